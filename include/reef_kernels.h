@@ -1,0 +1,246 @@
+/*
+ * Device-side boundary of the MI355X REEF build: what a model's code objects
+ * (<model>.raw.co, <model>.be.co, <model>.trans.co) export and how the host
+ * launches them.  Plain C, shared by the HIP kernels, the C++ executor and the
+ * Python model generator (which mirrors the attribute slots below).
+ *
+ * The reference resolves every graph-JSON `kernels[i].name` with
+ * hipModuleGetFunction and binds `kernels[i].args` (storage indices)
+ * positionally to the kernel's pointer parameters
+ * (src/reef/executor/executor_base.cpp:46-75, 211-223).  Its kernels are TVM
+ * output with shapes baked in, one symbol per layer instance.  Here the
+ * kernels are hand-written and shape-generic, so one symbol serves every layer
+ * of a family and the per-layer shape travels with the launch:
+ *
+ *   kernels[i].name           entry symbol (REEF_K_* below)
+ *   kernels[i].launch_params  [tasks,1,1, 256,1,1]   (logical workgroups x threads)
+ *   kernels[i].args           storage indices  -> ReefOpDesc.ptr[j], in order
+ *   kernels[i].attrs          int list         -> ReefOpDesc.attr[j], in order
+ *                              (added key; the reference parser ignores keys it
+ *                               does not look up, src/reef/executor/model.cpp:23-51)
+ *
+ * Three flavours of every entry, one per code object, as in the reference's
+ * model directories (src/reef/server/scheduler.cpp:62-65, src/reef/test/test.cpp:15-22):
+ *
+ *   raw    K(ReefOpDesc d)
+ *          grid = launch_params; replaces the plain TVM kernels.
+ *   be     K(int* preempted, int* task_slot, ReefOpDesc d)
+ *          replaces script/best_effort_kernel.py:22-29: a workgroup returns at
+ *          once when *preempted != 0, re-polls the flag inside its main loop,
+ *          and thread 0 adds 1 to *task_slot only when the workgroup completed.
+ *   trans  K(ReefDkpArgs a)   and   merge_framework_<n>(ReefDkpArgs a)
+ *          replaces the 11-argument dynamic-kernel-padding entry and the
+ *          merge_framework_* proxies (script/transform_kernel.py:345-352,
+ *          689-718; script/generate_asm_loop.py:189-321): one launch hosts a
+ *          real-time side and a best-effort side, each walking its own task
+ *          range with a persistent-workgroup loop.
+ *
+ * Every workgroup has 256 threads (4 wavefronts), 1-D.  A kernel body never
+ * reads blockIdx: it receives a logical task index, so any physical workgroup
+ * may run any task, which is what makes co-run results bit-identical to solo.
+ */
+#ifndef REEF_KERNELS_H
+#define REEF_KERNELS_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define REEF_WG_THREADS 256
+#define REEF_MAX_PTRS 8
+#define REEF_MAX_ATTRS 24
+
+typedef struct ReefOpDesc {
+    void* ptr[REEF_MAX_PTRS];      /* storages, JSON `args` order */
+    int32_t attr[REEF_MAX_ATTRS];  /* JSON `attrs` order */
+} ReefOpDesc;
+
+/* One side of a dynamic-kernel-padding launch
+ * (func/layers/task_num/task_offset/param of transform_kernel.py:345-352). */
+typedef struct ReefDkpSide {
+    int32_t op;           /* REEF_OP_* (replaces the device function pointer) */
+    int32_t layers;       /* workgroup layers this side may occupy per virtual CU */
+    int32_t task_num;     /* tasks to run in this launch */
+    int32_t task_offset;  /* first task */
+    ReefOpDesc desc;
+} ReefDkpSide;
+
+typedef struct ReefDkpArgs {
+    ReefDkpSide l;         /* real-time side  (virtual CUs below the partition) */
+    ReefDkpSide r;         /* best-effort side */
+    int32_t cu_partition;  /* virtual CUs given to side l, multiple of num_xcds */
+    int32_t num_cus;       /* virtual CUs per layer (grid = layers * num_cus) */
+    int32_t num_xcds;      /* 8 on MI355X; 1 reproduces the reference's flat mapping */
+    int32_t reserved;
+    int32_t* task_slot_r;  /* optional completion counter of side r (may be null) */
+} ReefDkpArgs;
+
+/* Op ids for ReefDkpSide.op (order is ABI). */
+enum {
+    REEF_OP_NONE = 0,
+    REEF_OP_CONV2D = 1,
+    REEF_OP_SPLITK_REDUCE = 2,
+    REEF_OP_DWCONV2D = 3,
+    REEF_OP_POOL2D = 4,
+    REEF_OP_GLOBAL_AVGPOOL = 5,
+    REEF_OP_ELTWISE = 6,
+    REEF_OP_DENSE = 7,
+    REEF_OP_SOFTMAX = 8,
+    REEF_OP_LAYERNORM = 9,
+    REEF_OP_BIAS_GELU = 10,
+    REEF_OP_EMBEDDING = 11,
+    REEF_OP_COPY = 12,
+    REEF_OP_TRANSPOSE = 13,
+    REEF_OP_GEMM = 14,
+    REEF_OP_MOCK_ADD = 15,
+    REEF_OP_MOCK_MULTIPLY = 16,
+    REEF_OP_COUNT
+};
+
+/* Entry symbols (graph-JSON kernel names). */
+#define REEF_K_CONV2D "reef_conv2d"
+#define REEF_K_SPLITK_REDUCE "reef_splitk_reduce"
+#define REEF_K_DWCONV2D "reef_dwconv2d"
+#define REEF_K_POOL2D "reef_pool2d"
+#define REEF_K_GLOBAL_AVGPOOL "reef_global_avgpool"
+#define REEF_K_ELTWISE "reef_eltwise"
+#define REEF_K_DENSE "reef_dense"
+#define REEF_K_SOFTMAX "reef_softmax"
+#define REEF_K_LAYERNORM "reef_layernorm"
+#define REEF_K_BIAS_GELU "reef_bias_gelu"
+#define REEF_K_EMBEDDING "reef_embedding"
+#define REEF_K_COPY "reef_copy"
+#define REEF_K_TRANSPOSE "reef_transpose"
+#define REEF_K_GEMM "reef_gemm"
+/* The reference's mocked model (resource/mocked_kernel/mocked_kernel.json)
+ * keeps its own names and its (64,1,1)x(4,8,4) launch. */
+#define REEF_K_MOCK_ADD "add"
+#define REEF_K_MOCK_MULTIPLY "multiply"
+
+/* Activation codes. */
+#define REEF_ACT_NONE 0
+#define REEF_ACT_RELU 1
+#define REEF_ACT_RELU6 2 /* clamp to [0, 6] */
+#define REEF_ACT_GELU 3  /* exact erf form, dense/gemm only */
+
+/* ---- reef_conv2d: fp32 implicit-GEMM convolution on MFMA (groups == 1) ----
+ * GEMM view: out[M=Cout][N=Ho*Wo] = W[M][K=Cin*kh*kw] x im2col(in)[K][N].
+ * ptr: in, W(OIHW), dst, then the optional operands in this order when their
+ *      flag bit is set: bias, residual, scale, shift.
+ *      dst is the output tensor when split_k == 1, else the split-K workspace
+ *      [split_k][Cout][Ho*Wo] that reef_splitk_reduce folds in a fixed order
+ *      (then the optional operands belong to the reduce launch instead).
+ * tasks = split_k * m_tiles * n_tiles;
+ * task -> (split = task / (m_tiles*n_tiles), m_tile, n_tile), n fastest. */
+enum {
+    REEF_CONV_CIN = 0, REEF_CONV_H, REEF_CONV_W, REEF_CONV_COUT, REEF_CONV_HO, REEF_CONV_WO,
+    REEF_CONV_KH, REEF_CONV_KW, REEF_CONV_SH, REEF_CONV_SW, REEF_CONV_PH, REEF_CONV_PW,
+    REEF_CONV_FLAGS,     /* REEF_F_* */
+    REEF_CONV_ACT,       /* REEF_ACT_* */
+    REEF_CONV_TILE,      /* REEF_TILE_* */
+    REEF_CONV_SPLIT_K,   /* >= 1 */
+    REEF_CONV_K_CHUNK,   /* K elements per split, multiple of the tile's BK */
+    REEF_CONV_M_TILES, REEF_CONV_N_TILES,
+    REEF_CONV_NATTR
+};
+#define REEF_F_BIAS 1
+#define REEF_F_RESIDUAL 2
+#define REEF_F_AFFINE 4 /* per-channel scale and shift after the sum */
+
+/* Tile configurations (BM x BN output tile per workgroup, BK = 32). */
+enum {
+    REEF_TILE_128x128 = 0,
+    REEF_TILE_128x64 = 1,
+    REEF_TILE_64x64 = 2,
+    REEF_TILE_128x32 = 3,
+    REEF_TILE_64x32 = 4,
+    REEF_TILE_COUNT
+};
+
+/* ---- reef_splitk_reduce: out = act(sum_s ws[s] (+res)(+bias)(*scale+shift)), s ascending ----
+ * ptr: ws, out, then optional bias, residual, scale, shift (same flag order).
+ * attr: M, N, split_k, flags, act.   tasks = ceil(M*N / 1024) (4 elements per thread). */
+enum { REEF_RED_M = 0, REEF_RED_N, REEF_RED_SPLIT_K, REEF_RED_FLAGS, REEF_RED_ACT, REEF_RED_NATTR };
+
+/* ---- reef_dwconv2d: depthwise k x k convolution + bias + activation (bandwidth-bound) ----
+ * ptr: in, W[C][kh][kw], out, bias(optional by flag).
+ * attr: C,H,W,Ho,Wo,kh,kw,sh,sw,ph,pw,flags,act.  tasks = ceil(C*Ho*Wo / 256). */
+enum {
+    REEF_DW_C = 0, REEF_DW_H, REEF_DW_W, REEF_DW_HO, REEF_DW_WO, REEF_DW_KH, REEF_DW_KW,
+    REEF_DW_SH, REEF_DW_SW, REEF_DW_PH, REEF_DW_PW, REEF_DW_FLAGS, REEF_DW_ACT, REEF_DW_NATTR
+};
+
+/* ---- reef_pool2d: max / average pooling (+bias +relu) ----
+ * ptr: in, out, bias(optional).  mode 0 max (pads with -FLT_MAX), 1 average.
+ * tasks = ceil(C*Ho*Wo / 256). */
+enum {
+    REEF_POOL_C = 0, REEF_POOL_H, REEF_POOL_W, REEF_POOL_HO, REEF_POOL_WO, REEF_POOL_KH,
+    REEF_POOL_KW, REEF_POOL_SH, REEF_POOL_SW, REEF_POOL_PH, REEF_POOL_PW, REEF_POOL_MODE,
+    REEF_POOL_COUNT_PAD, REEF_POOL_FLAGS, REEF_POOL_ACT, REEF_POOL_NATTR
+};
+
+/* ---- reef_global_avgpool: out[c] = sum(in[c][:]) * (1/HW).  ptr: in, out.
+ * attr: C, HW.  tasks = ceil(C / 4) (one wavefront per channel). */
+enum { REEF_GAP_C = 0, REEF_GAP_HW, REEF_GAP_NATTR };
+
+/* ---- reef_eltwise: out = act(a (+b) (*scale[c]) (+shift[c])), c = i / inner ----
+ * ptr: a, out, then optional b, scale, shift by flag.  attr: C, inner, flags, act.
+ * tasks = ceil(C*inner / 1024). */
+enum { REEF_ELT_C = 0, REEF_ELT_INNER, REEF_ELT_FLAGS, REEF_ELT_ACT, REEF_ELT_NATTR };
+#define REEF_ELT_F_B 1
+#define REEF_ELT_F_SCALE 2
+#define REEF_ELT_F_SHIFT 4
+
+/* ---- reef_dense: y[r][o] = act(sum_k x[r][k] W[o][k] + b[o]), few rows (GEMV, bandwidth-bound) ----
+ * ptr: x, W, y, bias(optional).  attr: rows, in_f, out_f, flags, act.
+ * tasks = ceil(out_f / 4) (one wavefront per output neuron). */
+enum { REEF_DENSE_ROWS = 0, REEF_DENSE_IN, REEF_DENSE_OUT, REEF_DENSE_FLAGS, REEF_DENSE_ACT, REEF_DENSE_NATTR };
+
+/* ---- reef_softmax: rows x cols, one wavefront per row.  ptr: in, out.  attr: rows, cols.
+ * tasks = ceil(rows / 4). */
+enum { REEF_SM_ROWS = 0, REEF_SM_COLS, REEF_SM_NATTR };
+
+/* ---- reef_layernorm: out = LN(x (+res)) * gamma + beta, one wavefront per row ----
+ * ptr: x, gamma, beta, out, res(optional).  attr: rows, cols, flags(bit0 = res), eps (float bits).
+ * tasks = ceil(rows / 4). */
+enum { REEF_LN_ROWS = 0, REEF_LN_COLS, REEF_LN_FLAGS, REEF_LN_EPS_BITS, REEF_LN_NATTR };
+
+/* ---- reef_bias_gelu: out = gelu_erf(x + bias[col]).  ptr: x, out, bias(optional).
+ * attr: rows, cols, flags.  tasks = ceil(rows*cols / 1024). */
+enum { REEF_GELU_ROWS = 0, REEF_GELU_COLS, REEF_GELU_FLAGS, REEF_GELU_NATTR };
+
+/* ---- reef_embedding: out[s][h] = tok[ids[s]][h] (+pos[s][h]) (+seg[h]) ----
+ * ptr: ids(int64), tok, out, pos(optional), seg(optional).
+ * attr: seq, hidden, flags(bit0 pos, bit1 seg), vocab.  tasks = ceil(seq*hidden/1024). */
+enum { REEF_EMB_SEQ = 0, REEF_EMB_HIDDEN, REEF_EMB_FLAGS, REEF_EMB_VOCAB, REEF_EMB_NATTR };
+
+/* ---- reef_copy: out[dst_off + i] = in[i].  ptr: in, out.  attr: count, dst_off.
+ * tasks = ceil(count / 1024). */
+enum { REEF_COPY_COUNT = 0, REEF_COPY_DST_OFF, REEF_COPY_NATTR };
+
+/* ---- reef_transpose: in [d0][d1][d2] -> out [d1][d0][d2] (+bias over (d1,d2)) ----
+ * ptr: in, out, bias(optional).  attr: d0, d1, d2, flags.  tasks = ceil(d0*d1*d2/1024). */
+enum { REEF_TR_D0 = 0, REEF_TR_D1, REEF_TR_D2, REEF_TR_FLAGS, REEF_TR_NATTR };
+
+/* ---- reef_gemm: batched fp32 GEMM on MFMA ----
+ * C[b][m][n] = act(alpha * sum_k A[b][m][k] * B(b,k,n) (+bias[n]))
+ * trans_b = 1: B stored [b][n][k] (dense layers, Q.K^T); 0: [b][k][n] (P.V).
+ * ptr: A, B, C, bias(optional).
+ * attr: batch, M, N, K, trans_b, flags, act, alpha (float bits), tile, m_tiles, n_tiles,
+ *       lda, ldb, ldc, strideA, strideB, strideC (elements).
+ * tasks = batch * m_tiles * n_tiles. */
+enum {
+    REEF_GEMM_BATCH = 0, REEF_GEMM_M, REEF_GEMM_N, REEF_GEMM_K, REEF_GEMM_TRANS_B,
+    REEF_GEMM_FLAGS, REEF_GEMM_ACT, REEF_GEMM_ALPHA_BITS, REEF_GEMM_TILE, REEF_GEMM_M_TILES,
+    REEF_GEMM_N_TILES, REEF_GEMM_LDA, REEF_GEMM_LDB, REEF_GEMM_LDC, REEF_GEMM_STRIDE_A,
+    REEF_GEMM_STRIDE_B, REEF_GEMM_STRIDE_C, REEF_GEMM_NATTR
+};
+
+/* ---- add / multiply (the reference's mocked model): ptr: a, b, out; no attrs ---- */
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* REEF_KERNELS_H */

@@ -1,0 +1,368 @@
+/*
+ * CPU oracle for the REEF hot path -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+ *
+ * Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may
+ * load this library.  The shipped library never links or calls it.
+ *
+ * Every function restates, as plain loops, the arithmetic of one kernel family
+ * of the reference's generated device code (the reference has no CPU path of
+ * its own; its kernels are TVM output with shapes baked in).  The citation on
+ * each function names the reference kernel whose per-element formula it
+ * follows.  Tensors are fp32, batch 1, NCHW activations / OIHW weights,
+ * row-major [rows][cols] matrices.
+ *
+ * Accumulation: `acc64 == 0` accumulates in fp32 with fused multiply-add in
+ * the reference's loop order (input channel outermost, then ky, kx), which is
+ * what the reference kernels do with __ocml_fma_f32; `acc64 != 0` accumulates
+ * in double and rounds once, which bounds the oracle's own rounding error.
+ *
+ * Pinning status (what checks each function, see tests/test_oracle_*.py):
+ *   conv2d / dense / batch_matmul / pools / softmax / layernorm / gelu /
+ *   eltwise / embedding / concat / transpose:
+ *     brute-force definitions on tiny shapes, algebraic invariants
+ *     (linearity, 1x1 conv == GEMM, softmax rows sum to 1, LN rows have
+ *     mean 0 / variance 1), and torch.nn.functional on CPU in fp64.
+ *   mocked add/multiply: the reference's closed form (3+3)*3 == 18.
+ *   The reference's ResNet-18 ten-float golden vector needs a weight blob that
+ *   is absent from the reference checkout: end-to-end parity with the TVM
+ *   model is "parity unpinned".
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#include <float.h>
+
+#define REEF_ACT_NONE 0
+#define REEF_ACT_RELU 1
+#define REEF_ACT_RELU6 2 /* clamp to [0, act_max] */
+
+static inline float apply_act(float v, int act, float act_max) {
+    if (act == REEF_ACT_RELU) return v > 0.0f ? v : 0.0f;
+    if (act == REEF_ACT_RELU6) {
+        v = v > 0.0f ? v : 0.0f;
+        return v < act_max ? v : act_max;
+    }
+    return v;
+}
+
+/*
+ * Fused convolution epilogue order, read off the reference kernels:
+ *   fused_nn_conv2d_add_nn_relu            relu(acc + bias[o])
+ *       resource/resnet152/resnet152.cu:376-713
+ *   fused_nn_conv2d_add                    acc + residual[o,y,x]
+ *       resource/resnet152/resnet152.cu:315-338
+ *   fused_nn_conv2d_add_add_nn_relu        relu((acc + residual) + bias[o])
+ *       resource/resnet152/resnet152.cu:2662
+ *   fused_nn_conv2d_add_multiply_add_nn_relu  relu(fma(acc + residual, scale[o], shift[o]))
+ *       resource/resnet152/resnet152.cu:340-363
+ * so the general form is: v = acc; v += residual; v += bias; v = fma(v, scale, shift); act.
+ * Depthwise convolution (mobilenet.cu fused_nn_conv2d_add_nn_relu_17_kernel0)
+ * is the groups == Cin case.
+ */
+void reef_oracle_conv2d(const float* in, const float* w, const float* bias,
+                        const float* residual, const float* scale, const float* shift,
+                        float* out, int Cin, int H, int W, int Cout, int kh, int kw,
+                        int sh, int sw, int ph, int pw, int groups, int act, float act_max,
+                        int acc64) {
+    const int Ho = (H + 2 * ph - kh) / sh + 1;
+    const int Wo = (W + 2 * pw - kw) / sw + 1;
+    const int cpg = Cin / groups;   /* input channels per group */
+    const int opg = Cout / groups;  /* output channels per group */
+#pragma omp parallel
+    {
+        float* accf = (float*)malloc(sizeof(float) * (size_t)Ho * Wo);
+        double* accd = acc64 ? (double*)malloc(sizeof(double) * (size_t)Ho * Wo) : NULL;
+#pragma omp for schedule(dynamic, 1)
+        for (int o = 0; o < Cout; ++o) {
+            const int g = o / opg;
+            if (acc64) memset(accd, 0, sizeof(double) * (size_t)Ho * Wo);
+            else memset(accf, 0, sizeof(float) * (size_t)Ho * Wo);
+            for (int ci = 0; ci < cpg; ++ci) {
+                const float* ip = in + (size_t)(g * cpg + ci) * H * W;
+                for (int ky = 0; ky < kh; ++ky) {
+                    for (int kx = 0; kx < kw; ++kx) {
+                        const float wv = w[(((size_t)o * cpg + ci) * kh + ky) * kw + kx];
+                        for (int y = 0; y < Ho; ++y) {
+                            const int iy = y * sh + ky - ph;
+                            if (iy < 0 || iy >= H) continue;
+                            /* x range with 0 <= x*sw + kx - pw < W */
+                            int x_lo = 0;
+                            if (pw - kx > 0) x_lo = (pw - kx + sw - 1) / sw;
+                            int x_hi = Wo;
+                            {
+                                int lim = W - 1 + pw - kx; /* x*sw <= lim */
+                                if (lim < 0) continue;
+                                int xh = lim / sw + 1;
+                                if (xh < x_hi) x_hi = xh;
+                            }
+                            const float* row = ip + (size_t)iy * W + (kx - pw);
+                            if (acc64) {
+                                double* a = accd + (size_t)y * Wo;
+                                for (int x = x_lo; x < x_hi; ++x)
+                                    a[x] += (double)row[x * sw] * (double)wv;
+                            } else {
+                                float* a = accf + (size_t)y * Wo;
+                                if (sw == 1) {
+                                    for (int x = x_lo; x < x_hi; ++x)
+                                        a[x] = fmaf(row[x], wv, a[x]);
+                                } else {
+                                    for (int x = x_lo; x < x_hi; ++x)
+                                        a[x] = fmaf(row[x * sw], wv, a[x]);
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+            float* op = out + (size_t)o * Ho * Wo;
+            const float* rp = residual ? residual + (size_t)o * Ho * Wo : NULL;
+            for (int i = 0; i < Ho * Wo; ++i) {
+                float v = acc64 ? (float)accd[i] : accf[i];
+                if (rp) v = v + rp[i];
+                if (bias) v = v + bias[o];
+                if (scale) v = fmaf(v, scale[o], shift[o]);
+                op[i] = apply_act(v, act, act_max);
+            }
+        }
+        free(accf);
+        if (accd) free(accd);
+    }
+}
+
+/*
+ * fused_nn_dense_add[_nn_relu]: y[r][o] = act(sum_k x[r][k] * W[o][k] + b[o])
+ * resource/resnet152/resnet152.cu:2-33 (one output neuron per block, k-loop,
+ * wave reduction, + bias).  rows > 1 covers the BERT projections
+ * (bert.cu:22-271, batch_matmul with a [out][in] weight).
+ * act: 0 none, 1 relu, 3 erf-GELU (bert.cu:167-173).
+ */
+static inline float gelu_erf(float x) {
+    /* x * (0.5 + 0.5 * erf(x * 0.70710678)) -- constants as in bert.cu:167-173 */
+    return x * (0.5f + 0.5f * erff(x * 0.70710678f));
+}
+
+void reef_oracle_dense(const float* x, const float* w, const float* bias, float* y, int rows,
+                       int in_f, int out_f, int act, int acc64) {
+#pragma omp parallel for schedule(static)
+    for (int o = 0; o < out_f; ++o) {
+        const float* wr = w + (size_t)o * in_f;
+        for (int r = 0; r < rows; ++r) {
+            const float* xr = x + (size_t)r * in_f;
+            float v;
+            if (acc64) {
+                double a = 0.0;
+                for (int k = 0; k < in_f; ++k) a += (double)xr[k] * (double)wr[k];
+                v = (float)a;
+            } else {
+                float a = 0.0f;
+                for (int k = 0; k < in_f; ++k) a = fmaf(xr[k], wr[k], a);
+                v = a;
+            }
+            if (bias) v += bias[o];
+            if (act == 1) v = v > 0.0f ? v : 0.0f;
+            else if (act == 3) v = gelu_erf(v);
+            y[(size_t)r * out_f + o] = v;
+        }
+    }
+}
+
+/*
+ * fused_nn_batch_matmul_{3,4,5} (bert.cu:22-271): C[b][m][n] = sum_k A[b][m][k] * B[b][n][k]
+ * (TVM batch_matmul contracts the LAST axis of both operands).  trans_b == 0
+ * gives the plain product sum_k A[b][m][k] * B[b][k][n] used for P.V.
+ * `alpha` scales the product (attention 1/sqrt(d)).
+ */
+void reef_oracle_batch_matmul(const float* a, const float* b, float* c, int batch, int M, int N,
+                              int K, int trans_b, float alpha, int acc64) {
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int bi = 0; bi < batch; ++bi) {
+        for (int m = 0; m < M; ++m) {
+            const float* ar = a + ((size_t)bi * M + m) * K;
+            for (int n = 0; n < N; ++n) {
+                double ad = 0.0;
+                float af = 0.0f;
+                for (int k = 0; k < K; ++k) {
+                    float bv = trans_b ? b[((size_t)bi * N + n) * K + k]
+                                       : b[((size_t)bi * K + k) * N + n];
+                    if (acc64) ad += (double)ar[k] * (double)bv;
+                    else af = fmaf(ar[k], bv, af);
+                }
+                float v = acc64 ? (float)ad : af;
+                c[((size_t)bi * M + m) * N + n] = v * alpha;
+            }
+        }
+    }
+}
+
+/*
+ * fused_nn_max_pool2d[_add_nn_relu] (resnet152.cu:365-374: padding value
+ * -3.402823e+38f, then + bias[c], relu) and fused_nn_avg_pool2d*
+ * (densenet/inception).  mode 0 = max, 1 = average.  For average pooling
+ * `count_include_pad` selects the divisor (window size vs valid taps).
+ */
+void reef_oracle_pool2d(const float* in, const float* bias, float* out, int C, int H, int W, int kh,
+                        int kw, int sh, int sw, int ph, int pw, int Ho, int Wo, int mode,
+                        int count_include_pad, int act) {
+#pragma omp parallel for schedule(static)
+    for (int c = 0; c < C; ++c) {
+        const float* ip = in + (size_t)c * H * W;
+        for (int y = 0; y < Ho; ++y) {
+            for (int x = 0; x < Wo; ++x) {
+                float m = -FLT_MAX;
+                float s = 0.0f;
+                int cnt = 0;
+                for (int dy = 0; dy < kh; ++dy) {
+                    for (int dx = 0; dx < kw; ++dx) {
+                        int iy = y * sh + dy - ph, ix = x * sw + dx - pw;
+                        if (iy < 0 || iy >= H || ix < 0 || ix >= W) continue;
+                        float v = ip[(size_t)iy * W + ix];
+                        m = v > m ? v : m;
+                        s += v;
+                        ++cnt;
+                    }
+                }
+                float v;
+                if (mode == 0) v = m;
+                else v = s / (float)(count_include_pad ? kh * kw : (cnt > 0 ? cnt : 1));
+                if (bias) v += bias[c];
+                if (act == 1) v = v > 0.0f ? v : 0.0f;
+                out[((size_t)c * Ho + y) * Wo + x] = v;
+            }
+        }
+    }
+}
+
+/* fused_nn_global_avg_pool2d (resnet152.cu:4390-4403): sum over H*W, times 1/(H*W). */
+void reef_oracle_global_avgpool(const float* in, float* out, int C, int HW) {
+    const float inv = 1.0f / (float)HW;
+    for (int c = 0; c < C; ++c) {
+        float s = 0.0f;
+        for (int i = 0; i < HW; ++i) s += in[(size_t)c * HW + i];
+        out[c] = s * inv;
+    }
+}
+
+/*
+ * Elementwise family: fused_add_* / fused_add_nn_relu* (resnet152.cu:771-773,
+ * 4056-4066, 4782-4784): out = act(a [+ b] [* scale[c]] [+ shift[c]]),
+ * channel c = i / inner.  `b` is a same-shape tensor; scale/shift are
+ * per-channel vectors.
+ */
+void reef_oracle_eltwise(const float* a, const float* b, const float* scale, const float* shift,
+                         float* out, int C, int inner, int act, float act_max) {
+    for (int c = 0; c < C; ++c) {
+        for (int i = 0; i < inner; ++i) {
+            size_t idx = (size_t)c * inner + i;
+            float v = a[idx];
+            if (b) v = v + b[idx];
+            if (scale) v = v * scale[c];
+            if (shift) v = v + shift[c];
+            out[idx] = apply_act(v, act, act_max);
+        }
+    }
+}
+
+/*
+ * fused_nn_softmax (resnet152.cu:775-841; bert.cu:3-13,159-166,327-337,389-396):
+ * per row: m = max, e = exp(x - m), out = e / sum(e).
+ */
+void reef_oracle_softmax(const float* in, float* out, int rows, int cols) {
+    for (int r = 0; r < rows; ++r) {
+        const float* x = in + (size_t)r * cols;
+        float* y = out + (size_t)r * cols;
+        float m = -FLT_MAX;
+        for (int i = 0; i < cols; ++i) m = x[i] > m ? x[i] : m;
+        float s = 0.0f;
+        for (int i = 0; i < cols; ++i) {
+            y[i] = expf(x[i] - m);
+            s += y[i];
+        }
+        for (int i = 0; i < cols; ++i) y[i] = y[i] / s;
+    }
+}
+
+/*
+ * LayerNorm as the reference splits it (bert.cu:175-205, 338-380):
+ * mean = sum(x)/n; var = sum((x-mean)^2)/n; out = (x-mean)/sqrt(var+eps)*gamma+beta.
+ * Optional residual `res` is added to x first (BERT add & norm).
+ */
+void reef_oracle_layernorm(const float* in, const float* res, const float* gamma,
+                           const float* beta, float* out, int rows, int cols, float eps) {
+    for (int r = 0; r < rows; ++r) {
+        const float* x = in + (size_t)r * cols;
+        const float* rr = res ? res + (size_t)r * cols : NULL;
+        float* y = out + (size_t)r * cols;
+        double s = 0.0;
+        for (int i = 0; i < cols; ++i) s += (double)(rr ? x[i] + rr[i] : x[i]);
+        float mean = (float)(s / cols);
+        double v = 0.0;
+        for (int i = 0; i < cols; ++i) {
+            float d = (rr ? x[i] + rr[i] : x[i]) - mean;
+            v += (double)d * d;
+        }
+        float var = (float)(v / cols);
+        float inv = 1.0f / sqrtf(var + eps);
+        for (int i = 0; i < cols; ++i) {
+            float d = (rr ? x[i] + rr[i] : x[i]) - mean;
+            y[i] = d * inv * gamma[i] + beta[i];
+        }
+    }
+}
+
+/* fused_reshape_add_multiply_erf_multiply_add_multiply_reshape (bert.cu:167-173):
+ * out = gelu_erf(x + bias[col]). */
+void reef_oracle_bias_gelu(const float* in, const float* bias, float* out, int rows, int cols) {
+    for (int r = 0; r < rows; ++r)
+        for (int c = 0; c < cols; ++c) {
+            float v = in[(size_t)r * cols + c] + (bias ? bias[c] : 0.0f);
+            out[(size_t)r * cols + c] = gelu_erf(v);
+        }
+}
+
+/*
+ * fused_cast_take_..._take_add_1 (bert.cu:14-21): token + position (+ segment)
+ * embedding gather, int64 ids.  out[s][h] = tok[ids[s]][h] + pos[s][h] + seg[h].
+ */
+void reef_oracle_embedding(const int64_t* ids, const float* tok, const float* pos,
+                           const float* seg, float* out, int seq, int hidden) {
+    for (int s = 0; s < seq; ++s)
+        for (int h = 0; h < hidden; ++h) {
+            float v = tok[(size_t)ids[s] * hidden + h];
+            if (pos) v += pos[(size_t)s * hidden + h];
+            if (seg) v += seg[h];
+            out[(size_t)s * hidden + h] = v;
+        }
+}
+
+/* fused_concatenate (inception.cu): copy `count` floats to out + offset. */
+void reef_oracle_copy(const float* in, float* out, size_t out_offset, size_t count) {
+    memcpy(out + out_offset, in, count * sizeof(float));
+}
+
+/*
+ * Head split / merge movers (bert.cu:273-326, 344-351, 381-388):
+ * in [d0][d1][d2] -> out [d1][d0][d2] (+ optional bias over the flattened
+ * (d1,d2) feature axis of the input row, which is how the reference fuses the
+ * projection bias into the transpose).
+ */
+void reef_oracle_transpose_102(const float* in, const float* bias, float* out, int d0, int d1,
+                               int d2) {
+    for (int a = 0; a < d0; ++a)
+        for (int b = 0; b < d1; ++b)
+            for (int c = 0; c < d2; ++c) {
+                float v = in[((size_t)a * d1 + b) * d2 + c];
+                if (bias) v += bias[(size_t)b * d2 + c];
+                out[((size_t)b * d0 + a) * d2 + c] = v;
+            }
+}
+
+/* mocked_kernel.cu:9-27: temp[blk*128+t] = a[t] (+|*) b[blk*128+t], 64 blocks x 128 threads. */
+void reef_oracle_mocked(const float* a, const float* b, float* out, int blocks, int threads,
+                        int is_multiply) {
+    for (int blk = 0; blk < blocks; ++blk)
+        for (int t = 0; t < threads; ++t) {
+            int i = blk * threads + t;
+            out[i] = is_multiply ? a[t] * b[i] : a[t] + b[i];
+        }
+}
