@@ -1,0 +1,97 @@
+/*
+ * reef_c.h -- flat C view of the executor and scheduler classes, for callers
+ * that cannot include C++ headers (the Python tests and benchmark bind it with
+ * ctypes).  Each function forwards to the C++ method of the same name, which in
+ * turn mirrors the reference class it replaces:
+ *   ExecutorBase     src/reef/executor/executor_base.h:17-69
+ *   TransExecutor    src/reef/executor/trans_executor.h:41-87
+ *   HybridExecutor   src/reef/executor/hybrid_executor.h:18-76
+ *   REEFScheduler    src/reef/server/scheduler.h:15-190
+ * Return value: reef::Status as an int (0 Succ, 1 Fail, 2 NotFound,
+ * 3 OutOfRange, 4 Full), as in src/reef/util/common.h:46-52.
+ */
+#ifndef REEF_C_H
+#define REEF_C_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct reef_executor_s* reef_executor_t;
+
+enum { REEF_EXECUTOR_BASE = 0, REEF_EXECUTOR_TRANS = 1, REEF_EXECUTOR_HYBRID = 2 };
+/* Which flavour a timing helper launches. */
+enum { REEF_RUN_DEFAULT = 0, REEF_RUN_PREEMPTIBLE = 1 };
+
+int reef_executor_create(int kind, reef_executor_t* out);
+void reef_executor_destroy(reef_executor_t e);
+/* ExecutorBase::load_model_from_file (executor_base.cpp:15-27); for a TransExecutor `co` is the trans.co. */
+int reef_executor_load(reef_executor_t e, const char* json_path, const char* co_path);
+/* HybridExecutor::load_hybrid_model_from_file (hybrid_executor.cpp:14-31) */
+int reef_executor_load_hybrid(reef_executor_t e, const char* json_path, const char* profile_path,
+                              const char* trans_co_path, const char* be_co_path);
+int reef_executor_load_param(reef_executor_t e, const char* param_path);
+int reef_executor_set_input(reef_executor_t e, const char* name, const void* data, size_t len);
+int reef_executor_set_input_idx(reef_executor_t e, int idx, const void* data, size_t len);
+int reef_executor_get_data_size(reef_executor_t e, const char* name, size_t* size);
+int reef_executor_get_output(reef_executor_t e, void* out, size_t len);
+int reef_executor_get_data(reef_executor_t e, int idx, void* out, size_t len);
+int reef_executor_execute(reef_executor_t e);
+int reef_executor_execute_to(reef_executor_t e, int idx);
+int reef_executor_execute_kernel(reef_executor_t e, int idx);
+int reef_executor_execute_preemptable(reef_executor_t e);
+int reef_executor_num_kernels(reef_executor_t e);
+/* Sets the executor's own 4-byte preemption flag (hybrid only) to `value`. */
+int reef_executor_poke_preempt_flag(reef_executor_t e, int value);
+/* Reads the per-kernel completion counters (hybrid only) into out[0..n). */
+int reef_executor_read_task_slots(reef_executor_t e, int* out, int n);
+/* Per-kernel resource record: out = {block_num, min_occupancy, vgprs, sgprs, lds, scratch, op}. */
+int reef_executor_kernel_info(reef_executor_t e, int idx, int out[7]);
+
+/*
+ * Measurement helpers (device events on the stream the kernels run on).
+ * time_kernel: `warmup` untimed launches of kernel idx, then `iters` timed
+ *   launches bracketed by two events; *avg_us = elapsed / iters.
+ * time_model:  `warmup` whole-model runs, then `iters` runs, each bracketed by
+ *   events and by host clocks; lat_us[i] = host-observed latency of run i
+ *   (launch of the first kernel to completion of the last), dev_us[i] = device
+ *   time between the events.  Either output may be NULL.
+ */
+int reef_executor_time_kernel(reef_executor_t e, int idx, int flavour, int warmup, int iters,
+                              float* avg_us);
+int reef_executor_time_model(reef_executor_t e, int flavour, int warmup, int iters, float* lat_us,
+                             float* dev_us);
+
+/* GPUConfig (src/reef/executor/hip/hip_impl.cpp:9-74) */
+int reef_gpuconfig_num_cus(void);
+int reef_gpuconfig_num_xcds(void);
+void reef_gpuconfig_override_geometry(int num_cus, int num_xcds);
+int reef_gpuconfig_calculate_occupancy(int shared_memory, int vgprs, int sgprs, int stack_size,
+                                       int block_threads);
+/* DKP arithmetic shared by TransExecutor and the scheduler. */
+int reef_dkp_logical_layers(int block_num, int num_cus);
+int reef_dkp_cu_partition(int block_num, int num_cus, int num_xcds);
+int reef_dkp_occupancy_class(int vgprs);
+/* Host replica of the device-side side/task walk (one physical workgroup):
+ * returns the number of tasks written to tasks[0..cap), *is_right = side. */
+int reef_dkp_walk(int block_idx, int num_cus, int num_xcds, int cu_partition, int layers_l,
+                  int task_num_l, int task_offset_l, int layers_r, int task_num_r,
+                  int task_offset_r, int* is_right, int* tasks, int cap);
+
+/* Parsers (src/reef/executor/model.cpp), exposed for format tests. */
+int reef_model_parse_summary(const char* json_path, int* n_storage, int* n_kernels, int* n_args,
+                             int* n_shared);
+int reef_profile_parse_summary(const char* json_path, int* model_latency, int* n_kernels,
+                               int* min_latency, int* n_latency_values);
+int reef_profile_roundtrip(const char* json_path, char* out, size_t cap);
+int reef_param_parse_summary(const char* param_path, const char* key, uint64_t* n_tensors,
+                             uint64_t* key_len, float* first, float* last);
+int reef_code_object_kernel_meta(const char* co_path, const char* kernel, int out[6]);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* REEF_C_H */

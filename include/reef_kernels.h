@@ -155,7 +155,8 @@ enum {
     REEF_TILE_128x64 = 1,
     REEF_TILE_64x64 = 2,
     REEF_TILE_128x32 = 3,
-    REEF_TILE_64x32 = 4,
+    REEF_TILE_32x128 = 4,
+    REEF_TILE_64x128 = 5,
     REEF_TILE_COUNT
 };
 

@@ -270,14 +270,14 @@ class GraphOracle:
     def run_kernel(self, k, acc64=False):
         name, a = k["name"], k.get("attrs", [])
         P = [self.storage[i] for i in k["args"]]
-        if name == "reef_conv2d":
+        if name.startswith("reef_conv2d"):
             Cin, H, W, Cout, Ho, Wo, kh, kw, sh, sw, ph, pw, flags, act, _tile, split_k = a[:16]
             if split_k > 1:
                 # The partial sums are an implementation detail of the device
                 # kernel; the oracle computes the whole convolution into slot 0
                 # of the workspace and leaves the other slots zero, which the
                 # ordered reduce then folds to the same mathematical result.
-                ws = P[2]
+                ws = P[2].view(np.float32)
                 ws[:] = 0
                 out = conv2d(P[0][:Cin * H * W].reshape(Cin, H, W),
                              P[1][:Cout * Cin * kh * kw].reshape(Cout, Cin, kh, kw),
@@ -294,8 +294,9 @@ class GraphOracle:
             M, N, split_k, flags, act = a[:5]
             bias, res, scale, shift = self._conv_opt(P, 2, flags)
             acc = np.zeros(M * N, np.float32)
+            ws = P[0].view(np.float32)
             for s in range(split_k):
-                acc = acc + P[0][s * M * N:(s + 1) * M * N]
+                acc = acc + ws[s * M * N:(s + 1) * M * N]
             v = acc.reshape(M, N)
             if res is not None:
                 v = v + res[:M * N].reshape(M, N)
@@ -363,7 +364,7 @@ class GraphOracle:
             bias = P[2] if flags & 1 else None
             y = transpose_102(P[0][:d0 * d1 * d2].reshape(d0, d1, d2), bias)
             P[1][:y.size] = y.reshape(-1)
-        elif name == "reef_gemm":
+        elif name.startswith("reef_gemm"):
             (batch, M, N, K, trans_b, flags, act, alpha_bits, _t, _mt, _nt, lda, ldb, ldc, sA, sB,
              sC) = a[:17]
             alpha = _bits_to_float(alpha_bits)

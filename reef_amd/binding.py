@@ -1,0 +1,162 @@
+"""ctypes binding of the flat C API (include/reef_c.h) of libreef_amd.so.
+
+The library is the product; this module only marshals arguments.  It raises if
+the library has not been built -- there is no fallback path.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+from .paths import LIB_PATH
+
+STATUS = {0: "Succ", 1: "Fail", 2: "NotFound", 3: "OutOfRange", 4: "Full"}
+BASE, TRANS, HYBRID = 0, 1, 2
+RUN_DEFAULT, RUN_PREEMPTIBLE = 0, 1
+
+_lib = None
+
+
+class ReefError(RuntimeError):
+    def __init__(self, what, status):
+        super().__init__("%s -> %s (%s)" % (what, STATUS.get(status, status), last_error()))
+        self.status = status
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("libreef_amd.so is not built: run __graft_entry__.build() "
+                               "(make -C reef_amd/csrc)")
+        _lib = ctypes.CDLL(LIB_PATH)
+        _lib.reef_hal_last_error.restype = ctypes.c_char_p
+    return _lib
+
+
+def last_error():
+    try:
+        return lib().reef_hal_last_error().decode()
+    except Exception:  # pragma: no cover
+        return ""
+
+
+def _check(what, st):
+    if st != 0:
+        raise ReefError(what, st)
+
+
+class Executor:
+    """ExecutorBase / TransExecutor / HybridExecutor behind one Python class."""
+
+    def __init__(self, kind=BASE):
+        self.kind = kind
+        self.h = ctypes.c_void_p()
+        _check("create", lib().reef_executor_create(kind, ctypes.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib().reef_executor_destroy(self.h)
+            self.h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @classmethod
+    def from_dir(cls, model_dir, name, kind=BASE, load_params=True):
+        """Loads <dir>/<name>.{json,profile.json,raw.co|trans.co,be.co,param}."""
+        e = cls(kind)
+        base = os.path.join(model_dir, name)
+        if kind == BASE:
+            e.load(base + ".json", base + ".raw.co")
+        elif kind == TRANS:
+            e.load(base + ".json", base + ".trans.co")
+        else:
+            e.load_hybrid(base + ".json", base + ".profile.json", base + ".trans.co", base + ".be.co")
+        if load_params and os.path.exists(base + ".param"):
+            e.load_param(base + ".param")
+        return e
+
+    def load(self, json_path, co_path):
+        _check("load_model_from_file",
+               lib().reef_executor_load(self.h, json_path.encode(), co_path.encode()))
+
+    def load_hybrid(self, json_path, profile_path, trans_co, be_co):
+        _check("load_hybrid_model_from_file",
+               lib().reef_executor_load_hybrid(self.h, json_path.encode(), profile_path.encode(),
+                                               trans_co.encode(), be_co.encode()))
+
+    def load_param(self, path):
+        _check("load_param_from_file", lib().reef_executor_load_param(self.h, path.encode()))
+
+    def set_input(self, name, arr):
+        arr = np.ascontiguousarray(arr)
+        return lib().reef_executor_set_input(self.h, name.encode(), arr.ctypes.data_as(ctypes.c_void_p),
+                                             ctypes.c_size_t(arr.nbytes))
+
+    def set_input_checked(self, name, arr):
+        _check("set_input(%s)" % name, self.set_input(name, arr))
+
+    def get_data_size(self, name):
+        sz = ctypes.c_size_t()
+        _check("get_data_size", lib().reef_executor_get_data_size(self.h, name.encode(), ctypes.byref(sz)))
+        return sz.value
+
+    def get_output(self, n=None):
+        if n is None:
+            n = self.get_data_size("output") // 4
+        out = np.empty(n, np.float32)
+        _check("get_output", lib().reef_executor_get_output(self.h, out.ctypes.data_as(ctypes.c_void_p),
+                                                           ctypes.c_size_t(out.nbytes)))
+        return out
+
+    def get_data(self, idx, n, dtype=np.float32):
+        out = np.empty(n, dtype)
+        _check("get_data", lib().reef_executor_get_data(self.h, idx, out.ctypes.data_as(ctypes.c_void_p),
+                                                       ctypes.c_size_t(out.nbytes)))
+        return out
+
+    def execute(self):
+        _check("execute", lib().reef_executor_execute(self.h))
+
+    def execute_to(self, idx):
+        _check("execute_to", lib().reef_executor_execute_to(self.h, idx))
+
+    def execute_kernel(self, idx):
+        _check("execute_kernel", lib().reef_executor_execute_kernel(self.h, idx))
+
+    def execute_preemptable(self):
+        _check("execute_preemptale", lib().reef_executor_execute_preemptable(self.h))
+
+    def num_kernels(self):
+        return lib().reef_executor_num_kernels(self.h)
+
+    def poke_preempt_flag(self, value):
+        _check("poke_preempt_flag", lib().reef_executor_poke_preempt_flag(self.h, int(value)))
+
+    def read_task_slots(self):
+        n = self.num_kernels()
+        out = (ctypes.c_int * n)()
+        _check("read_task_slots", lib().reef_executor_read_task_slots(self.h, out, n))
+        return list(out)
+
+    def kernel_info(self, idx):
+        out = (ctypes.c_int * 7)()
+        _check("kernel_info", lib().reef_executor_kernel_info(self.h, idx, out))
+        keys = ("block_num", "min_occupancy", "vgprs", "sgprs", "lds", "scratch", "op")
+        return dict(zip(keys, out))
+
+    def time_kernel(self, idx, flavour=RUN_DEFAULT, warmup=5, iters=50):
+        us = ctypes.c_float()
+        _check("time_kernel", lib().reef_executor_time_kernel(self.h, idx, flavour, warmup, iters,
+                                                             ctypes.byref(us)))
+        return us.value
+
+    def time_model(self, flavour=RUN_DEFAULT, warmup=5, iters=50):
+        lat = (ctypes.c_float * iters)()
+        dev = (ctypes.c_float * iters)()
+        _check("time_model", lib().reef_executor_time_model(self.h, flavour, warmup, iters, lat, dev))
+        return np.array(lat, np.float64), np.array(dev, np.float64)

@@ -1,0 +1,266 @@
+// Flat C view of the executors (include/reef_c.h).
+#include <chrono>
+#include <cstring>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "executor/hybrid_executor.h"
+#include "hal/code_object.h"
+#include "reef_c.h"
+
+using namespace reef;
+using namespace reef::executor;
+
+struct reef_executor_s {
+    int kind;
+    std::unique_ptr<ExecutorBase> exe;
+    HybridExecutor* hybrid() { return kind == REEF_EXECUTOR_HYBRID ? static_cast<HybridExecutor*>(exe.get()) : nullptr; }
+    TransExecutor* trans() { return kind >= REEF_EXECUTOR_TRANS ? static_cast<TransExecutor*>(exe.get()) : nullptr; }
+};
+
+namespace {
+// Opens up launch_range / launch_preempt_kernel for the timing helpers.
+Status launch_all(reef_executor_s* e, int flavour, int begin, int end) {
+    if (flavour == REEF_RUN_PREEMPTIBLE) {
+        HybridExecutor* h = e->hybrid();
+        if (!h) return Status::Fail;
+        for (int i = begin; i < end; ++i) RETURN_STATUS(h->launch_preempt_kernel(i, h->stream()));
+        return Status::Succ;
+    }
+    return e->exe->launch_range(begin, end, e->exe->stream());
+}
+}  // namespace
+
+extern "C" {
+
+int reef_executor_create(int kind, reef_executor_t* out) {
+    reef_executor_s* e = new reef_executor_s;
+    e->kind = kind;
+    if (kind == REEF_EXECUTOR_BASE) e->exe.reset(new ExecutorBase);
+    else if (kind == REEF_EXECUTOR_TRANS) e->exe.reset(new TransExecutor);
+    else if (kind == REEF_EXECUTOR_HYBRID) e->exe.reset(new HybridExecutor);
+    else { delete e; return Status::OutOfRange; }
+    *out = e;
+    return Status::Succ;
+}
+void reef_executor_destroy(reef_executor_t e) { delete e; }
+
+int reef_executor_load(reef_executor_t e, const char* json_path, const char* co_path) {
+    return e->exe->load_model_from_file(json_path, co_path);
+}
+int reef_executor_load_hybrid(reef_executor_t e, const char* json_path, const char* profile_path,
+                              const char* trans_co_path, const char* be_co_path) {
+    HybridExecutor* h = e->hybrid();
+    if (!h) return Status::Fail;
+    return h->load_hybrid_model_from_file(json_path, profile_path, trans_co_path, be_co_path);
+}
+int reef_executor_load_param(reef_executor_t e, const char* p) { return e->exe->load_param_from_file(p); }
+int reef_executor_set_input(reef_executor_t e, const char* name, const void* data, size_t len) {
+    return e->exe->set_input(std::string(name), data, len);
+}
+int reef_executor_set_input_idx(reef_executor_t e, int idx, const void* data, size_t len) {
+    return e->exe->set_input(idx, data, len);
+}
+int reef_executor_get_data_size(reef_executor_t e, const char* name, size_t* size) {
+    return e->exe->get_data_size(name, *size);
+}
+int reef_executor_get_output(reef_executor_t e, void* out, size_t len) { return e->exe->get_output(out, len); }
+int reef_executor_get_data(reef_executor_t e, int idx, void* out, size_t len) {
+    return e->exe->get_data(idx, out, len);
+}
+int reef_executor_execute(reef_executor_t e) { return e->exe->execute(e->exe->stream()); }
+int reef_executor_execute_to(reef_executor_t e, int idx) { return e->exe->execute_to(idx, e->exe->stream()); }
+int reef_executor_execute_kernel(reef_executor_t e, int idx) {
+    return e->exe->execute_kernel(idx, e->exe->stream());
+}
+int reef_executor_execute_preemptable(reef_executor_t e) {
+    HybridExecutor* h = e->hybrid();
+    if (!h) return Status::Fail;
+    return h->execute_preemptale(h->stream());
+}
+int reef_executor_num_kernels(reef_executor_t e) { return (int)e->exe->num_kernels(); }
+
+namespace {
+struct HybridPeek : public HybridExecutor {
+    GPUDevicePtr_t flag() const { return preempt_flag; }
+    GPUDevicePtr_t slots() const { return task_slot_base; }
+};
+}  // namespace
+
+int reef_executor_poke_preempt_flag(reef_executor_t e, int value) {
+    HybridExecutor* h = e->hybrid();
+    if (!h) return Status::Fail;
+    GPUDevicePtr_t flag = static_cast<HybridPeek*>(h)->flag();
+    if (reef_hal_memcpy_h2d(flag, &value, 4) != 0) return Status::Fail;
+    return Status::Succ;
+}
+int reef_executor_read_task_slots(reef_executor_t e, int* out, int n) {
+    HybridExecutor* h = e->hybrid();
+    if (!h || n > (int)h->num_kernels()) return Status::Fail;
+    if (reef_hal_memcpy_d2h(out, static_cast<HybridPeek*>(h)->slots(), (size_t)n * 4) != 0) return Status::Fail;
+    return Status::Succ;
+}
+int reef_executor_kernel_info(reef_executor_t e, int idx, int out[7]) {
+    TransExecutor* t = e->trans();
+    if (!t || idx < 0 || idx >= (int)t->num_kernels()) return Status::OutOfRange;
+    const TransExecutor::KernelArg& ka = t->kernel_args()[idx];
+    out[0] = ka.block_num;
+    out[1] = ka.min_occupancy;
+    out[2] = ka.resource.vgprs;
+    out[3] = ka.resource.sgprs;
+    out[4] = ka.resource.shared_memory;
+    out[5] = ka.resource.stack_size;
+    out[6] = ka.op;
+    return Status::Succ;
+}
+
+int reef_executor_time_kernel(reef_executor_t e, int idx, int flavour, int warmup, int iters,
+                              float* avg_us) {
+    if (idx < 0 || idx >= (int)e->exe->num_kernels() || iters <= 0) return Status::OutOfRange;
+    GPUStream_t s = e->exe->stream();
+    for (int i = 0; i < warmup; ++i) RETURN_STATUS(launch_all(e, flavour, idx, idx + 1));
+    reef_event_t a, b;
+    GPU_RETURN_STATUS(reef_hal_event_create(&a));
+    GPU_RETURN_STATUS(reef_hal_event_create(&b));
+    GPU_RETURN_STATUS(reef_hal_stream_sync(s));
+    GPU_RETURN_STATUS(reef_hal_event_record(a, s));
+    for (int i = 0; i < iters; ++i) RETURN_STATUS(launch_all(e, flavour, idx, idx + 1));
+    GPU_RETURN_STATUS(reef_hal_event_record(b, s));
+    GPU_RETURN_STATUS(reef_hal_event_sync(b));
+    float us = 0.f;
+    GPU_RETURN_STATUS(reef_hal_event_elapsed_us(a, b, &us));
+    *avg_us = us / (float)iters;
+    reef_hal_event_destroy(a);
+    reef_hal_event_destroy(b);
+    return Status::Succ;
+}
+
+int reef_executor_time_model(reef_executor_t e, int flavour, int warmup, int iters, float* lat_us,
+                             float* dev_us) {
+    GPUStream_t s = e->exe->stream();
+    const int n = (int)e->exe->num_kernels();
+    reef_event_t a, b;
+    GPU_RETURN_STATUS(reef_hal_event_create(&a));
+    GPU_RETURN_STATUS(reef_hal_event_create(&b));
+    for (int it = -warmup; it < iters; ++it) {
+        GPU_RETURN_STATUS(reef_hal_stream_sync(s));
+        auto t0 = std::chrono::steady_clock::now();
+        GPU_RETURN_STATUS(reef_hal_event_record(a, s));
+        RETURN_STATUS(launch_all(e, flavour, 0, n));
+        GPU_RETURN_STATUS(reef_hal_event_record(b, s));
+        GPU_RETURN_STATUS(reef_hal_stream_sync(s));
+        auto t1 = std::chrono::steady_clock::now();
+        if (it >= 0) {
+            if (lat_us) lat_us[it] = std::chrono::duration<float, std::micro>(t1 - t0).count();
+            if (dev_us) GPU_RETURN_STATUS(reef_hal_event_elapsed_us(a, b, &dev_us[it]));
+        }
+    }
+    reef_hal_event_destroy(a);
+    reef_hal_event_destroy(b);
+    return Status::Succ;
+}
+
+int reef_gpuconfig_num_cus(void) { return (int)GPUConfig::get_num_cus(); }
+int reef_gpuconfig_num_xcds(void) { return (int)GPUConfig::get_num_xcds(); }
+void reef_gpuconfig_override_geometry(int num_cus, int num_xcds) {
+    GPUConfig::override_geometry((uint32_t)num_cus, (uint32_t)num_xcds);
+}
+int reef_gpuconfig_calculate_occupancy(int shared_memory, int vgprs, int sgprs, int stack_size,
+                                       int block_threads) {
+    GPUConfig::KernelResource kr{shared_memory, vgprs, sgprs, stack_size};
+    return GPUConfig::calculate_occupancy(kr, block_threads);
+}
+int reef_dkp_logical_layers(int block_num, int num_cus) {
+    return TransExecutor::logical_layers(block_num, num_cus);
+}
+int reef_dkp_cu_partition(int block_num, int num_cus, int num_xcds) {
+    return TransExecutor::cu_partition_for(block_num, num_cus, num_xcds);
+}
+int reef_dkp_occupancy_class(int vgprs) {
+    GPUConfig::KernelResource kr{0, vgprs, 0, 0};
+    return TransExecutor::occupancy_class(kr);
+}
+
+// Same arithmetic as dkp_walk in kernels/reef_entries.hip, on the host.
+int reef_dkp_walk(int b, int C, int X, int cu_partition, int layers_l, int task_num_l,
+                  int task_offset_l, int layers_r, int task_num_r, int task_offset_r, int* is_right,
+                  int* tasks, int cap) {
+    const int layer = b / C, cu = b - layer * C;
+    const int xcd = cu % X, slot = cu / X;
+    const int rt_slots = cu_partition / X;
+    int span, cu_idx, layers, task_num, task_offset;
+    if (slot < rt_slots) {
+        *is_right = 0;
+        span = rt_slots * X; cu_idx = slot * X + xcd;
+        layers = layers_l; task_num = task_num_l; task_offset = task_offset_l;
+    } else {
+        *is_right = 1;
+        span = C - rt_slots * X; cu_idx = (slot - rt_slots) * X + xcd;
+        layers = layers_r; task_num = task_num_r; task_offset = task_offset_r;
+    }
+    if (layer >= layers) return 0;
+    int n = 0;
+    const int step = layers * span, end = task_offset + task_num;
+    for (int i = span * layer + cu_idx + task_offset; i < end; i += step) {
+        if (n < cap) tasks[n] = i;
+        ++n;
+    }
+    return n;
+}
+
+int reef_model_parse_summary(const char* json_path, int* n_storage, int* n_kernels, int* n_args,
+                             int* n_shared) {
+    std::unique_ptr<Model> m(Model::from_json(json_path));
+    if (!m) return Status::NotFound;
+    *n_storage = (int)m->storage.size();
+    *n_kernels = (int)m->kernels.size();
+    *n_args = (int)m->args.size();
+    *n_shared = (int)m->shared_memory.size();
+    return Status::Succ;
+}
+int reef_profile_parse_summary(const char* json_path, int* model_latency, int* n_kernels,
+                               int* min_latency, int* n_latency_values) {
+    std::unique_ptr<ModelProfile> p(ModelProfile::from_json(json_path));
+    if (!p) return Status::NotFound;
+    *model_latency = p->model_latency;
+    *n_kernels = (int)p->kernel_latency.size();
+    int mn = 1 << 30, cnt = 0;
+    for (auto& kv : p->kernel_latency)
+        for (int v : kv.second.latency) { mn = std::min(mn, v); ++cnt; }
+    *min_latency = cnt ? mn : 0;
+    *n_latency_values = cnt;
+    return Status::Succ;
+}
+int reef_profile_roundtrip(const char* json_path, char* out, size_t cap) {
+    std::unique_ptr<ModelProfile> p(ModelProfile::from_json(json_path));
+    if (!p) return Status::NotFound;
+    std::string s = p->to_json();
+    if (s.size() + 1 > cap) return Status::OutOfRange;
+    std::memcpy(out, s.c_str(), s.size() + 1);
+    return Status::Succ;
+}
+int reef_param_parse_summary(const char* param_path, const char* key, uint64_t* n_tensors,
+                             uint64_t* key_len, float* first, float* last) {
+    std::unique_ptr<ModelParam> p(ModelParamParser::parse_from_file(param_path));
+    if (!p) return Status::NotFound;
+    *n_tensors = p->size();
+    auto it = p->find(key);
+    if (it == p->end()) return Status::NotFound;
+    *key_len = it->second.size();
+    *first = it->second.front();
+    *last = it->second.back();
+    return Status::Succ;
+}
+int reef_code_object_kernel_meta(const char* co_path, const char* kernel, int out[6]) {
+    std::map<std::string, reef::hal::KernelMeta> meta;
+    std::string err;
+    if (!reef::hal::read_code_object_metadata(co_path, &meta, &err)) return Status::Fail;
+    auto it = meta.find(kernel);
+    if (it == meta.end()) return Status::NotFound;
+    out[0] = it->second.vgprs; out[1] = it->second.agprs; out[2] = it->second.sgprs;
+    out[3] = it->second.lds; out[4] = it->second.scratch; out[5] = it->second.kernarg;
+    return Status::Succ;
+}
+
+}  // extern "C"

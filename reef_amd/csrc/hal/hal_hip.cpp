@@ -1,0 +1,307 @@
+// HIP backend of the C-ABI layer (stock ROCm, no patched runtime).
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+#include <deque>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "hal/code_object.h"
+#include "reef_hal.h"
+
+struct reef_module_s {
+    hipModule_t mod;
+    std::map<std::string, reef::hal::KernelMeta> meta;
+    std::vector<reef_function_s*> fns;
+};
+struct reef_function_s {
+    hipFunction_t fn;
+    reef::hal::KernelMeta meta;
+    bool has_meta;
+    std::string name;
+};
+
+namespace {
+
+struct Held {
+    hipFunction_t fn;
+    uint32_t grid[3], block[3], lds;
+    std::vector<char> kernarg;
+};
+
+}  // namespace
+
+// A stream with an optional launch window.  `done` is a pinned host word the
+// device writes after every kernel of a windowed stream; submitted - *done is
+// the number of kernels still on the device.
+struct reef_stream_s {
+    hipStream_t s;
+    int window;
+    uint32_t submitted;
+    volatile uint32_t* done;
+    std::deque<Held> held;
+};
+
+namespace {
+
+int fail(hipError_t e, const char* what) {
+    std::string m = std::string(what) + ": " + hipGetErrorString(e);
+    reef_hal_set_error(m.c_str());
+    return 1;
+}
+#define HIPCHK(call)                          \
+    do {                                      \
+        hipError_t _e = (call);               \
+        if (_e != hipSuccess) return fail(_e, #call); \
+    } while (0)
+
+int g_device = 0;
+
+int h_init(int device) {
+    HIPCHK(hipInit(0));
+    int n = 0;
+    HIPCHK(hipGetDeviceCount(&n));
+    if (device < 0 || device >= n) {
+        reef_hal_set_error("reef_hal_init: no such device");
+        return 1;
+    }
+    g_device = device;
+    HIPCHK(hipSetDevice(device));
+    return 0;
+}
+
+int h_device_info(reef_device_info* out) {
+    if (!out) return 1;
+    std::memset(out, 0, sizeof(*out));
+    hipDeviceProp_t p;
+    HIPCHK(hipGetDeviceProperties(&p, g_device));
+    out->num_cus = p.multiProcessorCount;
+    out->num_xcds = 8;
+    if (out->num_cus % out->num_xcds != 0) out->num_xcds = 1;
+    out->simds_per_cu = 4;
+    out->max_waves_per_simd = 8;
+    out->vgprs_per_simd = 512;
+    out->vgpr_granule = 8;
+    out->lds_bytes_per_cu = 160 * 1024;
+    out->lds_granule = 1280;
+    out->max_wg_per_cu = 32;
+    out->clock_khz = p.clockRate;
+    std::strncpy(out->arch, p.gcnArchName, sizeof(out->arch) - 1);
+    if (char* c = std::strchr(out->arch, ':')) *c = 0;
+    return 0;
+}
+
+int h_module_load(const char* path, reef_module_t* out) {
+    reef_module_s* m = new reef_module_s;
+    hipError_t e = hipModuleLoad(&m->mod, path);
+    if (e != hipSuccess) {
+        delete m;
+        return fail(e, (std::string("hipModuleLoad ") + path).c_str());
+    }
+    std::string err;
+    if (!reef::hal::read_code_object_metadata(path, &m->meta, &err)) m->meta.clear();
+    *out = m;
+    return 0;
+}
+
+int h_module_unload(reef_module_t m) {
+    if (!m) return 0;
+    hipError_t e = hipModuleUnload(m->mod);
+    for (auto* f : m->fns) delete f;
+    delete m;
+    return e == hipSuccess ? 0 : fail(e, "hipModuleUnload");
+}
+
+int h_module_get_function(reef_module_t m, const char* name, reef_function_t* out) {
+    hipFunction_t fn;
+    hipError_t e = hipModuleGetFunction(&fn, m->mod, name);
+    if (e != hipSuccess) return fail(e, (std::string("hipModuleGetFunction ") + name).c_str());
+    reef_function_s* f = new reef_function_s;
+    f->fn = fn;
+    f->name = name;
+    auto it = m->meta.find(name);
+    f->has_meta = it != m->meta.end();
+    if (f->has_meta) f->meta = it->second;
+    m->fns.push_back(f);
+    *out = f;
+    return 0;
+}
+
+int h_function_resource(reef_function_t f, reef_kernel_resource* out) {
+    if (!f->has_meta) {
+        reef_hal_set_error(("no metadata for kernel " + f->name).c_str());
+        return 1;
+    }
+    out->shared_memory = f->meta.lds;
+    out->vgprs = (f->meta.vgprs + 3) / 4 * 4 + f->meta.agprs;
+    out->sgprs = f->meta.sgprs;
+    out->stack_size = f->meta.scratch;
+    return 0;
+}
+
+int h_malloc(size_t bytes, int kind, reef_devptr_t* out) {
+    if (bytes == 0) bytes = 4;
+    switch (kind) {
+        case REEF_MEM_DEVICE: HIPCHK(hipMalloc(out, bytes)); break;
+        case REEF_MEM_DEVICE_FINEGRAINED:
+            HIPCHK(hipExtMallocWithFlags(out, bytes, hipDeviceMallocFinegrained));
+            break;
+        case REEF_MEM_HOST_PINNED: HIPCHK(hipHostMalloc(out, bytes, hipHostMallocDefault)); break;
+        default: reef_hal_set_error("reef_hal_malloc: bad kind"); return 1;
+    }
+    return 0;
+}
+int h_free(reef_devptr_t p, int kind) {
+    if (kind == REEF_MEM_HOST_PINNED) HIPCHK(hipHostFree(p));
+    else HIPCHK(hipFree(p));
+    return 0;
+}
+int h_memset(reef_devptr_t p, int byte, size_t n) { HIPCHK(hipMemset(p, byte, n)); return 0; }
+int h_h2d(reef_devptr_t d, const void* s, size_t n) { HIPCHK(hipMemcpy(d, s, n, hipMemcpyHostToDevice)); return 0; }
+int h_d2h(void* d, reef_devptr_t s, size_t n) { HIPCHK(hipMemcpy(d, s, n, hipMemcpyDeviceToHost)); return 0; }
+int h_h2d_async(reef_devptr_t d, const void* s, size_t n, reef_stream_t st) {
+    HIPCHK(hipMemcpyAsync(d, s, n, hipMemcpyHostToDevice, st ? st->s : nullptr));
+    return 0;
+}
+int h_d2h_async(void* d, reef_devptr_t s, size_t n, reef_stream_t st) {
+    HIPCHK(hipMemcpyAsync(d, s, n, hipMemcpyDeviceToHost, st ? st->s : nullptr));
+    return 0;
+}
+
+int h_stream_create(int window, reef_stream_t* out) {
+    reef_stream_s* st = new reef_stream_s;
+    st->window = window;
+    st->submitted = 0;
+    st->done = nullptr;
+    hipError_t e = hipStreamCreateWithFlags(&st->s, hipStreamNonBlocking);
+    if (e != hipSuccess) { delete st; return fail(e, "hipStreamCreateWithFlags"); }
+    if (window > 0) {
+        void* p = nullptr;
+        e = hipHostMalloc(&p, 64, hipHostMallocDefault);
+        if (e != hipSuccess) { hipStreamDestroy(st->s); delete st; return fail(e, "hipHostMalloc"); }
+        st->done = (volatile uint32_t*)p;
+        *st->done = 0;
+    }
+    *out = st;
+    return 0;
+}
+int h_stream_destroy(reef_stream_t st) {
+    if (!st) return 0;
+    hipStreamSynchronize(st->s);
+    hipStreamDestroy(st->s);
+    if (st->done) hipHostFree((void*)st->done);
+    delete st;
+    return 0;
+}
+
+int submit(reef_stream_t st, hipFunction_t fn, const uint32_t* g, const uint32_t* b, uint32_t lds,
+           const void* kernarg, size_t bytes) {
+    size_t sz = bytes;
+    void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(kernarg),
+                     HIP_LAUNCH_PARAM_BUFFER_SIZE, &sz, HIP_LAUNCH_PARAM_END};
+    HIPCHK(hipModuleLaunchKernel(fn, g[0], g[1], g[2], b[0], b[1], b[2], lds, st ? st->s : nullptr,
+                                 nullptr, extra));
+    if (st && st->window > 0) {
+        ++st->submitted;
+        HIPCHK(hipStreamWriteValue32(st->s, (void*)st->done, st->submitted, 0));
+    }
+    return 0;
+}
+
+inline uint32_t in_flight(reef_stream_t st) { return st->submitted - *st->done; }
+
+int h_stream_pump(reef_stream_t st) {
+    if (!st || st->window <= 0) return 0;
+    while (!st->held.empty() && (int)in_flight(st) < st->window) {
+        Held& h = st->held.front();
+        int rc = submit(st, h.fn, h.grid, h.block, h.lds, h.kernarg.data(), h.kernarg.size());
+        st->held.pop_front();
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+int h_launch(reef_function_t f, const uint32_t* g, const uint32_t* b, uint32_t lds, reef_stream_t st,
+             const void* kernarg, size_t bytes) {
+    if (st && st->window > 0) {
+        if (int rc = h_stream_pump(st)) return rc;
+        if (!st->held.empty() || (int)in_flight(st) >= st->window) {
+            Held h;
+            h.fn = f->fn;
+            std::memcpy(h.grid, g, sizeof(h.grid));
+            std::memcpy(h.block, b, sizeof(h.block));
+            h.lds = lds;
+            h.kernarg.assign((const char*)kernarg, (const char*)kernarg + bytes);
+            st->held.push_back(std::move(h));
+            return 0;
+        }
+    }
+    return submit(st, f->fn, g, b, lds, kernarg, bytes);
+}
+
+int h_stream_sync(reef_stream_t st) {
+    if (st && st->window > 0) {
+        while (!st->held.empty()) {
+            if (int rc = h_stream_pump(st)) return rc;
+        }
+    }
+    HIPCHK(hipStreamSynchronize(st ? st->s : nullptr));
+    return 0;
+}
+int h_stream_query(reef_stream_t st, int* idle) {
+    if (st && st->window > 0) {
+        if (int rc = h_stream_pump(st)) return rc;
+        if (!st->held.empty()) { *idle = 0; return 0; }
+    }
+    hipError_t e = hipStreamQuery(st ? st->s : nullptr);
+    if (e == hipSuccess) *idle = 1;
+    else if (e == hipErrorNotReady) *idle = 0;
+    else return fail(e, "hipStreamQuery");
+    return 0;
+}
+int h_device_sync() { HIPCHK(hipDeviceSynchronize()); return 0; }
+
+int h_write_value32(reef_stream_t st, reef_devptr_t p, int32_t v) {
+    HIPCHK(hipStreamWriteValue32(st ? st->s : nullptr, p, (uint32_t)v, 0));
+    return 0;
+}
+int h_clear_queue(reef_stream_t st, uint64_t* n) {
+    uint64_t d = 0;
+    if (st) { d = st->held.size(); st->held.clear(); }
+    if (n) *n = d;
+    return 0;
+}
+int h_reset_cus() { return 0; }
+
+int h_event_create(reef_event_t* out) {
+    hipEvent_t e;
+    HIPCHK(hipEventCreate(&e));
+    *out = (reef_event_t)e;
+    return 0;
+}
+int h_event_destroy(reef_event_t e) { HIPCHK(hipEventDestroy((hipEvent_t)e)); return 0; }
+int h_event_record(reef_event_t e, reef_stream_t st) {
+    HIPCHK(hipEventRecord((hipEvent_t)e, st ? st->s : nullptr));
+    return 0;
+}
+int h_event_sync(reef_event_t e) { HIPCHK(hipEventSynchronize((hipEvent_t)e)); return 0; }
+int h_event_elapsed_us(reef_event_t a, reef_event_t b, float* us) {
+    float ms = 0.f;
+    HIPCHK(hipEventElapsedTime(&ms, (hipEvent_t)a, (hipEvent_t)b));
+    *us = ms * 1000.0f;
+    return 0;
+}
+
+const reef_hal_backend kHip = {
+    h_init, h_device_info, h_module_load, h_module_unload, h_module_get_function,
+    h_function_resource, h_malloc, h_free, h_memset, h_h2d, h_d2h, h_h2d_async, h_d2h_async,
+    h_stream_create, h_stream_destroy, h_stream_sync, h_stream_query, h_device_sync, h_stream_pump,
+    h_launch, h_write_value32, h_clear_queue, h_reset_cus,
+    h_event_create, h_event_destroy, h_event_record, h_event_sync, h_event_elapsed_us,
+};
+
+}  // namespace
+
+extern "C" const reef_hal_backend* reef_hal_hip_backend(void) { return &kHip; }

@@ -1,0 +1,309 @@
+// Bandwidth-bound kernels: split-K reduce, depthwise conv, pooling, elementwise,
+// GEMV, softmax, LayerNorm, GELU, embedding, copy, transpose, and the
+// reference's mocked add/multiply.  No matrix cores: coalesced 128-bit accesses
+// where the layout allows, one wavefront per row for the reductions.
+//
+// Reference kernels these replace (generated code, shapes baked in):
+//   pooling            resource/resnet152/resnet152.cu:365-374, 4390-4403
+//   elementwise add    resource/resnet152/resnet152.cu:771-773, 4056-4066, 4782-4784
+//   dense (GEMV)       resource/resnet152/resnet152.cu:2-33
+//   softmax            resource/resnet152/resnet152.cu:775-841; resource/bert/bert.cu:3-13,159-166
+//   LayerNorm (5 kernels there, one here)   resource/bert/bert.cu:175-205, 338-380
+//   bias + erf GELU    resource/bert/bert.cu:167-173
+//   embedding gather   resource/bert/bert.cu:14-21
+//   movers             resource/bert/bert.cu:273-326, 344-351, 381-388
+//   depthwise conv     resource/mobilenet/mobilenet.cu (fused_nn_conv2d_add_nn_relu_17_kernel0)
+//   mocked add/multiply  resource/mocked_kernel/mocked_kernel.cu:9-27
+#pragma once
+#include <float.h>
+
+#include "reef_common.hpp"
+
+namespace reef_dev {
+
+// out = act(sum_{s ascending} ws[s] (+res)(+bias)(*scale+shift)); 4 elements per thread.
+__device__ __forceinline__ void splitk_reduce_body(const ReefOpDesc& d, int task) {
+    const int* a = d.attr;
+    const int M = a[REEF_RED_M], N = a[REEF_RED_N], S = a[REEF_RED_SPLIT_K];
+    const size_t MN = (size_t)M * N;
+    const float* ws = (const float*)d.ptr[0];
+    float* out = (float*)d.ptr[1];
+    Epilogue ep;
+    ep.unpack(d, 2, a[REEF_RED_FLAGS], a[REEF_RED_ACT]);
+    const size_t i0 = ((size_t)task * kThreads + threadIdx.x) * 4;
+    if (i0 >= MN) return;
+    if ((MN & 3) == 0) {
+        f32x4 acc = *(const f32x4*)(ws + i0);
+        for (int s = 1; s < S; ++s) acc += *(const f32x4*)(ws + (size_t)s * MN + i0);
+        f32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = ep.apply(acc[e], (int)((i0 + e) / N), i0 + e);
+        *(f32x4*)(out + i0) = o;
+    } else {
+        for (int e = 0; e < 4 && i0 + e < MN; ++e) {
+            float acc = ws[i0 + e];
+            for (int s = 1; s < S; ++s) acc += ws[(size_t)s * MN + i0 + e];
+            out[i0 + e] = ep.apply(acc, (int)((i0 + e) / N), i0 + e);
+        }
+    }
+}
+
+__device__ __forceinline__ void dwconv2d_body(const ReefOpDesc& d, int task) {
+    const int* a = d.attr;
+    const int C = a[REEF_DW_C], H = a[REEF_DW_H], W = a[REEF_DW_W], Ho = a[REEF_DW_HO],
+              Wo = a[REEF_DW_WO], kh = a[REEF_DW_KH], kw = a[REEF_DW_KW], sh = a[REEF_DW_SH],
+              sw = a[REEF_DW_SW], ph = a[REEF_DW_PH], pw = a[REEF_DW_PW];
+    const int idx = task * kThreads + threadIdx.x;
+    if (idx >= C * Ho * Wo) return;
+    const int c = idx / (Ho * Wo);
+    const int r = idx - c * Ho * Wo;
+    const int y = r / Wo, x = r - y * Wo;
+    const float* in = (const float*)d.ptr[0] + (size_t)c * H * W;
+    const float* w = (const float*)d.ptr[1] + (size_t)c * kh * kw;
+    float acc = 0.0f;
+    for (int ky = 0; ky < kh; ++ky) {
+        const int iy = y * sh + ky - ph;
+        if ((unsigned)iy >= (unsigned)H) continue;
+        for (int kx = 0; kx < kw; ++kx) {
+            const int ix = x * sw + kx - pw;
+            if ((unsigned)ix < (unsigned)W) acc = fmaf(in[iy * W + ix], w[ky * kw + kx], acc);
+        }
+    }
+    if (a[REEF_DW_FLAGS] & 1) acc += ((const float*)d.ptr[3])[c];
+    ((float*)d.ptr[2])[idx] = act_apply(acc, a[REEF_DW_ACT]);
+}
+
+__device__ __forceinline__ void pool2d_body(const ReefOpDesc& d, int task) {
+    const int* a = d.attr;
+    const int C = a[REEF_POOL_C], H = a[REEF_POOL_H], W = a[REEF_POOL_W], Ho = a[REEF_POOL_HO],
+              Wo = a[REEF_POOL_WO], kh = a[REEF_POOL_KH], kw = a[REEF_POOL_KW],
+              sh = a[REEF_POOL_SH], sw = a[REEF_POOL_SW], ph = a[REEF_POOL_PH],
+              pw = a[REEF_POOL_PW], mode = a[REEF_POOL_MODE];
+    const int idx = task * kThreads + threadIdx.x;
+    if (idx >= C * Ho * Wo) return;
+    const int c = idx / (Ho * Wo);
+    const int r = idx - c * Ho * Wo;
+    const int y = r / Wo, x = r - y * Wo;
+    const float* in = (const float*)d.ptr[0] + (size_t)c * H * W;
+    float m = -FLT_MAX, s = 0.0f;
+    int cnt = 0;
+    for (int dy = 0; dy < kh; ++dy) {
+        const int iy = y * sh + dy - ph;
+        if ((unsigned)iy >= (unsigned)H) continue;
+        for (int dx = 0; dx < kw; ++dx) {
+            const int ix = x * sw + dx - pw;
+            if ((unsigned)ix >= (unsigned)W) continue;
+            const float v = in[iy * W + ix];
+            m = fmaxf(m, v);
+            s += v;
+            ++cnt;
+        }
+    }
+    float v;
+    if (mode == 0) v = m;
+    else v = s / (float)(a[REEF_POOL_COUNT_PAD] ? kh * kw : (cnt > 0 ? cnt : 1));
+    if (a[REEF_POOL_FLAGS] & 1) v += ((const float*)d.ptr[2])[c];
+    ((float*)d.ptr[1])[idx] = act_apply(v, a[REEF_POOL_ACT]);
+}
+
+// one wavefront per channel
+__device__ __forceinline__ void global_avgpool_body(const ReefOpDesc& d, int task) {
+    const int C = d.attr[REEF_GAP_C], HW = d.attr[REEF_GAP_HW];
+    const int c = task * 4 + (threadIdx.x >> 6);
+    if (c >= C) return;
+    const float* in = (const float*)d.ptr[0] + (size_t)c * HW;
+    float s = 0.0f;
+    for (int i = threadIdx.x & 63; i < HW; i += 64) s += in[i];
+    s = wave_sum(s);
+    if ((threadIdx.x & 63) == 0) ((float*)d.ptr[1])[c] = s * (1.0f / (float)HW);
+}
+
+__device__ __forceinline__ void eltwise_body(const ReefOpDesc& d, int task) {
+    const int* at = d.attr;
+    const int C = at[REEF_ELT_C], inner = at[REEF_ELT_INNER], flags = at[REEF_ELT_FLAGS],
+              act = at[REEF_ELT_ACT];
+    const float* a = (const float*)d.ptr[0];
+    float* out = (float*)d.ptr[1];
+    int p = 2;
+    const float* b = (flags & REEF_ELT_F_B) ? (const float*)d.ptr[p++] : nullptr;
+    const float* scale = (flags & REEF_ELT_F_SCALE) ? (const float*)d.ptr[p++] : nullptr;
+    const float* shift = (flags & REEF_ELT_F_SHIFT) ? (const float*)d.ptr[p++] : nullptr;
+    const size_t total = (size_t)C * inner;
+    const size_t i0 = ((size_t)task * kThreads + threadIdx.x) * 4;
+    if (i0 >= total) return;
+    if ((inner & 3) == 0) {
+        const int c = (int)(i0 / inner);
+        f32x4 v = *(const f32x4*)(a + i0);
+        if (b) v += *(const f32x4*)(b + i0);
+        if (scale) v *= scale[c];
+        if (shift) v += shift[c];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = act_apply(v[e], act);
+        *(f32x4*)(out + i0) = v;
+    } else {
+        for (int e = 0; e < 4 && i0 + e < total; ++e) {
+            const int c = (int)((i0 + e) / inner);
+            float v = a[i0 + e];
+            if (b) v += b[i0 + e];
+            if (scale) v *= scale[c];
+            if (shift) v += shift[c];
+            out[i0 + e] = act_apply(v, act);
+        }
+    }
+}
+
+// GEMV: one wavefront per output neuron, 128-bit loads along k.
+__device__ __forceinline__ void dense_body(const ReefOpDesc& d, int task) {
+    const int* a = d.attr;
+    const int rows = a[REEF_DENSE_ROWS], in_f = a[REEF_DENSE_IN], out_f = a[REEF_DENSE_OUT],
+              act = a[REEF_DENSE_ACT];
+    const int o = task * 4 + (threadIdx.x >> 6);
+    if (o >= out_f) return;
+    const int lane = threadIdx.x & 63;
+    const float* w = (const float*)d.ptr[1] + (size_t)o * in_f;
+    const float bias = (a[REEF_DENSE_FLAGS] & 1) ? ((const float*)d.ptr[3])[o] : 0.0f;
+    for (int r = 0; r < rows; ++r) {
+        const float* x = (const float*)d.ptr[0] + (size_t)r * in_f;
+        float s = 0.0f;
+        if ((in_f & 3) == 0) {
+            for (int k = lane * 4; k < in_f; k += 256) {
+                const f32x4 xv = *(const f32x4*)(x + k), wv = *(const f32x4*)(w + k);
+                s = fmaf(xv.x, wv.x, s);
+                s = fmaf(xv.y, wv.y, s);
+                s = fmaf(xv.z, wv.z, s);
+                s = fmaf(xv.w, wv.w, s);
+            }
+        } else {
+            for (int k = lane; k < in_f; k += 64) s = fmaf(x[k], w[k], s);
+        }
+        s = wave_sum(s);
+        if (lane == 0) {
+            float v = s + bias;
+            if (act == REEF_ACT_RELU) v = fmaxf(v, 0.0f);
+            else if (act == REEF_ACT_GELU) v = gelu_erf(v);
+            ((float*)d.ptr[2])[(size_t)r * out_f + o] = v;
+        }
+    }
+}
+
+// one wavefront per row: max, exp, sum, divide
+__device__ __forceinline__ void softmax_body(const ReefOpDesc& d, int task) {
+    const int rows = d.attr[REEF_SM_ROWS], cols = d.attr[REEF_SM_COLS];
+    const int r = task * 4 + (threadIdx.x >> 6);
+    if (r >= rows) return;
+    const int lane = threadIdx.x & 63;
+    const float* x = (const float*)d.ptr[0] + (size_t)r * cols;
+    float* y = (float*)d.ptr[1] + (size_t)r * cols;
+    float m = -FLT_MAX;
+    for (int i = lane; i < cols; i += 64) m = fmaxf(m, x[i]);
+    m = wave_max(m);
+    float s = 0.0f;
+    for (int i = lane; i < cols; i += 64) s += expf(x[i] - m);
+    s = wave_sum(s);
+    for (int i = lane; i < cols; i += 64) y[i] = expf(x[i] - m) / s;
+}
+
+// one wavefront per row; two-pass mean / variance as the reference splits it
+__device__ __forceinline__ void layernorm_body(const ReefOpDesc& d, int task) {
+    const int rows = d.attr[REEF_LN_ROWS], cols = d.attr[REEF_LN_COLS];
+    const int r = task * 4 + (threadIdx.x >> 6);
+    if (r >= rows) return;
+    const int lane = threadIdx.x & 63;
+    const float eps = __int_as_float(d.attr[REEF_LN_EPS_BITS]);
+    const float* x = (const float*)d.ptr[0] + (size_t)r * cols;
+    const float* gamma = (const float*)d.ptr[1];
+    const float* beta = (const float*)d.ptr[2];
+    float* y = (float*)d.ptr[3] + (size_t)r * cols;
+    const float* res = (d.attr[REEF_LN_FLAGS] & 1) ? (const float*)d.ptr[4] + (size_t)r * cols : nullptr;
+    float s = 0.0f;
+    for (int i = lane; i < cols; i += 64) s += res ? x[i] + res[i] : x[i];
+    const float mean = wave_sum(s) / (float)cols;
+    float v = 0.0f;
+    for (int i = lane; i < cols; i += 64) {
+        const float dlt = (res ? x[i] + res[i] : x[i]) - mean;
+        v = fmaf(dlt, dlt, v);
+    }
+    const float inv = 1.0f / sqrtf(wave_sum(v) / (float)cols + eps);
+    for (int i = lane; i < cols; i += 64) {
+        const float dlt = (res ? x[i] + res[i] : x[i]) - mean;
+        y[i] = dlt * inv * gamma[i] + beta[i];
+    }
+}
+
+__device__ __forceinline__ void bias_gelu_body(const ReefOpDesc& d, int task) {
+    const int rows = d.attr[REEF_GELU_ROWS], cols = d.attr[REEF_GELU_COLS];
+    const float* x = (const float*)d.ptr[0];
+    float* y = (float*)d.ptr[1];
+    const float* bias = (d.attr[REEF_GELU_FLAGS] & 1) ? (const float*)d.ptr[2] : nullptr;
+    const size_t total = (size_t)rows * cols;
+    const size_t i0 = ((size_t)task * kThreads + threadIdx.x) * 4;
+    for (int e = 0; e < 4 && i0 + e < total; ++e) {
+        const int c = (int)((i0 + e) % cols);
+        y[i0 + e] = gelu_erf(x[i0 + e] + (bias ? bias[c] : 0.0f));
+    }
+}
+
+__device__ __forceinline__ void embedding_body(const ReefOpDesc& d, int task) {
+    const int seq = d.attr[REEF_EMB_SEQ], hidden = d.attr[REEF_EMB_HIDDEN],
+              flags = d.attr[REEF_EMB_FLAGS];
+    const long long* ids = (const long long*)d.ptr[0];
+    const float* tok = (const float*)d.ptr[1];
+    float* out = (float*)d.ptr[2];
+    int p = 3;
+    const float* pos = (flags & 1) ? (const float*)d.ptr[p++] : nullptr;
+    const float* seg = (flags & 2) ? (const float*)d.ptr[p++] : nullptr;
+    const size_t total = (size_t)seq * hidden;
+    const size_t i0 = ((size_t)task * kThreads + threadIdx.x) * 4;
+    for (int e = 0; e < 4 && i0 + e < total; ++e) {
+        const int s = (int)((i0 + e) / hidden), h = (int)((i0 + e) - (size_t)s * hidden);
+        float v = tok[(size_t)ids[s] * hidden + h];
+        if (pos) v += pos[i0 + e];
+        if (seg) v += seg[h];
+        out[i0 + e] = v;
+    }
+}
+
+__device__ __forceinline__ void copy_body(const ReefOpDesc& d, int task) {
+    const int count = d.attr[REEF_COPY_COUNT], dst_off = d.attr[REEF_COPY_DST_OFF];
+    const float* in = (const float*)d.ptr[0];
+    float* out = (float*)d.ptr[1] + dst_off;
+    const int i0 = (task * kThreads + threadIdx.x) * 4;
+    if (i0 >= count) return;
+    if (((count | dst_off) & 3) == 0) {
+        *(f32x4*)(out + i0) = *(const f32x4*)(in + i0);
+    } else {
+        for (int e = 0; e < 4 && i0 + e < count; ++e) out[i0 + e] = in[i0 + e];
+    }
+}
+
+// in [d0][d1][d2] -> out [d1][d0][d2] (+ bias[d1][d2])
+__device__ __forceinline__ void transpose_body(const ReefOpDesc& d, int task) {
+    const int d0 = d.attr[REEF_TR_D0], d1 = d.attr[REEF_TR_D1], d2 = d.attr[REEF_TR_D2];
+    const float* in = (const float*)d.ptr[0];
+    float* out = (float*)d.ptr[1];
+    const float* bias = (d.attr[REEF_TR_FLAGS] & 1) ? (const float*)d.ptr[2] : nullptr;
+    const size_t total = (size_t)d0 * d1 * d2;
+    const size_t i0 = ((size_t)task * kThreads + threadIdx.x) * 4;
+    for (int e = 0; e < 4 && i0 + e < total; ++e) {
+        const size_t i = i0 + e;  // output index (b, a, c)
+        const int c = (int)(i % d2);
+        const int a = (int)((i / d2) % d0);
+        const int b = (int)(i / ((size_t)d2 * d0));
+        float v = in[((size_t)a * d1 + b) * d2 + c];
+        if (bias) v += bias[(size_t)b * d2 + c];
+        out[i] = v;
+    }
+}
+
+// The reference's mocked model: logical block = task, 128 logical threads;
+// out[task*128 + t] = a[t] (+|*) b[task*128 + t]   (mocked_kernel.cu:9-27)
+template <bool MUL>
+__device__ __forceinline__ void mocked_body(const ReefOpDesc& d, int task, int t) {
+    const float* a = (const float*)d.ptr[0];
+    const float* b = (const float*)d.ptr[1];
+    float* out = (float*)d.ptr[2];
+    const int i = task * 128 + t;
+    out[i] = MUL ? a[t] * b[i] : a[t] + b[i];
+}
+
+}  // namespace reef_dev

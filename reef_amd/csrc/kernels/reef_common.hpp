@@ -1,0 +1,87 @@
+// Shared device helpers for the gfx950 REEF kernels: preemption polling
+// policies, wavefront reductions, optional-operand unpacking.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "reef_kernels.h"
+
+namespace reef_dev {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int kWave = 64;
+constexpr int kThreads = REEF_WG_THREADS;
+
+// ---- preemption polling -------------------------------------------------
+// The reference's best-effort wrapper reads *preempted once at block start
+// (script/best_effort_kernel.py:22-29) and relies on a patched driver to kill
+// running wavefronts (src/reef/server/scheduler.cpp:331-333).  Stock ROCm has
+// no such call, so long-running bodies re-read the flag inside their main loop
+// and the whole workgroup leaves together.  The flag lives in memory the host
+// can write while kernels run; it is read with a system-scope relaxed atomic so
+// the load is not served from a stale cache line.
+struct NoPoll {
+    static constexpr bool enabled = false;
+    __device__ __forceinline__ int load() const { return 0; }
+};
+struct FlagPoll {
+    static constexpr bool enabled = true;
+    const int* flag;
+    __device__ __forceinline__ int load() const {
+        return __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+__device__ __forceinline__ float act_apply(float v, int act) {
+    if (act == REEF_ACT_RELU) return fmaxf(v, 0.0f);
+    if (act == REEF_ACT_RELU6) return fminf(fmaxf(v, 0.0f), 6.0f);
+    return v;
+}
+
+__device__ __forceinline__ float gelu_erf(float x) {
+    return x * (0.5f + 0.5f * erff(x * 0.70710678f));
+}
+
+// Optional operands of the conv / reduce epilogue follow the fixed pointers in
+// flag-bit order: bias, residual, scale, shift.
+struct Epilogue {
+    const float* bias;
+    const float* residual;
+    const float* scale;
+    const float* shift;
+    int act;
+    __device__ __forceinline__ void unpack(const ReefOpDesc& d, int first, int flags, int act_) {
+        int p = first;
+        bias = (flags & REEF_F_BIAS) ? (const float*)d.ptr[p++] : nullptr;
+        residual = (flags & REEF_F_RESIDUAL) ? (const float*)d.ptr[p++] : nullptr;
+        if (flags & REEF_F_AFFINE) {
+            scale = (const float*)d.ptr[p];
+            shift = (const float*)d.ptr[p + 1];
+        } else {
+            scale = shift = nullptr;
+        }
+        act = act_;
+    }
+    // v = acc; v += residual; v += bias; v = fma(v, scale, shift); act
+    __device__ __forceinline__ float apply(float v, int ch, size_t idx) const {
+        if (residual) v = v + residual[idx];
+        if (bias) v = v + bias[ch];
+        if (scale) v = fmaf(v, scale[ch], shift[ch]);
+        return act_apply(v, act);
+    }
+};
+
+}  // namespace reef_dev

@@ -1,0 +1,387 @@
+"""Graph builder that writes REEF model directories for the gfx950 kernels.
+
+Writes the reference's model resource format (graph JSON + ``.param`` +
+``.profile.json``; reader src/reef/executor/model.cpp:13-156, writers
+script/generate_final_schedule.py:109-144 and script/tvm_generate_model.py:66-76)
+with one added key per kernel, ``attrs`` (the shape attributes the shape-generic
+kernels need, include/reef_kernels.h), plus ``op`` for human readers.  JSON
+values are restricted to ints, strings, lists and dicts, which is all the
+reference's parser accepts (src/reef/util/json.cpp).
+
+Every tensor gets its own storage (no buffer reuse), as the reference forces for
+its own models (script/generate_final_schedule.py:37-40), so a best-effort task
+can be restarted from any kernel after a preemption.
+"""
+import json
+import math
+import os
+import shutil
+import struct
+
+import numpy as np
+
+from . import rng, tiling
+from ..paths import code_object
+
+ACT_NONE, ACT_RELU, ACT_RELU6, ACT_GELU = 0, 1, 2, 3
+F_BIAS, F_RESIDUAL, F_AFFINE = 1, 2, 4
+WG = 256
+
+
+def float_bits(x):
+    return struct.unpack("<i", struct.pack("<f", float(x)))[0]
+
+
+class Tensor:
+    """A storage index plus its logical shape."""
+
+    def __init__(self, idx, shape):
+        self.idx = idx
+        self.shape = tuple(int(s) for s in shape)
+
+    @property
+    def size(self):
+        return int(np.prod(self.shape))
+
+
+class GraphBuilder:
+    def __init__(self, name, seed=rng.BASE_SEED, weight_std=None):
+        self.name = name
+        self.seed = seed
+        self.weight_std = weight_std   # fixed std (BERT: 0.02); None = He-normal
+        self.storage = []
+        self.kernels = []
+        self.graph_args = []
+        self.params = []               # (key, float32 array)
+        self.flops = 0                 # algorithmic FLOPs of contractions
+        self.kernel_flops = []         # per kernel call
+        self.kernel_bytes = []         # algorithmic bytes per kernel call
+        self.kernel_est_us = []
+        self._np = 0
+
+    # ------------------------------------------------------------ storages
+    def _storage(self, name, size, stype="float32"):
+        self.storage.append({"name": name, "size": int(size), "stype": stype})
+        return len(self.storage) - 1
+
+    def input(self, name, shape, stype="float32"):
+        idx = self._storage(name, int(np.prod(shape)), stype)
+        self.graph_args.append(idx)
+        return Tensor(idx, shape)
+
+    def temp(self, shape, name="null"):
+        return Tensor(self._storage(name, int(np.prod(shape))), shape)
+
+    def workspace(self, n_floats):
+        return Tensor(self._storage("temp_arg", int(n_floats) * 4, "byte"), (n_floats,))
+
+    def param(self, shape, std=None, kind="normal", value=None):
+        key = "p%d" % self._np
+        self._np += 1
+        n = int(np.prod(shape))
+        if value is not None:
+            arr = np.full(n, value, np.float32)
+        elif kind == "normal":
+            arr = rng.normal_f32(self.name + "/" + key, n, std, self.seed)
+        else:
+            raise ValueError(kind)
+        idx = self._storage(key, n)
+        self.graph_args.append(idx)
+        self.params.append((key, arr))
+        return Tensor(idx, shape)
+
+    def mark_output(self, t):
+        self.storage[t.idx]["name"] = "output"
+
+    # ------------------------------------------------------------ kernels
+    def _emit(self, name, tasks, args, attrs, op, flops=0, nbytes=0, est_us=1.0, block=(WG, 1, 1)):
+        self.kernels.append({
+            "name": name,
+            "launch_params": [int(tasks), 1, 1, block[0], block[1], block[2]],
+            "args": [int(a) for a in args],
+            "attrs": [int(a) for a in attrs],
+            "op": op,
+        })
+        self.kernel_flops.append(int(flops))
+        self.kernel_bytes.append(int(nbytes))
+        self.kernel_est_us.append(float(est_us))
+
+    def conv2d(self, x, cout, k, stride=1, pad=0, bias=True, act=ACT_RELU, residual=None,
+               affine=False, force=None):
+        """Fused conv + (residual) + (bias) + (scale, shift) + activation on MFMA."""
+        kh, kw = (k, k) if isinstance(k, int) else k
+        sh, sw = (stride, stride) if isinstance(stride, int) else stride
+        ph, pw = (pad, pad) if isinstance(pad, int) else pad
+        cin, H, W = x.shape
+        Ho = (H + 2 * ph - kh) // sh + 1
+        Wo = (W + 2 * pw - kw) // sw + 1
+        M, N, K = cout, Ho * Wo, cin * kh * kw
+        std = self.weight_std if self.weight_std is not None else math.sqrt(2.0 / K)
+        w = self.param((cout, cin, kh, kw), std)
+        flags = 0
+        opt = []
+        if bias:
+            flags |= F_BIAS
+            opt.append(self.param((cout,), 0.01).idx)
+        if residual is not None:
+            flags |= F_RESIDUAL
+            assert residual.shape == (cout, Ho, Wo), (residual.shape, (cout, Ho, Wo))
+            opt.append(residual.idx)
+        if affine:
+            flags |= F_AFFINE
+            opt.append(self.param((cout,), 0.1, value=None).idx)   # scale ~ N(0, 0.1) + 1 below
+            self.params[-1] = (self.params[-1][0], self.params[-1][1] + 1.0)
+            opt.append(self.param((cout,), 0.01).idx)
+        out = self.temp((cout, Ho, Wo))
+        t = force or tiling.choose(M, N, K)
+        flops = 2 * M * N * K
+        self.flops += flops
+        nbytes = 4 * (x.size + M * K + M * N + (M if bias else 0) + (M * N if residual is not None else 0)
+                      + (2 * M if affine else 0))
+        base = [cin, H, W, cout, Ho, Wo, kh, kw, sh, sw, ph, pw]
+        kname = "reef_conv2d_" + t["tile"]
+        if t["split_k"] == 1:
+            attrs = base + [flags, act, t["tile_id"], 1, t["k_chunk"], t["m_tiles"], t["n_tiles"]]
+            self._emit(kname, t["tasks"], [x.idx, w.idx, out.idx] + opt, attrs, "conv2d", flops,
+                       nbytes, t["est_us"])
+        else:
+            ws = self.workspace(t["split_k"] * M * N)
+            attrs = base + [0, ACT_NONE, t["tile_id"], t["split_k"], t["k_chunk"], t["m_tiles"],
+                            t["n_tiles"]]
+            self._emit(kname, t["tasks"], [x.idx, w.idx, ws.idx], attrs, "conv2d", flops,
+                       4 * (x.size + M * K + t["split_k"] * M * N), t["est_us"])
+            self._emit("reef_splitk_reduce", math.ceil(M * N / 1024), [ws.idx, out.idx] + opt,
+                       [M, N, t["split_k"], flags, act], "splitk_reduce", 0,
+                       4 * ((t["split_k"] + 1) * M * N), 2.0)
+        return out
+
+    def dwconv2d(self, x, k, stride=1, pad=0, bias=True, act=ACT_RELU6):
+        C, H, W = x.shape
+        Ho = (H + 2 * pad - k) // stride + 1
+        Wo = (W + 2 * pad - k) // stride + 1
+        std = self.weight_std if self.weight_std is not None else math.sqrt(2.0 / (k * k))
+        w = self.param((C, 1, k, k), std)
+        args = [x.idx, w.idx, None]
+        flags = 0
+        if bias:
+            flags |= 1
+            b = self.param((C,), 0.01)
+        out = self.temp((C, Ho, Wo))
+        args[2] = out.idx
+        if bias:
+            args.append(b.idx)
+        self.flops += 2 * C * Ho * Wo * k * k
+        self._emit("reef_dwconv2d", math.ceil(out.size / WG), args,
+                   [C, H, W, Ho, Wo, k, k, stride, stride, pad, pad, flags, act], "dwconv2d",
+                   2 * C * Ho * Wo * k * k, 4 * (x.size + out.size + C * k * k + C), 2.0)
+        return out
+
+    def pool2d(self, x, k, stride, pad, mode="max", bias=False, act=ACT_NONE, count_include_pad=False,
+               ceil_mode=False):
+        C, H, W = x.shape
+        kh, kw = (k, k) if isinstance(k, int) else k
+        rnd = math.ceil if ceil_mode else math.floor
+        Ho = int(rnd((H + 2 * pad - kh) / stride)) + 1
+        Wo = int(rnd((W + 2 * pad - kw) / stride)) + 1
+        out = self.temp((C, Ho, Wo))
+        args = [x.idx, out.idx]
+        flags = 0
+        if bias:
+            flags = 1
+            args.append(self.param((C,), 0.01).idx)
+        self._emit("reef_pool2d", math.ceil(out.size / WG), args,
+                   [C, H, W, Ho, Wo, kh, kw, stride, stride, pad, pad, 0 if mode == "max" else 1,
+                    1 if count_include_pad else 0, flags, act], "pool2d", 0,
+                   4 * (x.size + out.size), 2.0)
+        return out
+
+    def global_avgpool(self, x):
+        C = x.shape[0]
+        out = self.temp((C,))
+        self._emit("reef_global_avgpool", math.ceil(C / 4), [x.idx, out.idx], [C, x.size // C],
+                   "global_avgpool", 0, 4 * (x.size + C), 2.0)
+        return out
+
+    def eltwise(self, a, b=None, scale=False, shift=False, act=ACT_NONE):
+        C = a.shape[0]
+        inner = a.size // C
+        out = self.temp(a.shape)
+        args = [a.idx, out.idx]
+        flags = 0
+        n_in = 1
+        if b is not None:
+            assert b.size == a.size
+            flags |= 1
+            args.append(b.idx)
+            n_in = 2
+        if scale:
+            flags |= 2
+            p = self.param((C,), 0.1)
+            self.params[-1] = (self.params[-1][0], self.params[-1][1] + 1.0)
+            args.append(p.idx)
+        if shift:
+            flags |= 4
+            args.append(self.param((C,), 0.01 if not isinstance(shift, float) else shift).idx)
+        self._emit("reef_eltwise", math.ceil(a.size / 1024), args, [C, inner, flags, act], "eltwise",
+                   0, 4 * (n_in + 1) * a.size, 2.0)
+        return out
+
+    def dense(self, x, out_f, bias=True, act=ACT_NONE, rows=1):
+        in_f = x.size // rows
+        std = self.weight_std if self.weight_std is not None else math.sqrt(2.0 / in_f)
+        w = self.param((out_f, in_f), std)
+        out = self.temp((rows, out_f))
+        args = [x.idx, w.idx, out.idx]
+        flags = 0
+        if bias:
+            flags = 1
+            args.append(self.param((out_f,), 0.01).idx)
+        self.flops += 2 * rows * in_f * out_f
+        self._emit("reef_dense", math.ceil(out_f / 4), args, [rows, in_f, out_f, flags, act],
+                   "dense", 2 * rows * in_f * out_f, 4 * (x.size + in_f * out_f + rows * out_f), 2.0)
+        return out
+
+    def softmax(self, x, rows, cols):
+        out = self.temp((rows, cols))
+        self._emit("reef_softmax", math.ceil(rows / 4), [x.idx, out.idx], [rows, cols], "softmax", 0,
+                   8 * rows * cols, 2.0)
+        return out
+
+    def layernorm(self, x, rows, cols, res=None, eps=1e-12):
+        gamma = self.param((cols,), 0.1)
+        self.params[-1] = (self.params[-1][0], self.params[-1][1] + 1.0)
+        beta = self.param((cols,), 0.01)
+        out = self.temp((rows, cols))
+        args = [x.idx, gamma.idx, beta.idx, out.idx]
+        flags = 0
+        if res is not None:
+            flags = 1
+            args.append(res.idx)
+        self._emit("reef_layernorm", math.ceil(rows / 4), args, [rows, cols, flags, float_bits(eps)],
+                   "layernorm", 0, 4 * rows * cols * (3 if res is not None else 2), 2.0)
+        return out
+
+    def bias_gelu(self, x, rows, cols, bias=True):
+        out = self.temp((rows, cols))
+        args = [x.idx, out.idx]
+        if bias:
+            args.append(self.param((cols,), 0.01).idx)
+        self._emit("reef_bias_gelu", math.ceil(rows * cols / 1024), args, [rows, cols, 1 if bias else 0],
+                   "bias_gelu", 0, 8 * rows * cols, 2.0)
+        return out
+
+    def embedding(self, ids, vocab, seq, hidden, pos=True, seg=True):
+        tok = self.param((vocab, hidden), self.weight_std or 0.02)
+        out = self.temp((seq, hidden))
+        args = [ids.idx, tok.idx, out.idx]
+        flags = 0
+        if pos:
+            flags |= 1
+            args.append(self.param((seq, hidden), self.weight_std or 0.02).idx)
+        if seg:
+            flags |= 2
+            args.append(self.param((hidden,), self.weight_std or 0.02).idx)
+        self._emit("reef_embedding", math.ceil(seq * hidden / 1024), args, [seq, hidden, flags, vocab],
+                   "embedding", 0, 4 * seq * hidden * 3, 2.0)
+        return out
+
+    def copy_into(self, src, dst, dst_off):
+        self._emit("reef_copy", math.ceil(src.size / 1024), [src.idx, dst.idx], [src.size, dst_off],
+                   "copy", 0, 8 * src.size, 2.0)
+
+    def transpose_102(self, x, d0, d1, d2, bias=None):
+        out = self.temp((d1, d0, d2))
+        args = [x.idx, out.idx]
+        flags = 0
+        if bias is not None:
+            flags = 1
+            args.append(bias.idx)
+        self._emit("reef_transpose", math.ceil(d0 * d1 * d2 / 1024), args, [d0, d1, d2, flags],
+                   "transpose", 0, 8 * d0 * d1 * d2, 2.0)
+        return out
+
+    def gemm(self, a, b, M, N, K, batch=1, trans_b=True, bias=None, act=ACT_NONE, alpha=1.0,
+             lda=None, ldb=None, ldc=None, stride_a=0, stride_b=0, stride_c=0, out=None):
+        """C[b] = act(alpha * A[b] x B[b] (+bias)); operands are storages with explicit strides."""
+        lda = K if lda is None else lda
+        ldb = (K if trans_b else N) if ldb is None else ldb
+        ldc = N if ldc is None else ldc
+        if out is None:
+            out = self.temp((batch, M, N))
+        t = tiling.choose(M, N, K, allow_split=False, tiles=tiling.GEMM_TILES)
+        args = [a.idx, b.idx, out.idx]
+        flags = 0
+        if bias is not None:
+            flags = 1
+            args.append(bias.idx)
+        flops = 2 * batch * M * N * K
+        self.flops += flops
+        self._emit("reef_gemm_" + t["tile"], batch * t["m_tiles"] * t["n_tiles"], args,
+                   [batch, M, N, K, 1 if trans_b else 0, flags, act, float_bits(alpha), t["tile_id"],
+                    t["m_tiles"], t["n_tiles"], lda, ldb, ldc, stride_a, stride_b, stride_c],
+                   "gemm", flops, 4 * batch * (M * K + N * K + M * N), t["est_us"])
+        return out
+
+    def mocked(self, name, a, b, out):
+        self._emit(name, 64, [a.idx, b.idx, out.idx], [], "mocked", 0, 3 * 8192 * 4, 14.0,
+                   block=(4, 8, 4))
+
+    # ------------------------------------------------------------ output
+    def model_dict(self):
+        shared = {}
+        for k in self.kernels:
+            n = k["name"]
+            if n.startswith("reef_conv2d_") or n.startswith("reef_gemm_"):
+                shared[n] = tiling.lds_bytes(n.split("_")[-1])
+            else:
+                shared[n] = 4   # the reference's floor (generate_final_schedule.py:117-143)
+        return {"storage": self.storage, "kernels": self.kernels, "args": self.graph_args,
+                "shared_memory": shared}
+
+    def profile_dict(self, measured_us=None, occupancy_levels=8):
+        """Estimated (or measured) per-kernel latency table, keyed by kernel name as the
+        reference's profile is (model.cpp:57-80).  Kernels sharing a name share one
+        entry; the table keeps the slowest instance, which keeps DKP conservative."""
+        lat = {}
+        total = 0
+        for i, k in enumerate(self.kernels):
+            us = measured_us[i] if measured_us is not None else self.kernel_est_us[i]
+            us = max(1, int(math.ceil(us)))
+            total += us
+            e = lat.setdefault(k["name"], {"total_latency": 0, "latency": [0] * occupancy_levels})
+            e["total_latency"] = max(e["total_latency"], us)
+            e["latency"] = [max(v, us) for v in e["latency"]]
+        return {"model_latency": total, "kernel_latency": lat}
+
+    def write(self, out_dir, link_code_objects=True, measured_us=None):
+        os.makedirs(out_dir, exist_ok=True)
+        base = os.path.join(out_dir, self.name)
+        with open(base + ".json", "w") as f:
+            json.dump(self.model_dict(), f)
+        with open(base + ".profile.json", "w") as f:
+            json.dump(self.profile_dict(measured_us), f, separators=(",", ":"))
+        if self.params:   # the file is optional (src/reef/server/server.cpp:64-68)
+            write_params(base + ".param", self.params)
+        if link_code_objects:
+            for fl in ("raw", "be", "trans"):
+                dst = "%s.%s.co" % (base, fl)
+                if os.path.lexists(dst):
+                    os.remove(dst)
+                shutil.copyfile(code_object(fl), dst)
+        meta = {"flops": self.flops, "kernel_flops": self.kernel_flops,
+                "kernel_bytes": self.kernel_bytes}
+        with open(base + ".meta.json", "w") as f:
+            json.dump(meta, f)
+        return base
+
+
+def write_params(path, params):
+    """``.param`` writer (script/tvm_generate_model.py:66-76)."""
+    with open(path, "wb") as f:
+        f.write(b"TVM_MODEL_PARAMS\0")
+        f.write(struct.pack("<Q", len(params)))
+        for key, arr in params:
+            arr = np.ascontiguousarray(arr, dtype="<f4").reshape(-1)
+            f.write(key.encode("ascii") + b"\0")
+            f.write(struct.pack("<Q", arr.size))
+            f.write(arr.tobytes())

@@ -1,0 +1,71 @@
+"""Tile and split-K choice for the implicit-GEMM convolution / GEMM kernels.
+
+The reference takes grid and block sizes from TVM's tuned schedules
+(script/generate_final_schedule.py:98: launch_params come from the raw
+schedule).  Here the generator picks, per layer, one of the compiled tile
+configurations and a split-K factor from a small analytic cost model of a
+256-CU part: batch-1 layers are tiny (49..3136 output pixels), so most need
+split-K to put a workgroup on every CU.
+"""
+import math
+
+# name -> (id, BM, BN, relative MFMA efficiency of the inner loop, workgroups per CU)
+TILES = {
+    "128x128": (0, 128, 128, 1.00, 2),
+    "128x64": (1, 128, 64, 0.85, 2),
+    "64x64": (2, 64, 64, 0.60, 4),
+    "128x32": (3, 128, 32, 0.60, 3),
+    "32x128": (4, 32, 128, 0.60, 3),
+    "64x128": (5, 64, 128, 0.85, 2),
+}
+GEMM_TILES = ("128x128", "64x64", "32x128")
+
+NUM_CUS = 256
+BK = 32
+# Cost model constants (microseconds); calibrated against measured kernels.
+T_STEP_128x128 = 1.9     # one BK=32 step of a 128x128 tile on one CU at efficiency 1.0
+T_FIXED = 2.0            # prologue + epilogue of a workgroup
+T_REDUCE_LAUNCH = 3.0    # extra launch of the split-K reduce
+HBM_BYTES_PER_US = 4.0e6
+
+
+def _steps_time(bm, bn, eff, steps):
+    return steps * T_STEP_128x128 * (bm * bn) / (128.0 * 128.0) / eff
+
+
+def choose(M, N, K, allow_split=True, tiles=None, max_split=32):
+    """Returns dict(tile, tile_id, BM, BN, split_k, k_chunk, m_tiles, n_tiles, tasks)."""
+    best = None
+    for name in (tiles or TILES.keys()):
+        tid, bm, bn, eff, occ = TILES[name]
+        m_tiles, n_tiles = math.ceil(M / bm), math.ceil(N / bn)
+        nt = m_tiles * n_tiles
+        splits = [1]
+        if allow_split:
+            splits += [s for s in (2, 3, 4, 6, 8, 12, 16, 24, 32) if s <= max_split]
+        for s in splits:
+            k_chunk = math.ceil(math.ceil(K / s) / BK) * BK
+            s_eff = math.ceil(K / k_chunk)
+            if s_eff != s and s != 1:
+                continue
+            wgs = nt * s_eff
+            rounds = math.ceil(wgs / (NUM_CUS * occ))
+            # co-resident workgroups share the CU's matrix pipe
+            share = min(occ, math.ceil(wgs / NUM_CUS))
+            t = rounds * (_steps_time(bm, bn, eff, k_chunk // BK) * share + T_FIXED)
+            if s_eff > 1:
+                t += T_REDUCE_LAUNCH + (s_eff + 1) * M * N * 4 / HBM_BYTES_PER_US
+            cand = (t, name, s_eff, k_chunk, m_tiles, n_tiles)
+            if best is None or cand[0] < best[0] - 1e-9:
+                best = cand
+    t, name, s, k_chunk, m_tiles, n_tiles = best
+    tid, bm, bn, _, _ = TILES[name]
+    return dict(tile=name, tile_id=tid, BM=bm, BN=bn, split_k=s, k_chunk=k_chunk,
+                m_tiles=m_tiles, n_tiles=n_tiles, tasks=s * m_tiles * n_tiles, est_us=t)
+
+
+def lds_bytes(tile):
+    _, bm, bn, _, _ = TILES[tile]
+    a = bm * 36
+    b = max(32 * bn, bn * 36)
+    return 2 * (a + b) * 4 + 16

@@ -1,0 +1,119 @@
+"""End-to-end and per-layer parity of whole models against the CPU oracle,
+through all three kernel flavours (raw / DKP single-sided / preemptible), and
+the bit-identity guarantees between flavours."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from reef_amd import binding as B
+from reef_amd.modelgen import nets
+from tests.helpers import compare_storages, max_rel_err, write_model, REL_TOL
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def resnet18_dir(tmp_path_factory):
+    g = nets.resnet(18)
+    return g, write_model(g, tmp_path_factory.mktemp("r18"))
+
+
+@pytest.fixture(scope="module")
+def resnet18_oracle(resnet18_dir):
+    g, d = resnet18_dir
+    model = json.load(open(os.path.join(d, g.name + ".json")))
+    orc = O.GraphOracle(model, os.path.join(d, g.name + ".param"))
+    x = nets.image_input("resnet18", (3, 224, 224))
+    orc.set_input("data", x)
+    orc.run()
+    return model, orc, x
+
+
+@pytest.mark.parametrize("kind,preemptible", [(B.BASE, False), (B.TRANS, False), (B.HYBRID, False),
+                                              (B.HYBRID, True)])
+def test_resnet18_per_layer(resnet18_dir, resnet18_oracle, kind, preemptible):
+    """ResNet-18, 3x224x224 (the reference's CPU-runnable configuration): every
+    intermediate tensor within 1e-4 of the oracle, in every flavour."""
+    g, d = resnet18_dir
+    model, orc, x = resnet18_oracle
+    exe = B.Executor.from_dir(d, g.name, kind)
+    exe.set_input_checked("data", x)
+    if preemptible:
+        exe.execute_preemptable()
+    else:
+        exe.execute()
+    worst = compare_storages(exe, orc, model, what="resnet18 kind=%d" % kind)
+    out = exe.get_output()
+    assert out.shape == (1000,) and abs(out.sum() - 1.0) < 1e-4
+    print("worst rel err %.2e at storage %s" % worst)
+
+
+def test_flavours_bit_identical(resnet18_dir, resnet18_oracle):
+    """raw, DKP and preemptible flavours run the same arithmetic per task: outputs
+    must be bit-identical (the DKP co-run == solo guarantee starts here)."""
+    g, d = resnet18_dir
+    _, _, x = resnet18_oracle
+    outs = []
+    last = []
+    for kind, pre in ((B.BASE, False), (B.TRANS, False), (B.HYBRID, True)):
+        exe = B.Executor.from_dir(d, g.name, kind)
+        exe.set_input_checked("data", x)
+        exe.execute_preemptable() if pre else exe.execute()
+        outs.append(exe.get_output())
+        # logits (input of the softmax) are a more sensitive probe than the softmax output
+        model = exe  # keep alive
+        last.append(exe.get_data(json.load(open(os.path.join(d, g.name + ".json")))["kernels"][-1]["args"][0], 1000))
+    for o, l in zip(outs[1:], last[1:]):
+        np.testing.assert_array_equal(o, outs[0])
+        np.testing.assert_array_equal(l, last[0])
+
+
+def test_resnet152_end_to_end(tmp_path):
+    """ResNet-152 at the benchmark shape: per-layer and end-to-end parity."""
+    g = nets.resnet(152)
+    d = write_model(g, tmp_path)
+    model = json.load(open(os.path.join(d, g.name + ".json")))
+    x = nets.image_input("resnet152", (3, 224, 224))
+    exe = B.Executor.from_dir(d, g.name, B.HYBRID)
+    exe.set_input_checked("data", x)
+    exe.execute()
+    orc = O.GraphOracle(model, os.path.join(d, g.name + ".param"))
+    orc.set_input("data", x)
+    orc.run()
+    worst = compare_storages(exe, orc, model, what="resnet152")
+    print("resnet152 worst per-layer rel err %.2e (storage %s)" % worst)
+    logits_idx = model["kernels"][-1]["args"][0]
+    assert max_rel_err(exe.get_data(logits_idx, 1000), orc.storage[logits_idx]) < REL_TOL
+    assert int(np.argmax(exe.get_output())) == int(np.argmax(orc.get("output")))
+    # rerun: same bits (no state left behind by split-K workspaces)
+    first = exe.get_data(logits_idx, 1000)
+    exe.execute()
+    np.testing.assert_array_equal(exe.get_data(logits_idx, 1000), first)
+
+
+def test_preempt_flag_stops_and_restart_is_bit_identical(resnet18_dir, resnet18_oracle):
+    """Flag set before launch: every workgroup leaves at once, no completion is
+    counted and the output stays untouched; after clearing the flag a rerun gives
+    the same bits as an uninterrupted run (idempotence, src/reef/test/test.cpp:448-489)."""
+    g, d = resnet18_dir
+    _, _, x = resnet18_oracle
+    exe = B.Executor.from_dir(d, g.name, B.HYBRID)
+    exe.set_input_checked("data", x)
+    exe.execute_preemptable()
+    ref = exe.get_output()
+    slots = exe.read_task_slots()
+    blocks = [exe.kernel_info(i)["block_num"] for i in range(exe.num_kernels())]
+    assert slots == blocks, "every workgroup of every kernel completed once"
+
+    exe2 = B.Executor.from_dir(d, g.name, B.HYBRID)
+    exe2.set_input_checked("data", x)
+    exe2.poke_preempt_flag(1)
+    exe2.execute_preemptable()
+    assert exe2.read_task_slots() == [0] * exe2.num_kernels()
+    assert (exe2.get_output() == 0).all(), "storages stay zero-filled"
+    exe2.poke_preempt_flag(0)
+    exe2.execute_preemptable()
+    np.testing.assert_array_equal(exe2.get_output(), ref)
