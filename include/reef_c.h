@@ -62,8 +62,59 @@ int reef_executor_kernel_info(reef_executor_t e, int idx, int out[7]);
  */
 int reef_executor_time_kernel(reef_executor_t e, int idx, int flavour, int warmup, int iters,
                               float* avg_us);
+/* time_kernel_dkp: kernel idx through the DKP flavour with `layers` workgroup layers per CU
+ * and the first `task_num` tasks only -- the measurement behind <model>.profile.json
+ * (latency[j] = one round of (j+1) x num_cus workgroups; the reference's profiler tool
+ * is not in its repository, resource/Makefile:32-36). */
+int reef_executor_time_kernel_dkp(reef_executor_t e, int idx, int layers, int task_num, int warmup,
+                                  int iters, float* avg_us);
 int reef_executor_time_model(reef_executor_t e, int flavour, int warmup, int iters, float* lat_us,
                              float* dev_us);
+
+/* ---- REEFScheduler (src/reef/server/scheduler.h:68-126) ---- */
+typedef struct reef_scheduler_s* reef_scheduler_t;
+enum { REEF_MODE_NOPREEMPT = 0, REEF_MODE_MULTISTREAM = 1, REEF_MODE_WAITPREEMPT = 2,
+       REEF_MODE_REEF = 3, REEF_MODE_RESET = 4 };
+enum { REEF_QUEUE_RT = 0, REEF_QUEUE_BE = 1 };
+int reef_scheduler_create(int mode, reef_scheduler_t* out);
+void reef_scheduler_destroy(reef_scheduler_t s);
+/* load_model(dir, name) (scheduler.cpp:57-68); `with_param` != 0 also loads <dir>/<name>.param */
+int reef_scheduler_load_model(reef_scheduler_t s, const char* dir, const char* name, int with_param,
+                              uint32_t* mid);
+int reef_scheduler_load_model_files(reef_scheduler_t s, const char* rt_co, const char* be_co,
+                                    const char* json, const char* profile, const char* param,
+                                    uint32_t* mid);
+int reef_scheduler_create_queue(reef_scheduler_t s, int queue_type, uint32_t* qid);
+int reef_scheduler_bind_model_queue(reef_scheduler_t s, uint32_t qid, uint32_t mid);
+int reef_scheduler_get_data_size(reef_scheduler_t s, uint32_t mid, const char* name, size_t* size);
+int reef_scheduler_set_input(reef_scheduler_t s, uint32_t mid, const void* data, size_t len,
+                             const char* name);
+int reef_scheduler_get_output(reef_scheduler_t s, uint32_t mid, void* data, size_t len);
+int reef_scheduler_new_task(reef_scheduler_t s, uint32_t mid, uint32_t* tid);
+int reef_scheduler_wait_task(reef_scheduler_t s, uint32_t tid);
+/* Task record: flags bit0 preempted, bit1 padded, bit2 padded to completion;
+ * stamps = submit, start, end in nanoseconds since the epoch; state = TaskState. */
+int reef_scheduler_task_info(reef_scheduler_t s, uint32_t tid, int* flags, int64_t stamps_ns[3],
+                             int* state);
+int reef_scheduler_run(reef_scheduler_t s);
+int reef_scheduler_shutdown(reef_scheduler_t s);
+int reef_scheduler_mode(reef_scheduler_t s);
+void reef_scheduler_set_wait_sync(reef_scheduler_t s, int value);
+void reef_scheduler_set_be_stream_cap(reef_scheduler_t s, int value);
+int64_t reef_scheduler_avg_preempt_latency(reef_scheduler_t s);
+int64_t reef_scheduler_max_preempt_latency(reef_scheduler_t s);
+int64_t reef_scheduler_avg_kernel_sel_latency(reef_scheduler_t s);
+uint64_t reef_scheduler_preempt_times(reef_scheduler_t s);
+uint64_t reef_scheduler_padded_kernels(reef_scheduler_t s);
+size_t reef_scheduler_preempt_samples(reef_scheduler_t s, int64_t* out, size_t cap);
+/* DKP decision for one (real-time kernel, best-effort kernel) pair (scheduler.cpp:533-602).
+ * rt / be = {block_num, min_occupancy, threads, vgprs, sgprs, lds, total_latency};
+ * be_latency[n_lat] = best-effort kernel latency per occupancy; proxy = {vgprs, sgprs, lds}.
+ * out = {merge, rt_occupancy, be_occupancy, final_occupancy, cu_partition, be_block_num,
+ *        merged_block_size, lds}. */
+int reef_dkp_decide(const int rt[7], const int be[7], const int* be_latency, int n_lat,
+                    int be_block_offset, const int proxy[3], int num_cus, int num_xcds, int out[8]);
+int reef_dkp_rollback(int launch_offset, int dropped, int window, int kernel_offset);
 
 /* GPUConfig (src/reef/executor/hip/hip_impl.cpp:9-74) */
 int reef_gpuconfig_num_cus(void);

@@ -268,7 +268,7 @@ class GraphOracle:
             else None
 
     def run_kernel(self, k, acc64=False):
-        name, a = k["name"], k.get("attrs", [])
+        name, a = k["name"].split("#")[0], k.get("attrs", [])
         P = [self.storage[i] for i in k["args"]]
         if name.startswith("reef_conv2d"):
             Cin, H, W, Cout, Ho, Wo, kh, kw, sh, sw, ph, pw, flags, act, _tile, split_k = a[:16]

@@ -155,8 +155,137 @@ class Executor:
                                                              ctypes.byref(us)))
         return us.value
 
+    def time_kernel_dkp(self, idx, layers, task_num, warmup=2, iters=10):
+        us = ctypes.c_float()
+        _check("time_kernel_dkp", lib().reef_executor_time_kernel_dkp(self.h, idx, layers, task_num,
+                                                                     warmup, iters, ctypes.byref(us)))
+        return us.value
+
     def time_model(self, flavour=RUN_DEFAULT, warmup=5, iters=50):
         lat = (ctypes.c_float * iters)()
         dev = (ctypes.c_float * iters)()
         _check("time_model", lib().reef_executor_time_model(self.h, flavour, warmup, iters, lat, dev))
         return np.array(lat, np.float64), np.array(dev, np.float64)
+
+
+MODE_NOPREEMPT, MODE_MULTISTREAM, MODE_WAITPREEMPT, MODE_REEF, MODE_RESET = range(5)
+QUEUE_RT, QUEUE_BE = 0, 1
+STATE_INIT, STATE_WAITING, STATE_EXECUTING, STATE_FINISH = range(4)
+
+
+class Scheduler:
+    """REEFScheduler (src/reef/server/scheduler.h) through the flat C API."""
+
+    def __init__(self, mode=MODE_REEF):
+        self.h = ctypes.c_void_p()
+        L = lib()
+        for fn in ("reef_scheduler_avg_preempt_latency", "reef_scheduler_max_preempt_latency",
+                   "reef_scheduler_avg_kernel_sel_latency"):
+            getattr(L, fn).restype = ctypes.c_int64
+        for fn in ("reef_scheduler_preempt_times", "reef_scheduler_padded_kernels"):
+            getattr(L, fn).restype = ctypes.c_uint64
+        L.reef_scheduler_preempt_samples.restype = ctypes.c_size_t
+        _check("scheduler_create", L.reef_scheduler_create(mode, ctypes.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib().reef_scheduler_destroy(self.h)
+            self.h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def load_model(self, model_dir, name, with_param=True):
+        mid = ctypes.c_uint32()
+        with_param = with_param and os.path.exists(os.path.join(model_dir, name + ".param"))
+        _check("load_model", lib().reef_scheduler_load_model(self.h, model_dir.encode(), name.encode(),
+                                                            int(with_param), ctypes.byref(mid)))
+        return mid.value
+
+    def create_queue(self, qtype):
+        qid = ctypes.c_uint32()
+        st = lib().reef_scheduler_create_queue(self.h, qtype, ctypes.byref(qid))
+        _check("create_queue", st)
+        return qid.value
+
+    def create_queue_status(self, qtype):
+        qid = ctypes.c_uint32()
+        return lib().reef_scheduler_create_queue(self.h, qtype, ctypes.byref(qid)), qid.value
+
+    def bind_model_queue(self, qid, mid):
+        return lib().reef_scheduler_bind_model_queue(self.h, qid, mid)
+
+    def get_data_size(self, mid, name):
+        sz = ctypes.c_size_t()
+        st = lib().reef_scheduler_get_data_size(self.h, mid, name.encode(), ctypes.byref(sz))
+        return st, sz.value
+
+    def set_input(self, mid, arr, name="data"):
+        arr = np.ascontiguousarray(arr)
+        return lib().reef_scheduler_set_input(self.h, mid, arr.ctypes.data_as(ctypes.c_void_p),
+                                              ctypes.c_size_t(arr.nbytes), name.encode())
+
+    def get_output(self, mid, n):
+        out = np.empty(n, np.float32)
+        _check("get_output", lib().reef_scheduler_get_output(self.h, mid, out.ctypes.data_as(ctypes.c_void_p),
+                                                            ctypes.c_size_t(out.nbytes)))
+        return out
+
+    def new_task(self, mid):
+        tid = ctypes.c_uint32()
+        _check("new_task", lib().reef_scheduler_new_task(self.h, mid, ctypes.byref(tid)))
+        return tid.value
+
+    def new_task_status(self, mid):
+        tid = ctypes.c_uint32()
+        return lib().reef_scheduler_new_task(self.h, mid, ctypes.byref(tid))
+
+    def wait_task(self, tid):
+        return lib().reef_scheduler_wait_task(self.h, tid)
+
+    def task_info(self, tid):
+        flags, state = ctypes.c_int(), ctypes.c_int()
+        stamps = (ctypes.c_int64 * 3)()
+        _check("task_info", lib().reef_scheduler_task_info(self.h, tid, ctypes.byref(flags), stamps,
+                                                          ctypes.byref(state)))
+        return {"preempted": bool(flags.value & 1), "padded": bool(flags.value & 2),
+                "padded_to_complete": bool(flags.value & 4), "submit": stamps[0], "start": stamps[1],
+                "end": stamps[2], "state": state.value}
+
+    def run(self):
+        _check("run", lib().reef_scheduler_run(self.h))
+
+    def shutdown(self):
+        _check("shutdown", lib().reef_scheduler_shutdown(self.h))
+
+    def mode(self):
+        return lib().reef_scheduler_mode(self.h)
+
+    def set_wait_sync(self, v):
+        lib().reef_scheduler_set_wait_sync(self.h, int(v))
+
+    def set_be_stream_cap(self, v):
+        lib().reef_scheduler_set_be_stream_cap(self.h, int(v))
+
+    def avg_preempt_latency(self):
+        return lib().reef_scheduler_avg_preempt_latency(self.h)
+
+    def max_preempt_latency(self):
+        return lib().reef_scheduler_max_preempt_latency(self.h)
+
+    def avg_kernel_sel_latency(self):
+        return lib().reef_scheduler_avg_kernel_sel_latency(self.h)
+
+    def preempt_times(self):
+        return lib().reef_scheduler_preempt_times(self.h)
+
+    def padded_kernels(self):
+        return lib().reef_scheduler_padded_kernels(self.h)
+
+    def preempt_samples(self, cap=100000):
+        buf = (ctypes.c_int64 * cap)()
+        n = lib().reef_scheduler_preempt_samples(self.h, buf, ctypes.c_size_t(cap))
+        return np.array(buf[:n], np.int64)

@@ -8,6 +8,7 @@
 #include "executor/hybrid_executor.h"
 #include "hal/code_object.h"
 #include "reef_c.h"
+#include "server/scheduler.h"
 
 using namespace reef;
 using namespace reef::executor;
@@ -136,6 +137,28 @@ int reef_executor_time_kernel(reef_executor_t e, int idx, int flavour, int warmu
     return Status::Succ;
 }
 
+int reef_executor_time_kernel_dkp(reef_executor_t e, int idx, int layers, int task_num, int warmup,
+                                  int iters, float* avg_us) {
+    TransExecutor* t = e->trans();
+    if (!t || idx < 0 || idx >= (int)t->num_kernels() || iters <= 0 || layers <= 0) return Status::OutOfRange;
+    GPUStream_t s = t->stream();
+    for (int i = 0; i < warmup; ++i) RETURN_STATUS(t->launch_kernel_dkp(idx, layers, task_num, s));
+    reef_event_t a, b;
+    GPU_RETURN_STATUS(reef_hal_event_create(&a));
+    GPU_RETURN_STATUS(reef_hal_event_create(&b));
+    GPU_RETURN_STATUS(reef_hal_stream_sync(s));
+    GPU_RETURN_STATUS(reef_hal_event_record(a, s));
+    for (int i = 0; i < iters; ++i) RETURN_STATUS(t->launch_kernel_dkp(idx, layers, task_num, s));
+    GPU_RETURN_STATUS(reef_hal_event_record(b, s));
+    GPU_RETURN_STATUS(reef_hal_event_sync(b));
+    float us = 0.f;
+    GPU_RETURN_STATUS(reef_hal_event_elapsed_us(a, b, &us));
+    *avg_us = us / (float)iters;
+    reef_hal_event_destroy(a);
+    reef_hal_event_destroy(b);
+    return Status::Succ;
+}
+
 int reef_executor_time_model(reef_executor_t e, int flavour, int warmup, int iters, float* lat_us,
                              float* dev_us) {
     GPUStream_t s = e->exe->stream();
@@ -159,6 +182,110 @@ int reef_executor_time_model(reef_executor_t e, int flavour, int warmup, int ite
     reef_hal_event_destroy(a);
     reef_hal_event_destroy(b);
     return Status::Succ;
+}
+
+}  // extern "C"
+
+struct reef_scheduler_s {
+    std::unique_ptr<reef::server::REEFScheduler> s;
+};
+
+extern "C" {
+
+using reef::server::REEFScheduler;
+
+int reef_scheduler_create(int mode, reef_scheduler_t* out) {
+    if (mode < 0 || mode > 4) return Status::OutOfRange;
+    reef_scheduler_s* h = new reef_scheduler_s;
+    h->s.reset(new REEFScheduler((REEFScheduler::ScheduleMode)mode));
+    *out = h;
+    return Status::Succ;
+}
+void reef_scheduler_destroy(reef_scheduler_t h) { delete h; }
+int reef_scheduler_load_model(reef_scheduler_t h, const char* dir, const char* name, int with_param,
+                              uint32_t* mid) {
+    if (!with_param) return h->s->load_model(std::string(dir), std::string(name), *mid);
+    const std::string base = std::string(dir) + "/" + name;
+    return h->s->load_model(base + ".trans.co", base + ".be.co", base + ".json",
+                            base + ".profile.json", base + ".param", *mid);
+}
+int reef_scheduler_load_model_files(reef_scheduler_t h, const char* rt_co, const char* be_co,
+                                    const char* json, const char* profile, const char* param,
+                                    uint32_t* mid) {
+    return h->s->load_model(rt_co, be_co, json, profile, param ? param : "", *mid);
+}
+int reef_scheduler_create_queue(reef_scheduler_t h, int queue_type, uint32_t* qid) {
+    return h->s->create_queue(queue_type == REEF_QUEUE_RT ? REEFScheduler::RealTimeQueue
+                                                          : REEFScheduler::BestEffortQueue, *qid);
+}
+int reef_scheduler_bind_model_queue(reef_scheduler_t h, uint32_t qid, uint32_t mid) {
+    return h->s->bind_model_queue(qid, mid);
+}
+int reef_scheduler_get_data_size(reef_scheduler_t h, uint32_t mid, const char* name, size_t* size) {
+    return h->s->get_data_size(mid, name, *size);
+}
+int reef_scheduler_set_input(reef_scheduler_t h, uint32_t mid, const void* data, size_t len,
+                             const char* name) {
+    return h->s->set_input(mid, data, len, name ? name : "data");
+}
+int reef_scheduler_get_output(reef_scheduler_t h, uint32_t mid, void* data, size_t len) {
+    return h->s->get_output(mid, data, len);
+}
+int reef_scheduler_new_task(reef_scheduler_t h, uint32_t mid, uint32_t* tid) {
+    return h->s->new_task(mid, *tid);
+}
+int reef_scheduler_wait_task(reef_scheduler_t h, uint32_t tid) { return h->s->wait_task(tid); }
+int reef_scheduler_task_info(reef_scheduler_t h, uint32_t tid, int* flags, int64_t stamps_ns[3],
+                             int* state) {
+    std::shared_ptr<REEFScheduler::Task> t;
+    Status st = h->s->get_task(tid, t);
+    if (st != Status::Succ) return st;
+    *flags = (t->is_preempted() ? 1 : 0) | (t->is_padded() ? 2 : 0) | (t->is_padded_to_complete() ? 4 : 0);
+    auto ts = t->get_timestamp();
+    for (int i = 0; i < 3; ++i)
+        stamps_ns[i] = std::chrono::duration_cast<std::chrono::nanoseconds>(ts[i].time_since_epoch()).count();
+    *state = (int)t->get_state();
+    return Status::Succ;
+}
+int reef_scheduler_run(reef_scheduler_t h) { return h->s->run(); }
+int reef_scheduler_shutdown(reef_scheduler_t h) { return h->s->shutdown(); }
+int reef_scheduler_mode(reef_scheduler_t h) { return (int)h->s->sche_mode(); }
+void reef_scheduler_set_wait_sync(reef_scheduler_t h, int v) { h->s->set_wait_sync(v != 0); }
+void reef_scheduler_set_be_stream_cap(reef_scheduler_t h, int v) { h->s->set_be_stream_cap(v); }
+int64_t reef_scheduler_avg_preempt_latency(reef_scheduler_t h) { return h->s->avg_preempt_latency(); }
+int64_t reef_scheduler_max_preempt_latency(reef_scheduler_t h) { return h->s->max_preempt_latency(); }
+int64_t reef_scheduler_avg_kernel_sel_latency(reef_scheduler_t h) { return h->s->avg_kernel_sel_latency(); }
+uint64_t reef_scheduler_preempt_times(reef_scheduler_t h) { return h->s->preempt_times(); }
+uint64_t reef_scheduler_padded_kernels(reef_scheduler_t h) { return h->s->padded_kernels(); }
+size_t reef_scheduler_preempt_samples(reef_scheduler_t h, int64_t* out, size_t cap) {
+    return h->s->preempt_latency_samples(out, cap);
+}
+
+int reef_dkp_decide(const int rt[7], const int be[7], const int* be_latency, int n_lat,
+                    int be_block_offset, const int proxy[3], int num_cus, int num_xcds, int out[8]) {
+    auto fill = [](TransExecutor::KernelArg& ka, const int v[7]) {
+        ka.block_num = v[0];
+        ka.min_occupancy = v[1];
+        ka.thread_dim = dim3u((uint32_t)v[2], 1, 1);
+        ka.task_dim = dim3u((uint32_t)v[0], 1, 1);
+        ka.resource = GPUConfig::KernelResource{v[5], v[3], v[4], 0};
+        ka.profile.total_latency = v[6];
+        ka.block_offset = 0;
+    };
+    TransExecutor::KernelArg rta, bea;
+    fill(rta, rt);
+    fill(bea, be);
+    bea.profile.latency.assign(be_latency, be_latency + n_lat);
+    GPUConfig::KernelResource pr{proxy[2], proxy[0], proxy[1], 0};
+    REEFScheduler::PadDecision d =
+        REEFScheduler::decide_padding(rta, bea, be_block_offset, pr, num_cus, num_xcds);
+    out[0] = d.merge; out[1] = d.rt_occupancy; out[2] = d.be_occupancy; out[3] = d.final_occupancy;
+    out[4] = d.cu_partition; out[5] = d.be_block_num; out[6] = d.merged_block_size;
+    out[7] = d.resource.shared_memory;
+    return Status::Succ;
+}
+int reef_dkp_rollback(int launch_offset, int dropped, int window, int kernel_offset) {
+    return REEFScheduler::rollback_kernel_offset(launch_offset, dropped, window, kernel_offset);
 }
 
 int reef_gpuconfig_num_cus(void) { return (int)GPUConfig::get_num_cus(); }

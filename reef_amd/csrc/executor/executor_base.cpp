@@ -24,6 +24,11 @@ Status ExecutorBase::load_model_from_GPU_module(const char* json_file_path, GPUM
     return init_executor_base(json_file_path, mod);
 }
 
+std::string ExecutorBase::kernel_symbol(const std::string& name) {
+    const size_t p = name.find('#');
+    return p == std::string::npos ? name : name.substr(0, p);
+}
+
 size_t ExecutorBase::storage_bytes(size_t idx) const {
     const StorageInfo& si = model->storage[idx];
     return Model::get_stype_size(si.stype) * si.size;
@@ -37,11 +42,14 @@ Status ExecutorBase::init_executor_base(const char* json_file_path, GPUModule_t 
     // kernels: one lookup per distinct name
     kernel_funcs.clear();
     for (KernelInfo& ki : model->kernels) {
-        auto it = kernels.find(ki.name);
+        // "symbol#instance": the part before '#' is the entry symbol, the whole
+        // string keys the per-kernel profile (one symbol serves many layers here).
+        const std::string sym = kernel_symbol(ki.name);
+        auto it = kernels.find(sym);
         if (it == kernels.end()) {
             GPUFunction_t fn;
-            GPU_RETURN_STATUS(reef_hal_module_get_function(mod, ki.name.c_str(), &fn));
-            it = kernels.emplace(ki.name, fn).first;
+            GPU_RETURN_STATUS(reef_hal_module_get_function(mod, sym.c_str(), &fn));
+            it = kernels.emplace(sym, fn).first;
         }
         kernel_funcs.push_back(it->second);
         if (ki.args.size() > REEF_MAX_PTRS || ki.attrs.size() > REEF_MAX_ATTRS) {

@@ -49,6 +49,9 @@ public:
     // Launches kernels [begin, end) without synchronising (for timing loops).
     Status launch_range(int begin, int end, GPUStream_t stream);
 
+    // Entry symbol of a graph-JSON kernel name ("symbol" or "symbol#instance").
+    static std::string kernel_symbol(const std::string& name);
+
     std::unique_ptr<Model> model;
 
 protected:

@@ -58,7 +58,7 @@ Status HybridExecutor::init_hybrid_executor(const char* json_file_path,
     preempt_kernels.resize(n);
     std::unordered_map<std::string, GPUFunction_t> seen;
     for (size_t i = 0; i < n; i++) {
-        const std::string& name = model->kernels[i].name;
+        const std::string name = kernel_symbol(model->kernels[i].name);
         auto it = seen.find(name);
         if (it == seen.end()) {
             GPUFunction_t fn;

@@ -56,7 +56,7 @@ Status TransExecutor::init_rt_executor(const char* json_file_path, GPUModule_t m
         const KernelInfo& ki = model->kernels[i];
         const uint32_t* lp = ki.launch_params;
         ka.kernel = kernel_funcs[i];
-        ka.op = op_from_name(ki.name);
+        ka.op = op_from_name(kernel_symbol(ki.name));
         ka.task_dim = dim3u(lp[0], lp[1], lp[2]);
         ka.thread_dim = dim3u(lp[3], lp[4], lp[5]);
         ka.block_num = (int)ka.task_dim.count();
@@ -112,6 +112,24 @@ Status TransExecutor::launch_kernel(int i, GPUStream_t stream) {
     a.num_xcds = (int)GPUConfig::get_num_xcds();
     a.task_slot_r = nullptr;
     const uint32_t grid[3] = {(uint32_t)(num_cus * ka.min_occupancy), 1, 1};
+    const uint32_t block[3] = {ka.thread_dim.count(), 1, 1};
+    GPU_RETURN_STATUS(reef_hal_launch(ka.kernel, grid, block, 0, stream, &a, sizeof(a)));
+    return Status::Succ;
+}
+
+// One single-sided launch with an explicit layer count and task range (profiling).
+Status TransExecutor::launch_kernel_dkp(int i, int layers, int task_num, GPUStream_t stream) {
+    const KernelArg& ka = trans_args[i];
+    const int num_cus = (int)GPUConfig::get_num_cus();
+    ReefDkpArgs a;
+    std::memset(&a, 0, sizeof(a));
+    fill_side(a.l, i, layers, std::min(task_num, ka.block_num), 0);
+    a.r = a.l;
+    a.r.task_num = 0;
+    a.cu_partition = num_cus;
+    a.num_cus = num_cus;
+    a.num_xcds = (int)GPUConfig::get_num_xcds();
+    const uint32_t grid[3] = {(uint32_t)(num_cus * layers), 1, 1};
     const uint32_t block[3] = {ka.thread_dim.count(), 1, 1};
     GPU_RETURN_STATUS(reef_hal_launch(ka.kernel, grid, block, 0, stream, &a, sizeof(a)));
     return Status::Succ;

@@ -42,6 +42,7 @@ public:
     static int op_from_name(const std::string& name);
 
     const std::vector<KernelArg>& kernel_args() const { return trans_args; }
+    Status launch_kernel_dkp(int kernel_offset, int layers, int task_num, GPUStream_t stream);
     // Occupancy class 1..8 (waves per SIMD) a merged launch needs
     // (trans_executor.cpp:175-199 picks among 10 gfx906 classes).
     static int occupancy_class(const GPUConfig::KernelResource& kr);

@@ -1,0 +1,580 @@
+#include "server/scheduler.h"
+
+#include <algorithm>
+#include <cstring>
+
+namespace reef {
+namespace server {
+
+using executor::GPUConfig;
+using executor::HybridExecutor;
+using executor::TransExecutor;
+typedef std::chrono::system_clock Clock;
+
+// ---------------------------------------------------------------- task queues
+void REEFScheduler::TaskQueue::push(std::shared_ptr<Task> t) {
+    std::lock_guard<std::mutex> lock(mtx);
+    tasks.push_back(std::move(t));
+    count.store(tasks.size(), std::memory_order_release);
+}
+std::shared_ptr<REEFScheduler::Task> REEFScheduler::TaskQueue::front() {
+    std::lock_guard<std::mutex> lock(mtx);
+    return tasks.empty() ? nullptr : tasks.front();
+}
+void REEFScheduler::TaskQueue::pop() {
+    std::lock_guard<std::mutex> lock(mtx);
+    if (!tasks.empty()) tasks.pop_front();
+    count.store(tasks.size(), std::memory_order_release);
+}
+
+// ---------------------------------------------------------------- life cycle
+REEFScheduler::REEFScheduler(ScheduleMode _mode)
+    : mode(_mode),
+      model_pool_size(0),
+      model_pool(model_pool_capacity),
+      task_idx_pool(0),
+      be_queues(max_num_be_queues),
+      be_queue_cnt(0),
+      pending_tasks(0),
+      wait_sync(false),
+      preempt_stream(nullptr),
+      preempt_flag(nullptr),
+      preempted(false),
+      _shutdown(false),
+      preempt_count(0),
+      preempt_latency_sum(0),
+      preempt_latency_max(0),
+      kernel_sel_count(0),
+      kernel_sel_latency_sum(0),
+      padded_kernel_count(0),
+      gpu_ready(false) {
+    // Window of kernels a best-effort stream keeps on the device
+    // (scheduler.cpp:29-33: 2, or 1024 when preemption waits for completion).
+    be_stream_device_queue_cap = (mode == WaitPreempt) ? 1024 : 2;
+}
+
+REEFScheduler::~REEFScheduler() {
+    if (scheduler) shutdown();
+}
+
+// Streams and the shared preemption flag (scheduler.cpp:24-28).
+Status REEFScheduler::ensure_gpu() {
+    if (gpu_ready) return Status::Succ;
+    GPU_RETURN_STATUS(reef_hal_init(0));
+    GPU_RETURN_STATUS(reef_hal_stream_create(0, &preempt_stream));
+    GPU_RETURN_STATUS(reef_hal_malloc(4, REEF_MEM_DEVICE_FINEGRAINED, &preempt_flag));
+    GPU_RETURN_STATUS(reef_hal_write_value32(preempt_stream, preempt_flag, 0));
+    GPU_RETURN_STATUS(reef_hal_stream_sync(preempt_stream));
+    gpu_ready = true;
+    return Status::Succ;
+}
+
+Status REEFScheduler::create_task_queue(std::shared_ptr<TaskQueue>& ret, bool rt) {
+    RETURN_STATUS(ensure_gpu());
+    executor::GPUStream_t stream;
+    if (rt) {
+        REEF_LOG_INFO("create rt stream");
+        GPU_RETURN_STATUS(reef_hal_stream_create(0, &stream));
+    } else {
+        REEF_LOG_INFO("create be stream");
+        GPU_RETURN_STATUS(reef_hal_stream_create(be_stream_device_queue_cap, &stream));
+    }
+    ret = std::make_shared<TaskQueue>();
+    ret->stream = stream;
+    return Status::Succ;
+}
+
+Status REEFScheduler::load_model(const std::string& model_dir, const std::string& model_name,
+                                 ModelID& mid) {
+    const std::string base = model_dir + "/" + model_name;
+    return load_model(base + ".trans.co", base + ".be.co", base + ".json", base + ".profile.json",
+                      "", mid);
+}
+
+Status REEFScheduler::load_model(const std::string& rt_co_path, const std::string& be_co_path,
+                                 const std::string& json_path, const std::string& profile_path,
+                                 const std::string& param_path, ModelID& mid) {
+    RETURN_STATUS(ensure_gpu());
+    std::shared_ptr<Model> model(new Model);
+    RETURN_STATUS(model->executor.load_hybrid_model_from_file(
+        json_path.c_str(), profile_path.c_str(), rt_co_path.c_str(), be_co_path.c_str()));
+    model->qid = rt_queue_id;  // real-time queue by default
+    if (!param_path.empty()) RETURN_STATUS(model->executor.load_param_from_file(param_path.c_str()));
+    const uint32_t idx = model_pool_size.fetch_add(1);
+    if (idx >= model_pool_capacity) {
+        REEF_LOG_ERROR("model pool is full");
+        model_pool_size.fetch_sub(1);
+        return Status::Fail;
+    }
+    RETURN_STATUS(model->executor.set_preempt_flag(preempt_flag));
+    model_pool[idx] = std::move(model);
+    REEF_LOG_INFO("load model from %s, idx %u", json_path.c_str(), idx);
+    mid = idx;
+    return Status::Succ;
+}
+
+Status REEFScheduler::create_queue(const TaskQueueType& qtp, QueueID& qid) {
+    if (qtp == TaskQueueType::RealTimeQueue) {
+        qid = rt_queue_id;
+        std::lock_guard<std::mutex> lock(be_queues_mtx);
+        if (!rt_queue) RETURN_STATUS(create_task_queue(rt_queue, true));
+        return Status::Succ;
+    }
+    std::shared_ptr<TaskQueue> q;
+    RETURN_STATUS(create_task_queue(q, false));
+    std::lock_guard<std::mutex> lock(be_queues_mtx);
+    const uint32_t idx = be_queue_cnt.load();
+    if (idx >= max_num_be_queues) RETURN_STATUS(Status::Full);
+    be_queues[idx] = std::move(q);
+    be_queue_cnt.store(idx + 1);
+    qid = idx;
+    return Status::Succ;
+}
+
+Status REEFScheduler::bind_model_queue(const QueueID& qid, const ModelID& mid) {
+    if (model_pool_size.load() <= mid) RETURN_STATUS(Status::OutOfRange);
+    if (be_queue_cnt.load() <= qid && qid != rt_queue_id) RETURN_STATUS(Status::OutOfRange);
+    model_pool[mid]->qid = qid;
+    return Status::Succ;
+}
+
+Status REEFScheduler::new_task(const ModelID& mid, TaskID& tid) {
+    if (model_pool_size.load() <= mid) RETURN_STATUS(Status::OutOfRange);
+    auto& model = model_pool[mid];
+    if (model->qid == rt_queue_id && !rt_queue) RETURN_STATUS(Status::NotFound);
+    std::shared_ptr<Task> task(new Task);
+    task->model = model;
+    task->id = task_idx_pool.fetch_add(1);
+    task->qid = model->qid;
+    task->block_offset = 0;
+    task->kernel_offset = 0;
+    task->launch_offset = 0;
+    task->state.store(TaskState::Init);
+    task->submit = Clock::now();
+    task->preempted = false;
+    task->padding = false;
+    task->padding_to_finish = false;
+    tid = task->id;
+    {
+        std::lock_guard<std::mutex> lock(task_pool_mtx);
+        task_pool.insert({tid, task});
+    }
+    if (model->qid == rt_queue_id) rt_queue->push(task);
+    else be_queues[model->qid]->push(task);
+    {
+        std::lock_guard<std::mutex> lock(task_cnt_mtx);
+        pending_tasks.fetch_add(1);
+    }
+    task_cnt_cv.notify_all();
+    return Status::Succ;
+}
+
+Status REEFScheduler::get_task(TaskID tid, std::shared_ptr<Task>& t) {
+    std::lock_guard<std::mutex> lock(task_pool_mtx);
+    auto it = task_pool.find(tid);
+    if (it == task_pool.end()) return Status::NotFound;
+    t = it->second;
+    return Status::Succ;
+}
+
+Status REEFScheduler::wait_task(TaskID tid) {
+    std::shared_ptr<Task> task;
+    RETURN_STATUS(get_task(tid, task));
+    std::unique_lock<std::mutex> lock(task->mtx);
+    task->cv.wait(lock, [&] { return task->state.load() == TaskState::Finish; });
+    return Status::Succ;
+}
+
+Status REEFScheduler::get_data_size(ModelID mid, const std::string& name, size_t& size) {
+    if (mid >= model_pool_size.load()) RETURN_STATUS(Status::OutOfRange);
+    return model_pool[mid]->executor.get_data_size(name, size);
+}
+Status REEFScheduler::set_input(ModelID mid, const void* data, size_t len, const std::string& name) {
+    if (mid >= model_pool_size.load()) RETURN_STATUS(Status::OutOfRange);
+    return model_pool[mid]->executor.set_input(name, data, len);
+}
+// The name is accepted and ignored, as in the reference (scheduler.cpp:226-230).
+Status REEFScheduler::get_output(ModelID mid, void* data, size_t len, const std::string&) {
+    if (mid >= model_pool_size.load()) RETURN_STATUS(Status::OutOfRange);
+    return model_pool[mid]->executor.get_output(data, len);
+}
+
+Status REEFScheduler::run() {
+    if (scheduler) RETURN_STATUS(Status::Fail);
+    {
+        std::lock_guard<std::mutex> lock(be_queues_mtx);
+        if (!rt_queue) RETURN_STATUS(create_task_queue(rt_queue, true));
+    }
+    _shutdown.store(false);
+    scheduler.reset(new std::thread([this] {
+        reef_hal_init(0);  // bind the device to this thread
+        while (!_shutdown.load()) {
+            if (pending_tasks.load() == 0) {
+                std::unique_lock<std::mutex> lock(task_cnt_mtx);
+                task_cnt_cv.wait_for(lock, std::chrono::milliseconds(2), [this] {
+                    return pending_tasks.load() != 0 || _shutdown.load();
+                });
+                continue;
+            }
+            loop_body();
+        }
+    }));
+    return Status::Succ;
+}
+
+Status REEFScheduler::shutdown() {
+    if (!scheduler) return Status::Succ;
+    _shutdown.store(true);
+    task_cnt_cv.notify_all();
+    scheduler->join();
+    scheduler.reset();
+    return Status::Succ;
+}
+
+void REEFScheduler::finish_task(const std::shared_ptr<Task>& task, TimePoint end) {
+    task->end = end;
+    {
+        std::lock_guard<std::mutex> lock(task->mtx);
+        task->state.store(TaskState::Finish);
+    }
+    task->cv.notify_all();
+    pending_tasks.fetch_sub(1);
+}
+
+// ---------------------------------------------------------------- scheduling loop
+// Real-time tasks to exhaustion, then one pass over the best-effort queues,
+// going back to real-time mode as soon as a real-time task shows up
+// (scheduler.cpp:262-303).
+void REEFScheduler::loop_body() {
+    for (;;) {
+        while (!rt_queue->empty()) {
+            preempt_be_tasks();
+            auto rt_task = rt_queue->front();
+            rt_queue->pop();
+            execute_rt_task(rt_task);
+        }
+        bool rt_arrived = false;
+        const uint32_t n = be_queue_cnt.load();
+        for (uint32_t i = 0; i < n && !rt_arrived; i++) {
+            auto& q = be_queues[i];
+            while (!q->empty()) {
+                if (!rt_queue->empty()) { rt_arrived = true; break; }
+                auto be_task = q->front();
+                execute_be_task(be_task, q);
+                if (!rt_queue->empty()) { rt_arrived = true; break; }
+                if (be_task->state.load() == TaskState::Finish) {
+                    q->pop();
+                    continue;
+                }
+                break;
+            }
+        }
+        if (!rt_arrived) return;
+    }
+}
+
+int REEFScheduler::rollback_kernel_offset(int launch_offset, int dropped, int window, int kernel_offset) {
+    return std::max(launch_offset - dropped - window, kernel_offset);
+}
+
+// Reset-based preemption (scheduler.cpp:305-346): raise the flag, drop what the
+// best-effort streams still hold on the host, roll every running task back to a
+// kernel that is certainly complete, and (optionally) wait until the kernels
+// that were already on the device have left.
+void REEFScheduler::preempt_reset() {
+    reef_hal_write_value32(preempt_stream, preempt_flag, 1);
+    const uint32_t n = be_queue_cnt.load();
+    for (uint32_t i = 0; i < n; i++) {
+        uint64_t dropped = 0;
+        reef_hal_stream_clear_queue(be_queues[i]->stream, &dropped);
+        auto task = be_queues[i]->front();
+        if (task && task->state.load() == TaskState::Executing) {
+            task->kernel_offset = rollback_kernel_offset(task->launch_offset, (int)dropped,
+                                                         be_stream_device_queue_cap,
+                                                         task->kernel_offset);
+            task->block_offset = 0;
+            task->state.store(TaskState::Waiting);
+            task->preempted = true;
+        }
+    }
+    for (int i = 0; i < be_stream_device_queue_cap + 1; i++) reef_hal_reset_cus();
+    reef_hal_stream_sync(preempt_stream);
+    if (wait_sync) {
+        for (uint32_t i = 0; i < n; i++) reef_hal_stream_sync(be_queues[i]->stream);
+    }
+}
+
+// Wait-based preemption (scheduler.cpp:348-372): raise the flag, let the device
+// drain, then find per task the first kernel whose workgroups did not all finish.
+void REEFScheduler::preempt_wait() {
+    int one = 1;
+    reef_hal_memcpy_h2d_async(preempt_flag, &one, 4, preempt_stream);
+    reef_hal_stream_sync(preempt_stream);
+    const uint32_t n = be_queue_cnt.load();
+    for (uint32_t i = 0; i < n; i++) {
+        uint64_t dropped = 0;
+        reef_hal_stream_clear_queue(be_queues[i]->stream, &dropped);
+        reef_hal_stream_sync(be_queues[i]->stream);
+    }
+    for (uint32_t i = 0; i < n; i++) {
+        auto be_task = be_queues[i]->front();
+        if (!be_task) continue;
+        auto& exe = be_task->model->executor;
+        exe.copy_be_kernel_offset(preempt_stream);
+        exe.reset_task_slots(preempt_stream);
+        reef_hal_stream_sync(preempt_stream);
+        const int off = exe.get_be_kernel_offset(be_task->kernel_offset);
+        be_task->kernel_offset = std::max(be_task->kernel_offset, off);
+    }
+}
+
+void REEFScheduler::preempt_be_tasks() {
+    if (preempted) return;
+    preempted = true;
+    REEF_LOG_INFO("preempt");
+    const auto t0 = std::chrono::steady_clock::now();
+    switch (mode) {
+        case ScheduleMode::NoPreempt: {
+            const uint32_t n = be_queue_cnt.load();
+            for (uint32_t i = 0; i < n; i++) reef_hal_stream_sync(be_queues[i]->stream);
+            for (uint32_t i = 0; i < n; i++) {
+                auto be_task = be_queues[i]->front();
+                if (be_task && be_task->state.load() == TaskState::Executing)
+                    be_task->kernel_offset = be_task->launch_offset + 1;
+            }
+            break;
+        }
+        case ScheduleMode::Reset:
+        case ScheduleMode::REEF: preempt_reset(); break;
+        case ScheduleMode::WaitPreempt: preempt_wait(); break;
+        default: break;
+    }
+    const auto t1 = std::chrono::steady_clock::now();
+    const int64_t us = std::chrono::duration_cast<std::chrono::nanoseconds>(t1 - t0).count() / 1000;
+    {
+        std::lock_guard<std::mutex> lock(stats_mtx);
+        preempt_count++;
+        preempt_latency_sum += (uint64_t)us;
+        preempt_latency_max = std::max(preempt_latency_max, us);
+        preempt_samples.push_back(us);
+    }
+    REEF_LOG_INFO("preempt latency: %lld us", (long long)us);
+
+    const uint32_t n = be_queue_cnt.load();
+    for (uint32_t i = 0; i < n; i++) {
+        auto be_task = be_queues[i]->front();
+        if (be_task && be_task->state.load() == TaskState::Executing)
+            be_task->state.store(TaskState::Waiting);
+    }
+}
+
+int64_t REEFScheduler::avg_preempt_latency() const {
+    std::lock_guard<std::mutex> lock(stats_mtx);
+    return preempt_count ? (int64_t)(preempt_latency_sum / preempt_count) : 0;
+}
+int64_t REEFScheduler::avg_kernel_sel_latency() const {
+    return kernel_sel_count ? (int64_t)(kernel_sel_latency_sum / kernel_sel_count) : 0;
+}
+size_t REEFScheduler::preempt_latency_samples(int64_t* out, size_t cap) const {
+    std::lock_guard<std::mutex> lock(stats_mtx);
+    const size_t n = std::min(cap, preempt_samples.size());
+    std::copy(preempt_samples.end() - n, preempt_samples.end(), out);
+    return n;
+}
+
+void REEFScheduler::reset_preempt_flag_async() {
+    reef_hal_write_value32(preempt_stream, preempt_flag, 0);
+}
+
+void REEFScheduler::execute_rt_task(std::shared_ptr<Task>& task) {
+    REEF_LOG_INFO("start rt task");
+    task->state.store(TaskState::Executing);
+    task->start = Clock::now();
+    if (mode == ScheduleMode::REEF) {
+        dynamic_kernel_padding(task);
+        reef_hal_stream_sync(rt_queue->stream);
+    } else {
+        task->model->executor.execute(rt_queue->stream);
+    }
+    finish_task(task, Clock::now());
+    REEF_LOG_INFO("rt task finish");
+}
+
+// ---------------------------------------------------------------- dynamic kernel padding
+// Can `be` ride along with `rt`, and with how many workgroups?  (scheduler.cpp:533-602)
+//   fits      : occupancy(max resource, max block) >= rt.min_occupancy
+//   be_occ    : the largest j+1 <= merged occupancy with be.latency[j] <= rt.total_latency
+//   partition : CUs the rt kernel really needs, in whole slots per XCD
+//   be_blocks : (CUs left) * (rt_latency / be_latency[be_occ-1]) * be_occ, clamped to what is left
+REEFScheduler::PadDecision REEFScheduler::decide_padding(const TransExecutor::KernelArg& rt,
+                                                         const TransExecutor::KernelArg& be,
+                                                         int be_block_offset,
+                                                         const GPUConfig::KernelResource& proxy,
+                                                         int num_cus, int num_xcds) {
+    PadDecision d;
+    d.rt_occupancy = rt.min_occupancy;
+    d.final_occupancy = rt.min_occupancy;
+    d.cu_partition = num_cus;
+    d.merged_block_size = std::max((int)rt.thread_dim.count(), (int)be.thread_dim.count());
+    d.resource = GPUConfig::max_resource(GPUConfig::max_resource(rt.resource, be.resource), proxy);
+    // the proxy's LDS is dynamic: it needs the larger of the two sides' static LDS
+    d.resource.shared_memory = std::max(rt.resource.shared_memory, be.resource.shared_memory);
+    const int merged_occupancy = GPUConfig::calculate_occupancy(d.resource, d.merged_block_size);
+    if (merged_occupancy < rt.min_occupancy) return d;
+
+    int be_occupancy = 0;
+    const int rt_latency = rt.profile.total_latency;
+    for (int j = merged_occupancy - 1; j >= 0; j--) {
+        if ((int)be.profile.latency.size() <= j) continue;
+        if (be.profile.latency[j] <= rt_latency) {
+            be_occupancy = j + 1;
+            break;
+        }
+    }
+    if (be_occupancy == 0) return d;
+    const int be_latency = std::max(be.profile.latency[be_occupancy - 1], 1);
+
+    const int partition = TransExecutor::cu_partition_for(rt.block_num, num_cus, num_xcds);
+    const int be_iters = rt_latency / be_latency;
+    int be_blocks = (num_cus - partition) * be_iters * be_occupancy;
+    be_blocks = std::min(be_blocks, be.block_num - be_block_offset);
+    if (be_blocks <= 0) return d;
+
+    d.merge = true;
+    d.be_occupancy = be_occupancy;
+    d.final_occupancy = std::max(rt.min_occupancy, be_occupancy);
+    d.cu_partition = partition;
+    d.be_block_num = be_blocks;
+    return d;
+}
+
+void REEFScheduler::dynamic_kernel_padding(std::shared_ptr<Task>& rt_task) {
+    HybridExecutor& rt_exe = rt_task->model->executor;
+    const int num_cus = (int)GPUConfig::get_num_cus();
+    const int num_xcds = (int)GPUConfig::get_num_xcds();
+    std::vector<std::shared_ptr<Task>> complete_be_tasks;
+    TimePoint current_time_point = Clock::now();
+    GPUConfig::KernelResource proxy_res{};
+    GPUConfig::get_kernel_resource(rt_exe.proxy_kernels[0], proxy_res);
+
+    const int n_rt = (int)rt_exe.num_kernels();
+    for (int i = 0; i < n_rt; i++) {
+        const auto sel_start = std::chrono::steady_clock::now();
+        const TransExecutor::KernelArg& rt_args = rt_exe.trans_args[i];
+        PadDecision dec;
+        std::shared_ptr<Task> be_task;
+        const TransExecutor::KernelArg* be_args = nullptr;
+        const uint32_t n_q = be_queue_cnt.load();
+        for (uint32_t q = 0; q < n_q; q++) {   // first queue whose head kernel fits (scheduler.cpp:533-602)
+            auto cand = be_queues[q]->front();
+            if (!cand) continue;
+            HybridExecutor& be_exe = cand->model->executor;
+            if (cand->kernel_offset >= (int)be_exe.num_kernels()) continue;
+            const TransExecutor::KernelArg& ka = be_exe.trans_args[cand->kernel_offset];
+            PadDecision d = decide_padding(rt_args, ka, cand->block_offset, proxy_res, num_cus, num_xcds);
+            if (!d.merge) continue;
+            dec = d;
+            be_task = cand;
+            be_args = &ka;
+            break;
+        }
+        const auto sel_end = std::chrono::steady_clock::now();
+        kernel_sel_count++;
+        kernel_sel_latency_sum +=
+            (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(sel_end - sel_start).count();
+
+        if (!be_task) {
+            // nothing fits: the real-time kernel alone, single-sided
+            rt_exe.launch_kernel(i, rt_queue->stream);
+        } else {
+            HybridExecutor& be_exe = be_task->model->executor;
+            ReefDkpArgs a;
+            std::memset(&a, 0, sizeof(a));
+            rt_exe.fill_side(a.l, i, dec.rt_occupancy, rt_args.block_num, rt_args.block_offset);
+            be_exe.fill_side(a.r, be_task->kernel_offset, dec.be_occupancy, dec.be_block_num,
+                             be_task->block_offset);
+            a.cu_partition = dec.cu_partition;
+            a.num_cus = num_cus;
+            a.num_xcds = num_xcds;
+            a.task_slot_r = nullptr;
+            if (be_task->start.time_since_epoch().count() == 0) be_task->start = current_time_point;
+            executor::GPUFunction_t proxy = rt_exe.get_proxy_kernel(dec.resource);
+            const uint32_t grid[3] = {(uint32_t)(dec.final_occupancy * num_cus), 1, 1};
+            const uint32_t block[3] = {(uint32_t)dec.merged_block_size, 1, 1};
+            reef_hal_launch(proxy, grid, block, (uint32_t)dec.resource.shared_memory, rt_queue->stream,
+                            &a, sizeof(a));
+            padded_kernel_count++;
+        }
+        current_time_point += std::chrono::microseconds(rt_args.profile.total_latency);
+
+        // progress of the padded best-effort task (scheduler.cpp:655-672)
+        if (be_task) {
+            be_task->padding = true;
+            be_task->block_offset += dec.be_block_num;
+            if (be_task->block_offset >= be_args->block_num) {
+                be_task->block_offset = 0;
+                be_task->kernel_offset++;
+                if (be_task->kernel_offset >= (int)be_task->model->executor.num_kernels()) {
+                    be_task->kernel_offset = 0;
+                    be_task->padding_to_finish = true;
+                    be_task->end = current_time_point;
+                    complete_be_tasks.push_back(be_task);
+                    be_queues[be_task->qid]->pop();
+                }
+            }
+        }
+    }
+    // Tasks that finished inside real-time shadows are reported once the
+    // real-time stream has drained (their last workgroups run on it).
+    if (!complete_be_tasks.empty()) {
+        reef_hal_stream_sync(rt_queue->stream);
+        for (auto& t : complete_be_tasks) finish_task(t, t->end);
+    }
+}
+
+// ---------------------------------------------------------------- best-effort execution
+// Incremental launch with a real-time check between launches, completion by
+// polling the stream (scheduler.cpp:685-740).
+void REEFScheduler::execute_be_task(std::shared_ptr<Task>& task, std::shared_ptr<TaskQueue>& tqueue) {
+    switch ((TaskState)task->state.load()) {
+        case TaskState::Finish: return;
+        case TaskState::Executing: {
+            if (executor::GPUStreamEmpty(tqueue->stream)) {
+                task->kernel_offset = 0;
+                task->block_offset = 0;
+                finish_task(task, Clock::now());
+            }
+            return;
+        }
+        case TaskState::Init:
+        case TaskState::Waiting: {
+            auto& exe = task->model->executor;
+            const int num_kernels = (int)exe.num_kernels();
+            if (task->state.load() == TaskState::Init && task->start.time_since_epoch().count() == 0)
+                task->start = Clock::now();
+            if (preempted) {
+                reset_preempt_flag_async();
+                preempted = false;
+                reef_hal_stream_sync(preempt_stream);
+            }
+            if (task->kernel_offset >= num_kernels) {
+                task->kernel_offset = 0;
+                task->block_offset = 0;
+                finish_task(task, Clock::now());
+                return;
+            }
+            task->state.store(TaskState::Executing);
+            task->block_offset = 0;
+            for (int i = task->kernel_offset; i < num_kernels; i++) {
+                exe.launch_preempt_kernel(i, tqueue->stream);
+                task->launch_offset = i;
+                if (!rt_queue->empty() && (mode == ScheduleMode::REEF || mode == ScheduleMode::Reset))
+                    return;  // preempt during launch
+            }
+            return;
+        }
+    }
+}
+
+}  // namespace server
+}  // namespace reef

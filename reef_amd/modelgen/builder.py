@@ -58,6 +58,9 @@ class GraphBuilder:
         self.kernel_bytes = []         # algorithmic bytes per kernel call
         self.kernel_est_us = []
         self._np = 0
+        # "symbol#instance" names give every kernel call its own profile entry
+        # (the profile is keyed by kernel name, model.cpp:57-80).
+        self.unique_names = True
 
     # ------------------------------------------------------------ storages
     def _storage(self, name, size, stype="float32"):
@@ -96,7 +99,7 @@ class GraphBuilder:
     # ------------------------------------------------------------ kernels
     def _emit(self, name, tasks, args, attrs, op, flops=0, nbytes=0, est_us=1.0, block=(WG, 1, 1)):
         self.kernels.append({
-            "name": name,
+            "name": "%s#%d" % (name, len(self.kernels)) if self.unique_names else name,
             "launch_params": [int(tasks), 1, 1, block[0], block[1], block[2]],
             "args": [int(a) for a in args],
             "attrs": [int(a) for a in attrs],
@@ -331,8 +334,9 @@ class GraphBuilder:
         shared = {}
         for k in self.kernels:
             n = k["name"]
-            if n.startswith("reef_conv2d_") or n.startswith("reef_gemm_"):
-                shared[n] = tiling.lds_bytes(n.split("_")[-1])
+            sym = n.split("#")[0]
+            if sym.startswith("reef_conv2d_") or sym.startswith("reef_gemm_"):
+                shared[n] = tiling.lds_bytes(sym.split("_")[-1])
             else:
                 shared[n] = 4   # the reference's floor (generate_final_schedule.py:117-143)
         return {"storage": self.storage, "kernels": self.kernels, "args": self.graph_args,

@@ -87,6 +87,7 @@ def mocked_kernel(name="mocked_kernel"):
     """The reference's mocked model (resource/mocked_kernel/mocked_kernel.json):
     temp = b + a[t]; output = temp[t] * c."""
     g = GraphBuilder(name)
+    g.unique_names = False   # keep the reference's kernel names and profile keys
     a = g.input("a", (8192,))
     b = g.input("b", (8192,))
     temp = g.temp((8192,), "temp")

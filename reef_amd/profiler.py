@@ -1,0 +1,50 @@
+"""Per-kernel latency profiles for a model directory, measured on the device.
+
+``<model>.profile.json`` drives dynamic kernel padding: ``total_latency`` is the
+solo duration of a kernel call and ``latency[j]`` the duration of one round of
+``(j + 1) * num_cus`` workgroups, i.e. at occupancy ``j + 1``
+(consumed in src/reef/server/scheduler.cpp:509,565-572,589-590).  The reference
+ships profiles made by a ``profiler`` binary that is not in its repository
+(resource/Makefile:32-36); this module is the equivalent for gfx950.
+All values are integer microseconds, at least 1.
+"""
+import json
+import math
+import os
+
+from . import binding as B
+
+
+def measure_profile(model_dir, name, iters=10, warmup=2, levels=8):
+    exe = B.Executor.from_dir(model_dir, name, B.HYBRID)
+    num_cus = B.lib().reef_gpuconfig_num_cus()
+    model = json.load(open(os.path.join(model_dir, name + ".json")))
+    kl = {}
+    for i, k in enumerate(model["kernels"]):
+        info = exe.kernel_info(i)
+        blocks = info["block_num"]
+        total = exe.time_kernel_dkp(i, info["min_occupancy"], blocks, warmup, iters)
+        max_occ = B.lib().reef_gpuconfig_calculate_occupancy(info["lds"], info["vgprs"], info["sgprs"],
+                                                             info["scratch"], 256)
+        lat = []
+        for j in range(min(levels, max(max_occ, 1))):
+            us = exe.time_kernel_dkp(i, j + 1, min(blocks, (j + 1) * num_cus), warmup, iters)
+            lat.append(max(1, int(math.ceil(us))))
+            if (j + 1) * num_cus >= blocks:
+                # more layers cannot hold more of this kernel's workgroups
+                lat += [lat[-1]] * (min(levels, max(max_occ, 1)) - len(lat))
+                break
+        e = kl.setdefault(k["name"], {"total_latency": 0, "latency": lat})
+        e["total_latency"] = max(e["total_latency"], max(1, int(math.ceil(total))))
+        e["latency"] = [max(a, b) for a, b in zip(e["latency"], lat)]
+    lat_us, _ = exe.time_model(B.RUN_DEFAULT, 3, 10)
+    prof = {"model_latency": int(math.ceil(float(lat_us.mean()))), "kernel_latency": kl}
+    exe.close()
+    return prof
+
+
+def write_profile(model_dir, name, **kw):
+    prof = measure_profile(model_dir, name, **kw)
+    with open(os.path.join(model_dir, name + ".profile.json"), "w") as f:
+        json.dump(prof, f, separators=(",", ":"))
+    return prof
