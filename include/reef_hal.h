@@ -55,6 +55,7 @@ typedef struct reef_device_info {
     int lds_bytes_per_cu;   /* 163840 */
     int lds_granule;        /* 1280 */
     int max_wg_per_cu;      /* 32 */
+    int max_threads_per_cu; /* 2048 */
     int clock_khz;
     char arch[32];          /* "gfx950" */
 } reef_device_info;

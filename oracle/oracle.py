@@ -278,7 +278,7 @@ class GraphOracle:
                 # of the workspace and leaves the other slots zero, which the
                 # ordered reduce then folds to the same mathematical result.
                 ws = P[2].view(np.float32)
-                ws[:] = 0
+                ws[:split_k * Cout * Ho * Wo] = 0
                 out = conv2d(P[0][:Cin * H * W].reshape(Cin, H, W),
                              P[1][:Cout * Cin * kh * kw].reshape(Cout, Cin, kh, kw),
                              stride=(sh, sw), pad=(ph, pw), acc64=acc64)

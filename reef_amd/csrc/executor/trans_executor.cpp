@@ -57,6 +57,10 @@ Status TransExecutor::init_rt_executor(const char* json_file_path, GPUModule_t m
         const uint32_t* lp = ki.launch_params;
         ka.kernel = kernel_funcs[i];
         ka.op = op_from_name(kernel_symbol(ki.name));
+        int tile = -1;
+        if (ka.op == REEF_OP_CONV2D && ki.attrs.size() > REEF_CONV_TILE) tile = ki.attrs[REEF_CONV_TILE];
+        if (ka.op == REEF_OP_GEMM && ki.attrs.size() > REEF_GEMM_TILE) tile = ki.attrs[REEF_GEMM_TILE];
+        ka.proxy_level = proxy_level(ka.op, tile);
         ka.task_dim = dim3u(lp[0], lp[1], lp[2]);
         ka.thread_dim = dim3u(lp[3], lp[4], lp[5]);
         ka.block_num = (int)ka.task_dim.count();
@@ -73,15 +77,11 @@ Status TransExecutor::init_rt_executor(const char* json_file_path, GPUModule_t m
 
     // proxies: one per occupancy class that the code object provides
     proxy_kernels.clear();
-    for (int i = 1; i <= 8; i++) {
+    for (int level = 0; level < kNumProxyLevels; level++) {
         GPUFunction_t f;
-        const std::string name = REEF_PROXY_KERNEL_PREFIX() + std::to_string(i);
-        if (reef_hal_module_get_function(module, name.c_str(), &f) != 0) break;
+        const std::string name = REEF_PROXY_KERNEL_PREFIX() + std::to_string(proxy_class_of_level(level));
+        GPU_RETURN_STATUS(reef_hal_module_get_function(module, name.c_str(), &f));
         proxy_kernels.push_back(f);
-    }
-    if (proxy_kernels.empty()) {
-        REEF_LOG_ERROR("code object has no %s1 proxy kernel", REEF_PROXY_KERNEL_PREFIX().c_str());
-        return Status::Fail;
     }
     GPUConfig::KernelResource kr;
     RETURN_STATUS(GPUConfig::get_kernel_resource(proxy_kernels[0], kr));
@@ -142,10 +142,25 @@ int TransExecutor::occupancy_class(const GPUConfig::KernelResource& kr) {
     return std::max(1, std::min(8, 512 / v));
 }
 
-GPUFunction_t TransExecutor::get_proxy_kernel(const GPUConfig::KernelResource& kr) {
-    int cls = occupancy_class(kr);
-    if (cls > (int)proxy_kernels.size()) cls = (int)proxy_kernels.size();
-    return proxy_kernels[cls - 1];
+int TransExecutor::proxy_class_of_level(int level) {
+    static const int cls[kNumProxyLevels] = {8, 4, 3, 2};
+    return cls[std::max(0, std::min(level, kNumProxyLevels - 1))];
+}
+
+// Which proxy holds the body of (op, tile): the bandwidth-bound ops are in every
+// proxy, the matrix-core tiles only in the classes whose register budget fits them.
+int TransExecutor::proxy_level(int op, int tile) {
+    if (op == REEF_OP_CONV2D) {
+        if (tile == REEF_TILE_64x64 || tile == REEF_TILE_128x32 || tile == REEF_TILE_32x128) return 1;
+        if (tile == REEF_TILE_128x64 || tile == REEF_TILE_64x128) return 2;
+        return 3;
+    }
+    if (op == REEF_OP_GEMM) return (tile == REEF_TILE_64x64 || tile == REEF_TILE_32x128) ? 2 : 3;
+    return 0;
+}
+
+GPUFunction_t TransExecutor::get_proxy_kernel(int level) {
+    return proxy_kernels[std::max(0, std::min(level, (int)proxy_kernels.size() - 1))];
 }
 
 }  // namespace executor

@@ -25,6 +25,7 @@ public:
     public:
         GPUFunction_t kernel;
         int op;                 // REEF_OP_* of this call (replaces funcion_pointer)
+        int proxy_level;        // smallest merge_framework class that contains this op
         dim3u task_dim;
         dim3u thread_dim;
         int block_num;
@@ -43,14 +44,19 @@ public:
 
     const std::vector<KernelArg>& kernel_args() const { return trans_args; }
     Status launch_kernel_dkp(int kernel_offset, int layers, int task_num, GPUStream_t stream);
-    // Occupancy class 1..8 (waves per SIMD) a merged launch needs
-    // (trans_executor.cpp:175-199 picks among 10 gfx906 classes).
+    // Waves per SIMD a register count allows on gfx950
+    // (trans_executor.cpp:175-199 picks among 10 gfx906 classes the same way).
     static int occupancy_class(const GPUConfig::KernelResource& kr);
+    // The code object carries one proxy per occupancy class that matters for
+    // this kernel set: merge_framework_8 / _4 / _3 / _2 = levels 0..3.
+    static constexpr int kNumProxyLevels = 4;
+    static int proxy_class_of_level(int level);
+    static int proxy_level(int op, int tile);
 
 protected:
     Status init_rt_executor(const char* json_file_path, GPUModule_t module);
     virtual Status launch_kernel(int kernel_offset, GPUStream_t stream) override;
-    GPUFunction_t get_proxy_kernel(const GPUConfig::KernelResource& kr);
+    GPUFunction_t get_proxy_kernel(int level);
     void fill_side(ReefDkpSide& side, int kernel_offset, int layers, int task_num, int task_offset) const;
 
 protected:

@@ -15,8 +15,8 @@ namespace reef {
 namespace hal {
 
 struct KernelMeta {
-    int vgprs = 0;    // arch VGPRs
-    int agprs = 0;    // accumulation VGPRs
+    int vgprs = 0;    // unified register count: arch VGPRs (rounded to 4) + AGPRs
+    int agprs = 0;    // accumulation VGPRs, included in vgprs
     int sgprs = 0;
     int lds = 0;      // static group segment bytes
     int scratch = 0;  // private segment bytes per lane

@@ -104,6 +104,8 @@ int reef_hal_occupancy(const reef_kernel_resource* res, int block_threads, int d
         blocks = std::min(blocks, di.lds_bytes_per_cu / need);
     }
     blocks = std::min(blocks, di.max_wg_per_cu);
+    if (di.max_threads_per_cu > 0)
+        blocks = std::min(blocks, di.max_threads_per_cu / (waves_per_wg * 64));
     *blocks_per_cu = std::max(blocks, 0);
     return 0;
 }

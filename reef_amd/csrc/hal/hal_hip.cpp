@@ -87,6 +87,7 @@ int h_device_info(reef_device_info* out) {
     out->lds_bytes_per_cu = 160 * 1024;
     out->lds_granule = 1280;
     out->max_wg_per_cu = 32;
+    out->max_threads_per_cu = 2048;
     out->clock_khz = p.clockRate;
     std::strncpy(out->arch, p.gcnArchName, sizeof(out->arch) - 1);
     if (char* c = std::strchr(out->arch, ':')) *c = 0;
@@ -135,7 +136,9 @@ int h_function_resource(reef_function_t f, reef_kernel_resource* out) {
         return 1;
     }
     out->shared_memory = f->meta.lds;
-    out->vgprs = (f->meta.vgprs + 3) / 4 * 4 + f->meta.agprs;
+    // On gfx90a and later .vgpr_count is already the unified total (arch VGPRs
+    // rounded to 4, plus AGPRs).
+    out->vgprs = f->meta.vgprs;
     out->sgprs = f->meta.sgprs;
     out->stack_size = f->meta.scratch;
     return 0;

@@ -77,6 +77,16 @@ struct OpMocked {
     }
 };
 
+// The launch arguments are read in place from the kernarg segment (constant
+// address space, scalar loads).  Going through the by-value parameter instead
+// makes the compiler copy the structs to scratch as soon as a side or an
+// optional-operand slot is selected at run time.
+template <class T>
+__device__ __forceinline__ const T& kernarg_at(int byte_offset) {
+    const char* base = (const char*)__builtin_amdgcn_kernarg_segment_ptr();
+    return *(const T*)(base + byte_offset);
+}
+
 #if REEF_FLAVOUR == 2
 // Side selection and first task of this workgroup.  Returns false when the
 // workgroup has nothing to do.
@@ -115,14 +125,14 @@ __device__ __forceinline__ bool dkp_walk(const ReefDkpArgs& a, DkpWalk& w) {
 // ---- entry generators ---------------------------------------------------------
 #if REEF_FLAVOUR == 0
 #define REEF_ENTRY(NAME, OP)                                                          \
-    extern "C" __global__ void __launch_bounds__(REEF_WG_THREADS) NAME(ReefOpDesc d) { \
+    extern "C" __global__ void __launch_bounds__(REEF_WG_THREADS) NAME(ReefOpDesc) {  \
         __shared__ __align__(16) char smem[OP::LDS > 0 ? OP::LDS : 16];               \
-        OP::run(d, (int)blockIdx.x, smem, NoPoll{});                                  \
+        OP::run(kernarg_at<ReefOpDesc>(0), (int)blockIdx.x, smem, NoPoll{});          \
     }
 #elif REEF_FLAVOUR == 1
 #define REEF_ENTRY(NAME, OP)                                                              \
     extern "C" __global__ void __launch_bounds__(REEF_WG_THREADS)                         \
-    NAME(int* preempted, int* task_slot, ReefOpDesc d) {                                  \
+    NAME(int* preempted, int* task_slot, ReefOpDesc) {                                    \
         __shared__ __align__(16) char smem[OP::LDS > 0 ? OP::LDS : 16];                   \
         __shared__ int s_pre;                                                             \
         const int t = threadIdx.x + threadIdx.y * blockDim.x + threadIdx.z * blockDim.x * blockDim.y; \
@@ -130,25 +140,20 @@ __device__ __forceinline__ bool dkp_walk(const ReefDkpArgs& a, DkpWalk& w) {
         if (t == 0) s_pre = poll.load();                                                  \
         __syncthreads();                                                                  \
         if (s_pre) return;                                                                \
-        const bool done = OP::run(d, (int)blockIdx.x, smem, poll);                        \
+        const bool done = OP::run(kernarg_at<ReefOpDesc>(16), (int)blockIdx.x, smem, poll); \
         if (done && t == 0) atomicAdd(task_slot, 1);                                      \
     }
 #else
 #define REEF_ENTRY(NAME, OP)                                                           \
-    extern "C" __global__ void __launch_bounds__(REEF_WG_THREADS) NAME(ReefDkpArgs a) { \
+    extern "C" __global__ void __launch_bounds__(REEF_WG_THREADS) NAME(ReefDkpArgs) {  \
         __shared__ __align__(16) char smem[OP::LDS > 0 ? OP::LDS : 16];                \
+        const ReefDkpArgs& a = kernarg_at<ReefDkpArgs>(0);                             \
         DkpWalk w;                                                                     \
         if (!dkp_walk(a, w)) return;                                                   \
-        if (w.right) {                                                                 \
-            for (int i = w.idx; i < w.end; i += w.step) {                              \
-                OP::run(a.r.desc, i, smem, NoPoll{});                                  \
-                __syncthreads();                                                       \
-            }                                                                          \
-        } else {                                                                       \
-            for (int i = w.idx; i < w.end; i += w.step) {                              \
-                OP::run(a.l.desc, i, smem, NoPoll{});                                  \
-                __syncthreads();                                                       \
-            }                                                                          \
+        const ReefDkpSide& side = w.right ? a.r : a.l;                                 \
+        for (int i = w.idx; i < w.end; i += w.step) {                                  \
+            OP::run(side.desc, i, smem, NoPoll{});                                     \
+            __syncthreads();                                                           \
         }                                                                              \
     }
 #endif
@@ -180,31 +185,44 @@ REEF_ENTRY(multiply, OpMocked<true>)
 #if REEF_FLAVOUR == 2
 // ---- merge_framework_<n>: two different ops in one launch ------------------------
 // The reference's proxies jump to a device function pointer per side
-// (script/transform_kernel.py:689-718).  Here the side carries an op id and the
-// proxy switches into the inlined body; LDS is dynamic (the host passes the
-// larger of the two sides' needs, as src/reef/server/scheduler.cpp:643-649 does).
+// (script/transform_kernel.py:689-718) and exist in ten variants whose register
+// budgets are patched to the gfx906 occupancy classes
+// (script/replace_register_usage.py:33-59).  Here the side carries an op id and
+// the proxy switches into the inlined body; the variants are the gfx950
+// occupancy classes that matter for this kernel set, <n> = wavefronts per SIMD:
+//   merge_framework_8  bandwidth-bound ops only                      (<= 64 registers)
+//   merge_framework_4  + conv tiles 64x64 / 128x32 / 32x128            (<= 128)
+//   merge_framework_3  + conv tiles 128x64 / 64x128, gemm 64x64 / 32x128 (<= 168)
+//   merge_framework_2  + the 128x128 tiles                             (<= 256)
+// LDS is dynamic (the host passes the larger of the two sides' needs, as
+// src/reef/server/scheduler.cpp:643-649 does).
 namespace {
+template <int LEVEL>
 __device__ __forceinline__ void run_op(const ReefDkpSide& s, int task, char* smem) {
     const ReefOpDesc& d = s.desc;
     const NoPoll np{};
     switch (s.op) {
         case REEF_OP_CONV2D:
-            switch (d.attr[REEF_CONV_TILE]) {
-                case REEF_TILE_128x128: OpConv<Tile128x128>::run(d, task, smem, np); break;
-                case REEF_TILE_128x64: OpConv<Tile128x64>::run(d, task, smem, np); break;
-                case REEF_TILE_64x64: OpConv<Tile64x64>::run(d, task, smem, np); break;
-                case REEF_TILE_128x32: OpConv<Tile128x32>::run(d, task, smem, np); break;
-                case REEF_TILE_32x128: OpConv<Tile32x128>::run(d, task, smem, np); break;
-                case REEF_TILE_64x128: OpConv<Tile64x128>::run(d, task, smem, np); break;
-                default: break;
+            if (LEVEL >= 1) {
+                switch (d.attr[REEF_CONV_TILE]) {
+                    case REEF_TILE_64x64: OpConv<Tile64x64>::run(d, task, smem, np); break;
+                    case REEF_TILE_128x32: OpConv<Tile128x32>::run(d, task, smem, np); break;
+                    case REEF_TILE_32x128: OpConv<Tile32x128>::run(d, task, smem, np); break;
+                    case REEF_TILE_128x64: if (LEVEL >= 2) OpConv<Tile128x64>::run(d, task, smem, np); break;
+                    case REEF_TILE_64x128: if (LEVEL >= 2) OpConv<Tile64x128>::run(d, task, smem, np); break;
+                    case REEF_TILE_128x128: if (LEVEL >= 3) OpConv<Tile128x128>::run(d, task, smem, np); break;
+                    default: break;
+                }
             }
             break;
         case REEF_OP_GEMM:
-            switch (d.attr[REEF_GEMM_TILE]) {
-                case REEF_TILE_128x128: OpGemm<Tile128x128>::run(d, task, smem, np); break;
-                case REEF_TILE_64x64: OpGemm<Tile64x64>::run(d, task, smem, np); break;
-                case REEF_TILE_32x128: OpGemm<Tile32x128>::run(d, task, smem, np); break;
-                default: break;
+            if (LEVEL >= 2) {
+                switch (d.attr[REEF_GEMM_TILE]) {
+                    case REEF_TILE_64x64: OpGemm<Tile64x64>::run(d, task, smem, np); break;
+                    case REEF_TILE_32x128: OpGemm<Tile32x128>::run(d, task, smem, np); break;
+                    case REEF_TILE_128x128: if (LEVEL >= 3) OpGemm<Tile128x128>::run(d, task, smem, np); break;
+                    default: break;
+                }
             }
             break;
         case REEF_OP_SPLITK_REDUCE: splitk_reduce_body(d, task); break;
@@ -226,23 +244,23 @@ __device__ __forceinline__ void run_op(const ReefDkpSide& s, int task, char* sme
 }
 }  // namespace
 
-#define REEF_PROXY(N)                                                                       \
-    extern "C" __global__ void __launch_bounds__(REEF_WG_THREADS) merge_framework_##N(ReefDkpArgs a) { \
+#define REEF_PROXY(N, LEVEL)                                                                \
+    extern "C" __global__ void __launch_bounds__(REEF_WG_THREADS)                           \
+    __attribute__((amdgpu_waves_per_eu(N, N))) merge_framework_##N(ReefDkpArgs) {           \
         extern __shared__ __align__(16) char dyn_smem[];                                    \
+        const ReefDkpArgs& a = kernarg_at<ReefDkpArgs>(0);                                  \
         DkpWalk w;                                                                          \
         if (!dkp_walk(a, w)) return;                                                        \
-        if (w.right) {                                                                      \
-            for (int i = w.idx; i < w.end; i += w.step) {                                   \
-                run_op(a.r, i, dyn_smem);                                                   \
-                __syncthreads();                                                            \
-                if (a.task_slot_r && threadIdx.x == 0) atomicAdd(a.task_slot_r, 1);         \
-            }                                                                               \
-        } else {                                                                            \
-            for (int i = w.idx; i < w.end; i += w.step) {                                   \
-                run_op(a.l, i, dyn_smem);                                                   \
-                __syncthreads();                                                            \
-            }                                                                               \
+        const ReefDkpSide& side = w.right ? a.r : a.l;                                      \
+        int* slot = w.right ? a.task_slot_r : nullptr;                                      \
+        for (int i = w.idx; i < w.end; i += w.step) {                                       \
+            run_op<LEVEL>(side, i, dyn_smem);                                               \
+            __syncthreads();                                                                \
+            if (slot && threadIdx.x == 0) atomicAdd(slot, 1);                               \
         }                                                                                   \
     }
-REEF_PROXY(1)
+REEF_PROXY(8, 0)
+REEF_PROXY(4, 1)
+REEF_PROXY(3, 2)
+REEF_PROXY(2, 3)
 #endif

@@ -454,8 +454,9 @@ void REEFScheduler::dynamic_kernel_padding(std::shared_ptr<Task>& rt_task) {
     const int num_xcds = (int)GPUConfig::get_num_xcds();
     std::vector<std::shared_ptr<Task>> complete_be_tasks;
     TimePoint current_time_point = Clock::now();
-    GPUConfig::KernelResource proxy_res{};
-    GPUConfig::get_kernel_resource(rt_exe.proxy_kernels[0], proxy_res);
+    GPUConfig::KernelResource proxy_res[TransExecutor::kNumProxyLevels];
+    for (int l = 0; l < TransExecutor::kNumProxyLevels; l++)
+        GPUConfig::get_kernel_resource(rt_exe.get_proxy_kernel(l), proxy_res[l]);
 
     const int n_rt = (int)rt_exe.num_kernels();
     for (int i = 0; i < n_rt; i++) {
@@ -471,7 +472,10 @@ void REEFScheduler::dynamic_kernel_padding(std::shared_ptr<Task>& rt_task) {
             HybridExecutor& be_exe = cand->model->executor;
             if (cand->kernel_offset >= (int)be_exe.num_kernels()) continue;
             const TransExecutor::KernelArg& ka = be_exe.trans_args[cand->kernel_offset];
-            PadDecision d = decide_padding(rt_args, ka, cand->block_offset, proxy_res, num_cus, num_xcds);
+            // the proxy class that holds both bodies sets the register budget of the launch
+            const int level = std::max(rt_args.proxy_level, ka.proxy_level);
+            PadDecision d = decide_padding(rt_args, ka, cand->block_offset, proxy_res[level], num_cus,
+                                           num_xcds);
             if (!d.merge) continue;
             dec = d;
             be_task = cand;
@@ -498,7 +502,8 @@ void REEFScheduler::dynamic_kernel_padding(std::shared_ptr<Task>& rt_task) {
             a.num_xcds = num_xcds;
             a.task_slot_r = nullptr;
             if (be_task->start.time_since_epoch().count() == 0) be_task->start = current_time_point;
-            executor::GPUFunction_t proxy = rt_exe.get_proxy_kernel(dec.resource);
+            executor::GPUFunction_t proxy =
+                rt_exe.get_proxy_kernel(std::max(rt_args.proxy_level, be_args->proxy_level));
             const uint32_t grid[3] = {(uint32_t)(dec.final_occupancy * num_cus), 1, 1};
             const uint32_t block[3] = {(uint32_t)dec.merged_block_size, 1, 1};
             reef_hal_launch(proxy, grid, block, (uint32_t)dec.resource.shared_memory, rt_queue->stream,

@@ -1,0 +1,216 @@
+"""Model resource formats: the product's parsers on the files the reference's own
+parser tests use (src/reef/test/test.cpp:59-91), the oracle's Python reader on the
+same files, and round trips through both writers."""
+import array
+import ctypes
+import json
+import os
+import re
+import struct
+
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from reef_amd import binding as B
+from reef_amd.modelgen import builder as MB
+
+L = B.lib()
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def model_summary(path):
+    v = [ctypes.c_int() for _ in range(4)]
+    st = L.reef_model_parse_summary(path.encode(), *[ctypes.byref(x) for x in v])
+    return st, [x.value for x in v]
+
+
+def profile_summary(path):
+    v = [ctypes.c_int() for _ in range(4)]
+    st = L.reef_profile_parse_summary(path.encode(), *[ctypes.byref(x) for x in v])
+    return st, [x.value for x in v]
+
+
+@pytest.mark.parametrize("name,n_storage,n_kernels", [("mocked_kernel", 5, 2), ("resnet152", 317, 207),
+                                                      ("resnet18", None, None), ("bert", None, None)])
+def test_parse_reference_graph_json(golden_dir, name, n_storage, n_kernels):
+    path = os.path.join(golden_dir, name + ".json")
+    ref = json.load(open(path))
+    st, (ns, nk, na, nsh) = model_summary(path)
+    assert st == 0
+    assert (ns, nk, na, nsh) == (len(ref["storage"]), len(ref["kernels"]), len(ref["args"]),
+                                 len(ref["shared_memory"]))
+    assert nk > 0                                  # parser.parse_model, test.cpp:59-65
+    if n_storage is not None:
+        assert (ns, nk) == (n_storage, n_kernels)
+    # the oracle's graph loader accepts the same file
+    orc = O.GraphOracle(ref)
+    assert len(orc.storage) == ns
+    if name == "resnet152":
+        assert orc.storage[0].size == 12288        # 3 x 64 x 64 input
+    if name == "bert":
+        assert orc.storage[0].dtype == np.int64 and ref["storage"][0]["stype"] == "int64"
+
+
+def test_parse_reference_profiles(golden_dir):
+    st, (ml, nk, mn, cnt) = profile_summary(os.path.join(golden_dir, "resnet18.profile.json"))
+    assert st == 0 and nk == 54 and mn > 0 and cnt > 0          # parser.parse_profile, test.cpp:79-91
+    st, (ml, nk, mn, cnt) = profile_summary(os.path.join(golden_dir, "mocked_kernel.profile.json"))
+    assert (st, ml, nk, mn, cnt) == (0, 30, 2, 14, 32)
+    st, (ml, nk, _, _) = profile_summary(os.path.join(golden_dir, "resnet152.profile.json"))
+    assert (st, ml) == (0, 13233) and nk == len(json.load(open(os.path.join(golden_dir, "resnet152.profile.json")))["kernel_latency"])
+
+
+def test_profile_to_json_round_trip(golden_dir, tmp_path):
+    for name in ("mocked_kernel", "resnet18", "resnet152"):
+        path = os.path.join(golden_dir, name + ".profile.json")
+        buf = ctypes.create_string_buffer(1 << 16)
+        assert L.reef_profile_roundtrip(path.encode(), buf, ctypes.c_size_t(len(buf))) == 0
+        assert json.loads(buf.value.decode()) == json.load(open(path))
+        # what to_json writes parses again to the same summary
+        p2 = tmp_path / (name + ".json")
+        p2.write_bytes(buf.value)
+        assert profile_summary(str(p2)) == profile_summary(path)
+
+
+def reference_style_param_file(path, params):
+    """Byte-for-byte what script/tvm_generate_model.py:66-76 (dump_params) writes."""
+    with open(path, "wb") as f:
+        f.write(bytes("TVM_MODEL_PARAMS\0", "ascii"))
+        f.write(array.array('Q', [len(params)]).tobytes())
+        for k, v in params.items():
+            p = array.array('f', v.flatten().tolist())
+            f.write(bytes(k, "ascii"))
+            f.write(bytes("\0", "ascii"))
+            f.write(array.array('Q', [len(p)]).tobytes())
+            f.write(p.tobytes())
+
+
+def param_summary(path, key):
+    n, klen = ctypes.c_uint64(), ctypes.c_uint64()
+    first, last = ctypes.c_float(), ctypes.c_float()
+    st = L.reef_param_parse_summary(path.encode(), key.encode(), ctypes.byref(n), ctypes.byref(klen),
+                                    ctypes.byref(first), ctypes.byref(last))
+    return st, n.value, klen.value, first.value, last.value
+
+
+def test_param_format_both_writers_both_readers(tmp_path):
+    rng = np.random.default_rng(3)
+    params = {"p0": rng.standard_normal((8, 3, 3, 3)).astype(np.float32),
+              "p22": rng.standard_normal(294912).astype(np.float32),   # the size test.cpp:76 expects of p22
+              "a_rather_long_parameter_name_1": np.arange(5, dtype=np.float32)}
+    ref_file, own_file = str(tmp_path / "ref.param"), str(tmp_path / "own.param")
+    reference_style_param_file(ref_file, params)
+    MB.write_params(own_file, [(k, v) for k, v in params.items()])
+    assert open(ref_file, "rb").read() == open(own_file, "rb").read()
+    for key, arr in params.items():
+        st, n, klen, first, last = param_summary(ref_file, key)
+        assert (st, n, klen) == (0, 3, arr.size)
+        assert first == arr.reshape(-1)[0] and last == arr.reshape(-1)[-1]
+    got = O.read_params(ref_file)
+    assert set(got) == set(params)
+    for k in params:
+        np.testing.assert_array_equal(got[k], params[k].reshape(-1))
+    assert param_summary(ref_file, "nope")[0] == 2
+
+
+def test_param_parser_rejects_malformed(tmp_path):
+    bad = tmp_path / "bad.param"
+    bad.write_bytes(b"NOT_A_PARAM_FILE\0" + struct.pack("<Q", 1))
+    assert param_summary(str(bad), "p0")[0] == 2
+    trunc = tmp_path / "trunc.param"
+    trunc.write_bytes(b"TVM_MODEL_PARAMS\0" + struct.pack("<Q", 1) + b"p0\0" + struct.pack("<Q", 10) + b"\0" * 8)
+    assert param_summary(str(trunc), "p0")[0] == 2
+    empty = tmp_path / "empty.param"
+    empty.write_bytes(b"TVM_MODEL_PARAMS\0" + struct.pack("<Q", 0))   # the reference asserts count != 0
+    assert param_summary(str(empty), "p0")[0] == 2
+    assert param_summary(str(tmp_path / "missing.param"), "p0")[0] == 2
+
+
+def test_json_subset_and_superset(tmp_path):
+    """Single-quoted strings and bare decimals as the reference's tokenizer takes them
+    (src/reef/util/json.cpp:39-74), plus standard JSON it rejects (true/false/null, exponents)."""
+    p = tmp_path / "m.json"
+    p.write_text("{'storage': [{'name': 'a', 'size': 4, 'stype': 'float32'}],\n"
+                 " \"kernels\": [{\"name\": \"add\", \"launch_params\": [1,1,1,4,8,4], \"args\": [0, 0, 0],"
+                 "  \"attrs\": [-3, 7], \"extra\": true, \"f\": 1.5e3, \"n\": null}],\n"
+                 " \"args\": [0], \"shared_memory\": {\"add\": 1024}}")
+    assert model_summary(str(p)) == (0, [1, 1, 1, 1])
+    for text in ("{", "{\"storage\": [}", "{\"storage\": [], \"kernels\": [{\"name\": \"k\", \"launch_params\": [1,2], \"args\": []}]}",
+                 "{\"storage\": [], \"kernels\": [{\"name\": \"k\", \"launch_params\": [1,1,1,1,1,1], \"args\": [3]}]}", "bogus"):
+        p.write_text(text)
+        assert model_summary(str(p))[0] == 2, text
+    assert model_summary(str(tmp_path / "missing.json"))[0] == 2
+
+
+def test_generated_model_is_reference_parsable_subset(tmp_path):
+    """Generated graph JSON holds only ints, strings, lists and dicts (what the reference's
+    parser accepts) and keeps its four top-level keys."""
+    from reef_amd.modelgen import nets
+    g = nets.resnet(18, image=(3, 32, 32), classes=8, name="t")
+    g.write(str(tmp_path), link_code_objects=False)
+    m = json.load(open(tmp_path / "t.json"))
+    assert set(m) == {"storage", "kernels", "args", "shared_memory"}
+
+    def walk(v):
+        if isinstance(v, dict):
+            assert all(isinstance(k, str) for k in v)
+            for x in v.values():
+                walk(x)
+        elif isinstance(v, list):
+            for x in v:
+                walk(x)
+        else:
+            assert isinstance(v, (int, str)) and not isinstance(v, bool), v
+    walk(m)
+    assert all(len(k["launch_params"]) == 6 for k in m["kernels"])
+    assert {s["stype"] for s in m["storage"]} <= {"float32", "int64", "byte", "uint1", "int32"}
+    st, (ns, nk, _, _) = model_summary(str(tmp_path / "t.json"))
+    assert (st, ns, nk) == (0, len(m["storage"]), len(m["kernels"]))
+    prof = json.load(open(tmp_path / "t.profile.json"))
+    assert set(prof["kernel_latency"]) == {k["name"] for k in m["kernels"]}
+
+
+def test_library_exports_every_declared_symbol():
+    """Every function declared in include/*.h is exported by libreef_amd.so."""
+    lib = B.lib()
+    declared = []
+    for h in ("reef_hal.h", "reef_c.h"):
+        text = open(os.path.join(ROOT, "include", h)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        text = re.sub(r"typedef struct reef_hal_backend \{.*?\} reef_hal_backend;", "", text, flags=re.S)
+        declared += re.findall(r"\b(reef_[a-z0-9_]+)\s*\(", text)
+    declared = sorted(set(declared))
+    assert len(declared) > 80
+    missing = [n for n in declared if not hasattr(lib, n)]
+    assert not missing, missing
+
+
+def test_code_object_metadata_reader():
+    """Kernel resources come from the code object's metadata note (host-only parse)."""
+    from reef_amd.paths import code_object
+    out = (ctypes.c_int * 6)()
+    for fl in ("raw", "be", "trans"):
+        co = code_object(fl).encode()
+        assert L.reef_code_object_kernel_meta(co, b"reef_conv2d_128x128", out) == 0
+        vg, ag, sg, lds, scratch, kernarg = list(out)
+        assert ag == 64 and 73744 <= lds <= 73744 + 16 and scratch == 0 and 64 + 40 <= vg <= 64 + 128
+        assert L.reef_code_object_kernel_meta(co, b"reef_eltwise", out) == 0
+        assert out[3] <= 16 and out[4] == 0
+        assert L.reef_code_object_kernel_meta(co, b"no_such_kernel", out) == 2
+    # kernarg block sizes: raw = ReefOpDesc (160 B), be = two pointers + desc
+    assert L.reef_code_object_kernel_meta(code_object("raw").encode(), b"reef_pool2d", out) == 0
+    assert out[5] == 160
+    assert L.reef_code_object_kernel_meta(code_object("be").encode(), b"reef_pool2d", out) == 0
+    assert out[5] >= 176           # + the compiler's hidden arguments
+    assert L.reef_code_object_kernel_meta(code_object("trans").encode(), b"reef_pool2d", out) == 0
+    assert out[5] == 376           # sizeof(ReefDkpArgs)
+    for cls, budget in ((8, 64), (4, 128), (3, 168), (2, 256)):
+        assert L.reef_code_object_kernel_meta(code_object("trans").encode(),
+                                              b"merge_framework_%d" % cls, out) == 0
+        assert out[4] == 0 and out[0] <= budget, "proxy class %d: no scratch, registers within budget" % cls
+    # no kernel of any flavour spills
+    for fl in ("raw", "be", "trans"):
+        for k in ("reef_conv2d_128x128", "reef_gemm_128x128", "reef_dense", "reef_layernorm", "add"):
+            assert L.reef_code_object_kernel_meta(code_object(fl).encode(), k.encode(), out) == 0
+            assert out[4] == 0, (fl, k)

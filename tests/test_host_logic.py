@@ -1,0 +1,217 @@
+"""Executors and scheduler on the recording backend (no GPU): argument binding,
+launch geometry per flavour, error codes, preemption rollback and idempotence,
+dynamic kernel padding bookkeeping.  The backend executes every completed
+"kernel" with the CPU oracle, so outputs are real."""
+import json
+import os
+import time
+
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from reef_amd import binding as B
+from reef_amd.modelgen import nets
+from tests.fakehal import FakeHal
+from tests.helpers import write_model
+
+THREE = np.full(8192, 3.0, np.float32)
+
+
+@pytest.fixture()
+def fake():
+    f = FakeHal().install()
+    yield f
+    f.remove()
+
+
+@pytest.fixture(scope="module")
+def small_dirs(tmp_path_factory):
+    out = {}
+    for g in (nets.mocked_kernel(), nets.resnet(18, image=(3, 32, 32), classes=16, name="tiny18")):
+        out[g.name] = (g, write_model(g, tmp_path_factory.mktemp(g.name)))
+    return out
+
+
+def oracle_output(g, d, x):
+    model = json.load(open(os.path.join(d, g.name + ".json")))
+    orc = O.GraphOracle(model, os.path.join(d, g.name + ".param"))
+    orc.set_input("data", x)
+    return orc.run().copy()
+
+
+@pytest.mark.parametrize("kind,pre", [(B.BASE, False), (B.TRANS, False), (B.HYBRID, False), (B.HYBRID, True)])
+def test_mocked_model_all_flavours(fake, small_dirs, kind, pre):
+    g, d = small_dirs["mocked_kernel"]
+    exe = B.Executor.from_dir(d, g.name, kind)
+    for n in "abc":
+        exe.set_input_checked(n, THREE)
+    exe.execute_preemptable() if pre else exe.execute()
+    np.testing.assert_array_equal(exe.get_output(), np.full(8192, 18.0, np.float32))
+    log = fake.log()
+    assert [e[0] for e in log] == ["add", "multiply"]
+    if kind == B.BASE or pre:
+        assert all(e[2] == 64 and e[3] == 128 for e in log)      # grid/block from the JSON
+    else:
+        assert all(e[2] == 256 * 1 and e[3] == 128 for e in log)  # num_cus * min_occupancy, flat block
+
+
+@pytest.mark.parametrize("kind,pre", [(B.BASE, False), (B.TRANS, False), (B.HYBRID, True)])
+def test_resnet_binding_matches_graph_oracle(fake, small_dirs, kind, pre):
+    g, d = small_dirs["tiny18"]
+    x = nets.image_input("t", (3, 32, 32))
+    exe = B.Executor.from_dir(d, g.name, kind)
+    exe.set_input_checked("data", x)
+    exe.execute_preemptable() if pre else exe.execute()
+    np.testing.assert_array_equal(exe.get_output(), oracle_output(g, d, x))
+    assert exe.num_kernels() == len(g.kernels) == len(fake.log())
+    if pre:
+        assert exe.read_task_slots() == [k["launch_params"][0] for k in g.kernels]
+
+
+def test_executor_error_codes(fake, small_dirs, tmp_path):
+    g, d = small_dirs["mocked_kernel"]
+    exe = B.Executor.from_dir(d, g.name, B.BASE)
+    assert exe.set_input("nope", THREE) == 2            # NotFound
+    assert exe.set_input("a", THREE[:100]) == 3         # OutOfRange: shorter than the storage
+    assert exe.get_data_size("output") == 8192 * 4
+    with pytest.raises(B.ReefError) as ei:
+        exe.get_output(10)                              # buffer too small -> Fail
+    assert ei.value.status == 1
+    with pytest.raises(B.ReefError) as ei:
+        exe.execute_to(99)
+    assert ei.value.status == 3
+    with pytest.raises(B.ReefError) as ei:
+        exe.execute_kernel(2)
+    assert ei.value.status == 3
+    with pytest.raises(B.ReefError) as ei:               # missing graph file
+        B.Executor(B.BASE).load(str(tmp_path / "none.json"), os.path.join(d, g.name + ".raw.co"))
+    assert ei.value.status == 2
+    with pytest.raises(B.ReefError) as ei:               # missing code object
+        B.Executor(B.BASE).load(os.path.join(d, g.name + ".json"), str(tmp_path / "none.co"))
+    assert ei.value.status == 1
+    fake.set_missing("multiply")
+    with pytest.raises(B.ReefError) as ei:               # symbol not in the code object
+        B.Executor.from_dir(d, g.name, B.BASE)
+    assert ei.value.status == 1
+
+
+def test_trans_needs_proxy_kernel(fake, small_dirs):
+    g, d = small_dirs["mocked_kernel"]
+    fake.set_missing("merge_framework_3")
+    with pytest.raises(B.ReefError):
+        B.Executor.from_dir(d, g.name, B.TRANS)
+
+
+def test_min_occupancy_and_kernel_info(fake, small_dirs):
+    g, d = small_dirs["tiny18"]
+    fake.set_kernel_resource("reef_eltwise", lds=0, vgprs=128, sgprs=32)
+    exe = B.Executor.from_dir(d, g.name, B.TRANS)
+    for i, k in enumerate(g.kernels):
+        info = exe.kernel_info(i)
+        blocks = k["launch_params"][0]
+        assert info["block_num"] == blocks
+        occ = B.lib().reef_gpuconfig_calculate_occupancy(info["lds"], info["vgprs"], info["sgprs"], 0, 256)
+        assert info["min_occupancy"] == max(1, min(-(-blocks // 256), occ))
+
+
+def run_scheduler_until(s, tid, timeout=20.0):
+    t0 = time.time()
+    while time.time() - t0 < timeout:
+        if s.task_info(tid)["state"] == B.STATE_FINISH:
+            return True
+        time.sleep(0.001)
+    return False
+
+
+@pytest.mark.parametrize("qtype", [B.QUEUE_RT, B.QUEUE_BE])
+@pytest.mark.parametrize("mode", [B.MODE_REEF, B.MODE_RESET, B.MODE_WAITPREEMPT, B.MODE_NOPREEMPT])
+def test_scheduler_single_task(fake, small_dirs, qtype, mode):
+    g, d = small_dirs["mocked_kernel"]
+    s = B.Scheduler(mode)
+    assert s.mode() == mode
+    s.run()
+    mid = s.load_model(d, g.name)
+    qid = s.create_queue(qtype)
+    assert s.bind_model_queue(qid, mid) == 0
+    for n in "abc":
+        assert s.set_input(mid, THREE, n) == 0
+    tid = s.new_task(mid)
+    assert s.wait_task(tid) == 0
+    np.testing.assert_array_equal(s.get_output(mid, 8192), np.full(8192, 18.0, np.float32))
+    assert s.wait_task(tid + 100) == 2       # NotFound
+    assert s.new_task_status(mid + 5) == 3   # OutOfRange
+    s.shutdown()
+
+
+def test_scheduler_preempt_rollback_and_idempotence(fake, small_dirs):
+    """A best-effort task is interrupted by a real-time task: queued launches are
+    dropped, in-flight kernels see the flag and skip, the task restarts from the
+    rolled-back kernel, and its output equals the uninterrupted result."""
+    gb, db = small_dirs["tiny18"]
+    gm, dm = small_dirs["mocked_kernel"]
+    x = nets.image_input("t", (3, 32, 32))
+    ref = oracle_output(gb, db, x)
+    fake.lib.fake_hal_set_auto_progress(1)
+    s = B.Scheduler(B.MODE_RESET)
+    s.run()
+    be_mid = s.load_model(db, gb.name)
+    rt_mid = s.load_model(dm, gm.name)
+    be_q, rt_q = s.create_queue(B.QUEUE_BE), s.create_queue(B.QUEUE_RT)
+    s.bind_model_queue(be_q, be_mid)
+    s.bind_model_queue(rt_q, rt_mid)
+    s.set_input(be_mid, x, "data")
+    for n in "abc":
+        s.set_input(rt_mid, THREE, n)
+    be_tid = s.new_task(be_mid)
+    t0 = time.time()
+    while fake.lib.fake_hal_completed() < 3 and time.time() - t0 < 10:
+        time.sleep(0.0002)
+    rt_tid = s.new_task(rt_mid)
+    assert s.wait_task(rt_tid) == 0 and s.wait_task(be_tid) == 0
+    np.testing.assert_array_equal(s.get_output(rt_mid, 8192), np.full(8192, 18.0, np.float32))
+    np.testing.assert_array_equal(s.get_output(be_mid, 16), ref)
+    be, rt = s.task_info(be_tid), s.task_info(rt_tid)
+    if be["preempted"]:
+        assert fake.lib.fake_hal_dropped() > 0 or fake.skipped > 0
+        assert rt["start"] >= be["start"] and be["end"] >= rt["end"]
+        assert s.preempt_times() == 1
+        # more launches than kernels: the tail was launched twice
+        assert fake.lib.fake_hal_launches() > len(gb.kernels) + 2
+    s.shutdown()
+    assert be["preempted"], "the real-time task arrived after the best-effort task had finished"
+
+
+def test_scheduler_dkp_pads_to_completion(fake, small_dirs):
+    """scheduler.mocked_kernel of the reference (src/reef/test/test.cpp:491-536):
+    best-effort mocked model + real-time network queued before run()."""
+    gr, dr = small_dirs["tiny18"]
+    gm, dm = small_dirs["mocked_kernel"]
+    x = nets.image_input("t", (3, 32, 32))
+    ref = oracle_output(gr, dr, x)
+    # profile: make every real-time kernel long enough to host the mocked kernels
+    prof = json.load(open(os.path.join(dr, gr.name + ".profile.json")))
+    for v in prof["kernel_latency"].values():
+        v["total_latency"] = 100
+    json.dump(prof, open(os.path.join(dr, gr.name + ".profile.json"), "w"))
+    s = B.Scheduler(B.MODE_REEF)
+    rt_mid = s.load_model(dr, gr.name)
+    be_mid = s.load_model(dm, gm.name)
+    rt_q, be_q = s.create_queue(B.QUEUE_RT), s.create_queue(B.QUEUE_BE)
+    s.bind_model_queue(rt_q, rt_mid)
+    s.bind_model_queue(be_q, be_mid)
+    s.set_input(rt_mid, x, "data")
+    for n in "abc":
+        s.set_input(be_mid, THREE, n)
+    be_tid = s.new_task(be_mid)
+    rt_tid = s.new_task(rt_mid)
+    s.run()
+    assert s.wait_task(be_tid) == 0 and s.wait_task(rt_tid) == 0
+    np.testing.assert_array_equal(s.get_output(rt_mid, 16), ref)
+    np.testing.assert_array_equal(s.get_output(be_mid, 8192), np.full(8192, 18.0, np.float32))
+    be = s.task_info(be_tid)
+    assert be["padded"] and be["padded_to_complete"] and not be["preempted"]
+    merged = [e for e in fake.log() if e[0].startswith("merge_framework_")]
+    assert len(merged) == s.padded_kernels() >= 2
+    assert s.avg_kernel_sel_latency() >= 0
+    s.shutdown()
