@@ -96,6 +96,7 @@ int reef_hal_memset(reef_devptr_t ptr, int byte, size_t bytes);
 int reef_hal_memcpy_h2d(reef_devptr_t dst, const void* src, size_t bytes);
 int reef_hal_memcpy_d2h(void* dst, reef_devptr_t src, size_t bytes);
 /* hipMemcpyHtoDAsync / hipMemcpyDtoHAsync     hybrid_executor.cpp:134,138; scheduler.cpp:353 */
+int reef_hal_memset_async(reef_devptr_t ptr, int byte, size_t bytes, reef_stream_t s);
 int reef_hal_memcpy_h2d_async(reef_devptr_t dst, const void* src, size_t bytes, reef_stream_t s);
 int reef_hal_memcpy_d2h_async(void* dst, reef_devptr_t src, size_t bytes, reef_stream_t s);
 
@@ -168,6 +169,7 @@ typedef struct reef_hal_backend {
     int (*event_record)(reef_event_t, reef_stream_t);
     int (*event_sync)(reef_event_t);
     int (*event_elapsed_us)(reef_event_t, reef_event_t, float*);
+    int (*memset_async)(reef_devptr_t, int, size_t, reef_stream_t);
 } reef_hal_backend;
 
 const reef_hal_backend* reef_hal_hip_backend(void);

@@ -49,7 +49,7 @@ extern "C" {
 #endif
 
 #define REEF_WG_THREADS 256
-#define REEF_MAX_PTRS 8
+#define REEF_MAX_PTRS 10
 #define REEF_MAX_ATTRS 24
 
 typedef struct ReefOpDesc {
@@ -128,10 +128,24 @@ enum {
 /* ---- reef_conv2d: fp32 implicit-GEMM convolution on MFMA (groups == 1) ----
  * GEMM view: out[M=Cout][N=Ho*Wo] = W[M][K=Cin*kh*kw] x im2col(in)[K][N].
  * ptr: in, W(OIHW), dst, then the optional operands in this order when their
- *      flag bit is set: bias, residual, scale, shift.
- *      dst is the output tensor when split_k == 1, else the split-K workspace
- *      [split_k][Cout][Ho*Wo] that reef_splitk_reduce folds in a fixed order
- *      (then the optional operands belong to the reduce launch instead).
+ *      flag bit is set: bias, residual, (scale, shift), (out2, shift2), (workspace, sync).
+ * Epilogue: v = acc (+residual) (+bias) (*scale + shift); out = act(v);
+ *           with REEF_F_DUAL also out2 = act2(act(v) + shift2[channel]).
+ * Split-K (split_k > 1), two forms:
+ *   plain : dst is the workspace [split_k][Cout][Ho*Wo]; every split stores its
+ *           partial tile and reef_splitk_reduce folds them (the optional operands
+ *           then belong to that launch).
+ *   REEF_F_FUSED_REDUCE : dst is the output; the workspace holds
+ *           [split_k][Cout][Ho*Wo] floats and the sync storage (one per model, named
+ *           "reef_sync", int32) holds one counter per output tile starting at
+ *           attr SYNC_OFF.  Every split stores its partial, then counts itself on the
+ *           tile's counter; the workgroup that arrives last adds the partials in
+ *           ascending split order, applies the epilogue and resets the counter.
+ *           The sum order is fixed, so the result does not depend on which
+ *           workgroup arrives last and equals the plain form bit for bit.
+ *           Counters are zero between complete runs of the kernel; after an
+ *           interrupted run the host clears the sync storage before the kernel is
+ *           run again (HybridExecutor::reset_sync_storage).
  * tasks = split_k * m_tiles * n_tiles;
  * task -> (split = task / (m_tiles*n_tiles), m_tile, n_tile), n fastest. */
 enum {
@@ -143,11 +157,15 @@ enum {
     REEF_CONV_SPLIT_K,   /* >= 1 */
     REEF_CONV_K_CHUNK,   /* K elements per split, multiple of the tile's BK */
     REEF_CONV_M_TILES, REEF_CONV_N_TILES,
+    REEF_CONV_ACT2,      /* activation of the second output (REEF_F_DUAL) */
+    REEF_CONV_SYNC_OFF,  /* first counter of this launch inside the sync storage (ints) */
     REEF_CONV_NATTR
 };
 #define REEF_F_BIAS 1
 #define REEF_F_RESIDUAL 2
 #define REEF_F_AFFINE 4 /* per-channel scale and shift after the sum */
+#define REEF_F_DUAL 8   /* second output out2 = act2(out + shift2[channel]) */
+#define REEF_F_FUSED_REDUCE 16 /* split-K folded inside the kernel by the last-arriving workgroup */
 
 /* Tile configurations (BM x BN output tile per workgroup, BK = 32). */
 enum {
@@ -161,9 +179,9 @@ enum {
 };
 
 /* ---- reef_splitk_reduce: out = act(sum_s ws[s] (+res)(+bias)(*scale+shift)), s ascending ----
- * ptr: ws, out, then optional bias, residual, scale, shift (same flag order).
- * attr: M, N, split_k, flags, act.   tasks = ceil(M*N / 1024) (4 elements per thread). */
-enum { REEF_RED_M = 0, REEF_RED_N, REEF_RED_SPLIT_K, REEF_RED_FLAGS, REEF_RED_ACT, REEF_RED_NATTR };
+ * ptr: ws, out, then optional bias, residual, (scale, shift), (out2, shift2) (same flag order).
+ * attr: M, N, split_k, flags, act, act2.   tasks = ceil(M*N / 1024) (4 elements per thread). */
+enum { REEF_RED_M = 0, REEF_RED_N, REEF_RED_SPLIT_K, REEF_RED_FLAGS, REEF_RED_ACT, REEF_RED_ACT2, REEF_RED_NATTR };
 
 /* ---- reef_dwconv2d: depthwise k x k convolution + bias + activation (bandwidth-bound) ----
  * ptr: in, W[C][kh][kw], out, bias(optional by flag).

@@ -272,27 +272,31 @@ class GraphOracle:
         P = [self.storage[i] for i in k["args"]]
         if name.startswith("reef_conv2d"):
             Cin, H, W, Cout, Ho, Wo, kh, kw, sh, sw, ph, pw, flags, act, _tile, split_k = a[:16]
-            if split_k > 1:
-                # The partial sums are an implementation detail of the device
-                # kernel; the oracle computes the whole convolution into slot 0
-                # of the workspace and leaves the other slots zero, which the
-                # ordered reduce then folds to the same mathematical result.
+            act2 = a[19] if len(a) > 19 else 0   # a[20]: first sync counter (device detail)
+            xin = P[0][:Cin * H * W].reshape(Cin, H, W)
+            wgt = P[1][:Cout * Cin * kh * kw].reshape(Cout, Cin, kh, kw)
+            if split_k > 1 and not (flags & 16):
+                # Plain split-K: the partial sums are an implementation detail of the
+                # device kernel; the oracle computes the whole convolution into slot 0
+                # of the workspace and leaves the other slots zero, which the ordered
+                # reduce then folds to the same mathematical result.
                 ws = P[2].view(np.float32)
                 ws[:split_k * Cout * Ho * Wo] = 0
-                out = conv2d(P[0][:Cin * H * W].reshape(Cin, H, W),
-                             P[1][:Cout * Cin * kh * kw].reshape(Cout, Cin, kh, kw),
-                             stride=(sh, sw), pad=(ph, pw), acc64=acc64)
+                out = conv2d(xin, wgt, stride=(sh, sw), pad=(ph, pw), acc64=acc64)
                 ws[:out.size] = out.reshape(-1)
                 return
-            bias, res, scale, shift = self._conv_opt(P, 3, flags)
-            out = conv2d(P[0][:Cin * H * W].reshape(Cin, H, W),
-                         P[1][:Cout * Cin * kh * kw].reshape(Cout, Cin, kh, kw), bias,
+            # single pass, or split-K folded inside the kernel (workspace untouched here)
+            bias, res, scale, shift, out2, shift2 = self._conv_opt(P, 3, flags)
+            out = conv2d(xin, wgt, bias,
                          None if res is None else res[:Cout * Ho * Wo].reshape(Cout, Ho, Wo),
                          scale, shift, (sh, sw), (ph, pw), 1, act, 6.0, acc64)
             P[2][:out.size] = out.reshape(-1)
+            if out2 is not None:
+                out2[:out.size] = eltwise(out.reshape(Cout, -1), shift=shift2[:Cout], act=act2).reshape(-1)
         elif name == "reef_splitk_reduce":
             M, N, split_k, flags, act = a[:5]
-            bias, res, scale, shift = self._conv_opt(P, 2, flags)
+            act2 = a[5] if len(a) > 5 else 0
+            bias, res, scale, shift, out2, shift2 = self._conv_opt(P, 2, flags)
             acc = np.zeros(M * N, np.float32)
             ws = P[0].view(np.float32)
             for s in range(split_k):
@@ -308,7 +312,10 @@ class GraphOracle:
                 v = np.maximum(v, 0)
             elif act == 2:
                 v = np.minimum(np.maximum(v, 0), 6.0)
-            P[1][:M * N] = v.astype(np.float32).reshape(-1)
+            v = v.astype(np.float32)
+            P[1][:M * N] = v.reshape(-1)
+            if out2 is not None:
+                out2[:M * N] = eltwise(v, shift=shift2[:M], act=act2).reshape(-1)
         elif name == "reef_dwconv2d":
             C, H, W, Ho, Wo, kh, kw, sh, sw, ph, pw, flags, act = a[:13]
             bias = P[3] if flags & 1 else None
@@ -395,7 +402,8 @@ class GraphOracle:
 
     @staticmethod
     def _conv_opt(P, pos, flags):
-        bias = res = scale = shift = None
+        """bias, residual, (scale, shift), (out2, shift2) follow the fixed operands in flag order."""
+        bias = res = scale = shift = out2 = shift2 = None
         if flags & 1:
             bias = P[pos]
             pos += 1
@@ -404,4 +412,7 @@ class GraphOracle:
             pos += 1
         if flags & 4:
             scale, shift = P[pos], P[pos + 1]
-        return bias, res, scale, shift
+            pos += 2
+        if flags & 8:
+            out2, shift2 = P[pos], P[pos + 1]
+        return bias, res, scale, shift, out2, shift2

@@ -16,7 +16,8 @@ struct BeKernarg {
 
 HybridExecutor::HybridExecutor()
     : preempt_mod(nullptr), trans_mod(nullptr), preempt_flag(nullptr), owns_flag(false),
-      task_slot_base(nullptr), task_slots_host_empty(nullptr), task_slots_host(nullptr) {}
+      task_slot_base(nullptr), task_slots_host_empty(nullptr), task_slots_host(nullptr),
+      sync_ptr(nullptr), sync_bytes(0) {}
 
 HybridExecutor::~HybridExecutor() {
     if (owns_flag && preempt_flag) reef_hal_free(preempt_flag, REEF_MEM_DEVICE_FINEGRAINED);
@@ -78,6 +79,12 @@ Status HybridExecutor::init_hybrid_executor(const char* json_file_path,
     GPU_RETURN_STATUS(reef_hal_malloc(std::max<size_t>(n, 1) * 4, REEF_MEM_DEVICE, &task_slot_base));
     GPU_RETURN_STATUS(reef_hal_memset(task_slot_base, 0, std::max<size_t>(n, 1) * 4));
 
+    size_t sync_idx;
+    if (find_storage_idx("reef_sync", sync_idx) == Status::Succ) {
+        sync_ptr = storage[sync_idx];
+        sync_bytes = storage_bytes(sync_idx);
+    }
+
     // 3. profile (hybrid_executor.cpp:92-97)
     model_profile.reset(ModelProfile::from_json(profile_file_path));
     if (!model_profile) RETURN_STATUS(Status::NotFound);
@@ -131,6 +138,12 @@ int HybridExecutor::get_be_kernel_offset(int begin) {
     for (size_t i = begin; i < num_kernels(); i++)
         if (task_slots_host[i] < trans_args[i].block_num) return (int)i;
     return (int)num_kernels();
+}
+
+Status HybridExecutor::reset_sync_storage(GPUStream_t stream) {
+    if (sync_bytes == 0) return Status::Succ;
+    GPU_RETURN_STATUS(reef_hal_memset_async(sync_ptr, 0, sync_bytes, stream));
+    return Status::Succ;
 }
 
 Status HybridExecutor::launch_preempt_kernel(int i, GPUStream_t stream) {

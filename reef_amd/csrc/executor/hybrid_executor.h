@@ -34,6 +34,11 @@ public:
     int get_be_kernel_offset(int begin);
 
     Status launch_preempt_kernel(int kernel_offset, GPUStream_t stream);
+    // Zeroes the model's "reef_sync" storage (the arrival counters of kernels that
+    // fold split-K internally) in stream order.  Needed before kernels of this model
+    // run again after an interrupted run; a no-op for models without that storage.
+    Status reset_sync_storage(GPUStream_t stream);
+    bool has_sync_storage() const { return sync_bytes > 0; }
     const ModelProfile* profile() const { return model_profile.get(); }
 
 protected:
@@ -50,6 +55,8 @@ protected:
     int* task_slots_host_empty;
     int* task_slots_host;
     std::shared_ptr<ModelProfile> model_profile;
+    GPUDevicePtr_t sync_ptr;
+    size_t sync_bytes;
 };
 
 }  // namespace executor

@@ -38,6 +38,9 @@ int reef_hal_memcpy_h2d(reef_devptr_t dst, const void* src, size_t bytes) {
 int reef_hal_memcpy_d2h(void* dst, reef_devptr_t src, size_t bytes) {
     return be()->memcpy_d2h(dst, src, bytes);
 }
+int reef_hal_memset_async(reef_devptr_t ptr, int byte, size_t bytes, reef_stream_t s) {
+    return be()->memset_async(ptr, byte, bytes, s);
+}
 int reef_hal_memcpy_h2d_async(reef_devptr_t dst, const void* src, size_t bytes, reef_stream_t s) {
     return be()->memcpy_h2d_async(dst, src, bytes, s);
 }

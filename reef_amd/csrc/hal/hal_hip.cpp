@@ -278,6 +278,16 @@ int h_clear_queue(reef_stream_t st, uint64_t* n) {
 }
 int h_reset_cus() { return 0; }
 
+int h_memset_async(reef_devptr_t p, int byte, size_t n, reef_stream_t st) {
+    // a windowed stream may hold launches on the host: the fill must not overtake them
+    if (st && st->window > 0 && !st->held.empty()) {
+        reef_hal_set_error("reef_hal_memset_async: stream holds launches on the host");
+        return 1;
+    }
+    HIPCHK(hipMemsetAsync(p, byte, n, st ? st->s : nullptr));
+    return 0;
+}
+
 int h_event_create(reef_event_t* out) {
     hipEvent_t e;
     HIPCHK(hipEventCreate(&e));
@@ -303,6 +313,7 @@ const reef_hal_backend kHip = {
     h_stream_create, h_stream_destroy, h_stream_sync, h_stream_query, h_device_sync, h_stream_pump,
     h_launch, h_write_value32, h_clear_queue, h_reset_cus,
     h_event_create, h_event_destroy, h_event_record, h_event_sync, h_event_elapsed_us,
+    h_memset_async,
 };
 
 }  // namespace

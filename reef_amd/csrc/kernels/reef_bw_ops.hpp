@@ -29,21 +29,19 @@ __device__ __forceinline__ void splitk_reduce_body(const ReefOpDesc& d, int task
     const float* ws = (const float*)d.ptr[0];
     float* out = (float*)d.ptr[1];
     Epilogue ep;
-    ep.unpack(d, 2, a[REEF_RED_FLAGS], a[REEF_RED_ACT]);
+    ep.unpack(d, 2, a[REEF_RED_FLAGS], a[REEF_RED_ACT], a[REEF_RED_ACT2]);
     const size_t i0 = ((size_t)task * kThreads + threadIdx.x) * 4;
     if (i0 >= MN) return;
     if ((MN & 3) == 0) {
         f32x4 acc = *(const f32x4*)(ws + i0);
         for (int s = 1; s < S; ++s) acc += *(const f32x4*)(ws + (size_t)s * MN + i0);
-        f32x4 o;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = ep.apply(acc[e], (int)((i0 + e) / N), i0 + e);
-        *(f32x4*)(out + i0) = o;
+        for (int e = 0; e < 4; ++e) ep.store(out, acc[e], (int)((i0 + e) / N), i0 + e);
     } else {
         for (int e = 0; e < 4 && i0 + e < MN; ++e) {
             float acc = ws[i0 + e];
             for (int s = 1; s < S; ++s) acc += ws[(size_t)s * MN + i0 + e];
-            out[i0 + e] = ep.apply(acc, (int)((i0 + e) / N), i0 + e);
+            ep.store(out, acc, (int)((i0 + e) / N), i0 + e);
         }
     }
 }

@@ -62,18 +62,33 @@ struct Epilogue {
     const float* residual;
     const float* scale;
     const float* shift;
-    int act;
-    __device__ __forceinline__ void unpack(const ReefOpDesc& d, int first, int flags, int act_) {
+    float* out2;
+    const float* shift2;
+    int act, act2;
+    int next;  // first pointer slot after the optional operands
+    __device__ __forceinline__ void unpack(const ReefOpDesc& d, int first, int flags, int act_,
+                                           int act2_ = 0) {
         int p = first;
         bias = (flags & REEF_F_BIAS) ? (const float*)d.ptr[p++] : nullptr;
         residual = (flags & REEF_F_RESIDUAL) ? (const float*)d.ptr[p++] : nullptr;
         if (flags & REEF_F_AFFINE) {
             scale = (const float*)d.ptr[p];
             shift = (const float*)d.ptr[p + 1];
+            p += 2;
         } else {
             scale = shift = nullptr;
         }
+        if (flags & REEF_F_DUAL) {
+            out2 = (float*)d.ptr[p];
+            shift2 = (const float*)d.ptr[p + 1];
+            p += 2;
+        } else {
+            out2 = nullptr;
+            shift2 = nullptr;
+        }
         act = act_;
+        act2 = act2_;
+        next = p;
     }
     // v = acc; v += residual; v += bias; v = fma(v, scale, shift); act
     __device__ __forceinline__ float apply(float v, int ch, size_t idx) const {
@@ -81,6 +96,12 @@ struct Epilogue {
         if (bias) v = v + bias[ch];
         if (scale) v = fmaf(v, scale[ch], shift[ch]);
         return act_apply(v, act);
+    }
+    // out[idx] = apply(...); out2[idx] = act2(out[idx] + shift2[ch])
+    __device__ __forceinline__ void store(float* out, float v, int ch, size_t idx) const {
+        const float o = apply(v, ch, idx);
+        out[idx] = o;
+        if (out2) out2[idx] = act_apply(o + shift2[ch], act2);
     }
 };
 

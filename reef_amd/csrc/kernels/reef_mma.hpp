@@ -277,37 +277,53 @@ __device__ __forceinline__ bool k_loop(LA& la, LB& lb, int nk, float* smem, f32x
 
 // ---- reef_conv2d ------------------------------------------------------------
 template <class T, class Poll>
-__device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d, int task, char* smem_raw,
+__device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, char* smem_raw,
                                             const Poll& poll) {
+  int M, N, split_k, split, rem, m0, n0;
+  float* smem = (float*)smem_raw;
+  f32x16 acc[T::TM][T::TN];
+  {
+    const ReefOpDesc& d = d_in;
     const int* a = d.attr;
-    const int M = a[REEF_CONV_COUT];
-    const int N = a[REEF_CONV_HO] * a[REEF_CONV_WO];
+    M = a[REEF_CONV_COUT];
+    N = a[REEF_CONV_HO] * a[REEF_CONV_WO];
     const int K = a[REEF_CONV_CIN] * a[REEF_CONV_KH] * a[REEF_CONV_KW];
-    const int split_k = a[REEF_CONV_SPLIT_K], k_chunk = a[REEF_CONV_K_CHUNK];
+    split_k = a[REEF_CONV_SPLIT_K];
+    const int k_chunk = a[REEF_CONV_K_CHUNK];
     const int n_tiles = a[REEF_CONV_N_TILES];
     const int tiles = a[REEF_CONV_M_TILES] * n_tiles;
-    const int split = task / tiles;
-    const int rem = task - split * tiles;
+    split = task / tiles;
+    rem = task - split * tiles;
     const int mt = rem / n_tiles, nt = rem - mt * n_tiles;
-    const int m0 = mt * T::BM, n0 = nt * T::BN;
+    m0 = mt * T::BM;
+    n0 = nt * T::BN;
     const int k_begin = split * k_chunk;
     const int k_end = min(K, k_begin + k_chunk);
     const int nk = (k_end - k_begin + 31) >> 5;
 
-    float* smem = (float*)smem_raw;
     ALoader<T> la;
     Im2colLoader<T> lb;
     la.init((const float*)d.ptr[1], K, m0, M, k_begin, k_end, (K & 3) == 0);
     lb.init((const float*)d.ptr[0], a, n0, N, k_begin, k_end);
 
-    f32x16 acc[T::TM][T::TN];
     if (!k_loop<T, false>(la, lb, nk, smem, acc, poll)) return false;
+  }
 
+    // Everything the epilogue needs is re-read from the argument block here, so the
+    // K loop does not carry the epilogue's pointers in scalar registers.
+    const ReefOpDesc* dp = &d_in;
+    asm volatile("" : "+s"(dp));
+    const ReefOpDesc& d = *dp;
+    const int* a = d.attr;
     const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5, wave = threadIdx.x >> 6;
     const int wm0 = (wave / T::WGN) * (T::TM * 32), wn0 = (wave % T::WGN) * (T::TN * 32);
     float* dst = (float*)d.ptr[2];
-    if (split_k > 1) {
-        dst += (size_t)split * M * N;
+    const int flags = a[REEF_CONV_FLAGS];
+    const size_t MN = (size_t)M * N;
+
+    if (split_k > 1 && !(flags & REEF_F_FUSED_REDUCE)) {
+        // plain split-K: partial tile to the workspace, reef_splitk_reduce folds
+        float* ws = dst + (size_t)split * MN;
 #pragma unroll
         for (int tm = 0; tm < T::TM; ++tm)
 #pragma unroll
@@ -316,12 +332,41 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d, int task, char*
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int m = m0 + wm0 + tm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                    if (m < M && n < N) dst[(size_t)m * N + n] = acc[tm][tn][r];
+                    if (m < M && n < N) ws[(size_t)m * N + n] = acc[tm][tn][r];
                 }
             }
-    } else {
-        Epilogue ep;
-        ep.unpack(d, 3, a[REEF_CONV_FLAGS], a[REEF_CONV_ACT]);
+        return true;
+    }
+
+    Epilogue ep;
+    ep.unpack(d, 3, flags, a[REEF_CONV_ACT], a[REEF_CONV_ACT2]);
+    if (split_k > 1) {
+        // fused split-K: store the partial, count in, the last arrival folds all
+        // partials in ascending split order (fixed order => same bits whoever is last)
+        float* ws = (float*)d.ptr[ep.next];
+        int* counters = (int*)d.ptr[ep.next + 1] + a[REEF_CONV_SYNC_OFF];
+        int* s_last = (int*)(smem + 2 * (T::A_FLOATS + T::B_FLOATS)) + 1;
+        float* part = ws + (size_t)split * MN;
+#pragma unroll
+        for (int tm = 0; tm < T::TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < T::TN; ++tn) {
+                const int n = n0 + wn0 + tn * 32 + l32;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = m0 + wm0 + tm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                    if (m < M && n < N) part[(size_t)m * N + n] = acc[tm][tn][r];
+                }
+            }
+        __threadfence();  // release the partial tile device-wide before counting in
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            const int old = atomicAdd(&counters[rem], 1);
+            *s_last = (old == split_k - 1);
+        }
+        __syncthreads();
+        if (!*s_last) return true;
+        __threadfence();  // acquire the other splits' partial tiles
 #pragma unroll
         for (int tm = 0; tm < T::TM; ++tm)
 #pragma unroll
@@ -332,11 +377,27 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d, int task, char*
                     const int m = m0 + wm0 + tm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
                     if (m < M && n < N) {
                         const size_t idx = (size_t)m * N + n;
-                        dst[idx] = ep.apply(acc[tm][tn][r], m, idx);
+                        float v = ws[idx];
+                        for (int s = 1; s < split_k; ++s) v += ws[(size_t)s * MN + idx];
+                        ep.store(dst, v, m, idx);
                     }
                 }
             }
+        if (threadIdx.x == 0) counters[rem] = 0;  // ready for the next run
+        return true;
     }
+
+#pragma unroll
+    for (int tm = 0; tm < T::TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < T::TN; ++tn) {
+            const int n = n0 + wn0 + tn * 32 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + wm0 + tm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                if (m < M && n < N) ep.store(dst, acc[tm][tn][r], m, (size_t)m * N + n);
+            }
+        }
     return true;
 }
 

@@ -154,6 +154,8 @@ Status REEFScheduler::new_task(const ModelID& mid, TaskID& tid) {
     task->preempted = false;
     task->padding = false;
     task->padding_to_finish = false;
+    task->sync_dirty = false;
+    task->sync_touched = false;
     tid = task->id;
     {
         std::lock_guard<std::mutex> lock(task_pool_mtx);
@@ -295,6 +297,7 @@ void REEFScheduler::preempt_reset() {
             task->block_offset = 0;
             task->state.store(TaskState::Waiting);
             task->preempted = true;
+            task->sync_dirty = true;
         }
     }
     for (int i = 0; i < be_stream_device_queue_cap + 1; i++) reef_hal_reset_cus();
@@ -471,6 +474,15 @@ void REEFScheduler::dynamic_kernel_padding(std::shared_ptr<Task>& rt_task) {
             if (!cand) continue;
             HybridExecutor& be_exe = cand->model->executor;
             if (cand->kernel_offset >= (int)be_exe.num_kernels()) continue;
+            if (cand->sync_dirty) {
+                // an interrupted run left arrival counters behind: pad this task only once
+                // its own stream has drained, and clear the counters first
+                if (be_exe.has_sync_storage()) {
+                    if (!executor::GPUStreamEmpty(be_queues[q]->stream)) continue;
+                    be_exe.reset_sync_storage(rt_queue->stream);
+                }
+                cand->sync_dirty = false;
+            }
             const TransExecutor::KernelArg& ka = be_exe.trans_args[cand->kernel_offset];
             // the proxy class that holds both bodies sets the register budget of the launch
             const int level = std::max(rt_args.proxy_level, ka.proxy_level);
@@ -515,6 +527,8 @@ void REEFScheduler::dynamic_kernel_padding(std::shared_ptr<Task>& rt_task) {
         // progress of the padded best-effort task (scheduler.cpp:655-672)
         if (be_task) {
             be_task->padding = true;
+            // a later restart in best-effort mode re-runs this kernel from its first block
+            be_task->sync_touched = true;
             be_task->block_offset += dec.be_block_num;
             if (be_task->block_offset >= be_args->block_num) {
                 be_task->block_offset = 0;
@@ -570,6 +584,13 @@ void REEFScheduler::execute_be_task(std::shared_ptr<Task>& task, std::shared_ptr
             }
             task->state.store(TaskState::Executing);
             task->block_offset = 0;
+            // Arrival counters of split-K kernels may be left over from an interrupted
+            // or partly padded run; the fill is ordered behind anything still draining
+            // on this stream.
+            if (task->sync_dirty || task->sync_touched) {
+                exe.reset_sync_storage(tqueue->stream);
+                task->sync_dirty = task->sync_touched = false;
+            }
             for (int i = task->kernel_offset; i < num_kernels; i++) {
                 exe.launch_preempt_kernel(i, tqueue->stream);
                 task->launch_offset = i;

@@ -71,6 +71,8 @@ public:
         bool preempted;
         bool padding;
         bool padding_to_finish;
+        bool sync_dirty;    // an interrupted run may have left split-K arrival counters non-zero
+        bool sync_touched;  // padding ran part of a kernel: counters hold live partial counts
 
     public:
         bool is_preempted() const { return preempted; }

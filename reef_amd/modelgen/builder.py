@@ -24,7 +24,7 @@ from . import rng, tiling
 from ..paths import code_object
 
 ACT_NONE, ACT_RELU, ACT_RELU6, ACT_GELU = 0, 1, 2, 3
-F_BIAS, F_RESIDUAL, F_AFFINE = 1, 2, 4
+F_BIAS, F_RESIDUAL, F_AFFINE, F_DUAL, F_FUSED_REDUCE = 1, 2, 4, 8, 16
 WG = 256
 
 
@@ -58,9 +58,12 @@ class GraphBuilder:
         self.kernel_bytes = []         # algorithmic bytes per kernel call
         self.kernel_est_us = []
         self._np = 0
+        self._sync_idx = None
         # "symbol#instance" names give every kernel call its own profile entry
         # (the profile is keyed by kernel name, model.cpp:57-80).
         self.unique_names = True
+        # split-K folded inside the conv kernel (False: separate reef_splitk_reduce launch)
+        self.fused_reduce = True
 
     # ------------------------------------------------------------ storages
     def _storage(self, name, size, stype="float32"):
@@ -93,6 +96,14 @@ class GraphBuilder:
         self.params.append((key, arr))
         return Tensor(idx, shape)
 
+    def _sync_counters(self, n):
+        """Reserves n counters in the model's sync storage; returns (storage idx, first counter)."""
+        if self._sync_idx is None:
+            self._sync_idx = self._storage("reef_sync", 0, "int32")
+        off = self.storage[self._sync_idx]["size"]
+        self.storage[self._sync_idx]["size"] = off + int(n)
+        return self._sync_idx, off
+
     def mark_output(self, t):
         self.storage[t.idx]["name"] = "output"
 
@@ -110,8 +121,12 @@ class GraphBuilder:
         self.kernel_est_us.append(float(est_us))
 
     def conv2d(self, x, cout, k, stride=1, pad=0, bias=True, act=ACT_RELU, residual=None,
-               affine=False, force=None):
-        """Fused conv + (residual) + (bias) + (scale, shift) + activation on MFMA."""
+               affine=False, force=None, dual_act=None, fused_reduce=None):
+        """Fused conv + (residual) + (bias) + (scale, shift) + activation on MFMA.
+        dual_act: also emit out2 = dual_act(out + shift2[c]) and return (out, out2).
+        fused_reduce: fold split-K inside the kernel (default: self.fused_reduce)."""
+        if fused_reduce is None:
+            fused_reduce = self.fused_reduce
         kh, kw = (k, k) if isinstance(k, int) else k
         sh, sw = (stride, stride) if isinstance(stride, int) else stride
         ph, pw = (pad, pad) if isinstance(pad, int) else pad
@@ -136,27 +151,46 @@ class GraphBuilder:
             self.params[-1] = (self.params[-1][0], self.params[-1][1] + 1.0)
             opt.append(self.param((cout,), 0.01).idx)
         out = self.temp((cout, Ho, Wo))
-        t = force or tiling.choose(M, N, K)
+        out2 = None
+        if dual_act is not None:
+            assert not affine
+            flags |= F_DUAL
+            out2 = self.temp((cout, Ho, Wo))
+            opt.append(out2.idx)
+            opt.append(self.param((cout,), 0.01).idx)
+        act2 = dual_act or ACT_NONE
+        t = force or tiling.choose(M, N, K, fused=fused_reduce)
         flops = 2 * M * N * K
         self.flops += flops
         nbytes = 4 * (x.size + M * K + M * N + (M if bias else 0) + (M * N if residual is not None else 0)
                       + (2 * M if affine else 0))
         base = [cin, H, W, cout, Ho, Wo, kh, kw, sh, sw, ph, pw]
         kname = "reef_conv2d_" + t["tile"]
+        if out2 is not None:
+            nbytes += 4 * (M * N + M)
         if t["split_k"] == 1:
-            attrs = base + [flags, act, t["tile_id"], 1, t["k_chunk"], t["m_tiles"], t["n_tiles"]]
+            attrs = base + [flags, act, t["tile_id"], 1, t["k_chunk"], t["m_tiles"], t["n_tiles"], act2]
             self._emit(kname, t["tasks"], [x.idx, w.idx, out.idx] + opt, attrs, "conv2d", flops,
                        nbytes, t["est_us"])
+        elif fused_reduce:
+            # workspace: split_k partial tensors; counters: one int per output tile in
+            # the model's single sync storage
+            ws = self.workspace(t["split_k"] * M * N)
+            sync_idx, sync_off = self._sync_counters(t["m_tiles"] * t["n_tiles"])
+            attrs = base + [flags | F_FUSED_REDUCE, act, t["tile_id"], t["split_k"], t["k_chunk"],
+                            t["m_tiles"], t["n_tiles"], act2, sync_off]
+            self._emit(kname, t["tasks"], [x.idx, w.idx, out.idx] + opt + [ws.idx, sync_idx], attrs,
+                       "conv2d", flops, nbytes, t["est_us"])
         else:
             ws = self.workspace(t["split_k"] * M * N)
             attrs = base + [0, ACT_NONE, t["tile_id"], t["split_k"], t["k_chunk"], t["m_tiles"],
-                            t["n_tiles"]]
+                            t["n_tiles"], ACT_NONE]
             self._emit(kname, t["tasks"], [x.idx, w.idx, ws.idx], attrs, "conv2d", flops,
                        4 * (x.size + M * K + t["split_k"] * M * N), t["est_us"])
             self._emit("reef_splitk_reduce", math.ceil(M * N / 1024), [ws.idx, out.idx] + opt,
-                       [M, N, t["split_k"], flags, act], "splitk_reduce", 0,
+                       [M, N, t["split_k"], flags, act, act2], "splitk_reduce", 0,
                        4 * ((t["split_k"] + 1) * M * N), 2.0)
-        return out
+        return out if out2 is None else (out, out2)
 
     def dwconv2d(self, x, k, stride=1, pad=0, bias=True, act=ACT_RELU6):
         C, H, W = x.shape

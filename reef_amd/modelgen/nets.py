@@ -34,7 +34,10 @@ def image_input(name, shape, seed=rng.BASE_SEED):
     return ((x - mean) / std).astype(np.float32)
 
 
-def resnet(num_layers=152, image=(3, 224, 224), classes=1000, name=None, seed=rng.BASE_SEED):
+def resnet(num_layers=152, image=(3, 224, 224), classes=1000, name=None, seed=rng.BASE_SEED,
+           fused_reduce=True, fuse_act=True):
+    """fused_reduce: fold split-K inside the conv kernels.  fuse_act: let the unit's last
+    conv also write the next unit's activated input (one kernel instead of conv + add/relu)."""
     if num_layers >= 50:
         bottleneck = True
         filters = [64, 256, 512, 1024, 2048]
@@ -44,6 +47,7 @@ def resnet(num_layers=152, image=(3, 224, 224), classes=1000, name=None, seed=rn
         filters = [64, 64, 128, 256, 512]
         units = {18: [2, 2, 2, 2], 34: [3, 4, 6, 3]}[num_layers]
     g = GraphBuilder(name or "resnet%d" % num_layers, seed)
+    g.fused_reduce = fused_reduce
     data = g.input("data", image)
     x = g.eltwise(data, shift=True)                                  # bn_data (shift only)
     x = g.conv2d(x, filters[0], 7, 2, 3, bias=True, act=ACT_RELU)    # conv0 + bn0 + relu
@@ -72,6 +76,9 @@ def resnet(num_layers=152, image=(3, 224, 224), classes=1000, name=None, seed=rn
             elif last_of_stage:
                 act = g.conv2d(y, cout, last_k, 1, last_p, bias=True, act=ACT_RELU,
                                residual=shortcut)
+            elif fuse_act:
+                raw, act = g.conv2d(y, cout, last_k, 1, last_p, bias=False, act=ACT_NONE,
+                                    residual=shortcut, dual_act=ACT_RELU)
             else:
                 raw = g.conv2d(y, cout, last_k, 1, last_p, bias=False, act=ACT_NONE,
                                residual=shortcut)

@@ -26,6 +26,7 @@ BK = 32
 T_STEP_128x128 = 1.9     # one BK=32 step of a 128x128 tile on one CU at efficiency 1.0
 T_FIXED = 2.0            # prologue + epilogue of a workgroup
 T_REDUCE_LAUNCH = 3.0    # extra launch of the split-K reduce
+T_FUSED_REDUCE = 1.0     # fence + last-arrival fold inside the conv kernel
 HBM_BYTES_PER_US = 4.0e6
 
 
@@ -33,7 +34,7 @@ def _steps_time(bm, bn, eff, steps):
     return steps * T_STEP_128x128 * (bm * bn) / (128.0 * 128.0) / eff
 
 
-def choose(M, N, K, allow_split=True, tiles=None, max_split=32):
+def choose(M, N, K, allow_split=True, tiles=None, max_split=32, fused=True):
     """Returns dict(tile, tile_id, BM, BN, split_k, k_chunk, m_tiles, n_tiles, tasks)."""
     best = None
     for name in (tiles or TILES.keys()):
@@ -54,7 +55,7 @@ def choose(M, N, K, allow_split=True, tiles=None, max_split=32):
             share = min(occ, math.ceil(wgs / NUM_CUS))
             t = rounds * (_steps_time(bm, bn, eff, k_chunk // BK) * share + T_FIXED)
             if s_eff > 1:
-                t += T_REDUCE_LAUNCH + (s_eff + 1) * M * N * 4 / HBM_BYTES_PER_US
+                t += (T_FUSED_REDUCE if fused else T_REDUCE_LAUNCH) + (s_eff + 1) * M * N * 4 / HBM_BYTES_PER_US
             cand = (t, name, s_eff, k_chunk, m_tiles, n_tiles)
             if best is None or cand[0] < best[0] - 1e-9:
                 best = cand

@@ -16,7 +16,7 @@ SO = os.path.join(HERE, "fake_hal", "libreef_fakehal.so")
 
 
 class OpDesc(ctypes.Structure):
-    _fields_ = [("ptr", ctypes.c_void_p * 8), ("attr", ctypes.c_int32 * 24)]
+    _fields_ = [("ptr", ctypes.c_void_p * 10), ("attr", ctypes.c_int32 * 24)]
 
 
 class BeArg(ctypes.Structure):
@@ -134,13 +134,13 @@ class FakeHal:
         if count is not None and first + count < total:
             return   # an earlier piece of a split launch: the last piece applies the kernel
         views = []
-        for i in range(8):
+        for i in range(10):
             dt = np.int64 if (symbol == "reef_embedding" and i == 0) else np.float32
             views.append(self._view(desc.ptr[i], dt))
         orc = O.GraphOracle.__new__(O.GraphOracle)
         orc.storage = views
         orc.model = {}
-        orc.run_kernel({"name": symbol, "attrs": attrs, "args": list(range(8)),
+        orc.run_kernel({"name": symbol, "attrs": attrs, "args": list(range(10)),
                         "launch_params": [blocks, 1, 1, 256, 1, 1]})
 
     def _on_kernel(self, symbol, module_path, kernarg, nbytes, grid, block, lds, stream):

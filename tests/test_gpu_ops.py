@@ -83,6 +83,39 @@ def test_conv_split_k_and_epilogues(tmp_path, tile, split):
     assert a.shape == b.shape
 
 
+@pytest.mark.parametrize("tile,split", [("64x64", 4), ("128x64", 6), ("128x32", 16), ("32x128", 3),
+                                        ("64x128", 2), ("128x128", 2)])
+def test_fused_split_k_equals_plain_split_k_bitwise(tmp_path, tile, split):
+    """Split-K folded inside the kernel by the last-arriving workgroup sums the partial
+    tiles in the same fixed order as the separate reduce launch: identical bits, also
+    for the second (activated) output and on a rerun (counters reset themselves)."""
+    cin, H, W, cout = 128, 14, 14, 192
+    g = MB.GraphBuilder("f")
+    x = g.input("data", (cin, H, W))
+    res = g.input("res", (cout, H, W))
+    f = forced(tile, cout, H * W, cin * 9, split)
+    outs = {}
+    for fused in (False, True):
+        g._np = 0          # same parameter names -> same seeded weights for both variants
+        a = g.conv2d(x, cout, 3, 1, 1, bias=True, act=MB.ACT_RELU, force=f, fused_reduce=fused)
+        b, b2 = g.conv2d(x, cout, 3, 1, 1, bias=False, act=MB.ACT_NONE, residual=res,
+                         dual_act=MB.ACT_RELU, force=f, fused_reduce=fused)
+        c = g.conv2d(x, cout, 3, 1, 1, bias=False, act=MB.ACT_RELU, residual=res, affine=True,
+                     force=f, fused_reduce=fused)
+        outs[fused] = (a, b, b2, c)
+    g.mark_output(outs[True][0])
+    # both variants read the same parameter storages by name: keep one copy of each key
+    seen = {}
+    g.params = [kv for kv in g.params if not (kv[0] in seen or seen.setdefault(kv[0], 0))]
+    exe, orc, model = run_both(g, tmp_path, {"data": rnd(cin, H, W), "res": rnd(cout, H, W)})
+    compare_storages(exe, orc, model, what="fused split-k %s x%d" % (tile, split))
+    for rerun in range(2):
+        for t_plain, t_fused in zip(outs[False], outs[True]):
+            np.testing.assert_array_equal(exe.get_data(t_plain.idx, t_plain.size),
+                                          exe.get_data(t_fused.idx, t_fused.size))
+        exe.execute()
+
+
 def test_conv_auto_heuristic_shapes(tmp_path):
     """The layer shapes of ResNet-152 at reduced channel counts, tiles picked by the generator."""
     g = MB.GraphBuilder("h")
