@@ -159,6 +159,7 @@ enum {
     REEF_CONV_M_TILES, REEF_CONV_N_TILES,
     REEF_CONV_ACT2,      /* activation of the second output (REEF_F_DUAL) */
     REEF_CONV_SYNC_OFF,  /* first counter of this launch inside the sync storage (ints) */
+    REEF_CONV_MODE,      /* REEF_CONV_MODE_*: must match the entry symbol's family */
     REEF_CONV_NATTR
 };
 #define REEF_F_BIAS 1
@@ -166,6 +167,14 @@ enum {
 #define REEF_F_AFFINE 4 /* per-channel scale and shift after the sum */
 #define REEF_F_DUAL 8   /* second output out2 = act2(out + shift2[channel]) */
 #define REEF_F_FUSED_REDUCE 16 /* split-K folded inside the kernel by the last-arriving workgroup */
+
+/* Loader families of the convolution; the entry symbol carries the family:
+ *   reef_conv2d_<tile>      general: im2col gather, needs K % 4 == 0
+ *   reef_conv2d_pw_<tile>   pointwise: 1x1, stride 1, no padding, N % 4 == 0, K % 4 == 0
+ *   reef_conv2d_u_<tile>    unaligned: im2col gather, any K */
+#define REEF_CONV_MODE_GENERAL 0
+#define REEF_CONV_MODE_POINTWISE 1
+#define REEF_CONV_MODE_UNALIGNED 2
 
 /* Tile configurations (BM x BN output tile per workgroup, BK = 32). */
 enum {
@@ -243,7 +252,9 @@ enum { REEF_COPY_COUNT = 0, REEF_COPY_DST_OFF, REEF_COPY_NATTR };
  * ptr: in, out, bias(optional).  attr: d0, d1, d2, flags.  tasks = ceil(d0*d1*d2/1024). */
 enum { REEF_TR_D0 = 0, REEF_TR_D1, REEF_TR_D2, REEF_TR_FLAGS, REEF_TR_NATTR };
 
-/* ---- reef_gemm: batched fp32 GEMM on MFMA ----
+/* ---- reef_gemm_nt_<tile> / reef_gemm_nn_<tile>: batched fp32 GEMM on MFMA ----
+ * nt: trans_b = 1 (K, lda, ldb and the batch strides must be multiples of 4);
+ * nn: trans_b = 0 (K and lda multiples of 4).
  * C[b][m][n] = act(alpha * sum_k A[b][m][k] * B(b,k,n) (+bias[n]))
  * trans_b = 1: B stored [b][n][k] (dense layers, Q.K^T); 0: [b][k][n] (P.V).
  * ptr: A, B, C, bias(optional).

@@ -57,10 +57,12 @@ Status TransExecutor::init_rt_executor(const char* json_file_path, GPUModule_t m
         const uint32_t* lp = ki.launch_params;
         ka.kernel = kernel_funcs[i];
         ka.op = op_from_name(kernel_symbol(ki.name));
-        int tile = -1;
-        if (ka.op == REEF_OP_CONV2D && ki.attrs.size() > REEF_CONV_TILE) tile = ki.attrs[REEF_CONV_TILE];
-        if (ka.op == REEF_OP_GEMM && ki.attrs.size() > REEF_GEMM_TILE) tile = ki.attrs[REEF_GEMM_TILE];
-        ka.proxy_level = proxy_level(ka.op, tile);
+        int tile = -1, mode = 0;
+        if (ka.op == REEF_OP_CONV2D && ki.attrs.size() > REEF_CONV_MODE) {
+            tile = ki.attrs[REEF_CONV_TILE];
+            mode = ki.attrs[REEF_CONV_MODE];
+        }
+        ka.proxy_level = proxy_level(ka.op, tile, mode);
         ka.task_dim = dim3u(lp[0], lp[1], lp[2]);
         ka.thread_dim = dim3u(lp[3], lp[4], lp[5]);
         ka.block_num = (int)ka.task_dim.count();
@@ -143,19 +145,21 @@ int TransExecutor::occupancy_class(const GPUConfig::KernelResource& kr) {
 }
 
 int TransExecutor::proxy_class_of_level(int level) {
-    static const int cls[kNumProxyLevels] = {8, 4, 3, 2};
+    static const int cls[kNumProxyLevels] = {8, 3, 2};
     return cls[std::max(0, std::min(level, kNumProxyLevels - 1))];
 }
 
-// Which proxy holds the body of (op, tile): the bandwidth-bound ops are in every
-// proxy, the matrix-core tiles only in the classes whose register budget fits them.
-int TransExecutor::proxy_level(int op, int tile) {
+// Which proxy holds the body of (op, tile, loader family): the bandwidth-bound ops
+// are in every proxy, a few matrix-core tiles in the classes whose register budget
+// fits them, and everything else in none (-1: that kernel is never merged).
+int TransExecutor::proxy_level(int op, int tile, int mode) {
     if (op == REEF_OP_CONV2D) {
-        if (tile == REEF_TILE_64x64 || tile == REEF_TILE_128x32 || tile == REEF_TILE_32x128) return 1;
-        if (tile == REEF_TILE_128x64 || tile == REEF_TILE_64x128) return 2;
-        return 3;
+        if (mode != REEF_CONV_MODE_GENERAL && mode != REEF_CONV_MODE_POINTWISE) return -1;
+        if (tile == REEF_TILE_64x64 || tile == REEF_TILE_128x32) return 1;
+        if (tile == REEF_TILE_128x64) return 2;
+        return -1;
     }
-    if (op == REEF_OP_GEMM) return (tile == REEF_TILE_64x64 || tile == REEF_TILE_32x128) ? 2 : 3;
+    if (op == REEF_OP_GEMM || op == REEF_OP_NONE) return -1;
     return 0;
 }
 

@@ -25,7 +25,7 @@ public:
     public:
         GPUFunction_t kernel;
         int op;                 // REEF_OP_* of this call (replaces funcion_pointer)
-        int proxy_level;        // smallest merge_framework class that contains this op
+        int proxy_level;        // smallest merge_framework class that contains this op, -1: none
         dim3u task_dim;
         dim3u thread_dim;
         int block_num;
@@ -48,10 +48,10 @@ public:
     // (trans_executor.cpp:175-199 picks among 10 gfx906 classes the same way).
     static int occupancy_class(const GPUConfig::KernelResource& kr);
     // The code object carries one proxy per occupancy class that matters for
-    // this kernel set: merge_framework_8 / _4 / _3 / _2 = levels 0..3.
-    static constexpr int kNumProxyLevels = 4;
+    // this kernel set: merge_framework_8 / _3 / _2 = levels 0..2.
+    static constexpr int kNumProxyLevels = 3;
     static int proxy_class_of_level(int level);
-    static int proxy_level(int op, int tile);
+    static int proxy_level(int op, int tile, int mode);
 
 protected:
     Status init_rt_executor(const char* json_file_path, GPUModule_t module);

@@ -34,6 +34,17 @@ struct FlagPoll {
     }
 };
 
+// Device-coherent accesses for data one workgroup hands to another inside a kernel
+// (split-K partial tiles).  The scope travels on the instruction, so no L2-wide
+// write-back or invalidate is needed -- a __threadfence() per workgroup costs two
+// orders of magnitude more here.
+__device__ __forceinline__ void store_agent(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_agent(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);

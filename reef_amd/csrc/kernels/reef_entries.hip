@@ -27,20 +27,20 @@ using namespace reef_dev;
 namespace {
 
 // ---- op functors: LDS need + body ------------------------------------------
-template <class T>
+template <class T, int MODE = CONV_GENERAL>
 struct OpConv {
     static constexpr int LDS = T::LDS_BYTES;
     template <class P>
     static __device__ __forceinline__ bool run(const ReefOpDesc& d, int task, char* smem, const P& p) {
-        return conv2d_body<T>(d, task, smem, p);
+        return conv2d_body<T, MODE>(d, task, smem, p);
     }
 };
-template <class T>
+template <class T, bool TRANS_B>
 struct OpGemm {
     static constexpr int LDS = T::LDS_BYTES;
     template <class P>
     static __device__ __forceinline__ bool run(const ReefOpDesc& d, int task, char* smem, const P& p) {
-        return gemm_body<T>(d, task, smem, p);
+        return gemm_body<T, TRANS_B>(d, task, smem, p);
     }
 };
 #define REEF_SIMPLE_OP(STRUCT, CALL)                                                            \
@@ -123,6 +123,7 @@ __device__ __forceinline__ bool dkp_walk(const ReefDkpArgs& a, DkpWalk& w) {
 }  // namespace
 
 // ---- entry generators ---------------------------------------------------------
+#define REEF_COMMA ,
 #if REEF_FLAVOUR == 0
 #define REEF_ENTRY(NAME, OP)                                                          \
     extern "C" __global__ void __launch_bounds__(REEF_WG_THREADS) NAME(ReefOpDesc) {  \
@@ -164,9 +165,24 @@ REEF_ENTRY(reef_conv2d_64x64, OpConv<Tile64x64>)
 REEF_ENTRY(reef_conv2d_128x32, OpConv<Tile128x32>)
 REEF_ENTRY(reef_conv2d_32x128, OpConv<Tile32x128>)
 REEF_ENTRY(reef_conv2d_64x128, OpConv<Tile64x128>)
-REEF_ENTRY(reef_gemm_128x128, OpGemm<Tile128x128>)
-REEF_ENTRY(reef_gemm_64x64, OpGemm<Tile64x64>)
-REEF_ENTRY(reef_gemm_32x128, OpGemm<Tile32x128>)
+REEF_ENTRY(reef_conv2d_pw_128x128, OpConv<Tile128x128 REEF_COMMA CONV_POINTWISE>)
+REEF_ENTRY(reef_conv2d_pw_128x64, OpConv<Tile128x64 REEF_COMMA CONV_POINTWISE>)
+REEF_ENTRY(reef_conv2d_pw_64x64, OpConv<Tile64x64 REEF_COMMA CONV_POINTWISE>)
+REEF_ENTRY(reef_conv2d_pw_128x32, OpConv<Tile128x32 REEF_COMMA CONV_POINTWISE>)
+REEF_ENTRY(reef_conv2d_pw_32x128, OpConv<Tile32x128 REEF_COMMA CONV_POINTWISE>)
+REEF_ENTRY(reef_conv2d_pw_64x128, OpConv<Tile64x128 REEF_COMMA CONV_POINTWISE>)
+REEF_ENTRY(reef_conv2d_u_128x128, OpConv<Tile128x128 REEF_COMMA CONV_UNALIGNED>)
+REEF_ENTRY(reef_conv2d_u_128x64, OpConv<Tile128x64 REEF_COMMA CONV_UNALIGNED>)
+REEF_ENTRY(reef_conv2d_u_64x64, OpConv<Tile64x64 REEF_COMMA CONV_UNALIGNED>)
+REEF_ENTRY(reef_conv2d_u_128x32, OpConv<Tile128x32 REEF_COMMA CONV_UNALIGNED>)
+REEF_ENTRY(reef_conv2d_u_32x128, OpConv<Tile32x128 REEF_COMMA CONV_UNALIGNED>)
+REEF_ENTRY(reef_conv2d_u_64x128, OpConv<Tile64x128 REEF_COMMA CONV_UNALIGNED>)
+REEF_ENTRY(reef_gemm_nt_128x128, OpGemm<Tile128x128 REEF_COMMA true>)
+REEF_ENTRY(reef_gemm_nt_64x64, OpGemm<Tile64x64 REEF_COMMA true>)
+REEF_ENTRY(reef_gemm_nt_32x128, OpGemm<Tile32x128 REEF_COMMA true>)
+REEF_ENTRY(reef_gemm_nn_128x128, OpGemm<Tile128x128 REEF_COMMA false>)
+REEF_ENTRY(reef_gemm_nn_64x64, OpGemm<Tile64x64 REEF_COMMA false>)
+REEF_ENTRY(reef_gemm_nn_32x128, OpGemm<Tile32x128 REEF_COMMA false>)
 REEF_ENTRY(reef_splitk_reduce, OpSplitKReduce)
 REEF_ENTRY(reef_dwconv2d, OpDwConv)
 REEF_ENTRY(reef_pool2d, OpPool)
@@ -190,10 +206,11 @@ REEF_ENTRY(multiply, OpMocked<true>)
 // (script/replace_register_usage.py:33-59).  Here the side carries an op id and
 // the proxy switches into the inlined body; the variants are the gfx950
 // occupancy classes that matter for this kernel set, <n> = wavefronts per SIMD:
-//   merge_framework_8  bandwidth-bound ops only                      (<= 64 registers)
-//   merge_framework_4  + conv tiles 64x64 / 128x32 / 32x128            (<= 128)
-//   merge_framework_3  + conv tiles 128x64 / 64x128, gemm 64x64 / 32x128 (<= 168)
-//   merge_framework_2  + the 128x128 tiles                             (<= 256)
+//   merge_framework_8  bandwidth-bound ops only                          (<= 64 registers)
+//   merge_framework_3  + conv (general, pointwise) tiles 64x64 / 128x32    (<= 168)
+//   merge_framework_2  + conv (general, pointwise) tile 128x64             (<= 256)
+// Kernels outside these sets (the other tiles, the unaligned-K convolution, GEMM)
+// are never merged: they run single-sided through their own entry.
 // LDS is dynamic (the host passes the larger of the two sides' needs, as
 // src/reef/server/scheduler.cpp:643-649 does).
 namespace {
@@ -204,24 +221,15 @@ __device__ __forceinline__ void run_op(const ReefDkpSide& s, int task, char* sme
     switch (s.op) {
         case REEF_OP_CONV2D:
             if (LEVEL >= 1) {
-                switch (d.attr[REEF_CONV_TILE]) {
-                    case REEF_TILE_64x64: OpConv<Tile64x64>::run(d, task, smem, np); break;
-                    case REEF_TILE_128x32: OpConv<Tile128x32>::run(d, task, smem, np); break;
-                    case REEF_TILE_32x128: OpConv<Tile32x128>::run(d, task, smem, np); break;
-                    case REEF_TILE_128x64: if (LEVEL >= 2) OpConv<Tile128x64>::run(d, task, smem, np); break;
-                    case REEF_TILE_64x128: if (LEVEL >= 2) OpConv<Tile64x128>::run(d, task, smem, np); break;
-                    case REEF_TILE_128x128: if (LEVEL >= 3) OpConv<Tile128x128>::run(d, task, smem, np); break;
-                    default: break;
-                }
-            }
-            break;
-        case REEF_OP_GEMM:
-            if (LEVEL >= 2) {
-                switch (d.attr[REEF_GEMM_TILE]) {
-                    case REEF_TILE_64x64: OpGemm<Tile64x64>::run(d, task, smem, np); break;
-                    case REEF_TILE_32x128: OpGemm<Tile32x128>::run(d, task, smem, np); break;
-                    case REEF_TILE_128x128: if (LEVEL >= 3) OpGemm<Tile128x128>::run(d, task, smem, np); break;
-                    default: break;
+                const int tile = d.attr[REEF_CONV_TILE];
+                if (d.attr[REEF_CONV_MODE] == CONV_POINTWISE) {
+                    if (tile == REEF_TILE_64x64) OpConv<Tile64x64, CONV_POINTWISE>::run(d, task, smem, np);
+                    else if (tile == REEF_TILE_128x32) OpConv<Tile128x32, CONV_POINTWISE>::run(d, task, smem, np);
+                    else if (LEVEL >= 2 && tile == REEF_TILE_128x64) OpConv<Tile128x64, CONV_POINTWISE>::run(d, task, smem, np);
+                } else if (d.attr[REEF_CONV_MODE] == CONV_GENERAL) {
+                    if (tile == REEF_TILE_64x64) OpConv<Tile64x64, CONV_GENERAL>::run(d, task, smem, np);
+                    else if (tile == REEF_TILE_128x32) OpConv<Tile128x32, CONV_GENERAL>::run(d, task, smem, np);
+                    else if (LEVEL >= 2 && tile == REEF_TILE_128x64) OpConv<Tile128x64, CONV_GENERAL>::run(d, task, smem, np);
                 }
             }
             break;
@@ -260,7 +268,6 @@ __device__ __forceinline__ void run_op(const ReefDkpSide& s, int task, char* sme
         }                                                                                   \
     }
 REEF_PROXY(8, 0)
-REEF_PROXY(4, 1)
-REEF_PROXY(3, 2)
-REEF_PROXY(2, 3)
+REEF_PROXY(3, 1)
+REEF_PROXY(2, 2)
 #endif

@@ -27,10 +27,15 @@
 
 namespace reef_dev {
 
-template <int WGM_, int WGN_, int TM_, int TN_>
+template <int WGM_, int WGN_, int TM_, int TN_, int DEPTH_>
 struct Tile {
     static constexpr int WGM = WGM_, WGN = WGN_, TM = TM_, TN = TN_;
     static constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32, BK = 32;
+    // K steps whose global loads are in flight at once.  A batch-1 layer gives a
+    // workgroup only a handful of K steps, each shorter than one trip to memory, so
+    // the loads of several steps have to be outstanding together.
+    static constexpr int DEPTH = DEPTH_;
+    static_assert(DEPTH_ % 2 == 0, "the LDS buffer of a step is picked by the stage's parity");
     static constexpr int LDA = BK + 4;
     static constexpr int A_FLOATS = BM * LDA;
     static constexpr int BK_FLOATS = BK * BN;   // B tile, k-major
@@ -40,96 +45,128 @@ struct Tile {
     static_assert(WGM * WGN == 4, "four wavefronts per workgroup");
 };
 
-typedef Tile<2, 2, 2, 2> Tile128x128;
-typedef Tile<2, 2, 2, 1> Tile128x64;
-typedef Tile<2, 2, 1, 1> Tile64x64;
-typedef Tile<4, 1, 1, 1> Tile128x32;
-typedef Tile<1, 4, 1, 1> Tile32x128;
-typedef Tile<2, 2, 1, 2> Tile64x128;
+typedef Tile<2, 2, 2, 2, 2> Tile128x128;
+typedef Tile<2, 2, 2, 1, 2> Tile128x64;
+typedef Tile<2, 2, 1, 1, 2> Tile64x64;
+typedef Tile<4, 1, 1, 1, 2> Tile128x32;
+typedef Tile<1, 4, 1, 1, 2> Tile32x128;
+typedef Tile<2, 2, 1, 2, 2> Tile64x128;
+
+// All tile loads are branch-free: an element outside the tensor (row >= M,
+// k >= k_end, padding) is loaded from the tensor's first element instead and
+// replaced by zero afterwards, so every load of a K step issues back to back.
 
 // ---- A tile: rows of a K-contiguous matrix -------------------------------
-template <class T>
+// VEC: rows are 16-byte aligned at every k that is a multiple of 4 (K % 4 == 0).
+// Addresses are a uniform base plus a 32-bit element offset per lane.
+template <class T, bool VEC>
 struct ALoader {
     static constexpr int NV = T::BM / 32;  // float4 per thread per tile
-    const float* base[NV];                 // row pointer + kq*4, or null when the row is outside M
-    int k;                                 // k of this thread's first float4 in the next tile
+    // Raw loaded values plus one validity bit per element group.  The zeroing of
+    // invalid elements happens when the tile is written to LDS, not at the load: a
+    // select right behind the load would make the wavefront wait for the data at
+    // once and nothing would be in flight across K steps.
+    struct Regs { f32x4 v[NV]; unsigned ok; };
+    const float* a0;        // tensor base (also the stand-in address)
+    unsigned rowoff[NV];    // row * lda (0 when the row is outside M)
+    unsigned rowmask;       // bit i: row i of this thread is inside M
+    int k;                  // k of this thread's float4 in the next tile
     int k_end;
-    bool vec;
-    f32x4 reg[NV];
 
     __device__ __forceinline__ void init(const float* a, int lda, int m0, int M, int k_begin,
-                                         int k_end_, bool vec_) {
+                                         int k_end_) {
         const int tid = threadIdx.x;
+        a0 = a;
         k_end = k_end_;
-        vec = vec_;
-        const int kq = tid & 7;
-        k = k_begin + kq * 4;
+        k = k_begin + (tid & 7) * 4;
+        rowmask = 0;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            int row = (tid >> 3) + 32 * i;
-            base[i] = (m0 + row < M) ? a + (size_t)(m0 + row) * lda : nullptr;
+            const int row = m0 + (tid >> 3) + 32 * i;
+            const bool ok = row < M;
+            rowoff[i] = ok ? (unsigned)row * (unsigned)lda : 0u;
+            rowmask |= (ok ? 1u : 0u) << i;
         }
     }
-    __device__ __forceinline__ void load() {
+    __device__ __forceinline__ void load(Regs& r) {
+        unsigned okbits = 0;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            f32x4 v = {0.f, 0.f, 0.f, 0.f};
-            if (base[i]) {
-                const float* p = base[i] + k;
-                if (vec) {
-                    if (k < k_end) v = *(const f32x4*)p;
-                } else {
-                    if (k + 0 < k_end) v.x = p[0];
-                    if (k + 1 < k_end) v.y = p[1];
-                    if (k + 2 < k_end) v.z = p[2];
-                    if (k + 3 < k_end) v.w = p[3];
+            const bool rok = (rowmask >> i) & 1;
+            if (VEC) {
+                const bool ok = rok && k < k_end;
+                const unsigned off = ok ? rowoff[i] + (unsigned)k : 0u;
+                r.v[i] = *(const f32x4*)(a0 + off);
+                okbits |= (ok ? 0xFu : 0u) << (4 * i);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const bool ok = rok && k + e < k_end;
+                    const unsigned off = ok ? rowoff[i] + (unsigned)(k + e) : 0u;
+                    r.v[i][e] = a0[off];
+                    okbits |= (ok ? 1u : 0u) << (4 * i + e);
                 }
             }
-            reg[i] = v;
         }
+        r.ok = okbits;
         k += 32;
     }
-    __device__ __forceinline__ void store(float* As) const {
+    __device__ __forceinline__ void store(const Regs& r, float* As) const {
         const int tid = threadIdx.x;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             int row = (tid >> 3) + 32 * i;
-            *(f32x4*)(As + row * T::LDA + (tid & 7) * 4) = reg[i];
+            f32x4 v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = ((r.ok >> (4 * i + e)) & 1u) ? r.v[i][e] : 0.f;
+            *(f32x4*)(As + row * T::LDA + (tid & 7) * 4) = v;
         }
     }
 };
 
 // ---- B tile for convolution: im2col gather, one n per thread --------------
+// Thread (n, row group): n = tid % BN fixed for the whole kernel, k rows
+// tid / BN + RS * i.  For BN >= 64 a wavefront works on one k row at a time, so
+// the (channel, ky, kx) decode of the row and its carries live in scalar
+// registers; per lane only the padding test (two precomputed bit masks) and one
+// offset add remain.
 template <class T>
 struct Im2colLoader {
     static constexpr int RS = kThreads / T::BN;  // k rows covered per pass
     static constexpr int NR = 32 / RS;           // rows per thread per tile
+    static constexpr bool UNIFORM = T::BN >= 64; // one k row per wavefront
+    struct Regs { float v[NR]; unsigned ok; };   // raw values + validity bits (zeroed at store)
     const float* in;
-    int H, W, HW, kh, kw;
-    int soff, iy0, ix0;
-    bool nvalid;
+    int HW, W, kh, kw;
+    unsigned ymask, xmask;  // bit ky / kx: that tap is inside the image for this thread's pixel
+    int soff;               // iy0 * W + ix0 of this thread's pixel (may be negative)
     int k, k_end, c, ky, kx;
     int dkx, dky, dc;
-    float reg[NR];
 
     __device__ __forceinline__ void init(const float* in_, const int* a, int n0, int N, int k_begin,
                                          int k_end_) {
         const int tid = threadIdx.x;
         in = in_;
-        H = a[REEF_CONV_H];
+        const int H = a[REEF_CONV_H];
         W = a[REEF_CONV_W];
         HW = H * W;
         kh = a[REEF_CONV_KH];
         kw = a[REEF_CONV_KW];
         const int Wo = a[REEF_CONV_WO];
         const int n = n0 + (tid & (T::BN - 1));
-        nvalid = n < N;
         const int y = n / Wo, x = n - y * Wo;
-        iy0 = y * a[REEF_CONV_SH] - a[REEF_CONV_PH];
-        ix0 = x * a[REEF_CONV_SW] - a[REEF_CONV_PW];
+        const int iy0 = y * a[REEF_CONV_SH] - a[REEF_CONV_PH];
+        const int ix0 = x * a[REEF_CONV_SW] - a[REEF_CONV_PW];
         soff = iy0 * W + ix0;
+        ymask = xmask = 0;
+        if (n < N) {
+            for (int t = 0; t < kh; ++t) ymask |= ((unsigned)(iy0 + t) < (unsigned)H ? 1u : 0u) << t;
+            for (int t = 0; t < kw; ++t) xmask |= ((unsigned)(ix0 + t) < (unsigned)W ? 1u : 0u) << t;
+        }
         k_end = k_end_;
-        k = k_begin + tid / T::BN;
+        int row0 = tid / T::BN;
+        if (UNIFORM) row0 = __builtin_amdgcn_readfirstlane(row0);
+        k = k_begin + row0;
         const int khw = kh * kw;
         c = k / khw;
         const int r = k - c * khw;
@@ -140,26 +177,82 @@ struct Im2colLoader {
         dky = t % kh;
         dc = t / kh;
     }
-    __device__ __forceinline__ void load() {
+    __device__ __forceinline__ void load(Regs& r) {
+        unsigned okbits = 0;
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
-            const bool ok = nvalid && k < k_end && (unsigned)(iy0 + ky) < (unsigned)H &&
-                            (unsigned)(ix0 + kx) < (unsigned)W;
-            const int off = c * HW + ky * W + kx + soff;
-            reg[i] = ok ? in[off] : 0.0f;
+            const bool ok = (k < k_end) && (((ymask >> ky) & (xmask >> kx) & 1u) != 0);
+            const unsigned off = ok ? (unsigned)(c * HW + ky * W + kx + soff) : 0u;
+            r.v[i] = in[off];
+            okbits |= (ok ? 1u : 0u) << i;
+            // advance (c, ky, kx) by RS rows, mixed radix (kh, kw), without branches
             k += RS;
             kx += dkx;
-            if (kx >= kw) { kx -= kw; ++ky; }
-            ky += dky;
-            if (ky >= kh) { ky -= kh; ++c; }
-            c += dc;
+            const int cx = kx >= kw ? 1 : 0;
+            kx -= kw & -cx;
+            ky += dky + cx;
+            const int cy = ky >= kh ? 1 : 0;
+            ky -= kh & -cy;
+            c += dc + cy;
         }
+        r.ok = okbits;
     }
-    __device__ __forceinline__ void store(float* Bs) const {
+    __device__ __forceinline__ void store(const Regs& r, float* Bs) const {
         const int tid = threadIdx.x;
         const int nl = tid & (T::BN - 1), kr0 = tid / T::BN;
 #pragma unroll
-        for (int i = 0; i < NR; ++i) Bs[(kr0 + RS * i) * T::BN + nl] = reg[i];
+        for (int i = 0; i < NR; ++i) Bs[(kr0 + RS * i) * T::BN + nl] = ((r.ok >> i) & 1u) ? r.v[i] : 0.0f;
+    }
+};
+
+// ---- B tile for pointwise convolution (1x1, stride 1, no padding, N % 4 == 0) ----
+// The im2col matrix is the input itself, [K = Cin][N = H*W] row-major: 128-bit
+// loads along n, 128-bit LDS stores, one offset add per K step.
+template <class T>
+struct PointwiseLoader {
+    static constexpr int C4 = T::BN / 4;                 // float4 per tile row
+    static constexpr int NF = 32 * C4 / kThreads;        // float4 per thread per tile
+    static constexpr int RSTEP = kThreads / C4;          // rows between a thread's float4s
+    static_assert(NF >= 1, "tile narrower than one pass");
+    struct Regs { f32x4 v[NF]; unsigned ok; };
+    const float* in;
+    unsigned off;   // element offset of this thread's first float4 in the next tile
+    unsigned step;  // RSTEP * N
+    unsigned tile;  // 32 * N
+    int k, k_end;
+    bool nvalid;
+
+    __device__ __forceinline__ void init(const float* in_, int n0, int N, int k_begin, int k_end_) {
+        const int tid = threadIdx.x;
+        in = in_;
+        const int row = tid / C4, col = (tid % C4) * 4;
+        nvalid = n0 + col < N;
+        k = k_begin + row;
+        k_end = k_end_;
+        off = (unsigned)k * (unsigned)N + (unsigned)(n0 + col);
+        step = (unsigned)RSTEP * (unsigned)N;
+        tile = 32u * (unsigned)N;
+    }
+    __device__ __forceinline__ void load(Regs& r) {
+        unsigned okbits = 0;
+#pragma unroll
+        for (int i = 0; i < NF; ++i) {
+            const bool ok = nvalid && (k + RSTEP * i) < k_end;
+            r.v[i] = *(const f32x4*)(in + (ok ? off + step * i : 0u));
+            okbits |= (ok ? 1u : 0u) << i;
+        }
+        r.ok = okbits;
+        off += tile;
+        k += 32;
+    }
+    __device__ __forceinline__ void store(const Regs& r, float* Bs) const {
+        const int tid = threadIdx.x;
+        const int row = tid / C4, col = (tid % C4) * 4;
+#pragma unroll
+        for (int i = 0; i < NF; ++i) {
+            const bool ok = (r.ok >> i) & 1u;
+            *(f32x4*)(Bs + (row + RSTEP * i) * T::BN + col) = ok ? r.v[i] : f32x4{0.f, 0.f, 0.f, 0.f};
+        }
     }
 };
 
@@ -168,30 +261,37 @@ template <class T>
 struct BknLoader {
     static constexpr int RS = kThreads / T::BN;
     static constexpr int NR = 32 / RS;
-    const float* col;  // B + n, or null
+    struct Regs { float v[NR]; unsigned ok; };
+    const float* b0;
+    int n;
+    bool nvalid;
     int ldb, k, k_end;
-    float reg[NR];
     __device__ __forceinline__ void init(const float* b, int ldb_, int n0, int N, int k_begin,
                                          int k_end_) {
         const int tid = threadIdx.x;
-        const int n = n0 + (tid & (T::BN - 1));
-        col = n < N ? b + n : nullptr;
+        n = n0 + (tid & (T::BN - 1));
+        nvalid = n < N;
+        b0 = b;
         ldb = ldb_;
         k = k_begin + tid / T::BN;
         k_end = k_end_;
     }
-    __device__ __forceinline__ void load() {
+    __device__ __forceinline__ void load(Regs& r) {
+        unsigned okbits = 0;
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
-            reg[i] = (col && k < k_end) ? col[(size_t)k * ldb] : 0.0f;
+            const bool ok = nvalid && k < k_end;
+            r.v[i] = b0[ok ? (unsigned)k * (unsigned)ldb + (unsigned)n : 0u];
+            okbits |= (ok ? 1u : 0u) << i;
             k += RS;
         }
+        r.ok = okbits;
     }
-    __device__ __forceinline__ void store(float* Bs) const {
+    __device__ __forceinline__ void store(const Regs& r, float* Bs) const {
         const int tid = threadIdx.x;
         const int nl = tid & (T::BN - 1), kr0 = tid / T::BN;
 #pragma unroll
-        for (int i = 0; i < NR; ++i) Bs[(kr0 + RS * i) * T::BN + nl] = reg[i];
+        for (int i = 0; i < NR; ++i) Bs[(kr0 + RS * i) * T::BN + nl] = ((r.ok >> i) & 1u) ? r.v[i] : 0.0f;
     }
 };
 
@@ -200,42 +300,54 @@ template <class T, bool B_NMAJOR>
 __device__ __forceinline__ void mma_step(const float* As, const float* Bs, f32x16 (&acc)[T::TM][T::TN],
                                          int wm0, int wn0) {
     const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
+    // All operand fragments of the K step are fetched from LDS first, then the 16 x
+    // TM x TN MFMAs issue back to back: one LDS round trip per step is exposed
+    // instead of one per group of four MFMAs.
+    f32x4 af[4][T::TM];
+    f32x4 bf[4][T::TN];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        f32x4 af[T::TM];
-        f32x4 bf[T::TN];
 #pragma unroll
         for (int tm = 0; tm < T::TM; ++tm)
-            af[tm] = *(const f32x4*)(As + (wm0 + tm * 32 + l32) * T::LDA + 8 * j + 4 * h);
+            af[j][tm] = *(const f32x4*)(As + (wm0 + tm * 32 + l32) * T::LDA + 8 * j + 4 * h);
 #pragma unroll
         for (int tn = 0; tn < T::TN; ++tn) {
             if (B_NMAJOR) {
-                bf[tn] = *(const f32x4*)(Bs + (wn0 + tn * 32 + l32) * T::LDA + 8 * j + 4 * h);
+                bf[j][tn] = *(const f32x4*)(Bs + (wn0 + tn * 32 + l32) * T::LDA + 8 * j + 4 * h);
             } else {
                 const float* bp = Bs + (8 * j + 4 * h) * T::BN + wn0 + tn * 32 + l32;
-                bf[tn].x = bp[0];
-                bf[tn].y = bp[T::BN];
-                bf[tn].z = bp[2 * T::BN];
-                bf[tn].w = bp[3 * T::BN];
+                bf[j][tn].x = bp[0];
+                bf[j][tn].y = bp[T::BN];
+                bf[j][tn].z = bp[2 * T::BN];
+                bf[j][tn].w = bp[3 * T::BN];
             }
         }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
             for (int tm = 0; tm < T::TM; ++tm)
 #pragma unroll
                 for (int tn = 0; tn < T::TN; ++tn)
-                    acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[tm][t], bf[tn][t],
+                    acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[j][tm][t], bf[j][tn][t],
                                                                        acc[tm][tn], 0, 0, 0);
-    }
 }
 
-// Double-buffered K loop shared by conv and GEMM.  Returns false when the
-// preemption flag was seen (the whole workgroup leaves together: the value
-// read by thread 0 is published through LDS before the step's barrier).
+// K loop shared by conv and GEMM.  Global loads run DEPTH steps ahead of the
+// matrix cores (register staging), LDS is double-buffered, one barrier per step:
+//   step it:  regs[it % DEPTH] -> LDS[it & 1];  issue loads of step it + DEPTH;
+//             barrier;  MFMAs on LDS[it & 1]
+// The barrier of step it also proves every wavefront finished the MFMAs of step
+// it - 1, whose LDS buffer step it + 1 overwrites.
+// Returns false when the preemption flag was seen.  The whole workgroup leaves
+// together: thread 0 reads the flag one step ahead (the load overlaps the MFMAs)
+// and publishes it through LDS before the step's barrier.
 template <class T, bool B_NMAJOR, class LA, class LB, class Poll>
 __device__ __forceinline__ bool k_loop(LA& la, LB& lb, int nk, float* smem, f32x16 (&acc)[T::TM][T::TN],
                                        const Poll& poll) {
+    constexpr int D = T::DEPTH;
     float* As = smem;
     float* Bs = smem + 2 * T::A_FLOATS;
     int* sflag = (int*)(smem + 2 * (T::A_FLOATS + T::B_FLOATS));
@@ -248,35 +360,49 @@ __device__ __forceinline__ bool k_loop(LA& la, LB& lb, int nk, float* smem, f32x
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[tm][tn][r] = 0.0f;
 
+    typename LA::Regs ra[D];
+    typename LB::Regs rb[D];
     if (Poll::enabled && threadIdx.x == 0) *sflag = 0;
-    la.load();
-    lb.load();
-    la.store(As);
-    lb.store(Bs);
-    __syncthreads();
-    for (int it = 0; it < nk; ++it) {
-        const int cur = it & 1;
-        const bool more = it + 1 < nk;
-        int pf = 0;
-        if (more) {
-            la.load();
-            lb.load();
-        }
-        if (Poll::enabled && threadIdx.x == 0) pf = poll.load();
-        mma_step<T, B_NMAJOR>(As + cur * T::A_FLOATS, Bs + cur * T::B_FLOATS, acc, wm0, wn0);
-        if (more) {
-            la.store(As + (cur ^ 1) * T::A_FLOATS);
-            lb.store(Bs + (cur ^ 1) * T::B_FLOATS);
-        }
-        if (Poll::enabled && threadIdx.x == 0 && pf) *sflag = 1;
-        __syncthreads();
-        if (Poll::enabled && *sflag) return false;
+    // Loads past the last K step are issued too: the loaders mask them (k >= k_end)
+    // to a stand-in address, which keeps the steady state free of branches.
+#pragma unroll
+    for (int s = 0; s < D; ++s) {
+        la.load(ra[s]);
+        lb.load(rb[s]);
     }
-    return true;
+    int pf = 0;
+    int it = 0;
+    for (;;) {
+#pragma unroll
+        for (int s = 0; s < D; ++s) {
+            if (it >= nk) return true;
+            const int cur = s & 1;  // D is even, so step parity == stage parity
+            la.store(ra[s], As + cur * T::A_FLOATS);
+            lb.store(rb[s], Bs + cur * T::B_FLOATS);
+            if (Poll::enabled && threadIdx.x == 0) {
+                if (pf) *sflag = 1;
+                pf = poll.load();
+            }
+            __syncthreads();
+            if (Poll::enabled && *sflag) return false;
+            // refill this stage next to the MFMAs: the address arithmetic of the
+            // loads fills the issue slots the dependent MFMA chain leaves free
+            la.load(ra[s]);
+            lb.load(rb[s]);
+            mma_step<T, B_NMAJOR>(As + cur * T::A_FLOATS, Bs + cur * T::B_FLOATS, acc, wm0, wn0);
+            ++it;
+        }
+    }
 }
 
 // ---- reef_conv2d ------------------------------------------------------------
-template <class T, class Poll>
+// MODE selects the tile loaders, one K loop per kernel symbol:
+//   CONV_GENERAL    im2col gather, 128-bit weight loads        (K % 4 == 0)
+//   CONV_POINTWISE  1x1 / stride 1 / no padding / N % 4 == 0:  128-bit loads on both operands
+//   CONV_UNALIGNED  im2col gather, element-wise weight loads    (any K; the 7x7x3 stem)
+enum { CONV_GENERAL = 0, CONV_POINTWISE = 1, CONV_UNALIGNED = 2 };
+
+template <class T, int MODE, class Poll>
 __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, char* smem_raw,
                                             const Poll& poll) {
   int M, N, split_k, split, rem, m0, n0;
@@ -301,12 +427,21 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
     const int k_end = min(K, k_begin + k_chunk);
     const int nk = (k_end - k_begin + 31) >> 5;
 
-    ALoader<T> la;
-    Im2colLoader<T> lb;
-    la.init((const float*)d.ptr[1], K, m0, M, k_begin, k_end, (K & 3) == 0);
-    lb.init((const float*)d.ptr[0], a, n0, N, k_begin, k_end);
-
-    if (!k_loop<T, false>(la, lb, nk, smem, acc, poll)) return false;
+    bool ok;
+    if (MODE == CONV_POINTWISE) {
+        ALoader<T, true> la;
+        PointwiseLoader<T> lp;
+        la.init((const float*)d.ptr[1], K, m0, M, k_begin, k_end);
+        lp.init((const float*)d.ptr[0], n0, N, k_begin, k_end);
+        ok = k_loop<T, false>(la, lp, nk, smem, acc, poll);
+    } else {
+        Im2colLoader<T> lb;
+        lb.init((const float*)d.ptr[0], a, n0, N, k_begin, k_end);
+        ALoader<T, MODE == CONV_GENERAL> la;
+        la.init((const float*)d.ptr[1], K, m0, M, k_begin, k_end);
+        ok = k_loop<T, false>(la, lb, nk, smem, acc, poll);
+    }
+    if (!ok) return false;
   }
 
     // Everything the epilogue needs is re-read from the argument block here, so the
@@ -355,18 +490,19 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int m = m0 + wm0 + tm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                    if (m < M && n < N) part[(size_t)m * N + n] = acc[tm][tn][r];
+                    if (m < M && n < N) store_agent(part + (size_t)m * N + n, acc[tm][tn][r]);
                 }
             }
-        __threadfence();  // release the partial tile device-wide before counting in
+        // every store of this workgroup has completed at device scope before it counts in
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
         if (threadIdx.x == 0) {
-            const int old = atomicAdd(&counters[rem], 1);
+            const int old = __hip_atomic_fetch_add(&counters[rem], 1, __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
             *s_last = (old == split_k - 1);
         }
         __syncthreads();
         if (!*s_last) return true;
-        __threadfence();  // acquire the other splits' partial tiles
 #pragma unroll
         for (int tm = 0; tm < T::TM; ++tm)
 #pragma unroll
@@ -377,13 +513,14 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
                     const int m = m0 + wm0 + tm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
                     if (m < M && n < N) {
                         const size_t idx = (size_t)m * N + n;
-                        float v = ws[idx];
-                        for (int s = 1; s < split_k; ++s) v += ws[(size_t)s * MN + idx];
+                        float v = load_agent(ws + idx);
+                        for (int s = 1; s < split_k; ++s) v += load_agent(ws + (size_t)s * MN + idx);
                         ep.store(dst, v, m, idx);
                     }
                 }
             }
-        if (threadIdx.x == 0) counters[rem] = 0;  // ready for the next run
+        if (threadIdx.x == 0)  // ready for the next run
+            __hip_atomic_store(&counters[rem], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         return true;
     }
 
@@ -402,7 +539,10 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
 }
 
 // ---- reef_gemm ----------------------------------------------------------------
-template <class T, class Poll>
+// TRANS_B: B stored [N][K] (dense layers, Q.K^T) -- both operands take 128-bit row
+// loads, so K, lda, ldb and the batch strides must be multiples of 4 floats.
+// !TRANS_B: B stored [K][N] (P.V) -- element-wise B loads, 128-bit A loads.
+template <class T, bool TRANS_B, class Poll>
 __device__ __forceinline__ bool gemm_body(const ReefOpDesc& d, int task, char* smem_raw,
                                           const Poll& poll) {
     const int* a = d.attr;
@@ -421,14 +561,14 @@ __device__ __forceinline__ bool gemm_body(const ReefOpDesc& d, int task, char* s
     float* smem = (float*)smem_raw;
     f32x16 acc[T::TM][T::TN];
 
-    ALoader<T> la;
-    la.init(A, lda, m0, M, 0, K, ((K | lda) & 3) == 0);
     bool ok;
-    if (a[REEF_GEMM_TRANS_B]) {
+    ALoader<T, true> la;
+    la.init(A, lda, m0, M, 0, K);
+    if (TRANS_B) {
         // B is [N][K]: stage it exactly like A (rows = n).
-        typedef Tile<T::WGN, T::WGM, T::TN, T::TM> TB;  // BM of TB == BN of T
-        ALoader<TB> lb;
-        lb.init(B, ldb, n0, N, 0, K, ((K | ldb) & 3) == 0);
+        typedef Tile<T::WGN, T::WGM, T::TN, T::TM, T::DEPTH> TB;  // BM of TB == BN of T
+        ALoader<TB, true> lb;
+        lb.init(B, ldb, n0, N, 0, K);
         ok = k_loop<T, true>(la, lb, nk, smem, acc, poll);
     } else {
         BknLoader<T> lb;

@@ -484,7 +484,9 @@ void REEFScheduler::dynamic_kernel_padding(std::shared_ptr<Task>& rt_task) {
                 cand->sync_dirty = false;
             }
             const TransExecutor::KernelArg& ka = be_exe.trans_args[cand->kernel_offset];
-            // the proxy class that holds both bodies sets the register budget of the launch
+            // the proxy class that holds both bodies sets the register budget of the launch;
+            // a kernel that is in no proxy runs single-sided
+            if (rt_args.proxy_level < 0 || ka.proxy_level < 0) continue;
             const int level = std::max(rt_args.proxy_level, ka.proxy_level);
             PadDecision d = decide_padding(rt_args, ka, cand->block_offset, proxy_res[level], num_cus,
                                            num_xcds);

@@ -63,7 +63,7 @@ class GraphBuilder:
         # (the profile is keyed by kernel name, model.cpp:57-80).
         self.unique_names = True
         # split-K folded inside the conv kernel (False: separate reef_splitk_reduce launch)
-        self.fused_reduce = True
+        self.fused_reduce = False
 
     # ------------------------------------------------------------ storages
     def _storage(self, name, size, stype="float32"):
@@ -165,11 +165,19 @@ class GraphBuilder:
         nbytes = 4 * (x.size + M * K + M * N + (M if bias else 0) + (M * N if residual is not None else 0)
                       + (2 * M if affine else 0))
         base = [cin, H, W, cout, Ho, Wo, kh, kw, sh, sw, ph, pw]
-        kname = "reef_conv2d_" + t["tile"]
+        # loader family: pointwise (1x1/s1/p0, N % 4 == 0), unaligned (K % 4 != 0), general
+        if (kh, kw, sh, sw, ph, pw) == (1, 1, 1, 1, 0, 0) and N % 4 == 0 and K % 4 == 0:
+            mode, fam = 1, "pw_"
+        elif K % 4 != 0:
+            mode, fam = 2, "u_"
+        else:
+            mode, fam = 0, ""
+        kname = "reef_conv2d_" + fam + t["tile"]
         if out2 is not None:
             nbytes += 4 * (M * N + M)
         if t["split_k"] == 1:
-            attrs = base + [flags, act, t["tile_id"], 1, t["k_chunk"], t["m_tiles"], t["n_tiles"], act2]
+            attrs = base + [flags, act, t["tile_id"], 1, t["k_chunk"], t["m_tiles"], t["n_tiles"], act2,
+                            0, mode]
             self._emit(kname, t["tasks"], [x.idx, w.idx, out.idx] + opt, attrs, "conv2d", flops,
                        nbytes, t["est_us"])
         elif fused_reduce:
@@ -178,13 +186,13 @@ class GraphBuilder:
             ws = self.workspace(t["split_k"] * M * N)
             sync_idx, sync_off = self._sync_counters(t["m_tiles"] * t["n_tiles"])
             attrs = base + [flags | F_FUSED_REDUCE, act, t["tile_id"], t["split_k"], t["k_chunk"],
-                            t["m_tiles"], t["n_tiles"], act2, sync_off]
+                            t["m_tiles"], t["n_tiles"], act2, sync_off, mode]
             self._emit(kname, t["tasks"], [x.idx, w.idx, out.idx] + opt + [ws.idx, sync_idx], attrs,
                        "conv2d", flops, nbytes, t["est_us"])
         else:
             ws = self.workspace(t["split_k"] * M * N)
             attrs = base + [0, ACT_NONE, t["tile_id"], t["split_k"], t["k_chunk"], t["m_tiles"],
-                            t["n_tiles"], ACT_NONE]
+                            t["n_tiles"], ACT_NONE, 0, mode]
             self._emit(kname, t["tasks"], [x.idx, w.idx, ws.idx], attrs, "conv2d", flops,
                        4 * (x.size + M * K + t["split_k"] * M * N), t["est_us"])
             self._emit("reef_splitk_reduce", math.ceil(M * N / 1024), [ws.idx, out.idx] + opt,
@@ -353,7 +361,11 @@ class GraphBuilder:
             args.append(bias.idx)
         flops = 2 * batch * M * N * K
         self.flops += flops
-        self._emit("reef_gemm_" + t["tile"], batch * t["m_tiles"] * t["n_tiles"], args,
+        assert K % 4 == 0 and lda % 4 == 0 and stride_a % 4 == 0, "gemm operands must be 16-byte aligned"
+        if trans_b:
+            assert ldb % 4 == 0 and stride_b % 4 == 0, "gemm operands must be 16-byte aligned"
+        self._emit("reef_gemm_%s_%s" % ("nt" if trans_b else "nn", t["tile"]),
+                   batch * t["m_tiles"] * t["n_tiles"], args,
                    [batch, M, N, K, 1 if trans_b else 0, flags, act, float_bits(alpha), t["tile_id"],
                     t["m_tiles"], t["n_tiles"], lda, ldb, ldc, stride_a, stride_b, stride_c],
                    "gemm", flops, 4 * batch * (M * K + N * K + M * N), t["est_us"])

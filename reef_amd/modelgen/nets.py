@@ -35,7 +35,7 @@ def image_input(name, shape, seed=rng.BASE_SEED):
 
 
 def resnet(num_layers=152, image=(3, 224, 224), classes=1000, name=None, seed=rng.BASE_SEED,
-           fused_reduce=True, fuse_act=True):
+           fused_reduce=False, fuse_act=True):
     """fused_reduce: fold split-K inside the conv kernels.  fuse_act: let the unit's last
     conv also write the next unit's activated input (one kernel instead of conv + add/relu)."""
     if num_layers >= 50:
