@@ -160,6 +160,7 @@ enum {
     REEF_CONV_ACT2,      /* activation of the second output (REEF_F_DUAL) */
     REEF_CONV_SYNC_OFF,  /* first counter of this launch inside the sync storage (ints) */
     REEF_CONV_MODE,      /* REEF_CONV_MODE_*: must match the entry symbol's family */
+    REEF_CONV_DST_OFF,   /* element offset added to dst (and out2): channel slice of a concat buffer */
     REEF_CONV_NATTR
 };
 #define REEF_F_BIAS 1
@@ -189,8 +190,9 @@ enum {
 
 /* ---- reef_splitk_reduce: out = act(sum_s ws[s] (+res)(+bias)(*scale+shift)), s ascending ----
  * ptr: ws, out, then optional bias, residual, (scale, shift), (out2, shift2) (same flag order).
- * attr: M, N, split_k, flags, act, act2.   tasks = ceil(M*N / 1024) (4 elements per thread). */
-enum { REEF_RED_M = 0, REEF_RED_N, REEF_RED_SPLIT_K, REEF_RED_FLAGS, REEF_RED_ACT, REEF_RED_ACT2, REEF_RED_NATTR };
+ * attr: M, N, split_k, flags, act, act2, dst_off (element offset added to out and out2).   tasks = ceil(M*N / 1024) (4 elements per thread). */
+enum { REEF_RED_M = 0, REEF_RED_N, REEF_RED_SPLIT_K, REEF_RED_FLAGS, REEF_RED_ACT, REEF_RED_ACT2,
+       REEF_RED_DST_OFF, REEF_RED_NATTR };
 
 /* ---- reef_dwconv2d: depthwise k x k convolution + bias + activation (bandwidth-bound) ----
  * ptr: in, W[C][kh][kw], out, bias(optional by flag).

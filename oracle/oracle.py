@@ -273,6 +273,7 @@ class GraphOracle:
         if name.startswith("reef_conv2d"):
             Cin, H, W, Cout, Ho, Wo, kh, kw, sh, sw, ph, pw, flags, act, _tile, split_k = a[:16]
             act2 = a[19] if len(a) > 19 else 0   # a[20]: first sync counter (device detail)
+            dst_off = a[22] if len(a) > 22 else 0  # a[21]: loader family (device detail)
             xin = P[0][:Cin * H * W].reshape(Cin, H, W)
             wgt = P[1][:Cout * Cin * kh * kw].reshape(Cout, Cin, kh, kw)
             if split_k > 1 and not (flags & 16):
@@ -290,12 +291,14 @@ class GraphOracle:
             out = conv2d(xin, wgt, bias,
                          None if res is None else res[:Cout * Ho * Wo].reshape(Cout, Ho, Wo),
                          scale, shift, (sh, sw), (ph, pw), 1, act, 6.0, acc64)
-            P[2][:out.size] = out.reshape(-1)
+            P[2][dst_off:dst_off + out.size] = out.reshape(-1)
             if out2 is not None:
-                out2[:out.size] = eltwise(out.reshape(Cout, -1), shift=shift2[:Cout], act=act2).reshape(-1)
+                out2[dst_off:dst_off + out.size] = eltwise(out.reshape(Cout, -1), shift=shift2[:Cout],
+                                                           act=act2).reshape(-1)
         elif name == "reef_splitk_reduce":
             M, N, split_k, flags, act = a[:5]
             act2 = a[5] if len(a) > 5 else 0
+            dst_off = a[6] if len(a) > 6 else 0
             bias, res, scale, shift, out2, shift2 = self._conv_opt(P, 2, flags)
             acc = np.zeros(M * N, np.float32)
             ws = P[0].view(np.float32)
@@ -313,9 +316,9 @@ class GraphOracle:
             elif act == 2:
                 v = np.minimum(np.maximum(v, 0), 6.0)
             v = v.astype(np.float32)
-            P[1][:M * N] = v.reshape(-1)
+            P[1][dst_off:dst_off + M * N] = v.reshape(-1)
             if out2 is not None:
-                out2[:M * N] = eltwise(v, shift=shift2[:M], act=act2).reshape(-1)
+                out2[dst_off:dst_off + M * N] = eltwise(v, shift=shift2[:M], act=act2).reshape(-1)
         elif name == "reef_dwconv2d":
             C, H, W, Ho, Wo, kh, kw, sh, sw, ph, pw, flags, act = a[:13]
             bias = P[3] if flags & 1 else None

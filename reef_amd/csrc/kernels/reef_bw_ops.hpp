@@ -27,9 +27,10 @@ __device__ __forceinline__ void splitk_reduce_body(const ReefOpDesc& d, int task
     const int M = a[REEF_RED_M], N = a[REEF_RED_N], S = a[REEF_RED_SPLIT_K];
     const size_t MN = (size_t)M * N;
     const float* ws = (const float*)d.ptr[0];
-    float* out = (float*)d.ptr[1];
+    float* out = (float*)d.ptr[1] + a[REEF_RED_DST_OFF];
     Epilogue ep;
     ep.unpack(d, 2, a[REEF_RED_FLAGS], a[REEF_RED_ACT], a[REEF_RED_ACT2]);
+    if (ep.out2) ep.out2 += a[REEF_RED_DST_OFF];
     const size_t i0 = ((size_t)task * kThreads + threadIdx.x) * 4;
     if (i0 >= MN) return;
     if ((MN & 3) == 0) {

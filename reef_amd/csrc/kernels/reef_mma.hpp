@@ -452,11 +452,14 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
     const int* a = d.attr;
     const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5, wave = threadIdx.x >> 6;
     const int wm0 = (wave / T::WGN) * (T::TM * 32), wn0 = (wave % T::WGN) * (T::TN * 32);
-    float* dst = (float*)d.ptr[2];
     const int flags = a[REEF_CONV_FLAGS];
     const size_t MN = (size_t)M * N;
+    // plain split-K writes partial tiles to the workspace; the offset belongs to the
+    // launch that writes the real output
+    const bool to_ws = split_k > 1 && !(flags & REEF_F_FUSED_REDUCE);
+    float* dst = (float*)d.ptr[2] + (to_ws ? 0 : a[REEF_CONV_DST_OFF]);
 
-    if (split_k > 1 && !(flags & REEF_F_FUSED_REDUCE)) {
+    if (to_ws) {
         // plain split-K: partial tile to the workspace, reef_splitk_reduce folds
         float* ws = dst + (size_t)split * MN;
 #pragma unroll
@@ -475,6 +478,7 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
 
     Epilogue ep;
     ep.unpack(d, 3, flags, a[REEF_CONV_ACT], a[REEF_CONV_ACT2]);
+    if (ep.out2) ep.out2 += a[REEF_CONV_DST_OFF];
     if (split_k > 1) {
         // fused split-K: store the partial, count in, the last arrival folds all
         // partials in ascending split order (fixed order => same bits whoever is last)

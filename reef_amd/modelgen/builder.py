@@ -121,10 +121,12 @@ class GraphBuilder:
         self.kernel_est_us.append(float(est_us))
 
     def conv2d(self, x, cout, k, stride=1, pad=0, bias=True, act=ACT_RELU, residual=None,
-               affine=False, force=None, dual_act=None, fused_reduce=None):
+               affine=False, force=None, dual_act=None, fused_reduce=None, out=None, out_channel=0):
         """Fused conv + (residual) + (bias) + (scale, shift) + activation on MFMA.
         dual_act: also emit out2 = dual_act(out + shift2[c]) and return (out, out2).
-        fused_reduce: fold split-K inside the kernel (default: self.fused_reduce)."""
+        fused_reduce: fold split-K inside the kernel (default: self.fused_reduce).
+        out / out_channel: write into channels [out_channel, out_channel + cout) of an existing
+        tensor (a concatenation buffer) instead of a new one."""
         if fused_reduce is None:
             fused_reduce = self.fused_reduce
         kh, kw = (k, k) if isinstance(k, int) else k
@@ -150,7 +152,12 @@ class GraphBuilder:
             opt.append(self.param((cout,), 0.1, value=None).idx)   # scale ~ N(0, 0.1) + 1 below
             self.params[-1] = (self.params[-1][0], self.params[-1][1] + 1.0)
             opt.append(self.param((cout,), 0.01).idx)
-        out = self.temp((cout, Ho, Wo))
+        dst_off = 0
+        if out is None:
+            out = self.temp((cout, Ho, Wo))
+        else:
+            assert out.shape[1:] == (Ho, Wo) and out_channel + cout <= out.shape[0]
+            dst_off = out_channel * Ho * Wo
         out2 = None
         if dual_act is not None:
             assert not affine
@@ -177,7 +184,7 @@ class GraphBuilder:
             nbytes += 4 * (M * N + M)
         if t["split_k"] == 1:
             attrs = base + [flags, act, t["tile_id"], 1, t["k_chunk"], t["m_tiles"], t["n_tiles"], act2,
-                            0, mode]
+                            0, mode, dst_off]
             self._emit(kname, t["tasks"], [x.idx, w.idx, out.idx] + opt, attrs, "conv2d", flops,
                        nbytes, t["est_us"])
         elif fused_reduce:
@@ -186,17 +193,17 @@ class GraphBuilder:
             ws = self.workspace(t["split_k"] * M * N)
             sync_idx, sync_off = self._sync_counters(t["m_tiles"] * t["n_tiles"])
             attrs = base + [flags | F_FUSED_REDUCE, act, t["tile_id"], t["split_k"], t["k_chunk"],
-                            t["m_tiles"], t["n_tiles"], act2, sync_off, mode]
+                            t["m_tiles"], t["n_tiles"], act2, sync_off, mode, dst_off]
             self._emit(kname, t["tasks"], [x.idx, w.idx, out.idx] + opt + [ws.idx, sync_idx], attrs,
                        "conv2d", flops, nbytes, t["est_us"])
         else:
             ws = self.workspace(t["split_k"] * M * N)
             attrs = base + [0, ACT_NONE, t["tile_id"], t["split_k"], t["k_chunk"], t["m_tiles"],
-                            t["n_tiles"], ACT_NONE, 0, mode]
+                            t["n_tiles"], ACT_NONE, 0, mode, 0]
             self._emit(kname, t["tasks"], [x.idx, w.idx, ws.idx], attrs, "conv2d", flops,
                        4 * (x.size + M * K + t["split_k"] * M * N), t["est_us"])
             self._emit("reef_splitk_reduce", math.ceil(M * N / 1024), [ws.idx, out.idx] + opt,
-                       [M, N, t["split_k"], flags, act, act2], "splitk_reduce", 0,
+                       [M, N, t["split_k"], flags, act, act2, dst_off], "splitk_reduce", 0,
                        4 * ((t["split_k"] + 1) * M * N), 2.0)
         return out if out2 is None else (out, out2)
 

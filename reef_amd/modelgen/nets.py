@@ -103,3 +103,234 @@ def mocked_kernel(name="mocked_kernel"):
     g.mocked("add", b, a, temp)
     g.mocked("multiply", temp, c, out)
     return g
+
+
+def mobilenet_v2(image=(3, 224, 224), classes=1000, name="mobilenetv2", seed=rng.BASE_SEED):
+    """MobileNetV2, width 1.0: 3x3/2 stem, 17 inverted-residual blocks (1x1 expand + ReLU6,
+    depthwise 3x3 + ReLU6, linear 1x1 projection, residual add when stride 1 and equal
+    channels), 1x1 to 1280, global average pool, classifier.  Batch norms are folded
+    into the convolutions as biases; the residual add is the projection's epilogue."""
+    g = GraphBuilder(name, seed)
+    x = g.input("data", image)
+    x = g.conv2d(x, 32, 3, 2, 1, bias=True, act=ACT_RELU6)
+    cfg = [(1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1), (6, 160, 3, 2),
+           (6, 320, 1, 1)]
+    cin = 32
+    for t, c, n, s in cfg:
+        for i in range(n):
+            stride = s if i == 0 else 1
+            y = x
+            if t != 1:
+                y = g.conv2d(y, cin * t, 1, 1, 0, bias=True, act=ACT_RELU6)
+            y = g.dwconv2d(y, 3, stride, 1, bias=True, act=ACT_RELU6)
+            res = x if (stride == 1 and cin == c) else None
+            x = g.conv2d(y, c, 1, 1, 0, bias=True, act=ACT_NONE, residual=res)
+            cin = c
+    x = g.conv2d(x, 1280, 1, 1, 0, bias=True, act=ACT_RELU6)
+    pooled = g.global_avgpool(x)
+    logits = g.dense(pooled, classes, bias=True)
+    out = g.softmax(logits, 1, classes)
+    g.mark_output(out)
+    return g
+
+
+def densenet(blocks=(6, 12, 48, 32), growth=32, image=(3, 224, 224), classes=1000, name="densenet201",
+             seed=rng.BASE_SEED):
+    """DenseNet-BC (201: blocks 6/12/48/32, growth 32): every layer reads the running
+    concatenation through its own BN + ReLU (an elementwise scale/shift kernel, it cannot
+    be folded into a convolution because each consumer has its own statistics), then
+    1x1 -> 128 (+bias, ReLU) and 3x3 -> 32, which writes straight into its channel slice
+    of the concatenation buffer."""
+    g = GraphBuilder(name, seed)
+    x = g.input("data", image)
+    x = g.conv2d(x, 2 * growth, 7, 2, 3, bias=True, act=ACT_RELU)
+    x = g.pool2d(x, 3, 2, 1, "max")
+    c = 2 * growth
+    for bi, n_layers in enumerate(blocks):
+        _, H, W = x.shape
+        total = c + n_layers * growth
+        buf = g.temp((total, H, W))
+        g.copy_into(x, buf, 0)
+        for li in range(n_layers):
+            cur = c + li * growth
+            view = type(x)(buf.idx, (cur, H, W))          # first `cur` channels of the buffer
+            a = g.eltwise(view, scale=True, shift=True, act=ACT_RELU)
+            y = g.conv2d(a, 4 * growth, 1, 1, 0, bias=True, act=ACT_RELU)
+            g.conv2d(y, growth, 3, 1, 1, bias=False, act=ACT_NONE, out=buf, out_channel=cur)
+        c = total
+        x = buf
+        if bi != len(blocks) - 1:
+            a = g.eltwise(x, scale=True, shift=True, act=ACT_RELU)
+            y = g.conv2d(a, c // 2, 1, 1, 0, bias=False, act=ACT_NONE)
+            x = g.pool2d(y, 2, 2, 0, "avg")
+            c = c // 2
+    a = g.eltwise(x, scale=True, shift=True, act=ACT_RELU)
+    pooled = g.global_avgpool(a)
+    logits = g.dense(pooled, classes, bias=True)
+    out = g.softmax(logits, 1, classes)
+    g.mark_output(out)
+    return g
+
+
+def inception_v3(image=(3, 299, 299), classes=1000, name="inceptionv3", seed=rng.BASE_SEED):
+    """Inception-v3 (the 299x299 network): every convolution is conv + folded BN + ReLU;
+    branch outputs are written straight into their channel slices of the block output."""
+    g = GraphBuilder(name, seed)
+    T = None
+
+    def conv(x, cout, k, s=1, p=0, out=None, ch=0):
+        return g.conv2d(x, cout, k, s, p, bias=True, act=ACT_RELU, out=out, out_channel=ch)
+
+    def block(x, branches, H, W):
+        """branches: list of (channels, fn(x, out, ch)); returns the concatenated tensor."""
+        total = sum(c for c, _ in branches)
+        out = g.temp((total, H, W))
+        ch = 0
+        for c, fn in branches:
+            fn(x, out, ch)
+            ch += c
+        return out
+
+    x = g.input("data", image)
+    x = conv(x, 32, 3, 2)            # 149
+    x = conv(x, 32, 3)               # 147
+    x = conv(x, 64, 3, 1, 1)         # 147
+    x = g.pool2d(x, 3, 2, 0, "max")  # 73
+    x = conv(x, 80, 1)
+    x = conv(x, 192, 3)              # 71
+    x = g.pool2d(x, 3, 2, 0, "max")  # 35
+
+    def inception_a(x, pool_ch):
+        _, H, W = x.shape
+        return block(x, [
+            (64, lambda x, o, c: conv(x, 64, 1, out=o, ch=c)),
+            (64, lambda x, o, c: conv(conv(x, 48, 1), 64, 5, 1, 2, out=o, ch=c)),
+            (96, lambda x, o, c: conv(conv(conv(x, 64, 1), 96, 3, 1, 1), 96, 3, 1, 1, out=o, ch=c)),
+            (pool_ch, lambda x, o, c: conv(g.pool2d(x, 3, 1, 1, "avg", count_include_pad=True), pool_ch, 1,
+                                           out=o, ch=c)),
+        ], H, W)
+
+    x = inception_a(x, 32)
+    x = inception_a(x, 64)
+    x = inception_a(x, 64)
+
+    def inception_b(x):
+        cin, H, W = x.shape
+        Ho = (H - 3) // 2 + 1
+        out = g.temp((384 + 96 + cin, Ho, Ho))
+        conv(x, 384, 3, 2, out=out, ch=0)
+        conv(conv(conv(x, 64, 1), 96, 3, 1, 1), 96, 3, 2, out=out, ch=384)
+        p = g.pool2d(x, 3, 2, 0, "max")
+        g.copy_into(p, out, (384 + 96) * Ho * Ho)
+        return out
+
+    x = inception_b(x)               # 768 x 17 x 17
+
+    def inception_c(x, c7):
+        _, H, W = x.shape
+        return block(x, [
+            (192, lambda x, o, c: conv(x, 192, 1, out=o, ch=c)),
+            (192, lambda x, o, c: conv(conv(conv(x, c7, 1), c7, (1, 7), 1, (0, 3)), 192, (7, 1), 1, (3, 0),
+                                       out=o, ch=c)),
+            (192, lambda x, o, c: conv(conv(conv(conv(conv(x, c7, 1), c7, (7, 1), 1, (3, 0)), c7, (1, 7), 1,
+                                                      (0, 3)), c7, (7, 1), 1, (3, 0)), 192, (1, 7), 1, (0, 3),
+                                       out=o, ch=c)),
+            (192, lambda x, o, c: conv(g.pool2d(x, 3, 1, 1, "avg", count_include_pad=True), 192, 1, out=o,
+                                       ch=c)),
+        ], H, W)
+
+    for c7 in (128, 160, 160, 192):
+        x = inception_c(x, c7)
+
+    def inception_d(x):
+        cin, H, W = x.shape
+        Ho = (H - 3) // 2 + 1
+        out = g.temp((320 + 192 + cin, Ho, Ho))
+        conv(conv(x, 192, 1), 320, 3, 2, out=out, ch=0)
+        y = conv(conv(conv(x, 192, 1), 192, (1, 7), 1, (0, 3)), 192, (7, 1), 1, (3, 0))
+        conv(y, 192, 3, 2, out=out, ch=320)
+        p = g.pool2d(x, 3, 2, 0, "max")
+        g.copy_into(p, out, (320 + 192) * Ho * Ho)
+        return out
+
+    x = inception_d(x)               # 1280 x 8 x 8
+
+    def inception_e(x):
+        _, H, W = x.shape
+
+        def b3(x, o, c):
+            y = conv(x, 384, 1)
+            conv(y, 384, (1, 3), 1, (0, 1), out=o, ch=c)
+            conv(y, 384, (3, 1), 1, (1, 0), out=o, ch=c + 384)
+
+        def b3dbl(x, o, c):
+            y = conv(conv(x, 448, 1), 384, 3, 1, 1)
+            conv(y, 384, (1, 3), 1, (0, 1), out=o, ch=c)
+            conv(y, 384, (3, 1), 1, (1, 0), out=o, ch=c + 384)
+
+        return block(x, [
+            (320, lambda x, o, c: conv(x, 320, 1, out=o, ch=c)),
+            (768, b3),
+            (768, b3dbl),
+            (192, lambda x, o, c: conv(g.pool2d(x, 3, 1, 1, "avg", count_include_pad=True), 192, 1, out=o,
+                                       ch=c)),
+        ], H, W)
+
+    x = inception_e(x)
+    x = inception_e(x)               # 2048 x 8 x 8
+    pooled = g.global_avgpool(x)
+    logits = g.dense(pooled, classes, bias=True)
+    out = g.softmax(logits, 1, classes)
+    g.mark_output(out)
+    return g
+
+
+def bert(layers=12, hidden=768, heads=12, ffn=3072, seq=128, vocab=30522, name="bert_base",
+         seed=rng.BASE_SEED):
+    """BERT encoder (base: 12 layers, hidden 768, 12 heads, FFN 3072, sequence 128), fp32,
+    weights ~ N(0, 0.02).  Token ids are an int64 input, as in the reference's BERT model
+    (resource/bert/bert.json storage[0]).  The per-head views of Q, K, V and of the context
+    are expressed as GEMM strides, so no transpose kernels are needed."""
+    g = GraphBuilder(name, seed, weight_std=0.02)
+    hd = hidden // heads
+    ids = g.input("input0", (seq,), "int64")
+    x = g.embedding(ids, vocab, seq, hidden, pos=True, seg=True)
+    x = g.layernorm(x, seq, hidden)
+    inv_sqrt = 1.0 / (hd ** 0.5)
+    for _ in range(layers):
+        proj = []
+        for _name in ("q", "k", "v"):
+            w = g.param((hidden, hidden), 0.02)
+            b = g.param((hidden,), 0.02)
+            proj.append(g.gemm(x, w, seq, hidden, hidden, trans_b=True, bias=b))
+        q, k, v = proj
+        scores = g.gemm(q, k, seq, seq, hd, batch=heads, trans_b=True, alpha=inv_sqrt,
+                        lda=hidden, ldb=hidden, ldc=seq, stride_a=hd, stride_b=hd, stride_c=seq * seq)
+        probs = g.softmax(scores, heads * seq, seq)
+        ctx = g.temp((seq, hidden))
+        g.gemm(probs, v, seq, hd, seq, batch=heads, trans_b=False, lda=seq, ldb=hidden, ldc=hidden,
+               stride_a=seq * seq, stride_b=hd, stride_c=hd, out=ctx)
+        wo = g.param((hidden, hidden), 0.02)
+        bo = g.param((hidden,), 0.02)
+        att = g.gemm(ctx, wo, seq, hidden, hidden, trans_b=True, bias=bo)
+        x = g.layernorm(att, seq, hidden, res=x)
+        w1 = g.param((ffn, hidden), 0.02)
+        b1 = g.param((ffn,), 0.02)
+        h = g.gemm(x, w1, seq, ffn, hidden, trans_b=True, bias=b1, act=ACT_GELU)
+        w2 = g.param((hidden, ffn), 0.02)
+        b2 = g.param((hidden,), 0.02)
+        y = g.gemm(h, w2, seq, hidden, ffn, trans_b=True, bias=b2)
+        x = g.layernorm(y, seq, hidden, res=x)
+    g.mark_output(x)
+    return g
+
+
+def token_input(name, seq, vocab, seed=rng.BASE_SEED):
+    return rng.randint(name + "/ids", seq, vocab, seed)
+
+
+BUILDERS = {
+    "resnet18": lambda: resnet(18), "resnet50": lambda: resnet(50), "resnet152": lambda: resnet(152),
+    "mobilenetv2": mobilenet_v2, "densenet201": densenet, "inceptionv3": inception_v3,
+    "bert_base": bert, "mocked_kernel": mocked_kernel,
+}

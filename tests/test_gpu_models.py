@@ -117,3 +117,34 @@ def test_preempt_flag_stops_and_restart_is_bit_identical(resnet18_dir, resnet18_
     exe2.poke_preempt_flag(0)
     exe2.execute_preemptable()
     np.testing.assert_array_equal(exe2.get_output(), ref)
+
+
+MODEL_INPUTS = {
+    "mobilenetv2": lambda: {"data": nets.image_input("mobilenetv2", (3, 224, 224))},
+    "densenet201": lambda: {"data": nets.image_input("densenet201", (3, 224, 224))},
+    "inceptionv3": lambda: {"data": nets.image_input("inceptionv3", (3, 299, 299))},
+    "bert_base": lambda: {"input0": nets.token_input("bert_base", 128, 30522)},
+}
+
+
+@pytest.mark.parametrize("name,preemptible", [("mobilenetv2", False), ("mobilenetv2", True),
+                                              ("densenet201", True), ("inceptionv3", False),
+                                              ("bert_base", True)])
+def test_benchmark_models_per_layer(tmp_path, name, preemptible):
+    """The other networks of the benchmark configurations at their full shapes
+    (MobileNetV2 1.0, DenseNet-201, Inception-v3 @299, BERT-base seq 128): every
+    intermediate tensor within 1e-4 of the CPU oracle."""
+    g = nets.BUILDERS[name]()
+    d = write_model(g, tmp_path)
+    model = json.load(open(os.path.join(d, g.name + ".json")))
+    inputs = MODEL_INPUTS[name]()
+    exe = B.Executor.from_dir(d, g.name, B.HYBRID)
+    orc = O.GraphOracle(model, os.path.join(d, g.name + ".param"))
+    for k, v in inputs.items():
+        exe.set_input_checked(k, v)
+        orc.set_input(k, v)
+    exe.execute_preemptable() if preemptible else exe.execute()
+    orc.run()
+    worst = compare_storages(exe, orc, model, what=name)
+    print("%s: %d kernels, worst per-layer rel err %.2e (storage %s)" % ((name, len(g.kernels)) + worst))
+    assert np.isfinite(exe.get_output()).all()
