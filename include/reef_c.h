@@ -107,6 +107,28 @@ int64_t reef_scheduler_avg_kernel_sel_latency(reef_scheduler_t s);
 uint64_t reef_scheduler_preempt_times(reef_scheduler_t s);
 uint64_t reef_scheduler_padded_kernels(reef_scheduler_t s);
 size_t reef_scheduler_preempt_samples(reef_scheduler_t s, int64_t* out, size_t cap);
+/* Average ns per reset-based preemption in: flag store, host-queue drop + rollback, device drain. */
+void reef_scheduler_preempt_phases(reef_scheduler_t s, int64_t out_ns[3]);
+/* ---- load generator: the request loops of the reference's example clients
+ * (src/example/rpc_client.cpp, rpc_client_cont.cpp:20-36) run in-process against a scheduler.
+ * One open-loop real-time client (exponential inter-arrival times, mean `mean_interval_us`;
+ * <= 0 means closed loop, back to back) and `n_be` closed-loop best-effort clients.  With
+ * requests + warmup == 0 only the best-effort clients run, for `be_only_ms`.
+ * Output arrays: rt_* hold `requests` entries, be_* hold `n_be`; any may be NULL. ---- */
+typedef struct {
+    uint32_t rt_model;
+    uint32_t n_be;
+    const uint32_t* be_models;
+    double mean_interval_us;
+    uint64_t seed;
+    int32_t warmup;
+    int32_t requests;
+    int32_t be_only_ms;
+} reef_load_config;
+int reef_loadgen_run(reef_scheduler_t s, const reef_load_config* cfg, int64_t* rt_latency_ns,
+                     int64_t* rt_queue_ns, int64_t* rt_exec_ns, uint64_t* be_completed,
+                     uint64_t* be_preempted, uint64_t* be_padded, double* recorded_span_s);
+
 /* DKP decision for one (real-time kernel, best-effort kernel) pair (scheduler.cpp:533-602).
  * rt / be = {block_num, min_occupancy, threads, vgprs, sgprs, lds, total_latency};
  * be_latency[n_lat] = best-effort kernel latency per occupancy; proxy = {vgprs, sgprs, lds}.

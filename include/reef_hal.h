@@ -119,6 +119,17 @@ int reef_hal_launch(reef_function_t fn, const uint32_t grid[3], const uint32_t b
 
 /* hipStreamWriteValue32             scheduler.cpp:27,309,448,458 */
 int reef_hal_write_value32(reef_stream_t s, reef_devptr_t ptr, int32_t value);
+/* The same write without a stream (scheduler.cpp:309 raises the preemption flag through a
+ * stream write and waits for that stream): `ptr` must come from reef_hal_malloc with
+ * REEF_MEM_DEVICE_FINEGRAINED.  On a device whose memory is host-visible the word is stored
+ * directly from the calling thread and is visible to running kernels about a microsecond later;
+ * otherwise the layer falls back to a stream write it waits for.  No ordering against any stream. */
+int reef_hal_host_write32(reef_devptr_t ptr, int32_t value);
+/* Wait until the kernels `s` already has ON THE DEVICE have finished; launches the stream still
+ * holds on the host stay there (hipStreamSynchronize after hipStreamClearQueue, scheduler.cpp:339).
+ * For a windowed stream this spins on the stream's completion counter instead of sleeping in
+ * the runtime. */
+int reef_hal_stream_wait_device(reef_stream_t s);
 /* hipStreamClearQueue (REEF-custom) scheduler.cpp:315 */
 int reef_hal_stream_clear_queue(reef_stream_t s, uint64_t* n_dropped);
 /* hipResetWavefronts (REEF-custom)  scheduler.cpp:333,341 */
@@ -170,6 +181,8 @@ typedef struct reef_hal_backend {
     int (*event_sync)(reef_event_t);
     int (*event_elapsed_us)(reef_event_t, reef_event_t, float*);
     int (*memset_async)(reef_devptr_t, int, size_t, reef_stream_t);
+    int (*host_write32)(reef_devptr_t, int32_t);
+    int (*stream_wait_device)(reef_stream_t);
 } reef_hal_backend;
 
 const reef_hal_backend* reef_hal_hip_backend(void);

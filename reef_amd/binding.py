@@ -289,3 +289,38 @@ class Scheduler:
         buf = (ctypes.c_int64 * cap)()
         n = lib().reef_scheduler_preempt_samples(self.h, buf, ctypes.c_size_t(cap))
         return np.array(buf[:n], np.int64)
+
+    def preempt_phases(self):
+        out = (ctypes.c_int64 * 3)()
+        lib().reef_scheduler_preempt_phases(self.h, out)
+        return {"flag_ns": out[0], "drop_ns": out[1], "drain_ns": out[2]}
+
+    def run_load(self, rt_mid, be_mids, requests, warmup=0, mean_interval_us=20000.0, seed=0x5EEF,
+                 be_only_ms=0):
+        """Drives the scheduler with one open-loop real-time client and len(be_mids)
+        closed-loop best-effort clients (the request loops of src/example/rpc_client_cont.cpp
+        without the RPC hop).  Returns latencies in microseconds and per-client counts."""
+
+        class Cfg(ctypes.Structure):
+            _fields_ = [("rt_model", ctypes.c_uint32), ("n_be", ctypes.c_uint32),
+                        ("be_models", ctypes.POINTER(ctypes.c_uint32)),
+                        ("mean_interval_us", ctypes.c_double), ("seed", ctypes.c_uint64),
+                        ("warmup", ctypes.c_int32), ("requests", ctypes.c_int32),
+                        ("be_only_ms", ctypes.c_int32)]
+
+        n_be = len(be_mids)
+        mids = (ctypes.c_uint32 * max(n_be, 1))(*be_mids)
+        cfg = Cfg(rt_mid, n_be, mids, float(mean_interval_us), seed, warmup, requests, be_only_ms)
+        lat = np.zeros(requests, np.int64)
+        que = np.zeros(requests, np.int64)
+        exe = np.zeros(requests, np.int64)
+        done = np.zeros(max(n_be, 1), np.uint64)
+        pre = np.zeros(max(n_be, 1), np.uint64)
+        pad = np.zeros(max(n_be, 1), np.uint64)
+        span = ctypes.c_double()
+        p = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+        _check("loadgen_run", lib().reef_loadgen_run(self.h, ctypes.byref(cfg), p(lat), p(que), p(exe),
+                                                     p(done), p(pre), p(pad), ctypes.byref(span)))
+        return {"rt_latency_us": lat / 1e3, "rt_queue_us": que / 1e3, "rt_exec_us": exe / 1e3,
+                "be_completed": done[:n_be], "be_preempted": pre[:n_be], "be_padded": pad[:n_be],
+                "span_s": span.value}

@@ -5,6 +5,7 @@
 #include <string>
 #include <vector>
 
+#include "client/loadgen.h"
 #include "executor/hybrid_executor.h"
 #include "hal/code_object.h"
 #include "reef_c.h"
@@ -259,6 +260,36 @@ uint64_t reef_scheduler_preempt_times(reef_scheduler_t h) { return h->s->preempt
 uint64_t reef_scheduler_padded_kernels(reef_scheduler_t h) { return h->s->padded_kernels(); }
 size_t reef_scheduler_preempt_samples(reef_scheduler_t h, int64_t* out, size_t cap) {
     return h->s->preempt_latency_samples(out, cap);
+}
+
+void reef_scheduler_preempt_phases(reef_scheduler_t h, int64_t out_ns[3]) { h->s->preempt_phase_avg_ns(out_ns); }
+
+int reef_loadgen_run(reef_scheduler_t h, const reef_load_config* c, int64_t* rt_latency_ns,
+                     int64_t* rt_queue_ns, int64_t* rt_exec_ns, uint64_t* be_completed,
+                     uint64_t* be_preempted, uint64_t* be_padded, double* recorded_span_s) {
+    if (!h || !c || c->warmup < 0 || c->requests < 0) return Status::OutOfRange;
+    reef::client::LoadConfig cfg;
+    cfg.rt_model = c->rt_model;
+    cfg.be_models.assign(c->be_models, c->be_models + c->n_be);
+    cfg.mean_interval_us = c->mean_interval_us;
+    cfg.seed = c->seed;
+    cfg.warmup = c->warmup;
+    cfg.requests = c->requests;
+    cfg.be_only_ms = c->be_only_ms;
+    reef::client::LoadResult r;
+    RETURN_STATUS(reef::client::run_load(*h->s, cfg, r));
+    for (size_t i = 0; i < r.rt_latency_ns.size(); i++) {
+        if (rt_latency_ns) rt_latency_ns[i] = r.rt_latency_ns[i];
+        if (rt_queue_ns) rt_queue_ns[i] = r.rt_queue_ns[i];
+        if (rt_exec_ns) rt_exec_ns[i] = r.rt_exec_ns[i];
+    }
+    for (size_t i = 0; i < r.be_completed.size(); i++) {
+        if (be_completed) be_completed[i] = r.be_completed[i];
+        if (be_preempted) be_preempted[i] = r.be_preempted[i];
+        if (be_padded) be_padded[i] = r.be_padded[i];
+    }
+    if (recorded_span_s) *recorded_span_s = r.recorded_span_s;
+    return Status::Succ;
 }
 
 int reef_dkp_decide(const int rt[7], const int be[7], const int* be_latency, int n_lat,

@@ -62,6 +62,8 @@ int reef_hal_launch(reef_function_t fn, const uint32_t grid[3], const uint32_t b
 int reef_hal_write_value32(reef_stream_t s, reef_devptr_t ptr, int32_t value) {
     return be()->write_value32(s, ptr, value);
 }
+int reef_hal_host_write32(reef_devptr_t ptr, int32_t value) { return be()->host_write32(ptr, value); }
+int reef_hal_stream_wait_device(reef_stream_t s) { return be()->stream_wait_device(s); }
 int reef_hal_stream_clear_queue(reef_stream_t s, uint64_t* n_dropped) {
     return be()->stream_clear_queue(s, n_dropped);
 }

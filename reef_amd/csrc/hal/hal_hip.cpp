@@ -2,7 +2,6 @@
 #include <hip/hip_runtime.h>
 
 #include <cstring>
-#include <deque>
 #include <map>
 #include <mutex>
 #include <string>
@@ -25,10 +24,34 @@ struct reef_function_s {
 
 namespace {
 
+// One launch a windowed stream keeps on the host.  The argument block is stored
+// inline and the queue is a ring that never shrinks, so that dropping the whole
+// queue (the first step of a preemption) costs no allocator calls.
+constexpr size_t kMaxHeldKernarg = 512;
 struct Held {
     hipFunction_t fn;
-    uint32_t grid[3], block[3], lds;
-    std::vector<char> kernarg;
+    uint32_t grid[3], block[3], lds, bytes;
+    alignas(16) char kernarg[kMaxHeldKernarg];
+};
+struct HeldRing {
+    std::vector<Held> slots;
+    size_t head = 0, count = 0;
+    bool empty() const { return count == 0; }
+    size_t size() const { return count; }
+    Held& front() { return slots[head]; }
+    void pop_front() { head = (head + 1) % slots.size(); --count; }
+    void clear() { head = 0; count = 0; }
+    Held& push_back() {
+        if (count == slots.size()) {
+            std::vector<Held> bigger(slots.empty() ? 1024 : slots.size() * 2);
+            for (size_t i = 0; i < count; i++) bigger[i] = slots[(head + i) % slots.size()];
+            slots.swap(bigger);
+            head = 0;
+        }
+        Held& h = slots[(head + count) % slots.size()];
+        ++count;
+        return h;
+    }
 };
 
 }  // namespace
@@ -41,7 +64,7 @@ struct reef_stream_s {
     int window;
     uint32_t submitted;
     volatile uint32_t* done;
-    std::deque<Held> held;
+    HeldRing held;
 };
 
 namespace {
@@ -58,6 +81,8 @@ int fail(hipError_t e, const char* what) {
     } while (0)
 
 int g_device = 0;
+bool g_host_visible = false;       // device memory can be stored to from the host (large BAR)
+hipStream_t g_flag_stream = nullptr;  // fallback path of host_write32
 
 int h_init(int device) {
     HIPCHK(hipInit(0));
@@ -69,6 +94,9 @@ int h_init(int device) {
     }
     g_device = device;
     HIPCHK(hipSetDevice(device));
+    int large_bar = 0;
+    if (hipDeviceGetAttribute(&large_bar, hipDeviceAttributeIsLargeBar, device) == hipSuccess)
+        g_host_visible = large_bar != 0;
     return 0;
 }
 
@@ -219,7 +247,7 @@ int h_stream_pump(reef_stream_t st) {
     if (!st || st->window <= 0) return 0;
     while (!st->held.empty() && (int)in_flight(st) < st->window) {
         Held& h = st->held.front();
-        int rc = submit(st, h.fn, h.grid, h.block, h.lds, h.kernarg.data(), h.kernarg.size());
+        int rc = submit(st, h.fn, h.grid, h.block, h.lds, h.kernarg, h.bytes);
         st->held.pop_front();
         if (rc) return rc;
     }
@@ -231,13 +259,17 @@ int h_launch(reef_function_t f, const uint32_t* g, const uint32_t* b, uint32_t l
     if (st && st->window > 0) {
         if (int rc = h_stream_pump(st)) return rc;
         if (!st->held.empty() || (int)in_flight(st) >= st->window) {
-            Held h;
+            if (bytes > kMaxHeldKernarg) {
+                reef_hal_set_error("reef_hal_launch: argument block too large for a windowed stream");
+                return 1;
+            }
+            Held& h = st->held.push_back();
             h.fn = f->fn;
             std::memcpy(h.grid, g, sizeof(h.grid));
             std::memcpy(h.block, b, sizeof(h.block));
             h.lds = lds;
-            h.kernarg.assign((const char*)kernarg, (const char*)kernarg + bytes);
-            st->held.push_back(std::move(h));
+            h.bytes = (uint32_t)bytes;
+            std::memcpy(h.kernarg, kernarg, bytes);
             return 0;
         }
     }
@@ -268,6 +300,29 @@ int h_device_sync() { HIPCHK(hipDeviceSynchronize()); return 0; }
 
 int h_write_value32(reef_stream_t st, reef_devptr_t p, int32_t v) {
     HIPCHK(hipStreamWriteValue32(st ? st->s : nullptr, p, (uint32_t)v, 0));
+    return 0;
+}
+int h_host_write32(reef_devptr_t p, int32_t v) {
+    if (g_host_visible) {
+        __atomic_store_n((volatile int32_t*)p, v, __ATOMIC_RELEASE);
+        __atomic_thread_fence(__ATOMIC_SEQ_CST);  // push the write-combined store out now
+        return 0;
+    }
+    if (!g_flag_stream) HIPCHK(hipStreamCreateWithFlags(&g_flag_stream, hipStreamNonBlocking));
+    HIPCHK(hipStreamWriteValue32(g_flag_stream, p, (uint32_t)v, 0));
+    HIPCHK(hipStreamSynchronize(g_flag_stream));
+    return 0;
+}
+int h_stream_wait_device(reef_stream_t st) {
+    if (st && st->window > 0) {
+        // bounded spin on the pinned completion word, then let the runtime sleep
+        for (long spins = 0; in_flight(st) != 0; ++spins) {
+            if (spins > 20000000L) break;
+            __builtin_ia32_pause();
+        }
+        if (in_flight(st) == 0) return 0;
+    }
+    HIPCHK(hipStreamSynchronize(st ? st->s : nullptr));
     return 0;
 }
 int h_clear_queue(reef_stream_t st, uint64_t* n) {
@@ -313,7 +368,7 @@ const reef_hal_backend kHip = {
     h_stream_create, h_stream_destroy, h_stream_sync, h_stream_query, h_device_sync, h_stream_pump,
     h_launch, h_write_value32, h_clear_queue, h_reset_cus,
     h_event_create, h_event_destroy, h_event_record, h_event_sync, h_event_elapsed_us,
-    h_memset_async,
+    h_memset_async, h_host_write32, h_stream_wait_device,
 };
 
 }  // namespace

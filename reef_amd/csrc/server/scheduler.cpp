@@ -48,6 +48,7 @@ REEFScheduler::REEFScheduler(ScheduleMode _mode)
       kernel_sel_latency_sum(0),
       padded_kernel_count(0),
       gpu_ready(false) {
+    preempt_phase_ns[0] = preempt_phase_ns[1] = preempt_phase_ns[2] = 0;
     // Window of kernels a best-effort stream keeps on the device
     // (scheduler.cpp:29-33: 2, or 1024 when preemption waits for completion).
     be_stream_device_queue_cap = (mode == WaitPreempt) ? 1024 : 2;
@@ -63,8 +64,7 @@ Status REEFScheduler::ensure_gpu() {
     GPU_RETURN_STATUS(reef_hal_init(0));
     GPU_RETURN_STATUS(reef_hal_stream_create(0, &preempt_stream));
     GPU_RETURN_STATUS(reef_hal_malloc(4, REEF_MEM_DEVICE_FINEGRAINED, &preempt_flag));
-    GPU_RETURN_STATUS(reef_hal_write_value32(preempt_stream, preempt_flag, 0));
-    GPU_RETURN_STATUS(reef_hal_stream_sync(preempt_stream));
+    GPU_RETURN_STATUS(reef_hal_memset(preempt_flag, 0, 4));
     gpu_ready = true;
     return Status::Succ;
 }
@@ -282,9 +282,14 @@ int REEFScheduler::rollback_kernel_offset(int launch_offset, int dropped, int wi
 // Reset-based preemption (scheduler.cpp:305-346): raise the flag, drop what the
 // best-effort streams still hold on the host, roll every running task back to a
 // kernel that is certainly complete, and (optionally) wait until the kernels
-// that were already on the device have left.
+// that were already on the device have left.  The flag is stored from this
+// thread straight into device memory: a stream write would queue behind whatever
+// best-effort kernel shares the hardware queue with the preemption stream.
 void REEFScheduler::preempt_reset() {
-    reef_hal_write_value32(preempt_stream, preempt_flag, 1);
+    typedef std::chrono::steady_clock Steady;
+    const auto t0 = Steady::now();
+    reef_hal_host_write32(preempt_flag, 1);
+    const auto t1 = Steady::now();
     const uint32_t n = be_queue_cnt.load();
     for (uint32_t i = 0; i < n; i++) {
         uint64_t dropped = 0;
@@ -301,10 +306,23 @@ void REEFScheduler::preempt_reset() {
         }
     }
     for (int i = 0; i < be_stream_device_queue_cap + 1; i++) reef_hal_reset_cus();
-    reef_hal_stream_sync(preempt_stream);
+    const auto t2 = Steady::now();
     if (wait_sync) {
-        for (uint32_t i = 0; i < n; i++) reef_hal_stream_sync(be_queues[i]->stream);
+        for (uint32_t i = 0; i < n; i++) reef_hal_stream_wait_device(be_queues[i]->stream);
     }
+    const auto t3 = Steady::now();
+    auto ns = [](Steady::time_point a, Steady::time_point b) {
+        return (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(b - a).count();
+    };
+    std::lock_guard<std::mutex> lock(stats_mtx);
+    preempt_phase_ns[0] += ns(t0, t1);
+    preempt_phase_ns[1] += ns(t1, t2);
+    preempt_phase_ns[2] += ns(t2, t3);
+}
+
+void REEFScheduler::preempt_phase_avg_ns(int64_t out[3]) const {
+    std::lock_guard<std::mutex> lock(stats_mtx);
+    for (int i = 0; i < 3; i++) out[i] = preempt_count ? (int64_t)(preempt_phase_ns[i] / preempt_count) : 0;
 }
 
 // Wait-based preemption (scheduler.cpp:348-372): raise the flag, let the device
@@ -386,7 +404,7 @@ size_t REEFScheduler::preempt_latency_samples(int64_t* out, size_t cap) const {
 }
 
 void REEFScheduler::reset_preempt_flag_async() {
-    reef_hal_write_value32(preempt_stream, preempt_flag, 0);
+    reef_hal_host_write32(preempt_flag, 0);
 }
 
 void REEFScheduler::execute_rt_task(std::shared_ptr<Task>& task) {
@@ -576,7 +594,6 @@ void REEFScheduler::execute_be_task(std::shared_ptr<Task>& task, std::shared_ptr
             if (preempted) {
                 reset_preempt_flag_async();
                 preempted = false;
-                reef_hal_stream_sync(preempt_stream);
             }
             if (task->kernel_offset >= num_kernels) {
                 task->kernel_offset = 0;

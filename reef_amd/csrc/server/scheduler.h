@@ -130,6 +130,9 @@ public:
     uint64_t padded_kernels() const { return padded_kernel_count; }
     // Copies the last `cap` preemption latencies (microseconds); returns how many.
     size_t preempt_latency_samples(int64_t* out, size_t cap) const;
+    // Average nanoseconds per reset-based preemption spent in: raising the flag, dropping the
+    // host queues + rollback, waiting for the device to drain (0 unless wait_sync).
+    void preempt_phase_avg_ns(int64_t out[3]) const;
 
 private:
     ScheduleMode mode;
@@ -179,6 +182,7 @@ private:
     uint64_t preempt_latency_sum;
     int64_t preempt_latency_max;
     std::vector<int64_t> preempt_samples;
+    uint64_t preempt_phase_ns[3];
     mutable std::mutex stats_mtx;
     uint64_t kernel_sel_count;
     uint64_t kernel_sel_latency_sum;

@@ -246,6 +246,22 @@ int f_memset_async(reef_devptr_t p, int b, size_t n, reef_stream_t st) {
     std::memset(p, b, n);
     return 0;
 }
+int f_host_write32(reef_devptr_t p, int32_t v) {
+    std::lock_guard<std::recursive_mutex> lock(g_mtx);
+    *(int32_t*)p = v;
+    return 0;
+}
+// everything already "on the device" completes; held launches stay held
+int f_stream_wait_device(reef_stream_t st) {
+    std::lock_guard<std::recursive_mutex> lock(g_mtx);
+    reef_stream_s* s = S(st);
+    while (!s->inflight.empty()) {
+        Op op = std::move(s->inflight.front());
+        s->inflight.pop_front();
+        complete(s, op);
+    }
+    return 0;
+}
 int f_event_create(reef_event_t* out) { *out = new reef_event_s{0}; return 0; }
 int f_event_destroy(reef_event_t e) { delete e; return 0; }
 int f_event_record(reef_event_t, reef_stream_t) { return 0; }
@@ -257,7 +273,7 @@ const reef_hal_backend kFake = {
     f_malloc, f_free, f_memset, f_h2d, f_d2h, f_h2d_async, f_d2h_async, f_stream_create,
     f_stream_destroy, f_stream_sync, f_stream_query, f_device_sync, f_stream_pump, f_launch,
     f_write_value32, f_clear_queue, f_reset_cus, f_event_create, f_event_destroy, f_event_record,
-    f_event_sync, f_event_elapsed, f_memset_async,
+    f_event_sync, f_event_elapsed, f_memset_async, f_host_write32, f_stream_wait_device,
 };
 
 }  // namespace
