@@ -1,15 +1,27 @@
 #!/usr/bin/env python3
 """Benchmark of the REEF hot path on one MI355X.
 
-Workload (N=1): ResNet-152 forward pass, batch 1, fp32 NCHW 3x224x224, seeded
-synthetic input and weights, one real-time client -- one "step" is one
-inference through the executor's real-time (DKP-capable) kernels.  Inputs and
-weights are resident in HBM before the timed region.
+Workload (N=1): one real-time client running ResNet-152 (batch 1, fp32 NCHW
+3x224x224) with Poisson arrivals, mean interval 20 ms, while 4 best-effort
+clients loop DenseNet-201 (growth 32, batch 1, 224x224) on the same GPU through
+one REEFScheduler.  All weights and inputs are seeded synthetic data, resident
+in HBM before the timed region.  One "step" is one real-time request; the
+value is the p99 of its latency (submit -> result ready at the scheduler API)
+over exactly --steps recorded requests, after --warmup unrecorded ones.
 
-Prints ONE JSON line: the metric, the roofline of the dominant kernel family
-(the fp32 implicit-GEMM convolution on the matrix cores) measured live with
-device events on the stream the kernels run on, and a CPU baseline (the CPU
-oracle executing the identical graph on the host cores).
+The same JSON line carries
+  * the same real-time request stream served with no best-effort load (same
+    seed, same arrival times), for the "within 5 % of solo" comparison;
+  * preemption latency (flag raised -> every best-effort stream drained);
+  * best-effort throughput with and without the real-time client;
+  * the roofline of the dominant kernel family of ResNet-152 (fp32 implicit-GEMM
+    convolution on the matrix cores), timed with device events on the stream
+    the kernels are launched on;
+  * a CPU baseline: the same ResNet-152 graph executed by the CPU oracle on the
+    host cores;
+  * two further co-location scenarios (dynamic kernel padding with a
+    MobileNetV2 best-effort client; Inception-v3 real-time with two BERT-base
+    best-effort clients), shorter runs.
 """
 import argparse
 import json
@@ -25,15 +37,17 @@ import numpy as np  # noqa: E402
 
 FP32_MFMA_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
 HBM_PEAK_GBS = 8000.0
+MEAN_INTERVAL_US = 20000.0
+SEED = 0x5EEF
 
 
-def percentile(a, q):
-    return float(np.percentile(np.asarray(a, np.float64), q))
+def pct(a, q):
+    return round(float(np.percentile(np.asarray(a, np.float64), q)) / 1e3, 4)
 
 
 def cpu_baseline(model_dir, name, x, budget_s=30.0):
     """The CPU oracle (a port of the same graph to plain C loops, OpenMP over the
-    host cores) timed on whole inferences of the same workload."""
+    host cores) timed on whole inferences of the same model."""
     from oracle import oracle as O
     model = json.load(open(os.path.join(model_dir, name + ".json")))
     orc = O.GraphOracle(model, os.path.join(model_dir, name + ".param"))
@@ -41,22 +55,100 @@ def cpu_baseline(model_dir, name, x, budget_s=30.0):
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
     times = []
     t_start = time.time()
-    while len(times) < 3 and (time.time() - t_start) < budget_s:
+    while len(times) < 5 and (time.time() - t_start) < budget_s:
         t0 = time.time()
         orc.run()
         times.append(time.time() - t0)
     return {"value": round(min(times) * 1e3, 2), "unit": "ms", "cores": cores, "kind": "port",
-            "sample": "%d whole ResNet-152 batch-1 inferences (22.56 GFLOP each), best of them"
-                      % len(times)}, orc
+            "sample": "%d whole ResNet-152 batch-1 inferences (22.56 GFLOP each) by the CPU oracle "
+                      "(C, OpenMP), best of them; TVM is not installed, so this stands in for the "
+                      "TVM-llvm build of the model" % len(times)}, orc
+
+
+def write_models(names, root):
+    from reef_amd.modelgen import nets
+    out = {}
+    for n in names:
+        g = nets.BUILDERS[n]()
+        d = os.path.dirname(g.write(os.path.join(root, g.name)))
+        out[n] = (g, d)
+    return out
+
+
+def model_input(name):
+    from reef_amd.modelgen import nets
+    if name == "bert_base":
+        return "input0", nets.token_input(name, 128, 30522)
+    side = 299 if name == "inceptionv3" else 224
+    return "data", nets.image_input(name, (3, side, side))
+
+
+def summarize(r, sched, n_be):
+    lat = r["rt_latency_us"]
+    return {"rt_ms": {"p50": pct(lat, 50), "p99": pct(lat, 99), "mean": round(float(lat.mean()) / 1e3, 4),
+                      "max": round(float(lat.max()) / 1e3, 4)},
+            "rt_exec_ms": {"p50": pct(r["rt_exec_us"], 50), "p99": pct(r["rt_exec_us"], 99)},
+            "rt_queue_ms": {"p50": pct(r["rt_queue_us"], 50), "p99": pct(r["rt_queue_us"], 99)},
+            "be_inferences_per_s": round(float(r["be_completed"].sum()) / r["span_s"], 2) if n_be else 0.0,
+            "be_completed": [int(v) for v in r["be_completed"]],
+            "be_preempted": [int(v) for v in r["be_preempted"]],
+            "be_padded": [int(v) for v in r["be_padded"]],
+            "span_s": round(r["span_s"], 3)}
+
+
+def corun(models, rt_name, be_name, n_be, mode, requests, warmup, wait_sync=True, solo=True):
+    """One scheduler, one real-time model, n_be best-effort clients of one model."""
+    from reef_amd import binding as B
+    s = B.Scheduler(mode)
+    s.set_wait_sync(wait_sync)
+    g_rt, d_rt = models[rt_name]
+    rt = s.load_model(d_rt, g_rt.name)
+    s.bind_model_queue(s.create_queue(B.QUEUE_RT), rt)
+    key, x = model_input(rt_name)
+    assert s.set_input(rt, x, key) == 0
+    bes = []
+    g_be, d_be = models[be_name]
+    bkey, bx = model_input(be_name)
+    for _ in range(n_be):
+        m = s.load_model(d_be, g_be.name)
+        s.bind_model_queue(s.create_queue(B.QUEUE_BE), m)
+        assert s.set_input(m, bx, bkey) == 0
+        bes.append(m)
+    s.run()
+    out = {"mode": {B.MODE_REEF: "REEF (reset-based preemption + dynamic kernel padding)",
+                    B.MODE_RESET: "Reset (reset-based preemption only)"}[mode],
+           "rt_model": g_rt.name, "be_model": g_be.name, "be_clients": n_be}
+    if solo:
+        r0 = s.run_load(rt, [], requests, warmup=warmup, mean_interval_us=MEAN_INTERVAL_US, seed=SEED)
+        out["solo"] = summarize(r0, s, 0)
+    rb = s.run_load(rt, bes, 0, be_only_ms=1500)
+    out["be_only_inferences_per_s"] = round(float(rb["be_completed"].sum()) / rb["span_s"], 2)
+    r1 = s.run_load(rt, bes, requests, warmup=warmup, mean_interval_us=MEAN_INTERVAL_US, seed=SEED)
+    out["loaded"] = summarize(r1, s, n_be)
+    ps = s.preempt_samples()
+    ps = ps[-(requests):] if len(ps) > requests else ps
+    out["preempt_us"] = {"n": int(len(ps)), "mean": round(float(ps.mean()), 2) if len(ps) else None,
+                         "p50": float(np.percentile(ps, 50)) if len(ps) else None,
+                         "p99": float(np.percentile(ps, 99)) if len(ps) else None,
+                         "max": int(ps.max()) if len(ps) else None,
+                         "what": "host span: flag stored into device memory -> host queues dropped -> "
+                                 "every best-effort stream has no kernel left on the device"
+                                 if wait_sync else "host span without waiting for the device to drain"}
+    out["preempt_phase_ns"] = s.preempt_phases()
+    out["padded_kernels"] = int(s.padded_kernels())
+    out["kernel_select_ns"] = int(s.avg_kernel_sel_latency())
+    s.shutdown()
+    s.close()
+    return out
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=400, help="recorded real-time requests")
+    ap.add_argument("--warmup", type=int, default=40, help="real-time requests before recording")
     ap.add_argument("--kernel-iters", type=int, default=20)
-    ap.add_argument("--model", default="resnet152")
+    ap.add_argument("--configs", default="3,4,5", help="co-location scenarios to run (3 is the headline)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--workdir", default=None)
     args = ap.parse_args()
@@ -64,34 +156,37 @@ def main():
         print("bench.py: this build runs on ONE GPU (replicas per GPU share nothing); "
               "--gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
+    configs = [int(c) for c in args.configs.split(",") if c]
 
     from reef_amd import binding as B
-    from reef_amd.modelgen import nets
 
-    layers = {"resnet152": 152, "resnet18": 18}[args.model]
-    g = nets.resnet(layers)
     tmp = tempfile.TemporaryDirectory(dir=args.workdir)
-    d = g.write(os.path.join(tmp.name, g.name))
-    d = os.path.dirname(d)
-    x = nets.image_input(g.name, (3, 224, 224))
+    names = ["resnet152", "densenet201"]
+    if 4 in configs:
+        names.append("mobilenetv2")
+    if 5 in configs:
+        names += ["inceptionv3", "bert_base"]
+    models = write_models(names, tmp.name)
+    g, d = models["resnet152"]
+    _, x = model_input("resnet152")
 
+    # ---- headline: RT ResNet-152 + 4 BE DenseNet-201 ----------------------------------
+    t0 = time.perf_counter()
+    head = corun(models, "resnet152", "densenet201", 4, B.MODE_REEF, args.steps, args.warmup)
+    wall_s = time.perf_counter() - t0
+    reset_only = corun(models, "resnet152", "densenet201", 4, B.MODE_RESET, args.steps, args.warmup,
+                       solo=False)
+
+    # ---- solo executor: whole-model device time and per-kernel durations ---------------
     exe = B.Executor.from_dir(d, g.name, B.HYBRID)
     exe.set_input_checked("data", x)
-
-    # ---- whole-model latency: W warm-up steps, then exactly K timed steps -------------
-    t0 = time.perf_counter()
-    lat_us, dev_us = exe.time_model(B.RUN_DEFAULT, args.warmup, args.steps)
-    wall_s = time.perf_counter() - t0
-    ms_per_step = float(lat_us.sum()) / args.steps / 1e3
-    p50, p99 = percentile(lat_us, 50) / 1e3, percentile(lat_us, 99) / 1e3
-
-    # ---- per-kernel durations (device events around back-to-back launches) ------------
+    lat_us, dev_us = exe.time_model(B.RUN_DEFAULT, 20, 200)
     n = exe.num_kernels()
     kus = np.array([exe.time_kernel(i, B.RUN_DEFAULT, 3, args.kernel_iters) for i in range(n)])
-    names = [k["name"].split("#")[0] for k in g.kernels]
+    names_k = [k["name"].split("#")[0] for k in g.kernels]
     flops = np.array(g.kernel_flops, np.float64)
     by = {}
-    for i, nm in enumerate(names):
+    for i, nm in enumerate(names_k):
         e = by.setdefault(nm, {"us": 0.0, "flops": 0.0, "bytes": 0.0, "launches": 0})
         e["us"] += kus[i]
         e["flops"] += flops[i]
@@ -104,28 +199,40 @@ def main():
     conv_us = sum(v["us"] for v in conv.values())
     conv_flops = sum(v["flops"] for v in conv.values())
     best_i = int(np.argmax(np.where(flops > 0, flops / np.maximum(kus, 1e-3), 0)))
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get(dom)
 
+    p99 = head["loaded"]["rt_ms"]["p99"]
+    solo_p99 = head["solo"]["rt_ms"]["p99"]
     out = {
-        "metric": "ResNet-152 batch-1 RT latency p99 (solo RT client)",
-        "value": round(p99, 4),
+        "metric": "ResNet-152 RT p99 latency w/ 4 BE clients",
+        "value": p99,
         "unit": "ms",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4),
+        "ms_per_step": head["loaded"]["rt_ms"]["mean"],
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "ResNet-152 v2 (TVM relay.testing wiring, BN folded), batch 1, fp32 NCHW "
-                               "3x224x224, seeded He-normal weights; one RT client, no BE load",
-                   "kernels_per_inference": n, "gflop_per_inference": round(g.flops / 1e9, 3)},
-        "rt_latency_ms": {"p50": round(p50, 4), "p99": round(p99, 4),
-                          "mean_device": round(float(dev_us.mean()) / 1e3, 4)},
-        "model_tflops": round(g.flops / (ms_per_step * 1e-3) / 1e12, 3),
+        "config": {"workload": "RT ResNet-152 (batch 1, fp32 NCHW 3x224x224, Poisson arrivals mean 20 ms, "
+                               "seed 0x5EEF) + 4 BE clients looping DenseNet-201 (growth 32, batch 1, "
+                               "224x224); seeded He-normal weights; REEF mode",
+                   "rt_kernels_per_inference": n, "rt_gflop_per_inference": round(g.flops / 1e9, 3)},
+        "rt_p99_vs_solo": round(p99 / solo_p99, 4),
+        "rt_p50_vs_solo": round(head["loaded"]["rt_ms"]["p50"] / head["solo"]["rt_ms"]["p50"], 4),
+        "preempt_us": head["preempt_us"],
+        "corun_resnet152_4x_densenet201": head,
+        "corun_reset_mode": reset_only,
+        "solo_back_to_back_ms": {"p50": pct(lat_us, 50), "p99": pct(lat_us, 99),
+                                 "mean_device": round(float(dev_us.mean()) / 1e3, 4)},
+        "model_tflops": round(g.flops / float(dev_us.mean()) / 1e6, 3),
         "conv_tflops_all_layers": round(conv_flops / conv_us / 1e6, 3),
-        "best_layer": {"kernel": names[best_i], "attrs": g.kernels[best_i]["attrs"][:12],
+        "best_layer": {"kernel": names_k[best_i], "attrs": g.kernels[best_i]["attrs"][:12],
                        "tflops": round(float(flops[best_i] / kus[best_i] / 1e6), 2)},
         "sum_kernel_us": round(float(kus.sum()), 1),
         "roofline": {
@@ -135,20 +242,32 @@ def main():
             "peak": FP32_MFMA_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(dom_tflops / FP32_MFMA_PEAK_TFLOPS, 4),
-            "traffic": None,
+            "traffic": traffic,
             "launches_per_inference": dom_e["launches"],
             "avg_launch_us": round(dom_e["us"] / dom_e["launches"], 3),
             "avg_launch_gflop": round(dom_e["flops"] / dom_e["launches"] / 1e9, 4),
         },
         "per_kernel": {k: {"launches": v["launches"], "avg_us": round(v["us"] / v["launches"], 3),
                            "tflops": round(v["flops"] / v["us"] / 1e6, 3),
-                           "gbs": round(v["bytes"] / v["us"] / 1e3, 1)} for k, v in sorted(by.items())},
+                           "frac_mfma_peak": round(v["flops"] / v["us"] / 1e6 / FP32_MFMA_PEAK_TFLOPS, 4),
+                           "gbs": round(v["bytes"] / v["us"] / 1e3, 1),
+                           "frac_hbm_peak": round(v["bytes"] / v["us"] / 1e3 / HBM_PEAK_GBS, 4)}
+                       for k, v in sorted(by.items())},
         "timed_region_wall_s": round(wall_s, 3),
     }
+    got = exe.get_output()
+    exe.close()
+    if 4 in configs:
+        k = max(args.steps // 2, 50)
+        out["corun_dkp_mobilenetv2"] = {
+            "reef": corun(models, "resnet152", "mobilenetv2", 1, B.MODE_REEF, k, 20),
+            "reset": corun(models, "resnet152", "mobilenetv2", 1, B.MODE_RESET, k, 20, solo=False)}
+    if 5 in configs:
+        k = max(args.steps // 2, 50)
+        out["corun_inceptionv3_2x_bert"] = corun(models, "inceptionv3", "bert_base", 2, B.MODE_REEF, k, 20)
     if not args.no_cpu:
         cb, orc = cpu_baseline(d, g.name, x)
         out["cpu_baseline"] = cb
-        got = exe.get_output()
         ref = orc.get("output")
         out["parity_max_abs_err_vs_oracle"] = float(np.abs(got - ref).max())
     print(json.dumps(out))

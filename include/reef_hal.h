@@ -41,6 +41,7 @@ typedef struct reef_module_s* reef_module_t;
 typedef struct reef_function_s* reef_function_t;
 typedef struct reef_stream_s* reef_stream_t;
 typedef struct reef_event_s* reef_event_t;
+typedef struct reef_graph_s* reef_graph_t;
 typedef void* reef_devptr_t;
 
 /* Static properties of the device the occupancy model needs.
@@ -144,6 +145,19 @@ int reef_hal_event_record(reef_event_t e, reef_stream_t s);
 int reef_hal_event_sync(reef_event_t e);
 int reef_hal_event_elapsed_us(reef_event_t start, reef_event_t stop, float* us);
 
+/* One submission for a recorded sequence of launches (no counterpart in the reference,
+ * which issues one hipModuleLaunchKernel per kernel, executor_base.cpp:191-221).  On this
+ * device a launch call costs the host 3-4 us, more than most batch-1 kernels run; a recorded
+ * sequence is replayed by the device at under 2 us per kernel.
+ *   graph_begin(s): launches issued on `s` by the calling thread are recorded, not run;
+ *   graph_end(s, &g): stops recording and builds the replayable sequence;
+ *   graph_launch(g, s): enqueues the whole sequence on `s` (any stream without a launch window).
+ * Only reef_hal_launch may be called on `s` between begin and end. */
+int reef_hal_graph_begin(reef_stream_t s);
+int reef_hal_graph_end(reef_stream_t s, reef_graph_t* out);
+int reef_hal_graph_launch(reef_graph_t g, reef_stream_t s);
+int reef_hal_graph_destroy(reef_graph_t g);
+
 /*
  * Backend table.  The functions above forward to the active backend; the HIP
  * backend is the default and the only one the library ships.  Host-logic tests
@@ -183,6 +197,10 @@ typedef struct reef_hal_backend {
     int (*memset_async)(reef_devptr_t, int, size_t, reef_stream_t);
     int (*host_write32)(reef_devptr_t, int32_t);
     int (*stream_wait_device)(reef_stream_t);
+    int (*graph_begin)(reef_stream_t);
+    int (*graph_end)(reef_stream_t, reef_graph_t*);
+    int (*graph_launch)(reef_graph_t, reef_stream_t);
+    int (*graph_destroy)(reef_graph_t);
 } reef_hal_backend;
 
 const reef_hal_backend* reef_hal_hip_backend(void);

@@ -177,7 +177,9 @@ enum {
 #define REEF_CONV_MODE_POINTWISE 1
 #define REEF_CONV_MODE_UNALIGNED 2
 
-/* Tile configurations (BM x BN output tile per workgroup, BK = 32). */
+/* Tile configurations: BM x BN output tile per workgroup.  Plain tiles walk K in steps of
+ * 32; a "k<n>" tile splits every step of 32*n k values across n wavefronts and sums the n
+ * partial tiles inside the workgroup (K_CHUNK is then a multiple of 32*n). */
 enum {
     REEF_TILE_128x128 = 0,
     REEF_TILE_128x64 = 1,
@@ -185,6 +187,9 @@ enum {
     REEF_TILE_128x32 = 3,
     REEF_TILE_32x128 = 4,
     REEF_TILE_64x128 = 5,
+    REEF_TILE_32x32k4 = 6,
+    REEF_TILE_64x32k2 = 7,
+    REEF_TILE_32x64k2 = 8,
     REEF_TILE_COUNT
 };
 

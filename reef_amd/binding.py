@@ -119,6 +119,9 @@ class Executor:
                                                        ctypes.c_size_t(out.nbytes)))
         return out
 
+    def set_graph_launch(self, on):
+        lib().reef_executor_set_graph_launch(self.h, int(bool(on)))
+
     def execute(self):
         _check("execute", lib().reef_executor_execute(self.h))
 

@@ -71,6 +71,7 @@ int reef_executor_get_output(reef_executor_t e, void* out, size_t len) { return 
 int reef_executor_get_data(reef_executor_t e, int idx, void* out, size_t len) {
     return e->exe->get_data(idx, out, len);
 }
+void reef_executor_set_graph_launch(reef_executor_t e, int on) { e->exe->set_graph_launch(on != 0); }
 int reef_executor_execute(reef_executor_t e) { return e->exe->execute(e->exe->stream()); }
 int reef_executor_execute_to(reef_executor_t e, int idx) { return e->exe->execute_to(idx, e->exe->stream()); }
 int reef_executor_execute_kernel(reef_executor_t e, int idx) {
@@ -171,7 +172,8 @@ int reef_executor_time_model(reef_executor_t e, int flavour, int warmup, int ite
         GPU_RETURN_STATUS(reef_hal_stream_sync(s));
         auto t0 = std::chrono::steady_clock::now();
         GPU_RETURN_STATUS(reef_hal_event_record(a, s));
-        RETURN_STATUS(launch_all(e, flavour, 0, n));
+        if (flavour == REEF_RUN_DEFAULT) RETURN_STATUS(e->exe->launch_model(s));
+        else RETURN_STATUS(launch_all(e, flavour, 0, n));
         GPU_RETURN_STATUS(reef_hal_event_record(b, s));
         GPU_RETURN_STATUS(reef_hal_stream_sync(s));
         auto t1 = std::chrono::steady_clock::now();

@@ -1,14 +1,18 @@
 #include "executor/executor_base.h"
 
+#include <cstdlib>
+
 #include <cstring>
 
 namespace reef {
 namespace executor {
 
 ExecutorBase::ExecutorBase()
-    : arena(nullptr), arena_bytes(0), base_mod(nullptr), s(nullptr), owns_stream(false) {}
+    : arena(nullptr), arena_bytes(0), base_mod(nullptr), s(nullptr), owns_stream(false),
+      use_graph(std::getenv("REEF_NO_GRAPH") == nullptr), model_graph(nullptr) {}
 
 ExecutorBase::~ExecutorBase() {
+    drop_graph();
     if (owns_stream && s) reef_hal_stream_destroy(s);
     if (arena) reef_hal_free(arena, REEF_MEM_DEVICE);
 }
@@ -170,8 +174,38 @@ Status ExecutorBase::execute(GPUStream_t stream) { return execute_to((int)num_ke
 
 Status ExecutorBase::execute_to(int idx, GPUStream_t stream) {
     if (idx < 0 || (size_t)idx > num_kernels()) RETURN_STATUS(Status::OutOfRange);
-    for (int i = 0; i < idx; i++) RETURN_STATUS(launch_kernel(i, stream));
+    if ((size_t)idx == num_kernels()) RETURN_STATUS(launch_model(stream));
+    else for (int i = 0; i < idx; i++) RETURN_STATUS(launch_kernel(i, stream));
     GPU_RETURN_STATUS(reef_hal_stream_sync(stream));
+    return Status::Succ;
+}
+
+void ExecutorBase::set_graph_launch(bool on) {
+    use_graph = on;
+    if (!on) drop_graph();
+}
+
+void ExecutorBase::drop_graph() {
+    if (model_graph) reef_hal_graph_destroy(model_graph);
+    model_graph = nullptr;
+}
+
+Status ExecutorBase::launch_model(GPUStream_t stream) {
+    const int n = (int)num_kernels();
+    if (!use_graph || !stream || n == 0) return launch_range(0, n, stream);
+    if (!model_graph) {
+        GPU_RETURN_STATUS(reef_hal_graph_begin(stream));
+        Status st = launch_range(0, n, stream);
+        reef_graph_t g = nullptr;
+        const int rc = reef_hal_graph_end(stream, &g);
+        if (st != Status::Succ) {
+            if (rc == 0) reef_hal_graph_destroy(g);
+            RETURN_STATUS(st);
+        }
+        GPU_RETURN_STATUS(rc);
+        model_graph = g;
+    }
+    GPU_RETURN_STATUS(reef_hal_graph_launch(model_graph, stream));
     return Status::Succ;
 }
 

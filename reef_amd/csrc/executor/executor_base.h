@@ -48,6 +48,14 @@ public:
 
     // Launches kernels [begin, end) without synchronising (for timing loops).
     Status launch_range(int begin, int end, GPUStream_t stream);
+    // Enqueues the whole model without synchronising.  The kernel sequence of a model
+    // never changes between runs (same functions, same argument blocks, same storages),
+    // so it is recorded once and replayed as ONE submission: the host pays one call
+    // instead of one per kernel.  set_graph_launch(false), or REEF_NO_GRAPH=1 in the
+    // environment, goes back to one launch call per kernel.
+    Status launch_model(GPUStream_t stream);
+    void set_graph_launch(bool on);
+    bool graph_launch() const { return use_graph; }
 
     // Entry symbol of a graph-JSON kernel name ("symbol" or "symbol#instance").
     static std::string kernel_symbol(const std::string& name);
@@ -70,6 +78,9 @@ protected:
     GPUModule_t base_mod;
     GPUStream_t s;
     bool owns_stream;
+    bool use_graph;
+    reef_graph_t model_graph;
+    void drop_graph();
 };
 
 }  // namespace executor

@@ -64,6 +64,10 @@ int reef_hal_write_value32(reef_stream_t s, reef_devptr_t ptr, int32_t value) {
 }
 int reef_hal_host_write32(reef_devptr_t ptr, int32_t value) { return be()->host_write32(ptr, value); }
 int reef_hal_stream_wait_device(reef_stream_t s) { return be()->stream_wait_device(s); }
+int reef_hal_graph_begin(reef_stream_t s) { return be()->graph_begin(s); }
+int reef_hal_graph_end(reef_stream_t s, reef_graph_t* out) { return be()->graph_end(s, out); }
+int reef_hal_graph_launch(reef_graph_t g, reef_stream_t s) { return be()->graph_launch(g, s); }
+int reef_hal_graph_destroy(reef_graph_t g) { return be()->graph_destroy(g); }
 int reef_hal_stream_clear_queue(reef_stream_t s, uint64_t* n_dropped) {
     return be()->stream_clear_queue(s, n_dropped);
 }

@@ -67,6 +67,11 @@ struct reef_stream_s {
     HeldRing held;
 };
 
+struct reef_graph_s {
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+};
+
 namespace {
 
 int fail(hipError_t e, const char* what) {
@@ -325,6 +330,42 @@ int h_stream_wait_device(reef_stream_t st) {
     HIPCHK(hipStreamSynchronize(st ? st->s : nullptr));
     return 0;
 }
+int h_graph_begin(reef_stream_t st) {
+    if (!st || st->window > 0) {
+        reef_hal_set_error("reef_hal_graph_begin: needs a stream without a launch window");
+        return 1;
+    }
+    HIPCHK(hipStreamBeginCapture(st->s, hipStreamCaptureModeThreadLocal));
+    return 0;
+}
+int h_graph_end(reef_stream_t st, reef_graph_t* out) {
+    if (!st || !out) return 1;
+    hipGraph_t g = nullptr;
+    HIPCHK(hipStreamEndCapture(st->s, &g));
+    hipGraphExec_t ge = nullptr;
+    hipError_t e = hipGraphInstantiate(&ge, g, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        hipGraphDestroy(g);
+        return fail(e, "hipGraphInstantiate");
+    }
+    *out = new reef_graph_s{g, ge};
+    return 0;
+}
+int h_graph_launch(reef_graph_t g, reef_stream_t st) {
+    if (!g || (st && st->window > 0)) {
+        reef_hal_set_error("reef_hal_graph_launch: bad graph or windowed stream");
+        return 1;
+    }
+    HIPCHK(hipGraphLaunch(g->exec, st ? st->s : nullptr));
+    return 0;
+}
+int h_graph_destroy(reef_graph_t g) {
+    if (!g) return 0;
+    hipGraphExecDestroy(g->exec);
+    hipGraphDestroy(g->graph);
+    delete g;
+    return 0;
+}
 int h_clear_queue(reef_stream_t st, uint64_t* n) {
     uint64_t d = 0;
     if (st) { d = st->held.size(); st->held.clear(); }
@@ -369,6 +410,7 @@ const reef_hal_backend kHip = {
     h_launch, h_write_value32, h_clear_queue, h_reset_cus,
     h_event_create, h_event_destroy, h_event_record, h_event_sync, h_event_elapsed_us,
     h_memset_async, h_host_write32, h_stream_wait_device,
+    h_graph_begin, h_graph_end, h_graph_launch, h_graph_destroy,
 };
 
 }  // namespace

@@ -34,8 +34,21 @@ __device__ __forceinline__ void splitk_reduce_body(const ReefOpDesc& d, int task
     const size_t i0 = ((size_t)task * kThreads + threadIdx.x) * 4;
     if (i0 >= MN) return;
     if ((MN & 3) == 0) {
-        f32x4 acc = *(const f32x4*)(ws + i0);
-        for (int s = 1; s < S; ++s) acc += *(const f32x4*)(ws + (size_t)s * MN + i0);
+        // The partial tensors were written by another kernel and come from memory: the loads
+        // of eight partials are issued together (a partial past S is loaded from the last one
+        // and dropped), the sums then run in ascending s as before.
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int s0 = 0; s0 < S; s0 += 8) {
+            f32x4 v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int s = min(s0 + j, S - 1);
+                v[j] = *(const f32x4*)(ws + (size_t)s * MN + i0);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (s0 + j < S) acc = (s0 + j == 0) ? v[j] : acc + v[j];
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) ep.store(out, acc[e], (int)((i0 + e) / N), i0 + e);
     } else {

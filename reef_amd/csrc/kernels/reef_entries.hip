@@ -165,24 +165,37 @@ REEF_ENTRY(reef_conv2d_64x64, OpConv<Tile64x64>)
 REEF_ENTRY(reef_conv2d_128x32, OpConv<Tile128x32>)
 REEF_ENTRY(reef_conv2d_32x128, OpConv<Tile32x128>)
 REEF_ENTRY(reef_conv2d_64x128, OpConv<Tile64x128>)
+REEF_ENTRY(reef_conv2d_32x32k4, OpConv<Tile32x32k4>)
+REEF_ENTRY(reef_conv2d_64x32k2, OpConv<Tile64x32k2>)
+REEF_ENTRY(reef_conv2d_32x64k2, OpConv<Tile32x64k2>)
 REEF_ENTRY(reef_conv2d_pw_128x128, OpConv<Tile128x128 REEF_COMMA CONV_POINTWISE>)
 REEF_ENTRY(reef_conv2d_pw_128x64, OpConv<Tile128x64 REEF_COMMA CONV_POINTWISE>)
 REEF_ENTRY(reef_conv2d_pw_64x64, OpConv<Tile64x64 REEF_COMMA CONV_POINTWISE>)
 REEF_ENTRY(reef_conv2d_pw_128x32, OpConv<Tile128x32 REEF_COMMA CONV_POINTWISE>)
 REEF_ENTRY(reef_conv2d_pw_32x128, OpConv<Tile32x128 REEF_COMMA CONV_POINTWISE>)
 REEF_ENTRY(reef_conv2d_pw_64x128, OpConv<Tile64x128 REEF_COMMA CONV_POINTWISE>)
+REEF_ENTRY(reef_conv2d_pw_32x32k4, OpConv<Tile32x32k4 REEF_COMMA CONV_POINTWISE>)
+REEF_ENTRY(reef_conv2d_pw_64x32k2, OpConv<Tile64x32k2 REEF_COMMA CONV_POINTWISE>)
+REEF_ENTRY(reef_conv2d_pw_32x64k2, OpConv<Tile32x64k2 REEF_COMMA CONV_POINTWISE>)
 REEF_ENTRY(reef_conv2d_u_128x128, OpConv<Tile128x128 REEF_COMMA CONV_UNALIGNED>)
 REEF_ENTRY(reef_conv2d_u_128x64, OpConv<Tile128x64 REEF_COMMA CONV_UNALIGNED>)
 REEF_ENTRY(reef_conv2d_u_64x64, OpConv<Tile64x64 REEF_COMMA CONV_UNALIGNED>)
 REEF_ENTRY(reef_conv2d_u_128x32, OpConv<Tile128x32 REEF_COMMA CONV_UNALIGNED>)
 REEF_ENTRY(reef_conv2d_u_32x128, OpConv<Tile32x128 REEF_COMMA CONV_UNALIGNED>)
 REEF_ENTRY(reef_conv2d_u_64x128, OpConv<Tile64x128 REEF_COMMA CONV_UNALIGNED>)
+REEF_ENTRY(reef_conv2d_u_32x32k4, OpConv<Tile32x32k4 REEF_COMMA CONV_UNALIGNED>)
+REEF_ENTRY(reef_conv2d_u_64x32k2, OpConv<Tile64x32k2 REEF_COMMA CONV_UNALIGNED>)
+REEF_ENTRY(reef_conv2d_u_32x64k2, OpConv<Tile32x64k2 REEF_COMMA CONV_UNALIGNED>)
 REEF_ENTRY(reef_gemm_nt_128x128, OpGemm<Tile128x128 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nt_64x64, OpGemm<Tile64x64 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nt_32x128, OpGemm<Tile32x128 REEF_COMMA true>)
+REEF_ENTRY(reef_gemm_nt_32x32k4, OpGemm<Tile32x32k4 REEF_COMMA true>)
+REEF_ENTRY(reef_gemm_nt_64x32k2, OpGemm<Tile64x32k2 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nn_128x128, OpGemm<Tile128x128 REEF_COMMA false>)
 REEF_ENTRY(reef_gemm_nn_64x64, OpGemm<Tile64x64 REEF_COMMA false>)
 REEF_ENTRY(reef_gemm_nn_32x128, OpGemm<Tile32x128 REEF_COMMA false>)
+REEF_ENTRY(reef_gemm_nn_32x32k4, OpGemm<Tile32x32k4 REEF_COMMA false>)
+REEF_ENTRY(reef_gemm_nn_64x32k2, OpGemm<Tile64x32k2 REEF_COMMA false>)
 REEF_ENTRY(reef_splitk_reduce, OpSplitKReduce)
 REEF_ENTRY(reef_dwconv2d, OpDwConv)
 REEF_ENTRY(reef_pool2d, OpPool)

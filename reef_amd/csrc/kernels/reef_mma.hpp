@@ -27,10 +27,16 @@
 
 namespace reef_dev {
 
-template <int WGM_, int WGN_, int TM_, int TN_, int DEPTH_>
+// KW_ > 1 splits K across wavefronts: the workgroup stages 32 * KW k values per
+// step, wavefront kw of a (row, column) group multiplies the kw-th 32 of them, and
+// the KW partial tiles are summed through LDS after the loop (always in the order
+// kw = 0, 1, ..).  A batch-1 layer has far fewer output tiles than the device has
+// matrix pipes; this puts all four pipes of a CU on one small tile without a
+// second kernel to fold partial sums.
+template <int WGM_, int WGN_, int TM_, int TN_, int DEPTH_, int KW_ = 1>
 struct Tile {
-    static constexpr int WGM = WGM_, WGN = WGN_, TM = TM_, TN = TN_;
-    static constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32, BK = 32;
+    static constexpr int WGM = WGM_, WGN = WGN_, TM = TM_, TN = TN_, KW = KW_;
+    static constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32, BK = 32 * KW;
     // K steps whose global loads are in flight at once.  A batch-1 layer gives a
     // workgroup only a handful of K steps, each shorter than one trip to memory, so
     // the loads of several steps have to be outstanding together.
@@ -42,7 +48,10 @@ struct Tile {
     static constexpr int BN_FLOATS = BN * LDA;  // B tile, n-major (trans_b GEMM)
     static constexpr int B_FLOATS = BN_FLOATS > BK_FLOATS ? BN_FLOATS : BK_FLOATS;
     static constexpr int LDS_BYTES = 2 * (A_FLOATS + B_FLOATS) * 4 + 16;
-    static_assert(WGM * WGN == 4, "four wavefronts per workgroup");
+    static constexpr int RPW = 16 / KW;  // accumulator rows-of-lanes each wavefront finishes
+    static_assert(WGM * WGN * KW == 4, "four wavefronts per workgroup");
+    static_assert(KW == 1 || 4 * TM * TN * 16 * 64 <= 2 * (A_FLOATS + B_FLOATS),
+                  "the partial tiles are exchanged through the staging buffers");
 };
 
 typedef Tile<2, 2, 2, 2, 2> Tile128x128;
@@ -51,6 +60,9 @@ typedef Tile<2, 2, 1, 1, 2> Tile64x64;
 typedef Tile<4, 1, 1, 1, 2> Tile128x32;
 typedef Tile<1, 4, 1, 1, 2> Tile32x128;
 typedef Tile<2, 2, 1, 2, 2> Tile64x128;
+typedef Tile<1, 1, 1, 1, 2, 4> Tile32x32k4;
+typedef Tile<2, 1, 1, 1, 2, 2> Tile64x32k2;
+typedef Tile<1, 2, 1, 1, 2, 2> Tile32x64k2;
 
 // All tile loads are branch-free: an element outside the tensor (row >= M,
 // k >= k_end, padding) is loaded from the tensor's first element instead and
@@ -61,7 +73,10 @@ typedef Tile<2, 2, 1, 2, 2> Tile64x128;
 // Addresses are a uniform base plus a 32-bit element offset per lane.
 template <class T, bool VEC>
 struct ALoader {
-    static constexpr int NV = T::BM / 32;  // float4 per thread per tile
+    static constexpr int TPR = T::BK / 4;          // threads (float4s) per tile row
+    static constexpr int RPP = kThreads / TPR;     // rows per pass
+    static constexpr int NV = T::BM / RPP;         // float4 per thread per tile
+    static_assert(NV >= 1 && NV <= 8, "validity bits of a tile fit one register");
     // Raw loaded values plus one validity bit per element group.  The zeroing of
     // invalid elements happens when the tile is written to LDS, not at the load: a
     // select right behind the load would make the wavefront wait for the data at
@@ -78,11 +93,11 @@ struct ALoader {
         const int tid = threadIdx.x;
         a0 = a;
         k_end = k_end_;
-        k = k_begin + (tid & 7) * 4;
+        k = k_begin + (tid % TPR) * 4;
         rowmask = 0;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            const int row = m0 + (tid >> 3) + 32 * i;
+            const int row = m0 + tid / TPR + RPP * i;
             const bool ok = row < M;
             rowoff[i] = ok ? (unsigned)row * (unsigned)lda : 0u;
             rowmask |= (ok ? 1u : 0u) << i;
@@ -109,17 +124,17 @@ struct ALoader {
             }
         }
         r.ok = okbits;
-        k += 32;
+        k += T::BK;
     }
     __device__ __forceinline__ void store(const Regs& r, float* As) const {
         const int tid = threadIdx.x;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            int row = (tid >> 3) + 32 * i;
+            int row = tid / TPR + RPP * i;
             f32x4 v;
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] = ((r.ok >> (4 * i + e)) & 1u) ? r.v[i][e] : 0.f;
-            *(f32x4*)(As + row * T::LDA + (tid & 7) * 4) = v;
+            *(f32x4*)(As + row * T::LDA + (tid % TPR) * 4) = v;
         }
     }
 };
@@ -133,8 +148,9 @@ struct ALoader {
 template <class T>
 struct Im2colLoader {
     static constexpr int RS = kThreads / T::BN;  // k rows covered per pass
-    static constexpr int NR = 32 / RS;           // rows per thread per tile
+    static constexpr int NR = T::BK / RS;        // rows per thread per tile
     static constexpr bool UNIFORM = T::BN >= 64; // one k row per wavefront
+    static_assert(NR <= 32, "validity bits of a tile fit one register");
     struct Regs { float v[NR]; unsigned ok; };   // raw values + validity bits (zeroed at store)
     const float* in;
     int HW, W, kh, kw;
@@ -211,14 +227,14 @@ struct Im2colLoader {
 template <class T>
 struct PointwiseLoader {
     static constexpr int C4 = T::BN / 4;                 // float4 per tile row
-    static constexpr int NF = 32 * C4 / kThreads;        // float4 per thread per tile
+    static constexpr int NF = T::BK * C4 / kThreads;     // float4 per thread per tile
     static constexpr int RSTEP = kThreads / C4;          // rows between a thread's float4s
     static_assert(NF >= 1, "tile narrower than one pass");
     struct Regs { f32x4 v[NF]; unsigned ok; };
     const float* in;
     unsigned off;   // element offset of this thread's first float4 in the next tile
     unsigned step;  // RSTEP * N
-    unsigned tile;  // 32 * N
+    unsigned tile;  // BK * N
     int k, k_end;
     bool nvalid;
 
@@ -231,7 +247,7 @@ struct PointwiseLoader {
         k_end = k_end_;
         off = (unsigned)k * (unsigned)N + (unsigned)(n0 + col);
         step = (unsigned)RSTEP * (unsigned)N;
-        tile = 32u * (unsigned)N;
+        tile = (unsigned)T::BK * (unsigned)N;
     }
     __device__ __forceinline__ void load(Regs& r) {
         unsigned okbits = 0;
@@ -243,7 +259,7 @@ struct PointwiseLoader {
         }
         r.ok = okbits;
         off += tile;
-        k += 32;
+        k += T::BK;
     }
     __device__ __forceinline__ void store(const Regs& r, float* Bs) const {
         const int tid = threadIdx.x;
@@ -260,7 +276,7 @@ struct PointwiseLoader {
 template <class T>
 struct BknLoader {
     static constexpr int RS = kThreads / T::BN;
-    static constexpr int NR = 32 / RS;
+    static constexpr int NR = T::BK / RS;
     struct Regs { float v[NR]; unsigned ok; };
     const float* b0;
     int n;
@@ -295,11 +311,73 @@ struct BknLoader {
     }
 };
 
+// ---- which part of the tile a wavefront owns ---------------------------------
+// Wavefronts are numbered (group, kw): the KW wavefronts of a group share one
+// TM*32 x TN*32 block of the tile and split the k values of every step.
+template <class T>
+struct WaveGeom {
+    int wk, wm0, wn0;
+    __device__ __forceinline__ WaveGeom() {
+        const int wave = threadIdx.x >> 6;
+        wk = wave % T::KW;
+        const int g = wave / T::KW;
+        wm0 = (g / T::WGN) * (T::TM * 32);
+        wn0 = (g % T::WGN) * (T::TN * 32);
+    }
+};
+
+// After the K loop: the values this wavefront writes out.  res[tm][tn][rr] is
+// accumulator element r = r0 + rr of the lane (row = 8*(r/4) + 4*(lane/32) + r%4,
+// col = lane%32).  With KW == 1 that is the wavefront's own accumulator (r0 = 0, all
+// 16 elements); otherwise the KW partial tiles of the group go through LDS, are
+// summed in the order kw = 0, 1, .., and each wavefront keeps 16/KW elements, so
+// the epilogue is spread over all wavefronts too.
+template <class T>
+__device__ __forceinline__ int finish_tile(const f32x16 (&acc)[T::TM][T::TN],
+                                           float (&res)[T::TM][T::TN][T::RPW], float* smem) {
+    if (T::KW == 1) {
+#pragma unroll
+        for (int tm = 0; tm < T::TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < T::TN; ++tn)
+#pragma unroll
+                for (int r = 0; r < T::RPW; ++r) res[tm][tn][r] = acc[tm][tn][r];
+        return 0;
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();  // every wavefront is done reading the staged tiles
+#pragma unroll
+    for (int tm = 0; tm < T::TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < T::TN; ++tn)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                smem[(((wave * T::TM + tm) * T::TN + tn) * 16 + r) * 64 + lane] = acc[tm][tn][r];
+    __syncthreads();
+    const int wk = wave % T::KW, first = wave - wk;
+    const int r0 = wk * T::RPW;
+#pragma unroll
+    for (int tm = 0; tm < T::TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < T::TN; ++tn)
+#pragma unroll
+            for (int rr = 0; rr < T::RPW; ++rr) {
+                float v = smem[(((first * T::TM + tm) * T::TN + tn) * 16 + r0 + rr) * 64 + lane];
+#pragma unroll
+                for (int s = 1; s < T::KW; ++s)
+                    v += smem[((((first + s) * T::TM + tm) * T::TN + tn) * 16 + r0 + rr) * 64 + lane];
+                res[tm][tn][rr] = v;
+            }
+    return r0;
+}
+
 // ---- the MFMA inner product over one staged K step -------------------------
 template <class T, bool B_NMAJOR>
 __device__ __forceinline__ void mma_step(const float* As, const float* Bs, f32x16 (&acc)[T::TM][T::TN],
-                                         int wm0, int wn0) {
+                                         int wm0, int wn0, int wk0) {
     const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
+    As += wk0;                                   // this wavefront's 32 k values of the step
+    Bs += B_NMAJOR ? wk0 : wk0 * T::BN;
     // All operand fragments of the K step are fetched from LDS first, then the 16 x
     // TM x TN MFMAs issue back to back: one LDS round trip per step is exposed
     // instead of one per group of four MFMAs.
@@ -351,8 +429,8 @@ __device__ __forceinline__ bool k_loop(LA& la, LB& lb, int nk, float* smem, f32x
     float* As = smem;
     float* Bs = smem + 2 * T::A_FLOATS;
     int* sflag = (int*)(smem + 2 * (T::A_FLOATS + T::B_FLOATS));
-    const int wave = threadIdx.x >> 6;
-    const int wm0 = (wave / T::WGN) * (T::TM * 32), wn0 = (wave % T::WGN) * (T::TN * 32);
+    const WaveGeom<T> wg;
+    const int wm0 = wg.wm0, wn0 = wg.wn0, wk0 = wg.wk * 32;
 #pragma unroll
     for (int tm = 0; tm < T::TM; ++tm)
 #pragma unroll
@@ -389,7 +467,7 @@ __device__ __forceinline__ bool k_loop(LA& la, LB& lb, int nk, float* smem, f32x
             // loads fills the issue slots the dependent MFMA chain leaves free
             la.load(ra[s]);
             lb.load(rb[s]);
-            mma_step<T, B_NMAJOR>(As + cur * T::A_FLOATS, Bs + cur * T::B_FLOATS, acc, wm0, wn0);
+            mma_step<T, B_NMAJOR>(As + cur * T::A_FLOATS, Bs + cur * T::B_FLOATS, acc, wm0, wn0, wk0);
             ++it;
         }
     }
@@ -425,7 +503,7 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
     n0 = nt * T::BN;
     const int k_begin = split * k_chunk;
     const int k_end = min(K, k_begin + k_chunk);
-    const int nk = (k_end - k_begin + 31) >> 5;
+    const int nk = (k_end - k_begin + T::BK - 1) / T::BK;
 
     bool ok;
     if (MODE == CONV_POINTWISE) {
@@ -443,6 +521,8 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
     }
     if (!ok) return false;
   }
+    float res[T::TM][T::TN][T::RPW];
+    const int r0 = finish_tile<T>(acc, res, smem);
 
     // Everything the epilogue needs is re-read from the argument block here, so the
     // K loop does not carry the epilogue's pointers in scalar registers.
@@ -450,8 +530,9 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
     asm volatile("" : "+s"(dp));
     const ReefOpDesc& d = *dp;
     const int* a = d.attr;
-    const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5, wave = threadIdx.x >> 6;
-    const int wm0 = (wave / T::WGN) * (T::TM * 32), wn0 = (wave % T::WGN) * (T::TN * 32);
+    const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
+    const WaveGeom<T> wg;
+    const int wm0 = wg.wm0, wn0 = wg.wn0;
     const int flags = a[REEF_CONV_FLAGS];
     const size_t MN = (size_t)M * N;
     // plain split-K writes partial tiles to the workspace; the offset belongs to the
@@ -468,9 +549,10 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
             for (int tn = 0; tn < T::TN; ++tn) {
                 const int n = n0 + wn0 + tn * 32 + l32;
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
+                for (int rr = 0; rr < T::RPW; ++rr) {
+                    const int r = r0 + rr;
                     const int m = m0 + wm0 + tm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                    if (m < M && n < N) ws[(size_t)m * N + n] = acc[tm][tn][r];
+                    if (m < M && n < N) ws[(size_t)m * N + n] = res[tm][tn][rr];
                 }
             }
         return true;
@@ -492,9 +574,10 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
             for (int tn = 0; tn < T::TN; ++tn) {
                 const int n = n0 + wn0 + tn * 32 + l32;
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
+                for (int rr = 0; rr < T::RPW; ++rr) {
+                    const int r = r0 + rr;
                     const int m = m0 + wm0 + tm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                    if (m < M && n < N) store_agent(part + (size_t)m * N + n, acc[tm][tn][r]);
+                    if (m < M && n < N) store_agent(part + (size_t)m * N + n, res[tm][tn][rr]);
                 }
             }
         // every store of this workgroup has completed at device scope before it counts in
@@ -513,7 +596,8 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
             for (int tn = 0; tn < T::TN; ++tn) {
                 const int n = n0 + wn0 + tn * 32 + l32;
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
+                for (int rr = 0; rr < T::RPW; ++rr) {
+                    const int r = r0 + rr;
                     const int m = m0 + wm0 + tm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
                     if (m < M && n < N) {
                         const size_t idx = (size_t)m * N + n;
@@ -534,9 +618,10 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
         for (int tn = 0; tn < T::TN; ++tn) {
             const int n = n0 + wn0 + tn * 32 + l32;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
+            for (int rr = 0; rr < T::RPW; ++rr) {
+                const int r = r0 + rr;
                 const int m = m0 + wm0 + tm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                if (m < M && n < N) ep.store(dst, acc[tm][tn][r], m, (size_t)m * N + n);
+                if (m < M && n < N) ep.store(dst, res[tm][tn][rr], m, (size_t)m * N + n);
             }
         }
     return true;
@@ -561,7 +646,7 @@ __device__ __forceinline__ bool gemm_body(const ReefOpDesc& d, int task, char* s
     const float* A = (const float*)d.ptr[0] + (size_t)b * a[REEF_GEMM_STRIDE_A];
     const float* B = (const float*)d.ptr[1] + (size_t)b * a[REEF_GEMM_STRIDE_B];
     float* C = (float*)d.ptr[2] + (size_t)b * a[REEF_GEMM_STRIDE_C];
-    const int nk = (K + 31) >> 5;
+    const int nk = (K + T::BK - 1) / T::BK;
     float* smem = (float*)smem_raw;
     f32x16 acc[T::TM][T::TN];
 
@@ -570,7 +655,7 @@ __device__ __forceinline__ bool gemm_body(const ReefOpDesc& d, int task, char* s
     la.init(A, lda, m0, M, 0, K);
     if (TRANS_B) {
         // B is [N][K]: stage it exactly like A (rows = n).
-        typedef Tile<T::WGN, T::WGM, T::TN, T::TM, T::DEPTH> TB;  // BM of TB == BN of T
+        typedef Tile<T::WGN, T::WGM, T::TN, T::TM, T::DEPTH, T::KW> TB;  // BM of TB == BN of T
         ALoader<TB, true> lb;
         lb.init(B, ldb, n0, N, 0, K);
         ok = k_loop<T, true>(la, lb, nk, smem, acc, poll);
@@ -580,9 +665,12 @@ __device__ __forceinline__ bool gemm_body(const ReefOpDesc& d, int task, char* s
         ok = k_loop<T, false>(la, lb, nk, smem, acc, poll);
     }
     if (!ok) return false;
+    float res[T::TM][T::TN][T::RPW];
+    const int r0 = finish_tile<T>(acc, res, smem);
 
-    const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5, wave = threadIdx.x >> 6;
-    const int wm0 = (wave / T::WGN) * (T::TM * 32), wn0 = (wave % T::WGN) * (T::TN * 32);
+    const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
+    const WaveGeom<T> wg;
+    const int wm0 = wg.wm0, wn0 = wg.wn0;
     const float* bias = (a[REEF_GEMM_FLAGS] & 1) ? (const float*)d.ptr[3] : nullptr;
     const float alpha = __int_as_float(a[REEF_GEMM_ALPHA_BITS]);
     const int act = a[REEF_GEMM_ACT];
@@ -593,10 +681,11 @@ __device__ __forceinline__ bool gemm_body(const ReefOpDesc& d, int task, char* s
             const int n = n0 + wn0 + tn * 32 + l32;
             const float bv = (bias && n < N) ? bias[n] : 0.0f;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
+            for (int rr = 0; rr < T::RPW; ++rr) {
+                const int r = r0 + rr;
                 const int m = m0 + wm0 + tm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
                 if (m < M && n < N) {
-                    float v = acc[tm][tn][r] * alpha + bv;
+                    float v = res[tm][tn][rr] * alpha + bv;
                     if (act == REEF_ACT_RELU) v = fmaxf(v, 0.0f);
                     else if (act == REEF_ACT_GELU) v = gelu_erf(v);
                     C[(size_t)m * ldc + n] = v;

@@ -411,7 +411,13 @@ void REEFScheduler::execute_rt_task(std::shared_ptr<Task>& task) {
     REEF_LOG_INFO("start rt task");
     task->state.store(TaskState::Executing);
     task->start = Clock::now();
+    bool be_waiting = false;
     if (mode == ScheduleMode::REEF) {
+        const uint32_t n_q = be_queue_cnt.load();
+        for (uint32_t q = 0; q < n_q && !be_waiting; q++) be_waiting = !be_queues[q]->empty();
+    }
+    if (be_waiting) {
+        // something to pad with: one launch per kernel, each with its own decision
         dynamic_kernel_padding(task);
         reef_hal_stream_sync(rt_queue->stream);
     } else {

@@ -166,7 +166,8 @@ class GraphBuilder:
             opt.append(out2.idx)
             opt.append(self.param((cout,), 0.01).idx)
         act2 = dual_act or ACT_NONE
-        t = force or tiling.choose(M, N, K, fused=fused_reduce)
+        t = force or tiling.choose(M, N, K, fused=fused_reduce,
+                                   pointwise=(kh, kw) == (1, 1))
         flops = 2 * M * N * K
         self.flops += flops
         nbytes = 4 * (x.size + M * K + M * N + (M if bias else 0) + (M * N if residual is not None else 0)

@@ -9,6 +9,8 @@ split-K to put a workgroup on every CU.
 """
 import math
 
+from .tuned import TUNED
+
 # name -> (id, BM, BN, relative MFMA efficiency of the inner loop, workgroups per CU)
 TILES = {
     "128x128": (0, 128, 128, 1.00, 2),
@@ -17,8 +19,30 @@ TILES = {
     "128x32": (3, 128, 32, 0.60, 3),
     "32x128": (4, 32, 128, 0.60, 3),
     "64x128": (5, 64, 128, 0.85, 2),
+    # k<n>: the workgroup's four wavefronts split K n ways on one small tile
+    "32x32k4": (6, 32, 32, 0.50, 2),
+    "64x32k2": (7, 64, 32, 0.55, 3),
+    "32x64k2": (8, 32, 64, 0.55, 3),
 }
-GEMM_TILES = ("128x128", "64x64", "32x128")
+# wavefronts that share one output block and split K inside the workgroup
+KW = {"32x32k4": 4, "64x32k2": 2, "32x64k2": 2}
+GEMM_TILES = ("128x128", "64x64", "32x128", "32x32k4", "64x32k2")
+
+
+def step_k(tile):
+    """k values a workgroup consumes per step of its K loop."""
+    return BK * KW.get(tile, 1)
+
+
+def forced(tile, M, N, K, split=1):
+    """The launch geometry of a given tile and split-K factor (no cost model)."""
+    tid, bm, bn, _, _ = TILES[tile]
+    bk = step_k(tile)
+    k_chunk = math.ceil(math.ceil(K / split) / bk) * bk
+    s = math.ceil(K / k_chunk)
+    mt, nt = math.ceil(M / bm), math.ceil(N / bn)
+    return dict(tile=tile, tile_id=tid, BM=bm, BN=bn, split_k=s, k_chunk=k_chunk, m_tiles=mt,
+                n_tiles=nt, tasks=s * mt * nt, est_us=1.0)
 
 NUM_CUS = 256
 BK = 32
@@ -34,8 +58,15 @@ def _steps_time(bm, bn, eff, steps):
     return steps * T_STEP_128x128 * (bm * bn) / (128.0 * 128.0) / eff
 
 
-def choose(M, N, K, allow_split=True, tiles=None, max_split=32, fused=True):
-    """Returns dict(tile, tile_id, BM, BN, split_k, k_chunk, m_tiles, n_tiles, tasks)."""
+def choose(M, N, K, allow_split=True, tiles=None, max_split=32, fused=True, pointwise=False):
+    """Returns dict(tile, tile_id, BM, BN, split_k, k_chunk, m_tiles, n_tiles, tasks).
+    Measured choices (tuned.py) win over the analytic model for the shapes they cover."""
+    if allow_split and tiles is None and not fused:
+        hit = TUNED.get((M, N, K, 1 if pointwise else 0))
+        if hit is not None:
+            t = forced(hit[0], M, N, K, hit[1])
+            t["est_us"] = hit[2]
+            return t
     best = None
     for name in (tiles or TILES.keys()):
         tid, bm, bn, eff, occ = TILES[name]
@@ -44,8 +75,9 @@ def choose(M, N, K, allow_split=True, tiles=None, max_split=32, fused=True):
         splits = [1]
         if allow_split:
             splits += [s for s in (2, 3, 4, 6, 8, 12, 16, 24, 32) if s <= max_split]
+        bk = step_k(name)
         for s in splits:
-            k_chunk = math.ceil(math.ceil(K / s) / BK) * BK
+            k_chunk = math.ceil(math.ceil(K / s) / bk) * bk
             s_eff = math.ceil(K / k_chunk)
             if s_eff != s and s != 1:
                 continue
@@ -53,7 +85,7 @@ def choose(M, N, K, allow_split=True, tiles=None, max_split=32, fused=True):
             rounds = math.ceil(wgs / (NUM_CUS * occ))
             # co-resident workgroups share the CU's matrix pipe
             share = min(occ, math.ceil(wgs / NUM_CUS))
-            t = rounds * (_steps_time(bm, bn, eff, k_chunk // BK) * share + T_FIXED)
+            t = rounds * (_steps_time(bm, bn, eff, k_chunk // bk) * share + T_FIXED)
             if s_eff > 1:
                 t += (T_FUSED_REDUCE if fused else T_REDUCE_LAUNCH) + (s_eff + 1) * M * N * 4 / HBM_BYTES_PER_US
             cand = (t, name, s_eff, k_chunk, m_tiles, n_tiles)
@@ -67,6 +99,7 @@ def choose(M, N, K, allow_split=True, tiles=None, max_split=32, fused=True):
 
 def lds_bytes(tile):
     _, bm, bn, _, _ = TILES[tile]
-    a = bm * 36
-    b = max(32 * bn, bn * 36)
+    bk = step_k(tile)
+    a = bm * (bk + 4)
+    b = max(bk * bn, bn * (bk + 4))
     return 2 * (a + b) * 4 + 16

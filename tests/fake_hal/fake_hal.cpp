@@ -42,6 +42,7 @@ struct reef_stream_s {
     std::deque<Op> inflight, held;
 };
 struct reef_event_s { int dummy; };
+struct reef_graph_s { std::vector<Op> ops; };
 
 namespace {
 
@@ -58,6 +59,8 @@ std::vector<std::string> g_missing;
 std::vector<reef_stream_s*> g_streams;
 reef_stream_s g_null_stream{0, 0, {}, {}};
 int g_next_stream = 1;
+std::map<reef_stream_s*, std::vector<Op>> g_recording;
+long g_graph_launches = 0;
 long g_launches = 0, g_completed = 0, g_dropped = 0;
 struct LogEntry { std::string symbol; int stream; uint32_t grid, block, lds; };
 std::vector<LogEntry> g_log;
@@ -218,6 +221,11 @@ int f_launch(reef_function_t f, const uint32_t* g, const uint32_t* b, uint32_t l
     std::memcpy(op.grid, g, sizeof(op.grid));
     std::memcpy(op.block, b, sizeof(op.block));
     op.kernarg.assign((const char*)kernarg, (const char*)kernarg + bytes);
+    auto rec = g_recording.find(S(st));
+    if (rec != g_recording.end()) {
+        rec->second.push_back(std::move(op));
+        return 0;
+    }
     ++g_launches;
     g_log.push_back(LogEntry{f->name, S(st)->id, g[0] * g[1] * g[2], b[0] * b[1] * b[2], lds});
     enqueue(S(st), std::move(op));
@@ -262,6 +270,36 @@ int f_stream_wait_device(reef_stream_t st) {
     }
     return 0;
 }
+// graphs: launches on a recording stream are kept aside and replayed as ordinary launches
+int f_graph_begin(reef_stream_t st) {
+    std::lock_guard<std::recursive_mutex> lock(g_mtx);
+    reef_stream_s* s = S(st);
+    if (s->window > 0 || g_recording.count(s)) return 1;
+    g_recording[s] = {};
+    return 0;
+}
+int f_graph_end(reef_stream_t st, reef_graph_t* out) {
+    std::lock_guard<std::recursive_mutex> lock(g_mtx);
+    auto it = g_recording.find(S(st));
+    if (it == g_recording.end()) return 1;
+    *out = new reef_graph_s{std::move(it->second)};
+    g_recording.erase(it);
+    return 0;
+}
+int f_graph_launch(reef_graph_t g, reef_stream_t st) {
+    std::lock_guard<std::recursive_mutex> lock(g_mtx);
+    if (!g || S(st)->window > 0) return 1;
+    ++g_graph_launches;
+    for (const Op& o : g->ops) {
+        Op op = o;
+        ++g_launches;
+        g_log.push_back(LogEntry{op.fn->name, S(st)->id, op.grid[0] * op.grid[1] * op.grid[2],
+                                 op.block[0] * op.block[1] * op.block[2], op.lds});
+        enqueue(S(st), std::move(op));
+    }
+    return 0;
+}
+int f_graph_destroy(reef_graph_t g) { delete g; return 0; }
 int f_event_create(reef_event_t* out) { *out = new reef_event_s{0}; return 0; }
 int f_event_destroy(reef_event_t e) { delete e; return 0; }
 int f_event_record(reef_event_t, reef_stream_t) { return 0; }
@@ -274,6 +312,7 @@ const reef_hal_backend kFake = {
     f_stream_destroy, f_stream_sync, f_stream_query, f_device_sync, f_stream_pump, f_launch,
     f_write_value32, f_clear_queue, f_reset_cus, f_event_create, f_event_destroy, f_event_record,
     f_event_sync, f_event_elapsed, f_memset_async, f_host_write32, f_stream_wait_device,
+    f_graph_begin, f_graph_end, f_graph_launch, f_graph_destroy,
 };
 
 }  // namespace
@@ -295,6 +334,8 @@ void fake_hal_set_auto_progress(int n) { g_auto_progress = n; }
 void fake_hal_reset(void) {
     std::lock_guard<std::recursive_mutex> lock(g_mtx);
     g_launches = g_completed = g_dropped = 0;
+    g_graph_launches = 0;
+    g_recording.clear();
     g_log.clear();
     g_res.clear();
     g_missing.clear();
@@ -313,6 +354,7 @@ size_t fake_hal_extent(const void* p) {
 long fake_hal_launches(void) { return g_launches; }
 long fake_hal_completed(void) { return g_completed; }
 long fake_hal_dropped(void) { return g_dropped; }
+long fake_hal_graph_launches(void) { return g_graph_launches; }
 long fake_hal_log_size(void) { std::lock_guard<std::recursive_mutex> lock(g_mtx); return (long)g_log.size(); }
 int fake_hal_log_entry(long i, char* symbol, size_t cap, int* stream, uint32_t* grid, uint32_t* block,
                        uint32_t* lds) {

@@ -63,7 +63,8 @@ class FakeHal:
         self.lib.fake_hal_backend.restype = ctypes.c_void_p
         self.lib.fake_hal_extent.restype = ctypes.c_size_t
         self.lib.fake_hal_extent.argtypes = [ctypes.c_void_p]
-        for f in ("fake_hal_launches", "fake_hal_completed", "fake_hal_dropped", "fake_hal_log_size"):
+        for f in ("fake_hal_launches", "fake_hal_completed", "fake_hal_dropped", "fake_hal_log_size",
+                  "fake_hal_graph_launches"):
             getattr(self.lib, f).restype = ctypes.c_long
         self.events = []          # (symbol, flavour, stream, grid, skipped)
         self.skipped = 0

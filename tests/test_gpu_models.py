@@ -148,3 +148,28 @@ def test_benchmark_models_per_layer(tmp_path, name, preemptible):
     worst = compare_storages(exe, orc, model, what=name)
     print("%s: %d kernels, worst per-layer rel err %.2e (storage %s)" % ((name, len(g.kernels)) + worst))
     assert np.isfinite(exe.get_output()).all()
+
+
+@pytest.mark.parametrize("kind", [B.BASE, B.HYBRID])
+def test_recorded_submission_replays_bit_identical(tmp_path, kind):
+    """A whole-model run replays a recorded launch sequence.  Several replays, with new inputs
+    copied in and other kernels run eagerly in between, each give exactly the output of the same
+    model launched one kernel at a time."""
+    g = nets.resnet(18)
+    d = write_model(g, tmp_path)
+    rec = B.Executor.from_dir(d, g.name, kind)
+    one = B.Executor.from_dir(d, g.name, kind)
+    one.set_graph_launch(False)
+    rng = np.random.default_rng(5)
+    for rep in range(4):
+        x = (nets.image_input("resnet18", (3, 224, 224)) * (1.0 + 0.25 * rep)
+             + rng.standard_normal((3, 224, 224)).astype(np.float32) * 0.1).astype(np.float32)
+        rec.set_input_checked("data", x)
+        one.set_input_checked("data", x)
+        rec.execute()
+        one.execute()
+        a, b = rec.get_output(), one.get_output()
+        assert np.isfinite(a).all()
+        np.testing.assert_array_equal(a, b, err_msg="replay %d" % rep)
+        rec.execute_to(7)          # eager partial run between replays
+    assert not np.array_equal(a, np.zeros_like(a))

@@ -69,6 +69,34 @@ def test_resnet_binding_matches_graph_oracle(fake, small_dirs, kind, pre):
         assert exe.read_task_slots() == [k["launch_params"][0] for k in g.kernels]
 
 
+@pytest.mark.parametrize("kind", [B.BASE, B.TRANS, B.HYBRID])
+def test_whole_model_runs_replay_one_recorded_submission(fake, small_dirs, kind):
+    """execute() records the model's launch sequence on first use and replays it as one
+    submission afterwards; switching that off goes back to one launch call per kernel.  Both
+    ways run the same kernels with the same arguments."""
+    g, d = small_dirs["tiny18"]
+    x = nets.image_input("t", (3, 32, 32))
+    want = oracle_output(g, d, x)
+    exe = B.Executor.from_dir(d, g.name, kind)
+    exe.set_input_checked("data", x)
+    n = exe.num_kernels()
+    for run in range(3):
+        exe.execute()
+        np.testing.assert_array_equal(exe.get_output(), want)
+        assert fake.lib.fake_hal_graph_launches() == run + 1
+        assert fake.lib.fake_hal_launches() == n * (run + 1)
+    log_graph = fake.log()[-n:]
+    exe.set_graph_launch(False)
+    exe.execute()
+    np.testing.assert_array_equal(exe.get_output(), want)
+    assert fake.lib.fake_hal_graph_launches() == 3
+    assert fake.log()[-n:] == log_graph
+    # partial runs never go through the recording
+    exe.set_graph_launch(True)
+    exe.execute_to(n - 1)
+    assert fake.lib.fake_hal_graph_launches() == 3
+
+
 def test_executor_error_codes(fake, small_dirs, tmp_path):
     g, d = small_dirs["mocked_kernel"]
     exe = B.Executor.from_dir(d, g.name, B.BASE)
