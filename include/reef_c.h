@@ -39,8 +39,8 @@ int reef_executor_set_input_idx(reef_executor_t e, int idx, const void* data, si
 int reef_executor_get_data_size(reef_executor_t e, const char* name, size_t* size);
 int reef_executor_get_output(reef_executor_t e, void* out, size_t len);
 int reef_executor_get_data(reef_executor_t e, int idx, void* out, size_t len);
-/* Whole-model runs replay a recorded launch sequence (one submission) unless switched off
- * here or by REEF_NO_GRAPH=1 in the environment; off = one launch call per kernel, as
+/* on: whole-model runs replay a recorded launch sequence (one submission); off (default,
+ * unless REEF_GRAPH=1 is in the environment): one launch call per kernel, as
  * executor_base.cpp:191-221 does. */
 void reef_executor_set_graph_launch(reef_executor_t e, int on);
 int reef_executor_execute(reef_executor_t e);

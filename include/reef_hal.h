@@ -147,8 +147,8 @@ int reef_hal_event_elapsed_us(reef_event_t start, reef_event_t stop, float* us);
 
 /* One submission for a recorded sequence of launches (no counterpart in the reference,
  * which issues one hipModuleLaunchKernel per kernel, executor_base.cpp:191-221).  On this
- * device a launch call costs the host 3-4 us, more than most batch-1 kernels run; a recorded
- * sequence is replayed by the device at under 2 us per kernel.
+ * device a launch call costs the host 3-4 us; a recorded sequence is replayed by the device
+ * at under 2 us per kernel, which matters once kernels are shorter than a launch call.
  *   graph_begin(s): launches issued on `s` by the calling thread are recorded, not run;
  *   graph_end(s, &g): stops recording and builds the replayable sequence;
  *   graph_launch(g, s): enqueues the whole sequence on `s` (any stream without a launch window).

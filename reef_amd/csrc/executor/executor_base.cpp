@@ -9,7 +9,7 @@ namespace executor {
 
 ExecutorBase::ExecutorBase()
     : arena(nullptr), arena_bytes(0), base_mod(nullptr), s(nullptr), owns_stream(false),
-      use_graph(std::getenv("REEF_NO_GRAPH") == nullptr), model_graph(nullptr) {}
+      use_graph(std::getenv("REEF_GRAPH") != nullptr), model_graph(nullptr) {}
 
 ExecutorBase::~ExecutorBase() {
     drop_graph();

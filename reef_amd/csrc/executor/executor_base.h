@@ -50,9 +50,12 @@ public:
     Status launch_range(int begin, int end, GPUStream_t stream);
     // Enqueues the whole model without synchronising.  The kernel sequence of a model
     // never changes between runs (same functions, same argument blocks, same storages),
-    // so it is recorded once and replayed as ONE submission: the host pays one call
-    // instead of one per kernel.  set_graph_launch(false), or REEF_NO_GRAPH=1 in the
-    // environment, goes back to one launch call per kernel.
+    // so it can be recorded once and replayed as ONE submission: the host then pays one
+    // call instead of one per kernel.  Off by default (set_graph_launch(true), or
+    // REEF_GRAPH=1 in the environment, turns it on): a launch call costs the host 3-4 us,
+    // which hides behind kernels that run 5-15 us each, while a replay starts about
+    // 0.1 ms later than the first direct launch would.  It pays for models whose kernels
+    // are shorter than a launch call.
     Status launch_model(GPUStream_t stream);
     void set_graph_launch(bool on);
     bool graph_launch() const { return use_graph; }

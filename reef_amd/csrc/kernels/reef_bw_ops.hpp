@@ -36,7 +36,17 @@ __device__ __forceinline__ void splitk_reduce_body(const ReefOpDesc& d, int task
     if ((MN & 3) == 0) {
         // The partial tensors were written by another kernel and come from memory: the loads
         // of eight partials are issued together (a partial past S is loaded from the last one
-        // and dropped), the sums then run in ascending s as before.
+        // and dropped), the sums then run in ascending s as before.  The epilogue operands
+        // are fetched first for the same reason.
+        f32x4 resv = {0.f, 0.f, 0.f, 0.f};
+        float biasv[4], sh2v[4];
+        if (ep.residual) resv = *(const f32x4*)(ep.residual + i0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int ch = (int)((i0 + e) / N);
+            biasv[e] = ep.bias ? ep.bias[ch] : 0.0f;
+            sh2v[e] = ep.shift2 ? ep.shift2[ch] : 0.0f;
+        }
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
         for (int s0 = 0; s0 < S; s0 += 8) {
             f32x4 v[8];
@@ -50,7 +60,8 @@ __device__ __forceinline__ void splitk_reduce_body(const ReefOpDesc& d, int task
                 if (s0 + j < S) acc = (s0 + j == 0) ? v[j] : acc + v[j];
         }
 #pragma unroll
-        for (int e = 0; e < 4; ++e) ep.store(out, acc[e], (int)((i0 + e) / N), i0 + e);
+        for (int e = 0; e < 4; ++e)
+            ep.store_pre(out, acc[e], (int)((i0 + e) / N), i0 + e, resv[e], biasv[e], sh2v[e]);
     } else {
         for (int e = 0; e < 4 && i0 + e < MN; ++e) {
             float acc = ws[i0 + e];

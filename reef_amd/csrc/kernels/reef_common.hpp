@@ -114,6 +114,17 @@ struct Epilogue {
         out[idx] = o;
         if (out2) out2[idx] = act_apply(o + shift2[ch], act2);
     }
+    // The same with residual[idx], bias[ch] and shift2[ch] already in registers (loaded at
+    // kernel start, so their trip to memory overlaps the main loop instead of following it).
+    __device__ __forceinline__ void store_pre(float* out, float v, int ch, size_t idx, float resv,
+                                              float biasv, float sh2v) const {
+        if (residual) v = v + resv;
+        if (bias) v = v + biasv;
+        if (scale) v = fmaf(v, scale[ch], shift[ch]);
+        const float o = act_apply(v, act);
+        out[idx] = o;
+        if (out2) out2[idx] = act_apply(o + sh2v, act2);
+    }
 };
 
 }  // namespace reef_dev

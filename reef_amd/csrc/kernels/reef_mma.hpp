@@ -486,6 +486,11 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
   int M, N, split_k, split, rem, m0, n0;
   float* smem = (float*)smem_raw;
   f32x16 acc[T::TM][T::TN];
+  // wave-split-K tiles leave each wavefront only 16/KW accumulator elements to write
+  // out: few enough to fetch their bias / residual / second shift ahead of the K loop
+  constexpr bool EARLY = T::KW > 1;
+  constexpr int ER = EARLY ? T::RPW : 1;
+  float e_bias[T::TM][ER], e_sh2[T::TM][ER], e_res[T::TM][T::TN][ER];
   {
     const ReefOpDesc& d = d_in;
     const int* a = d.attr;
@@ -504,6 +509,35 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
     const int k_begin = split * k_chunk;
     const int k_end = min(K, k_begin + k_chunk);
     const int nk = (k_end - k_begin + T::BK - 1) / T::BK;
+
+    if (EARLY) {
+        // Epilogue operands of the few outputs this wavefront will write: issued now, used
+        // after the K loop.
+        const int flags = a[REEF_CONV_FLAGS];
+        if (split_k == 1) {
+            Epilogue ep;
+            ep.unpack(d, 3, flags, 0, 0);
+            const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
+            const WaveGeom<T> wg;
+            const int r0 = wg.wk * T::RPW;
+#pragma unroll
+            for (int tm = 0; tm < T::TM; ++tm)
+#pragma unroll
+                for (int rr = 0; rr < T::RPW; ++rr) {
+                    const int r = r0 + rr;
+                    const int m = m0 + wg.wm0 + tm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                    const bool mok = m < M;
+                    e_bias[tm][rr] = (ep.bias && mok) ? ep.bias[m] : 0.0f;
+                    e_sh2[tm][rr] = (ep.shift2 && mok) ? ep.shift2[m] : 0.0f;
+#pragma unroll
+                    for (int tn = 0; tn < T::TN; ++tn) {
+                        const int n = n0 + wg.wn0 + tn * 32 + l32;
+                        e_res[tm][tn][rr] = (ep.residual && mok && n < N) ? ep.residual[(size_t)m * N + n] : 0.0f;
+                    }
+                }
+        }
+        asm volatile("" ::: "memory");  // keeps the loads above the K loop
+    }
 
     bool ok;
     if (MODE == CONV_POINTWISE) {
@@ -621,7 +655,13 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
             for (int rr = 0; rr < T::RPW; ++rr) {
                 const int r = r0 + rr;
                 const int m = m0 + wm0 + tm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                if (m < M && n < N) ep.store(dst, res[tm][tn][rr], m, (size_t)m * N + n);
+                if (m < M && n < N) {
+                    if (EARLY)
+                        ep.store_pre(dst, res[tm][tn][rr], m, (size_t)m * N + n, e_res[tm][tn][rr],
+                                     e_bias[tm][rr], e_sh2[tm][rr]);
+                    else
+                        ep.store(dst, res[tm][tn][rr], m, (size_t)m * N + n);
+                }
             }
         }
     return true;

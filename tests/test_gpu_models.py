@@ -158,6 +158,7 @@ def test_recorded_submission_replays_bit_identical(tmp_path, kind):
     g = nets.resnet(18)
     d = write_model(g, tmp_path)
     rec = B.Executor.from_dir(d, g.name, kind)
+    rec.set_graph_launch(True)
     one = B.Executor.from_dir(d, g.name, kind)
     one.set_graph_launch(False)
     rng = np.random.default_rng(5)

@@ -71,13 +71,14 @@ def test_resnet_binding_matches_graph_oracle(fake, small_dirs, kind, pre):
 
 @pytest.mark.parametrize("kind", [B.BASE, B.TRANS, B.HYBRID])
 def test_whole_model_runs_replay_one_recorded_submission(fake, small_dirs, kind):
-    """execute() records the model's launch sequence on first use and replays it as one
-    submission afterwards; switching that off goes back to one launch call per kernel.  Both
-    ways run the same kernels with the same arguments."""
+    """With graph launch on, execute() records the model's launch sequence on first use and
+    replays it as one submission afterwards; off means one launch call per kernel.  Both ways
+    run the same kernels with the same arguments."""
     g, d = small_dirs["tiny18"]
     x = nets.image_input("t", (3, 32, 32))
     want = oracle_output(g, d, x)
     exe = B.Executor.from_dir(d, g.name, kind)
+    exe.set_graph_launch(True)
     exe.set_input_checked("data", x)
     n = exe.num_kernels()
     for run in range(3):
