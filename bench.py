@@ -96,11 +96,14 @@ def summarize(r, sched, n_be):
             "span_s": round(r["span_s"], 3)}
 
 
-def corun(models, rt_name, be_name, n_be, mode, requests, warmup, wait_sync=True, solo=True):
+def corun(models, rt_name, be_name, n_be, mode, requests, warmup, wait_sync=True, solo=True,
+          dkp_slack=None):
     """One scheduler, one real-time model, n_be best-effort clients of one model."""
     from reef_amd import binding as B
     s = B.Scheduler(mode)
     s.set_wait_sync(wait_sync)
+    if dkp_slack is not None:
+        s.set_dkp_slack_percent(dkp_slack)
     g_rt, d_rt = models[rt_name]
     rt = s.load_model(d_rt, g_rt.name)
     s.bind_model_queue(s.create_queue(B.QUEUE_RT), rt)

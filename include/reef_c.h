@@ -105,6 +105,9 @@ int reef_scheduler_shutdown(reef_scheduler_t s);
 int reef_scheduler_mode(reef_scheduler_t s);
 void reef_scheduler_set_wait_sync(reef_scheduler_t s, int value);
 void reef_scheduler_set_be_stream_cap(reef_scheduler_t s, int value);
+/* Share (percent) of a real-time kernel's profiled latency that padded best-effort workgroups
+ * may take; 100 is the reference's rule (scheduler.cpp:565-572). */
+void reef_scheduler_set_dkp_slack_percent(reef_scheduler_t s, int value);
 int64_t reef_scheduler_avg_preempt_latency(reef_scheduler_t s);
 int64_t reef_scheduler_max_preempt_latency(reef_scheduler_t s);
 int64_t reef_scheduler_avg_kernel_sel_latency(reef_scheduler_t s);

@@ -273,6 +273,9 @@ class Scheduler:
     def set_be_stream_cap(self, v):
         lib().reef_scheduler_set_be_stream_cap(self.h, int(v))
 
+    def set_dkp_slack_percent(self, v):
+        lib().reef_scheduler_set_dkp_slack_percent(self.h, int(v))
+
     def avg_preempt_latency(self):
         return lib().reef_scheduler_avg_preempt_latency(self.h)
 

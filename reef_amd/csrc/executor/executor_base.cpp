@@ -86,9 +86,6 @@ Status ExecutorBase::init_executor_base(const char* json_file_path, GPUModule_t 
         for (size_t j = 0; j < ki.attrs.size(); ++j) d.attr[j] = ki.attrs[j];
     }
 
-    REEF_LOG_INFO("create base model stream");
-    GPU_RETURN_STATUS(reef_hal_stream_create(0, &s));
-    owns_stream = true;
     return Status::Succ;
 }
 
@@ -165,8 +162,21 @@ Status ExecutorBase::find_storage_idx(const std::string& name, size_t& idx) {
 }
 
 size_t ExecutorBase::num_kernels() const { return model->kernels.size(); }
-void ExecutorBase::set_stream(GPUStream_t stream) { s = stream; }
-GPUStream_t ExecutorBase::stream() const { return s; }
+void ExecutorBase::set_stream(GPUStream_t stream) {
+    if (owns_stream && s) reef_hal_stream_destroy(s);
+    owns_stream = false;
+    s = stream;
+}
+// The model's own stream is made on first use: an executor that a scheduler drives
+// runs on the scheduler's streams and never needs one, and every stream that exists
+// takes a share of the few hardware queues.
+GPUStream_t ExecutorBase::stream() {
+    if (!s) {
+        REEF_LOG_INFO("create base model stream");
+        if (reef_hal_stream_create(0, &s) == 0) owns_stream = true;
+    }
+    return s;
+}
 
 // The reference's execute(stream) drops its argument and runs on the default
 // stream (executor_base.cpp:191-194); here the stream is honoured.

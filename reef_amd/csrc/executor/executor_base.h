@@ -44,7 +44,7 @@ public:
 
     size_t num_kernels() const;
     void set_stream(GPUStream_t stream);
-    GPUStream_t stream() const;
+    GPUStream_t stream();
 
     // Launches kernels [begin, end) without synchronising (for timing loops).
     Status launch_range(int begin, int end, GPUStream_t stream);

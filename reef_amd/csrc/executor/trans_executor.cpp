@@ -157,6 +157,8 @@ int TransExecutor::proxy_level(int op, int tile, int mode) {
         if (mode != REEF_CONV_MODE_GENERAL && mode != REEF_CONV_MODE_POINTWISE) return -1;
         if (tile == REEF_TILE_64x64 || tile == REEF_TILE_128x32) return 1;
         if (tile == REEF_TILE_128x64) return 2;
+        if (tile == REEF_TILE_32x32k4 || tile == REEF_TILE_64x32k2 || tile == REEF_TILE_32x64k2)
+            return 2;
         return -1;
     }
     if (op == REEF_OP_GEMM || op == REEF_OP_NONE) return -1;

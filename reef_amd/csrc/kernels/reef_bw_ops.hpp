@@ -22,6 +22,7 @@
 namespace reef_dev {
 
 // out = act(sum_{s ascending} ws[s] (+res)(+bias)(*scale+shift)); 4 elements per thread.
+template <int BATCH>
 __device__ __forceinline__ void splitk_reduce_body(const ReefOpDesc& d, int task) {
     const int* a = d.attr;
     const int M = a[REEF_RED_M], N = a[REEF_RED_N], S = a[REEF_RED_SPLIT_K];
@@ -35,7 +36,7 @@ __device__ __forceinline__ void splitk_reduce_body(const ReefOpDesc& d, int task
     if (i0 >= MN) return;
     if ((MN & 3) == 0) {
         // The partial tensors were written by another kernel and come from memory: the loads
-        // of eight partials are issued together (a partial past S is loaded from the last one
+        // of BATCH partials are issued together (a partial past S is loaded from the last one
         // and dropped), the sums then run in ascending s as before.  The epilogue operands
         // are fetched first for the same reason.
         f32x4 resv = {0.f, 0.f, 0.f, 0.f};
@@ -48,15 +49,15 @@ __device__ __forceinline__ void splitk_reduce_body(const ReefOpDesc& d, int task
             sh2v[e] = ep.shift2 ? ep.shift2[ch] : 0.0f;
         }
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-        for (int s0 = 0; s0 < S; s0 += 8) {
-            f32x4 v[8];
+        for (int s0 = 0; s0 < S; s0 += BATCH) {
+            f32x4 v[BATCH];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
+            for (int j = 0; j < BATCH; ++j) {
                 const int s = min(s0 + j, S - 1);
                 v[j] = *(const f32x4*)(ws + (size_t)s * MN + i0);
             }
 #pragma unroll
-            for (int j = 0; j < 8; ++j)
+            for (int j = 0; j < BATCH; ++j)
                 if (s0 + j < S) acc = (s0 + j == 0) ? v[j] : acc + v[j];
         }
 #pragma unroll

@@ -52,7 +52,7 @@ struct OpGemm {
             return true;                                                                        \
         }                                                                                       \
     };
-REEF_SIMPLE_OP(OpSplitKReduce, splitk_reduce_body)
+REEF_SIMPLE_OP(OpSplitKReduce, splitk_reduce_body<8>)
 REEF_SIMPLE_OP(OpDwConv, dwconv2d_body)
 REEF_SIMPLE_OP(OpPool, pool2d_body)
 REEF_SIMPLE_OP(OpGap, global_avgpool_body)
@@ -221,7 +221,8 @@ REEF_ENTRY(multiply, OpMocked<true>)
 // occupancy classes that matter for this kernel set, <n> = wavefronts per SIMD:
 //   merge_framework_8  bandwidth-bound ops only                          (<= 64 registers)
 //   merge_framework_3  + conv (general, pointwise) tiles 64x64 / 128x32    (<= 168)
-//   merge_framework_2  + conv (general, pointwise) tile 128x64             (<= 256)
+//   merge_framework_2  + conv (general, pointwise) tile 128x64 and the
+//                        wave-split-K tiles                                   (<= 256)
 // Kernels outside these sets (the other tiles, the unaligned-K convolution, GEMM)
 // are never merged: they run single-sided through their own entry.
 // LDS is dynamic (the host passes the larger of the two sides' needs, as
@@ -238,15 +239,25 @@ __device__ __forceinline__ void run_op(const ReefDkpSide& s, int task, char* sme
                 if (d.attr[REEF_CONV_MODE] == CONV_POINTWISE) {
                     if (tile == REEF_TILE_64x64) OpConv<Tile64x64, CONV_POINTWISE>::run(d, task, smem, np);
                     else if (tile == REEF_TILE_128x32) OpConv<Tile128x32, CONV_POINTWISE>::run(d, task, smem, np);
+                    else if (LEVEL >= 2 && tile == REEF_TILE_32x32k4) OpConv<Tile32x32k4, CONV_POINTWISE>::run(d, task, smem, np);
+                    else if (LEVEL >= 2 && tile == REEF_TILE_64x32k2) OpConv<Tile64x32k2, CONV_POINTWISE>::run(d, task, smem, np);
+                    else if (LEVEL >= 2 && tile == REEF_TILE_32x64k2) OpConv<Tile32x64k2, CONV_POINTWISE>::run(d, task, smem, np);
                     else if (LEVEL >= 2 && tile == REEF_TILE_128x64) OpConv<Tile128x64, CONV_POINTWISE>::run(d, task, smem, np);
                 } else if (d.attr[REEF_CONV_MODE] == CONV_GENERAL) {
                     if (tile == REEF_TILE_64x64) OpConv<Tile64x64, CONV_GENERAL>::run(d, task, smem, np);
                     else if (tile == REEF_TILE_128x32) OpConv<Tile128x32, CONV_GENERAL>::run(d, task, smem, np);
                     else if (LEVEL >= 2 && tile == REEF_TILE_128x64) OpConv<Tile128x64, CONV_GENERAL>::run(d, task, smem, np);
+                    else if (LEVEL >= 2 && tile == REEF_TILE_32x32k4) OpConv<Tile32x32k4, CONV_GENERAL>::run(d, task, smem, np);
+                    else if (LEVEL >= 2 && tile == REEF_TILE_64x32k2) OpConv<Tile64x32k2, CONV_GENERAL>::run(d, task, smem, np);
+                    else if (LEVEL >= 2 && tile == REEF_TILE_32x64k2) OpConv<Tile32x64k2, CONV_GENERAL>::run(d, task, smem, np);
                 }
             }
             break;
-        case REEF_OP_SPLITK_REDUCE: splitk_reduce_body(d, task); break;
+        case REEF_OP_SPLITK_REDUCE:
+            // fewer partial loads in flight where the class allows 64 registers only
+            if (LEVEL == 0) splitk_reduce_body<4>(d, task);
+            else splitk_reduce_body<8>(d, task);
+            break;
         case REEF_OP_DWCONV2D: dwconv2d_body(d, task); break;
         case REEF_OP_POOL2D: pool2d_body(d, task); break;
         case REEF_OP_GLOBAL_AVGPOOL: global_avgpool_body(d, task); break;

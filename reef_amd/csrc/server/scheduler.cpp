@@ -1,6 +1,7 @@
 #include "server/scheduler.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 
 namespace reef {
@@ -52,17 +53,28 @@ REEFScheduler::REEFScheduler(ScheduleMode _mode)
     // Window of kernels a best-effort stream keeps on the device
     // (scheduler.cpp:29-33: 2, or 1024 when preemption waits for completion).
     be_stream_device_queue_cap = (mode == WaitPreempt) ? 1024 : 2;
+    dkp_slack_percent = 50;
+    if (const char* e = std::getenv("REEF_DKP_SLACK")) dkp_slack_percent = std::atoi(e);
 }
 
 REEFScheduler::~REEFScheduler() {
     if (scheduler) shutdown();
+    // give the hardware queues back: a later scheduler in the same process would otherwise
+    // share them with streams nobody uses
+    for (auto& q : be_queues)
+        if (q && q->stream) reef_hal_stream_destroy(q->stream);
+    if (rt_queue && rt_queue->stream) reef_hal_stream_destroy(rt_queue->stream);
+    if (preempt_stream) reef_hal_stream_destroy(preempt_stream);
+    model_pool.clear();
+    if (preempt_flag) reef_hal_free(preempt_flag, REEF_MEM_DEVICE_FINEGRAINED);
 }
 
 // Streams and the shared preemption flag (scheduler.cpp:24-28).
 Status REEFScheduler::ensure_gpu() {
     if (gpu_ready) return Status::Succ;
     GPU_RETURN_STATUS(reef_hal_init(0));
-    GPU_RETURN_STATUS(reef_hal_stream_create(0, &preempt_stream));
+    // only wait-based preemption orders anything on a stream of its own
+    if (mode == WaitPreempt) GPU_RETURN_STATUS(reef_hal_stream_create(0, &preempt_stream));
     GPU_RETURN_STATUS(reef_hal_malloc(4, REEF_MEM_DEVICE_FINEGRAINED, &preempt_flag));
     GPU_RETURN_STATUS(reef_hal_memset(preempt_flag, 0, 4));
     gpu_ready = true;
@@ -430,14 +442,14 @@ void REEFScheduler::execute_rt_task(std::shared_ptr<Task>& task) {
 // ---------------------------------------------------------------- dynamic kernel padding
 // Can `be` ride along with `rt`, and with how many workgroups?  (scheduler.cpp:533-602)
 //   fits      : occupancy(max resource, max block) >= rt.min_occupancy
-//   be_occ    : the largest j+1 <= merged occupancy with be.latency[j] <= rt.total_latency
+//   be_occ    : the largest j+1 <= merged occupancy with be.latency[j] <= rt.total_latency * slack
 //   partition : CUs the rt kernel really needs, in whole slots per XCD
-//   be_blocks : (CUs left) * (rt_latency / be_latency[be_occ-1]) * be_occ, clamped to what is left
+//   be_blocks : (CUs left) * (rt_latency * slack / be_latency[be_occ-1]) * be_occ, clamped to what is left
 REEFScheduler::PadDecision REEFScheduler::decide_padding(const TransExecutor::KernelArg& rt,
                                                          const TransExecutor::KernelArg& be,
                                                          int be_block_offset,
                                                          const GPUConfig::KernelResource& proxy,
-                                                         int num_cus, int num_xcds) {
+                                                         int num_cus, int num_xcds, int slack_percent) {
     PadDecision d;
     d.rt_occupancy = rt.min_occupancy;
     d.final_occupancy = rt.min_occupancy;
@@ -451,9 +463,10 @@ REEFScheduler::PadDecision REEFScheduler::decide_padding(const TransExecutor::Ke
 
     int be_occupancy = 0;
     const int rt_latency = rt.profile.total_latency;
+    const int be_budget = (int)((int64_t)rt_latency * slack_percent / 100);
     for (int j = merged_occupancy - 1; j >= 0; j--) {
         if ((int)be.profile.latency.size() <= j) continue;
-        if (be.profile.latency[j] <= rt_latency) {
+        if (be.profile.latency[j] <= be_budget) {
             be_occupancy = j + 1;
             break;
         }
@@ -462,7 +475,7 @@ REEFScheduler::PadDecision REEFScheduler::decide_padding(const TransExecutor::Ke
     const int be_latency = std::max(be.profile.latency[be_occupancy - 1], 1);
 
     const int partition = TransExecutor::cu_partition_for(rt.block_num, num_cus, num_xcds);
-    const int be_iters = rt_latency / be_latency;
+    const int be_iters = be_budget / be_latency;
     int be_blocks = (num_cus - partition) * be_iters * be_occupancy;
     be_blocks = std::min(be_blocks, be.block_num - be_block_offset);
     if (be_blocks <= 0) return d;
@@ -513,7 +526,7 @@ void REEFScheduler::dynamic_kernel_padding(std::shared_ptr<Task>& rt_task) {
             if (rt_args.proxy_level < 0 || ka.proxy_level < 0) continue;
             const int level = std::max(rt_args.proxy_level, ka.proxy_level);
             PadDecision d = decide_padding(rt_args, ka, cand->block_offset, proxy_res[level], num_cus,
-                                           num_xcds);
+                                           num_xcds, dkp_slack_percent);
             if (!d.merge) continue;
             dec = d;
             be_task = cand;

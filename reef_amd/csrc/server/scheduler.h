@@ -98,7 +98,7 @@ public:
                                       const executor::TransExecutor::KernelArg& be,
                                       int be_block_offset,
                                       const executor::GPUConfig::KernelResource& proxy,
-                                      int num_cus, int num_xcds);
+                                      int num_cus, int num_xcds, int slack_percent = 100);
     // Rollback after a reset (scheduler.cpp:320-323).
     static int rollback_kernel_offset(int launch_offset, int dropped, int window, int kernel_offset);
 
@@ -121,6 +121,16 @@ public:
     ScheduleMode sche_mode() const { return mode; }
     void set_wait_sync(bool value) { wait_sync = value; }
     void set_be_stream_cap(int value) { be_stream_device_queue_cap = value; }
+    // Share of a real-time kernel's profiled latency that padded best-effort workgroups may
+    // take (100 = the reference's rule, be.latency <= rt.latency, scheduler.cpp:565-572).
+    // The merged launch ends when its slowest workgroup ends, and on this device kernels run
+    // for microseconds, so a best-effort workgroup predicted to take exactly as long as the
+    // real-time kernel usually ends after it; a smaller share keeps that out of the
+    // real-time latency at the price of fewer padded kernels.  Default 50 (REEF_DKP_SLACK in
+    // the environment overrides): measured on MI355X with ResNet-152 real-time, 100 costs the
+    // real-time task 7 % (DenseNet-201 best-effort) for 2-4 % best-effort throughput, 50
+    // costs it under 1 %.
+    void set_dkp_slack_percent(int value) { dkp_slack_percent = value; }
     Status run();
     Status shutdown();
     int64_t avg_preempt_latency() const;     // microseconds
@@ -176,6 +186,7 @@ private:
     executor::GPUDevicePtr_t preempt_flag;
     bool preempted;
     int be_stream_device_queue_cap;
+    int dkp_slack_percent;
     std::atomic<bool> _shutdown;
 
     uint64_t preempt_count;
