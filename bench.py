@@ -65,6 +65,22 @@ def cpu_baseline(model_dir, name, x, budget_s=30.0):
                       "TVM-llvm build of the model" % len(times)}, orc
 
 
+def calibrate_copy(mib, root):
+    """A plain copy kernel over a known number of bytes: what the memory counters read for
+    it fixes their scale."""
+    from reef_amd import binding as B
+    from reef_amd.modelgen import builder as MB
+    n = mib * 1024 * 1024 // 4
+    g = MB.GraphBuilder("copycal")
+    x = g.input("data", (n,))
+    g.copy_into(x, g.temp((n,), name="output"), 0)
+    d = os.path.dirname(g.write(os.path.join(root, g.name)))
+    exe = B.Executor.from_dir(d, g.name, B.BASE)
+    for _ in range(20):
+        exe.execute()
+    exe.close()
+
+
 def write_models(names, root):
     from reef_amd.modelgen import nets
     out = {}
@@ -153,6 +169,13 @@ def main():
     ap.add_argument("--kernel-iters", type=int, default=20)
     ap.add_argument("--configs", default="3,4,5", help="co-location scenarios to run (3 is the headline)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--solo-only", action="store_true",
+                    help="only the solo ResNet-152 executor part (whole-model and per-kernel timing); "
+                         "the value is then the solo p99 -- this is the command the kernel profiles "
+                         "under profiles/ are taken with")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
+                    help="also run a plain copy kernel over this many MiB 20 times (scale for the "
+                         "FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--workdir", default=None)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -164,7 +187,9 @@ def main():
     from reef_amd import binding as B
 
     tmp = tempfile.TemporaryDirectory(dir=args.workdir)
-    names = ["resnet152", "densenet201"]
+    names = ["resnet152"] if args.solo_only else ["resnet152", "densenet201"]
+    if args.solo_only:
+        configs = []
     if 4 in configs:
         names.append("mobilenetv2")
     if 5 in configs:
@@ -173,17 +198,27 @@ def main():
     g, d = models["resnet152"]
     _, x = model_input("resnet152")
 
+    if args.calibrate_copy:
+        calibrate_copy(args.calibrate_copy, tmp.name)
+
     # ---- headline: RT ResNet-152 + 4 BE DenseNet-201 ----------------------------------
-    t0 = time.perf_counter()
-    head = corun(models, "resnet152", "densenet201", 4, B.MODE_REEF, args.steps, args.warmup)
-    wall_s = time.perf_counter() - t0
-    reset_only = corun(models, "resnet152", "densenet201", 4, B.MODE_RESET, args.steps, args.warmup,
-                       solo=False)
+    head = reset_only = None
+    wall_s = 0.0
+    if not args.solo_only:
+        t0 = time.perf_counter()
+        head = corun(models, "resnet152", "densenet201", 4, B.MODE_REEF, args.steps, args.warmup)
+        wall_s = time.perf_counter() - t0
+        reset_only = corun(models, "resnet152", "densenet201", 4, B.MODE_RESET, args.steps, args.warmup,
+                           solo=False)
 
     # ---- solo executor: whole-model device time and per-kernel durations ---------------
     exe = B.Executor.from_dir(d, g.name, B.HYBRID)
     exe.set_input_checked("data", x)
-    lat_us, dev_us = exe.time_model(B.RUN_DEFAULT, 20, 200)
+    t0 = time.perf_counter()
+    solo_iters = args.steps if args.solo_only else 200
+    lat_us, dev_us = exe.time_model(B.RUN_DEFAULT, args.warmup if args.solo_only else 20, solo_iters)
+    if args.solo_only:
+        wall_s = time.perf_counter() - t0
     n = exe.num_kernels()
     kus = np.array([exe.time_kernel(i, B.RUN_DEFAULT, 3, args.kernel_iters) for i in range(n)])
     names_k = [k["name"].split("#")[0] for k in g.kernels]
@@ -207,16 +242,21 @@ def main():
     if os.path.exists(tpath):
         traffic = json.load(open(tpath)).get(dom)
 
-    p99 = head["loaded"]["rt_ms"]["p99"]
-    solo_p99 = head["solo"]["rt_ms"]["p99"]
+    if args.solo_only:
+        p99 = pct(lat_us, 99)
+        solo_p99 = p99
+    else:
+        p99 = head["loaded"]["rt_ms"]["p99"]
+        solo_p99 = head["solo"]["rt_ms"]["p99"]
     out = {
-        "metric": "ResNet-152 RT p99 latency w/ 4 BE clients",
+        "metric": "ResNet-152 RT p99 latency, solo, back to back" if args.solo_only
+                  else "ResNet-152 RT p99 latency w/ 4 BE clients",
         "value": p99,
         "unit": "ms",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": head["loaded"]["rt_ms"]["mean"],
+        "ms_per_step": round(float(lat_us.mean()) / 1e3, 4) if args.solo_only else head["loaded"]["rt_ms"]["mean"],
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
@@ -227,8 +267,9 @@ def main():
                                "224x224); seeded He-normal weights; REEF mode",
                    "rt_kernels_per_inference": n, "rt_gflop_per_inference": round(g.flops / 1e9, 3)},
         "rt_p99_vs_solo": round(p99 / solo_p99, 4),
-        "rt_p50_vs_solo": round(head["loaded"]["rt_ms"]["p50"] / head["solo"]["rt_ms"]["p50"], 4),
-        "preempt_us": head["preempt_us"],
+        "rt_p50_vs_solo": None if args.solo_only
+        else round(head["loaded"]["rt_ms"]["p50"] / head["solo"]["rt_ms"]["p50"], 4),
+        "preempt_us": None if args.solo_only else head["preempt_us"],
         "corun_resnet152_4x_densenet201": head,
         "corun_reset_mode": reset_only,
         "solo_back_to_back_ms": {"p50": pct(lat_us, 50), "p99": pct(lat_us, 99),

@@ -473,6 +473,20 @@ __device__ __forceinline__ bool k_loop(LA& la, LB& lb, int nk, float* smem, f32x
     }
 }
 
+// ---- task -> tile order that keeps neighbours on one XCD ---------------------
+// The dispatcher hands workgroup j to XCD j % 8 and every XCD has its own L2.  Tiles
+// are numbered (split, m tile, n tile) row-major, so neighbours in that order share
+// weight rows and input columns; handing XCD x the x-th CONTIGUOUS eighth of the
+// order (instead of every eighth tile) lets one L2 fetch those once for all of them.
+// Without it a 32-row weight tile used by seven column tiles is fetched by seven L2s.
+// A bijection on [0, total): chunk x holds total/8 tiles, plus one if x < total % 8.
+__device__ __forceinline__ int xcd_chunked(int task, int total) {
+    constexpr int X = 8;
+    const int x = task % X, l = task / X;
+    const int base = total / X, r = total - base * X;
+    return x * base + min(x, r) + l;
+}
+
 // ---- reef_conv2d ------------------------------------------------------------
 // MODE selects the tile loaders, one K loop per kernel symbol:
 //   CONV_GENERAL    im2col gather, 128-bit weight loads        (K % 4 == 0)
@@ -501,6 +515,7 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
     const int k_chunk = a[REEF_CONV_K_CHUNK];
     const int n_tiles = a[REEF_CONV_N_TILES];
     const int tiles = a[REEF_CONV_M_TILES] * n_tiles;
+    task = xcd_chunked(task, tiles * split_k);
     split = task / tiles;
     rem = task - split * tiles;
     const int mt = rem / n_tiles, nt = rem - mt * n_tiles;
