@@ -143,6 +143,10 @@ int reef_loadgen_run(reef_scheduler_t s, const reef_load_config* cfg, int64_t* r
  *        merged_block_size, lds}. */
 int reef_dkp_decide(const int rt[7], const int be[7], const int* be_latency, int n_lat,
                     int be_block_offset, const int proxy[3], int num_cus, int num_xcds, int out[8]);
+/* The same with the share (percent) of rt's latency that best-effort work may take; 100 above. */
+int reef_dkp_decide_slack(const int rt[7], const int be[7], const int* be_latency, int n_lat,
+                          int be_block_offset, const int proxy[3], int num_cus, int num_xcds,
+                          int slack_percent, int out[8]);
 int reef_dkp_rollback(int launch_offset, int dropped, int window, int kernel_offset);
 
 /* GPUConfig (src/reef/executor/hip/hip_impl.cpp:9-74) */

@@ -297,6 +297,12 @@ int reef_loadgen_run(reef_scheduler_t h, const reef_load_config* c, int64_t* rt_
 
 int reef_dkp_decide(const int rt[7], const int be[7], const int* be_latency, int n_lat,
                     int be_block_offset, const int proxy[3], int num_cus, int num_xcds, int out[8]) {
+    return reef_dkp_decide_slack(rt, be, be_latency, n_lat, be_block_offset, proxy, num_cus, num_xcds,
+                                 100, out);
+}
+int reef_dkp_decide_slack(const int rt[7], const int be[7], const int* be_latency, int n_lat,
+                          int be_block_offset, const int proxy[3], int num_cus, int num_xcds,
+                          int slack_percent, int out[8]) {
     auto fill = [](TransExecutor::KernelArg& ka, const int v[7]) {
         ka.block_num = v[0];
         ka.min_occupancy = v[1];
@@ -312,7 +318,7 @@ int reef_dkp_decide(const int rt[7], const int be[7], const int* be_latency, int
     bea.profile.latency.assign(be_latency, be_latency + n_lat);
     GPUConfig::KernelResource pr{proxy[2], proxy[0], proxy[1], 0};
     REEFScheduler::PadDecision d =
-        REEFScheduler::decide_padding(rta, bea, be_block_offset, pr, num_cus, num_xcds);
+        REEFScheduler::decide_padding(rta, bea, be_block_offset, pr, num_cus, num_xcds, slack_percent);
     out[0] = d.merge; out[1] = d.rt_occupancy; out[2] = d.be_occupancy; out[3] = d.final_occupancy;
     out[4] = d.cu_partition; out[5] = d.be_block_num; out[6] = d.merged_block_size;
     out[7] = d.resource.shared_memory;

@@ -182,3 +182,45 @@ def test_dkp_resnet_in_resnet_shadow(dirs):
     assert be["padded"]
     print("padded kernels:", s.padded_kernels(), "kernel selection ns:", s.avg_kernel_sel_latency())
     s.shutdown()
+
+
+@pytest.mark.parametrize("mode", [B.MODE_RESET, B.MODE_REEF])
+def test_load_generator_preemption_under_load(dirs, mode):
+    """One open-loop real-time client (ResNet-18, exponential gaps, mean 3 ms) against three
+    closed-loop best-effort ResNet-50 clients: dozens of preemptions, and afterwards every model
+    still holds exactly the output of an uninterrupted solo run.  With wait_sync the recorded
+    preemption span covers the drain of every best-effort stream; it has to stay far below a
+    best-effort inference (which is what a scheduler without preemption would wait for)."""
+    x50 = nets.image_input("resnet50", (3, 224, 224))
+    x18 = nets.image_input("resnet18", (3, 224, 224))
+    ref_be = solo_output(dirs["resnet50"], "resnet50", x50)
+    ref_rt = solo_output(dirs["resnet18"], "resnet18", x18)
+    s = B.Scheduler(mode)
+    s.set_wait_sync(True)
+    rt_mid = s.load_model(dirs["resnet18"], "resnet18")
+    s.bind_model_queue(s.create_queue(B.QUEUE_RT), rt_mid)
+    s.set_input(rt_mid, x18, "data")
+    bes = []
+    for _ in range(3):
+        m = s.load_model(dirs["resnet50"], "resnet50")
+        s.bind_model_queue(s.create_queue(B.QUEUE_BE), m)
+        s.set_input(m, x50, "data")
+        bes.append(m)
+    s.run()
+    r = s.run_load(rt_mid, bes, requests=60, warmup=10, mean_interval_us=3000.0, seed=11)
+    assert len(r["rt_latency_us"]) == 60 and (r["rt_exec_us"] > 0).all()
+    assert r["be_completed"].sum() > 0
+    assert r["be_preempted"].sum() > 0
+    ps = s.preempt_samples()
+    assert len(ps) >= 30
+    print("mode %d: rt p50 %.0f us, preempt mean %.1f max %d us over %d, BE done %s preempted %s padded %s"
+          % (mode, np.percentile(r["rt_latency_us"], 50), ps.mean(), ps.max(), len(ps),
+             r["be_completed"], r["be_preempted"], r["be_padded"]))
+    assert ps.mean() < 200 and np.percentile(ps, 95) < 400      # microseconds
+    np.testing.assert_array_equal(s.get_output(rt_mid, 1000), ref_rt)
+    # let every best-effort client finish one more uninterrupted inference, then compare
+    r2 = s.run_load(rt_mid, bes, requests=0, be_only_ms=30)
+    assert (r2["be_completed"] > 0).all()
+    for m in bes:
+        np.testing.assert_array_equal(s.get_output(m, 1000), ref_be)
+    s.shutdown()

@@ -2,6 +2,7 @@
 launch geometry per flavour, error codes, preemption rollback and idempotence,
 dynamic kernel padding bookkeeping.  The backend executes every completed
 "kernel" with the CPU oracle, so outputs are real."""
+import ctypes
 import json
 import os
 import time
@@ -244,3 +245,67 @@ def test_scheduler_dkp_pads_to_completion(fake, small_dirs):
     assert len(merged) == s.padded_kernels() >= 2
     assert s.avg_kernel_sel_latency() >= 0
     s.shutdown()
+
+
+def test_load_generator_counts_and_outputs(fake, small_dirs):
+    """The in-process clients (request loops of src/example/rpc_client_cont.cpp:20-36): one open-loop
+    real-time client with exponential gaps, two closed-loop best-effort clients.  Every recorded
+    request has submit <= start <= end, best-effort clients complete work, and the models'
+    outputs stay those of the oracle whatever got preempted on the way."""
+    gb, db = small_dirs["tiny18"]
+    gm, dm = small_dirs["mocked_kernel"]
+    x = nets.image_input("t", (3, 32, 32))
+    ref = oracle_output(gb, db, x)
+    fake.lib.fake_hal_set_auto_progress(4)
+    s = B.Scheduler(B.MODE_RESET)
+    s.set_wait_sync(True)
+    rt_mid = s.load_model(dm, gm.name)
+    s.bind_model_queue(s.create_queue(B.QUEUE_RT), rt_mid)
+    for n in "abc":
+        s.set_input(rt_mid, THREE, n)
+    bes = []
+    for _ in range(2):
+        m = s.load_model(db, gb.name)
+        s.bind_model_queue(s.create_queue(B.QUEUE_BE), m)
+        s.set_input(m, x, "data")
+        bes.append(m)
+    s.run()
+    r = s.run_load(rt_mid, bes, requests=12, warmup=3, mean_interval_us=25000.0, seed=7)
+    assert len(r["rt_latency_us"]) == 12
+    assert (r["rt_queue_us"] >= 0).all() and (r["rt_exec_us"] >= 0).all()
+    np.testing.assert_allclose(r["rt_latency_us"], r["rt_queue_us"] + r["rt_exec_us"], atol=1e-3)
+    assert r["span_s"] > 12 * 0.005
+    assert r["be_completed"].sum() > 0 and (r["be_preempted"] <= r["be_completed"]).all()
+    assert s.preempt_times() > 0
+    ph = s.preempt_phases()
+    assert ph["flag_ns"] >= 0 and ph["drop_ns"] >= 0 and ph["drain_ns"] >= 0
+    np.testing.assert_array_equal(s.get_output(rt_mid, 8192), np.full(8192, 18.0, np.float32))
+    for m in bes:
+        np.testing.assert_array_equal(s.get_output(m, 16), ref)
+    # best-effort only
+    r2 = s.run_load(rt_mid, bes, requests=0, be_only_ms=50)
+    assert len(r2["rt_latency_us"]) == 0 and r2["be_completed"].sum() > 0
+    s.shutdown()
+
+
+def test_dkp_slack_limits_padding(fake):
+    """set_dkp_slack_percent: best-effort work must fit the given share of the real-time kernel's
+    latency (100 = be.latency <= rt.latency, src/reef/server/scheduler.cpp:565-572)."""
+    L = B.lib()
+    rt = (ctypes.c_int * 7)(64, 1, 256, 64, 32, 0, 100)       # 64 blocks, latency 100 us
+    be = (ctypes.c_int * 7)(512, 1, 256, 64, 32, 0, 0)
+    lat = (ctypes.c_int * 4)(60, 70, 90, 120)                 # per occupancy 1..4
+    proxy = (ctypes.c_int * 3)(64, 32, 0)
+    out = (ctypes.c_int * 8)()
+    got = {}
+    for slack in (100, 80, 65, 50):
+        assert L.reef_dkp_decide_slack(rt, be, lat, 4, 0, proxy, 256, 8, slack, out) == 0
+        got[slack] = list(out)
+    assert got[100][0] == 1 and got[100][2] == 3     # occupancy 3: 90 <= 100
+    assert got[80][0] == 1 and got[80][2] == 2       # 70 <= 80
+    assert got[65][0] == 1 and got[65][2] == 1       # 60 <= 65
+    assert got[50][0] == 0                           # nothing fits half the latency
+    # be_blocks = (256 - partition) * (budget / be_latency) * be_occ
+    part = got[100][4]
+    assert got[100][5] == min(512, (256 - part) * (100 // 90) * 3)
+    assert got[65][5] == min(512, (256 - part) * (65 // 60) * 1)
