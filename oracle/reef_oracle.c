@@ -22,7 +22,15 @@
  *     brute-force definitions on tiny shapes, algebraic invariants
  *     (linearity, 1x1 conv == GEMM, softmax rows sum to 1, LN rows have
  *     mean 0 / variance 1), and torch.nn.functional on CPU in fp64.
- *   mocked add/multiply: the reference's closed form (3+3)*3 == 18.
+ *   conv2d (all five fused epilogue families), per-channel add (+relu),
+ *   max-pool+add+relu, global average pool, flatten, dense+add: additionally
+ *     the reference's OWN generated kernels (resource/resnet152/resnet152.cu,
+ *     compiled for gfx950 into oracle/_ref by `make ref`) run on the GPU on
+ *     random operands; the oracle reproduces 24 of its 25 convolution kernels
+ *     and all of the others named here (tests/test_gpu_reference_kernels.py,
+ *     which also says why one convolution kernel and softmax are no witnesses).
+ *   mocked add/multiply: the reference's closed form (3+3)*3 == 18, also on the
+ *     reference's own mocked kernels.
  *   The reference's ResNet-18 ten-float golden vector needs a weight blob that
  *   is absent from the reference checkout: end-to-end parity with the TVM
  *   model is "parity unpinned".
