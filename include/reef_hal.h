@@ -19,7 +19,10 @@
  * driver).  This layer provides the same contract without patches:
  *   - a stream created with launch_window = w keeps at most w kernels on the
  *     device; further launches wait in a host-side queue of the stream and
- *     move to the device as earlier kernels complete (reef_hal_stream_pump);
+ *     move to the device as earlier kernels complete.  In the HIP backend a
+ *     feeder thread per windowed stream does that (REEF_HAL_FEEDER=0 in the
+ *     environment: the caller's thread does it inside reef_hal_launch /
+ *     reef_hal_stream_query / reef_hal_stream_pump instead);
  *   - reef_hal_stream_clear_queue drops the host-side queue and reports how
  *     many launches it dropped, which is what the scheduler's rollback formula
  *     consumes (src/reef/server/scheduler.cpp:313-329);

@@ -29,6 +29,10 @@ def lib():
         if not os.path.exists(LIB_PATH):
             raise RuntimeError("libreef_amd.so is not built: run __graft_entry__.build() "
                                "(make -C reef_amd/csrc)")
+        # One real-time stream and several best-effort streams have to run side by side; with
+        # the runtime's default of 4 hardware queues per process they share queues.  The runtime
+        # reads this when it is loaded, so it has to be in the environment before the CDLL call.
+        os.environ.setdefault("GPU_MAX_HW_QUEUES", "8")
         _lib = ctypes.CDLL(LIB_PATH)
         _lib.reef_hal_last_error.restype = ctypes.c_char_p
     return _lib

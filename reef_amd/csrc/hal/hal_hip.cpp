@@ -1,10 +1,16 @@
 // HIP backend of the C-ABI layer (stock ROCm, no patched runtime).
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+#include <chrono>
+#include <condition_variable>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <mutex>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "hal/code_object.h"
@@ -59,12 +65,32 @@ struct HeldRing {
 // A stream with an optional launch window.  `done` is a pinned host word the
 // device writes after every kernel of a windowed stream; submitted - *done is
 // the number of kernels still on the device.
+//
+// A windowed stream has a feeder thread of its own that moves held launches to the
+// device as the window frees up.  The caller of reef_hal_launch (the scheduler
+// thread) then only copies the launch into the ring; the two runtime calls per
+// kernel (launch + completion write, 5-6 us together) are paid by the feeder, one
+// per stream, so several best-effort streams are fed in parallel instead of one
+// after the other from the scheduler's loop.  `mtx` guards the ring and `submitted`
+// and is only held for copies; `submit_mtx` is held around the runtime calls on the
+// HIP stream.  A launch counts as in flight from the moment the feeder takes it out
+// of the ring, so "ring dropped + at most `window` kernels not known complete" -- what
+// the rollback after a preemption relies on -- holds at every instant.
 struct reef_stream_s {
     hipStream_t s;
     int window;
     uint32_t submitted;
     volatile uint32_t* done;
     HeldRing held;
+    std::mutex mtx;
+    std::mutex submit_mtx;
+    std::condition_variable cv;
+    std::thread feeder;
+    std::atomic<bool> stop{false};
+    std::atomic<int> feeder_error{0};
+    std::atomic<size_t> held_count{0};   // mirror of held.size(), readable without mtx
+    std::atomic<uint32_t> enqueued{0};   // highest seq whose runtime calls have returned
+    bool has_feeder = false;
 };
 
 struct reef_graph_s {
@@ -206,6 +232,66 @@ int h_d2h_async(void* d, reef_devptr_t s, size_t n, reef_stream_t st) {
     return 0;
 }
 
+int submit(reef_stream_t st, hipFunction_t fn, const uint32_t* g, const uint32_t* b, uint32_t lds,
+           const void* kernarg, size_t bytes, uint32_t seq);
+inline uint32_t in_flight(reef_stream_t st) { return st->submitted - *st->done; }
+
+// Moves held launches to the device while the window has room.  Caller holds st->mtx.
+int pump_locked(reef_stream_t st) {
+    while (!st->held.empty() && (int)in_flight(st) < st->window) {
+        Held& h = st->held.front();
+        int rc = submit(st, h.fn, h.grid, h.block, h.lds, h.kernarg, h.bytes, ++st->submitted);
+        st->held.pop_front();
+        st->held_count.store(st->held.size(), std::memory_order_release);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+// The feeder looks at the ring size and the window through lock-free mirrors and only
+// takes the locks when there is a launch to move: a thread that re-takes a mutex in a
+// tight loop starves whoever else wants it (here the scheduler thread in the middle of
+// a preemption) for milliseconds.
+void feeder_main(reef_stream_s* st) {
+    hipSetDevice(g_device);
+    int idle_spins = 0;
+    Held h;
+    while (!st->stop.load(std::memory_order_acquire)) {
+        if (st->held_count.load(std::memory_order_acquire) == 0) {
+            // nothing to feed: after a while sleep until a launch is held (bounded, so that a
+            // missed wake-up costs little)
+            if (++idle_spins > 2000) {
+                std::unique_lock<std::mutex> lock(st->mtx);
+                if (st->held.empty()) st->cv.wait_for(lock, std::chrono::microseconds(200));
+                idle_spins = 0;
+            } else {
+                __builtin_ia32_pause();
+            }
+            continue;
+        }
+        idle_spins = 0;
+        // `submitted` only changes in this thread while a feeder exists
+        if ((int)in_flight(st) >= st->window) {
+            __builtin_ia32_pause();
+            continue;
+        }
+        std::lock_guard<std::mutex> sub(st->submit_mtx);
+        uint32_t seq = 0;
+        {
+            std::lock_guard<std::mutex> lock(st->mtx);
+            if (st->held.empty()) continue;   // dropped in the meantime
+            h = st->held.front();
+            st->held.pop_front();
+            st->held_count.store(st->held.size(), std::memory_order_release);
+            seq = ++st->submitted;   // in flight from now on
+        }
+        if (submit(st, h.fn, h.grid, h.block, h.lds, h.kernarg, h.bytes, seq) != 0)
+            st->feeder_error.store(1);
+    }
+}
+
+bool g_use_feeder = true;
+
 int h_stream_create(int window, reef_stream_t* out) {
     reef_stream_s* st = new reef_stream_s;
     st->window = window;
@@ -219,12 +305,22 @@ int h_stream_create(int window, reef_stream_t* out) {
         if (e != hipSuccess) { hipStreamDestroy(st->s); delete st; return fail(e, "hipHostMalloc"); }
         st->done = (volatile uint32_t*)p;
         *st->done = 0;
+        if (const char* v = std::getenv("REEF_HAL_FEEDER")) g_use_feeder = std::atoi(v) != 0;
+        if (g_use_feeder) {
+            st->has_feeder = true;
+            st->feeder = std::thread(feeder_main, st);
+        }
     }
     *out = st;
     return 0;
 }
 int h_stream_destroy(reef_stream_t st) {
     if (!st) return 0;
+    if (st->has_feeder) {
+        st->stop.store(true, std::memory_order_release);
+        st->cv.notify_all();
+        st->feeder.join();
+    }
     hipStreamSynchronize(st->s);
     hipStreamDestroy(st->s);
     if (st->done) hipHostFree((void*)st->done);
@@ -232,68 +328,89 @@ int h_stream_destroy(reef_stream_t st) {
     return 0;
 }
 
+// `seq` != 0: the launch belongs to a windowed stream and is its seq-th; the device writes
+// seq to the stream's completion word when the kernel has finished.
 int submit(reef_stream_t st, hipFunction_t fn, const uint32_t* g, const uint32_t* b, uint32_t lds,
-           const void* kernarg, size_t bytes) {
+           const void* kernarg, size_t bytes, uint32_t seq) {
     size_t sz = bytes;
     void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(kernarg),
                      HIP_LAUNCH_PARAM_BUFFER_SIZE, &sz, HIP_LAUNCH_PARAM_END};
     HIPCHK(hipModuleLaunchKernel(fn, g[0], g[1], g[2], b[0], b[1], b[2], lds, st ? st->s : nullptr,
                                  nullptr, extra));
-    if (st && st->window > 0) {
-        ++st->submitted;
-        HIPCHK(hipStreamWriteValue32(st->s, (void*)st->done, st->submitted, 0));
+    if (seq != 0) {
+        HIPCHK(hipStreamWriteValue32(st->s, (void*)st->done, seq, 0));
+        st->enqueued.store(seq, std::memory_order_release);
     }
     return 0;
 }
 
-inline uint32_t in_flight(reef_stream_t st) { return st->submitted - *st->done; }
-
 int h_stream_pump(reef_stream_t st) {
     if (!st || st->window <= 0) return 0;
-    while (!st->held.empty() && (int)in_flight(st) < st->window) {
-        Held& h = st->held.front();
-        int rc = submit(st, h.fn, h.grid, h.block, h.lds, h.kernarg, h.bytes);
-        st->held.pop_front();
-        if (rc) return rc;
-    }
-    return 0;
+    if (st->has_feeder) return st->feeder_error.load() ? 1 : 0;   // the feeder does it
+    std::lock_guard<std::mutex> lock(st->mtx);
+    return pump_locked(st);
 }
 
 int h_launch(reef_function_t f, const uint32_t* g, const uint32_t* b, uint32_t lds, reef_stream_t st,
              const void* kernarg, size_t bytes) {
     if (st && st->window > 0) {
-        if (int rc = h_stream_pump(st)) return rc;
-        if (!st->held.empty() || (int)in_flight(st) >= st->window) {
-            if (bytes > kMaxHeldKernarg) {
-                reef_hal_set_error("reef_hal_launch: argument block too large for a windowed stream");
-                return 1;
-            }
-            Held& h = st->held.push_back();
-            h.fn = f->fn;
-            std::memcpy(h.grid, g, sizeof(h.grid));
-            std::memcpy(h.block, b, sizeof(h.block));
-            h.lds = lds;
-            h.bytes = (uint32_t)bytes;
-            std::memcpy(h.kernarg, kernarg, bytes);
-            return 0;
+        if (bytes > kMaxHeldKernarg) {
+            reef_hal_set_error("reef_hal_launch: argument block too large for a windowed stream");
+            return 1;
         }
+        std::unique_lock<std::mutex> lock(st->mtx);
+        if (!st->has_feeder) {
+            if (int rc = pump_locked(st)) return rc;
+            if (st->held.empty() && (int)in_flight(st) < st->window)
+                return submit(st, f->fn, g, b, lds, kernarg, bytes, ++st->submitted);
+        }
+        const bool was_empty = st->held.empty();
+        Held& h = st->held.push_back();
+        h.fn = f->fn;
+        std::memcpy(h.grid, g, sizeof(h.grid));
+        std::memcpy(h.block, b, sizeof(h.block));
+        h.lds = lds;
+        h.bytes = (uint32_t)bytes;
+        std::memcpy(h.kernarg, kernarg, bytes);
+        st->held_count.store(st->held.size(), std::memory_order_release);
+        lock.unlock();
+        if (st->has_feeder && was_empty) st->cv.notify_one();
+        return st->feeder_error.load() ? 1 : 0;
     }
-    return submit(st, f->fn, g, b, lds, kernarg, bytes);
+    return submit(st, f->fn, g, b, lds, kernarg, bytes, 0);
 }
 
+// Waits until the ring of a windowed stream is empty (everything handed to the device).
+int drain_ring(reef_stream_t st) {
+    for (;;) {
+        {
+            std::lock_guard<std::mutex> lock(st->mtx);
+            if (!st->has_feeder) {
+                if (int rc = pump_locked(st)) return rc;
+            }
+            if (st->held.empty()) return st->feeder_error.load() ? 1 : 0;
+        }
+        __builtin_ia32_pause();
+    }
+}
 int h_stream_sync(reef_stream_t st) {
     if (st && st->window > 0) {
-        while (!st->held.empty()) {
-            if (int rc = h_stream_pump(st)) return rc;
-        }
+        if (int rc = drain_ring(st)) return rc;
+        std::lock_guard<std::mutex> sub(st->submit_mtx);   // a launch the feeder has in hand is enqueued
     }
     HIPCHK(hipStreamSynchronize(st ? st->s : nullptr));
     return 0;
 }
 int h_stream_query(reef_stream_t st, int* idle) {
     if (st && st->window > 0) {
-        if (int rc = h_stream_pump(st)) return rc;
+        std::lock_guard<std::mutex> lock(st->mtx);
+        if (!st->has_feeder) {
+            if (int rc = pump_locked(st)) return rc;
+        }
         if (!st->held.empty()) { *idle = 0; return 0; }
+        // everything is on the device: the completion word says whether it is done
+        *idle = in_flight(st) == 0 ? 1 : 0;
+        return st->feeder_error.load() ? 1 : 0;
     }
     hipError_t e = hipStreamQuery(st ? st->s : nullptr);
     if (e == hipSuccess) *idle = 1;
@@ -320,12 +437,18 @@ int h_host_write32(reef_devptr_t p, int32_t v) {
 }
 int h_stream_wait_device(reef_stream_t st) {
     if (st && st->window > 0) {
+        // What the device has been given by now.  A launch the feeder has taken out of the ring
+        // but whose runtime call has not returned yet is not waited for (the runtime blocks a
+        // launching thread for milliseconds now and then): it reaches the device later, reads the
+        // raised flag and leaves at once.
+        const uint32_t target = st->has_feeder ? st->enqueued.load(std::memory_order_acquire)
+                                               : st->submitted;
         // bounded spin on the pinned completion word, then let the runtime sleep
-        for (long spins = 0; in_flight(st) != 0; ++spins) {
+        for (long spins = 0; (int32_t)(*st->done - target) < 0; ++spins) {
             if (spins > 20000000L) break;
             __builtin_ia32_pause();
         }
-        if (in_flight(st) == 0) return 0;
+        if ((int32_t)(*st->done - target) >= 0) return 0;
     }
     HIPCHK(hipStreamSynchronize(st ? st->s : nullptr));
     return 0;
@@ -368,7 +491,13 @@ int h_graph_destroy(reef_graph_t g) {
 }
 int h_clear_queue(reef_stream_t st, uint64_t* n) {
     uint64_t d = 0;
-    if (st) { d = st->held.size(); st->held.clear(); }
+    if (st) {
+        // a launch the feeder has already taken out of the ring counts as in flight, not as dropped
+        std::lock_guard<std::mutex> lock(st->mtx);
+        d = st->held.size();
+        st->held.clear();
+        st->held_count.store(0, std::memory_order_release);
+    }
     if (n) *n = d;
     return 0;
 }
@@ -376,9 +505,11 @@ int h_reset_cus() { return 0; }
 
 int h_memset_async(reef_devptr_t p, int byte, size_t n, reef_stream_t st) {
     // a windowed stream may hold launches on the host: the fill must not overtake them
-    if (st && st->window > 0 && !st->held.empty()) {
-        reef_hal_set_error("reef_hal_memset_async: stream holds launches on the host");
-        return 1;
+    if (st && st->window > 0) {
+        if (int rc = drain_ring(st)) return rc;
+        std::lock_guard<std::mutex> sub(st->submit_mtx);   // behind a launch the feeder has in hand
+        HIPCHK(hipMemsetAsync(p, byte, n, st->s));
+        return 0;
     }
     HIPCHK(hipMemsetAsync(p, byte, n, st ? st->s : nullptr));
     return 0;

@@ -1,6 +1,7 @@
 #include "server/scheduler.h"
 
 #include <algorithm>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 
