@@ -650,8 +650,17 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
                     const int m = m0 + wm0 + tm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
                     if (m < M && n < N) {
                         const size_t idx = (size_t)m * N + n;
-                        float v = load_agent(ws + idx);
-                        for (int s = 1; s < split_k; ++s) v += load_agent(ws + (size_t)s * MN + idx);
+                        // loads of eight partials in flight together, sums in ascending s
+                        float v = 0.0f;
+                        for (int s0 = 0; s0 < split_k; s0 += 8) {
+                            float p[8];
+#pragma unroll
+                            for (int j = 0; j < 8; ++j)
+                                p[j] = load_agent(ws + (size_t)min(s0 + j, split_k - 1) * MN + idx);
+#pragma unroll
+                            for (int j = 0; j < 8; ++j)
+                                if (s0 + j < split_k) v = (s0 + j == 0) ? p[j] : v + p[j];
+                        }
                         ep.store(dst, v, m, idx);
                     }
                 }

@@ -59,7 +59,7 @@ def test_conv_tiles(tmp_path, tile, case):
 
 
 @pytest.mark.parametrize("split", [2, 3, 8])
-@pytest.mark.parametrize("tile", ["64x64", "128x64", "128x32"])
+@pytest.mark.parametrize("tile", ["64x64", "128x64", "128x32", "32x32k4", "64x32k2", "32x64k2"])
 def test_conv_split_k_and_epilogues(tmp_path, tile, split):
     cin, H, W, cout = 96, 14, 14, 160
     g = MB.GraphBuilder("s")
