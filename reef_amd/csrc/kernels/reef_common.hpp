@@ -45,6 +45,32 @@ __device__ __forceinline__ float load_agent(const float* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// ---- buffer addressing ------------------------------------------------------------
+// Tile loads and output stores go through buffer instructions: the tensor is described by a
+// resource (base, size in bytes) held in scalar registers, the lane supplies a 32-bit byte
+// offset, and the hardware checks the offset against the size -- a load outside the tensor
+// returns 0 and a store outside it is dropped.  Everything a tile loader or an epilogue would
+// otherwise do per element with compares, selects and exec masks (row >= M, k >= k_end,
+// padding taps, the ragged last tile) becomes: pick kOutside as the offset.  Tensors are
+// smaller than 1 GiB, so kOutside is outside every one of them, and so is the sum of a valid
+// offset and kOutside or of two kOutside (offsets are built as row part + column part).
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+constexpr unsigned kOutside = 0x40000000u;
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ float buf_load(rsrc_t r, unsigned byte_off) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)byte_off, 0, 0));
+}
+__device__ __forceinline__ f32x4 buf_load4(rsrc_t r, unsigned byte_off) {
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0));
+}
+__device__ __forceinline__ void buf_store(rsrc_t r, unsigned byte_off, float v) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, (int)byte_off, 0, 0);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);

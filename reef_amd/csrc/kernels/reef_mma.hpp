@@ -64,78 +64,59 @@ typedef Tile<1, 1, 1, 1, 2, 4> Tile32x32k4;
 typedef Tile<2, 1, 1, 1, 2, 2> Tile64x32k2;
 typedef Tile<1, 2, 1, 1, 2, 2> Tile32x64k2;
 
-// All tile loads are branch-free: an element outside the tensor (row >= M,
-// k >= k_end, padding) is loaded from the tensor's first element instead and
-// replaced by zero afterwards, so every load of a K step issues back to back.
+// All tile loads are buffer loads: an element outside the tensor or outside this launch's K
+// range (row >= M, k >= k_end, a padding tap) is addressed at kOutside and comes back as 0, so
+// a K step's loads issue back to back with one compare-and-select per load and nothing to
+// patch up afterwards.
 
 // ---- A tile: rows of a K-contiguous matrix -------------------------------
 // VEC: rows are 16-byte aligned at every k that is a multiple of 4 (K % 4 == 0).
-// Addresses are a uniform base plus a 32-bit element offset per lane.
 template <class T, bool VEC>
 struct ALoader {
     static constexpr int TPR = T::BK / 4;          // threads (float4s) per tile row
     static constexpr int RPP = kThreads / TPR;     // rows per pass
     static constexpr int NV = T::BM / RPP;         // float4 per thread per tile
-    static_assert(NV >= 1 && NV <= 8, "validity bits of a tile fit one register");
-    // Raw loaded values plus one validity bit per element group.  The zeroing of
-    // invalid elements happens when the tile is written to LDS, not at the load: a
-    // select right behind the load would make the wavefront wait for the data at
-    // once and nothing would be in flight across K steps.
-    struct Regs { f32x4 v[NV]; unsigned ok; };
-    const float* a0;        // tensor base (also the stand-in address)
-    unsigned rowoff[NV];    // row * lda (0 when the row is outside M)
-    unsigned rowmask;       // bit i: row i of this thread is inside M
+    static_assert(NV >= 1, "tile shorter than one pass");
+    struct Regs { f32x4 v[NV]; };
+    rsrc_t rs;
+    unsigned rowoff[NV];    // byte offset of the row (kOutside when the row is outside M)
     int k;                  // k of this thread's float4 in the next tile
     int k_end;
 
-    __device__ __forceinline__ void init(const float* a, int lda, int m0, int M, int k_begin,
-                                         int k_end_) {
+    // `bytes`: size of the matrix from `a` on
+    __device__ __forceinline__ void init(const float* a, unsigned bytes, int lda, int m0, int M,
+                                         int k_begin, int k_end_) {
         const int tid = threadIdx.x;
-        a0 = a;
+        rs = make_rsrc(a, bytes);
         k_end = k_end_;
         k = k_begin + (tid % TPR) * 4;
-        rowmask = 0;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int row = m0 + tid / TPR + RPP * i;
-            const bool ok = row < M;
-            rowoff[i] = ok ? (unsigned)row * (unsigned)lda : 0u;
-            rowmask |= (ok ? 1u : 0u) << i;
+            rowoff[i] = row < M ? (unsigned)row * (unsigned)lda * 4u : kOutside;
         }
     }
     __device__ __forceinline__ void load(Regs& r) {
-        unsigned okbits = 0;
+        if (VEC) {
+            // k and k_end are multiples of 4 here: the float4 is inside or outside as a whole
+            const unsigned koff = k < k_end ? (unsigned)k * 4u : kOutside;
 #pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            const bool rok = (rowmask >> i) & 1;
-            if (VEC) {
-                const bool ok = rok && k < k_end;
-                const unsigned off = ok ? rowoff[i] + (unsigned)k : 0u;
-                r.v[i] = *(const f32x4*)(a0 + off);
-                okbits |= (ok ? 0xFu : 0u) << (4 * i);
-            } else {
+            for (int i = 0; i < NV; ++i) r.v[i] = buf_load4(rs, rowoff[i] + koff);
+        } else {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const bool ok = rok && k + e < k_end;
-                    const unsigned off = ok ? rowoff[i] + (unsigned)(k + e) : 0u;
-                    r.v[i][e] = a0[off];
-                    okbits |= (ok ? 1u : 0u) << (4 * i + e);
-                }
+            for (int e = 0; e < 4; ++e) {
+                const unsigned koff = k + e < k_end ? (unsigned)(k + e) * 4u : kOutside;
+#pragma unroll
+                for (int i = 0; i < NV; ++i) r.v[i][e] = buf_load(rs, rowoff[i] + koff);
             }
         }
-        r.ok = okbits;
         k += T::BK;
     }
     __device__ __forceinline__ void store(const Regs& r, float* As) const {
         const int tid = threadIdx.x;
 #pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            int row = tid / TPR + RPP * i;
-            f32x4 v;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = ((r.ok >> (4 * i + e)) & 1u) ? r.v[i][e] : 0.f;
-            *(f32x4*)(As + row * T::LDA + (tid % TPR) * 4) = v;
-        }
+        for (int i = 0; i < NV; ++i)
+            *(f32x4*)(As + (tid / TPR + RPP * i) * T::LDA + (tid % TPR) * 4) = r.v[i];
     }
 };
 
@@ -150,9 +131,8 @@ struct Im2colLoader {
     static constexpr int RS = kThreads / T::BN;  // k rows covered per pass
     static constexpr int NR = T::BK / RS;        // rows per thread per tile
     static constexpr bool UNIFORM = T::BN >= 64; // one k row per wavefront
-    static_assert(NR <= 32, "validity bits of a tile fit one register");
-    struct Regs { float v[NR]; unsigned ok; };   // raw values + validity bits (zeroed at store)
-    const float* in;
+    struct Regs { float v[NR]; };
+    rsrc_t rs;
     int HW, W, kh, kw;
     unsigned ymask, xmask;  // bit ky / kx: that tap is inside the image for this thread's pixel
     int soff;               // iy0 * W + ix0 of this thread's pixel (may be negative)
@@ -162,10 +142,10 @@ struct Im2colLoader {
     __device__ __forceinline__ void init(const float* in_, const int* a, int n0, int N, int k_begin,
                                          int k_end_) {
         const int tid = threadIdx.x;
-        in = in_;
         const int H = a[REEF_CONV_H];
         W = a[REEF_CONV_W];
         HW = H * W;
+        rs = make_rsrc(in_, (unsigned)a[REEF_CONV_CIN] * (unsigned)HW * 4u);
         kh = a[REEF_CONV_KH];
         kw = a[REEF_CONV_KW];
         const int Wo = a[REEF_CONV_WO];
@@ -194,13 +174,10 @@ struct Im2colLoader {
         dc = t / kh;
     }
     __device__ __forceinline__ void load(Regs& r) {
-        unsigned okbits = 0;
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
             const bool ok = (k < k_end) && (((ymask >> ky) & (xmask >> kx) & 1u) != 0);
-            const unsigned off = ok ? (unsigned)(c * HW + ky * W + kx + soff) : 0u;
-            r.v[i] = in[off];
-            okbits |= (ok ? 1u : 0u) << i;
+            r.v[i] = buf_load(rs, ok ? (unsigned)(c * HW + ky * W + kx + soff) * 4u : kOutside);
             // advance (c, ky, kx) by RS rows, mixed radix (kh, kw), without branches
             k += RS;
             kx += dkx;
@@ -211,13 +188,12 @@ struct Im2colLoader {
             ky -= kh & -cy;
             c += dc + cy;
         }
-        r.ok = okbits;
     }
     __device__ __forceinline__ void store(const Regs& r, float* Bs) const {
         const int tid = threadIdx.x;
         const int nl = tid & (T::BN - 1), kr0 = tid / T::BN;
 #pragma unroll
-        for (int i = 0; i < NR; ++i) Bs[(kr0 + RS * i) * T::BN + nl] = ((r.ok >> i) & 1u) ? r.v[i] : 0.0f;
+        for (int i = 0; i < NR; ++i) Bs[(kr0 + RS * i) * T::BN + nl] = r.v[i];
     }
 };
 
@@ -230,34 +206,31 @@ struct PointwiseLoader {
     static constexpr int NF = T::BK * C4 / kThreads;     // float4 per thread per tile
     static constexpr int RSTEP = kThreads / C4;          // rows between a thread's float4s
     static_assert(NF >= 1, "tile narrower than one pass");
-    struct Regs { f32x4 v[NF]; unsigned ok; };
-    const float* in;
-    unsigned off;   // element offset of this thread's first float4 in the next tile
-    unsigned step;  // RSTEP * N
-    unsigned tile;  // BK * N
+    struct Regs { f32x4 v[NF]; };
+    rsrc_t rs;
+    unsigned off;   // byte offset of this thread's first float4 in the next tile
+    unsigned step;  // RSTEP rows in bytes
+    unsigned tile;  // BK rows in bytes
     int k, k_end;
-    bool nvalid;
 
-    __device__ __forceinline__ void init(const float* in_, int n0, int N, int k_begin, int k_end_) {
+    // K = all rows of the matrix (the buffer ends there), k_end = this launch's last row + 1
+    __device__ __forceinline__ void init(const float* in_, int n0, int N, int K, int k_begin, int k_end_) {
         const int tid = threadIdx.x;
-        in = in_;
+        rs = make_rsrc(in_, (unsigned)K * (unsigned)N * 4u);
         const int row = tid / C4, col = (tid % C4) * 4;
-        nvalid = n0 + col < N;
         k = k_begin + row;
         k_end = k_end_;
-        off = (unsigned)k * (unsigned)N + (unsigned)(n0 + col);
-        step = (unsigned)RSTEP * (unsigned)N;
-        tile = (unsigned)T::BK * (unsigned)N;
+        // a column past N stays outside for every row
+        off = n0 + col < N ? ((unsigned)k * (unsigned)N + (unsigned)(n0 + col)) * 4u : kOutside;
+        step = (unsigned)RSTEP * (unsigned)N * 4u;
+        tile = (unsigned)T::BK * (unsigned)N * 4u;
     }
     __device__ __forceinline__ void load(Regs& r) {
-        unsigned okbits = 0;
 #pragma unroll
-        for (int i = 0; i < NF; ++i) {
-            const bool ok = nvalid && (k + RSTEP * i) < k_end;
-            r.v[i] = *(const f32x4*)(in + (ok ? off + step * i : 0u));
-            okbits |= (ok ? 1u : 0u) << i;
-        }
-        r.ok = okbits;
+        for (int i = 0; i < NF; ++i)
+            r.v[i] = buf_load4(rs, (k + RSTEP * i) < k_end ? off + step * i : kOutside);
+        // (an offset that started at kOutside stays outside: the rows of a tensor below 1 GiB do
+        // not carry it around the 32-bit range)
         off += tile;
         k += T::BK;
     }
@@ -265,10 +238,7 @@ struct PointwiseLoader {
         const int tid = threadIdx.x;
         const int row = tid / C4, col = (tid % C4) * 4;
 #pragma unroll
-        for (int i = 0; i < NF; ++i) {
-            const bool ok = (r.ok >> i) & 1u;
-            *(f32x4*)(Bs + (row + RSTEP * i) * T::BN + col) = ok ? r.v[i] : f32x4{0.f, 0.f, 0.f, 0.f};
-        }
+        for (int i = 0; i < NF; ++i) *(f32x4*)(Bs + (row + RSTEP * i) * T::BN + col) = r.v[i];
     }
 };
 
@@ -277,37 +247,33 @@ template <class T>
 struct BknLoader {
     static constexpr int RS = kThreads / T::BN;
     static constexpr int NR = T::BK / RS;
-    struct Regs { float v[NR]; unsigned ok; };
-    const float* b0;
-    int n;
-    bool nvalid;
-    int ldb, k, k_end;
-    __device__ __forceinline__ void init(const float* b, int ldb_, int n0, int N, int k_begin,
-                                         int k_end_) {
+    struct Regs { float v[NR]; };
+    rsrc_t rs;
+    unsigned noff;   // byte offset of this thread's column (kOutside when it is past N)
+    unsigned ldb4;   // row pitch in bytes
+    int k, k_end;
+    __device__ __forceinline__ void init(const float* b, unsigned bytes, int ldb, int n0, int N,
+                                         int k_begin, int k_end_) {
         const int tid = threadIdx.x;
-        n = n0 + (tid & (T::BN - 1));
-        nvalid = n < N;
-        b0 = b;
-        ldb = ldb_;
+        rs = make_rsrc(b, bytes);
+        const int n = n0 + (tid & (T::BN - 1));
+        noff = n < N ? (unsigned)n * 4u : kOutside;
+        ldb4 = (unsigned)ldb * 4u;
         k = k_begin + tid / T::BN;
         k_end = k_end_;
     }
     __device__ __forceinline__ void load(Regs& r) {
-        unsigned okbits = 0;
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
-            const bool ok = nvalid && k < k_end;
-            r.v[i] = b0[ok ? (unsigned)k * (unsigned)ldb + (unsigned)n : 0u];
-            okbits |= (ok ? 1u : 0u) << i;
+            r.v[i] = buf_load(rs, k < k_end ? (unsigned)k * ldb4 + noff : kOutside);
             k += RS;
         }
-        r.ok = okbits;
     }
     __device__ __forceinline__ void store(const Regs& r, float* Bs) const {
         const int tid = threadIdx.x;
         const int nl = tid & (T::BN - 1), kr0 = tid / T::BN;
 #pragma unroll
-        for (int i = 0; i < NR; ++i) Bs[(kr0 + RS * i) * T::BN + nl] = ((r.ok >> i) & 1u) ? r.v[i] : 0.0f;
+        for (int i = 0; i < NR; ++i) Bs[(kr0 + RS * i) * T::BN + nl] = r.v[i];
     }
 };
 
@@ -494,6 +460,55 @@ __device__ __forceinline__ int xcd_chunked(int task, int total) {
 //   CONV_UNALIGNED  im2col gather, element-wise weight loads    (any K; the 7x7x3 stem)
 enum { CONV_GENERAL = 0, CONV_POINTWISE = 1, CONV_UNALIGNED = 2 };
 
+// Epilogue operands of a convolution as buffers.  Optional operands follow the three fixed
+// pointers in flag order (bias, residual, scale + shift, second output + its shift).  A
+// per-channel vector is `channels` floats long and a full tensor `MN` floats, so an offset
+// computed for a row >= M falls outside by itself; only a column >= N has to be turned into
+// kOutside by the caller (it would land in the next row).
+struct ConvEpilogue {
+    rsrc_t out, out2, res, bias, scale, shift, shift2;
+    bool has_res, has_bias, has_affine, has_dual;
+    int act, act2;
+    unsigned doff4;   // byte offset of this layer's slice inside the output tensor(s)
+    __device__ __forceinline__ void init(const ReefOpDesc& d, int flags, int act_, int act2_, int M,
+                                         unsigned MN4, unsigned doff4_) {
+        int p = 3;
+        const unsigned M4 = (unsigned)M * 4u;
+        doff4 = doff4_;
+        out = make_rsrc(d.ptr[2], doff4 + MN4);
+        has_bias = flags & REEF_F_BIAS;
+        has_res = flags & REEF_F_RESIDUAL;
+        has_affine = flags & REEF_F_AFFINE;
+        has_dual = flags & REEF_F_DUAL;
+        bias = res = scale = shift = out2 = shift2 = out;
+        if (has_bias) bias = make_rsrc(d.ptr[p++], M4);
+        if (has_res) res = make_rsrc(d.ptr[p++], MN4);
+        if (has_affine) {
+            scale = make_rsrc(d.ptr[p], M4);
+            shift = make_rsrc(d.ptr[p + 1], M4);
+            p += 2;
+        }
+        if (has_dual) {
+            out2 = make_rsrc(d.ptr[p], doff4 + MN4);
+            shift2 = make_rsrc(d.ptr[p + 1], M4);
+            p += 2;
+        }
+        act = act_;
+        act2 = act2_;
+    }
+    // off = (m * N + n) * 4 or outside; m4 = m * 4.  v = acc; v += residual; v += bias;
+    // v = fma(v, scale, shift); act  -- then out2 = act2(out + shift2).
+    __device__ __forceinline__ void finish(float v, unsigned off, unsigned m4, float resv, float biasv,
+                                           float sh2v) const {
+        if (has_res) v = v + resv;
+        if (has_bias) v = v + biasv;
+        if (has_affine) v = fmaf(v, buf_load(scale, m4), buf_load(shift, m4));
+        const float o = act_apply(v, act);
+        buf_store(out, off + doff4, o);
+        if (has_dual) buf_store(out2, off + doff4, act_apply(o + sh2v, act2));
+    }
+};
+
 template <class T, int MODE, class Poll>
 __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, char* smem_raw,
                                             const Poll& poll) {
@@ -505,6 +520,9 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
   constexpr bool EARLY = T::KW > 1;
   constexpr int ER = EARLY ? T::RPW : 1;
   float e_bias[T::TM][ER], e_sh2[T::TM][ER], e_res[T::TM][T::TN][ER];
+  const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
+  const WaveGeom<T> wg;
+  const int r0 = wg.wk * T::RPW;   // first accumulator element this wavefront writes out
   {
     const ReefOpDesc& d = d_in;
     const int* a = d.attr;
@@ -528,28 +546,24 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
     if (EARLY) {
         // Epilogue operands of the few outputs this wavefront will write: issued now, used
         // after the K loop.
-        const int flags = a[REEF_CONV_FLAGS];
         if (split_k == 1) {
-            Epilogue ep;
-            ep.unpack(d, 3, flags, 0, 0);
-            const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
-            const WaveGeom<T> wg;
-            const int r0 = wg.wk * T::RPW;
+            ConvEpilogue ep;
+            ep.init(d, a[REEF_CONV_FLAGS], 0, 0, M, (unsigned)M * (unsigned)N * 4u, 0);
 #pragma unroll
-            for (int tm = 0; tm < T::TM; ++tm)
+            for (int tm = 0; tm < T::TM; ++tm) {
+                const unsigned mb = (unsigned)(m0 + wg.wm0 + tm * 32 + 4 * h + 8 * (r0 >> 2));
 #pragma unroll
                 for (int rr = 0; rr < T::RPW; ++rr) {
-                    const int r = r0 + rr;
-                    const int m = m0 + wg.wm0 + tm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                    const bool mok = m < M;
-                    e_bias[tm][rr] = (ep.bias && mok) ? ep.bias[m] : 0.0f;
-                    e_sh2[tm][rr] = (ep.shift2 && mok) ? ep.shift2[m] : 0.0f;
+                    const unsigned m = mb + 8 * (rr >> 2) + (rr & 3);
+                    e_bias[tm][rr] = ep.has_bias ? buf_load(ep.bias, m * 4u) : 0.0f;
+                    e_sh2[tm][rr] = ep.has_dual ? buf_load(ep.shift2, m * 4u) : 0.0f;
 #pragma unroll
                     for (int tn = 0; tn < T::TN; ++tn) {
-                        const int n = n0 + wg.wn0 + tn * 32 + l32;
-                        e_res[tm][tn][rr] = (ep.residual && mok && n < N) ? ep.residual[(size_t)m * N + n] : 0.0f;
+                        const unsigned n = (unsigned)(n0 + wg.wn0 + tn * 32 + l32);
+                        e_res[tm][tn][rr] = ep.has_res ? buf_load(ep.res, (m * (unsigned)N + n) * 4u) : 0.0f;
                     }
                 }
+            }
         }
         asm volatile("" ::: "memory");  // keeps the loads above the K loop
     }
@@ -558,20 +572,20 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
     if (MODE == CONV_POINTWISE) {
         ALoader<T, true> la;
         PointwiseLoader<T> lp;
-        la.init((const float*)d.ptr[1], K, m0, M, k_begin, k_end);
-        lp.init((const float*)d.ptr[0], n0, N, k_begin, k_end);
+        la.init((const float*)d.ptr[1], (unsigned)M * (unsigned)K * 4u, K, m0, M, k_begin, k_end);
+        lp.init((const float*)d.ptr[0], n0, N, K, k_begin, k_end);
         ok = k_loop<T, false>(la, lp, nk, smem, acc, poll);
     } else {
         Im2colLoader<T> lb;
         lb.init((const float*)d.ptr[0], a, n0, N, k_begin, k_end);
         ALoader<T, MODE == CONV_GENERAL> la;
-        la.init((const float*)d.ptr[1], K, m0, M, k_begin, k_end);
+        la.init((const float*)d.ptr[1], (unsigned)M * (unsigned)K * 4u, K, m0, M, k_begin, k_end);
         ok = k_loop<T, false>(la, lb, nk, smem, acc, poll);
     }
     if (!ok) return false;
   }
     float res[T::TM][T::TN][T::RPW];
-    const int r0 = finish_tile<T>(acc, res, smem);
+    finish_tile<T>(acc, res, smem);
 
     // Everything the epilogue needs is re-read from the argument block here, so the
     // K loop does not carry the epilogue's pointers in scalar registers.
@@ -579,40 +593,59 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
     asm volatile("" : "+s"(dp));
     const ReefOpDesc& d = *dp;
     const int* a = d.attr;
-    const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
-    const WaveGeom<T> wg;
-    const int wm0 = wg.wm0, wn0 = wg.wn0;
     const int flags = a[REEF_CONV_FLAGS];
-    const size_t MN = (size_t)M * N;
-    // plain split-K writes partial tiles to the workspace; the offset belongs to the
-    // launch that writes the real output
-    const bool to_ws = split_k > 1 && !(flags & REEF_F_FUSED_REDUCE);
-    float* dst = (float*)d.ptr[2] + (to_ws ? 0 : a[REEF_CONV_DST_OFF]);
+    const unsigned MN4 = (unsigned)M * (unsigned)N * 4u;
+    const unsigned row4 = (unsigned)N * 4u;
+    const bool fused = split_k > 1 && (flags & REEF_F_FUSED_REDUCE);
 
-    if (to_ws) {
-        // plain split-K: partial tile to the workspace, reef_splitk_reduce folds
-        float* ws = dst + (size_t)split * MN;
+    if (!fused) {
+        // One pass over this wavefront's outputs.  Offsets are 32-bit byte offsets built from a
+        // per-lane base plus compile-time row steps; a column past N makes the base kOutside, a
+        // row past M runs off the end of the buffer: no compares per element.
+        const bool to_ws = split_k > 1;   // plain split-K: partial tile to the workspace
+        ConvEpilogue ep;
+        rsrc_t ws;
+        if (to_ws) ws = make_rsrc((const float*)d.ptr[2] + (size_t)split * M * N, MN4);
+        else ep.init(d, flags, a[REEF_CONV_ACT], a[REEF_CONV_ACT2], M, MN4, (unsigned)a[REEF_CONV_DST_OFF] * 4u);
 #pragma unroll
-        for (int tm = 0; tm < T::TM; ++tm)
+        for (int tm = 0; tm < T::TM; ++tm) {
+            const unsigned mb = (unsigned)(m0 + wg.wm0 + tm * 32 + 4 * h + 8 * (r0 >> 2));
 #pragma unroll
             for (int tn = 0; tn < T::TN; ++tn) {
-                const int n = n0 + wn0 + tn * 32 + l32;
+                const unsigned n = (unsigned)(n0 + wg.wn0 + tn * 32 + l32);
+                const unsigned base = n < (unsigned)N ? (mb * (unsigned)N + n) * 4u : kOutside;
 #pragma unroll
                 for (int rr = 0; rr < T::RPW; ++rr) {
-                    const int r = r0 + rr;
-                    const int m = m0 + wm0 + tm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                    if (m < M && n < N) ws[(size_t)m * N + n] = res[tm][tn][rr];
+                    const unsigned c = 8 * (rr >> 2) + (rr & 3);
+                    const unsigned off = base + c * row4;
+                    const float v = res[tm][tn][rr];
+                    if (to_ws) {
+                        buf_store(ws, off, v);
+                    } else {
+                        const unsigned m4 = (mb + c) * 4u;
+                        if (EARLY) {
+                            ep.finish(v, off, m4, e_res[tm][tn][rr], e_bias[tm][rr], e_sh2[tm][rr]);
+                        } else {
+                            ep.finish(v, off, m4, ep.has_res ? buf_load(ep.res, off) : 0.0f,
+                                      ep.has_bias ? buf_load(ep.bias, m4) : 0.0f,
+                                      ep.has_dual ? buf_load(ep.shift2, m4) : 0.0f);
+                        }
+                    }
                 }
             }
+        }
         return true;
     }
 
+    // fused split-K: store the partial, count in, the last arrival folds all partials in
+    // ascending split order (fixed order => same bits whoever is last)
+    const int wm0 = wg.wm0, wn0 = wg.wn0;
+    const size_t MN = (size_t)M * N;
+    float* dst = (float*)d.ptr[2] + a[REEF_CONV_DST_OFF];
     Epilogue ep;
     ep.unpack(d, 3, flags, a[REEF_CONV_ACT], a[REEF_CONV_ACT2]);
     if (ep.out2) ep.out2 += a[REEF_CONV_DST_OFF];
-    if (split_k > 1) {
-        // fused split-K: store the partial, count in, the last arrival folds all
-        // partials in ascending split order (fixed order => same bits whoever is last)
+    {
         float* ws = (float*)d.ptr[ep.next];
         int* counters = (int*)d.ptr[ep.next + 1] + a[REEF_CONV_SYNC_OFF];
         int* s_last = (int*)(smem + 2 * (T::A_FLOATS + T::B_FLOATS)) + 1;
@@ -669,26 +702,6 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
             __hip_atomic_store(&counters[rem], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         return true;
     }
-
-#pragma unroll
-    for (int tm = 0; tm < T::TM; ++tm)
-#pragma unroll
-        for (int tn = 0; tn < T::TN; ++tn) {
-            const int n = n0 + wn0 + tn * 32 + l32;
-#pragma unroll
-            for (int rr = 0; rr < T::RPW; ++rr) {
-                const int r = r0 + rr;
-                const int m = m0 + wm0 + tm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                if (m < M && n < N) {
-                    if (EARLY)
-                        ep.store_pre(dst, res[tm][tn][rr], m, (size_t)m * N + n, e_res[tm][tn][rr],
-                                     e_bias[tm][rr], e_sh2[tm][rr]);
-                    else
-                        ep.store(dst, res[tm][tn][rr], m, (size_t)m * N + n);
-                }
-            }
-        }
-    return true;
 }
 
 // ---- reef_gemm ----------------------------------------------------------------
@@ -716,16 +729,16 @@ __device__ __forceinline__ bool gemm_body(const ReefOpDesc& d, int task, char* s
 
     bool ok;
     ALoader<T, true> la;
-    la.init(A, lda, m0, M, 0, K);
+    la.init(A, ((unsigned)(M - 1) * (unsigned)lda + (unsigned)K) * 4u, lda, m0, M, 0, K);
     if (TRANS_B) {
         // B is [N][K]: stage it exactly like A (rows = n).
         typedef Tile<T::WGN, T::WGM, T::TN, T::TM, T::DEPTH, T::KW> TB;  // BM of TB == BN of T
         ALoader<TB, true> lb;
-        lb.init(B, ldb, n0, N, 0, K);
+        lb.init(B, ((unsigned)(N - 1) * (unsigned)ldb + (unsigned)K) * 4u, ldb, n0, N, 0, K);
         ok = k_loop<T, true>(la, lb, nk, smem, acc, poll);
     } else {
         BknLoader<T> lb;
-        lb.init(B, ldb, n0, N, 0, K);
+        lb.init(B, ((unsigned)(K - 1) * (unsigned)ldb + (unsigned)N) * 4u, ldb, n0, N, 0, K);
         ok = k_loop<T, false>(la, lb, nk, smem, acc, poll);
     }
     if (!ok) return false;
