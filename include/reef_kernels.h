@@ -172,10 +172,15 @@ enum {
 /* Loader families of the convolution; the entry symbol carries the family:
  *   reef_conv2d_<tile>      general: im2col gather, needs K % 4 == 0
  *   reef_conv2d_pw_<tile>   pointwise: 1x1, stride 1, no padding, N % 4 == 0, K % 4 == 0
- *   reef_conv2d_u_<tile>    unaligned: im2col gather, any K */
+ *   reef_conv2d_u_<tile>    unaligned: im2col gather, any K
+ *   reef_conv2d_d<R>_16x16k4  direct: R = kh*kw taps compiled in (1, 9); operands go from memory
+ *                           straight into 16x16x4 MFMAs, the four wavefronts split the input
+ *                           channels.  d1 needs Cin % 8 == 0 (any stride); K_CHUNK is a multiple
+ *                           of R (d9) or 8 (d1) and splits K on channel boundaries. */
 #define REEF_CONV_MODE_GENERAL 0
 #define REEF_CONV_MODE_POINTWISE 1
 #define REEF_CONV_MODE_UNALIGNED 2
+#define REEF_CONV_MODE_DIRECT 3
 
 /* Tile configurations: BM x BN output tile per workgroup.  Plain tiles walk K in steps of
  * 32; a "k<n>" tile splits every step of 32*n k values across n wavefronts and sums the n
@@ -190,6 +195,7 @@ enum {
     REEF_TILE_32x32k4 = 6,
     REEF_TILE_64x32k2 = 7,
     REEF_TILE_32x64k2 = 8,
+    REEF_TILE_16x16k4 = 9,   /* direct family only */
     REEF_TILE_COUNT
 };
 

@@ -35,6 +35,14 @@ struct OpConv {
         return conv2d_body<T, MODE>(d, task, smem, p);
     }
 };
+template <int R>
+struct OpConvDirect {
+    static constexpr int LDS = TileD16::LDS_BYTES;
+    template <class P>
+    static __device__ __forceinline__ bool run(const ReefOpDesc& d, int task, char* smem, const P& p) {
+        return conv2d_direct_body<R>(d, task, smem, p);
+    }
+};
 template <class T, bool TRANS_B>
 struct OpGemm {
     static constexpr int LDS = T::LDS_BYTES;
@@ -186,6 +194,8 @@ REEF_ENTRY(reef_conv2d_u_64x128, OpConv<Tile64x128 REEF_COMMA CONV_UNALIGNED>)
 REEF_ENTRY(reef_conv2d_u_32x32k4, OpConv<Tile32x32k4 REEF_COMMA CONV_UNALIGNED>)
 REEF_ENTRY(reef_conv2d_u_64x32k2, OpConv<Tile64x32k2 REEF_COMMA CONV_UNALIGNED>)
 REEF_ENTRY(reef_conv2d_u_32x64k2, OpConv<Tile32x64k2 REEF_COMMA CONV_UNALIGNED>)
+REEF_ENTRY(reef_conv2d_d1_16x16k4, OpConvDirect<1>)
+REEF_ENTRY(reef_conv2d_d9_16x16k4, OpConvDirect<9>)
 REEF_ENTRY(reef_gemm_nt_128x128, OpGemm<Tile128x128 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nt_64x64, OpGemm<Tile64x64 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nt_32x128, OpGemm<Tile32x128 REEF_COMMA true>)

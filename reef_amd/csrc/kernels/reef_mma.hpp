@@ -704,6 +704,197 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
     }
 }
 
+// ---- reef_conv2d_d<R>: operands straight from memory into the matrix cores ----------------
+// A batch-1 layer is latency bound: every weight is used once per inference, so each K step of
+// the tiled kernels above waits a full memory round trip (global -> registers -> LDS -> barrier).
+// This family removes the staging.  A workgroup owns a 16 x 16 output tile and its four
+// wavefronts split the input channels; v_mfma_f32_16x16x4f32 takes one A value (row = lane % 16,
+// k = lane / 16) and one B value (column = lane % 16, k = lane / 16) per lane, which a lane can
+// load directly:
+//   R > 1 (R = kh * kw taps): k slot kq = lane / 16 is input channel c + kq; the lane loads the
+//          R contiguous weights W[m][c + kq][0..R) and the R taps in[c + kq][iy(t)][ix(t)] of
+//          its output pixel; MFMA t multiplies tap t of four channels.  Tap offsets and their
+//          padding validity are fixed per lane for the whole kernel.
+//   R = 1: k slot kq covers eight channels c + 8 kq .. + 8: two 128-bit weight loads and eight
+//          pixel loads; MFMA j multiplies channel j of each slot.  Any stride.
+// No LDS and no barrier inside the K loop, so NS steps of loads are in flight per wavefront
+// (a wavefront may have 63 vector-memory instructions outstanding; NS steps are 60 of them).  The four
+// partial tiles are summed through LDS in wavefront order and thread t writes output element
+// (t / 16, t % 16), so stores are 64-byte runs along a row.  The sum order over k differs from
+// the tiled kernels (it is fixed, so results are reproducible run to run).
+struct TileD16 {
+    static constexpr int BM = 16, BN = 16;
+    static constexpr int LDS_BYTES = 4 * 256 * 4 + 16;
+};
+
+template <int R>
+struct DirectGeom {
+    static constexpr int CPL = R == 1 ? 8 : 1;   // channels per k slot and step
+    static constexpr int RC = R * CPL;           // A values (= B values = MFMAs) per lane and step
+    static constexpr int STEP_C = 16 * CPL;      // channels a workgroup consumes per step
+    static constexpr int LOADS = (RC / 4) + (RC % 4) + RC;  // vector-memory instructions per step
+    static constexpr int NS = 60 / LOADS;         // steps of loads in flight per wavefront
+};
+
+template <int R, class Poll>
+__device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int task, char* smem_raw,
+                                                   const Poll& poll) {
+    typedef DirectGeom<R> G;
+    constexpr int RC = G::RC, NS = G::NS;
+    float* smem = (float*)smem_raw;
+    int* sflag = (int*)(smem + 4 * 256);
+    const ReefOpDesc& d = d_in;
+    const int* a = d.attr;
+    const int lane = threadIdx.x & 63, i16 = lane & 15, kq = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int M = a[REEF_CONV_COUT], C = a[REEF_CONV_CIN];
+    const int H = a[REEF_CONV_H], W = a[REEF_CONV_W], Wo = a[REEF_CONV_WO];
+    const int N = a[REEF_CONV_HO] * Wo;
+    const int K = C * R;
+    const int split_k = a[REEF_CONV_SPLIT_K];
+    const int n_tiles = a[REEF_CONV_N_TILES];
+    const int tiles = a[REEF_CONV_M_TILES] * n_tiles;
+    task = xcd_chunked(task, tiles * split_k);
+    const int split = task / tiles;
+    const int rem = task - split * tiles;
+    const int mt = rem / n_tiles, nt = rem - mt * n_tiles;
+    const int m0 = mt * 16, n0 = nt * 16;
+    const int c_chunk = a[REEF_CONV_K_CHUNK] / R;
+    const int cb = split * c_chunk;
+    const int ce = min(C, cb + c_chunk);
+    const int nsteps = (ce - cb + G::STEP_C - 1) / G::STEP_C;
+    const unsigned HW4 = (unsigned)(H * W) * 4u;
+    const unsigned MN4 = (unsigned)M * (unsigned)N * 4u;
+    const int flags = a[REEF_CONV_FLAGS];
+
+    // epilogue operands of the one output element this thread writes, fetched ahead of the K loop
+    const int orow = threadIdx.x >> 4, ocol = threadIdx.x & 15;
+    const unsigned om = (unsigned)(m0 + orow), on = (unsigned)(n0 + ocol);
+    const unsigned ooff = on < (unsigned)N ? (om * (unsigned)N + on) * 4u : kOutside;
+    const bool to_ws = split_k > 1;
+    ConvEpilogue ep;
+    float e_bias = 0.0f, e_res = 0.0f, e_sh2 = 0.0f;
+    if (!to_ws) {
+        ep.init(d, flags, a[REEF_CONV_ACT], a[REEF_CONV_ACT2], M, MN4, (unsigned)a[REEF_CONV_DST_OFF] * 4u);
+        if (ep.has_bias) e_bias = buf_load(ep.bias, om * 4u);
+        if (ep.has_res) e_res = buf_load(ep.res, ooff);
+        if (ep.has_dual) e_sh2 = buf_load(ep.shift2, om * 4u);
+    }
+
+    // per-lane operand offsets
+    const rsrc_t rs_a = make_rsrc(d.ptr[1], (unsigned)M * (unsigned)K * 4u);
+    const rsrc_t rs_b = make_rsrc(d.ptr[0], (unsigned)C * HW4);
+    const int lane_c = cb + (wave * 4 + kq) * G::CPL;     // first channel of this lane's k slot
+    const unsigned va = ((unsigned)(m0 + i16) * (unsigned)K + (unsigned)(lane_c * R)) * 4u;
+    unsigned vb[R];
+    {
+        const int n = n0 + i16;
+        const int oy = n / Wo, ox = n - oy * Wo;
+        const int kw_ = a[REEF_CONV_KW];
+#pragma unroll
+        for (int t = 0; t < R; ++t) {
+            const int ky = t / kw_, kx = t - ky * kw_;
+            const int iy = oy * a[REEF_CONV_SH] + ky - a[REEF_CONV_PH];
+            const int ix = ox * a[REEF_CONV_SW] + kx - a[REEF_CONV_PW];
+            const bool ok = n < N && (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
+            vb[t] = ok ? (unsigned)(iy * W + ix) * 4u + (unsigned)lane_c * HW4 : kOutside;
+        }
+    }
+    // steps this lane's k slot stays inside the channel range of the split
+    const int lane_steps = lane_c < ce ? (ce - lane_c + G::STEP_C - 1) / G::STEP_C : 0;
+
+    float ra[NS][RC], rb[NS][RC];
+    auto load_step = [&](int s, int step) {
+        // offsets are below kOutside (a power of two), so or-ing it in moves them outside
+        const unsigned outm = step < lane_steps ? 0u : kOutside;
+        const unsigned sa = (unsigned)step * (unsigned)(G::STEP_C * R) * 4u;   // uniform
+        const unsigned sb = (unsigned)step * (unsigned)G::STEP_C * HW4;         // uniform
+        const unsigned oa = va | outm;
+#pragma unroll
+        for (int q = 0; q < RC / 4; ++q) {
+            const f32x4 v = __builtin_bit_cast(
+                f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, (int)(oa + 16u * q), (int)sa, 0));
+            ra[s][4 * q] = v[0]; ra[s][4 * q + 1] = v[1]; ra[s][4 * q + 2] = v[2]; ra[s][4 * q + 3] = v[3];
+        }
+#pragma unroll
+        for (int q = RC / 4 * 4; q < RC; ++q)
+            ra[s][q] = __builtin_bit_cast(
+                float, __builtin_amdgcn_raw_buffer_load_b32(rs_a, (int)(oa + 4u * q), (int)sa, 0));
+#pragma unroll
+        for (int q = 0; q < RC; ++q) {
+            // R > 1: tap q of the slot's channel; R == 1: channel q of the slot
+            const unsigned ob = (R > 1 ? vb[q] : vb[0]) | outm;
+            const unsigned sq = R > 1 ? sb : sb + (unsigned)q * HW4;
+            rb[s][q] = __builtin_bit_cast(
+                float, __builtin_amdgcn_raw_buffer_load_b32(rs_b, (int)ob, (int)sq, 0));
+        }
+    };
+
+    // oldest step first: the wait before a step's MFMAs counts the loads issued after its own
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        load_step(s, s);
+        asm volatile("" ::: "memory");
+    }
+    if (Poll::enabled) {
+        if (threadIdx.x == 0) *sflag = 0;
+        __syncthreads();
+    }
+
+    // Whole groups of NS steps with no condition inside (a loop with per-step conditions gets
+    // reordered around the loads), then the remaining steps, whose loads are already under way.
+    f32x4 acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = {0.0f, 0.0f, 0.0f, 0.0f};
+    auto mma_stage = [&](int s) {
+#pragma unroll
+        for (int q = 0; q < RC; ++q) {
+            if (q & 1) acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[s][q], rb[s][q], acc1, 0, 0, 0);
+            else acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[s][q], rb[s][q], acc0, 0, 0, 0);
+        }
+    };
+    int pf = 0;
+    int it = 0;
+    bool left = false;
+    for (; it + NS <= nsteps; it += NS) {
+        if (Poll::enabled) {
+            // the flag is read one group ahead; a wavefront that sees it tells the others
+            // through LDS and all of them leave after the barrier below
+            if (pf) {
+                *sflag = 1;
+                left = true;
+                break;
+            }
+            pf = poll.load();
+        }
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            mma_stage(s);
+            load_step(s, it + s + NS);
+            // keeps each step's refill behind its own MFMAs instead of at the end of the group
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    if (!left) {
+#pragma unroll
+        for (int s = 0; s < NS - 1; ++s)
+            if (it + s < nsteps) mma_stage(s);
+    }
+
+    // partial tile of this wavefront -> LDS; element j of a lane is row 4 * (lane / 16) + j
+    float* part = smem + wave * 256;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) part[(4 * kq + j) * 16 + i16] = acc0[j] + acc1[j];
+    __syncthreads();
+    if (Poll::enabled && *sflag) return false;
+    const float v = ((smem[threadIdx.x] + smem[256 + threadIdx.x]) + smem[512 + threadIdx.x]) + smem[768 + threadIdx.x];
+    if (to_ws) {
+        const rsrc_t ws = make_rsrc((const float*)d.ptr[2] + (size_t)split * M * N, MN4);
+        buf_store(ws, ooff, v);
+    } else {
+        ep.finish(v, ooff, om * 4u, e_res, e_bias, e_sh2);
+    }
+    return true;
+}
+
 // ---- reef_gemm ----------------------------------------------------------------
 // TRANS_B: B stored [N][K] (dense layers, Q.K^T) -- both operands take 128-bit row
 // loads, so K, lda, ldb and the batch strides must be multiples of 4 floats.

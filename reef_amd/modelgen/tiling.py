@@ -23,21 +23,35 @@ TILES = {
     "32x32k4": (6, 32, 32, 0.50, 2),
     "64x32k2": (7, 64, 32, 0.55, 3),
     "32x64k2": (8, 32, 64, 0.55, 3),
+    # direct family (reef_conv2d_d<taps>_16x16k4): never picked by the analytic model, only
+    # through the measured table or an explicit request
+    "16x16k4": (9, 16, 16, 0.40, 2),
 }
+DIRECT_TILE = "16x16k4"
+DIRECT_TAPS = (1, 9)    # filter sizes kh*kw the direct family is compiled for
 # wavefronts that share one output block and split K inside the workgroup
 KW = {"32x32k4": 4, "64x32k2": 2, "32x64k2": 2}
 GEMM_TILES = ("128x128", "64x64", "32x128", "32x32k4", "64x32k2")
 
 
-def step_k(tile):
-    """k values a workgroup consumes per step of its K loop."""
+def step_k(tile, taps=1):
+    """k values a workgroup consumes per step of its K loop (taps = kh*kw, direct family only:
+    a step is 16 channels of a filter with taps > 1, 128 channels of a 1x1 filter)."""
+    if tile == DIRECT_TILE:
+        return 128 if taps == 1 else 16 * taps
     return BK * KW.get(tile, 1)
 
 
-def forced(tile, M, N, K, split=1):
+def direct_ok(cin, kh, kw):
+    """Whether the direct family has a kernel for this filter."""
+    taps = kh * kw
+    return taps in DIRECT_TAPS and (taps > 1 or cin % 8 == 0)
+
+
+def forced(tile, M, N, K, split=1, taps=1):
     """The launch geometry of a given tile and split-K factor (no cost model)."""
     tid, bm, bn, _, _ = TILES[tile]
-    bk = step_k(tile)
+    bk = step_k(tile, taps)
     k_chunk = math.ceil(math.ceil(K / split) / bk) * bk
     s = math.ceil(K / k_chunk)
     mt, nt = math.ceil(M / bm), math.ceil(N / bn)
@@ -58,17 +72,19 @@ def _steps_time(bm, bn, eff, steps):
     return steps * T_STEP_128x128 * (bm * bn) / (128.0 * 128.0) / eff
 
 
-def choose(M, N, K, allow_split=True, tiles=None, max_split=32, fused=True, pointwise=False):
+def choose(M, N, K, allow_split=True, tiles=None, max_split=32, fused=True, pointwise=False,
+           taps=1, direct=False):
     """Returns dict(tile, tile_id, BM, BN, split_k, k_chunk, m_tiles, n_tiles, tasks).
-    Measured choices (tuned.py) win over the analytic model for the shapes they cover."""
+    Measured choices (tuned.py) win over the analytic model for the shapes they cover; an entry
+    that names the direct tile counts only if the caller says the filter qualifies."""
     if allow_split and tiles is None and not fused:
         hit = TUNED.get((M, N, K, 1 if pointwise else 0))
-        if hit is not None:
-            t = forced(hit[0], M, N, K, hit[1])
+        if hit is not None and (hit[0] != DIRECT_TILE or direct):
+            t = forced(hit[0], M, N, K, hit[1], taps)
             t["est_us"] = hit[2]
             return t
     best = None
-    for name in (tiles or TILES.keys()):
+    for name in (tiles or [t for t in TILES if t != DIRECT_TILE]):
         tid, bm, bn, eff, occ = TILES[name]
         m_tiles, n_tiles = math.ceil(M / bm), math.ceil(N / bn)
         nt = m_tiles * n_tiles
@@ -98,6 +114,8 @@ def choose(M, N, K, allow_split=True, tiles=None, max_split=32, fused=True, poin
 
 
 def lds_bytes(tile):
+    if tile == DIRECT_TILE:
+        return 4 * 256 * 4 + 16     # four partial 16x16 tiles + the leave flag
     _, bm, bn, _, _ = TILES[tile]
     bk = step_k(tile)
     a = bm * (bk + 4)

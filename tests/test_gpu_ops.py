@@ -18,14 +18,8 @@ def rnd(*shape):
     return RNG.standard_normal(shape).astype(np.float32)
 
 
-def forced(tile, M, N, K, split):
-    tid, bm, bn, _, _ = tiling.TILES[tile]
-    import math
-    k_chunk = math.ceil(math.ceil(K / split) / 32) * 32
-    s = math.ceil(K / k_chunk)
-    mt, nt = math.ceil(M / bm), math.ceil(N / bn)
-    return dict(tile=tile, tile_id=tid, BM=bm, BN=bn, split_k=s, k_chunk=k_chunk, m_tiles=mt,
-                n_tiles=nt, tasks=s * mt * nt, est_us=1.0)
+def forced(tile, M, N, K, split, taps=1):
+    return tiling.forced(tile, M, N, K, split, taps)
 
 
 CONV_CASES = [
@@ -51,26 +45,28 @@ def test_conv_tiles(tmp_path, tile, case):
     kh, kw = (k, k) if isinstance(k, int) else k
     ph, pw = (p, p) if isinstance(p, int) else p
     Ho, Wo = (H + 2 * ph - kh) // s + 1, (W + 2 * pw - kw) // s + 1
+    if tile == tiling.DIRECT_TILE and not tiling.direct_ok(cin, kh, kw):
+        pytest.skip("the direct family is compiled for 1x1 (Cin % 8 == 0) and 9-tap filters")
     y = g.conv2d(x, cout, k, s, p, bias=True, act=MB.ACT_RELU,
-                 force=forced(tile, cout, Ho * Wo, cin * kh * kw, 1))
+                 force=forced(tile, cout, Ho * Wo, cin * kh * kw, 1, kh * kw))
     g.mark_output(y)
     exe, orc, model = run_both(g, tmp_path, {"data": rnd(cin, H, W)})
     compare_storages(exe, orc, model, what="conv %s %s" % (tile, case))
 
 
 @pytest.mark.parametrize("split", [2, 3, 8])
-@pytest.mark.parametrize("tile", ["64x64", "128x64", "128x32", "32x32k4", "64x32k2", "32x64k2"])
+@pytest.mark.parametrize("tile", ["64x64", "128x64", "128x32", "32x32k4", "64x32k2", "32x64k2", "16x16k4"])
 def test_conv_split_k_and_epilogues(tmp_path, tile, split):
     cin, H, W, cout = 96, 14, 14, 160
     g = MB.GraphBuilder("s")
     x = g.input("data", (cin, H, W))
     res = g.input("res", (cout, H, W))
-    f = forced(tile, cout, H * W, cin * 9, split)
+    f = forced(tile, cout, H * W, cin * 9, split, 9)
     y1 = g.conv2d(x, cout, 3, 1, 1, bias=True, act=MB.ACT_RELU, force=f)
     y2 = g.conv2d(x, cout, 3, 1, 1, bias=False, act=MB.ACT_NONE, residual=res, force=f)
     y3 = g.conv2d(x, cout, 3, 1, 1, bias=True, act=MB.ACT_RELU, residual=res, force=f)
     y4 = g.conv2d(x, cout, 3, 1, 1, bias=False, act=MB.ACT_RELU, residual=res, affine=True, force=f)
-    f1 = forced(tile, cout, H * W, cin * 9, 1)
+    f1 = forced(tile, cout, H * W, cin * 9, 1, 9)
     y5 = g.conv2d(x, cout, 3, 1, 1, bias=False, act=MB.ACT_RELU, residual=res, affine=True, force=f1)
     y6 = g.conv2d(x, cout, 3, 1, 1, bias=True, act=MB.ACT_RELU6, force=f1)
     g.mark_output(y6)
@@ -114,6 +110,33 @@ def test_fused_split_k_equals_plain_split_k_bitwise(tmp_path, tile, split):
             np.testing.assert_array_equal(exe.get_data(t_plain.idx, t_plain.size),
                                           exe.get_data(t_fused.idx, t_fused.size))
         exe.execute()
+
+
+@pytest.mark.parametrize("split", [1, 2])
+def test_conv_direct_family_epilogues(tmp_path, split):
+    """Direct-operand family (16x16 tiles, channels split over the wavefronts): every epilogue
+    form, a second output, a channel slice of a concatenation buffer, ragged M / N / Cin, and
+    a strided 1x1, each with and without split-K across workgroups."""
+    cin, H, W, cout = 72, 13, 13, 88          # Cin % 16 != 0, M % 16 != 0, N = 169
+    g = MB.GraphBuilder("d")
+    x = g.input("data", (cin, H, W))
+    res = g.input("res", (cout, H, W))
+    M, N = cout, H * W
+    f9 = forced("16x16k4", M, N, cin * 9, split, 9)
+    f1 = forced("16x16k4", M, N, cin, split, 1)
+    g.conv2d(x, cout, 3, 1, 1, bias=True, act=MB.ACT_RELU, residual=res, force=f9)
+    g.conv2d(x, cout, 3, 1, 1, bias=False, act=MB.ACT_RELU, residual=res, affine=True, force=f9)
+    g.conv2d(x, cout, 3, 1, 1, bias=False, act=MB.ACT_NONE, residual=res, dual_act=MB.ACT_RELU, force=f9)
+    g.conv2d(x, cout, 1, 1, 0, bias=True, act=MB.ACT_RELU6, force=f1)
+    g.conv2d(x, cout, 1, 1, 0, bias=False, act=MB.ACT_NONE, residual=res, dual_act=MB.ACT_RELU, force=f1)
+    cat = g.temp((2 * cout, H, W))
+    g.conv2d(x, cout, 3, 1, 1, force=f9, out=cat, out_channel=0)
+    g.conv2d(x, cout, 1, 1, 0, force=f1, out=cat, out_channel=cout)
+    Ho = (H - 1) // 2 + 1
+    y = g.conv2d(x, cout, 1, 2, 0, force=forced("16x16k4", M, Ho * Ho, cin, split, 1))
+    g.mark_output(y)
+    exe, orc, model = run_both(g, tmp_path, {"data": rnd(cin, H, W), "res": rnd(cout, H, W)})
+    compare_storages(exe, orc, model, what="direct family x%d" % split)
 
 
 def test_conv_auto_heuristic_shapes(tmp_path):
