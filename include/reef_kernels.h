@@ -173,10 +173,10 @@ enum {
  *   reef_conv2d_<tile>      general: im2col gather, needs K % 4 == 0
  *   reef_conv2d_pw_<tile>   pointwise: 1x1, stride 1, no padding, N % 4 == 0, K % 4 == 0
  *   reef_conv2d_u_<tile>    unaligned: im2col gather, any K
- *   reef_conv2d_d<R>_16x16k4  direct: R = kh*kw taps compiled in (1, 9); operands go from memory
+ *   reef_conv2d_d<R>_16x16k4  direct: R = kh*kw taps compiled in (1, 3, 7, 9); operands go from memory
  *                           straight into 16x16x4 MFMAs, the four wavefronts split the input
  *                           channels.  d1 needs Cin % 8 == 0 (any stride); K_CHUNK is a multiple
- *                           of R (d9) or 8 (d1) and splits K on channel boundaries. */
+ *                           of R (R > 1) or 8 (d1) and splits K on channel boundaries. */
 #define REEF_CONV_MODE_GENERAL 0
 #define REEF_CONV_MODE_POINTWISE 1
 #define REEF_CONV_MODE_UNALIGNED 2

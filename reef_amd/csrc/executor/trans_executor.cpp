@@ -57,12 +57,13 @@ Status TransExecutor::init_rt_executor(const char* json_file_path, GPUModule_t m
         const uint32_t* lp = ki.launch_params;
         ka.kernel = kernel_funcs[i];
         ka.op = op_from_name(kernel_symbol(ki.name));
-        int tile = -1, mode = 0;
+        int tile = -1, mode = 0, taps = 0;
         if (ka.op == REEF_OP_CONV2D && ki.attrs.size() > REEF_CONV_MODE) {
             tile = ki.attrs[REEF_CONV_TILE];
             mode = ki.attrs[REEF_CONV_MODE];
+            taps = ki.attrs[REEF_CONV_KH] * ki.attrs[REEF_CONV_KW];
         }
-        ka.proxy_level = proxy_level(ka.op, tile, mode);
+        ka.proxy_level = proxy_level(ka.op, tile, mode, taps);
         ka.task_dim = dim3u(lp[0], lp[1], lp[2]);
         ka.thread_dim = dim3u(lp[3], lp[4], lp[5]);
         ka.block_num = (int)ka.task_dim.count();
@@ -152,8 +153,9 @@ int TransExecutor::proxy_class_of_level(int level) {
 // Which proxy holds the body of (op, tile, loader family): the bandwidth-bound ops
 // are in every proxy, a few matrix-core tiles in the classes whose register budget
 // fits them, and everything else in none (-1: that kernel is never merged).
-int TransExecutor::proxy_level(int op, int tile, int mode) {
+int TransExecutor::proxy_level(int op, int tile, int mode, int taps) {
     if (op == REEF_OP_CONV2D) {
+        if (mode == REEF_CONV_MODE_DIRECT) return (taps == 1 || taps == 9) ? 1 : -1;
         if (mode != REEF_CONV_MODE_GENERAL && mode != REEF_CONV_MODE_POINTWISE) return -1;
         if (tile == REEF_TILE_64x64 || tile == REEF_TILE_128x32) return 1;
         if (tile == REEF_TILE_128x64) return 2;

@@ -51,7 +51,7 @@ public:
     // this kernel set: merge_framework_8 / _3 / _2 = levels 0..2.
     static constexpr int kNumProxyLevels = 3;
     static int proxy_class_of_level(int level);
-    static int proxy_level(int op, int tile, int mode);
+    static int proxy_level(int op, int tile, int mode, int taps = 0);
 
 protected:
     Status init_rt_executor(const char* json_file_path, GPUModule_t module);

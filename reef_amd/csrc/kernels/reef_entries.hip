@@ -195,6 +195,8 @@ REEF_ENTRY(reef_conv2d_u_32x32k4, OpConv<Tile32x32k4 REEF_COMMA CONV_UNALIGNED>)
 REEF_ENTRY(reef_conv2d_u_64x32k2, OpConv<Tile64x32k2 REEF_COMMA CONV_UNALIGNED>)
 REEF_ENTRY(reef_conv2d_u_32x64k2, OpConv<Tile32x64k2 REEF_COMMA CONV_UNALIGNED>)
 REEF_ENTRY(reef_conv2d_d1_16x16k4, OpConvDirect<1>)
+REEF_ENTRY(reef_conv2d_d3_16x16k4, OpConvDirect<3>)
+REEF_ENTRY(reef_conv2d_d7_16x16k4, OpConvDirect<7>)
 REEF_ENTRY(reef_conv2d_d9_16x16k4, OpConvDirect<9>)
 REEF_ENTRY(reef_gemm_nt_128x128, OpGemm<Tile128x128 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nt_64x64, OpGemm<Tile64x64 REEF_COMMA true>)
@@ -230,7 +232,8 @@ REEF_ENTRY(multiply, OpMocked<true>)
 // the proxy switches into the inlined body; the variants are the gfx950
 // occupancy classes that matter for this kernel set, <n> = wavefronts per SIMD:
 //   merge_framework_8  bandwidth-bound ops only                          (<= 64 registers)
-//   merge_framework_3  + conv (general, pointwise) tiles 64x64 / 128x32    (<= 168)
+//   merge_framework_3  + conv (general, pointwise) tiles 64x64 / 128x32,
+//                        direct family with 1 and 9 taps                      (<= 168)
 //   merge_framework_2  + conv (general, pointwise) tile 128x64 and the
 //                        wave-split-K tiles                                   (<= 256)
 // Kernels outside these sets (the other tiles, the unaligned-K convolution, GEMM)
@@ -246,7 +249,11 @@ __device__ __forceinline__ void run_op(const ReefDkpSide& s, int task, char* sme
         case REEF_OP_CONV2D:
             if (LEVEL >= 1) {
                 const int tile = d.attr[REEF_CONV_TILE];
-                if (d.attr[REEF_CONV_MODE] == CONV_POINTWISE) {
+                if (d.attr[REEF_CONV_MODE] == REEF_CONV_MODE_DIRECT) {
+                    const int taps = d.attr[REEF_CONV_KH] * d.attr[REEF_CONV_KW];
+                    if (taps == 1) OpConvDirect<1>::run(d, task, smem, np);
+                    else if (taps == 9) OpConvDirect<9>::run(d, task, smem, np);
+                } else if (d.attr[REEF_CONV_MODE] == CONV_POINTWISE) {
                     if (tile == REEF_TILE_64x64) OpConv<Tile64x64, CONV_POINTWISE>::run(d, task, smem, np);
                     else if (tile == REEF_TILE_128x32) OpConv<Tile128x32, CONV_POINTWISE>::run(d, task, smem, np);
                     else if (LEVEL >= 2 && tile == REEF_TILE_32x32k4) OpConv<Tile32x32k4, CONV_POINTWISE>::run(d, task, smem, np);

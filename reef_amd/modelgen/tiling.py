@@ -28,7 +28,7 @@ TILES = {
     "16x16k4": (9, 16, 16, 0.40, 2),
 }
 DIRECT_TILE = "16x16k4"
-DIRECT_TAPS = (1, 9)    # filter sizes kh*kw the direct family is compiled for
+DIRECT_TAPS = (1, 3, 7, 9)    # filter sizes kh*kw the direct family is compiled for
 # wavefronts that share one output block and split K inside the workgroup
 KW = {"32x32k4": 4, "64x32k2": 2, "32x64k2": 2}
 GEMM_TILES = ("128x128", "64x64", "32x128", "32x32k4", "64x32k2")

@@ -33,6 +33,8 @@ CONV_CASES = [
     (16, 17, 17, 24, 5, 1, 2),
     (40, 15, 15, 136, 3, 2, 1),
     (256, 7, 7, 64, 3, 1, 1),        # N = 49
+    (32, 8, 10, 48, (1, 3), 1, (0, 1)),
+    (32, 10, 8, 48, (3, 1), 2, (1, 0)),
 ]
 
 
@@ -46,7 +48,7 @@ def test_conv_tiles(tmp_path, tile, case):
     ph, pw = (p, p) if isinstance(p, int) else p
     Ho, Wo = (H + 2 * ph - kh) // s + 1, (W + 2 * pw - kw) // s + 1
     if tile == tiling.DIRECT_TILE and not tiling.direct_ok(cin, kh, kw):
-        pytest.skip("the direct family is compiled for 1x1 (Cin % 8 == 0) and 9-tap filters")
+        pytest.skip("the direct family is compiled for 1x1 (Cin % 8 == 0) and 3-, 7-, 9-tap filters")
     y = g.conv2d(x, cout, k, s, p, bias=True, act=MB.ACT_RELU,
                  force=forced(tile, cout, Ho * Wo, cin * kh * kw, 1, kh * kw))
     g.mark_output(y)
