@@ -724,7 +724,8 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
 // the tiled kernels (it is fixed, so results are reproducible run to run).
 struct TileD16 {
     static constexpr int BM = 16, BN = 16;
-    static constexpr int LDS_BYTES = 4 * 256 * 4 + 16;
+    static constexpr int PART = 320;   // floats per wavefront's partial tile in LDS (256 + row-group skew)
+    static constexpr int LDS_BYTES = 4 * PART * 4 + 16;
 };
 
 template <int R>
@@ -742,7 +743,7 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     typedef DirectGeom<R> G;
     constexpr int RC = G::RC, NS = G::NS;
     float* smem = (float*)smem_raw;
-    int* sflag = (int*)(smem + 4 * 256);
+    int* sflag = (int*)(smem + 4 * TileD16::PART);
     const ReefOpDesc& d = d_in;
     const int* a = d.attr;
     const int lane = threadIdx.x & 63, i16 = lane & 15, kq = lane >> 4;
@@ -879,13 +880,15 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
             if (it + s < nsteps) mma_stage(s);
     }
 
-    // partial tile of this wavefront -> LDS; element j of a lane is row 4 * (lane / 16) + j
-    float* part = smem + wave * 256;
+    // partial tile of this wavefront -> LDS; element j of a lane is row 4 * (lane / 16) + j.
+    // Each group of four rows is skewed by 16 floats so the four k slots write to different banks.
+    float* part = smem + wave * TileD16::PART;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) part[(4 * kq + j) * 16 + i16] = acc0[j] + acc1[j];
+    for (int j = 0; j < 4; ++j) part[(5 * kq + j) * 16 + i16] = acc0[j] + acc1[j];
     __syncthreads();
     if (Poll::enabled && *sflag) return false;
-    const float v = ((smem[threadIdx.x] + smem[256 + threadIdx.x]) + smem[512 + threadIdx.x]) + smem[768 + threadIdx.x];
+    const float* mine = smem + threadIdx.x + (threadIdx.x >> 6) * 16;
+    const float v = ((mine[0] + mine[TileD16::PART]) + mine[2 * TileD16::PART]) + mine[3 * TileD16::PART];
     if (to_ws) {
         const rsrc_t ws = make_rsrc((const float*)d.ptr[2] + (size_t)split * M * N, MN4);
         buf_store(ws, ooff, v);

@@ -115,7 +115,7 @@ def choose(M, N, K, allow_split=True, tiles=None, max_split=32, fused=True, poin
 
 def lds_bytes(tile):
     if tile == DIRECT_TILE:
-        return 4 * 256 * 4 + 16     # four partial 16x16 tiles + the leave flag
+        return 4 * 320 * 4 + 16     # four partial 16x16 tiles (skewed rows) + the leave flag
     _, bm, bn, _, _ = TILES[tile]
     bk = step_k(tile)
     a = bm * (bk + 4)
