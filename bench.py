@@ -19,6 +19,8 @@ The same JSON line carries
     the kernels are launched on;
   * a CPU baseline: the same ResNet-152 graph executed by the CPU oracle on the
     host cores;
+  * the convolution tiles on two device-filling layers (`steady_state_conv`), to separate what
+    the K loop sustains from what a batch-1 launch allows;
   * two further co-location scenarios (dynamic kernel padding with a
     MobileNetV2 best-effort client; Inception-v3 real-time with two BERT-base
     best-effort clients), shorter runs.
@@ -63,6 +65,33 @@ def cpu_baseline(model_dir, name, x, budget_s=30.0):
             "sample": "%d whole ResNet-152 batch-1 inferences (22.56 GFLOP each) by the CPU oracle "
                       "(C, OpenMP), best of them; TVM is not installed, so this stands in for the "
                       "TVM-llvm build of the model" % len(times)}, orc
+
+
+def steady_state_conv(root, iters):
+    """The staged convolution tiles on two layers large enough to fill the device (12544 and
+    3136 output pixels): what the K loop sustains when a launch is not latency bound."""
+    from reef_amd import binding as B
+    from reef_amd.modelgen import builder as MB
+    from reef_amd.modelgen import tiling
+    cases = [("3x3 256->256 @112x112", 256, 112, 256, 3, 1, "128x64"),
+             ("1x1 1024->1024 @56x56", 1024, 56, 1024, 1, 0, "64x64")]
+    g = MB.GraphBuilder("steady")
+    meta = []
+    for label, cin, hw, cout, k, pad, tile in cases:
+        x = g.input("in_%d_%d" % (cin, hw), (cin, hw, hw))
+        g.conv2d(x, cout, k, 1, pad, bias=True, act=MB.ACT_RELU,
+                 force=tiling.forced(tile, cout, hw * hw, cin * k * k, 1, k * k))
+        meta.append((label, tile, len(g.kernels) - 1, 2.0 * cout * hw * hw * cin * k * k))
+    d = os.path.dirname(g.write(os.path.join(root, g.name)))
+    exe = B.Executor.from_dir(d, g.name, B.BASE)
+    out = []
+    for label, tile, idx, fl in meta:
+        us = exe.time_kernel(idx, B.RUN_DEFAULT, 3, iters)
+        out.append({"layer": label, "kernel": g.kernels[idx]["name"].split("#")[0], "us": round(us, 2),
+                    "tflops": round(fl / us / 1e6, 2),
+                    "frac_mfma_peak": round(fl / us / 1e6 / FP32_MFMA_PEAK_TFLOPS, 4)})
+    exe.close()
+    return out
 
 
 def calibrate_copy(mib, root):
@@ -301,6 +330,7 @@ def main():
     }
     got = exe.get_output()
     exe.close()
+    out["steady_state_conv"] = steady_state_conv(tmp.name, max(args.kernel_iters, 5))
     if 4 in configs:
         k = max(args.steps // 2, 50)
         out["corun_dkp_mobilenetv2"] = {
