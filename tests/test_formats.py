@@ -215,3 +215,47 @@ def test_code_object_metadata_reader():
                   "reef_gemm_nn_64x64", "reef_dense", "reef_layernorm", "add"):
             assert L.reef_code_object_kernel_meta(code_object(fl).encode(), k.encode(), out) == 0
             assert out[4] == 0, (fl, k)
+
+
+def test_benchmark_models_name_only_compiled_kernels_without_scratch():
+    """Every kernel symbol the generator emits for the four CNNs and BERT exists in all three
+    code objects, uses no scratch memory, and the three proxies stay inside their register
+    classes (waves per SIMD 8 / 3 / 2 on a 512-entry register file)."""
+    import ctypes
+    from reef_amd.modelgen import nets
+    from reef_amd.paths import code_object
+    L = B.lib()
+    out = (ctypes.c_int * 6)()
+    symbols = set()
+    for name in ("resnet152", "densenet201", "inceptionv3", "mobilenetv2", "bert_base"):
+        g = nets.BUILDERS[name]()
+        symbols |= {k["name"].split("#")[0] for k in g.kernels}
+    assert any(s.startswith("reef_conv2d_d") for s in symbols)      # the direct family is in use
+    for fl in ("raw", "be", "trans"):
+        co = code_object(fl).encode()
+        for sym in sorted(symbols):
+            assert L.reef_code_object_kernel_meta(co, sym.encode(), out) == 0, (fl, sym)
+            assert out[4] == 0, "%s in %s.co uses %d bytes of scratch" % (sym, fl, out[4])
+    co = code_object("trans").encode()
+    for n, budget in ((8, 64), (3, 168), (2, 256)):
+        assert L.reef_code_object_kernel_meta(co, ("merge_framework_%d" % n).encode(), out) == 0
+        assert out[4] == 0 and out[0] + out[1] <= budget, (n, list(out))
+
+
+def test_direct_tile_geometry():
+    """Launch geometry of the direct family: K is split on channel boundaries, in whole steps
+    (16 channels of a filter with several taps, 128 channels of a 1x1 filter)."""
+    from reef_amd.modelgen import tiling
+    f = tiling.forced("16x16k4", 256, 196, 2304, 1, 9)
+    assert (f["m_tiles"], f["n_tiles"], f["split_k"], f["k_chunk"], f["tasks"]) == (16, 13, 1, 2304, 208)
+    f = tiling.forced("16x16k4", 88, 169, 72 * 9, 2, 9)
+    assert f["k_chunk"] % (16 * 9) == 0 and f["split_k"] == 2 and f["k_chunk"] * 2 >= 72 * 9
+    f = tiling.forced("16x16k4", 512, 49, 1024, 3, 1)
+    assert f["k_chunk"] % 128 == 0 and f["split_k"] * f["k_chunk"] >= 1024
+    assert tiling.direct_ok(256, 3, 3) and tiling.direct_ok(64, 1, 1) and tiling.direct_ok(24, 1, 7)
+    assert not tiling.direct_ok(3, 7, 7) and not tiling.direct_ok(20, 1, 1) and not tiling.direct_ok(16, 5, 5)
+    # the analytic model never picks the direct tile; only the measured table may, and only
+    # when the caller vouches for the filter
+    t = tiling.choose(256, 196, 2304, fused=False, pointwise=False, taps=9, direct=False)
+    assert t["tile"] != "16x16k4"
+    assert tiling.lds_bytes("16x16k4") == 4 * 320 * 4 + 16
