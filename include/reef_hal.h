@@ -76,7 +76,10 @@ enum { REEF_MEM_DEVICE = 0, REEF_MEM_DEVICE_FINEGRAINED = 1, REEF_MEM_HOST_PINNE
 
 const char* reef_hal_last_error(void);
 
-/* hipInit + hipDeviceGet            executor_base.cpp:19-22 */
+/* hipInit + hipDeviceGet            executor_base.cpp:19-22
+ * The HIP backend also opens the runtime's pool of hardware queues with idle streams that live as
+ * long as the process, so streams created later are spread over different hardware queues instead
+ * of sharing one by accident of creation order (REEF_HAL_HOLD_QUEUES=0: off). */
 int reef_hal_init(int device);
 /* GPUConfig::get_num_cus            hip_impl.cpp:9-12 */
 int reef_hal_device_info(reef_device_info* out);
