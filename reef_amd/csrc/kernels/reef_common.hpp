@@ -44,6 +44,12 @@ __device__ __forceinline__ void store_agent(float* p, float v) {
 __device__ __forceinline__ float load_agent(const float* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// Waits until every vector-memory operation this lane has issued, device-scope stores included,
+// has been acknowledged; keeps the compiler from moving memory operations across it.
+__device__ __forceinline__ void partial_stores_done() {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+}
 
 // ---- buffer addressing ------------------------------------------------------------
 // Tile loads and output stores go through buffer instructions: the tensor is described by a

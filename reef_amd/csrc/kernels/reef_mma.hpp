@@ -469,6 +469,7 @@ struct ConvEpilogue {
     rsrc_t out, out2, res, bias, scale, shift, shift2;
     bool has_res, has_bias, has_affine, has_dual;
     int act, act2;
+    int next;         // first pointer slot after the optional operands
     unsigned doff4;   // byte offset of this layer's slice inside the output tensor(s)
     __device__ __forceinline__ void init(const ReefOpDesc& d, int flags, int act_, int act2_, int M,
                                          unsigned MN4, unsigned doff4_) {
@@ -495,6 +496,7 @@ struct ConvEpilogue {
         }
         act = act_;
         act2 = act2_;
+        next = p;
     }
     // off = (m * N + n) * 4 or outside; m4 = m * 4.  v = acc; v += residual; v += bias;
     // v = fma(v, scale, shift); act  -- then out2 = act2(out + shift2).
@@ -662,8 +664,11 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
                     if (m < M && n < N) store_agent(part + (size_t)m * N + n, res[tm][tn][rr]);
                 }
             }
-        // every store of this workgroup has completed at device scope before it counts in
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        // Every store of this workgroup has completed at device scope before it counts in.  The
+        // stores carry device scope themselves, so they are complete once acknowledged: each
+        // lane waits for its own (a workgroup-scope fence alone does not wait for outstanding
+        // stores on this target), then the barrier collects all lanes.
+        partial_stores_done();
         __syncthreads();
         if (threadIdx.x == 0) {
             const int old = __hip_atomic_fetch_add(&counters[rem], 1, __ATOMIC_RELAXED,
@@ -722,28 +727,40 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
 // partial tiles are summed through LDS in wavefront order and thread t writes output element
 // (t / 16, t % 16), so stores are 64-byte runs along a row.  The sum order over k differs from
 // the tiled kernels (it is fixed, so results are reproducible run to run).
+template <int TN_>
 struct TileD16 {
-    static constexpr int BM = 16, BN = 16;
-    static constexpr int PART = 320;   // floats per wavefront's partial tile in LDS (256 + row-group skew)
-    static constexpr int LDS_BYTES = 4 * PART * 4 + 16;
+    static constexpr int TN = TN_;      // 16-pixel column groups per workgroup: the tile is 16 x 16 TN
+    static constexpr int BM = 16, BN = 16 * TN;
+    static constexpr int PART = 320;    // floats per 16 x 16 partial tile in LDS (256 + row-group skew)
+    static constexpr int LDS_BYTES = 4 * TN * PART * 4 + 16;
 };
 
-template <int R>
+template <int R, int TN>
 struct DirectGeom {
     static constexpr int CPL = R == 1 ? 8 : 1;   // channels per k slot and step
-    static constexpr int RC = R * CPL;           // A values (= B values = MFMAs) per lane and step
+    static constexpr int RC = R * CPL;           // A values per lane and step (x TN B values and MFMAs)
     static constexpr int STEP_C = 16 * CPL;      // channels a workgroup consumes per step
-    static constexpr int LOADS = (RC / 4) + (RC % 4) + RC;  // vector-memory instructions per step
-    static constexpr int NS = 60 / LOADS;         // steps of loads in flight per wavefront
+    static constexpr int LOADS = (RC / 4) + (RC % 4) + TN * RC;  // vector-memory instructions per step
+    static constexpr int NS = 60 / LOADS < 2 ? 2 : 60 / LOADS;   // steps of loads in flight per wavefront
 };
 
-template <int R, class Poll>
+// TN > 1 widens the tile along the pixels: every weight value a lane has loaded is multiplied
+// with TN pixel groups, so the weight rows -- the larger, cold operand -- are streamed by a
+// TN-th of the workgroups.  What a CU can pull from memory per microsecond is what bounds these
+// kernels at batch 1 (a lone workgroup on an idle device takes as long as 208 of them), so fewer,
+// wider tiles are combined with a split of K across workgroups to keep every CU busy with a
+// shorter stream; REEF_F_FUSED_REDUCE then folds the split inside this launch: a workgroup
+// stores its partial tile, counts itself in, and the last one to arrive for a tile adds the
+// partial tiles in ascending split order (fixed order, so the result does not depend on who is
+// last) and runs the epilogue.
+template <int R, int TN, class Poll>
 __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int task, char* smem_raw,
                                                    const Poll& poll) {
-    typedef DirectGeom<R> G;
+    typedef DirectGeom<R, TN> G;
+    typedef TileD16<TN> TD;
     constexpr int RC = G::RC, NS = G::NS;
     float* smem = (float*)smem_raw;
-    int* sflag = (int*)(smem + 4 * TileD16::PART);
+    int* sflag = (int*)(smem + 4 * TN * TD::PART);
     const ReefOpDesc& d = d_in;
     const int* a = d.attr;
     const int lane = threadIdx.x & 63, i16 = lane & 15, kq = lane >> 4;
@@ -759,7 +776,7 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     const int split = task / tiles;
     const int rem = task - split * tiles;
     const int mt = rem / n_tiles, nt = rem - mt * n_tiles;
-    const int m0 = mt * 16, n0 = nt * 16;
+    const int m0 = mt * 16, n0 = nt * TD::BN;
     const int c_chunk = a[REEF_CONV_K_CHUNK] / R;
     const int cb = split * c_chunk;
     const int ce = min(C, cb + c_chunk);
@@ -767,19 +784,31 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     const unsigned HW4 = (unsigned)(H * W) * 4u;
     const unsigned MN4 = (unsigned)M * (unsigned)N * 4u;
     const int flags = a[REEF_CONV_FLAGS];
+    const bool fused = split_k > 1 && (flags & REEF_F_FUSED_REDUCE);
+    const bool to_ws = split_k > 1 && !fused;   // plain split-K: partial tile to the workspace
 
-    // epilogue operands of the one output element this thread writes, fetched ahead of the K loop
+    // epilogue operands of the TN output elements this thread writes (element g: row t / 16,
+    // column 16 g + t % 16 of the tile), fetched ahead of the K loop
     const int orow = threadIdx.x >> 4, ocol = threadIdx.x & 15;
-    const unsigned om = (unsigned)(m0 + orow), on = (unsigned)(n0 + ocol);
-    const unsigned ooff = on < (unsigned)N ? (om * (unsigned)N + on) * 4u : kOutside;
-    const bool to_ws = split_k > 1;
+    const unsigned om = (unsigned)(m0 + orow);
+    unsigned ooff[TN];
+#pragma unroll
+    for (int g = 0; g < TN; ++g) {
+        const unsigned on = (unsigned)(n0 + 16 * g + ocol);
+        ooff[g] = on < (unsigned)N ? (om * (unsigned)N + on) * 4u : kOutside;
+    }
     ConvEpilogue ep;
-    float e_bias = 0.0f, e_res = 0.0f, e_sh2 = 0.0f;
+    float e_bias = 0.0f, e_sh2 = 0.0f, e_res[TN];
+#pragma unroll
+    for (int g = 0; g < TN; ++g) e_res[g] = 0.0f;
     if (!to_ws) {
         ep.init(d, flags, a[REEF_CONV_ACT], a[REEF_CONV_ACT2], M, MN4, (unsigned)a[REEF_CONV_DST_OFF] * 4u);
         if (ep.has_bias) e_bias = buf_load(ep.bias, om * 4u);
-        if (ep.has_res) e_res = buf_load(ep.res, ooff);
         if (ep.has_dual) e_sh2 = buf_load(ep.shift2, om * 4u);
+        if (ep.has_res) {
+#pragma unroll
+            for (int g = 0; g < TN; ++g) e_res[g] = buf_load(ep.res, ooff[g]);
+        }
     }
 
     // per-lane operand offsets
@@ -787,24 +816,27 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     const rsrc_t rs_b = make_rsrc(d.ptr[0], (unsigned)C * HW4);
     const int lane_c = cb + (wave * 4 + kq) * G::CPL;     // first channel of this lane's k slot
     const unsigned va = ((unsigned)(m0 + i16) * (unsigned)K + (unsigned)(lane_c * R)) * 4u;
-    unsigned vb[R];
+    unsigned vb[TN][R];
     {
-        const int n = n0 + i16;
-        const int oy = n / Wo, ox = n - oy * Wo;
         const int kw_ = a[REEF_CONV_KW];
 #pragma unroll
-        for (int t = 0; t < R; ++t) {
-            const int ky = t / kw_, kx = t - ky * kw_;
-            const int iy = oy * a[REEF_CONV_SH] + ky - a[REEF_CONV_PH];
-            const int ix = ox * a[REEF_CONV_SW] + kx - a[REEF_CONV_PW];
-            const bool ok = n < N && (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
-            vb[t] = ok ? (unsigned)(iy * W + ix) * 4u + (unsigned)lane_c * HW4 : kOutside;
+        for (int g = 0; g < TN; ++g) {
+            const int n = n0 + 16 * g + i16;
+            const int oy = n / Wo, ox = n - oy * Wo;
+#pragma unroll
+            for (int t = 0; t < R; ++t) {
+                const int ky = t / kw_, kx = t - ky * kw_;
+                const int iy = oy * a[REEF_CONV_SH] + ky - a[REEF_CONV_PH];
+                const int ix = ox * a[REEF_CONV_SW] + kx - a[REEF_CONV_PW];
+                const bool ok = n < N && (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
+                vb[g][t] = ok ? (unsigned)(iy * W + ix) * 4u + (unsigned)lane_c * HW4 : kOutside;
+            }
         }
     }
     // steps this lane's k slot stays inside the channel range of the split
     const int lane_steps = lane_c < ce ? (ce - lane_c + G::STEP_C - 1) / G::STEP_C : 0;
 
-    float ra[NS][RC], rb[NS][RC];
+    float ra[NS][RC], rb[NS][TN][RC];
     auto load_step = [&](int s, int step) {
         // offsets are below kOutside (a power of two), so or-ing it in moves them outside
         const unsigned outm = step < lane_steps ? 0u : kOutside;
@@ -822,13 +854,15 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
             ra[s][q] = __builtin_bit_cast(
                 float, __builtin_amdgcn_raw_buffer_load_b32(rs_a, (int)(oa + 4u * q), (int)sa, 0));
 #pragma unroll
-        for (int q = 0; q < RC; ++q) {
-            // R > 1: tap q of the slot's channel; R == 1: channel q of the slot
-            const unsigned ob = (R > 1 ? vb[q] : vb[0]) | outm;
-            const unsigned sq = R > 1 ? sb : sb + (unsigned)q * HW4;
-            rb[s][q] = __builtin_bit_cast(
-                float, __builtin_amdgcn_raw_buffer_load_b32(rs_b, (int)ob, (int)sq, 0));
-        }
+        for (int g = 0; g < TN; ++g)
+#pragma unroll
+            for (int q = 0; q < RC; ++q) {
+                // R > 1: tap q of the slot's channel; R == 1: channel q of the slot
+                const unsigned ob = (R > 1 ? vb[g][q] : vb[g][0]) | outm;
+                const unsigned sq = R > 1 ? sb : sb + (unsigned)q * HW4;
+                rb[s][g][q] = __builtin_bit_cast(
+                    float, __builtin_amdgcn_raw_buffer_load_b32(rs_b, (int)ob, (int)sq, 0));
+            }
     };
 
     // oldest step first: the wait before a step's MFMAs counts the loads issued after its own
@@ -844,13 +878,19 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
 
     // Whole groups of NS steps with no condition inside (a loop with per-step conditions gets
     // reordered around the loads), then the remaining steps, whose loads are already under way.
-    f32x4 acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = {0.0f, 0.0f, 0.0f, 0.0f};
+    // Two accumulators per pixel group, so consecutive MFMAs never depend on each other.
+    f32x4 acc[TN][2];
+#pragma unroll
+    for (int g = 0; g < TN; ++g) {
+        acc[g][0] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        acc[g][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
     auto mma_stage = [&](int s) {
 #pragma unroll
-        for (int q = 0; q < RC; ++q) {
-            if (q & 1) acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[s][q], rb[s][q], acc1, 0, 0, 0);
-            else acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[s][q], rb[s][q], acc0, 0, 0, 0);
-        }
+        for (int q = 0; q < RC; ++q)
+#pragma unroll
+            for (int g = 0; g < TN; ++g)
+                acc[g][q & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[s][q], rb[s][g][q], acc[g][q & 1], 0, 0, 0);
     };
     int pf = 0;
     int it = 0;
@@ -880,21 +920,70 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
             if (it + s < nsteps) mma_stage(s);
     }
 
-    // partial tile of this wavefront -> LDS; element j of a lane is row 4 * (lane / 16) + j.
+    // partial tiles of this wavefront -> LDS; element j of a lane is row 4 * (lane / 16) + j.
     // Each group of four rows is skewed by 16 floats so the four k slots write to different banks.
-    float* part = smem + wave * TileD16::PART;
+    float* part = smem + wave * (TN * TD::PART);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) part[(5 * kq + j) * 16 + i16] = acc0[j] + acc1[j];
+    for (int g = 0; g < TN; ++g)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            part[g * TD::PART + (5 * kq + j) * 16 + i16] = acc[g][0][j] + acc[g][1][j];
     __syncthreads();
     if (Poll::enabled && *sflag) return false;
     const float* mine = smem + threadIdx.x + (threadIdx.x >> 6) * 16;
-    const float v = ((mine[0] + mine[TileD16::PART]) + mine[2 * TileD16::PART]) + mine[3 * TileD16::PART];
+    float v[TN];
+#pragma unroll
+    for (int g = 0; g < TN; ++g) {
+        const float* e = mine + g * TD::PART;
+        v[g] = ((e[0] + e[TN * TD::PART]) + e[2 * TN * TD::PART]) + e[3 * TN * TD::PART];
+    }
     if (to_ws) {
         const rsrc_t ws = make_rsrc((const float*)d.ptr[2] + (size_t)split * M * N, MN4);
-        buf_store(ws, ooff, v);
-    } else {
-        ep.finish(v, ooff, om * 4u, e_res, e_bias, e_sh2);
+#pragma unroll
+        for (int g = 0; g < TN; ++g) buf_store(ws, ooff[g], v[g]);
+        return true;
     }
+    if (!fused) {
+#pragma unroll
+        for (int g = 0; g < TN; ++g) ep.finish(v[g], ooff[g], om * 4u, e_res[g], e_bias, e_sh2);
+        return true;
+    }
+
+    // split-K folded inside the launch
+    const size_t MN = (size_t)M * N;
+    float* ws = (float*)d.ptr[ep.next];
+    int* counters = (int*)d.ptr[ep.next + 1] + a[REEF_CONV_SYNC_OFF];
+    int* s_last = sflag + 1;
+#pragma unroll
+    for (int g = 0; g < TN; ++g)
+        if (ooff[g] != kOutside && om < (unsigned)M) store_agent(ws + (size_t)split * MN + (ooff[g] >> 2), v[g]);
+    // every store of this workgroup has completed at device scope before it counts in
+    partial_stores_done();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int old = __hip_atomic_fetch_add(&counters[rem], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *s_last = (old == split_k - 1);
+    }
+    __syncthreads();
+    if (!*s_last) return true;
+#pragma unroll
+    for (int g = 0; g < TN; ++g) {
+        if (ooff[g] != kOutside && om < (unsigned)M) {
+            const float* src = ws + (ooff[g] >> 2);
+            float sum = 0.0f;
+            for (int s0 = 0; s0 < split_k; s0 += 4) {
+                float p[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) p[j] = load_agent(src + (size_t)min(s0 + j, split_k - 1) * MN);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (s0 + j < split_k) sum = (s0 + j == 0) ? p[j] : sum + p[j];
+            }
+            ep.finish(sum, ooff[g], om * 4u, e_res[g], e_bias, e_sh2);
+        }
+    }
+    if (threadIdx.x == 0)  // ready for the next run
+        __hip_atomic_store(&counters[rem], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return true;
 }
 

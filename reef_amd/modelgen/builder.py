@@ -168,6 +168,8 @@ class GraphBuilder:
         act2 = dual_act or ACT_NONE
         t = force or tiling.choose(M, N, K, fused=fused_reduce, pointwise=(kh, kw) == (1, 1),
                                    taps=kh * kw, direct=tiling.direct_ok(cin, kh, kw))
+        if t.get("fused"):
+            fused_reduce = True       # the measured table asks for the split folded into the launch
         flops = 2 * M * N * K
         self.flops += flops
         nbytes = 4 * (x.size + M * K + M * N + (M if bias else 0) + (M * N if residual is not None else 0)
@@ -175,8 +177,8 @@ class GraphBuilder:
         base = [cin, H, W, cout, Ho, Wo, kh, kw, sh, sw, ph, pw]
         # loader family: direct (only with its own tile), pointwise (1x1/s1/p0, N % 4 == 0),
         # unaligned (K % 4 != 0), general
-        if t["tile"] == tiling.DIRECT_TILE:
-            assert tiling.direct_ok(cin, kh, kw) and not fused_reduce, (cin, kh, kw)
+        if t["tile"] in tiling.DIRECT_TILES:
+            assert tiling.direct_ok(cin, kh, kw, t["tile"]), (cin, kh, kw, t["tile"])
             assert t["k_chunk"] % (kh * kw * (8 if kh * kw == 1 else 1)) == 0
             mode, fam = 3, "d%d_" % (kh * kw)
         elif (kh, kw, sh, sw, ph, pw) == (1, 1, 1, 1, 0, 0) and N % 4 == 0 and K % 4 == 0:

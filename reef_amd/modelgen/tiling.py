@@ -26,9 +26,13 @@ TILES = {
     # direct family (reef_conv2d_d<taps>_16x16k4): never picked by the analytic model, only
     # through the measured table or an explicit request
     "16x16k4": (9, 16, 16, 0.40, 2),
+    "16x32k4": (10, 16, 32, 0.40, 2),
+    "16x64k4": (11, 16, 64, 0.40, 2),
 }
 DIRECT_TILE = "16x16k4"
+DIRECT_TILES = ("16x16k4", "16x32k4", "16x64k4")
 DIRECT_TAPS = (1, 3, 7, 9)    # filter sizes kh*kw the direct family is compiled for
+DIRECT_WIDE_TAPS = (1, 9)     # ... and those that also have the 32- and 64-pixel wide tiles
 # wavefronts that share one output block and split K inside the workgroup
 KW = {"32x32k4": 4, "64x32k2": 2, "32x64k2": 2}
 GEMM_TILES = ("128x128", "64x64", "32x128", "32x32k4", "64x32k2")
@@ -37,15 +41,17 @@ GEMM_TILES = ("128x128", "64x64", "32x128", "32x32k4", "64x32k2")
 def step_k(tile, taps=1):
     """k values a workgroup consumes per step of its K loop (taps = kh*kw, direct family only:
     a step is 16 channels of a filter with taps > 1, 128 channels of a 1x1 filter)."""
-    if tile == DIRECT_TILE:
+    if tile in DIRECT_TILES:
         return 128 if taps == 1 else 16 * taps
     return BK * KW.get(tile, 1)
 
 
-def direct_ok(cin, kh, kw):
-    """Whether the direct family has a kernel for this filter."""
+def direct_ok(cin, kh, kw, tile=DIRECT_TILE):
+    """Whether the direct family has a kernel for this filter (and tile)."""
     taps = kh * kw
-    return taps in DIRECT_TAPS and (taps > 1 or cin % 8 == 0)
+    if taps not in (DIRECT_TAPS if tile == DIRECT_TILE else DIRECT_WIDE_TAPS):
+        return False
+    return taps > 1 or cin % 8 == 0
 
 
 def forced(tile, M, N, K, split=1, taps=1):
@@ -79,12 +85,14 @@ def choose(M, N, K, allow_split=True, tiles=None, max_split=32, fused=True, poin
     that names the direct tile counts only if the caller says the filter qualifies."""
     if allow_split and tiles is None and not fused:
         hit = TUNED.get((M, N, K, 1 if pointwise else 0))
-        if hit is not None and (hit[0] != DIRECT_TILE or direct):
-            t = forced(hit[0], M, N, K, hit[1], taps)
+        if hit is not None and (hit[0] not in DIRECT_TILES or direct):
+            # a negative split factor in the table: the split is folded inside the launch
+            t = forced(hit[0], M, N, K, abs(hit[1]), taps)
             t["est_us"] = hit[2]
+            t["fused"] = hit[1] < 0
             return t
     best = None
-    for name in (tiles or [t for t in TILES if t != DIRECT_TILE]):
+    for name in (tiles or [t for t in TILES if t not in DIRECT_TILES]):
         tid, bm, bn, eff, occ = TILES[name]
         m_tiles, n_tiles = math.ceil(M / bm), math.ceil(N / bn)
         nt = m_tiles * n_tiles
@@ -114,8 +122,9 @@ def choose(M, N, K, allow_split=True, tiles=None, max_split=32, fused=True, poin
 
 
 def lds_bytes(tile):
-    if tile == DIRECT_TILE:
-        return 4 * 320 * 4 + 16     # four partial 16x16 tiles (skewed rows) + the leave flag
+    if tile in DIRECT_TILES:
+        # four wavefronts x BN/16 partial 16x16 tiles (skewed rows) + the leave / last-arrival flags
+        return 4 * (TILES[tile][2] // 16) * 320 * 4 + 16
     _, bm, bn, _, _ = TILES[tile]
     bk = step_k(tile)
     a = bm * (bk + 4)

@@ -47,8 +47,9 @@ def test_conv_tiles(tmp_path, tile, case):
     kh, kw = (k, k) if isinstance(k, int) else k
     ph, pw = (p, p) if isinstance(p, int) else p
     Ho, Wo = (H + 2 * ph - kh) // s + 1, (W + 2 * pw - kw) // s + 1
-    if tile == tiling.DIRECT_TILE and not tiling.direct_ok(cin, kh, kw):
-        pytest.skip("the direct family is compiled for 1x1 (Cin % 8 == 0) and 3-, 7-, 9-tap filters")
+    if tile in tiling.DIRECT_TILES and not tiling.direct_ok(cin, kh, kw, tile):
+        pytest.skip("the direct family is compiled for 1x1 (Cin % 8 == 0) and 3-, 7-, 9-tap filters, "
+                    "its wide tiles for 1 and 9 taps")
     y = g.conv2d(x, cout, k, s, p, bias=True, act=MB.ACT_RELU,
                  force=forced(tile, cout, Ho * Wo, cin * kh * kw, 1, kh * kw))
     g.mark_output(y)
@@ -114,31 +115,53 @@ def test_fused_split_k_equals_plain_split_k_bitwise(tmp_path, tile, split):
         exe.execute()
 
 
-@pytest.mark.parametrize("split", [1, 2])
-def test_conv_direct_family_epilogues(tmp_path, split):
-    """Direct-operand family (16x16 tiles, channels split over the wavefronts): every epilogue
-    form, a second output, a channel slice of a concatenation buffer, ragged M / N / Cin, and
-    a strided 1x1, each with and without split-K across workgroups."""
+@pytest.mark.parametrize("split,fused", [(1, False), (2, False), (2, True), (3, True)])
+@pytest.mark.parametrize("tile", list(tiling.DIRECT_TILES))
+def test_conv_direct_family_epilogues(tmp_path, tile, split, fused):
+    """Direct-operand family (16 x 16/32/64 tiles, channels split over the wavefronts): every
+    epilogue form, a second output, a channel slice of a concatenation buffer, ragged M / N / Cin,
+    and a strided 1x1; without split-K, with a separate reduce launch, and with the split folded
+    inside the launch.  The folded form must hold the same bits as the separate reduce (both
+    add the partial tiles in ascending split order), also on a second run (counters reset)."""
     cin, H, W, cout = 72, 13, 13, 88          # Cin % 16 != 0, M % 16 != 0, N = 169
     g = MB.GraphBuilder("d")
     x = g.input("data", (cin, H, W))
     res = g.input("res", (cout, H, W))
     M, N = cout, H * W
-    f9 = forced("16x16k4", M, N, cin * 9, split, 9)
-    f1 = forced("16x16k4", M, N, cin, split, 1)
-    g.conv2d(x, cout, 3, 1, 1, bias=True, act=MB.ACT_RELU, residual=res, force=f9)
-    g.conv2d(x, cout, 3, 1, 1, bias=False, act=MB.ACT_RELU, residual=res, affine=True, force=f9)
-    g.conv2d(x, cout, 3, 1, 1, bias=False, act=MB.ACT_NONE, residual=res, dual_act=MB.ACT_RELU, force=f9)
-    g.conv2d(x, cout, 1, 1, 0, bias=True, act=MB.ACT_RELU6, force=f1)
-    g.conv2d(x, cout, 1, 1, 0, bias=False, act=MB.ACT_NONE, residual=res, dual_act=MB.ACT_RELU, force=f1)
-    cat = g.temp((2 * cout, H, W))
-    g.conv2d(x, cout, 3, 1, 1, force=f9, out=cat, out_channel=0)
-    g.conv2d(x, cout, 1, 1, 0, force=f1, out=cat, out_channel=cout)
+    f9 = forced(tile, M, N, cin * 9, split, 9)
+    f1 = forced(tile, M, N, cin, split, 1)
     Ho = (H - 1) // 2 + 1
-    y = g.conv2d(x, cout, 1, 2, 0, force=forced("16x16k4", M, Ho * Ho, cin, split, 1))
-    g.mark_output(y)
+    fs = forced(tile, M, Ho * Ho, cin, split, 1)
+
+    def layers(fz):
+        g._np = 0          # same parameter names -> same seeded weights for every variant
+        outs = [g.conv2d(x, cout, 3, 1, 1, bias=True, act=MB.ACT_RELU, residual=res, force=f9, fused_reduce=fz),
+                g.conv2d(x, cout, 3, 1, 1, bias=False, act=MB.ACT_RELU, residual=res, affine=True, force=f9,
+                         fused_reduce=fz)]
+        outs += list(g.conv2d(x, cout, 3, 1, 1, bias=False, act=MB.ACT_NONE, residual=res,
+                              dual_act=MB.ACT_RELU, force=f9, fused_reduce=fz))
+        outs.append(g.conv2d(x, cout, 1, 1, 0, bias=True, act=MB.ACT_RELU6, force=f1, fused_reduce=fz))
+        outs += list(g.conv2d(x, cout, 1, 1, 0, bias=False, act=MB.ACT_NONE, residual=res,
+                              dual_act=MB.ACT_RELU, force=f1, fused_reduce=fz))
+        cat = g.temp((2 * cout, H, W))
+        g.conv2d(x, cout, 3, 1, 1, force=f9, out=cat, out_channel=0, fused_reduce=fz)
+        g.conv2d(x, cout, 1, 1, 0, force=f1, out=cat, out_channel=cout, fused_reduce=fz)
+        outs.append(cat)
+        outs.append(g.conv2d(x, cout, 1, 2, 0, force=fs, fused_reduce=fz))
+        return outs
+
+    first = layers(fused)
+    plain = layers(False) if fused else None
+    g.mark_output(first[-1])
+    seen = {}
+    g.params = [kv for kv in g.params if not (kv[0] in seen or seen.setdefault(kv[0], 0))]
     exe, orc, model = run_both(g, tmp_path, {"data": rnd(cin, H, W), "res": rnd(cout, H, W)})
-    compare_storages(exe, orc, model, what="direct family x%d" % split)
+    compare_storages(exe, orc, model, what="direct family %s x%d%s" % (tile, split, " fused" if fused else ""))
+    if fused:
+        for rerun in range(2):
+            for a, b in zip(first, plain):
+                np.testing.assert_array_equal(exe.get_data(a.idx, a.size), exe.get_data(b.idx, b.size))
+            exe.execute()
 
 
 def test_conv_auto_heuristic_shapes(tmp_path):

@@ -89,6 +89,28 @@ def test_resnet18_through_queue(dirs, qtype, mode):
     s.shutdown()
 
 
+def test_folded_split_k_stable_over_many_best_effort_runs(dirs):
+    """ResNet-50 holds convolutions whose split-K is folded inside the launch (partial tiles,
+    arrival counter, last workgroup adds them up).  Forty runs through a best-effort queue
+    (windowed stream, launches from the feeder thread) give the same bits as a solo run every
+    time: the partial tiles are complete before a workgroup counts itself in."""
+    import json
+    x = nets.image_input("resnet50", (3, 224, 224))
+    model = json.load(open(os.path.join(dirs["resnet50"], "resnet50.json")))
+    folded = [k for k in model["kernels"] if k["name"].startswith("reef_conv2d_d") and k["attrs"][12] & 16]
+    assert folded, "no convolution of this model folds its split-K; the test would prove nothing"
+    ref = solo_output(dirs["resnet50"], "resnet50", x)
+    s = B.Scheduler(B.MODE_REEF)
+    s.run()
+    mid = s.load_model(dirs["resnet50"], "resnet50")
+    s.bind_model_queue(s.create_queue(B.QUEUE_BE), mid)
+    assert s.set_input(mid, x, "data") == 0
+    for _ in range(40):
+        assert s.wait_task(s.new_task(mid)) == 0
+        np.testing.assert_array_equal(s.get_output(mid, 1000), ref)
+    s.shutdown()
+
+
 def test_preempt_restart_bit_identical(dirs):
     """scheduler.resnet18_param_preempt: a best-effort task is submitted, a real-time
     task arrives while it runs; the best-effort output must equal an uninterrupted
