@@ -156,7 +156,7 @@ int TransExecutor::proxy_class_of_level(int level) {
 int TransExecutor::proxy_level(int op, int tile, int mode, int taps) {
     if (op == REEF_OP_CONV2D) {
         if (mode == REEF_CONV_MODE_DIRECT)
-            return (tile == REEF_TILE_16x16k4 && (taps == 1 || taps == 9)) ? 1 : -1;
+            return ((tile == REEF_TILE_16x16k4 || tile == REEF_TILE_16x32k4) && (taps == 1 || taps == 9)) ? 1 : -1;
         if (mode != REEF_CONV_MODE_GENERAL && mode != REEF_CONV_MODE_POINTWISE) return -1;
         if (tile == REEF_TILE_64x64 || tile == REEF_TILE_128x32) return 1;
         if (tile == REEF_TILE_128x64) return 2;

@@ -237,7 +237,7 @@ REEF_ENTRY(multiply, OpMocked<true>)
 // occupancy classes that matter for this kernel set, <n> = wavefronts per SIMD:
 //   merge_framework_8  bandwidth-bound ops only                          (<= 64 registers)
 //   merge_framework_3  + conv (general, pointwise) tiles 64x64 / 128x32,
-//                        direct family with 1 and 9 taps                      (<= 168)
+//                        direct family with 1 and 9 taps, 16x16 and 16x32    (<= 168)
 //   merge_framework_2  + conv (general, pointwise) tile 128x64 and the
 //                        wave-split-K tiles                                   (<= 256)
 // Kernels outside these sets (the other tiles, the unaligned-K convolution, GEMM)
@@ -255,8 +255,13 @@ __device__ __forceinline__ void run_op(const ReefDkpSide& s, int task, char* sme
                 const int tile = d.attr[REEF_CONV_TILE];
                 if (d.attr[REEF_CONV_MODE] == REEF_CONV_MODE_DIRECT) {
                     const int taps = d.attr[REEF_CONV_KH] * d.attr[REEF_CONV_KW];
-                    if (taps == 1) OpConvDirect<1>::run(d, task, smem, np);
-                    else if (taps == 9) OpConvDirect<9>::run(d, task, smem, np);
+                    if (tile == REEF_TILE_16x16k4) {
+                        if (taps == 1) OpConvDirect<1>::run(d, task, smem, np);
+                        else if (taps == 9) OpConvDirect<9>::run(d, task, smem, np);
+                    } else if (tile == REEF_TILE_16x32k4) {
+                        if (taps == 1) OpConvDirect<1, 2>::run(d, task, smem, np);
+                        else if (taps == 9) OpConvDirect<9, 2>::run(d, task, smem, np);
+                    }
                 } else if (d.attr[REEF_CONV_MODE] == CONV_POINTWISE) {
                     if (tile == REEF_TILE_64x64) OpConv<Tile64x64, CONV_POINTWISE>::run(d, task, smem, np);
                     else if (tile == REEF_TILE_128x32) OpConv<Tile128x32, CONV_POINTWISE>::run(d, task, smem, np);

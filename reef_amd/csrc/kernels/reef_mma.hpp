@@ -741,7 +741,8 @@ struct DirectGeom {
     static constexpr int RC = R * CPL;           // A values per lane and step (x TN B values and MFMAs)
     static constexpr int STEP_C = 16 * CPL;      // channels a workgroup consumes per step
     static constexpr int LOADS = (RC / 4) + (RC % 4) + TN * RC;  // vector-memory instructions per step
-    static constexpr int NS = 60 / LOADS < 2 ? 2 : 60 / LOADS;   // steps of loads in flight per wavefront
+    // steps of loads in flight per wavefront: up to 60 load instructions, 2 to 6 steps
+    static constexpr int NS = 60 / LOADS < 2 ? 2 : (60 / LOADS > 6 ? 6 : 60 / LOADS);
 };
 
 // TN > 1 widens the tile along the pixels: every weight value a lane has loaded is multiplied
@@ -772,9 +773,14 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     const int split_k = a[REEF_CONV_SPLIT_K];
     const int n_tiles = a[REEF_CONV_N_TILES];
     const int tiles = a[REEF_CONV_M_TILES] * n_tiles;
+    const int flags = a[REEF_CONV_FLAGS];
+    const bool fused = split_k > 1 && (flags & REEF_F_FUSED_REDUCE);
+    const bool to_ws = split_k > 1 && !fused;   // plain split-K: partial tile to the workspace
     task = xcd_chunked(task, tiles * split_k);
-    const int split = task / tiles;
-    const int rem = task - split * tiles;
+    // Folded split: the workgroups of one tile are neighbours in the task order, so they run on
+    // one XCD and meet in its L2; otherwise split-major like the staged tiles.
+    const int split = fused ? task % split_k : task / tiles;
+    const int rem = fused ? task / split_k : task - split * tiles;
     const int mt = rem / n_tiles, nt = rem - mt * n_tiles;
     const int m0 = mt * 16, n0 = nt * TD::BN;
     const int c_chunk = a[REEF_CONV_K_CHUNK] / R;
@@ -783,9 +789,6 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     const int nsteps = (ce - cb + G::STEP_C - 1) / G::STEP_C;
     const unsigned HW4 = (unsigned)(H * W) * 4u;
     const unsigned MN4 = (unsigned)M * (unsigned)N * 4u;
-    const int flags = a[REEF_CONV_FLAGS];
-    const bool fused = split_k > 1 && (flags & REEF_F_FUSED_REDUCE);
-    const bool to_ws = split_k > 1 && !fused;   // plain split-K: partial tile to the workspace
 
     // epilogue operands of the TN output elements this thread writes (element g: row t / 16,
     // column 16 g + t % 16 of the tile), fetched ahead of the K loop
