@@ -173,7 +173,7 @@ enum {
  *   reef_conv2d_<tile>      general: im2col gather, needs K % 4 == 0
  *   reef_conv2d_pw_<tile>   pointwise: 1x1, stride 1, no padding, N % 4 == 0, K % 4 == 0
  *   reef_conv2d_u_<tile>    unaligned: im2col gather, any K
- *   reef_conv2d_d<R>_16x<BN>k4  direct: R = kh*kw taps compiled in (1, 3, 7, 9; BN = 32, 64 for 1 and 9); operands go from memory
+ *   reef_conv2d_d<R>_16x<BN>k4  direct: R = kh*kw taps compiled in (1, 3, 7, 9 for BN = 16, 32; 1, 9 for 16x64 and 32x32d4); operands go from memory
  *                           straight into 16x16x4 MFMAs, the four wavefronts split the input
  *                           channels.  d1 needs Cin % 8 == 0 (any stride); K_CHUNK is a multiple
  *                           of R (R > 1) or 8 (d1) and splits K on channel boundaries. */
@@ -198,6 +198,7 @@ enum {
     REEF_TILE_16x16k4 = 9,   /* direct family only */
     REEF_TILE_16x32k4 = 10,  /* direct family, 1 and 9 taps */
     REEF_TILE_16x64k4 = 11,  /* direct family, 1 and 9 taps */
+    REEF_TILE_32x32d4 = 12,  /* direct family, 1 and 9 taps (symbol suffix 32x32d4) */
     REEF_TILE_COUNT
 };
 

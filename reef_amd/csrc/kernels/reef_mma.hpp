@@ -727,41 +727,43 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
 // partial tiles are summed through LDS in wavefront order and thread t writes output element
 // (t / 16, t % 16), so stores are 64-byte runs along a row.  The sum order over k differs from
 // the tiled kernels (it is fixed, so results are reproducible run to run).
-template <int TN_>
+template <int TN_, int TM_ = 1>
 struct TileD16 {
-    static constexpr int TN = TN_;      // 16-pixel column groups per workgroup: the tile is 16 x 16 TN
-    static constexpr int BM = 16, BN = 16 * TN;
+    static constexpr int TN = TN_;      // 16-pixel column groups per workgroup
+    static constexpr int TM = TM_;      // 16-row groups per workgroup: the tile is 16 TM x 16 TN
+    static constexpr int BM = 16 * TM, BN = 16 * TN;
     static constexpr int PART = 320;    // floats per 16 x 16 partial tile in LDS (256 + row-group skew)
-    static constexpr int LDS_BYTES = 4 * TN * PART * 4 + 16;
+    static constexpr int SUBS = TM * TN;
+    static constexpr int LDS_BYTES = 4 * SUBS * PART * 4 + 16;
 };
 
-template <int R, int TN>
+template <int R, int TN, int TM = 1>
 struct DirectGeom {
     static constexpr int CPL = R == 1 ? 8 : 1;   // channels per k slot and step
     static constexpr int RC = R * CPL;           // A values per lane and step (x TN B values and MFMAs)
     static constexpr int STEP_C = 16 * CPL;      // channels a workgroup consumes per step
-    static constexpr int LOADS = (RC / 4) + (RC % 4) + TN * RC;  // vector-memory instructions per step
+    static constexpr int LOADS = TM * ((RC / 4) + (RC % 4)) + TN * RC;  // vector-memory instructions per step
     // steps of loads in flight per wavefront: up to 60 load instructions, 2 to 6 steps
     static constexpr int NS = 60 / LOADS < 2 ? 2 : (60 / LOADS > 6 ? 6 : 60 / LOADS);
 };
 
 // TN > 1 widens the tile along the pixels: every weight value a lane has loaded is multiplied
 // with TN pixel groups, so the weight rows -- the larger, cold operand -- are streamed by a
-// TN-th of the workgroups.  What a CU can pull from memory per microsecond is what bounds these
+// TN-th of the workgroups.  TM > 1 does the same along the output channels for the input values.  What a CU can pull from memory per microsecond is what bounds these
 // kernels at batch 1 (a lone workgroup on an idle device takes as long as 208 of them), so fewer,
 // wider tiles are combined with a split of K across workgroups to keep every CU busy with a
 // shorter stream; REEF_F_FUSED_REDUCE then folds the split inside this launch: a workgroup
 // stores its partial tile, counts itself in, and the last one to arrive for a tile adds the
 // partial tiles in ascending split order (fixed order, so the result does not depend on who is
 // last) and runs the epilogue.
-template <int R, int TN, class Poll>
+template <int R, int TN, int TM, class Poll>
 __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int task, char* smem_raw,
                                                    const Poll& poll) {
-    typedef DirectGeom<R, TN> G;
-    typedef TileD16<TN> TD;
+    typedef DirectGeom<R, TN, TM> G;
+    typedef TileD16<TN, TM> TD;
     constexpr int RC = G::RC, NS = G::NS;
     float* smem = (float*)smem_raw;
-    int* sflag = (int*)(smem + 4 * TN * TD::PART);
+    int* sflag = (int*)(smem + 4 * TD::SUBS * TD::PART);
     const ReefOpDesc& d = d_in;
     const int* a = d.attr;
     const int lane = threadIdx.x & 63, i16 = lane & 15, kq = lane >> 4;
@@ -782,7 +784,7 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     const int split = fused ? task % split_k : task / tiles;
     const int rem = fused ? task / split_k : task - split * tiles;
     const int mt = rem / n_tiles, nt = rem - mt * n_tiles;
-    const int m0 = mt * 16, n0 = nt * TD::BN;
+    const int m0 = mt * TD::BM, n0 = nt * TD::BN;
     const int c_chunk = a[REEF_CONV_K_CHUNK] / R;
     const int cb = split * c_chunk;
     const int ce = min(C, cb + c_chunk);
@@ -790,27 +792,37 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     const unsigned HW4 = (unsigned)(H * W) * 4u;
     const unsigned MN4 = (unsigned)M * (unsigned)N * 4u;
 
-    // epilogue operands of the TN output elements this thread writes (element g: row t / 16,
-    // column 16 g + t % 16 of the tile), fetched ahead of the K loop
+    // epilogue operands of the TM x TN output elements this thread writes (element (h, g): row
+    // 16 h + t / 16, column 16 g + t % 16 of the tile), fetched ahead of the K loop
     const int orow = threadIdx.x >> 4, ocol = threadIdx.x & 15;
-    const unsigned om = (unsigned)(m0 + orow);
-    unsigned ooff[TN];
+    unsigned om[TM], ooff[TM][TN];
 #pragma unroll
-    for (int g = 0; g < TN; ++g) {
-        const unsigned on = (unsigned)(n0 + 16 * g + ocol);
-        ooff[g] = on < (unsigned)N ? (om * (unsigned)N + on) * 4u : kOutside;
+    for (int h = 0; h < TM; ++h) {
+        om[h] = (unsigned)(m0 + 16 * h + orow);
+#pragma unroll
+        for (int g = 0; g < TN; ++g) {
+            const unsigned on = (unsigned)(n0 + 16 * g + ocol);
+            ooff[h][g] = on < (unsigned)N ? (om[h] * (unsigned)N + on) * 4u : kOutside;
+        }
     }
     ConvEpilogue ep;
-    float e_bias = 0.0f, e_sh2 = 0.0f, e_res[TN];
+    float e_bias[TM], e_sh2[TM], e_res[TM][TN];
 #pragma unroll
-    for (int g = 0; g < TN; ++g) e_res[g] = 0.0f;
+    for (int h = 0; h < TM; ++h) {
+        e_bias[h] = e_sh2[h] = 0.0f;
+#pragma unroll
+        for (int g = 0; g < TN; ++g) e_res[h][g] = 0.0f;
+    }
     if (!to_ws) {
         ep.init(d, flags, a[REEF_CONV_ACT], a[REEF_CONV_ACT2], M, MN4, (unsigned)a[REEF_CONV_DST_OFF] * 4u);
-        if (ep.has_bias) e_bias = buf_load(ep.bias, om * 4u);
-        if (ep.has_dual) e_sh2 = buf_load(ep.shift2, om * 4u);
-        if (ep.has_res) {
 #pragma unroll
-            for (int g = 0; g < TN; ++g) e_res[g] = buf_load(ep.res, ooff[g]);
+        for (int h = 0; h < TM; ++h) {
+            if (ep.has_bias) e_bias[h] = buf_load(ep.bias, om[h] * 4u);
+            if (ep.has_dual) e_sh2[h] = buf_load(ep.shift2, om[h] * 4u);
+            if (ep.has_res) {
+#pragma unroll
+                for (int g = 0; g < TN; ++g) e_res[h][g] = buf_load(ep.res, ooff[h][g]);
+            }
         }
     }
 
@@ -818,7 +830,10 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     const rsrc_t rs_a = make_rsrc(d.ptr[1], (unsigned)M * (unsigned)K * 4u);
     const rsrc_t rs_b = make_rsrc(d.ptr[0], (unsigned)C * HW4);
     const int lane_c = cb + (wave * 4 + kq) * G::CPL;     // first channel of this lane's k slot
-    const unsigned va = ((unsigned)(m0 + i16) * (unsigned)K + (unsigned)(lane_c * R)) * 4u;
+    unsigned va[TM];
+#pragma unroll
+    for (int h = 0; h < TM; ++h)
+        va[h] = ((unsigned)(m0 + 16 * h + i16) * (unsigned)K + (unsigned)(lane_c * R)) * 4u;
     unsigned vb[TN][R];
     {
         const int kw_ = a[REEF_CONV_KW];
@@ -839,23 +854,27 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     // steps this lane's k slot stays inside the channel range of the split
     const int lane_steps = lane_c < ce ? (ce - lane_c + G::STEP_C - 1) / G::STEP_C : 0;
 
-    float ra[NS][RC], rb[NS][TN][RC];
+    float ra[NS][TM][RC], rb[NS][TN][RC];
     auto load_step = [&](int s, int step) {
         // offsets are below kOutside (a power of two), so or-ing it in moves them outside
         const unsigned outm = step < lane_steps ? 0u : kOutside;
         const unsigned sa = (unsigned)step * (unsigned)(G::STEP_C * R) * 4u;   // uniform
         const unsigned sb = (unsigned)step * (unsigned)G::STEP_C * HW4;         // uniform
-        const unsigned oa = va | outm;
 #pragma unroll
-        for (int q = 0; q < RC / 4; ++q) {
-            const f32x4 v = __builtin_bit_cast(
-                f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, (int)(oa + 16u * q), (int)sa, 0));
-            ra[s][4 * q] = v[0]; ra[s][4 * q + 1] = v[1]; ra[s][4 * q + 2] = v[2]; ra[s][4 * q + 3] = v[3];
+        for (int h = 0; h < TM; ++h) {
+            const unsigned oa = va[h] | outm;
+#pragma unroll
+            for (int q = 0; q < RC / 4; ++q) {
+                const f32x4 v = __builtin_bit_cast(
+                    f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, (int)(oa + 16u * q), (int)sa, 0));
+                ra[s][h][4 * q] = v[0]; ra[s][h][4 * q + 1] = v[1];
+                ra[s][h][4 * q + 2] = v[2]; ra[s][h][4 * q + 3] = v[3];
+            }
+#pragma unroll
+            for (int q = RC / 4 * 4; q < RC; ++q)
+                ra[s][h][q] = __builtin_bit_cast(
+                    float, __builtin_amdgcn_raw_buffer_load_b32(rs_a, (int)(oa + 4u * q), (int)sa, 0));
         }
-#pragma unroll
-        for (int q = RC / 4 * 4; q < RC; ++q)
-            ra[s][q] = __builtin_bit_cast(
-                float, __builtin_amdgcn_raw_buffer_load_b32(rs_a, (int)(oa + 4u * q), (int)sa, 0));
 #pragma unroll
         for (int g = 0; g < TN; ++g)
 #pragma unroll
@@ -882,18 +901,23 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     // Whole groups of NS steps with no condition inside (a loop with per-step conditions gets
     // reordered around the loads), then the remaining steps, whose loads are already under way.
     // Two accumulators per pixel group, so consecutive MFMAs never depend on each other.
-    f32x4 acc[TN][2];
+    f32x4 acc[TM][TN][2];
 #pragma unroll
-    for (int g = 0; g < TN; ++g) {
-        acc[g][0] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-        acc[g][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    }
+    for (int h = 0; h < TM; ++h)
+#pragma unroll
+        for (int g = 0; g < TN; ++g) {
+            acc[h][g][0] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            acc[h][g][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
     auto mma_stage = [&](int s) {
 #pragma unroll
         for (int q = 0; q < RC; ++q)
 #pragma unroll
-            for (int g = 0; g < TN; ++g)
-                acc[g][q & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[s][q], rb[s][g][q], acc[g][q & 1], 0, 0, 0);
+            for (int h = 0; h < TM; ++h)
+#pragma unroll
+                for (int g = 0; g < TN; ++g)
+                    acc[h][g][q & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[s][h][q], rb[s][g][q],
+                                                                            acc[h][g][q & 1], 0, 0, 0);
     };
     int pf = 0;
     int it = 0;
@@ -925,30 +949,40 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
 
     // partial tiles of this wavefront -> LDS; element j of a lane is row 4 * (lane / 16) + j.
     // Each group of four rows is skewed by 16 floats so the four k slots write to different banks.
-    float* part = smem + wave * (TN * TD::PART);
+    float* part = smem + wave * (TD::SUBS * TD::PART);
 #pragma unroll
-    for (int g = 0; g < TN; ++g)
+    for (int h = 0; h < TM; ++h)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            part[g * TD::PART + (5 * kq + j) * 16 + i16] = acc[g][0][j] + acc[g][1][j];
+        for (int g = 0; g < TN; ++g)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                part[(h * TN + g) * TD::PART + (5 * kq + j) * 16 + i16] = acc[h][g][0][j] + acc[h][g][1][j];
     __syncthreads();
     if (Poll::enabled && *sflag) return false;
     const float* mine = smem + threadIdx.x + (threadIdx.x >> 6) * 16;
-    float v[TN];
+    constexpr int WSTRIDE = TD::SUBS * TD::PART;   // one wavefront's partial tiles
+    float v[TM][TN];
 #pragma unroll
-    for (int g = 0; g < TN; ++g) {
-        const float* e = mine + g * TD::PART;
-        v[g] = ((e[0] + e[TN * TD::PART]) + e[2 * TN * TD::PART]) + e[3 * TN * TD::PART];
-    }
+    for (int h = 0; h < TM; ++h)
+#pragma unroll
+        for (int g = 0; g < TN; ++g) {
+            const float* e = mine + (h * TN + g) * TD::PART;
+            v[h][g] = ((e[0] + e[WSTRIDE]) + e[2 * WSTRIDE]) + e[3 * WSTRIDE];
+        }
     if (to_ws) {
         const rsrc_t ws = make_rsrc((const float*)d.ptr[2] + (size_t)split * M * N, MN4);
 #pragma unroll
-        for (int g = 0; g < TN; ++g) buf_store(ws, ooff[g], v[g]);
+        for (int h = 0; h < TM; ++h)
+#pragma unroll
+            for (int g = 0; g < TN; ++g) buf_store(ws, ooff[h][g], v[h][g]);
         return true;
     }
     if (!fused) {
 #pragma unroll
-        for (int g = 0; g < TN; ++g) ep.finish(v[g], ooff[g], om * 4u, e_res[g], e_bias, e_sh2);
+        for (int h = 0; h < TM; ++h)
+#pragma unroll
+            for (int g = 0; g < TN; ++g)
+                ep.finish(v[h][g], ooff[h][g], om[h] * 4u, e_res[h][g], e_bias[h], e_sh2[h]);
         return true;
     }
 
@@ -958,8 +992,11 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     int* counters = (int*)d.ptr[ep.next + 1] + a[REEF_CONV_SYNC_OFF];
     int* s_last = sflag + 1;
 #pragma unroll
-    for (int g = 0; g < TN; ++g)
-        if (ooff[g] != kOutside && om < (unsigned)M) store_agent(ws + (size_t)split * MN + (ooff[g] >> 2), v[g]);
+    for (int h = 0; h < TM; ++h)
+#pragma unroll
+        for (int g = 0; g < TN; ++g)
+            if (ooff[h][g] != kOutside && om[h] < (unsigned)M)
+                store_agent(ws + (size_t)split * MN + (ooff[h][g] >> 2), v[h][g]);
     // every store of this workgroup has completed at device scope before it counts in
     partial_stores_done();
     __syncthreads();
@@ -970,21 +1007,23 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     __syncthreads();
     if (!*s_last) return true;
 #pragma unroll
-    for (int g = 0; g < TN; ++g) {
-        if (ooff[g] != kOutside && om < (unsigned)M) {
-            const float* src = ws + (ooff[g] >> 2);
-            float sum = 0.0f;
-            for (int s0 = 0; s0 < split_k; s0 += 4) {
-                float p[4];
+    for (int h = 0; h < TM; ++h)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) p[j] = load_agent(src + (size_t)min(s0 + j, split_k - 1) * MN);
+        for (int g = 0; g < TN; ++g) {
+            if (ooff[h][g] != kOutside && om[h] < (unsigned)M) {
+                const float* src = ws + (ooff[h][g] >> 2);
+                float sum = 0.0f;
+                for (int s0 = 0; s0 < split_k; s0 += 4) {
+                    float p[4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    if (s0 + j < split_k) sum = (s0 + j == 0) ? p[j] : sum + p[j];
+                    for (int j = 0; j < 4; ++j) p[j] = load_agent(src + (size_t)min(s0 + j, split_k - 1) * MN);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (s0 + j < split_k) sum = (s0 + j == 0) ? p[j] : sum + p[j];
+                }
+                ep.finish(sum, ooff[h][g], om[h] * 4u, e_res[h][g], e_bias[h], e_sh2[h]);
             }
-            ep.finish(sum, ooff[g], om * 4u, e_res[g], e_bias, e_sh2);
         }
-    }
     if (threadIdx.x == 0)  // ready for the next run
         __hip_atomic_store(&counters[rem], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return true;

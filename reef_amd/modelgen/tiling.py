@@ -28,11 +28,12 @@ TILES = {
     "16x16k4": (9, 16, 16, 0.40, 2),
     "16x32k4": (10, 16, 32, 0.40, 2),
     "16x64k4": (11, 16, 64, 0.40, 2),
+    "32x32d4": (12, 32, 32, 0.40, 2),   # direct; the name differs from the staged 32x32k4
 }
 DIRECT_TILE = "16x16k4"
-DIRECT_TILES = ("16x16k4", "16x32k4", "16x64k4")
-DIRECT_TAPS = (1, 3, 7, 9)    # filter sizes kh*kw the direct family is compiled for
-DIRECT_WIDE_TAPS = (1, 9)     # ... and those that also have the 32- and 64-pixel wide tiles
+DIRECT_TILES = ("16x16k4", "16x32k4", "16x64k4", "32x32d4")
+# filter sizes kh*kw each direct tile is compiled for
+DIRECT_TAPS = {"16x16k4": (1, 3, 7, 9), "16x32k4": (1, 3, 7, 9), "16x64k4": (1, 9), "32x32d4": (1, 9)}
 # wavefronts that share one output block and split K inside the workgroup
 KW = {"32x32k4": 4, "64x32k2": 2, "32x64k2": 2}
 GEMM_TILES = ("128x128", "64x64", "32x128", "32x32k4", "64x32k2")
@@ -49,7 +50,7 @@ def step_k(tile, taps=1):
 def direct_ok(cin, kh, kw, tile=DIRECT_TILE):
     """Whether the direct family has a kernel for this filter (and tile)."""
     taps = kh * kw
-    if taps not in (DIRECT_TAPS if tile == DIRECT_TILE else DIRECT_WIDE_TAPS):
+    if taps not in DIRECT_TAPS[tile]:
         return False
     return taps > 1 or cin % 8 == 0
 
@@ -123,8 +124,8 @@ def choose(M, N, K, allow_split=True, tiles=None, max_split=32, fused=True, poin
 
 def lds_bytes(tile):
     if tile in DIRECT_TILES:
-        # four wavefronts x BN/16 partial 16x16 tiles (skewed rows) + the leave / last-arrival flags
-        return 4 * (TILES[tile][2] // 16) * 320 * 4 + 16
+        # four wavefronts x (BM/16)(BN/16) partial 16x16 tiles (skewed rows) + leave / last-arrival flags
+        return 4 * (TILES[tile][1] // 16) * (TILES[tile][2] // 16) * 320 * 4 + 16
     _, bm, bn, _, _ = TILES[tile]
     bk = step_k(tile)
     a = bm * (bk + 4)

@@ -253,6 +253,10 @@ def test_direct_tile_geometry():
     f = tiling.forced("16x16k4", 512, 49, 1024, 3, 1)
     assert f["k_chunk"] % 128 == 0 and f["split_k"] * f["k_chunk"] >= 1024
     assert tiling.direct_ok(256, 3, 3) and tiling.direct_ok(64, 1, 1) and tiling.direct_ok(24, 1, 7)
+    assert tiling.direct_ok(24, 1, 7, "16x32k4") and not tiling.direct_ok(24, 1, 7, "16x64k4")
+    f = tiling.forced("32x32d4", 256, 196, 2304, 4, 9)
+    assert (f["m_tiles"], f["n_tiles"], f["split_k"], f["tasks"]) == (8, 7, 4, 224)
+    assert tiling.lds_bytes("32x32d4") == 4 * 4 * 320 * 4 + 16
     assert not tiling.direct_ok(3, 7, 7) and not tiling.direct_ok(20, 1, 1) and not tiling.direct_ok(16, 5, 5)
     # the analytic model never picks the direct tile; only the measured table may, and only
     # when the caller vouches for the filter
