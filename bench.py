@@ -142,7 +142,7 @@ def summarize(r, sched, n_be):
 
 
 def corun(models, rt_name, be_name, n_be, mode, requests, warmup, wait_sync=True, solo=True,
-          dkp_slack=None):
+          dkp_slack=None, interval_us=MEAN_INTERVAL_US):
     """One scheduler, one real-time model, n_be best-effort clients of one model."""
     from reef_amd import binding as B
     s = B.Scheduler(mode)
@@ -167,11 +167,11 @@ def corun(models, rt_name, be_name, n_be, mode, requests, warmup, wait_sync=True
                     B.MODE_RESET: "Reset (reset-based preemption only)"}[mode],
            "rt_model": g_rt.name, "be_model": g_be.name, "be_clients": n_be}
     if solo:
-        r0 = s.run_load(rt, [], requests, warmup=warmup, mean_interval_us=MEAN_INTERVAL_US, seed=SEED)
+        r0 = s.run_load(rt, [], requests, warmup=warmup, mean_interval_us=interval_us, seed=SEED)
         out["solo"] = summarize(r0, s, 0)
     rb = s.run_load(rt, bes, 0, be_only_ms=1500)
     out["be_only_inferences_per_s"] = round(float(rb["be_completed"].sum()) / rb["span_s"], 2)
-    r1 = s.run_load(rt, bes, requests, warmup=warmup, mean_interval_us=MEAN_INTERVAL_US, seed=SEED)
+    r1 = s.run_load(rt, bes, requests, warmup=warmup, mean_interval_us=interval_us, seed=SEED)
     out["loaded"] = summarize(r1, s, n_be)
     ps = s.preempt_samples()
     ps = ps[-(requests):] if len(ps) > requests else ps
@@ -196,7 +196,9 @@ def main():
     ap.add_argument("--steps", type=int, default=400, help="recorded real-time requests")
     ap.add_argument("--warmup", type=int, default=40, help="real-time requests before recording")
     ap.add_argument("--kernel-iters", type=int, default=20)
-    ap.add_argument("--configs", default="3,4,5", help="co-location scenarios to run (3 is the headline)")
+    ap.add_argument("--configs", default="3,4,5",
+                    help="co-location scenarios to run (3 is the headline; 6 = dynamic kernel padding under "
+                         "a real-time request every 2 ms, not in the default set)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--solo-only", action="store_true",
                     help="only the solo ResNet-152 executor part (whole-model and per-kernel timing); "
@@ -219,7 +221,7 @@ def main():
     names = ["resnet152"] if args.solo_only else ["resnet152", "densenet201"]
     if args.solo_only:
         configs = []
-    if 4 in configs:
+    if 4 in configs or 6 in configs:
         names.append("mobilenetv2")
     if 5 in configs:
         names += ["inceptionv3", "bert_base"]
@@ -339,6 +341,17 @@ def main():
     if 5 in configs:
         k = max(args.steps // 2, 50)
         out["corun_inceptionv3_2x_bert"] = corun(models, "inceptionv3", "bert_base", 2, B.MODE_REEF, k, 20)
+    if 6 in configs:
+        # dynamic kernel padding where it can matter: real-time requests every 2 ms on average
+        # keep the device busy about three quarters of the time
+        k = max(args.steps, 200)
+        out["corun_dkp_high_rt_load"] = {
+            "rt_mean_interval_us": 2000.0,
+            "reef_slack50": corun(models, "resnet152", "mobilenetv2", 1, B.MODE_REEF, k, 20, interval_us=2000.0),
+            "reef_slack100": corun(models, "resnet152", "mobilenetv2", 1, B.MODE_REEF, k, 20, solo=False,
+                                   dkp_slack=100, interval_us=2000.0),
+            "reset": corun(models, "resnet152", "mobilenetv2", 1, B.MODE_RESET, k, 20, solo=False,
+                           interval_us=2000.0)}
     if not args.no_cpu:
         cb, orc = cpu_baseline(d, g.name, x)
         out["cpu_baseline"] = cb
