@@ -712,10 +712,10 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
 // ---- reef_conv2d_d<R>: operands straight from memory into the matrix cores ----------------
 // A batch-1 layer is latency bound: every weight is used once per inference, so each K step of
 // the tiled kernels above waits a full memory round trip (global -> registers -> LDS -> barrier).
-// This family removes the staging.  A workgroup owns a 16 x 16 output tile and its four
-// wavefronts split the input channels; v_mfma_f32_16x16x4f32 takes one A value (row = lane % 16,
-// k = lane / 16) and one B value (column = lane % 16, k = lane / 16) per lane, which a lane can
-// load directly:
+// This family removes the staging.  A workgroup owns a 16 TM x 16 TN output tile (16 x 16 in the
+// basic form) and its four wavefronts split the input channels; v_mfma_f32_16x16x4f32 takes one
+// A value (row = lane % 16, k = lane / 16) and one B value (column = lane % 16, k = lane / 16)
+// per lane, which a lane can load directly:
 //   R > 1 (R = kh * kw taps): k slot kq = lane / 16 is input channel c + kq; the lane loads the
 //          R contiguous weights W[m][c + kq][0..R) and the R taps in[c + kq][iy(t)][ix(t)] of
 //          its output pixel; MFMA t multiplies tap t of four channels.  Tap offsets and their
@@ -723,9 +723,9 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
 //   R = 1: k slot kq covers eight channels c + 8 kq .. + 8: two 128-bit weight loads and eight
 //          pixel loads; MFMA j multiplies channel j of each slot.  Any stride.
 // No LDS and no barrier inside the K loop, so NS steps of loads are in flight per wavefront
-// (a wavefront may have 63 vector-memory instructions outstanding; NS steps are 60 of them).  The four
-// partial tiles are summed through LDS in wavefront order and thread t writes output element
-// (t / 16, t % 16), so stores are 64-byte runs along a row.  The sum order over k differs from
+// (a wavefront may have 63 vector-memory instructions outstanding; NS steps are up to 60 of
+// them).  The four partial tiles are summed through LDS in wavefront order and thread t writes
+// output element (t / 16, t % 16) of every 16 x 16 sub-tile, so stores are 64-byte runs along a row.  The sum order over k differs from
 // the tiled kernels (it is fixed, so results are reproducible run to run).
 template <int TN_, int TM_ = 1>
 struct TileD16 {
@@ -749,8 +749,8 @@ struct DirectGeom {
 
 // TN > 1 widens the tile along the pixels: every weight value a lane has loaded is multiplied
 // with TN pixel groups, so the weight rows -- the larger, cold operand -- are streamed by a
-// TN-th of the workgroups.  TM > 1 does the same along the output channels for the input values.  What a CU can pull from memory per microsecond is what bounds these
-// kernels at batch 1 (a lone workgroup on an idle device takes as long as 208 of them), so fewer,
+// TN-th of the workgroups.  TM > 1 does the same along the output channels for the input values.
+// What a CU can pull from memory per microsecond is what bounds these kernels at batch 1 (a lone workgroup on an idle device takes as long as 208 of them), so fewer,
 // wider tiles are combined with a split of K across workgroups to keep every CU busy with a
 // shorter stream; REEF_F_FUSED_REDUCE then folds the split inside this launch: a workgroup
 // stores its partial tile, counts itself in, and the last one to arrive for a tile adds the
