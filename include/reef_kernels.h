@@ -168,6 +168,9 @@ enum {
 #define REEF_F_AFFINE 4 /* per-channel scale and shift after the sum */
 #define REEF_F_DUAL 8   /* second output out2 = act2(out + shift2[channel]) */
 #define REEF_F_FUSED_REDUCE 16 /* split-K folded inside the kernel by the last-arriving workgroup */
+#define REEF_F_PRE_ACT 32      /* the input is read through relu(in * pre_scale[c] + pre_shift[c]); the two
+                                  vectors follow the optional operands (before workspace and counters);
+                                  symbols reef_conv2d_p1_<tile>: 1x1 filters, no padding */
 
 /* Loader families of the convolution; the entry symbol carries the family:
  *   reef_conv2d_<tile>      general: im2col gather, needs K % 4 == 0
@@ -181,6 +184,7 @@ enum {
 #define REEF_CONV_MODE_POINTWISE 1
 #define REEF_CONV_MODE_UNALIGNED 2
 #define REEF_CONV_MODE_DIRECT 3
+#define REEF_CONV_MODE_DIRECT_PRE 4   /* direct, 1 tap, with REEF_F_PRE_ACT (reef_conv2d_p1_<tile>) */
 
 /* Tile configurations: BM x BN output tile per workgroup.  Plain tiles walk K in steps of
  * 32; a "k<n>" tile splits every step of 32*n k values across n wavefronts and sums the n

@@ -276,6 +276,14 @@ class GraphOracle:
             dst_off = a[22] if len(a) > 22 else 0  # a[21]: loader family (device detail)
             xin = P[0][:Cin * H * W].reshape(Cin, H, W)
             wgt = P[1][:Cout * Cin * kh * kw].reshape(Cout, Cin, kh, kw)
+            if flags & 32:
+                # pre-activation: the layer reads relu(in * scale[c] + shift[c]); the two vectors
+                # follow the optional operands (a plain split-K launch has none)
+                plain = split_k > 1 and not (flags & 16)
+                pos = 3 if plain else 3 + bool(flags & 1) + bool(flags & 2) + 2 * bool(flags & 4) + 2 * bool(flags & 8)
+                ps = P[pos][:Cin].astype(np.float64)[:, None, None]
+                pt = P[pos + 1][:Cin].astype(np.float64)[:, None, None]
+                xin = np.maximum(xin.astype(np.float64) * ps + pt, 0.0).astype(np.float32)
             if split_k > 1 and not (flags & 16):
                 # Plain split-K: the partial sums are an implementation detail of the
                 # device kernel; the oracle computes the whole convolution into slot 0

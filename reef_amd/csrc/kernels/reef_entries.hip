@@ -35,12 +35,12 @@ struct OpConv {
         return conv2d_body<T, MODE>(d, task, smem, p);
     }
 };
-template <int R, int TN = 1, int TM = 1>
+template <int R, int TN = 1, int TM = 1, bool PRE = false>
 struct OpConvDirect {
     static constexpr int LDS = TileD16<TN, TM>::LDS_BYTES;
     template <class P>
     static __device__ __forceinline__ bool run(const ReefOpDesc& d, int task, char* smem, const P& p) {
-        return conv2d_direct_body<R, TN, TM>(d, task, smem, p);
+        return conv2d_direct_body<R, TN, TM, PRE>(d, task, smem, p);
     }
 };
 template <class T, bool TRANS_B>
@@ -204,6 +204,9 @@ REEF_ENTRY(reef_conv2d_d1_16x64k4, OpConvDirect<1 REEF_COMMA 4>)
 REEF_ENTRY(reef_conv2d_d9_16x64k4, OpConvDirect<9 REEF_COMMA 4>)
 REEF_ENTRY(reef_conv2d_d3_16x32k4, OpConvDirect<3 REEF_COMMA 2>)
 REEF_ENTRY(reef_conv2d_d7_16x32k4, OpConvDirect<7 REEF_COMMA 2>)
+REEF_ENTRY(reef_conv2d_p1_16x16k4, OpConvDirect<1 REEF_COMMA 1 REEF_COMMA 1 REEF_COMMA true>)
+REEF_ENTRY(reef_conv2d_p1_16x32k4, OpConvDirect<1 REEF_COMMA 2 REEF_COMMA 1 REEF_COMMA true>)
+REEF_ENTRY(reef_conv2d_p1_32x32d4, OpConvDirect<1 REEF_COMMA 2 REEF_COMMA 2 REEF_COMMA true>)
 REEF_ENTRY(reef_conv2d_d1_32x32d4, OpConvDirect<1 REEF_COMMA 2 REEF_COMMA 2>)
 REEF_ENTRY(reef_conv2d_d9_32x32d4, OpConvDirect<9 REEF_COMMA 2 REEF_COMMA 2>)
 REEF_ENTRY(reef_gemm_nt_128x128, OpGemm<Tile128x128 REEF_COMMA true>)

@@ -737,12 +737,13 @@ struct TileD16 {
     static constexpr int LDS_BYTES = 4 * SUBS * PART * 4 + 16;
 };
 
-template <int R, int TN, int TM = 1>
+template <int R, int TN, int TM = 1, bool PRE = false>
 struct DirectGeom {
     static constexpr int CPL = R == 1 ? 8 : 1;   // channels per k slot and step
     static constexpr int RC = R * CPL;           // A values per lane and step (x TN B values and MFMAs)
     static constexpr int STEP_C = 16 * CPL;      // channels a workgroup consumes per step
-    static constexpr int LOADS = TM * ((RC / 4) + (RC % 4)) + TN * RC;  // vector-memory instructions per step
+    // vector-memory instructions per step (PRE: two 128-bit loads each of input scale and shift)
+    static constexpr int LOADS = TM * ((RC / 4) + (RC % 4)) + TN * RC + (PRE ? 4 : 0);
     // steps of loads in flight per wavefront: up to 60 load instructions, 2 to 6 steps
     static constexpr int NS = 60 / LOADS < 2 ? 2 : (60 / LOADS > 6 ? 6 : 60 / LOADS);
 };
@@ -756,10 +757,18 @@ struct DirectGeom {
 // stores its partial tile, counts itself in, and the last one to arrive for a tile adds the
 // partial tiles in ascending split order (fixed order, so the result does not depend on who is
 // last) and runs the epilogue.
-template <int R, int TN, int TM, class Poll>
+//
+// PRE (1-tap kernels only, symbols reef_conv2d_p1_*): the layer reads its input through a
+// per-channel scale, shift and ReLU -- the pre-activation of a DenseNet layer, which cannot be
+// folded into the producing convolution because every consumer of the concatenation has its own.
+// The eight input values a lane loads per step are eight consecutive channels, so their scales
+// and shifts are two 128-bit loads each; a channel past the split loads scale = shift = 0 and
+// contributes relu(0) = 0.  REEF_F_PRE_ACT; the two vectors follow the optional epilogue operands.
+template <int R, int TN, int TM, bool PRE, class Poll>
 __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int task, char* smem_raw,
                                                    const Poll& poll) {
-    typedef DirectGeom<R, TN, TM> G;
+    static_assert(!PRE || R == 1, "the pre-activation form exists for 1-tap filters only");
+    typedef DirectGeom<R, TN, TM, PRE> G;
     typedef TileD16<TN, TM> TD;
     constexpr int RC = G::RC, NS = G::NS;
     float* smem = (float*)smem_raw;
@@ -806,6 +815,7 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
         }
     }
     ConvEpilogue ep;
+    ep.next = 3;   // plain split-K launches carry no epilogue operands
     float e_bias[TM], e_sh2[TM], e_res[TM][TN];
 #pragma unroll
     for (int h = 0; h < TM; ++h) {
@@ -854,7 +864,15 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     // steps this lane's k slot stays inside the channel range of the split
     const int lane_steps = lane_c < ce ? (ce - lane_c + G::STEP_C - 1) / G::STEP_C : 0;
 
+    // operands that follow the optional epilogue operands: (pre-activation scale, shift), then
+    // (workspace, arrival counters) of a folded split
+    const int aux = ep.next + (PRE ? 2 : 0);
+    const rsrc_t rs_ps = make_rsrc(d.ptr[PRE ? ep.next : 0], (unsigned)C * 4u);
+    const rsrc_t rs_pt = make_rsrc(d.ptr[PRE ? ep.next + 1 : 0], (unsigned)C * 4u);
+    const unsigned vpre = (unsigned)lane_c * 4u;
+
     float ra[NS][TM][RC], rb[NS][TN][RC];
+    float rps[NS][PRE ? 8 : 1], rpt[NS][PRE ? 8 : 1];
     auto load_step = [&](int s, int step) {
         // offsets are below kOutside (a power of two), so or-ing it in moves them outside
         const unsigned outm = step < lane_steps ? 0u : kOutside;
@@ -874,6 +892,22 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
             for (int q = RC / 4 * 4; q < RC; ++q)
                 ra[s][h][q] = __builtin_bit_cast(
                     float, __builtin_amdgcn_raw_buffer_load_b32(rs_a, (int)(oa + 4u * q), (int)sa, 0));
+        }
+        if (PRE) {
+            const unsigned op = vpre | outm;
+            const unsigned sp = (unsigned)step * (unsigned)G::STEP_C * 4u;   // uniform
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const f32x4 sc = __builtin_bit_cast(
+                    f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_ps, (int)(op + 16u * q), (int)sp, 0));
+                const f32x4 sh = __builtin_bit_cast(
+                    f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_pt, (int)(op + 16u * q), (int)sp, 0));
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    rps[s][PRE ? 4 * q + e : 0] = sc[e];
+                    rpt[s][PRE ? 4 * q + e : 0] = sh[e];
+                }
+            }
         }
 #pragma unroll
         for (int g = 0; g < TN; ++g)
@@ -910,6 +944,13 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
             acc[h][g][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
         }
     auto mma_stage = [&](int s) {
+        if (PRE) {
+#pragma unroll
+            for (int g = 0; g < TN; ++g)
+#pragma unroll
+                for (int q = 0; q < RC; ++q)
+                    rb[s][g][q] = fmaxf(fmaf(rb[s][g][q], rps[s][PRE ? q : 0], rpt[s][PRE ? q : 0]), 0.0f);
+        }
 #pragma unroll
         for (int q = 0; q < RC; ++q)
 #pragma unroll
@@ -988,8 +1029,8 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
 
     // split-K folded inside the launch
     const size_t MN = (size_t)M * N;
-    float* ws = (float*)d.ptr[ep.next];
-    int* counters = (int*)d.ptr[ep.next + 1] + a[REEF_CONV_SYNC_OFF];
+    float* ws = (float*)d.ptr[aux];
+    int* counters = (int*)d.ptr[aux + 1] + a[REEF_CONV_SYNC_OFF];
     int* s_last = sflag + 1;
 #pragma unroll
     for (int h = 0; h < TM; ++h)

@@ -24,7 +24,7 @@ from . import rng, tiling
 from ..paths import code_object
 
 ACT_NONE, ACT_RELU, ACT_RELU6, ACT_GELU = 0, 1, 2, 3
-F_BIAS, F_RESIDUAL, F_AFFINE, F_DUAL, F_FUSED_REDUCE = 1, 2, 4, 8, 16
+F_BIAS, F_RESIDUAL, F_AFFINE, F_DUAL, F_FUSED_REDUCE, F_PRE_ACT = 1, 2, 4, 8, 16, 32
 WG = 256
 
 
@@ -121,8 +121,12 @@ class GraphBuilder:
         self.kernel_est_us.append(float(est_us))
 
     def conv2d(self, x, cout, k, stride=1, pad=0, bias=True, act=ACT_RELU, residual=None,
-               affine=False, force=None, dual_act=None, fused_reduce=None, out=None, out_channel=0):
+               affine=False, force=None, dual_act=None, fused_reduce=None, out=None, out_channel=0,
+               pre_act=False):
         """Fused conv + (residual) + (bias) + (scale, shift) + activation on MFMA.
+        pre_act: the layer reads its input through a per-channel scale, shift and ReLU of its own
+        (DenseNet pre-activation); folded into the convolution's input loads where a kernel for it
+        exists (1x1 filters on the direct tiles), a separate elementwise launch otherwise.
         dual_act: also emit out2 = dual_act(out + shift2[c]) and return (out, out2).
         fused_reduce: fold split-K inside the kernel (default: self.fused_reduce).
         out / out_channel: write into channels [out_channel, out_channel + cout) of an existing
@@ -170,6 +174,15 @@ class GraphBuilder:
                                    taps=kh * kw, direct=tiling.direct_ok(cin, kh, kw))
         if t.get("fused"):
             fused_reduce = True       # the measured table asks for the split folded into the launch
+        pre = []
+        if pre_act:
+            if (t["tile"] in tiling.PRE_ACT_TILES and (kh, kw, ph, pw) == (1, 1, 0, 0)
+                    and tiling.direct_ok(cin, kh, kw, t["tile"])):
+                ps = self.param((cin,), 0.1)
+                self.params[-1] = (self.params[-1][0], self.params[-1][1] + 1.0)   # scale ~ 1 + N(0, 0.1)
+                pre = [ps.idx, self.param((cin,), 0.01).idx]
+            else:
+                x = self.eltwise(x, scale=True, shift=True, act=ACT_RELU)
         flops = 2 * M * N * K
         self.flops += flops
         nbytes = 4 * (x.size + M * K + M * N + (M if bias else 0) + (M * N if residual is not None else 0)
@@ -180,7 +193,7 @@ class GraphBuilder:
         if t["tile"] in tiling.DIRECT_TILES:
             assert tiling.direct_ok(cin, kh, kw, t["tile"]), (cin, kh, kw, t["tile"])
             assert t["k_chunk"] % (kh * kw * (8 if kh * kw == 1 else 1)) == 0
-            mode, fam = 3, "d%d_" % (kh * kw)
+            mode, fam = (4, "p1_") if pre else (3, "d%d_" % (kh * kw))
         elif (kh, kw, sh, sw, ph, pw) == (1, 1, 1, 1, 0, 0) and N % 4 == 0 and K % 4 == 0:
             mode, fam = 1, "pw_"
         elif K % 4 != 0:
@@ -190,10 +203,13 @@ class GraphBuilder:
         kname = "reef_conv2d_" + fam + t["tile"]
         if out2 is not None:
             nbytes += 4 * (M * N + M)
+        if pre:
+            flags |= F_PRE_ACT
+            nbytes += 4 * 2 * cin
         if t["split_k"] == 1:
             attrs = base + [flags, act, t["tile_id"], 1, t["k_chunk"], t["m_tiles"], t["n_tiles"], act2,
                             0, mode, dst_off]
-            self._emit(kname, t["tasks"], [x.idx, w.idx, out.idx] + opt, attrs, "conv2d", flops,
+            self._emit(kname, t["tasks"], [x.idx, w.idx, out.idx] + opt + pre, attrs, "conv2d", flops,
                        nbytes, t["est_us"])
         elif fused_reduce:
             # workspace: split_k partial tensors; counters: one int per output tile in
@@ -202,16 +218,16 @@ class GraphBuilder:
             sync_idx, sync_off = self._sync_counters(t["m_tiles"] * t["n_tiles"])
             attrs = base + [flags | F_FUSED_REDUCE, act, t["tile_id"], t["split_k"], t["k_chunk"],
                             t["m_tiles"], t["n_tiles"], act2, sync_off, mode, dst_off]
-            self._emit(kname, t["tasks"], [x.idx, w.idx, out.idx] + opt + [ws.idx, sync_idx], attrs,
+            self._emit(kname, t["tasks"], [x.idx, w.idx, out.idx] + opt + pre + [ws.idx, sync_idx], attrs,
                        "conv2d", flops, nbytes, t["est_us"])
         else:
             ws = self.workspace(t["split_k"] * M * N)
-            attrs = base + [0, ACT_NONE, t["tile_id"], t["split_k"], t["k_chunk"], t["m_tiles"],
-                            t["n_tiles"], ACT_NONE, 0, mode, 0]
-            self._emit(kname, t["tasks"], [x.idx, w.idx, ws.idx], attrs, "conv2d", flops,
+            attrs = base + [F_PRE_ACT if pre else 0, ACT_NONE, t["tile_id"], t["split_k"], t["k_chunk"],
+                            t["m_tiles"], t["n_tiles"], ACT_NONE, 0, mode, 0]
+            self._emit(kname, t["tasks"], [x.idx, w.idx, ws.idx] + pre, attrs, "conv2d", flops,
                        4 * (x.size + M * K + t["split_k"] * M * N), t["est_us"])
             self._emit("reef_splitk_reduce", math.ceil(M * N / 1024), [ws.idx, out.idx] + opt,
-                       [M, N, t["split_k"], flags, act, act2, dst_off], "splitk_reduce", 0,
+                       [M, N, t["split_k"], flags & ~F_PRE_ACT, act, act2, dst_off], "splitk_reduce", 0,
                        4 * ((t["split_k"] + 1) * M * N), 2.0)
         return out if out2 is None else (out, out2)
 

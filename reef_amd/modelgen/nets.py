@@ -137,8 +137,9 @@ def mobilenet_v2(image=(3, 224, 224), classes=1000, name="mobilenetv2", seed=rng
 def densenet(blocks=(6, 12, 48, 32), growth=32, image=(3, 224, 224), classes=1000, name="densenet201",
              seed=rng.BASE_SEED):
     """DenseNet-BC (201: blocks 6/12/48/32, growth 32): every layer reads the running
-    concatenation through its own BN + ReLU (an elementwise scale/shift kernel, it cannot
-    be folded into a convolution because each consumer has its own statistics), then
+    concatenation through its own BN + ReLU (it cannot be folded into the producing
+    convolution because each consumer has its own statistics; it is folded into the input
+    loads of the consuming 1x1 convolution where a kernel for that exists), then
     1x1 -> 128 (+bias, ReLU) and 3x3 -> 32, which writes straight into its channel slice
     of the concatenation buffer."""
     g = GraphBuilder(name, seed)
@@ -154,14 +155,12 @@ def densenet(blocks=(6, 12, 48, 32), growth=32, image=(3, 224, 224), classes=100
         for li in range(n_layers):
             cur = c + li * growth
             view = type(x)(buf.idx, (cur, H, W))          # first `cur` channels of the buffer
-            a = g.eltwise(view, scale=True, shift=True, act=ACT_RELU)
-            y = g.conv2d(a, 4 * growth, 1, 1, 0, bias=True, act=ACT_RELU)
+            y = g.conv2d(view, 4 * growth, 1, 1, 0, bias=True, act=ACT_RELU, pre_act=True)
             g.conv2d(y, growth, 3, 1, 1, bias=False, act=ACT_NONE, out=buf, out_channel=cur)
         c = total
         x = buf
         if bi != len(blocks) - 1:
-            a = g.eltwise(x, scale=True, shift=True, act=ACT_RELU)
-            y = g.conv2d(a, c // 2, 1, 1, 0, bias=False, act=ACT_NONE)
+            y = g.conv2d(x, c // 2, 1, 1, 0, bias=False, act=ACT_NONE, pre_act=True)
             x = g.pool2d(y, 2, 2, 0, "avg")
             c = c // 2
     a = g.eltwise(x, scale=True, shift=True, act=ACT_RELU)

@@ -164,6 +164,32 @@ def test_conv_direct_family_epilogues(tmp_path, tile, split, fused):
             exe.execute()
 
 
+@pytest.mark.parametrize("split,fused", [(1, False), (2, False), (2, True)])
+@pytest.mark.parametrize("tile", list(tiling.PRE_ACT_TILES))
+def test_conv_pre_activation_folded_into_the_loads(tmp_path, tile, split, fused):
+    """1x1 convolution that reads its input through a per-channel scale, shift and ReLU (the
+    DenseNet pre-activation) inside its own loads: equals the oracle, which applies the
+    pre-activation first, for ragged M / N / Cin, with a residual and second output, into a slice
+    of a concatenation buffer, with plain and folded split-K."""
+    cin, H, W, cout = 200, 13, 13, 88         # Cin % 128 != 0, M % 16 != 0, N = 169
+    g = MB.GraphBuilder("p")
+    x = g.input("data", (cin, H, W))
+    res = g.input("res", (cout, H, W))
+    f = forced(tile, cout, H * W, cin, split, 1)
+    g.conv2d(x, cout, 1, 1, 0, bias=True, act=MB.ACT_RELU, force=f, fused_reduce=fused, pre_act=True)
+    g.conv2d(x, cout, 1, 1, 0, bias=False, act=MB.ACT_NONE, residual=res, dual_act=MB.ACT_RELU, force=f,
+             fused_reduce=fused, pre_act=True)
+    cat = g.temp((2 * cout, H, W))
+    g.conv2d(x, cout, 1, 1, 0, force=f, out=cat, out_channel=cout, fused_reduce=fused, pre_act=True)
+    # a filter the folded form does not cover falls back to a separate elementwise launch
+    y = g.conv2d(x, cout, 3, 1, 1, force=forced(tile, cout, H * W, cin * 9, 1, 9), pre_act=True)
+    g.mark_output(y)
+    names = [k["name"].split("#")[0] for k in g.kernels]
+    assert names.count("reef_conv2d_p1_" + tile) == 3 and names.count("reef_eltwise") == 1
+    exe, orc, model = run_both(g, tmp_path, {"data": rnd(cin, H, W), "res": rnd(cout, H, W)})
+    compare_storages(exe, orc, model, what="pre-activation %s x%d%s" % (tile, split, " fused" if fused else ""))
+
+
 def test_conv_auto_heuristic_shapes(tmp_path):
     """The layer shapes of ResNet-152 at reduced channel counts, tiles picked by the generator."""
     g = MB.GraphBuilder("h")
