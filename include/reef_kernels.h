@@ -272,8 +272,10 @@ enum { REEF_COPY_COUNT = 0, REEF_COPY_DST_OFF, REEF_COPY_NATTR };
  * ptr: in, out, bias(optional).  attr: d0, d1, d2, flags.  tasks = ceil(d0*d1*d2/1024). */
 enum { REEF_TR_D0 = 0, REEF_TR_D1, REEF_TR_D2, REEF_TR_FLAGS, REEF_TR_NATTR };
 
-/* ---- reef_gemm_nt_<tile> / reef_gemm_nn_<tile>: batched fp32 GEMM on MFMA ----
+/* ---- reef_gemm_nt_<tile> / reef_gemm_ntd_<tile> / reef_gemm_nn_<tile>: batched fp32 GEMM on MFMA ----
  * nt: trans_b = 1 (K, lda, ldb and the batch strides must be multiples of 4);
+ * ntd: trans_b = 1, operands straight from memory into 16x16x4 MFMAs (tiles 16x16k4, 16x32k4,
+ *      32x32d4; K a multiple of 8, lda, ldb and the batch strides multiples of 4);
  * nn: trans_b = 0 (K and lda multiples of 4).
  * C[b][m][n] = act(alpha * sum_k A[b][m][k] * B(b,k,n) (+bias[n]))
  * trans_b = 1: B stored [b][n][k] (dense layers, Q.K^T); 0: [b][k][n] (P.V).

@@ -51,6 +51,14 @@ struct OpGemm {
         return gemm_body<T, TRANS_B>(d, task, smem, p);
     }
 };
+template <int TM, int TN>
+struct OpGemmNtDirect {
+    static constexpr int LDS = TileD16<TN, TM>::LDS_BYTES;
+    template <class P>
+    static __device__ __forceinline__ bool run(const ReefOpDesc& d, int task, char* smem, const P& p) {
+        return gemm_nt_direct_body<TM, TN>(d, task, smem, p);
+    }
+};
 #define REEF_SIMPLE_OP(STRUCT, CALL)                                                            \
     struct STRUCT {                                                                             \
         static constexpr int LDS = 0;                                                           \
@@ -214,6 +222,9 @@ REEF_ENTRY(reef_gemm_nt_64x64, OpGemm<Tile64x64 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nt_32x128, OpGemm<Tile32x128 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nt_32x32k4, OpGemm<Tile32x32k4 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nt_64x32k2, OpGemm<Tile64x32k2 REEF_COMMA true>)
+REEF_ENTRY(reef_gemm_ntd_16x16k4, OpGemmNtDirect<1 REEF_COMMA 1>)
+REEF_ENTRY(reef_gemm_ntd_16x32k4, OpGemmNtDirect<1 REEF_COMMA 2>)
+REEF_ENTRY(reef_gemm_ntd_32x32d4, OpGemmNtDirect<2 REEF_COMMA 2>)
 REEF_ENTRY(reef_gemm_nn_128x128, OpGemm<Tile128x128 REEF_COMMA false>)
 REEF_ENTRY(reef_gemm_nn_64x64, OpGemm<Tile64x64 REEF_COMMA false>)
 REEF_ENTRY(reef_gemm_nn_32x128, OpGemm<Tile32x128 REEF_COMMA false>)

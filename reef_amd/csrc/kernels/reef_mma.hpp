@@ -1138,4 +1138,160 @@ __device__ __forceinline__ bool gemm_body(const ReefOpDesc& d, int task, char* s
     return true;
 }
 
+// ---- reef_gemm_ntd: C = act(alpha A B^T + bias) with both operands straight from memory -----
+// The direct scheme of reef_conv2d_d1 applied to a GEMM whose operands are both K-contiguous
+// (dense layers, Q K^T): a lane of the A side (row = lane % 16 of a 16-row group, k slot =
+// lane / 16) and a lane of the B side (column = lane % 16 of a 16-column group) each load the
+// eight consecutive k values of their slot with two 128-bit loads; MFMA j multiplies value j of
+// every slot.  The four wavefronts split K (a step is 128 k values), the partial tiles meet in
+// LDS, thread t writes element (t / 16, t % 16) of every 16 x 16 sub-tile.  K % 8 == 0, lda, ldb
+// and the batch strides multiples of 4.  No split of K across workgroups.
+template <int TM, int TN, class Poll>
+__device__ __forceinline__ bool gemm_nt_direct_body(const ReefOpDesc& d, int task, char* smem_raw,
+                                                    const Poll& poll) {
+    typedef TileD16<TN, TM> TD;
+    constexpr int LOADS = 2 * (TM + TN);
+    constexpr int NS = 60 / LOADS > 6 ? 6 : 60 / LOADS;
+    float* smem = (float*)smem_raw;
+    int* sflag = (int*)(smem + 4 * TD::SUBS * TD::PART);
+    const int* a = d.attr;
+    const int lane = threadIdx.x & 63, i16 = lane & 15, kq = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int M = a[REEF_GEMM_M], N = a[REEF_GEMM_N], K = a[REEF_GEMM_K];
+    const int n_tiles = a[REEF_GEMM_N_TILES];
+    const int tiles = a[REEF_GEMM_M_TILES] * n_tiles;
+    const int b = task / tiles;
+    const int rem = task - b * tiles;
+    const int mt = rem / n_tiles, nt = rem - mt * n_tiles;
+    const int m0 = mt * TD::BM, n0 = nt * TD::BN;
+    const unsigned lda = (unsigned)a[REEF_GEMM_LDA], ldb = (unsigned)a[REEF_GEMM_LDB],
+                   ldc = (unsigned)a[REEF_GEMM_LDC];
+    const rsrc_t rs_a = make_rsrc((const float*)d.ptr[0] + (size_t)b * a[REEF_GEMM_STRIDE_A],
+                                  ((unsigned)(M - 1) * lda + (unsigned)K) * 4u);
+    const rsrc_t rs_b = make_rsrc((const float*)d.ptr[1] + (size_t)b * a[REEF_GEMM_STRIDE_B],
+                                  ((unsigned)(N - 1) * ldb + (unsigned)K) * 4u);
+    const rsrc_t rs_c = make_rsrc((const float*)d.ptr[2] + (size_t)b * a[REEF_GEMM_STRIDE_C],
+                                  ((unsigned)(M - 1) * ldc + (unsigned)N) * 4u);
+    const bool has_bias = a[REEF_GEMM_FLAGS] & 1;
+    const rsrc_t rs_bias = make_rsrc(d.ptr[has_bias ? 3 : 2], (unsigned)N * 4u);
+
+    // the outputs of this thread and their bias, ahead of the K loop
+    const int orow = threadIdx.x >> 4, ocol = threadIdx.x & 15;
+    unsigned ooff[TM][TN];
+    float e_bias[TN];
+#pragma unroll
+    for (int g = 0; g < TN; ++g) {
+        const unsigned n = (unsigned)(n0 + 16 * g + ocol);
+        e_bias[g] = has_bias ? buf_load(rs_bias, n * 4u) : 0.0f;
+#pragma unroll
+        for (int h = 0; h < TM; ++h) {
+            const unsigned m = (unsigned)(m0 + 16 * h + orow);
+            ooff[h][g] = n < (unsigned)N ? (m * ldc + n) * 4u : kOutside;
+        }
+    }
+
+    const int lane_k = (wave * 4 + kq) * 8;          // first k of this lane's slot
+    const int nsteps = (K + 127) / 128;
+    const int lane_steps = lane_k < K ? (K - lane_k + 127) / 128 : 0;
+    unsigned va[TM], vb[TN];
+#pragma unroll
+    for (int h = 0; h < TM; ++h) va[h] = ((unsigned)(m0 + 16 * h + i16) * lda + (unsigned)lane_k) * 4u;
+#pragma unroll
+    for (int g = 0; g < TN; ++g) vb[g] = ((unsigned)(n0 + 16 * g + i16) * ldb + (unsigned)lane_k) * 4u;
+
+    float ra[NS][TM][8], rb[NS][TN][8];
+    auto load8 = [&](float (&dst)[8], rsrc_t rs, unsigned off, unsigned soff) {
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const f32x4 v = __builtin_bit_cast(
+                f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, (int)(off + 16u * q), (int)soff, 0));
+            dst[4 * q] = v[0]; dst[4 * q + 1] = v[1]; dst[4 * q + 2] = v[2]; dst[4 * q + 3] = v[3];
+        }
+    };
+    auto load_step = [&](int s, int step) {
+        const unsigned outm = step < lane_steps ? 0u : kOutside;
+        const unsigned so = (unsigned)step * 512u;   // 128 k values, uniform
+#pragma unroll
+        for (int h = 0; h < TM; ++h) load8(ra[s][h], rs_a, va[h] | outm, so);
+#pragma unroll
+        for (int g = 0; g < TN; ++g) load8(rb[s][g], rs_b, vb[g] | outm, so);
+    };
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        load_step(s, s);
+        asm volatile("" ::: "memory");
+    }
+    if (Poll::enabled) {
+        if (threadIdx.x == 0) *sflag = 0;
+        __syncthreads();
+    }
+    f32x4 acc[TM][TN][2];
+#pragma unroll
+    for (int h = 0; h < TM; ++h)
+#pragma unroll
+        for (int g = 0; g < TN; ++g) {
+            acc[h][g][0] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            acc[h][g][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    auto mma_stage = [&](int s) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+#pragma unroll
+            for (int h = 0; h < TM; ++h)
+#pragma unroll
+                for (int g = 0; g < TN; ++g)
+                    acc[h][g][q & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[s][h][q], rb[s][g][q],
+                                                                            acc[h][g][q & 1], 0, 0, 0);
+    };
+    int pf = 0, it = 0;
+    bool left = false;
+    for (; it + NS <= nsteps; it += NS) {
+        if (Poll::enabled) {
+            if (pf) {
+                *sflag = 1;
+                left = true;
+                break;
+            }
+            pf = poll.load();
+        }
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            mma_stage(s);
+            load_step(s, it + s + NS);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    if (!left) {
+#pragma unroll
+        for (int s = 0; s < NS - 1; ++s)
+            if (it + s < nsteps) mma_stage(s);
+    }
+
+    float* part = smem + wave * (TD::SUBS * TD::PART);
+#pragma unroll
+    for (int h = 0; h < TM; ++h)
+#pragma unroll
+        for (int g = 0; g < TN; ++g)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                part[(h * TN + g) * TD::PART + (5 * kq + j) * 16 + i16] = acc[h][g][0][j] + acc[h][g][1][j];
+    __syncthreads();
+    if (Poll::enabled && *sflag) return false;
+    const float* mine = smem + threadIdx.x + (threadIdx.x >> 6) * 16;
+    constexpr int WSTRIDE = TD::SUBS * TD::PART;
+    const float alpha = __int_as_float(a[REEF_GEMM_ALPHA_BITS]);
+    const int act = a[REEF_GEMM_ACT];
+#pragma unroll
+    for (int h = 0; h < TM; ++h)
+#pragma unroll
+        for (int g = 0; g < TN; ++g) {
+            const float* e = mine + (h * TN + g) * TD::PART;
+            float v = (((e[0] + e[WSTRIDE]) + e[2 * WSTRIDE]) + e[3 * WSTRIDE]) * alpha + e_bias[g];
+            if (act == REEF_ACT_RELU) v = fmaxf(v, 0.0f);
+            else if (act == REEF_ACT_GELU) v = gelu_erf(v);
+            buf_store(rs_c, ooff[h][g], v);
+        }
+    return true;
+}
+
 }  // namespace reef_dev

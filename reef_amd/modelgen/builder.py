@@ -377,14 +377,22 @@ class GraphBuilder:
         return out
 
     def gemm(self, a, b, M, N, K, batch=1, trans_b=True, bias=None, act=ACT_NONE, alpha=1.0,
-             lda=None, ldb=None, ldc=None, stride_a=0, stride_b=0, stride_c=0, out=None):
-        """C[b] = act(alpha * A[b] x B[b] (+bias)); operands are storages with explicit strides."""
+             lda=None, ldb=None, ldc=None, stride_a=0, stride_b=0, stride_c=0, out=None, force_tile=None):
+        """C[b] = act(alpha * A[b] x B[b] (+bias)); operands are storages with explicit strides.
+        force_tile: a staged tile name or, for trans_b, one of tiling.GEMM_DIRECT_TILES."""
         lda = K if lda is None else lda
         ldb = (K if trans_b else N) if ldb is None else ldb
         ldc = N if ldc is None else ldc
         if out is None:
             out = self.temp((batch, M, N))
-        t = tiling.choose(M, N, K, allow_split=False, tiles=tiling.GEMM_TILES)
+        direct_ok = (trans_b and K % 8 == 0 and lda % 4 == 0 and ldb % 4 == 0 and stride_a % 4 == 0
+                     and stride_b % 4 == 0)
+        if force_tile is not None:
+            t = tiling.forced(force_tile, M, N, K, 1)
+        else:
+            t = tiling.choose_gemm(M, N, K, batch, direct_ok)
+        direct = t["tile"] in tiling.GEMM_DIRECT_TILES
+        assert direct_ok or not direct, "this GEMM has no direct form"
         args = [a.idx, b.idx, out.idx]
         flags = 0
         if bias is not None:
@@ -395,7 +403,7 @@ class GraphBuilder:
         assert K % 4 == 0 and lda % 4 == 0 and stride_a % 4 == 0, "gemm operands must be 16-byte aligned"
         if trans_b:
             assert ldb % 4 == 0 and stride_b % 4 == 0, "gemm operands must be 16-byte aligned"
-        self._emit("reef_gemm_%s_%s" % ("nt" if trans_b else "nn", t["tile"]),
+        self._emit("reef_gemm_%s_%s" % ("ntd" if direct else "nt" if trans_b else "nn", t["tile"]),
                    batch * t["m_tiles"] * t["n_tiles"], args,
                    [batch, M, N, K, 1 if trans_b else 0, flags, act, float_bits(alpha), t["tile_id"],
                     t["m_tiles"], t["n_tiles"], lda, ldb, ldc, stride_a, stride_b, stride_c],

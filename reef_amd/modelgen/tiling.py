@@ -40,6 +40,31 @@ KW = {"32x32k4": 4, "64x32k2": 2, "32x64k2": 2}
 GEMM_TILES = ("128x128", "64x64", "32x128", "32x32k4", "64x32k2")
 
 
+GEMM_DIRECT_TILES = ("16x16k4", "16x32k4", "32x32d4")   # reef_gemm_ntd_<tile>
+
+
+def choose_gemm(M, N, K, batch=1, direct_ok=False):
+    """Tile of a GEMM.  Without a measured table: the staged choice of the analytic model,
+    against the direct tiles (both operands K-contiguous) scored by the rule the batch-1
+    convolutions were found to follow -- a workgroup's time grows with the cache lines it has to
+    pull in, (BM + BN) K / 32 of them, and workgroups beyond one per CU queue up."""
+    staged = choose(M, N, K, allow_split=False, tiles=GEMM_TILES)
+    if not direct_ok:
+        return staged
+
+    def cost(bm, bn):
+        wgs = batch * math.ceil(M / bm) * math.ceil(N / bn)
+        return math.ceil(wgs / NUM_CUS) * (bm + bn) * K / 32.0
+    best = min(GEMM_DIRECT_TILES, key=lambda t: (cost(TILES[t][1], TILES[t][2]), -TILES[t][1] * TILES[t][2]))
+    _, bm, bn, _, _ = TILES[staged["tile"]]
+    if cost(bm, bn) * GEMM_STAGED_BONUS <= cost(TILES[best][1], TILES[best][2]):
+        return staged
+    return forced(best, M, N, K, 1)
+
+
+GEMM_STAGED_BONUS = 1.0
+
+
 def step_k(tile, taps=1):
     """k values a workgroup consumes per step of its K loop (taps = kh*kw, direct family only:
     a step is 16 channels of a filter with taps > 1, 128 channels of a 1x1 filter)."""

@@ -268,6 +268,28 @@ def test_transformer_ops(tmp_path):
     compare_storages(exe, orc, model, what="transformer ops")
 
 
+@pytest.mark.parametrize("tile", list(tiling.GEMM_DIRECT_TILES))
+def test_gemm_nt_direct_tiles(tmp_path, tile):
+    """C = act(alpha A B^T + bias) with both operands loaded straight into the matrix cores:
+    ragged M and N, K not a multiple of the 128-wide step, bias + GELU, alpha, a batched product
+    over strided views (the Q K^T of an attention head: lda = ldb = hidden > K)."""
+    seq, hid, heads = 40, 200, 5          # M = 40 (2.5 row groups), K = 200 = 128 + 72
+    hd = hid // heads                     # 40: K of the batched product, one partial step
+    g = MB.GraphBuilder("gd", weight_std=0.05)
+    x = g.input("x", (seq, hid))
+    w = g.param((3 * hid + 8, hid), 0.05)                 # N = 608: ragged against 16 / 32
+    bias = g.param((3 * hid + 8,), 0.02)
+    y = g.gemm(x, w, seq, 3 * hid + 8, hid, trans_b=True, bias=bias, act=MB.ACT_GELU, force_tile=tile)
+    z = g.gemm(x, w, seq, 3 * hid + 8, hid, trans_b=True, alpha=0.5, force_tile=tile)
+    # heads as strided views of x: A[b] = x[:, b*hd:(b+1)*hd], same for B; C[b] = [seq, seq]
+    s_ = g.gemm(x, x, seq, seq, hd, batch=heads, trans_b=True, alpha=0.25, lda=hid, ldb=hid,
+                stride_a=hd, stride_b=hd, stride_c=seq * seq, force_tile=tile)
+    g.mark_output(s_)
+    assert all(k["name"].startswith("reef_gemm_ntd_" + tile) for k in g.kernels)
+    exe, orc, model = run_both(g, tmp_path, {"x": rnd(seq, hid)})
+    compare_storages(exe, orc, model, what="direct gemm " + tile)
+
+
 def test_mocked_model_closed_form(tmp_path):
     """The reference's executor_base.mocked_kernel test: a = b = c = 3 -> 18 everywhere
     (src/reef/test/test.cpp:102-116)."""
