@@ -263,3 +263,17 @@ def test_direct_tile_geometry():
     t = tiling.choose(256, 196, 2304, fused=False, pointwise=False, taps=9, direct=False)
     assert t["tile"] != "16x16k4"
     assert tiling.lds_bytes("16x16k4") == 4 * 320 * 4 + 16
+
+
+def test_gemm_tile_choice_follows_the_line_rule():
+    """BERT-base's products: the generator takes a direct tile where a workgroup's stream of
+    cache lines, (BM + BN) K / 32 times the workgroups queued per CU, is shorter than the staged
+    tile's, and never without K-contiguous, 16-byte aligned operands."""
+    from reef_amd.modelgen import tiling
+    assert tiling.choose_gemm(128, 768, 768, 1, True)["tile"] == "16x32k4"       # projections
+    assert tiling.choose_gemm(128, 768, 3072, 1, True)["tile"] == "16x32k4"      # FFN down
+    assert tiling.choose_gemm(128, 3072, 768, 1, True)["tile"] == "32x32k4"      # FFN up: staged
+    assert tiling.choose_gemm(128, 768, 768, 1, False)["tile"] in tiling.GEMM_TILES
+    for t in tiling.GEMM_DIRECT_TILES:
+        f = tiling.forced(t, 128, 768, 768, 1)
+        assert f["split_k"] == 1 and f["tasks"] == f["m_tiles"] * f["n_tiles"]
