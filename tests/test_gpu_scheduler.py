@@ -246,3 +246,55 @@ def test_load_generator_preemption_under_load(dirs, mode):
     for m in bes:
         np.testing.assert_array_equal(s.get_output(m, 1000), ref_be)
     s.shutdown()
+
+
+def test_pre_activation_and_folded_split_survive_preemption(tmp_path_factory):
+    """Best-effort clients running a DenseNet (pre-activation folded into its 1x1 convolutions,
+    split-K folded inside launches) and a BERT encoder (direct GEMMs) are preempted dozens of
+    times by a real-time ResNet-18; afterwards every model holds exactly the output of an
+    uninterrupted solo run."""
+    from reef_amd import profiler
+    models = {"densenet_s": nets.densenet(blocks=(3, 4, 6, 4), name="densenet_s"),
+              "bert_s": nets.bert(layers=2, name="bert_s"),
+              "resnet18": nets.resnet(18)}
+    d = {}
+    for k, g in models.items():
+        d[k] = write_model(g, tmp_path_factory.mktemp(k))
+        profiler.write_profile(d[k], k)
+    syms = {k["name"].split("#")[0] for k in models["densenet_s"].kernels}
+    assert any(s_.startswith("reef_conv2d_p1_") for s_ in syms)
+    assert any(s_.startswith("reef_gemm_ntd_") for s_ in {k["name"].split("#")[0] for k in models["bert_s"].kernels})
+    x = nets.image_input("resnet18", (3, 224, 224))
+    ids = nets.token_input("bert_s", 128, 30522)
+    refs = {}
+    for k in ("densenet_s", "resnet18"):
+        refs[k] = solo_output(d[k], k, x)
+    s = B.Scheduler(B.MODE_REEF)
+    s.set_wait_sync(True)
+    rt = s.load_model(d["resnet18"], "resnet18")
+    s.bind_model_queue(s.create_queue(B.QUEUE_RT), rt)
+    s.set_input(rt, x, "data")
+    bes = []
+    for _ in range(2):
+        m = s.load_model(d["densenet_s"], "densenet_s")
+        s.bind_model_queue(s.create_queue(B.QUEUE_BE), m)
+        s.set_input(m, x, "data")
+        bes.append(m)
+    bert = s.load_model(d["bert_s"], "bert_s")
+    s.bind_model_queue(s.create_queue(B.QUEUE_BE), bert)
+    assert s.set_input(bert, ids, "input0") == 0
+    s.run()
+    # the encoder's reference: its own first uninterrupted run on this scheduler
+    r0 = s.run_load(rt, [bert], requests=0, be_only_ms=20)
+    assert r0["be_completed"].sum() > 0
+    n_out = 128 * 768
+    bert_ref = s.get_output(bert, n_out).copy()
+    r = s.run_load(rt, bes + [bert], requests=60, warmup=5, mean_interval_us=1500.0, seed=3)
+    assert r["be_preempted"].sum() > 10 and r["be_completed"].sum() > 0
+    r2 = s.run_load(rt, bes + [bert], requests=0, be_only_ms=30)
+    assert (r2["be_completed"] > 0).all()
+    np.testing.assert_array_equal(s.get_output(rt, 1000), refs["resnet18"])
+    for m in bes:
+        np.testing.assert_array_equal(s.get_output(m, 1000), refs["densenet_s"])
+    np.testing.assert_array_equal(s.get_output(bert, n_out), bert_ref)
+    s.shutdown()
