@@ -104,7 +104,11 @@ int reef_scheduler_run(reef_scheduler_t s);
 int reef_scheduler_shutdown(reef_scheduler_t s);
 int reef_scheduler_mode(reef_scheduler_t s);
 void reef_scheduler_set_wait_sync(reef_scheduler_t s, int value);
-void reef_scheduler_set_be_stream_cap(reef_scheduler_t s, int value);
+/* Launch window of best-effort streams (set_be_stream_cap, scheduler.h:120).  Only while no
+ * best-effort queue exists: Fail afterwards (the streams were created with the old window). */
+int reef_scheduler_set_be_stream_cap(reef_scheduler_t s, int value);
+/* Tasks submitted and not yet finished. */
+uint64_t reef_scheduler_pending_tasks(reef_scheduler_t s);
 /* Share (percent) of a real-time kernel's profiled latency that padded best-effort workgroups
  * may take; 100 is the reference's rule (scheduler.cpp:565-572). */
 void reef_scheduler_set_dkp_slack_percent(reef_scheduler_t s, int value);

@@ -189,7 +189,8 @@ class Scheduler:
         for fn in ("reef_scheduler_avg_preempt_latency", "reef_scheduler_max_preempt_latency",
                    "reef_scheduler_avg_kernel_sel_latency"):
             getattr(L, fn).restype = ctypes.c_int64
-        for fn in ("reef_scheduler_preempt_times", "reef_scheduler_padded_kernels"):
+        for fn in ("reef_scheduler_preempt_times", "reef_scheduler_padded_kernels",
+                   "reef_scheduler_pending_tasks"):
             getattr(L, fn).restype = ctypes.c_uint64
         L.reef_scheduler_preempt_samples.restype = ctypes.c_size_t
         _check("scheduler_create", L.reef_scheduler_create(mode, ctypes.byref(self.h)))
@@ -275,7 +276,10 @@ class Scheduler:
         lib().reef_scheduler_set_wait_sync(self.h, int(v))
 
     def set_be_stream_cap(self, v):
-        lib().reef_scheduler_set_be_stream_cap(self.h, int(v))
+        return lib().reef_scheduler_set_be_stream_cap(self.h, int(v))
+
+    def pending_tasks(self):
+        return lib().reef_scheduler_pending_tasks(self.h)
 
     def set_dkp_slack_percent(self, v):
         lib().reef_scheduler_set_dkp_slack_percent(self.h, int(v))

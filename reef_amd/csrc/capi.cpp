@@ -254,7 +254,8 @@ int reef_scheduler_run(reef_scheduler_t h) { return h->s->run(); }
 int reef_scheduler_shutdown(reef_scheduler_t h) { return h->s->shutdown(); }
 int reef_scheduler_mode(reef_scheduler_t h) { return (int)h->s->sche_mode(); }
 void reef_scheduler_set_wait_sync(reef_scheduler_t h, int v) { h->s->set_wait_sync(v != 0); }
-void reef_scheduler_set_be_stream_cap(reef_scheduler_t h, int v) { h->s->set_be_stream_cap(v); }
+int reef_scheduler_set_be_stream_cap(reef_scheduler_t h, int v) { return (int)h->s->set_be_stream_cap(v); }
+uint64_t reef_scheduler_pending_tasks(reef_scheduler_t h) { return h->s->num_pending_tasks(); }
 void reef_scheduler_set_dkp_slack_percent(reef_scheduler_t h, int v) { h->s->set_dkp_slack_percent(v); }
 int64_t reef_scheduler_avg_preempt_latency(reef_scheduler_t h) { return h->s->avg_preempt_latency(); }
 int64_t reef_scheduler_max_preempt_latency(reef_scheduler_t h) { return h->s->max_preempt_latency(); }

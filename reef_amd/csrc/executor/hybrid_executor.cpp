@@ -128,6 +128,16 @@ void HybridExecutor::reset_task_slots(GPUStream_t stream) {
     reef_hal_memcpy_h2d_async(task_slot_base, task_slots_host_empty, 4 * num_kernels(), stream);
 }
 
+// Zeroes the completion counters of kernels [first, n) in stream order.
+Status HybridExecutor::reset_task_slots_from(int first, GPUStream_t stream) {
+    const int n = (int)num_kernels();
+    if (first < 0) first = 0;
+    if (first >= n) return Status::Succ;
+    GPU_RETURN_STATUS(reef_hal_memset_async((char*)task_slot_base + (size_t)first * 4, 0,
+                                            (size_t)(n - first) * 4, stream));
+    return Status::Succ;
+}
+
 void HybridExecutor::copy_be_kernel_offset(GPUStream_t stream) {
     reef_hal_memcpy_d2h_async(task_slots_host, task_slot_base, 4 * num_kernels(), stream);
 }

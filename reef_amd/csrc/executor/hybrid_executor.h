@@ -30,6 +30,7 @@ public:
 
     Status reset_task_slot_async(int kernel_offset, GPUStream_t stream);
     void reset_task_slots(GPUStream_t stream);
+    Status reset_task_slots_from(int first_kernel, GPUStream_t stream);
     void copy_be_kernel_offset(GPUStream_t stream);
     int get_be_kernel_offset(int begin);
 

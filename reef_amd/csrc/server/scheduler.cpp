@@ -246,10 +246,13 @@ Status REEFScheduler::shutdown() {
     return Status::Succ;
 }
 
+// Finishing is idempotent: a task is reported (and counted out of pending_tasks) once,
+// whichever path notices its completion first.
 void REEFScheduler::finish_task(const std::shared_ptr<Task>& task, TimePoint end) {
-    task->end = end;
     {
         std::lock_guard<std::mutex> lock(task->mtx);
+        if (task->state.load() == TaskState::Finish) return;
+        task->end = end;
         task->state.store(TaskState::Finish);
     }
     task->cv.notify_all();
@@ -276,11 +279,14 @@ void REEFScheduler::loop_body() {
                 if (!rt_queue->empty()) { rt_arrived = true; break; }
                 auto be_task = q->front();
                 execute_be_task(be_task, q);
-                if (!rt_queue->empty()) { rt_arrived = true; break; }
+                // A finished task leaves its queue before anything else can look at the
+                // queue head: a real-time arrival in this instant must not find it there
+                // (the padding pass would run its kernels a second time).
                 if (be_task->state.load() == TaskState::Finish) {
                     q->pop();
                     continue;
                 }
+                if (!rt_queue->empty()) { rt_arrived = true; break; }
                 break;
             }
         }
@@ -339,26 +345,30 @@ void REEFScheduler::preempt_phase_avg_ns(int64_t out[3]) const {
 }
 
 // Wait-based preemption (scheduler.cpp:348-372): raise the flag, let the device
-// drain, then find per task the first kernel whose workgroups did not all finish.
+// drain, then find per running task the first kernel whose workgroups did not all
+// finish (HybridExecutor::get_be_kernel_offset, hybrid_executor.cpp:141-151).
+// The completion counters of the kernels a run is about to launch are zeroed on the
+// task's own stream when the run (re)starts (execute_be_task), so a count read here
+// belongs to this run only; a task that has not been launched yet is left alone.
 void REEFScheduler::preempt_wait() {
-    int one = 1;
-    reef_hal_memcpy_h2d_async(preempt_flag, &one, 4, preempt_stream);
-    reef_hal_stream_sync(preempt_stream);
+    reef_hal_host_write32(preempt_flag, 1);
     const uint32_t n = be_queue_cnt.load();
     for (uint32_t i = 0; i < n; i++) {
         uint64_t dropped = 0;
         reef_hal_stream_clear_queue(be_queues[i]->stream, &dropped);
-        reef_hal_stream_sync(be_queues[i]->stream);
     }
+    for (uint32_t i = 0; i < n; i++) reef_hal_stream_sync(be_queues[i]->stream);
     for (uint32_t i = 0; i < n; i++) {
         auto be_task = be_queues[i]->front();
-        if (!be_task) continue;
+        if (!be_task || be_task->state.load() != TaskState::Executing) continue;
         auto& exe = be_task->model->executor;
         exe.copy_be_kernel_offset(preempt_stream);
-        exe.reset_task_slots(preempt_stream);
         reef_hal_stream_sync(preempt_stream);
         const int off = exe.get_be_kernel_offset(be_task->kernel_offset);
         be_task->kernel_offset = std::max(be_task->kernel_offset, off);
+        be_task->block_offset = 0;
+        be_task->preempted = true;
+        be_task->sync_dirty = true;
     }
 }
 
@@ -509,7 +519,7 @@ void REEFScheduler::dynamic_kernel_padding(std::shared_ptr<Task>& rt_task) {
         const uint32_t n_q = be_queue_cnt.load();
         for (uint32_t q = 0; q < n_q; q++) {   // first queue whose head kernel fits (scheduler.cpp:533-602)
             auto cand = be_queues[q]->front();
-            if (!cand) continue;
+            if (!cand || cand->state.load() == TaskState::Finish) continue;
             HybridExecutor& be_exe = cand->model->executor;
             if (cand->kernel_offset >= (int)be_exe.num_kernels()) continue;
             if (cand->sync_dirty) {
@@ -630,6 +640,9 @@ void REEFScheduler::execute_be_task(std::shared_ptr<Task>& task, std::shared_ptr
                 exe.reset_sync_storage(tqueue->stream);
                 task->sync_dirty = task->sync_touched = false;
             }
+            // wait-based preemption reads the completion counters of this run: the kernels
+            // about to be launched start from zero (a model keeps the counts of earlier runs)
+            if (mode == ScheduleMode::WaitPreempt) exe.reset_task_slots_from(task->kernel_offset, tqueue->stream);
             for (int i = task->kernel_offset; i < num_kernels; i++) {
                 exe.launch_preempt_kernel(i, tqueue->stream);
                 task->launch_offset = i;

@@ -120,7 +120,15 @@ public:
     Status get_task(TaskID tid, std::shared_ptr<Task>& t);
     ScheduleMode sche_mode() const { return mode; }
     void set_wait_sync(bool value) { wait_sync = value; }
-    void set_be_stream_cap(int value) { be_stream_device_queue_cap = value; }
+    // The window is a property of the best-effort streams, which are created with it; it can
+    // only change while no best-effort queue exists (afterwards the rollback after a
+    // preemption would assume a window the streams do not have).  Returns Fail then.
+    Status set_be_stream_cap(int value) {
+        if (be_queue_cnt.load() != 0 || value < 1) return Status::Fail;
+        be_stream_device_queue_cap = value;
+        return Status::Succ;
+    }
+    uint64_t num_pending_tasks() const { return pending_tasks.load(); }
     // Share of a real-time kernel's profiled latency that padded best-effort workgroups may
     // take (100 = the reference's rule, be.latency <= rt.latency, scheduler.cpp:565-572).
     // The merged launch ends when its slowest workgroup ends, and on this device kernels run

@@ -309,3 +309,98 @@ def test_dkp_slack_limits_padding(fake):
     part = got[100][4]
     assert got[100][5] == min(512, (256 - part) * (100 // 90) * 3)
     assert got[65][5] == min(512, (256 - part) * (65 // 60) * 1)
+
+
+def test_finished_best_effort_task_is_never_run_or_counted_twice(fake, small_dirs):
+    """A real-time task that arrives in the instant a best-effort task completes must not find
+    the completed task at the head of its queue: it would be padded into real-time kernels a
+    second time and counted out of the pending tasks twice.  Many short best-effort tasks with
+    real-time arrivals at random moments; afterwards every task is finished exactly once (the
+    pending count is back at zero, not below) and outputs are intact."""
+    gm, dm = small_dirs["mocked_kernel"]
+    gr, dr = small_dirs["tiny18"]
+    x = nets.image_input("t", (3, 32, 32))
+    ref = oracle_output(gr, dr, x)
+    prof = json.load(open(os.path.join(dr, gr.name + ".profile.json")))
+    for v in prof["kernel_latency"].values():
+        v["total_latency"] = 100      # every real-time kernel can host the mocked kernels
+    json.dump(prof, open(os.path.join(dr, gr.name + ".profile.json"), "w"))
+    fake.lib.fake_hal_set_auto_progress(2)
+    s = B.Scheduler(B.MODE_REEF)
+    rt_mid = s.load_model(dr, gr.name)
+    be_mid = s.load_model(dm, gm.name)
+    s.bind_model_queue(s.create_queue(B.QUEUE_RT), rt_mid)
+    s.bind_model_queue(s.create_queue(B.QUEUE_BE), be_mid)
+    s.set_input(rt_mid, x, "data")
+    for n in "abc":
+        s.set_input(be_mid, THREE, n)
+    s.run()
+    rng = np.random.default_rng(5)
+    for rep in range(60):
+        be_tid = s.new_task(be_mid)
+        time.sleep(float(rng.uniform(0, 0.002)))
+        rt_tid = s.new_task(rt_mid)
+        be2 = s.new_task(be_mid)
+        for t in (be_tid, rt_tid, be2):
+            assert run_scheduler_until(s, t), "task %d never finished (rep %d)" % (t, rep)
+        np.testing.assert_array_equal(s.get_output(be_mid, 8192), np.full(8192, 18.0, np.float32))
+    t0 = time.time()
+    while s.pending_tasks() != 0 and time.time() - t0 < 2:
+        time.sleep(0.001)
+    assert s.pending_tasks() == 0
+    np.testing.assert_array_equal(s.get_output(rt_mid, 16), ref)
+    s.shutdown()
+
+
+def test_wait_preempt_second_run_restarts_at_the_interrupted_kernel(fake, small_dirs):
+    """Wait-based preemption (src/reef/server/scheduler.cpp:348-372) finds the restart point from
+    per-kernel completion counters.  The counters of a model survive a run, so a second,
+    interrupted run must not mistake the first run's counts for its own: its output still
+    equals the uninterrupted result and the interrupted tail is launched again."""
+    gb, db = small_dirs["tiny18"]
+    gm, dm = small_dirs["mocked_kernel"]
+    x = nets.image_input("t", (3, 32, 32))
+    ref = oracle_output(gb, db, x)
+    fake.lib.fake_hal_set_auto_progress(1)
+    s = B.Scheduler(B.MODE_WAITPREEMPT)
+    s.run()
+    be_mid = s.load_model(db, gb.name)
+    rt_mid = s.load_model(dm, gm.name)
+    s.bind_model_queue(s.create_queue(B.QUEUE_BE), be_mid)
+    s.bind_model_queue(s.create_queue(B.QUEUE_RT), rt_mid)
+    s.set_input(be_mid, x, "data")
+    for n in "abc":
+        s.set_input(rt_mid, THREE, n)
+    # a clean first run leaves every counter at its kernel's workgroup count
+    assert s.wait_task(s.new_task(be_mid)) == 0
+    np.testing.assert_array_equal(s.get_output(be_mid, 16), ref)
+    n_kernels = len(gb.kernels)
+    preempted = 0
+    for rep in range(6):
+        # a different input each time, so a skipped kernel would leave stale activations behind
+        xi = (x * (1.0 + 0.25 * rep)).astype(np.float32)
+        want = oracle_output(gb, db, xi)
+        s.set_input(be_mid, xi, "data")
+        done0 = fake.lib.fake_hal_completed()
+        launches0 = fake.lib.fake_hal_launches()
+        be_tid = s.new_task(be_mid)
+        t0 = time.time()
+        while fake.lib.fake_hal_completed() < done0 + 3 + rep and time.time() - t0 < 10:
+            time.sleep(0.0002)
+        rt_tid = s.new_task(rt_mid)
+        assert s.wait_task(rt_tid) == 0 and s.wait_task(be_tid) == 0
+        np.testing.assert_array_equal(s.get_output(be_mid, 16), want)
+        if s.task_info(be_tid)["preempted"]:
+            preempted += 1
+            # everything the model has was launched at least once in this run
+            assert fake.lib.fake_hal_launches() - launches0 >= n_kernels + 2
+    assert preempted > 0, "no run was interrupted"
+    s.shutdown()
+
+
+def test_be_stream_cap_is_fixed_once_a_best_effort_queue_exists(fake, small_dirs):
+    s = B.Scheduler(B.MODE_RESET)
+    assert s.set_be_stream_cap(3) == 0
+    assert s.set_be_stream_cap(0) == 1           # a window of zero kernels makes no sense
+    s.create_queue(B.QUEUE_BE)
+    assert s.set_be_stream_cap(1) == 1           # Fail: the stream exists with a window of 3
