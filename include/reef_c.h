@@ -94,6 +94,8 @@ int reef_scheduler_get_data_size(reef_scheduler_t s, uint32_t mid, const char* n
 int reef_scheduler_set_input(reef_scheduler_t s, uint32_t mid, const void* data, size_t len,
                              const char* name);
 int reef_scheduler_get_output(reef_scheduler_t s, uint32_t mid, void* data, size_t len);
+/* ExecutorBase::get_data (executor_base.cpp:153-162) of a model the scheduler holds. */
+int reef_scheduler_get_data(reef_scheduler_t s, uint32_t mid, int idx, void* data, size_t len);
 int reef_scheduler_new_task(reef_scheduler_t s, uint32_t mid, uint32_t* tid);
 int reef_scheduler_wait_task(reef_scheduler_t s, uint32_t tid);
 /* Task record: flags bit0 preempted, bit1 padded, bit2 padded to completion;
@@ -117,6 +119,9 @@ int64_t reef_scheduler_max_preempt_latency(reef_scheduler_t s);
 int64_t reef_scheduler_avg_kernel_sel_latency(reef_scheduler_t s);
 uint64_t reef_scheduler_preempt_times(reef_scheduler_t s);
 uint64_t reef_scheduler_padded_kernels(reef_scheduler_t s);
+/* Merged launches by the op of their best-effort side: out[i] for REEF_OP_* = i (reef_kernels.h),
+ * i < n.  Returns the number of op ids. */
+int reef_scheduler_padded_by_op(reef_scheduler_t s, uint64_t* out, int n);
 size_t reef_scheduler_preempt_samples(reef_scheduler_t s, int64_t* out, size_t cap);
 /* Average ns per reset-based preemption in: flag store, host-queue drop + rollback, device drain. */
 void reef_scheduler_preempt_phases(reef_scheduler_t s, int64_t out_ns[3]);

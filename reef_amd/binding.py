@@ -242,6 +242,12 @@ class Scheduler:
                                                             ctypes.c_size_t(out.nbytes)))
         return out
 
+    def get_data(self, mid, idx, n, dtype=np.float32):
+        out = np.empty(n, dtype)
+        _check("get_data", lib().reef_scheduler_get_data(self.h, mid, idx, out.ctypes.data_as(ctypes.c_void_p),
+                                                        ctypes.c_size_t(out.nbytes)))
+        return out
+
     def new_task(self, mid):
         tid = ctypes.c_uint32()
         _check("new_task", lib().reef_scheduler_new_task(self.h, mid, ctypes.byref(tid)))
@@ -298,6 +304,12 @@ class Scheduler:
 
     def padded_kernels(self):
         return lib().reef_scheduler_padded_kernels(self.h)
+
+    def padded_by_op(self):
+        """Merged launches by the best-effort side's op id (REEF_OP_* of include/reef_kernels.h)."""
+        buf = (ctypes.c_uint64 * 32)()
+        n = lib().reef_scheduler_padded_by_op(self.h, buf, 32)
+        return [int(buf[i]) for i in range(n)]
 
     def preempt_samples(self, cap=100000):
         buf = (ctypes.c_int64 * cap)()

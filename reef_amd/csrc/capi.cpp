@@ -231,6 +231,9 @@ int reef_scheduler_set_input(reef_scheduler_t h, uint32_t mid, const void* data,
                              const char* name) {
     return h->s->set_input(mid, data, len, name ? name : "data");
 }
+int reef_scheduler_get_data(reef_scheduler_t h, uint32_t mid, int idx, void* data, size_t len) {
+    return (int)h->s->get_data(mid, idx, data, len);
+}
 int reef_scheduler_get_output(reef_scheduler_t h, uint32_t mid, void* data, size_t len) {
     return h->s->get_output(mid, data, len);
 }
@@ -262,6 +265,12 @@ int64_t reef_scheduler_max_preempt_latency(reef_scheduler_t h) { return h->s->ma
 int64_t reef_scheduler_avg_kernel_sel_latency(reef_scheduler_t h) { return h->s->avg_kernel_sel_latency(); }
 uint64_t reef_scheduler_preempt_times(reef_scheduler_t h) { return h->s->preempt_times(); }
 uint64_t reef_scheduler_padded_kernels(reef_scheduler_t h) { return h->s->padded_kernels(); }
+int reef_scheduler_padded_by_op(reef_scheduler_t h, uint64_t* out, int n) {
+    uint64_t v[REEF_OP_COUNT];
+    h->s->padded_kernels_by_op(v);
+    for (int i = 0; i < n; i++) out[i] = i < REEF_OP_COUNT ? v[i] : 0;
+    return REEF_OP_COUNT;
+}
 size_t reef_scheduler_preempt_samples(reef_scheduler_t h, int64_t* out, size_t cap) {
     return h->s->preempt_latency_samples(out, cap);
 }

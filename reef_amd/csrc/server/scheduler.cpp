@@ -214,6 +214,11 @@ Status REEFScheduler::get_output(ModelID mid, void* data, size_t len, const std:
     return model_pool[mid]->executor.get_output(data, len);
 }
 
+Status REEFScheduler::get_data(ModelID mid, int idx, void* data, size_t len) {
+    if (mid >= model_pool_size.load()) RETURN_STATUS(Status::OutOfRange);
+    return model_pool[mid]->executor.get_data(idx, data, len);
+}
+
 Status REEFScheduler::run() {
     if (scheduler) RETURN_STATUS(Status::Fail);
     {
@@ -571,6 +576,7 @@ void REEFScheduler::dynamic_kernel_padding(std::shared_ptr<Task>& rt_task) {
             reef_hal_launch(proxy, grid, block, (uint32_t)dec.resource.shared_memory, rt_queue->stream,
                             &a, sizeof(a));
             padded_kernel_count++;
+            if (be_args->op >= 0 && be_args->op < REEF_OP_COUNT) padded_by_op[be_args->op]++;
         }
         current_time_point += std::chrono::microseconds(rt_args.profile.total_latency);
 

@@ -115,6 +115,8 @@ public:
     Status get_data_size(ModelID mid, const std::string& name, size_t& size);
     Status set_input(ModelID mid, const void* data, size_t len, const std::string& name = "data");
     Status get_output(ModelID mid, void* data, size_t len, const std::string& name = "output");
+    // ExecutorBase::get_data of a loaded model (executor_base.cpp:153-162): any storage by index.
+    Status get_data(ModelID mid, int idx, void* data, size_t len);
     Status new_task(const ModelID& mid, TaskID& tid);
     Status wait_task(TaskID tid);
     Status get_task(TaskID tid, std::shared_ptr<Task>& t);
@@ -146,6 +148,10 @@ public:
     uint64_t preempt_times() const { return preempt_count; }
     int64_t max_preempt_latency() const { return preempt_latency_max; }
     uint64_t padded_kernels() const { return padded_kernel_count; }
+    // Merged launches so far by the op of their best-effort side (index = REEF_OP_*).
+    void padded_kernels_by_op(uint64_t out[REEF_OP_COUNT]) const {
+        for (int i = 0; i < REEF_OP_COUNT; i++) out[i] = padded_by_op[i];
+    }
     // Copies the last `cap` preemption latencies (microseconds); returns how many.
     size_t preempt_latency_samples(int64_t* out, size_t cap) const;
     // Average nanoseconds per reset-based preemption spent in: raising the flag, dropping the
@@ -206,6 +212,7 @@ private:
     uint64_t kernel_sel_count;
     uint64_t kernel_sel_latency_sum;
     uint64_t padded_kernel_count;
+    uint64_t padded_by_op[REEF_OP_COUNT] = {};
     bool gpu_ready;
 
 private:
