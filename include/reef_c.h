@@ -123,6 +123,12 @@ uint64_t reef_scheduler_padded_kernels(reef_scheduler_t s);
  * i < n.  Returns the number of op ids. */
 int reef_scheduler_padded_by_op(reef_scheduler_t s, uint64_t* out, int n);
 size_t reef_scheduler_preempt_samples(reef_scheduler_t s, int64_t* out, size_t cap);
+/* The same preemptions timed by the device (nanoseconds): flag store -> the last best-effort
+ * workgroup that was on the device has left, from the device wall clock that workgroup wrote,
+ * mapped to the host clock by a clock exchange whose half-length clock_sync_error_ns returns
+ * (-1: this backend has no device clock).  Only with wait_sync on. */
+size_t reef_scheduler_preempt_device_samples(reef_scheduler_t s, int64_t* out_ns, size_t cap);
+int64_t reef_scheduler_clock_sync_error_ns(reef_scheduler_t s);
 /* Average ns per reset-based preemption in: flag store, host-queue drop + rollback, device drain. */
 void reef_scheduler_preempt_phases(reef_scheduler_t s, int64_t out_ns[3]);
 /* ---- load generator: the request loops of the reference's example clients
@@ -157,6 +163,26 @@ int reef_dkp_decide_slack(const int rt[7], const int be[7], const int* be_latenc
                           int be_block_offset, const int proxy[3], int num_cus, int num_xcds,
                           int slack_percent, int out[8]);
 int reef_dkp_rollback(int launch_offset, int dropped, int window, int kernel_offset);
+
+/* ---- one fused convolution on plain device pointers ----
+ * The call one generated kernel of the reference's fused_nn_conv2d_* family serves
+ * (resource/resnet152/resnet152.cu:376,715: in, W, out, bias; :35: in, W, out, residual), for
+ * callers that hold tensors of their own instead of a model directory:
+ *   out[o][y][x] = act(sum_{c,ky,kx} in[c][y*s+ky-p][x*s+kx-p] * w[o][c][ky][kx] + residual[o][y][x] + bias[o])
+ * NCHW / OIHW fp32, batch 1; bias and residual may be NULL.  All pointers are device memory.
+ * `stream` is a hipStream_t (NULL: the default stream).  The kernels and the split of K are
+ * chosen by the library; a split is folded inside the launch through partial tiles and arrival
+ * counters (fixed summation order), which need memory beyond the operands. */
+typedef struct {
+    int32_t cin, h, w, cout, kh, kw, stride_h, stride_w, pad_h, pad_w;
+    int32_t act;   /* REEF_ACT_NONE / REEF_ACT_RELU / REEF_ACT_RELU6 of reef_kernels.h */
+} reef_conv2d_desc;
+/* Loads the gfx950 kernels (a reef_kernels.raw.co) for the current device. */
+int reef_ops_init(const char* kernels_co_path);
+/* Takes the partial-tile workspace and the counters from hipMalloc for the duration of the call
+ * and returns them before it returns (it waits for the stream then). */
+int reef_ops_conv2d(const reef_conv2d_desc* c, const float* in, const float* w, const float* bias,
+                    const float* residual, float* out, void* stream);
 
 /* GPUConfig (src/reef/executor/hip/hip_impl.cpp:9-74) */
 int reef_gpuconfig_num_cus(void);

@@ -70,7 +70,23 @@ typedef struct reef_kernel_resource {
     int vgprs;         /* arch VGPRs + AGPRs */
     int sgprs;
     int stack_size;    /* scratch bytes per lane */
+    int agprs;         /* the accumulation registers among `vgprs` (they sit behind the arch VGPRs) */
 } reef_kernel_resource;
+
+/* Completion record of a launch on a windowed stream in REEF_COMPLETE_IN_KERNEL mode: the first
+ * 32 bytes of the kernel's argument block.  The caller leaves it zero; the layer fills it when
+ * the launch goes to the device.  The kernel's workgroups count themselves out on *exit_count
+ * as they leave; the last one sets the counter back to zero, stores the device wall clock to
+ * *exit_ticks and then `seq` to *done_word (both host-visible).  A kernel that finds done_word
+ * NULL (launched on a stream without that mode) does none of this. */
+typedef struct reef_hal_completion {
+    uint32_t* done_word;
+    uint64_t* exit_ticks;
+    uint32_t* exit_count;
+    uint32_t seq;
+    uint32_t reserved;
+} reef_hal_completion;
+enum { REEF_COMPLETE_STREAM_WRITE = 0, REEF_COMPLETE_IN_KERNEL = 1 };
 
 enum { REEF_MEM_DEVICE = 0, REEF_MEM_DEVICE_FINEGRAINED = 1, REEF_MEM_HOST_PINNED = 2 };
 
@@ -91,6 +107,11 @@ int reef_hal_module_unload(reef_module_t mod);
 int reef_hal_module_get_function(reef_module_t mod, const char* name, reef_function_t* out);
 /* hipFuncGetWGInfo                  hip_impl.cpp:34-42 (read from the code object's metadata) */
 int reef_hal_function_resource(reef_function_t fn, reef_kernel_resource* out);
+/* Device address of a kernel's first instruction: GPUConfig::get_kernel_address, hip_impl.cpp:16-32
+ * (there read out of the kernel descriptor through the patched runtime's hipFuncGetWGInfo; here
+ * from the device variable <name>_entry the code object publishes beside each kernel of the
+ * padding flavour).  What a merge_framework_<n> proxy jumps to. */
+int reef_hal_module_kernel_entry(reef_module_t mod, const char* name, uint64_t* address);
 /* GPUConfig::calculate_occupancy    hip_impl.cpp:55-74 -> workgroups resident per CU */
 int reef_hal_occupancy(const reef_kernel_resource* res, int block_threads, int dyn_lds,
                        int* blocks_per_cu);
@@ -111,6 +132,24 @@ int reef_hal_memcpy_d2h_async(void* dst, reef_devptr_t src, size_t bytes, reef_s
  * launch_window <= 0: no limit. */
 int reef_hal_stream_create(int launch_window, reef_stream_t* out);
 int reef_hal_stream_destroy(reef_stream_t s);
+/* How a windowed stream learns that a kernel has finished (the reference's patched runtime
+ * tracks its launch window inside the driver, scheduler.cpp:45):
+ *   REEF_COMPLETE_STREAM_WRITE  the layer appends a stream write of the launch's sequence
+ *                               number after every kernel (on this runtime a small kernel of
+ *                               its own, about 2 us of device time per launch);
+ *   REEF_COMPLETE_IN_KERNEL     every kernel launched on the stream starts its argument block
+ *                               with a reef_hal_completion and signals by itself.
+ * Set before the first launch on the stream. */
+int reef_hal_stream_set_completion(reef_stream_t s, int mode);
+/* Launches handed to the device so far on a windowed stream, and how many have signalled. */
+int reef_hal_stream_progress(reef_stream_t s, uint32_t* submitted, uint32_t* done);
+/* Device wall clock at which launch `seq` of a windowed stream in REEF_COMPLETE_IN_KERNEL mode
+ * left the device (its last workgroup); kept for the 8 most recent launches.  0 if unknown. */
+int reef_hal_stream_exit_ticks(reef_stream_t s, uint32_t seq, uint64_t* ticks);
+/* One correlated reading of the host's monotonic clock (ns) and the device wall clock (ticks at
+ * *ticks_per_us): a probe kernel answers a host-written word with its clock; the host time is
+ * the middle of the exchange and *err_ns half its length (best of several exchanges). */
+int reef_hal_clock_sync(int64_t* host_ns, uint64_t* device_ticks, int64_t* err_ns, int* ticks_per_us);
 /* hipStreamSynchronize / hipStreamQuery / hipDeviceSynchronize   scheduler.cpp:335,339,356; hip_impl.cpp:77-80 */
 int reef_hal_stream_sync(reef_stream_t s);
 int reef_hal_stream_query(reef_stream_t s, int* idle);
@@ -207,6 +246,11 @@ typedef struct reef_hal_backend {
     int (*graph_end)(reef_stream_t, reef_graph_t*);
     int (*graph_launch)(reef_graph_t, reef_stream_t);
     int (*graph_destroy)(reef_graph_t);
+    int (*stream_set_completion)(reef_stream_t, int);
+    int (*stream_progress)(reef_stream_t, uint32_t*, uint32_t*);
+    int (*stream_exit_ticks)(reef_stream_t, uint32_t, uint64_t*);
+    int (*clock_sync)(int64_t*, uint64_t*, int64_t*, int*);
+    int (*module_kernel_entry)(reef_module_t, const char*, uint64_t*);
 } reef_hal_backend;
 
 const reef_hal_backend* reef_hal_hip_backend(void);

@@ -24,10 +24,13 @@
  *
  *   raw    K(ReefOpDesc d)
  *          grid = launch_params; replaces the plain TVM kernels.
- *   be     K(int* preempted, int* task_slot, ReefOpDesc d)
- *          replaces script/best_effort_kernel.py:22-29: a workgroup returns at
+ *   be     K(ReefBeArgs a)  =  (completion record, int* preempted, int* task_slot, ReefOpDesc d)
+ *          replaces script/best_effort_kernel.py:22-29: a workgroup leaves at
  *          once when *preempted != 0, re-polls the flag inside its main loop,
  *          and thread 0 adds 1 to *task_slot only when the workgroup completed.
+ *          The completion record (reef_hal.h) lets the launch-window stream the
+ *          kernel runs on see it finish without a second device operation: every
+ *          workgroup counts itself out as it leaves, preempted or not.
  *   trans  K(ReefDkpArgs a)   and   merge_framework_<n>(ReefDkpArgs a)
  *          replaces the 11-argument dynamic-kernel-padding entry and the
  *          merge_framework_* proxies (script/transform_kernel.py:345-352,
@@ -57,6 +60,19 @@ typedef struct ReefOpDesc {
     int32_t attr[REEF_MAX_ATTRS];  /* JSON `attrs` order */
 } ReefOpDesc;
 
+/* Argument block of the best-effort flavour.  The first 32 bytes are the
+ * reef_hal_completion of reef_hal.h (all zero: nothing is signalled). */
+typedef struct ReefBeArgs {
+    uint32_t* done_word;
+    uint64_t* exit_ticks;
+    uint32_t* exit_count;
+    uint32_t seq;
+    uint32_t reserved;
+    int32_t* preempted;
+    int32_t* task_slot;
+    ReefOpDesc desc;
+} ReefBeArgs;
+
 /* One side of a dynamic-kernel-padding launch
  * (func/layers/task_num/task_offset/param of transform_kernel.py:345-352). */
 typedef struct ReefDkpSide {
@@ -74,7 +90,12 @@ typedef struct ReefDkpArgs {
     int32_t num_cus;       /* virtual CUs per layer (grid = layers * num_cus) */
     int32_t num_xcds;      /* 8 on MI355X; 1 reproduces the reference's flat mapping */
     int32_t reserved;
-    int32_t* task_slot_r;  /* optional completion counter of side r (may be null) */
+    int32_t* task_slot_r;  /* unused, null */
+    /* First instruction of each side's own kernel (the reference's func_l / func_r,
+     * transform_kernel.py:345-352): read by the merge_framework_<n> proxies only, which jump
+     * there; a kernel launched directly ignores them. */
+    const void* entry_l;
+    const void* entry_r;
 } ReefDkpArgs;
 
 /* Op ids for ReefDkpSide.op (order is ABI). */
@@ -179,12 +200,18 @@ enum {
  *   reef_conv2d_d<R>_16x<BN>k4  direct: R = kh*kw taps compiled in (1, 3, 7, 9 for BN = 16, 32; 1, 9 for 16x64 and 32x32d4); operands go from memory
  *                           straight into 16x16x4 MFMAs, the four wavefronts split the input
  *                           channels.  d1 needs Cin % 8 == 0 (any stride); K_CHUNK is a multiple
- *                           of R (R > 1) or 8 (d1) and splits K on channel boundaries. */
+ *                           of R (R > 1) or 8 (d1) and splits K on channel boundaries.
+ *   reef_conv2d_r9_g<G>[m2] row form of the direct 3x3 / stride 1 / padding 1 convolution: every input value
+ *                           is loaded once per tile and the horizontal taps come from neighbouring lanes. */
 #define REEF_CONV_MODE_GENERAL 0
 #define REEF_CONV_MODE_POINTWISE 1
 #define REEF_CONV_MODE_UNALIGNED 2
 #define REEF_CONV_MODE_DIRECT 3
 #define REEF_CONV_MODE_DIRECT_PRE 4   /* direct, 1 tap, with REEF_F_PRE_ACT (reef_conv2d_p1_<tile>) */
+#define REEF_CONV_MODE_ROWS 5         /* direct, row form: 3x3 / stride 1 / padding 1 (reef_conv2d_r9_g<G>[m2]).
+                                         The output tile is 16 (m2: 32) channels x G image rows x one 14-column
+                                         segment; N_TILES = ceil(Ho / G) * ceil(Wo / 14), spatial tile index =
+                                         row tile * segments + segment.  K_CHUNK a multiple of 144. */
 
 /* Tile configurations: BM x BN output tile per workgroup.  Plain tiles walk K in steps of
  * 32; a "k<n>" tile splits every step of 32*n k values across n wavefronts and sums the n
@@ -203,6 +230,12 @@ enum {
     REEF_TILE_16x32k4 = 10,  /* direct family, 1 and 9 taps */
     REEF_TILE_16x64k4 = 11,  /* direct family, 1 and 9 taps */
     REEF_TILE_32x32d4 = 12,  /* direct family, 1 and 9 taps (symbol suffix 32x32d4) */
+    REEF_TILE_R9G1 = 13,     /* row form (REEF_CONV_MODE_ROWS): 16 channels x 1, 2, 4, 7 image rows */
+    REEF_TILE_R9G2 = 14,
+    REEF_TILE_R9G4 = 15,
+    REEF_TILE_R9G7 = 16,
+    REEF_TILE_R9G2M2 = 17,   /* 32 channels x 2, 4 image rows */
+    REEF_TILE_R9G4M2 = 18,
     REEF_TILE_COUNT
 };
 

@@ -193,6 +193,8 @@ class Scheduler:
                    "reef_scheduler_pending_tasks"):
             getattr(L, fn).restype = ctypes.c_uint64
         L.reef_scheduler_preempt_samples.restype = ctypes.c_size_t
+        L.reef_scheduler_preempt_device_samples.restype = ctypes.c_size_t
+        L.reef_scheduler_clock_sync_error_ns.restype = ctypes.c_int64
         _check("scheduler_create", L.reef_scheduler_create(mode, ctypes.byref(self.h)))
 
     def close(self):
@@ -316,6 +318,15 @@ class Scheduler:
         n = lib().reef_scheduler_preempt_samples(self.h, buf, ctypes.c_size_t(cap))
         return np.array(buf[:n], np.int64)
 
+    def preempt_device_samples(self, cap=100000):
+        """Preemption latencies measured by the device, in microseconds."""
+        buf = (ctypes.c_int64 * cap)()
+        n = lib().reef_scheduler_preempt_device_samples(self.h, buf, ctypes.c_size_t(cap))
+        return np.array(buf[:n], np.float64) / 1e3
+
+    def clock_sync_error_us(self):
+        return lib().reef_scheduler_clock_sync_error_ns(self.h) / 1e3
+
     def preempt_phases(self):
         out = (ctypes.c_int64 * 3)()
         lib().reef_scheduler_preempt_phases(self.h, out)
@@ -350,3 +361,63 @@ class Scheduler:
         return {"rt_latency_us": lat / 1e3, "rt_queue_us": que / 1e3, "rt_exec_us": exe / 1e3,
                 "be_completed": done[:n_be], "be_preempted": pre[:n_be], "be_padded": pad[:n_be],
                 "span_s": span.value}
+
+
+# ---- device memory and the single-convolution entry points ---------------------------------
+class DeviceBuffer:
+    """Device memory from the C-ABI layer (reef_hal_malloc), for callers of the op-level entry
+    points that hold their tensors themselves."""
+
+    def __init__(self, nbytes):
+        L = lib()
+        _check("hal_init", L.reef_hal_init(0))
+        self.ptr = ctypes.c_void_p()
+        self.nbytes = int(nbytes)
+        _check("hal_malloc", L.reef_hal_malloc(ctypes.c_size_t(max(self.nbytes, 4)), 0, ctypes.byref(self.ptr)))
+
+    @classmethod
+    def from_array(cls, arr):
+        arr = np.ascontiguousarray(arr)
+        b = cls(arr.nbytes)
+        _check("h2d", lib().reef_hal_memcpy_h2d(b.ptr, arr.ctypes.data_as(ctypes.c_void_p), ctypes.c_size_t(arr.nbytes)))
+        return b
+
+    def to_array(self, dtype=np.float32):
+        out = np.empty(self.nbytes // np.dtype(dtype).itemsize, dtype)
+        _check("d2h", lib().reef_hal_memcpy_d2h(out.ctypes.data_as(ctypes.c_void_p), self.ptr, ctypes.c_size_t(out.nbytes)))
+        return out
+
+    def fill(self, byte=0):
+        _check("memset", lib().reef_hal_memset(self.ptr, int(byte), ctypes.c_size_t(self.nbytes)))
+
+    def free(self):
+        if self.ptr:
+            lib().reef_hal_free(self.ptr, 0)
+            self.ptr = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Conv2dDesc(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in ("cin", "h", "w", "cout", "kh", "kw", "stride_h", "stride_w",
+                                              "pad_h", "pad_w", "act")]
+
+
+def ops_init(kernels_co=None):
+    from .paths import BUILD_DIR
+    path = kernels_co or os.path.join(BUILD_DIR, "reef_kernels.raw.co")
+    _check("reef_ops_init", lib().reef_ops_init(path.encode()))
+
+
+def ops_conv2d(desc, inp, w, bias, residual, out, noalloc=False):
+    """reef_ops_conv2d / reef_ops_conv2d_noalloc on DeviceBuffers, default stream; returns the status."""
+    fn = lib().reef_ops_conv2d_noalloc if noalloc else lib().reef_ops_conv2d
+    st = fn(ctypes.byref(desc), inp.ptr, w.ptr, bias.ptr if bias is not None else None,
+            residual.ptr if residual is not None else None, out.ptr, None)
+    if st == 0:
+        _check("device_sync", lib().reef_hal_device_sync())
+    return st

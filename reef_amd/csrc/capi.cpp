@@ -271,6 +271,10 @@ int reef_scheduler_padded_by_op(reef_scheduler_t h, uint64_t* out, int n) {
     for (int i = 0; i < n; i++) out[i] = i < REEF_OP_COUNT ? v[i] : 0;
     return REEF_OP_COUNT;
 }
+size_t reef_scheduler_preempt_device_samples(reef_scheduler_t h, int64_t* out_ns, size_t cap) {
+    return h->s->preempt_device_samples(out_ns, cap);
+}
+int64_t reef_scheduler_clock_sync_error_ns(reef_scheduler_t h) { return h->s->clock_sync_error_ns(); }
 size_t reef_scheduler_preempt_samples(reef_scheduler_t h, int64_t* out, size_t cap) {
     return h->s->preempt_latency_samples(out, cap);
 }
@@ -320,12 +324,14 @@ int reef_dkp_decide_slack(const int rt[7], const int be[7], const int* be_latenc
         ka.task_dim = dim3u((uint32_t)v[0], 1, 1);
         ka.resource = GPUConfig::KernelResource{v[5], v[3], v[4], 0};
         ka.profile.total_latency = v[6];
+        ka.profile.total_latency_ns = v[6] * 1000;
         ka.block_offset = 0;
     };
     TransExecutor::KernelArg rta, bea;
     fill(rta, rt);
     fill(bea, be);
     bea.profile.latency.assign(be_latency, be_latency + n_lat);
+    for (int j = 0; j < n_lat; j++) bea.profile.latency_ns.push_back(be_latency[j] * 1000);
     GPUConfig::KernelResource pr{proxy[2], proxy[0], proxy[1], 0};
     REEFScheduler::PadDecision d =
         REEFScheduler::decide_padding(rta, bea, be_block_offset, pr, num_cus, num_xcds, slack_percent);

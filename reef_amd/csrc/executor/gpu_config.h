@@ -37,9 +37,13 @@ public:
     static Status get_kernel_resource(GPUFunction_t func, KernelResource& ret);  // hip_impl.cpp:34-42
 
     static KernelResource max_resource(const KernelResource& a, const KernelResource& b) {  // :45-53
+        // registers: the architectural VGPRs and the accumulation registers behind them are
+        // two ranges of one file, so the union needs the larger of each
         KernelResource r;
         r.sgprs = std::max(a.sgprs, b.sgprs);
-        r.vgprs = std::max(a.vgprs, b.vgprs);
+        r.agprs = std::max(a.agprs, b.agprs);
+        const int arch = std::max(a.vgprs - a.agprs, b.vgprs - b.agprs);
+        r.vgprs = std::max(std::max(a.vgprs, b.vgprs), r.agprs ? align_up(arch, 4) + r.agprs : arch);
         r.shared_memory = std::max(a.shared_memory, b.shared_memory);
         r.stack_size = std::max(a.stack_size, b.stack_size);
         return r;

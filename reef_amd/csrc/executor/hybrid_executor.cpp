@@ -1,18 +1,13 @@
 #include "executor/hybrid_executor.h"
 
+#include <cstddef>
 #include <cstring>
 
 namespace reef {
 namespace executor {
 
-namespace {
-// Kernel parameter block of the best-effort flavour.
-struct BeKernarg {
-    int* preempted;
-    int* task_slot;
-    ReefOpDesc desc;
-};
-}  // namespace
+static_assert(sizeof(reef_hal_completion) == 32 && offsetof(ReefBeArgs, preempted) == 32,
+              "the best-effort argument block starts with the C-ABI layer's completion record");
 
 HybridExecutor::HybridExecutor()
     : preempt_mod(nullptr), trans_mod(nullptr), preempt_flag(nullptr), owns_flag(false),
@@ -158,7 +153,8 @@ Status HybridExecutor::reset_sync_storage(GPUStream_t stream) {
 
 Status HybridExecutor::launch_preempt_kernel(int i, GPUStream_t stream) {
     const KernelArg& ka = trans_args[i];
-    BeKernarg arg;
+    ReefBeArgs arg;
+    std::memset(&arg, 0, sizeof(reef_hal_completion));   // filled by the layer on a windowed stream
     arg.preempted = (int*)preempt_flag;
     arg.task_slot = (int*)((char*)task_slot_base + i * 4);
     arg.desc = descs[i];

@@ -109,6 +109,16 @@ ModelProfile* ModelProfile::from_json_text(const std::string& text, std::string*
         if (const JsonValue* t = kv.second->get("total_latency")) kp.total_latency = (int)t->as_int();
         if (const JsonValue* l = kv.second->get("latency"))
             for (const auto& v : l->lval) kp.latency.push_back((int)v->as_int());
+        const JsonValue* tn = kv.second->get("total_latency_ns");
+        const JsonValue* ln = kv.second->get("latency_ns");
+        if (tn && ln && ln->lval.size() == kp.latency.size()) {
+            kp.has_ns = true;
+            kp.total_latency_ns = (int)tn->as_int();
+            for (const auto& v : ln->lval) kp.latency_ns.push_back((int)v->as_int());
+        } else {
+            kp.total_latency_ns = kp.total_latency * 1000;
+            for (int v : kp.latency) kp.latency_ns.push_back(v * 1000);
+        }
         p->kernel_latency.emplace(kv.first, std::move(kp));
     }
     return p.release();
@@ -138,7 +148,16 @@ std::string ModelProfile::to_json() const {
             if (j) ss << ",";
             ss << kv.second.latency[j];
         }
-        ss << "]}";
+        ss << "]";
+        if (kv.second.has_ns) {
+            ss << ", \"total_latency_ns\":" << kv.second.total_latency_ns << ", \"latency_ns\":[";
+            for (size_t j = 0; j < kv.second.latency_ns.size(); ++j) {
+                if (j) ss << ",";
+                ss << kv.second.latency_ns[j];
+            }
+            ss << "]";
+        }
+        ss << "}";
     }
     ss << "}}";
     return ss.str();

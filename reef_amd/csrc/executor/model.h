@@ -47,6 +47,13 @@ class KernelProfile {
 public:
     std::vector<int> latency;  // microseconds at occupancy 1, 2, ...
     int total_latency = 0;
+    // The same in nanoseconds, from the optional keys "latency_ns" / "total_latency_ns" (kernels on
+    // this device run for a few microseconds, so whole microseconds are too coarse to decide what
+    // fits beside what; the reference's reader ignores keys it does not look up, model.cpp:57-80).
+    // Filled from the microsecond values when the keys are absent.
+    std::vector<int> latency_ns;
+    int total_latency_ns = 0;
+    bool has_ns = false;
 };
 
 class ModelProfile {

@@ -57,13 +57,8 @@ Status TransExecutor::init_rt_executor(const char* json_file_path, GPUModule_t m
         const uint32_t* lp = ki.launch_params;
         ka.kernel = kernel_funcs[i];
         ka.op = op_from_name(kernel_symbol(ki.name));
-        int tile = -1, mode = 0, taps = 0;
-        if (ka.op == REEF_OP_CONV2D && ki.attrs.size() > REEF_CONV_MODE) {
-            tile = ki.attrs[REEF_CONV_TILE];
-            mode = ki.attrs[REEF_CONV_MODE];
-            taps = ki.attrs[REEF_CONV_KH] * ki.attrs[REEF_CONV_KW];
-        }
-        ka.proxy_level = proxy_level(ka.op, tile, mode, taps);
+        ka.entry = 0;
+        GPU_RETURN_STATUS(reef_hal_module_kernel_entry(module, kernel_symbol(ki.name).c_str(), &ka.entry));
         ka.task_dim = dim3u(lp[0], lp[1], lp[2]);
         ka.thread_dim = dim3u(lp[3], lp[4], lp[5]);
         ka.block_num = (int)ka.task_dim.count();
@@ -78,17 +73,16 @@ Status TransExecutor::init_rt_executor(const char* json_file_path, GPUModule_t m
         ka.min_occupancy = std::max(layers, 1);
     }
 
-    // proxies: one per occupancy class that the code object provides
+    // proxies: every register class of the code object (trans_executor.cpp:100-124 resolves 20)
     proxy_kernels.clear();
-    for (int level = 0; level < kNumProxyLevels; level++) {
-        GPUFunction_t f;
-        const std::string name = REEF_PROXY_KERNEL_PREFIX() + std::to_string(proxy_class_of_level(level));
-        GPU_RETURN_STATUS(reef_hal_module_get_function(module, name.c_str(), &f));
-        proxy_kernels.push_back(f);
+    for (int p = 0; p < kNumProxies; p++) {
+        Proxy px;
+        px.name = REEF_PROXY_KERNEL_PREFIX() + kProxyNames[p];
+        GPU_RETURN_STATUS(reef_hal_module_get_function(module, px.name.c_str(), &px.kernel));
+        RETURN_STATUS(GPUConfig::get_kernel_resource(px.kernel, px.resource));
+        proxy_kernels.push_back(px);
     }
-    GPUConfig::KernelResource kr;
-    RETURN_STATUS(GPUConfig::get_kernel_resource(proxy_kernels[0], kr));
-    max_stack_size = kr.stack_size;
+    max_stack_size = proxy_kernels[0].resource.stack_size;
     return Status::Succ;
 }
 
@@ -145,31 +139,23 @@ int TransExecutor::occupancy_class(const GPUConfig::KernelResource& kr) {
     return std::max(1, std::min(8, 512 / v));
 }
 
-int TransExecutor::proxy_class_of_level(int level) {
-    static const int cls[kNumProxyLevels] = {8, 3, 2};
-    return cls[std::max(0, std::min(level, kNumProxyLevels - 1))];
-}
+const char* const TransExecutor::kProxyNames[] = {"8", "5", "4", "3", "3b", "2", "2b", "2c", "1"};
 
-// Which proxy holds the body of (op, tile, loader family): the bandwidth-bound ops
-// are in every proxy, a few matrix-core tiles in the classes whose register budget
-// fits them, and everything else in none (-1: that kernel is never merged).
-int TransExecutor::proxy_level(int op, int tile, int mode, int taps) {
-    if (op == REEF_OP_CONV2D) {
-        if (mode == REEF_CONV_MODE_DIRECT)
-            return ((tile == REEF_TILE_16x16k4 || tile == REEF_TILE_16x32k4) && (taps == 1 || taps == 9)) ? 1 : -1;
-        if (mode != REEF_CONV_MODE_GENERAL && mode != REEF_CONV_MODE_POINTWISE) return -1;
-        if (tile == REEF_TILE_64x64 || tile == REEF_TILE_128x32) return 1;
-        if (tile == REEF_TILE_128x64) return 2;
-        if (tile == REEF_TILE_32x32k4 || tile == REEF_TILE_64x32k2 || tile == REEF_TILE_32x64k2)
-            return 2;
-        return -1;
+int TransExecutor::select_proxy(const std::vector<Proxy>& proxies, const GPUConfig::KernelResource& l,
+                                const GPUConfig::KernelResource& r) {
+    if (l.stack_size > 0 || r.stack_size > 0) return -1;   // a proxy starts its wavefronts without scratch
+    const int arch = std::max(l.vgprs - l.agprs, r.vgprs - r.agprs);
+    const int acc = std::max(l.agprs, r.agprs);
+    const int sgprs = std::max(l.sgprs, r.sgprs);
+    for (size_t p = 0; p < proxies.size(); p++) {
+        const GPUConfig::KernelResource& pr = proxies[p].resource;
+        if (arch <= pr.vgprs - pr.agprs && acc <= pr.agprs && sgprs <= pr.sgprs) return (int)p;
     }
-    if (op == REEF_OP_GEMM || op == REEF_OP_NONE) return -1;
-    return 0;
+    return -1;
 }
 
-GPUFunction_t TransExecutor::get_proxy_kernel(int level) {
-    return proxy_kernels[std::max(0, std::min(level, (int)proxy_kernels.size() - 1))];
+GPUFunction_t TransExecutor::get_proxy_kernel(int index) {
+    return proxy_kernels[std::max(0, std::min(index, (int)proxy_kernels.size() - 1))].kernel;
 }
 
 }  // namespace executor

@@ -5,10 +5,10 @@
 // covers occupancy x num_cus physical workgroups that walk the logical tasks
 // with a persistent loop.
 //
-// What changed for MI355X: the side descriptor carries an op id and a
-// ReefOpDesc instead of a device function pointer and a float** table
-// (no pointer table in device memory, no proxy trampolines in assembly), and
-// the CU geometry (256 virtual CUs in 8 XCD groups) comes from the device.
+// What changed for MI355X: the side descriptor carries a ReefOpDesc (shapes and
+// pointers by value) instead of a float** table in device memory, the proxy
+// classes are the gfx950 register classes, and the CU geometry (256 virtual
+// CUs in 8 XCD groups) comes from the device.
 #pragma once
 #include "executor/executor_base.h"
 
@@ -24,8 +24,8 @@ public:
     class KernelArg {  // trans_executor.h:47-63
     public:
         GPUFunction_t kernel;
-        int op;                 // REEF_OP_* of this call (replaces funcion_pointer)
-        int proxy_level;        // smallest merge_framework class that contains this op, -1: none
+        int op;                 // REEF_OP_* of this call
+        uint64_t entry;         // device address of the kernel's first instruction (funcion_pointer, trans_executor.h:50)
         dim3u task_dim;
         dim3u thread_dim;
         int block_num;
@@ -47,21 +47,35 @@ public:
     // Waves per SIMD a register count allows on gfx950
     // (trans_executor.cpp:175-199 picks among 10 gfx906 classes the same way).
     static int occupancy_class(const GPUConfig::KernelResource& kr);
-    // The code object carries one proxy per occupancy class that matters for
-    // this kernel set: merge_framework_8 / _3 / _2 = levels 0..2.
-    static constexpr int kNumProxyLevels = 3;
-    static int proxy_class_of_level(int level);
-    static int proxy_level(int op, int tile, int mode, int taps = 0);
+    // The merge_framework_<n> proxies of the code object, most wavefronts per SIMD first.  A
+    // proxy fixes the register file of a merged launch: `resource.vgprs - resource.agprs`
+    // architectural VGPRs and `resource.agprs` accumulation registers.
+    struct Proxy {
+        std::string name;
+        GPUFunction_t kernel;
+        GPUConfig::KernelResource resource;
+    };
+    static const char* const kProxyNames[];
+    static constexpr int kNumProxies = 9;
+    // First proxy (= most wavefronts) whose two register ranges hold both kernels; -1 when a
+    // kernel needs scratch memory or more registers than any proxy has
+    // (trans_executor.cpp:175-199 picks among 10 + 10 gfx906 classes the same way).
+    static int select_proxy(const std::vector<Proxy>& proxies, const GPUConfig::KernelResource& l,
+                            const GPUConfig::KernelResource& r);
+    int select_proxy(const GPUConfig::KernelResource& l, const GPUConfig::KernelResource& r) const {
+        return select_proxy(proxy_kernels, l, r);
+    }
+    const std::vector<Proxy>& proxies() const { return proxy_kernels; }
 
 protected:
     Status init_rt_executor(const char* json_file_path, GPUModule_t module);
     virtual Status launch_kernel(int kernel_offset, GPUStream_t stream) override;
-    GPUFunction_t get_proxy_kernel(int level);
+    GPUFunction_t get_proxy_kernel(int index);
     void fill_side(ReefDkpSide& side, int kernel_offset, int layers, int task_num, int task_offset) const;
 
 protected:
     std::vector<KernelArg> trans_args;
-    std::vector<GPUFunction_t> proxy_kernels;
+    std::vector<Proxy> proxy_kernels;
     int max_stack_size;
 
     virtual std::string REEF_PROXY_KERNEL_PREFIX() const { return "merge_framework_"; }

@@ -27,7 +27,12 @@ int reef_hal_module_get_function(reef_module_t mod, const char* name, reef_funct
     return be()->module_get_function(mod, name, out);
 }
 int reef_hal_function_resource(reef_function_t fn, reef_kernel_resource* out) {
+    out->agprs = 0;   // a backend that knows nothing of accumulation registers leaves it
     return be()->function_resource(fn, out);
+}
+int reef_hal_module_kernel_entry(reef_module_t mod, const char* name, uint64_t* address) {
+    if (!be()->module_kernel_entry) { if (address) *address = 0; return 0; }   // a backend without device code
+    return be()->module_kernel_entry(mod, name, address);
 }
 int reef_hal_malloc(size_t bytes, int kind, reef_devptr_t* out) { return be()->malloc_(bytes, kind, out); }
 int reef_hal_free(reef_devptr_t ptr, int kind) { return be()->free_(ptr, kind); }
@@ -68,6 +73,21 @@ int reef_hal_graph_begin(reef_stream_t s) { return be()->graph_begin(s); }
 int reef_hal_graph_end(reef_stream_t s, reef_graph_t* out) { return be()->graph_end(s, out); }
 int reef_hal_graph_launch(reef_graph_t g, reef_stream_t s) { return be()->graph_launch(g, s); }
 int reef_hal_graph_destroy(reef_graph_t g) { return be()->graph_destroy(g); }
+int reef_hal_stream_set_completion(reef_stream_t s, int mode) {
+    return be()->stream_set_completion ? be()->stream_set_completion(s, mode) : 0;
+}
+int reef_hal_stream_progress(reef_stream_t s, uint32_t* submitted, uint32_t* done) {
+    if (!be()->stream_progress) { reef_hal_set_error("stream_progress: not in this backend"); return 1; }
+    return be()->stream_progress(s, submitted, done);
+}
+int reef_hal_stream_exit_ticks(reef_stream_t s, uint32_t seq, uint64_t* ticks) {
+    if (!be()->stream_exit_ticks) { if (ticks) *ticks = 0; return 0; }
+    return be()->stream_exit_ticks(s, seq, ticks);
+}
+int reef_hal_clock_sync(int64_t* host_ns, uint64_t* device_ticks, int64_t* err_ns, int* ticks_per_us) {
+    if (!be()->clock_sync) { reef_hal_set_error("clock_sync: not in this backend"); return 1; }
+    return be()->clock_sync(host_ns, device_ticks, err_ns, ticks_per_us);
+}
 int reef_hal_stream_clear_queue(reef_stream_t s, uint64_t* n_dropped) {
     return be()->stream_clear_queue(s, n_dropped);
 }

@@ -16,6 +16,10 @@
 #include "hal/code_object.h"
 #include "reef_hal.h"
 
+// hal_device.hip
+int reef_hal_hip_clock_probe(hipStream_t stream, int64_t* host_ns, uint64_t* device_ticks, int64_t* err_ns,
+                             int* ticks_per_us);
+
 struct reef_module_s {
     hipModule_t mod;
     std::map<std::string, reef::hal::KernelMeta> meta;
@@ -76,9 +80,14 @@ struct HeldRing {
 // HIP stream.  A launch counts as in flight from the moment the feeder takes it out
 // of the ring, so "ring dropped + at most `window` kernels not known complete" -- what
 // the rollback after a preemption relies on -- holds at every instant.
+constexpr int kExitRing = 8;   // launches whose exit clock is kept
+
 struct reef_stream_s {
     hipStream_t s;
     int window;
+    int completion = REEF_COMPLETE_STREAM_WRITE;
+    volatile uint64_t* exit_ticks = nullptr;   // pinned, kExitRing slots (slot = seq % kExitRing)
+    uint32_t* exit_count = nullptr;            // device counter of workgroups that have left
     uint32_t submitted;
     volatile uint32_t* done;
     HeldRing held;
@@ -227,6 +236,19 @@ int h_function_resource(reef_function_t f, reef_kernel_resource* out) {
     out->vgprs = f->meta.vgprs;
     out->sgprs = f->meta.sgprs;
     out->stack_size = f->meta.scratch;
+    out->agprs = f->meta.agprs;
+    return 0;
+}
+
+int h_module_kernel_entry(reef_module_t m, const char* name, uint64_t* address) {
+    if (!m || !name || !address) { reef_hal_set_error("reef_hal_module_kernel_entry: null argument"); return 1; }
+    hipDeviceptr_t var = nullptr;
+    size_t bytes = 0;
+    const std::string sym = std::string(name) + "_entry";
+    hipError_t e = hipModuleGetGlobal(&var, &bytes, m->mod, sym.c_str());
+    if (e != hipSuccess) return fail(e, ("hipModuleGetGlobal " + sym).c_str());
+    if (bytes != sizeof(uint64_t)) { reef_hal_set_error((sym + ": not an 8-byte variable").c_str()); return 1; }
+    HIPCHK(hipMemcpy(address, var, sizeof(uint64_t), hipMemcpyDeviceToHost));
     return 0;
 }
 
@@ -328,10 +350,18 @@ int h_stream_create(int window, reef_stream_t* out) {
     if (e != hipSuccess) { delete st; return fail(e, "hipStreamCreateWithFlags"); }
     if (window > 0) {
         void* p = nullptr;
-        e = hipHostMalloc(&p, 64, hipHostMallocDefault);
+        // one pinned block: the completion word, and from byte 64 on the exit clocks of the
+        // last launches (8-byte slots)
+        e = hipHostMalloc(&p, 64 + 8 * kExitRing, hipHostMallocDefault);
         if (e != hipSuccess) { hipStreamDestroy(st->s); delete st; return fail(e, "hipHostMalloc"); }
+        std::memset(p, 0, 64 + 8 * kExitRing);
         st->done = (volatile uint32_t*)p;
-        *st->done = 0;
+        st->exit_ticks = (volatile uint64_t*)((char*)p + 64);
+        void* cnt = nullptr;
+        e = hipMalloc(&cnt, 64);
+        if (e == hipSuccess) e = hipMemset(cnt, 0, 64);
+        if (e != hipSuccess) { hipStreamDestroy(st->s); hipHostFree(p); delete st; return fail(e, "hipMalloc"); }
+        st->exit_count = (uint32_t*)cnt;
         if (const char* v = std::getenv("REEF_HAL_FEEDER")) g_use_feeder = std::atoi(v) != 0;
         if (g_use_feeder) {
             st->has_feeder = true;
@@ -351,6 +381,7 @@ int h_stream_destroy(reef_stream_t st) {
     hipStreamSynchronize(st->s);
     hipStreamDestroy(st->s);
     if (st->done) hipHostFree((void*)st->done);
+    if (st->exit_count) hipFree(st->exit_count);
     delete st;
     return 0;
 }
@@ -360,12 +391,30 @@ int h_stream_destroy(reef_stream_t st) {
 int submit(reef_stream_t st, hipFunction_t fn, const uint32_t* g, const uint32_t* b, uint32_t lds,
            const void* kernarg, size_t bytes, uint32_t seq) {
     size_t sz = bytes;
+    alignas(16) char patched[kMaxHeldKernarg];
+    const bool in_kernel = seq != 0 && st->completion == REEF_COMPLETE_IN_KERNEL;
+    if (in_kernel) {
+        // the kernel signals by itself: its argument block starts with the completion record
+        if (bytes < sizeof(reef_hal_completion) || bytes > sizeof(patched)) {
+            reef_hal_set_error("reef_hal_launch: argument block cannot hold a completion record");
+            return 1;
+        }
+        std::memcpy(patched, kernarg, bytes);
+        reef_hal_completion c;
+        c.done_word = (uint32_t*)st->done;
+        c.exit_ticks = (uint64_t*)&st->exit_ticks[seq % kExitRing];
+        c.exit_count = st->exit_count;
+        c.seq = seq;
+        c.reserved = 0;
+        std::memcpy(patched, &c, sizeof(c));
+        kernarg = patched;
+    }
     void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(kernarg),
                      HIP_LAUNCH_PARAM_BUFFER_SIZE, &sz, HIP_LAUNCH_PARAM_END};
     HIPCHK(hipModuleLaunchKernel(fn, g[0], g[1], g[2], b[0], b[1], b[2], lds, st ? st->s : nullptr,
                                  nullptr, extra));
     if (seq != 0) {
-        HIPCHK(hipStreamWriteValue32(st->s, (void*)st->done, seq, 0));
+        if (!in_kernel) HIPCHK(hipStreamWriteValue32(st->s, (void*)st->done, seq, 0));
         st->enqueued.store(seq, std::memory_order_release);
     }
     return 0;
@@ -437,6 +486,13 @@ int h_stream_query(reef_stream_t st, int* idle) {
         if (!st->held.empty()) { *idle = 0; return 0; }
         // everything is on the device: the completion word says whether it is done
         *idle = in_flight(st) == 0 ? 1 : 0;
+        if (*idle && st->completion == REEF_COMPLETE_IN_KERNEL) {
+            // the last workgroup signals just before the kernel retires: "idle" is only reported
+            // once the runtime agrees, so that whoever reads the results next sees them all
+            hipError_t e = hipStreamQuery(st->s);
+            if (e == hipErrorNotReady) *idle = 0;
+            else if (e != hipSuccess) return fail(e, "hipStreamQuery");
+        }
         return st->feeder_error.load() ? 1 : 0;
     }
     hipError_t e = hipStreamQuery(st ? st->s : nullptr);
@@ -479,6 +535,41 @@ int h_stream_wait_device(reef_stream_t st) {
     }
     HIPCHK(hipStreamSynchronize(st ? st->s : nullptr));
     return 0;
+}
+int h_stream_set_completion(reef_stream_t st, int mode) {
+    if (!st || st->window <= 0) return 0;
+    if (const char* v = std::getenv("REEF_HAL_COMPLETION"))   // "stream": keep the stream write
+        if (std::strcmp(v, "stream") == 0) mode = REEF_COMPLETE_STREAM_WRITE;
+    std::lock_guard<std::mutex> lock(st->mtx);
+    if (st->submitted != 0) {
+        reef_hal_set_error("reef_hal_stream_set_completion: the stream has launches already");
+        return 1;
+    }
+    st->completion = mode;
+    return 0;
+}
+int h_stream_progress(reef_stream_t st, uint32_t* submitted, uint32_t* done) {
+    if (!st || st->window <= 0) {
+        reef_hal_set_error("reef_hal_stream_progress: needs a stream with a launch window");
+        return 1;
+    }
+    std::lock_guard<std::mutex> lock(st->mtx);
+    if (submitted) *submitted = st->submitted;
+    if (done) *done = *st->done;
+    return 0;
+}
+int h_stream_exit_ticks(reef_stream_t st, uint32_t seq, uint64_t* ticks) {
+    if (!ticks) return 1;
+    *ticks = 0;
+    if (!st || st->window <= 0 || st->completion != REEF_COMPLETE_IN_KERNEL || seq == 0) return 0;
+    const uint32_t done = *st->done;
+    if ((int32_t)(done - seq) < 0 || done - seq >= (uint32_t)kExitRing) return 0;   // not yet, or overwritten
+    *ticks = st->exit_ticks[seq % kExitRing];
+    return 0;
+}
+int h_clock_sync(int64_t* host_ns, uint64_t* device_ticks, int64_t* err_ns, int* ticks_per_us) {
+    if (!g_flag_stream) HIPCHK(hipStreamCreateWithFlags(&g_flag_stream, hipStreamNonBlocking));
+    return reef_hal_hip_clock_probe(g_flag_stream, host_ns, device_ticks, err_ns, ticks_per_us);
 }
 int h_graph_begin(reef_stream_t st) {
     if (!st || st->window > 0) {
@@ -569,6 +660,8 @@ const reef_hal_backend kHip = {
     h_event_create, h_event_destroy, h_event_record, h_event_sync, h_event_elapsed_us,
     h_memset_async, h_host_write32, h_stream_wait_device,
     h_graph_begin, h_graph_end, h_graph_launch, h_graph_destroy,
+    h_stream_set_completion, h_stream_progress, h_stream_exit_ticks, h_clock_sync,
+    h_module_kernel_entry,
 };
 
 }  // namespace

@@ -5,10 +5,11 @@
 // reference's tests only, src/reef/test/test.cpp:19).
 //
 //   raw    K(ReefOpDesc)                               plain launch, task = blockIdx.x
-//   be     K(int* preempted, int* task_slot, ReefOpDesc)
+//   be     K(ReefBeArgs) = (completion record, int* preempted, int* task_slot, ReefOpDesc)
 //          script/best_effort_kernel.py:22-29 restated: leave at once when the
 //          flag is set, poll it again inside long bodies, count completed
-//          workgroups in *task_slot.
+//          workgroups in *task_slot; the last workgroup to leave tells the
+//          launch-window stream that the kernel is done.
 //   trans  K(ReefDkpArgs) and merge_framework_<n>(ReefDkpArgs)
 //          script/generate_asm_loop.py:227-321 / transform_kernel.py:423-478
 //          restated: pick the side from the virtual CU id, then walk that
@@ -35,14 +36,17 @@ struct OpConv {
         return conv2d_body<T, MODE>(d, task, smem, p);
     }
 };
-template <int R, int TN = 1, int TM = 1, bool PRE = false>
+template <int R, int TN = 1, int TM = 1, bool PRE = false, bool ROWS = false>
 struct OpConvDirect {
     static constexpr int LDS = TileD16<TN, TM>::LDS_BYTES;
     template <class P>
     static __device__ __forceinline__ bool run(const ReefOpDesc& d, int task, char* smem, const P& p) {
-        return conv2d_direct_body<R, TN, TM, PRE>(d, task, smem, p);
+        return conv2d_direct_body<R, TN, TM, PRE, ROWS>(d, task, smem, p);
     }
 };
+// row form of the 3x3 convolution: G image rows x one 14-column segment per workgroup
+template <int G, int TM = 1>
+using OpConvRows = OpConvDirect<9, G, TM, false, true>;
 template <class T, bool TRANS_B>
 struct OpGemm {
     static constexpr int LDS = T::LDS_BYTES;
@@ -87,7 +91,11 @@ struct OpMocked {
     static constexpr int LDS = 0;
     template <class P>
     static __device__ __forceinline__ bool run(const ReefOpDesc& d, int task, char*, const P&) {
+#if REEF_FLAVOUR == 2
+        const int t = threadIdx.x;   // the padding flavour is launched with a flat workgroup
+#else
         const int t = threadIdx.x + threadIdx.y * blockDim.x + threadIdx.z * blockDim.x * blockDim.y;
+#endif
         if (t < 128) mocked_body<MUL>(d, task, t);
         return true;
     }
@@ -147,20 +155,44 @@ __device__ __forceinline__ bool dkp_walk(const ReefDkpArgs& a, DkpWalk& w) {
         OP::run(kernarg_at<ReefOpDesc>(0), (int)blockIdx.x, smem, NoPoll{});          \
     }
 #elif REEF_FLAVOUR == 1
+namespace {
+// A best-effort workgroup counts itself out as it leaves (finished or preempted).  The last
+// one of the launch puts the counter back to zero for the next launch on the stream, stores
+// the device clock and then the launch's sequence number where the host sees them.  All with
+// ordinary vector stores whose scope travels on the instruction; the clock is acknowledged
+// before the sequence number is sent.
+__device__ __forceinline__ void be_signal_exit(const ReefBeArgs& a, int t) {
+    if (a.done_word == nullptr) return;   // not on a launch-window stream
+    __syncthreads();                      // every thread of the workgroup is past its work
+    if (t != 0) return;
+    const unsigned total = gridDim.x * gridDim.y * gridDim.z;
+    const unsigned old = __hip_atomic_fetch_add(a.exit_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (old != total - 1) return;
+    __hip_atomic_store(a.exit_count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(a.exit_ticks, (uint64_t)wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __hip_atomic_store(a.done_word, a.seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+}  // namespace
 #define REEF_ENTRY(NAME, OP)                                                              \
-    extern "C" __global__ void __launch_bounds__(REEF_WG_THREADS)                         \
-    NAME(int* preempted, int* task_slot, ReefOpDesc) {                                    \
+    extern "C" __global__ void __launch_bounds__(REEF_WG_THREADS) NAME(ReefBeArgs) {      \
         __shared__ __align__(16) char smem[OP::LDS > 0 ? OP::LDS : 16];                   \
         __shared__ int s_pre;                                                             \
+        const ReefBeArgs& a = kernarg_at<ReefBeArgs>(0);                                  \
         const int t = threadIdx.x + threadIdx.y * blockDim.x + threadIdx.z * blockDim.x * blockDim.y; \
-        FlagPoll poll{preempted};                                                         \
+        FlagPoll poll{a.preempted};                                                       \
         if (t == 0) s_pre = poll.load();                                                  \
         __syncthreads();                                                                  \
-        if (s_pre) return;                                                                \
-        const bool done = OP::run(kernarg_at<ReefOpDesc>(16), (int)blockIdx.x, smem, poll); \
-        if (done && t == 0) atomicAdd(task_slot, 1);                                      \
+        bool done = false;                                                                \
+        if (!s_pre) done = OP::run(a.desc, (int)blockIdx.x, smem, poll);                  \
+        if (done && t == 0) atomicAdd(a.task_slot, 1);                                    \
+        be_signal_exit(a, t);                                                             \
     }
 #else
+// Every entry also publishes the address of its first instruction in a device variable
+// <name>_entry: what the reference reads out of the kernel descriptor on the host
+// (GPUConfig::get_kernel_address, src/reef/executor/hip/hip_impl.cpp:16-32) and passes to its
+// proxies as func_l / func_r.  A merge_framework_<n> proxy jumps there.
 #define REEF_ENTRY(NAME, OP)                                                           \
     extern "C" __global__ void __launch_bounds__(REEF_WG_THREADS) NAME(ReefDkpArgs) {  \
         __shared__ __align__(16) char smem[OP::LDS > 0 ? OP::LDS : 16];                \
@@ -172,7 +204,8 @@ __device__ __forceinline__ bool dkp_walk(const ReefDkpArgs& a, DkpWalk& w) {
             OP::run(side.desc, i, smem, NoPoll{});                                     \
             __syncthreads();                                                           \
         }                                                                              \
-    }
+    }                                                                                  \
+    extern "C" __device__ __attribute__((used)) void* const NAME##_entry = (void*)NAME;
 #endif
 
 REEF_ENTRY(reef_conv2d_128x128, OpConv<Tile128x128>)
@@ -217,6 +250,12 @@ REEF_ENTRY(reef_conv2d_p1_16x32k4, OpConvDirect<1 REEF_COMMA 2 REEF_COMMA 1 REEF
 REEF_ENTRY(reef_conv2d_p1_32x32d4, OpConvDirect<1 REEF_COMMA 2 REEF_COMMA 2 REEF_COMMA true>)
 REEF_ENTRY(reef_conv2d_d1_32x32d4, OpConvDirect<1 REEF_COMMA 2 REEF_COMMA 2>)
 REEF_ENTRY(reef_conv2d_d9_32x32d4, OpConvDirect<9 REEF_COMMA 2 REEF_COMMA 2>)
+REEF_ENTRY(reef_conv2d_r9_g1, OpConvRows<1>)
+REEF_ENTRY(reef_conv2d_r9_g2, OpConvRows<2>)
+REEF_ENTRY(reef_conv2d_r9_g4, OpConvRows<4>)
+REEF_ENTRY(reef_conv2d_r9_g7, OpConvRows<7>)
+REEF_ENTRY(reef_conv2d_r9_g2m2, OpConvRows<2 REEF_COMMA 2>)
+REEF_ENTRY(reef_conv2d_r9_g4m2, OpConvRows<4 REEF_COMMA 2>)
 REEF_ENTRY(reef_gemm_nt_128x128, OpGemm<Tile128x128 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nt_64x64, OpGemm<Tile64x64 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nt_32x128, OpGemm<Tile32x128 REEF_COMMA true>)
@@ -246,96 +285,61 @@ REEF_ENTRY(add, OpMocked<false>)
 REEF_ENTRY(multiply, OpMocked<true>)
 
 #if REEF_FLAVOUR == 2
-// ---- merge_framework_<n>: two different ops in one launch ------------------------
-// The reference's proxies jump to a device function pointer per side
-// (script/transform_kernel.py:689-718) and exist in ten variants whose register
-// budgets are patched to the gfx906 occupancy classes
-// (script/replace_register_usage.py:33-59).  Here the side carries an op id and
-// the proxy switches into the inlined body; the variants are the gfx950
-// occupancy classes that matter for this kernel set, <n> = wavefronts per SIMD:
-//   merge_framework_8  bandwidth-bound ops only                          (<= 64 registers)
-//   merge_framework_3  + conv (general, pointwise) tiles 64x64 / 128x32,
-//                        direct family with 1 and 9 taps, 16x16 and 16x32    (<= 168)
-//   merge_framework_2  + conv (general, pointwise) tile 128x64 and the
-//                        wave-split-K tiles                                   (<= 256)
-// Kernels outside these sets (the other tiles, the unaligned-K convolution, GEMM)
-// are never merged: they run single-sided through their own entry.
-// LDS is dynamic (the host passes the larger of the two sides' needs, as
-// src/reef/server/scheduler.cpp:643-649 does).
-namespace {
-template <int LEVEL>
-__device__ __forceinline__ void run_op(const ReefDkpSide& s, int task, char* smem) {
-    const ReefOpDesc& d = s.desc;
-    const NoPoll np{};
-    switch (s.op) {
-        case REEF_OP_CONV2D:
-            if (LEVEL >= 1) {
-                const int tile = d.attr[REEF_CONV_TILE];
-                if (d.attr[REEF_CONV_MODE] == REEF_CONV_MODE_DIRECT) {
-                    const int taps = d.attr[REEF_CONV_KH] * d.attr[REEF_CONV_KW];
-                    if (tile == REEF_TILE_16x16k4) {
-                        if (taps == 1) OpConvDirect<1>::run(d, task, smem, np);
-                        else if (taps == 9) OpConvDirect<9>::run(d, task, smem, np);
-                    } else if (tile == REEF_TILE_16x32k4) {
-                        if (taps == 1) OpConvDirect<1, 2>::run(d, task, smem, np);
-                        else if (taps == 9) OpConvDirect<9, 2>::run(d, task, smem, np);
-                    }
-                } else if (d.attr[REEF_CONV_MODE] == CONV_POINTWISE) {
-                    if (tile == REEF_TILE_64x64) OpConv<Tile64x64, CONV_POINTWISE>::run(d, task, smem, np);
-                    else if (tile == REEF_TILE_128x32) OpConv<Tile128x32, CONV_POINTWISE>::run(d, task, smem, np);
-                    else if (LEVEL >= 2 && tile == REEF_TILE_32x32k4) OpConv<Tile32x32k4, CONV_POINTWISE>::run(d, task, smem, np);
-                    else if (LEVEL >= 2 && tile == REEF_TILE_64x32k2) OpConv<Tile64x32k2, CONV_POINTWISE>::run(d, task, smem, np);
-                    else if (LEVEL >= 2 && tile == REEF_TILE_32x64k2) OpConv<Tile32x64k2, CONV_POINTWISE>::run(d, task, smem, np);
-                    else if (LEVEL >= 2 && tile == REEF_TILE_128x64) OpConv<Tile128x64, CONV_POINTWISE>::run(d, task, smem, np);
-                } else if (d.attr[REEF_CONV_MODE] == CONV_GENERAL) {
-                    if (tile == REEF_TILE_64x64) OpConv<Tile64x64, CONV_GENERAL>::run(d, task, smem, np);
-                    else if (tile == REEF_TILE_128x32) OpConv<Tile128x32, CONV_GENERAL>::run(d, task, smem, np);
-                    else if (LEVEL >= 2 && tile == REEF_TILE_128x64) OpConv<Tile128x64, CONV_GENERAL>::run(d, task, smem, np);
-                    else if (LEVEL >= 2 && tile == REEF_TILE_32x32k4) OpConv<Tile32x32k4, CONV_GENERAL>::run(d, task, smem, np);
-                    else if (LEVEL >= 2 && tile == REEF_TILE_64x32k2) OpConv<Tile64x32k2, CONV_GENERAL>::run(d, task, smem, np);
-                    else if (LEVEL >= 2 && tile == REEF_TILE_32x64k2) OpConv<Tile32x64k2, CONV_GENERAL>::run(d, task, smem, np);
-                }
-            }
-            break;
-        case REEF_OP_SPLITK_REDUCE:
-            // fewer partial loads in flight where the class allows 64 registers only
-            if (LEVEL == 0) splitk_reduce_body<4>(d, task);
-            else splitk_reduce_body<8>(d, task);
-            break;
-        case REEF_OP_DWCONV2D: dwconv2d_body(d, task); break;
-        case REEF_OP_POOL2D: pool2d_body(d, task); break;
-        case REEF_OP_GLOBAL_AVGPOOL: global_avgpool_body(d, task); break;
-        case REEF_OP_ELTWISE: eltwise_body(d, task); break;
-        case REEF_OP_DENSE: dense_body(d, task); break;
-        case REEF_OP_SOFTMAX: softmax_body(d, task); break;
-        case REEF_OP_LAYERNORM: layernorm_body(d, task); break;
-        case REEF_OP_BIAS_GELU: bias_gelu_body(d, task); break;
-        case REEF_OP_EMBEDDING: embedding_body(d, task); break;
-        case REEF_OP_COPY: copy_body(d, task); break;
-        case REEF_OP_TRANSPOSE: transpose_body(d, task); break;
-        case REEF_OP_MOCK_ADD: if (threadIdx.x < 128) mocked_body<false>(d, task, threadIdx.x); break;
-        case REEF_OP_MOCK_MULTIPLY: if (threadIdx.x < 128) mocked_body<true>(d, task, threadIdx.x); break;
-        default: break;
+// ---- merge_framework_<n>: two different kernels in one launch ---------------------------
+// As in the reference (script/transform_kernel.py:689-718) a proxy is a trampoline: it finds
+// the side of its workgroup and jumps to the first instruction of that side's own kernel,
+// whose address the host passes in (entry_l / entry_r, the reference's func_l / func_r).  The
+// kernel then runs exactly as if it had been launched directly: it reads the same argument
+// block, finds the same side and walks that side's tasks.  Any two kernels of this code object
+// can share a launch that way, and each runs the very code of its solo launch.
+//
+// What makes the jump legal is that a proxy starts its wavefronts in the state every kernel
+// here expects: argument block address in s[0:1], workgroup id in s2, packed work-item id in
+// v0, no other preloaded registers, no scratch, the same floating-point mode (all kernels are
+// built from this one source with one set of flags, none uses blockIdx.y/z or hidden
+// arguments), and LDS from offset 0 (the launch passes the larger static need of the two
+// sides as dynamic LDS, src/reef/server/scheduler.cpp:643-649).  The proxy's own kernel
+// descriptor fixes the register file of the launch, so, like the reference's ten variants
+// whose register counts are patched to the gfx906 occupancy classes
+// (script/replace_register_usage.py:33-59), there is one proxy per gfx950 register class:
+// <n> wavefronts per SIMD = 512 / n unified registers, split into V architectural VGPRs (the
+// accumulation registers start behind them) and A accumulation registers.  The counts are
+// claimed by naming the last register of each kind as clobbered.  The host picks the class
+// with the most wavefronts whose V and A hold both kernels (TransExecutor::select_proxy).
+//
+//   proxy                 V    A   unified  wavefronts/SIMD
+//   merge_framework_8     64    0     64    8   bandwidth-bound kernels
+//   merge_framework_5     96    0     96    5
+//   merge_framework_4     96   32    128    4
+//   merge_framework_3    136   32    168    3   direct / row convolutions, 64x64 and 128x32 staged tiles
+//   merge_framework_3b   152   16    168    3
+//   merge_framework_2    192   64    256    2   wide tiles
+//   merge_framework_2b   224   32    256    2
+//   merge_framework_2c   128  128    256    2
+//   merge_framework_1    256  256    512    1   everything else
+#define REEF_PROXY(NAME, LAST_V, LAST_A_CLOBBER)                                             \
+    extern "C" __global__ void __launch_bounds__(REEF_WG_THREADS) NAME(ReefDkpArgs) {        \
+        const ReefDkpArgs& a = kernarg_at<ReefDkpArgs>(0);                                   \
+        const void* kernarg = __builtin_amdgcn_kernarg_segment_ptr();                        \
+        const unsigned wg = __builtin_amdgcn_workgroup_id_x();                               \
+        const unsigned tid = __builtin_amdgcn_workitem_id_x();                               \
+        const int C = a.num_cus, X = a.num_xcds;                                             \
+        const int cu = (int)wg % C;                                                          \
+        const bool right = cu / X >= a.cu_partition / X;   /* the side test of dkp_walk */   \
+        const void* target = right ? a.entry_r : a.entry_l;                                  \
+        asm volatile("s_setpc_b64 %3"                                                        \
+                     :                                                                       \
+                     : "{s[0:1]}"(kernarg), "{s2}"(wg), "{v0}"(tid), "s"(target)             \
+                     : "s99", "vcc", LAST_V LAST_A_CLOBBER, "memory");                       \
+        __builtin_unreachable();                                                             \
     }
-}
-}  // namespace
-
-#define REEF_PROXY(N, LEVEL)                                                                \
-    extern "C" __global__ void __launch_bounds__(REEF_WG_THREADS)                           \
-    __attribute__((amdgpu_waves_per_eu(N, N))) merge_framework_##N(ReefDkpArgs) {           \
-        extern __shared__ __align__(16) char dyn_smem[];                                    \
-        const ReefDkpArgs& a = kernarg_at<ReefDkpArgs>(0);                                  \
-        DkpWalk w;                                                                          \
-        if (!dkp_walk(a, w)) return;                                                        \
-        const ReefDkpSide& side = w.right ? a.r : a.l;                                      \
-        int* slot = w.right ? a.task_slot_r : nullptr;                                      \
-        for (int i = w.idx; i < w.end; i += w.step) {                                       \
-            run_op<LEVEL>(side, i, dyn_smem);                                               \
-            __syncthreads();                                                                \
-            if (slot && threadIdx.x == 0) atomicAdd(slot, 1);                               \
-        }                                                                                   \
-    }
-REEF_PROXY(8, 0)
-REEF_PROXY(3, 1)
-REEF_PROXY(2, 2)
+REEF_PROXY(merge_framework_8, "v63", )
+REEF_PROXY(merge_framework_5, "v95", )
+REEF_PROXY(merge_framework_4, "v95", REEF_COMMA "a31")
+REEF_PROXY(merge_framework_3, "v135", REEF_COMMA "a31")
+REEF_PROXY(merge_framework_3b, "v151", REEF_COMMA "a15")
+REEF_PROXY(merge_framework_2, "v191", REEF_COMMA "a63")
+REEF_PROXY(merge_framework_2b, "v223", REEF_COMMA "a31")
+REEF_PROXY(merge_framework_2c, "v127", REEF_COMMA "a127")
+REEF_PROXY(merge_framework_1, "v255", REEF_COMMA "a255")
 #endif

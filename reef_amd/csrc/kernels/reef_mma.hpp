@@ -737,16 +737,39 @@ struct TileD16 {
     static constexpr int LDS_BYTES = 4 * SUBS * PART * 4 + 16;
 };
 
-template <int R, int TN, int TM = 1, bool PRE = false>
+template <int R, int TN, int TM = 1, bool PRE = false, bool ROWS = false>
 struct DirectGeom {
     static constexpr int CPL = R == 1 ? 8 : 1;   // channels per k slot and step
     static constexpr int RC = R * CPL;           // A values per lane and step (x TN B values and MFMAs)
     static constexpr int STEP_C = 16 * CPL;      // channels a workgroup consumes per step
+    // B values a lane loads per step: every tap of every pixel group, or (row form) one value
+    // per input row of the tile
+    static constexpr int NB = ROWS ? TN + 2 : TN * RC;
     // vector-memory instructions per step (PRE: two 128-bit loads each of input scale and shift)
-    static constexpr int LOADS = TM * ((RC / 4) + (RC % 4)) + TN * RC + (PRE ? 4 : 0);
-    // steps of loads in flight per wavefront: up to 60 load instructions, 2 to 6 steps
-    static constexpr int NS = 60 / LOADS < 2 ? 2 : (60 / LOADS > 6 ? 6 : 60 / LOADS);
+    static constexpr int LOADS = TM * ((RC / 4) + (RC % 4)) + NB + (PRE ? 4 : 0);
+    // steps of loads in flight per wavefront: up to 60 load instructions, 2 to 6 (row form: 8) steps
+    static constexpr int NS_MAX = ROWS ? 8 : 6;
+    static constexpr int NS = 60 / LOADS < 2 ? 2 : (60 / LOADS > NS_MAX ? NS_MAX : 60 / LOADS);
 };
+
+// Row form (ROWS; 3x3 filters, stride 1, padding 1; symbols reef_conv2d_r9_g<G>[m2]): the tile is
+// G image rows x one 14-column segment of the output.  Pixel group g is image row y0 + g and the
+// 16 lanes of a k slot are the columns of the segment: lanes 0..13 hold columns x0 .. x0 + 13,
+// lane 14 the column right of the segment and lane 15 the column left of it (zero outside the
+// image).  A lane loads ONE value per input row y0 - 1 .. y0 + G of its channel; the three
+// horizontal taps of a row are that value (kx = 1) and its rotations by one lane within the
+// 16-lane row (kx = 0: from lane - 1, lane 0 from lane 15; kx = 2: from lane + 1, lane 13 from
+// lane 14), the three vertical taps are the rows g, g + 1, g + 2.  Every input value is fetched
+// once per tile instead of once per tap: G + 2 loads per step instead of 9 G, so the loads of
+// up to eight K steps are in flight per wavefront.  Lanes 14 and 15 compute columns nobody
+// stores.  Same sum order over k as the tap form (channel-major steps, taps in filter order).
+constexpr int kRowSeg = 14;
+__device__ __forceinline__ float lane_from_left(float v) {   // lane i <- lane (i - 1) mod 16 of its row
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x121, 0xF, 0xF, false));
+}
+__device__ __forceinline__ float lane_from_right(float v) {  // lane i <- lane (i + 1) mod 16 of its row
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x12F, 0xF, 0xF, false));
+}
 
 // TN > 1 widens the tile along the pixels: every weight value a lane has loaded is multiplied
 // with TN pixel groups, so the weight rows -- the larger, cold operand -- are streamed by a
@@ -764,11 +787,12 @@ struct DirectGeom {
 // The eight input values a lane loads per step are eight consecutive channels, so their scales
 // and shifts are two 128-bit loads each; a channel past the split loads scale = shift = 0 and
 // contributes relu(0) = 0.  REEF_F_PRE_ACT; the two vectors follow the optional epilogue operands.
-template <int R, int TN, int TM, bool PRE, class Poll>
+template <int R, int TN, int TM, bool PRE, bool ROWS, class Poll>
 __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int task, char* smem_raw,
                                                    const Poll& poll) {
     static_assert(!PRE || R == 1, "the pre-activation form exists for 1-tap filters only");
-    typedef DirectGeom<R, TN, TM, PRE> G;
+    static_assert(!ROWS || R == 9, "the row form exists for 3x3 filters only");
+    typedef DirectGeom<R, TN, TM, PRE, ROWS> G;
     typedef TileD16<TN, TM> TD;
     constexpr int RC = G::RC, NS = G::NS;
     float* smem = (float*)smem_raw;
@@ -794,6 +818,10 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     const int rem = fused ? task / split_k : task - split * tiles;
     const int mt = rem / n_tiles, nt = rem - mt * n_tiles;
     const int m0 = mt * TD::BM, n0 = nt * TD::BN;
+    // row form: spatial tile nt -> (row tile, column segment)
+    const int segs = ROWS ? (W + kRowSeg - 1) / kRowSeg : 1;
+    const int y0 = ROWS ? (nt / segs) * TN : 0;
+    const int x0 = ROWS ? (nt % segs) * kRowSeg : 0;
     const int c_chunk = a[REEF_CONV_K_CHUNK] / R;
     const int cb = split * c_chunk;
     const int ce = min(C, cb + c_chunk);
@@ -810,8 +838,13 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
         om[h] = (unsigned)(m0 + 16 * h + orow);
 #pragma unroll
         for (int g = 0; g < TN; ++g) {
-            const unsigned on = (unsigned)(n0 + 16 * g + ocol);
-            ooff[h][g] = on < (unsigned)N ? (om[h] * (unsigned)N + on) * 4u : kOutside;
+            if (ROWS) {
+                const bool ok = ocol < kRowSeg && x0 + ocol < W && y0 + g < H;
+                ooff[h][g] = ok ? (om[h] * (unsigned)N + (unsigned)((y0 + g) * W + x0 + ocol)) * 4u : kOutside;
+            } else {
+                const unsigned on = (unsigned)(n0 + 16 * g + ocol);
+                ooff[h][g] = on < (unsigned)N ? (om[h] * (unsigned)N + on) * 4u : kOutside;
+            }
         }
     }
     ConvEpilogue ep;
@@ -844,8 +877,17 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
 #pragma unroll
     for (int h = 0; h < TM; ++h)
         va[h] = ((unsigned)(m0 + 16 * h + i16) * (unsigned)K + (unsigned)(lane_c * R)) * 4u;
-    unsigned vb[TN][R];
-    {
+    unsigned vb[ROWS ? TN + 2 : TN][ROWS ? 1 : R];
+    if (ROWS) {
+        // one value per input row: column of this lane (lane 15: left of the segment)
+        const int ix = i16 == 15 ? x0 - 1 : x0 + i16;
+#pragma unroll
+        for (int r = 0; r < TN + 2; ++r) {
+            const int iy = y0 - 1 + r;
+            const bool ok = (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
+            vb[ROWS ? r : 0][0] = ok ? (unsigned)(iy * W + ix) * 4u + (unsigned)lane_c * HW4 : kOutside;
+        }
+    } else {
         const int kw_ = a[REEF_CONV_KW];
 #pragma unroll
         for (int g = 0; g < TN; ++g) {
@@ -857,7 +899,7 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
                 const int iy = oy * a[REEF_CONV_SH] + ky - a[REEF_CONV_PH];
                 const int ix = ox * a[REEF_CONV_SW] + kx - a[REEF_CONV_PW];
                 const bool ok = n < N && (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
-                vb[g][t] = ok ? (unsigned)(iy * W + ix) * 4u + (unsigned)lane_c * HW4 : kOutside;
+                vb[ROWS ? 0 : g][ROWS ? 0 : t] = ok ? (unsigned)(iy * W + ix) * 4u + (unsigned)lane_c * HW4 : kOutside;
             }
         }
     }
@@ -871,7 +913,8 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     const rsrc_t rs_pt = make_rsrc(d.ptr[PRE ? ep.next + 1 : 0], (unsigned)C * 4u);
     const unsigned vpre = (unsigned)lane_c * 4u;
 
-    float ra[NS][TM][RC], rb[NS][TN][RC];
+    constexpr int NB = G::NB;
+    float ra[NS][TM][RC], rb[NS][NB];
     float rps[NS][PRE ? 8 : 1], rpt[NS][PRE ? 8 : 1];
     auto load_step = [&](int s, int step) {
         // offsets are below kOutside (a power of two), so or-ing it in moves them outside
@@ -909,16 +952,23 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
                 }
             }
         }
+        if (ROWS) {
 #pragma unroll
-        for (int g = 0; g < TN; ++g)
+            for (int r = 0; r < NB; ++r)
+                rb[s][r] = __builtin_bit_cast(
+                    float, __builtin_amdgcn_raw_buffer_load_b32(rs_b, (int)(vb[ROWS ? r : 0][0] | outm), (int)sb, 0));
+        } else {
 #pragma unroll
-            for (int q = 0; q < RC; ++q) {
-                // R > 1: tap q of the slot's channel; R == 1: channel q of the slot
-                const unsigned ob = (R > 1 ? vb[g][q] : vb[g][0]) | outm;
-                const unsigned sq = R > 1 ? sb : sb + (unsigned)q * HW4;
-                rb[s][g][q] = __builtin_bit_cast(
-                    float, __builtin_amdgcn_raw_buffer_load_b32(rs_b, (int)ob, (int)sq, 0));
-            }
+            for (int g = 0; g < TN; ++g)
+#pragma unroll
+                for (int q = 0; q < RC; ++q) {
+                    // R > 1: tap q of the slot's channel; R == 1: channel q of the slot
+                    const unsigned ob = (R > 1 ? vb[ROWS ? 0 : g][ROWS ? 0 : q] : vb[ROWS ? 0 : g][0]) | outm;
+                    const unsigned sq = R > 1 ? sb : sb + (unsigned)q * HW4;
+                    rb[s][ROWS ? 0 : g * RC + q] = __builtin_bit_cast(
+                        float, __builtin_amdgcn_raw_buffer_load_b32(rs_b, (int)ob, (int)sq, 0));
+                }
+        }
     };
 
     // oldest step first: the wait before a step's MFMAs counts the loads issued after its own
@@ -944,12 +994,31 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
             acc[h][g][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
         }
     auto mma_stage = [&](int s) {
+        if (ROWS) {
+            // taps of input row r: the loaded value and its two neighbours within the 16-lane row
+            float bt[NB][3];
+#pragma unroll
+            for (int r = 0; r < NB; ++r) {
+                bt[r][0] = lane_from_left(rb[s][r]);
+                bt[r][1] = rb[s][r];
+                bt[r][2] = lane_from_right(rb[s][r]);
+            }
+#pragma unroll
+            for (int q = 0; q < RC; ++q)
+#pragma unroll
+                for (int h = 0; h < TM; ++h)
+#pragma unroll
+                    for (int g = 0; g < TN; ++g)
+                        acc[h][g][q & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                            ra[s][h][q], bt[ROWS ? g + q / 3 : 0][q % 3], acc[h][g][q & 1], 0, 0, 0);
+            return;
+        }
         if (PRE) {
 #pragma unroll
             for (int g = 0; g < TN; ++g)
 #pragma unroll
                 for (int q = 0; q < RC; ++q)
-                    rb[s][g][q] = fmaxf(fmaf(rb[s][g][q], rps[s][PRE ? q : 0], rpt[s][PRE ? q : 0]), 0.0f);
+                    rb[s][ROWS ? 0 : g * RC + q] = fmaxf(fmaf(rb[s][ROWS ? 0 : g * RC + q], rps[s][PRE ? q : 0], rpt[s][PRE ? q : 0]), 0.0f);
         }
 #pragma unroll
         for (int q = 0; q < RC; ++q)
@@ -957,7 +1026,7 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
             for (int h = 0; h < TM; ++h)
 #pragma unroll
                 for (int g = 0; g < TN; ++g)
-                    acc[h][g][q & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[s][h][q], rb[s][g][q],
+                    acc[h][g][q & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[s][h][q], rb[s][ROWS ? 0 : g * RC + q],
                                                                             acc[h][g][q & 1], 0, 0, 0);
     };
     int pf = 0;

@@ -78,6 +78,7 @@ Status REEFScheduler::ensure_gpu() {
     if (mode == WaitPreempt) GPU_RETURN_STATUS(reef_hal_stream_create(0, &preempt_stream));
     GPU_RETURN_STATUS(reef_hal_malloc(4, REEF_MEM_DEVICE_FINEGRAINED, &preempt_flag));
     GPU_RETURN_STATUS(reef_hal_memset(preempt_flag, 0, 4));
+    sync_clock();
     gpu_ready = true;
     return Status::Succ;
 }
@@ -91,6 +92,8 @@ Status REEFScheduler::create_task_queue(std::shared_ptr<TaskQueue>& ret, bool rt
     } else {
         REEF_LOG_INFO("create be stream");
         GPU_RETURN_STATUS(reef_hal_stream_create(be_stream_device_queue_cap, &stream));
+        // best-effort kernels tell the stream themselves when they are done (ReefBeArgs)
+        GPU_RETURN_STATUS(reef_hal_stream_set_completion(stream, REEF_COMPLETE_IN_KERNEL));
     }
     ret = std::make_shared<TaskQueue>();
     ret->stream = stream;
@@ -315,9 +318,18 @@ void REEFScheduler::preempt_reset() {
     reef_hal_host_write32(preempt_flag, 1);
     const auto t1 = Steady::now();
     const uint32_t n = be_queue_cnt.load();
+    // launches each stream has handed to the device by now (a launch its feeder thread is
+    // passing to the runtime this instant included) and how many of them are still there
+    uint32_t target[max_num_be_queues], busy[max_num_be_queues];
     for (uint32_t i = 0; i < n; i++) {
         uint64_t dropped = 0;
         reef_hal_stream_clear_queue(be_queues[i]->stream, &dropped);
+        uint32_t sub = 0, done = 0;
+        target[i] = busy[i] = 0;
+        if (clk_valid && reef_hal_stream_progress(be_queues[i]->stream, &sub, &done) == 0) {
+            target[i] = sub;
+            busy[i] = sub - done;
+        }
         auto task = be_queues[i]->front();
         if (task && task->state.load() == TaskState::Executing) {
             task->kernel_offset = rollback_kernel_offset(task->launch_offset, (int)dropped,
@@ -338,10 +350,77 @@ void REEFScheduler::preempt_reset() {
     auto ns = [](Steady::time_point a, Steady::time_point b) {
         return (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(b - a).count();
     };
+    // the device's own account: when did the last workgroup of each stream's newest launch leave
+    if (clk_valid && wait_sync) {
+        const int64_t t0_ns = std::chrono::duration_cast<std::chrono::nanoseconds>(t1.time_since_epoch()).count();
+        int64_t worst = -1;
+        bool any = false, late = false;
+        std::lock_guard<std::mutex> lock(stats_mtx);
+        const size_t slot = preempt_device_ns.size();
+        for (uint32_t i = 0; i < n; i++) {
+            if (busy[i] == 0) continue;
+            any = true;
+            uint64_t ticks = 0;
+            reef_hal_stream_exit_ticks(be_queues[i]->stream, target[i], &ticks);
+            if (ticks == 0) {   // still inside the runtime call or on the device: completed later
+                late_samples.push_back(LateSample{slot, i, target[i], t0_ns});
+                late = true;
+                continue;
+            }
+            worst = std::max(worst, std::max<int64_t>(device_ticks_to_host_ns(ticks) - t0_ns, 0));
+        }
+        if (any) preempt_device_ns.push_back(late ? -(worst + 2) : worst);   // <= -1: open, holds the worst so far
+    }
     std::lock_guard<std::mutex> lock(stats_mtx);
     preempt_phase_ns[0] += ns(t0, t1);
     preempt_phase_ns[1] += ns(t1, t2);
     preempt_phase_ns[2] += ns(t2, t3);
+}
+
+// Host clock <-> device wall clock, one exchange (see reef_hal_clock_sync).
+void REEFScheduler::sync_clock() {
+    int64_t h = 0, err = 0;
+    uint64_t d = 0;
+    int tpu = 0;
+    if (reef_hal_clock_sync(&h, &d, &err, &tpu) != 0 || tpu <= 0) return;   // a backend without a device clock
+    std::lock_guard<std::mutex> lock(stats_mtx);
+    clk_host_ns = h;
+    clk_dev_ticks = d;
+    clk_err_ns = err;
+    clk_ticks_per_us = tpu;
+    clk_synced_at_ns = h;
+    clk_valid = true;
+}
+
+int64_t REEFScheduler::device_ticks_to_host_ns(uint64_t ticks) const {
+    const int64_t dt = (int64_t)(ticks - clk_dev_ticks);
+    return clk_host_ns + dt * 1000 / clk_ticks_per_us;
+}
+
+// Samples that waited for a launch which reached the device after the flag was raised: that
+// launch has long left by the time a real-time task is done.
+void REEFScheduler::resolve_late_samples() {
+    std::lock_guard<std::mutex> lock(stats_mtx);
+    for (const LateSample& l : late_samples) {
+        if (l.slot >= preempt_device_ns.size() || preempt_device_ns[l.slot] > -1) continue;
+        int64_t worst = -(preempt_device_ns[l.slot] + 2);
+        uint64_t ticks = 0;
+        if (l.queue < be_queue_cnt.load()) reef_hal_stream_exit_ticks(be_queues[l.queue]->stream, l.seq, &ticks);
+        if (ticks != 0) worst = std::max(worst, std::max<int64_t>(device_ticks_to_host_ns(ticks) - l.t0_ns, 0));
+        preempt_device_ns[l.slot] = -(worst + 2);
+    }
+    for (const LateSample& l : late_samples)
+        if (l.slot < preempt_device_ns.size() && preempt_device_ns[l.slot] <= -1)
+            preempt_device_ns[l.slot] = std::max<int64_t>(-(preempt_device_ns[l.slot] + 2), 0);
+    late_samples.clear();
+}
+
+size_t REEFScheduler::preempt_device_samples(int64_t* out_ns, size_t cap) const {
+    std::lock_guard<std::mutex> lock(stats_mtx);
+    size_t k = 0;
+    for (size_t i = 0; i < preempt_device_ns.size() && k < cap; i++)
+        if (preempt_device_ns[i] >= 0) out_ns[k++] = preempt_device_ns[i];
+    return k;
 }
 
 void REEFScheduler::preempt_phase_avg_ns(int64_t out[3]) const {
@@ -453,6 +532,14 @@ void REEFScheduler::execute_rt_task(std::shared_ptr<Task>& task) {
     }
     finish_task(task, Clock::now());
     REEF_LOG_INFO("rt task finish");
+    // off the real-time path: complete preemption samples that waited for a late launch, and
+    // renew the clock mapping when it is older than 100 ms (the two clocks drift)
+    if (clk_valid) {
+        if (!late_samples.empty()) resolve_late_samples();
+        const int64_t now = std::chrono::duration_cast<std::chrono::nanoseconds>(
+                                std::chrono::steady_clock::now().time_since_epoch()).count();
+        if (now - clk_synced_at_ns > 100000000) sync_clock();
+    }
 }
 
 // ---------------------------------------------------------------- dynamic kernel padding
@@ -477,23 +564,25 @@ REEFScheduler::PadDecision REEFScheduler::decide_padding(const TransExecutor::Ke
     const int merged_occupancy = GPUConfig::calculate_occupancy(d.resource, d.merged_block_size);
     if (merged_occupancy < rt.min_occupancy) return d;
 
+    // latencies in nanoseconds (from the profile's *_ns keys, else microseconds x 1000)
     int be_occupancy = 0;
-    const int rt_latency = rt.profile.total_latency;
-    const int be_budget = (int)((int64_t)rt_latency * slack_percent / 100);
+    const int64_t rt_latency = rt.profile.total_latency_ns;
+    const int64_t be_budget = rt_latency * slack_percent / 100;
+    const std::vector<int>& be_lat = be.profile.latency_ns;
     for (int j = merged_occupancy - 1; j >= 0; j--) {
-        if ((int)be.profile.latency.size() <= j) continue;
-        if (be.profile.latency[j] <= be_budget) {
+        if ((int)be_lat.size() <= j) continue;
+        if (be_lat[j] <= be_budget) {
             be_occupancy = j + 1;
             break;
         }
     }
     if (be_occupancy == 0) return d;
-    const int be_latency = std::max(be.profile.latency[be_occupancy - 1], 1);
+    const int64_t be_latency = std::max(be_lat[be_occupancy - 1], 1);
 
     const int partition = TransExecutor::cu_partition_for(rt.block_num, num_cus, num_xcds);
-    const int be_iters = be_budget / be_latency;
-    int be_blocks = (num_cus - partition) * be_iters * be_occupancy;
-    be_blocks = std::min(be_blocks, be.block_num - be_block_offset);
+    const int64_t be_iters = be_budget / be_latency;
+    int64_t be_blocks64 = (int64_t)(num_cus - partition) * be_iters * be_occupancy;
+    int be_blocks = (int)std::min<int64_t>(be_blocks64, be.block_num - be_block_offset);
     if (be_blocks <= 0) return d;
 
     d.merge = true;
@@ -510,9 +599,7 @@ void REEFScheduler::dynamic_kernel_padding(std::shared_ptr<Task>& rt_task) {
     const int num_xcds = (int)GPUConfig::get_num_xcds();
     std::vector<std::shared_ptr<Task>> complete_be_tasks;
     TimePoint current_time_point = Clock::now();
-    GPUConfig::KernelResource proxy_res[TransExecutor::kNumProxyLevels];
-    for (int l = 0; l < TransExecutor::kNumProxyLevels; l++)
-        GPUConfig::get_kernel_resource(rt_exe.get_proxy_kernel(l), proxy_res[l]);
+    const std::vector<TransExecutor::Proxy>& proxies = rt_exe.proxies();
 
     const int n_rt = (int)rt_exe.num_kernels();
     for (int i = 0; i < n_rt; i++) {
@@ -521,6 +608,7 @@ void REEFScheduler::dynamic_kernel_padding(std::shared_ptr<Task>& rt_task) {
         PadDecision dec;
         std::shared_ptr<Task> be_task;
         const TransExecutor::KernelArg* be_args = nullptr;
+        int proxy_idx = -1;
         const uint32_t n_q = be_queue_cnt.load();
         for (uint32_t q = 0; q < n_q; q++) {   // first queue whose head kernel fits (scheduler.cpp:533-602)
             auto cand = be_queues[q]->front();
@@ -537,14 +625,15 @@ void REEFScheduler::dynamic_kernel_padding(std::shared_ptr<Task>& rt_task) {
                 cand->sync_dirty = false;
             }
             const TransExecutor::KernelArg& ka = be_exe.trans_args[cand->kernel_offset];
-            // the proxy class that holds both bodies sets the register budget of the launch;
-            // a kernel that is in no proxy runs single-sided
-            if (rt_args.proxy_level < 0 || ka.proxy_level < 0) continue;
-            const int level = std::max(rt_args.proxy_level, ka.proxy_level);
-            PadDecision d = decide_padding(rt_args, ka, cand->block_offset, proxy_res[level], num_cus,
+            // the proxy whose two register ranges hold both kernels sets the register budget of
+            // the launch (scheduler.cpp:613-642 / trans_executor.cpp:175-199)
+            const int px = TransExecutor::select_proxy(proxies, rt_args.resource, ka.resource);
+            if (px < 0) continue;
+            PadDecision d = decide_padding(rt_args, ka, cand->block_offset, proxies[px].resource, num_cus,
                                            num_xcds, dkp_slack_percent);
             if (!d.merge) continue;
             dec = d;
+            proxy_idx = px;
             be_task = cand;
             be_args = &ka;
             break;
@@ -568,9 +657,10 @@ void REEFScheduler::dynamic_kernel_padding(std::shared_ptr<Task>& rt_task) {
             a.num_cus = num_cus;
             a.num_xcds = num_xcds;
             a.task_slot_r = nullptr;
+            a.entry_l = (const void*)(uintptr_t)rt_args.entry;
+            a.entry_r = (const void*)(uintptr_t)be_args->entry;
             if (be_task->start.time_since_epoch().count() == 0) be_task->start = current_time_point;
-            executor::GPUFunction_t proxy =
-                rt_exe.get_proxy_kernel(std::max(rt_args.proxy_level, be_args->proxy_level));
+            executor::GPUFunction_t proxy = rt_exe.get_proxy_kernel(proxy_idx);
             const uint32_t grid[3] = {(uint32_t)(dec.final_occupancy * num_cus), 1, 1};
             const uint32_t block[3] = {(uint32_t)dec.merged_block_size, 1, 1};
             reef_hal_launch(proxy, grid, block, (uint32_t)dec.resource.shared_memory, rt_queue->stream,

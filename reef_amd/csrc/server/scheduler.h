@@ -154,6 +154,15 @@ public:
     }
     // Copies the last `cap` preemption latencies (microseconds); returns how many.
     size_t preempt_latency_samples(int64_t* out, size_t cap) const;
+    // The same preemptions timed by the device: nanoseconds from the flag store (host clock)
+    // to the moment the last best-effort workgroup that was on the device left it (device wall
+    // clock written by that workgroup, mapped to the host clock through reef_hal_clock_sync).
+    // A launch that a stream's feeder thread was handing to the runtime while the flag was
+    // raised is counted too: its sample is completed when it has left the device.  Only
+    // preemptions that found best-effort kernels on the device have a sample.
+    size_t preempt_device_samples(int64_t* out_ns, size_t cap) const;
+    // Half the length of the host-device clock exchange the mapping rests on (nanoseconds), -1: no mapping.
+    int64_t clock_sync_error_ns() const { return clk_valid ? clk_err_ns : -1; }
     // Average nanoseconds per reset-based preemption spent in: raising the flag, dropping the
     // host queues + rollback, waiting for the device to drain (0 unless wait_sync).
     void preempt_phase_avg_ns(int64_t out[3]) const;
@@ -208,6 +217,17 @@ private:
     int64_t preempt_latency_max;
     std::vector<int64_t> preempt_samples;
     uint64_t preempt_phase_ns[3];
+    // device-side timing of preemptions
+    struct LateSample { size_t slot; uint32_t queue; uint32_t seq; int64_t t0_ns; };
+    std::vector<int64_t> preempt_device_ns;   // -1: still waiting for a late launch
+    std::vector<LateSample> late_samples;
+    bool clk_valid = false;
+    int64_t clk_host_ns = 0, clk_err_ns = 0, clk_synced_at_ns = 0;
+    uint64_t clk_dev_ticks = 0;
+    int clk_ticks_per_us = 100;
+    void sync_clock();
+    int64_t device_ticks_to_host_ns(uint64_t ticks) const;
+    void resolve_late_samples();
     mutable std::mutex stats_mtx;
     uint64_t kernel_sel_count;
     uint64_t kernel_sel_latency_sum;

@@ -171,7 +171,8 @@ class GraphBuilder:
             opt.append(self.param((cout,), 0.01).idx)
         act2 = dual_act or ACT_NONE
         t = force or tiling.choose(M, N, K, fused=fused_reduce, pointwise=(kh, kw) == (1, 1),
-                                   taps=kh * kw, direct=tiling.direct_ok(cin, kh, kw))
+                                   taps=kh * kw, direct=tiling.direct_ok(cin, kh, kw),
+                                   rows=tiling.rows_ok(kh, kw, sh, sw, ph, pw), image=(Ho, Wo))
         if t.get("fused"):
             fused_reduce = True       # the measured table asks for the split folded into the launch
         pre = []
@@ -190,7 +191,10 @@ class GraphBuilder:
         base = [cin, H, W, cout, Ho, Wo, kh, kw, sh, sw, ph, pw]
         # loader family: direct (only with its own tile), pointwise (1x1/s1/p0, N % 4 == 0),
         # unaligned (K % 4 != 0), general
-        if t["tile"] in tiling.DIRECT_TILES:
+        if t["tile"] in tiling.ROW_TILES:
+            assert tiling.rows_ok(kh, kw, sh, sw, ph, pw) and t["k_chunk"] % 144 == 0
+            mode, fam = 5, "r9_"
+        elif t["tile"] in tiling.DIRECT_TILES:
             assert tiling.direct_ok(cin, kh, kw, t["tile"]), (cin, kh, kw, t["tile"])
             assert t["k_chunk"] % (kh * kw * (8 if kh * kw == 1 else 1)) == 0
             mode, fam = (4, "p1_") if pre else (3, "d%d_" % (kh * kw))

@@ -29,7 +29,18 @@ TILES = {
     "16x32k4": (10, 16, 32, 0.40, 2),
     "16x64k4": (11, 16, 64, 0.40, 2),
     "32x32d4": (12, 32, 32, 0.40, 2),   # direct; the name differs from the staged 32x32k4
+    # row form of the direct 3x3 / stride 1 / padding 1 convolution (reef_conv2d_r9_<name>): BM output
+    # channels x G image rows x one 14-column segment; BN here is the nominal 16 G lanes it computes
+    "g1": (13, 16, 16, 0.40, 2),
+    "g2": (14, 16, 32, 0.40, 2),
+    "g4": (15, 16, 64, 0.40, 2),
+    "g7": (16, 16, 112, 0.40, 2),
+    "g2m2": (17, 32, 32, 0.40, 2),
+    "g4m2": (18, 32, 64, 0.40, 2),
 }
+# row form: image rows per tile
+ROW_TILES = {"g1": 1, "g2": 2, "g4": 4, "g7": 7, "g2m2": 2, "g4m2": 4}
+ROW_SEG = 14
 DIRECT_TILE = "16x16k4"
 DIRECT_TILES = ("16x16k4", "16x32k4", "16x64k4", "32x32d4")
 # filter sizes kh*kw each direct tile is compiled for
@@ -81,8 +92,27 @@ def direct_ok(cin, kh, kw, tile=DIRECT_TILE):
     return taps > 1 or cin % 8 == 0
 
 
+def rows_ok(kh, kw, sh, sw, ph, pw):
+    """Whether the row form has a kernel for this filter."""
+    return (kh, kw, sh, sw, ph, pw) == (3, 3, 1, 1, 1, 1)
+
+
+def forced_rows(tile, M, H, W, K, split=1):
+    """Launch geometry of a row-form tile: spatial tiles are G image rows x one 14-column segment."""
+    tid, bm, _, _, _ = TILES[tile]
+    G = ROW_TILES[tile]
+    bk = 16 * 9
+    k_chunk = math.ceil(math.ceil(K / split) / bk) * bk
+    s = math.ceil(K / k_chunk)
+    mt = math.ceil(M / bm)
+    nt = math.ceil(H / G) * math.ceil(W / ROW_SEG)
+    return dict(tile=tile, tile_id=tid, BM=bm, BN=16 * G, split_k=s, k_chunk=k_chunk, m_tiles=mt,
+                n_tiles=nt, tasks=s * mt * nt, est_us=1.0)
+
+
 def forced(tile, M, N, K, split=1, taps=1):
     """The launch geometry of a given tile and split-K factor (no cost model)."""
+    assert tile not in ROW_TILES, "row-form tiles take the image shape: forced_rows"
     tid, bm, bn, _, _ = TILES[tile]
     bk = step_k(tile, taps)
     k_chunk = math.ceil(math.ceil(K / split) / bk) * bk
@@ -106,12 +136,19 @@ def _steps_time(bm, bn, eff, steps):
 
 
 def choose(M, N, K, allow_split=True, tiles=None, max_split=32, fused=True, pointwise=False,
-           taps=1, direct=False):
+           taps=1, direct=False, rows=False, image=None):
     """Returns dict(tile, tile_id, BM, BN, split_k, k_chunk, m_tiles, n_tiles, tasks).
     Measured choices (tuned.py) win over the analytic model for the shapes they cover; an entry
     that names the direct tile counts only if the caller says the filter qualifies."""
     if allow_split and tiles is None and not fused:
         hit = TUNED.get((M, N, K, 1 if pointwise else 0))
+        if hit is not None and hit[0] in ROW_TILES:
+            if rows and image is not None:
+                t = forced_rows(hit[0], M, image[0], image[1], K, abs(hit[1]))
+                t["est_us"] = hit[2]
+                t["fused"] = hit[1] < 0
+                return t
+            hit = None
         if hit is not None and (hit[0] not in DIRECT_TILES or direct):
             # a negative split factor in the table: the split is folded inside the launch
             t = forced(hit[0], M, N, K, abs(hit[1]), taps)
@@ -119,7 +156,7 @@ def choose(M, N, K, allow_split=True, tiles=None, max_split=32, fused=True, poin
             t["fused"] = hit[1] < 0
             return t
     best = None
-    for name in (tiles or [t for t in TILES if t not in DIRECT_TILES]):
+    for name in (tiles or [t for t in TILES if t not in DIRECT_TILES and t not in ROW_TILES]):
         tid, bm, bn, eff, occ = TILES[name]
         m_tiles, n_tiles = math.ceil(M / bm), math.ceil(N / bn)
         nt = m_tiles * n_tiles
@@ -149,7 +186,7 @@ def choose(M, N, K, allow_split=True, tiles=None, max_split=32, fused=True, poin
 
 
 def lds_bytes(tile):
-    if tile in DIRECT_TILES:
+    if tile in DIRECT_TILES or tile in ROW_TILES:
         # four wavefronts x (BM/16)(BN/16) partial 16x16 tiles (skewed rows) + leave / last-arrival flags
         return 4 * (TILES[tile][1] // 16) * (TILES[tile][2] // 16) * 320 * 4 + 16
     _, bm, bn, _, _ = TILES[tile]

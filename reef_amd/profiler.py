@@ -6,7 +6,10 @@ solo duration of a kernel call and ``latency[j]`` the duration of one round of
 (consumed in src/reef/server/scheduler.cpp:509,565-572,589-590).  The reference
 ships profiles made by a ``profiler`` binary that is not in its repository
 (resource/Makefile:32-36); this module is the equivalent for gfx950.
-All values are integer microseconds, at least 1.
+``total_latency`` / ``latency`` are integer microseconds, at least 1, as the reference's files
+hold them; ``total_latency_ns`` / ``latency_ns`` carry the same measurements in nanoseconds
+(extra keys the reference's reader does not look up): kernels run for 3-15 us on this device,
+so whole microseconds cannot tell which best-effort kernel fits beside which real-time kernel.
 """
 import json
 import math
@@ -29,14 +32,16 @@ def measure_profile(model_dir, name, iters=10, warmup=2, levels=8):
         lat = []
         for j in range(min(levels, max(max_occ, 1))):
             us = exe.time_kernel_dkp(i, j + 1, min(blocks, (j + 1) * num_cus), warmup, iters)
-            lat.append(max(1, int(math.ceil(us))))
+            lat.append(max(1, int(round(us * 1000))))
             if (j + 1) * num_cus >= blocks:
                 # more layers cannot hold more of this kernel's workgroups
                 lat += [lat[-1]] * (min(levels, max(max_occ, 1)) - len(lat))
                 break
-        e = kl.setdefault(k["name"], {"total_latency": 0, "latency": lat})
-        e["total_latency"] = max(e["total_latency"], max(1, int(math.ceil(total))))
-        e["latency"] = [max(a, b) for a, b in zip(e["latency"], lat)]
+        e = kl.setdefault(k["name"], {"total_latency": 0, "latency": [], "total_latency_ns": 0, "latency_ns": lat})
+        e["total_latency_ns"] = max(e["total_latency_ns"], max(1, int(round(total * 1000))))
+        e["latency_ns"] = [max(a, b) for a, b in zip(e["latency_ns"], lat)]
+        e["total_latency"] = max(1, -(-e["total_latency_ns"] // 1000))
+        e["latency"] = [max(1, -(-v // 1000)) for v in e["latency_ns"]]
     lat_us, _ = exe.time_model(B.RUN_DEFAULT, 3, 10)
     prof = {"model_latency": int(math.ceil(float(lat_us.mean()))), "kernel_latency": kl}
     exe.close()

@@ -20,7 +20,10 @@ class OpDesc(ctypes.Structure):
 
 
 class BeArg(ctypes.Structure):
-    _fields_ = [("preempted", ctypes.c_void_p), ("task_slot", ctypes.c_void_p), ("desc", OpDesc)]
+    # ReefBeArgs of include/reef_kernels.h: the C-ABI layer's completion record comes first
+    _fields_ = [("done_word", ctypes.c_void_p), ("exit_ticks", ctypes.c_void_p), ("exit_count", ctypes.c_void_p),
+                ("seq", ctypes.c_uint32), ("reserved", ctypes.c_uint32),
+                ("preempted", ctypes.c_void_p), ("task_slot", ctypes.c_void_p), ("desc", OpDesc)]
 
 
 class DkpSide(ctypes.Structure):
@@ -31,7 +34,7 @@ class DkpSide(ctypes.Structure):
 class DkpArgs(ctypes.Structure):
     _fields_ = [("l", DkpSide), ("r", DkpSide), ("cu_partition", ctypes.c_int32),
                 ("num_cus", ctypes.c_int32), ("num_xcds", ctypes.c_int32), ("reserved", ctypes.c_int32),
-                ("task_slot_r", ctypes.c_void_p)]
+                ("task_slot_r", ctypes.c_void_p), ("entry_l", ctypes.c_void_p), ("entry_r", ctypes.c_void_p)]
 
 
 class DeviceInfo(ctypes.Structure):
@@ -54,8 +57,9 @@ CB_TYPE = ctypes.CFUNCTYPE(None, ctypes.c_char_p, ctypes.c_char_p, ctypes.c_void
 
 class FakeHal:
     def __init__(self):
-        if not os.path.exists(SO) or os.path.getmtime(SO) < os.path.getmtime(
-                os.path.join(HERE, "fake_hal", "fake_hal.cpp")):
+        deps = [os.path.join(HERE, "fake_hal", "fake_hal.cpp"),
+                os.path.join(os.path.dirname(HERE), "include", "reef_hal.h")]   # the backend table's layout
+        if not os.path.exists(SO) or os.path.getmtime(SO) < max(os.path.getmtime(d) for d in deps):
             subprocess.check_call(["make", "-B", "-C", os.path.join(HERE, "fake_hal")],
                                   stdout=subprocess.DEVNULL)
         self.core = B.lib()

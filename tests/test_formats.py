@@ -204,11 +204,15 @@ def test_code_object_metadata_reader():
     assert L.reef_code_object_kernel_meta(code_object("be").encode(), b"reef_pool2d", out) == 0
     assert out[5] >= 192           # + the compiler's hidden arguments
     assert L.reef_code_object_kernel_meta(code_object("trans").encode(), b"reef_pool2d", out) == 0
-    assert out[5] == 408           # sizeof(ReefDkpArgs)
-    for cls, budget in ((8, 64), (3, 168), (2, 256)):
+    assert out[5] == 424           # sizeof(ReefDkpArgs)
+    # the proxies claim exactly the register ranges of their class: (arch VGPRs, accumulation registers)
+    for cls, (arch, acc) in {"8": (64, 0), "5": (96, 0), "4": (96, 32), "3": (136, 32), "3b": (152, 16),
+                             "2": (192, 64), "2b": (224, 32), "2c": (128, 128), "1": (256, 256)}.items():
         assert L.reef_code_object_kernel_meta(code_object("trans").encode(),
-                                              b"merge_framework_%d" % cls, out) == 0
-        assert out[4] == 0 and out[0] <= budget, "proxy class %d: no scratch, registers within budget" % cls
+                                              ("merge_framework_" + cls).encode(), out) == 0
+        assert out[4] == 0 and out[3] == 0 and out[5] == 424, "proxy %s: no scratch, no LDS of its own" % cls
+        assert (out[0] - out[1], out[1]) == (arch, acc), (cls, list(out))
+        assert 512 // ((out[0] + 7) // 8 * 8) == int(cls[0]), "proxy %s: wavefronts per SIMD" % cls
     # no kernel of any flavour spills
     for fl in ("raw", "be", "trans"):
         for k in ("reef_conv2d_128x128", "reef_conv2d_pw_64x64", "reef_conv2d_u_64x128", "reef_gemm_nt_128x128",
@@ -219,8 +223,7 @@ def test_code_object_metadata_reader():
 
 def test_benchmark_models_name_only_compiled_kernels_without_scratch():
     """Every kernel symbol the generator emits for the four CNNs and BERT exists in all three
-    code objects, uses no scratch memory, and the three proxies stay inside their register
-    classes (waves per SIMD 8 / 3 / 2 on a 512-entry register file)."""
+    code objects, uses no scratch memory, and has a proxy whose register ranges hold it."""
     import ctypes
     from reef_amd.modelgen import nets
     from reef_amd.paths import code_object
@@ -237,9 +240,15 @@ def test_benchmark_models_name_only_compiled_kernels_without_scratch():
             assert L.reef_code_object_kernel_meta(co, sym.encode(), out) == 0, (fl, sym)
             assert out[4] == 0, "%s in %s.co uses %d bytes of scratch" % (sym, fl, out[4])
     co = code_object("trans").encode()
-    for n, budget in ((8, 64), (3, 168), (2, 256)):
-        assert L.reef_code_object_kernel_meta(co, ("merge_framework_%d" % n).encode(), out) == 0
-        assert out[4] == 0 and out[0] + out[1] <= budget, (n, list(out))
+    # every one of those kernels fits the register ranges of some proxy with any other
+    proxies = []
+    for n in ("8", "5", "4", "3", "3b", "2", "2b", "2c", "1"):
+        assert L.reef_code_object_kernel_meta(co, ("merge_framework_" + n).encode(), out) == 0
+        assert out[4] == 0
+        proxies.append((out[0] - out[1], out[1], out[2]))
+    for sym in sorted(symbols):
+        assert L.reef_code_object_kernel_meta(co, sym.encode(), out) == 0
+        assert any(out[0] - out[1] <= v and out[1] <= a and out[2] <= s for v, a, s in proxies), (sym, list(out))
 
 
 def test_direct_tile_geometry():
@@ -277,3 +286,76 @@ def test_gemm_tile_choice_follows_the_line_rule():
     for t in tiling.GEMM_DIRECT_TILES:
         f = tiling.forced(t, 128, 768, 768, 1)
         assert f["split_k"] == 1 and f["tasks"] == f["m_tiles"] * f["n_tiles"]
+
+
+def _kernel_descriptors(path):
+    """name -> 64-byte kernel descriptor, from the code object's dynamic symbols <name>.kd."""
+    import struct
+    blob = open(path, "rb").read()
+    magic = b"__CLANG_OFFLOAD_BUNDLE__"
+    if blob.startswith(magic):          # hipcc --genco wraps the ELF in an offload bundle
+        n, = struct.unpack_from("<Q", blob, len(magic))
+        pos = len(magic) + 8
+        for _ in range(n):
+            off, size, tlen = struct.unpack_from("<QQQ", blob, pos)
+            triple = blob[pos + 24:pos + 24 + tlen]
+            pos += 24 + tlen
+            if b"gfx950" in triple:
+                blob = blob[off:off + size]
+                break
+    assert blob[:4] == b"\x7fELF" and blob[4] == 2
+    shoff, = struct.unpack_from("<Q", blob, 0x28)
+    shentsize, shnum, _ = struct.unpack_from("<HHH", blob, 0x3A)
+    secs = [struct.unpack_from("<IIQQQQIIQQ", blob, shoff + i * shentsize) for i in range(shnum)]
+    out = {}
+    for (_, typ, _, _, off, size, link, _, _, entsize) in secs:
+        if typ not in (2, 11):      # SHT_SYMTAB, SHT_DYNSYM
+            continue
+        stroff = secs[link][4]
+        for k in range(size // entsize):
+            st_name, _, _, shndx, value, _ = struct.unpack_from("<IBBHQQ", blob, off + k * entsize)
+            end = blob.index(b"\0", stroff + st_name)
+            name = blob[stroff + st_name:end].decode()
+            if not name.endswith(".kd") or shndx == 0 or shndx >= shnum:
+                continue
+            sec = secs[shndx]
+            fo = sec[4] + (value - sec[3])
+            out[name[:-3]] = blob[fo:fo + 64]
+    return out
+
+
+def test_every_padding_kernel_starts_its_wavefronts_in_the_same_state():
+    """A merge_framework_<n> proxy jumps to the first instruction of another kernel of the code
+    object, so all of them must ask the hardware for the same initial wavefront state: the same
+    preloaded scalar registers (argument block address only, then the workgroup id x), no scratch,
+    no hidden arguments, the same floating-point mode bits."""
+    import struct
+    from reef_amd.paths import code_object
+    kds = _kernel_descriptors(code_object("trans"))
+    assert len(kds) > 80 and "merge_framework_3" in kds and "reef_conv2d_d9_16x32k4" in kds
+    ref = None
+    for name, kd in sorted(kds.items()):
+        group_seg, private_seg, kernarg = struct.unpack_from("<III", kd, 0)
+        rsrc3, rsrc1, rsrc2 = struct.unpack_from("<III", kd, 44)
+        props, preload = struct.unpack_from("<HH", kd, 56)
+        state = {
+            "private_segment": private_seg,
+            "kernarg_size": kernarg,
+            "float_mode_dx10_ieee": (rsrc1 >> 12) & 0xFFF & ~0x100,      # rounding, denormals, priv=0, dx10 clamp, debug, ieee
+            "enable_private_segment": rsrc2 & 1,
+            "user_sgpr_count": (rsrc2 >> 1) & 0x1F,
+            "workgroup_id_xyz_info": (rsrc2 >> 7) & 0xF,
+            "exceptions": rsrc2 >> 13,
+            "kernel_code_properties": props,
+            "kernarg_preload": preload,
+            "tg_split": (rsrc3 >> 16) & 1,
+        }
+        if ref is None:
+            ref = state
+            # argument block address in s[0:1] is the only user register; workgroup id x follows in s2
+            assert state["user_sgpr_count"] == 2 and state["kernel_code_properties"] == 0x8
+            assert state["workgroup_id_xyz_info"] == 1 and state["private_segment"] == 0
+            assert state["kernarg_size"] == 424 and state["kernarg_preload"] == 0
+        assert state == ref, (name, state, ref)
+        if name.startswith("merge_framework_"):
+            assert group_seg == 0, name     # LDS of a merged launch is all dynamic, from offset 0

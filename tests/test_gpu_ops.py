@@ -50,8 +50,13 @@ def test_conv_tiles(tmp_path, tile, case):
     if tile in tiling.DIRECT_TILES and not tiling.direct_ok(cin, kh, kw, tile):
         pytest.skip("the direct family is compiled for 1x1 (Cin % 8 == 0) and 3-, 7-, 9-tap filters, "
                     "its wide tiles for 1 and 9 taps")
-    y = g.conv2d(x, cout, k, s, p, bias=True, act=MB.ACT_RELU,
-                 force=forced(tile, cout, Ho * Wo, cin * kh * kw, 1, kh * kw))
+    if tile in tiling.ROW_TILES:
+        if not tiling.rows_ok(kh, kw, s, s, ph, pw):
+            pytest.skip("the row form is compiled for 3x3 / stride 1 / padding 1")
+        f = tiling.forced_rows(tile, cout, Ho, Wo, cin * 9, 1)
+    else:
+        f = forced(tile, cout, Ho * Wo, cin * kh * kw, 1, kh * kw)
+    y = g.conv2d(x, cout, k, s, p, bias=True, act=MB.ACT_RELU, force=f)
     g.mark_output(y)
     exe, orc, model = run_both(g, tmp_path, {"data": rnd(cin, H, W)})
     compare_storages(exe, orc, model, what="conv %s %s" % (tile, case))
@@ -113,6 +118,49 @@ def test_fused_split_k_equals_plain_split_k_bitwise(tmp_path, tile, split):
             np.testing.assert_array_equal(exe.get_data(t_plain.idx, t_plain.size),
                                           exe.get_data(t_fused.idx, t_fused.size))
         exe.execute()
+
+
+@pytest.mark.parametrize("split,fused", [(1, False), (2, False), (2, True), (5, True)])
+@pytest.mark.parametrize("shape", [(72, 13, 13, 88), (40, 30, 37, 24), (32, 7, 7, 48), (16, 5, 50, 16)])
+@pytest.mark.parametrize("tile", list(tiling.ROW_TILES))
+def test_conv_row_form(tmp_path, tile, shape, split, fused):
+    """Row form of the 3x3 / stride 1 / padding 1 convolution (G image rows x 14-column segments,
+    horizontal taps from neighbouring lanes): images narrower and wider than a segment, widths
+    that are no multiple of 14, heights that are no multiple of G, ragged M and Cin; every
+    epilogue form, a second output and a channel slice; single pass, separate reduce, and the
+    split folded inside the launch, which must give the bits of the separate reduce."""
+    cin, H, W, cout = shape
+    g = MB.GraphBuilder("r")
+    x = g.input("data", (cin, H, W))
+    res = g.input("res", (cout, H, W))
+    f = tiling.forced_rows(tile, cout, H, W, cin * 9, split)
+    if f["split_k"] != split:
+        pytest.skip("too few channels for this split")
+    fu = fused if split > 1 else None
+    outs = {}
+    for variant in ((False, True) if fused else (fused,)):
+        g._np = 0
+        v = variant if split > 1 else None
+        a = g.conv2d(x, cout, 3, 1, 1, bias=True, act=MB.ACT_RELU, force=f, fused_reduce=v)
+        b, b2 = g.conv2d(x, cout, 3, 1, 1, bias=False, act=MB.ACT_NONE, residual=res,
+                         dual_act=MB.ACT_RELU, force=f, fused_reduce=v)
+        c = g.conv2d(x, cout, 3, 1, 1, bias=False, act=MB.ACT_RELU6, residual=res, affine=True,
+                     force=f, fused_reduce=v)
+        cat = g.temp((cout + 24, H, W))
+        e = g.conv2d(x, cout, 3, 1, 1, bias=True, act=MB.ACT_NONE, force=f, fused_reduce=v, out=cat,
+                     out_channel=16)
+        outs[variant] = (a, b, b2, c, cat)
+    g.mark_output(outs[fused][0])
+    seen = {}
+    g.params = [kv for kv in g.params if not (kv[0] in seen or seen.setdefault(kv[0], 0))]
+    exe, orc, model = run_both(g, tmp_path, {"data": rnd(cin, H, W), "res": rnd(cout, H, W)})
+    compare_storages(exe, orc, model, what="row form %s %s x%d fused=%s" % (tile, shape, split, fused))
+    if fused:
+        for rerun in range(2):
+            for t_plain, t_fused in zip(outs[False], outs[True]):
+                np.testing.assert_array_equal(exe.get_data(t_plain.idx, t_plain.size),
+                                              exe.get_data(t_fused.idx, t_fused.size))
+            exe.execute()
 
 
 @pytest.mark.parametrize("split,fused", [(1, False), (2, False), (2, True), (3, True)])
