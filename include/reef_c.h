@@ -183,6 +183,21 @@ int reef_ops_init(const char* kernels_co_path);
  * and returns them before it returns (it waits for the stream then). */
 int reef_ops_conv2d(const reef_conv2d_desc* c, const float* in, const float* w, const float* bias,
                     const float* residual, float* out, void* stream);
+/* The same convolution for callers that cannot allocate (code under stream capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * The partial tiles and arrival counters of a split K live in a fixed array in device memory
+ * that belongs to this library (4 MiB of partial tiles + 16384 counters per GPU, held until the
+ * process ends); the call allocates and frees nothing, enqueues a small fill kernel that zeroes
+ * the counters it needs and then the convolution, and returns without waiting.  A layer whose
+ * split needs more than the array holds is refused with Status::Fail and a message saying so
+ * (reef_ops_scratch_bytes() = bytes of partial tiles the array holds; the library's own choice
+ * of split stays within it for every shape it accepts).  reef_ops_init must have
+ * run with the device current.  Every call on a GPU uses that GPU's one array: calls that
+ * overlap on one GPU (two streams, two threads) race on it -- serialise them.  Bit-identical
+ * to reef_ops_conv2d. */
+int reef_ops_conv2d_noalloc(const reef_conv2d_desc* c, const float* in, const float* w, const float* bias,
+                            const float* residual, float* out, void* stream);
+size_t reef_ops_scratch_bytes(void);
 
 /* GPUConfig (src/reef/executor/hip/hip_impl.cpp:9-74) */
 int reef_gpuconfig_num_cus(void);

@@ -4,8 +4,12 @@
 // K across workgroups when the layer alone cannot fill the device, and folds the split inside
 // the launch (partial tiles + arrival counters, summed in ascending split order).
 //
-// reef_ops_conv2d (include/reef_c.h) takes the partial-tile workspace and the counters from
-// hipMalloc for the duration of the call.
+// Two entry points (include/reef_c.h):
+//   reef_ops_conv2d          takes the partial-tile workspace and the counters from hipMalloc
+//                            for the duration of the call;
+//   reef_ops_conv2d_noalloc  takes them from a fixed array in device memory that belongs to
+//                            this library -- no allocation of any kind, for callers that
+//                            cannot allocate (stream capture, serving loops).
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -20,6 +24,16 @@
 
 namespace {
 
+// ---- scratch of the allocation-free entry point -------------------------------------------
+// [0, kCounterBytes): one arrival counter per output tile; [kCounterBytes, ..): partial tiles.
+constexpr size_t kCounterBytes = 64 * 1024;
+// The plan below puts at most 256 workgroups on a split layer and a workgroup's tile has at
+// most 64 x 64 outputs, so no layer needs more than 256 x 4096 partial sums = 4 MiB; the
+// size check in the entry point guards that bound.
+constexpr size_t kWorkspaceBytes = 4u * 1024 * 1024;
+constexpr size_t kScratchBytes = kCounterBytes + kWorkspaceBytes;
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kScratchBytes];
+
 // Fills n 32-bit words (a captured stream must not hold a memset node: a small kernel instead).
 __global__ void fill_words(uint32_t* p, uint32_t value, size_t n) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -32,6 +46,7 @@ struct DeviceState {
     hipModule_t module = nullptr;
     hipFunction_t rows_g2 = nullptr, d1 = nullptr, d3 = nullptr, d7 = nullptr, d9 = nullptr, general = nullptr,
                   unaligned = nullptr;
+    unsigned char* scratch_ptr = nullptr;   // device address of `scratch` on this GPU
 };
 DeviceState g_dev[kMaxDevices];
 std::mutex g_mtx;
@@ -43,9 +58,9 @@ int fail(const std::string& m) {
 }
 int hip_fail(hipError_t e, const char* what) { return fail(std::string(what) + ": " + hipGetErrorString(e)); }
 
-// Loads the kernels.  Once per device, with
+// Loads the kernels and finds this GPU's copy of the scratch array.  Once per device, with
 // that device current.
-int ensure_device(DeviceState** out) {
+int ensure_device(DeviceState** out, bool may_set_up = true) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
@@ -53,6 +68,7 @@ int ensure_device(DeviceState** out) {
     std::lock_guard<std::mutex> lock(g_mtx);
     DeviceState& d = g_dev[dev];
     if (!d.ready) {
+        if (!may_set_up) return fail("reef_ops_conv2d_noalloc: reef_ops_init has not run with this device current");
         if (g_co_path.empty()) return fail("reef_ops_init has not been called");
         e = hipModuleLoad(&d.module, g_co_path.c_str());
         if (e != hipSuccess) return hip_fail(e, ("hipModuleLoad " + g_co_path).c_str());
@@ -65,6 +81,10 @@ int ensure_device(DeviceState** out) {
             e = hipModuleGetFunction(s.fn, d.module, s.name);
             if (e != hipSuccess) return hip_fail(e, (std::string("hipModuleGetFunction ") + s.name).c_str());
         }
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+        d.scratch_ptr = (unsigned char*)p;
         d.ready = true;
     }
     *out = &d;
@@ -173,6 +193,8 @@ int reef_ops_init(const char* kernels_co_path) {
     return ensure_device(&d);
 }
 
+size_t reef_ops_scratch_bytes(void) { return kWorkspaceBytes; }
+
 int reef_ops_conv2d(const reef_conv2d_desc* c, const float* in, const float* w, const float* bias,
                     const float* residual, float* out, void* stream) {
     DeviceState* d = nullptr;
@@ -200,6 +222,32 @@ int reef_ops_conv2d(const reef_conv2d_desc* c, const float* in, const float* w, 
         if (rc == 0 && e != hipSuccess) rc = hip_fail(e, "hipStreamSynchronize");
     }
     return rc;
+}
+
+int reef_ops_conv2d_noalloc(const reef_conv2d_desc* c, const float* in, const float* w, const float* bias,
+                            const float* residual, float* out, void* stream) {
+    DeviceState* d = nullptr;
+    if (int rc = ensure_device(&d, false)) return rc;   // set-up (module load, scratch address) is reef_ops_init's
+    Plan p;
+    if (int rc = make_plan(*d, c, in, w, bias, residual, out, &p)) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    if (p.split_k > 1) {
+        if (p.ws_floats * 4 > kWorkspaceBytes || (size_t)p.tiles * 4 > kCounterBytes) {
+            char msg[200];
+            std::snprintf(msg, sizeof(msg),
+                          "reef_ops_conv2d_noalloc: the layer needs %zu bytes of partial tiles and %d counters; "
+                          "the fixed scratch holds %zu bytes and %zu counters",
+                          p.ws_floats * 4, p.tiles, kWorkspaceBytes, kCounterBytes / 4);
+            return fail(msg);
+        }
+        uint32_t* cnt = (uint32_t*)d->scratch_ptr;
+        float* ws = (float*)(d->scratch_ptr + kCounterBytes);
+        // the array keeps what the last call left: the counters of this launch start at zero
+        hipLaunchKernelGGL(fill_words, dim3((p.tiles + 255) / 256), dim3(256), 0, s, cnt, 0u, (size_t)p.tiles);
+        p.desc.ptr[p.ws_slot] = ws;
+        p.desc.ptr[p.sync_slot] = cnt;
+    }
+    return launch(p, s);
 }
 
 }  // extern "C"
