@@ -172,7 +172,10 @@ def corun(models, rt_name, be_name, n_be, mode, requests, warmup, wait_sync=True
         bes.append(m)
     s.run()
     out = {"mode": {B.MODE_REEF: "REEF (reset-based preemption + dynamic kernel padding)",
-                    B.MODE_RESET: "Reset (reset-based preemption only)"}[mode],
+                    B.MODE_RESET: "Reset (reset-based preemption only)",
+                    B.MODE_WAITPREEMPT: "WaitPreempt (flag, then wait for everything launched)",
+                    B.MODE_NOPREEMPT: "NoPreempt (wait for the best-effort runs in flight)",
+                    B.MODE_MULTISTREAM: "MultiStream (no switch: real-time kernels beside best-effort ones)"}[mode],
            "rt_model": g_rt.name, "be_model": g_be.name, "be_clients": n_be}
     if solo:
         r0 = s.run_load(rt, [], requests, warmup=warmup, mean_interval_us=interval_us, seed=SEED)
@@ -215,9 +218,9 @@ def main():
     ap.add_argument("--steps", type=int, default=400, help="recorded real-time requests")
     ap.add_argument("--warmup", type=int, default=40, help="real-time requests before recording")
     ap.add_argument("--kernel-iters", type=int, default=20)
-    ap.add_argument("--configs", default="3,4,5",
+    ap.add_argument("--configs", default="3,4,5,6,7",
                     help="co-location scenarios to run (3 is the headline; 6 = dynamic kernel padding under "
-                         "a real-time request every 2 ms, not in the default set)")
+                         "a real-time request every 2 ms; 7 = the headline workload in every schedule mode)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--solo-only", action="store_true",
                     help="only the solo ResNet-152 executor part (whole-model and per-kernel timing); "
@@ -374,6 +377,21 @@ def main():
                                    dkp_slack=100, interval_us=2000.0),
             "reset": corun(models, "resnet152", "mobilenetv2", 1, B.MODE_RESET, k, 20, solo=False,
                            interval_us=2000.0)}
+    if 7 in configs and head is not None:
+        # the reference's evaluation baselines (scheduler.h:22-28) on the headline workload
+        k = max(args.steps // 4, 50)
+        runs = {"REEF": head, "Reset": reset_only}
+        for label, m in (("WaitPreempt", B.MODE_WAITPREEMPT), ("NoPreempt", B.MODE_NOPREEMPT),
+                         ("MultiStream", B.MODE_MULTISTREAM)):
+            runs[label] = corun(models, "resnet152", "densenet201", 4, m, k, 20, solo=False)
+        out["schedule_modes"] = {
+            label: {"rt_ms_p50": r["loaded"]["rt_ms"]["p50"], "rt_ms_p99": r["loaded"]["rt_ms"]["p99"],
+                    "rt_exec_ms_p50": r["loaded"]["rt_exec_ms"]["p50"],
+                    "rt_exec_ms_p99": r["loaded"]["rt_exec_ms"]["p99"],
+                    "be_inferences_per_s": r["loaded"]["be_inferences_per_s"],
+                    "switch_us_mean": r["preempt_us"]["mean"], "switch_us_p99": r["preempt_us"]["p99"],
+                    "rt_requests": r["preempt_us"]["n"]}
+            for label, r in runs.items()}
     if not args.no_cpu:
         cb, orc = cpu_baseline(d, g.name, x)
         out["cpu_baseline"] = cb

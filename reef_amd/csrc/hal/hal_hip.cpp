@@ -303,7 +303,7 @@ int pump_locked(reef_stream_t st) {
 // a preemption) for milliseconds.
 void feeder_main(reef_stream_s* st) {
     hipSetDevice(g_device);
-    int idle_spins = 0;
+    int idle_spins = 0, full_spins = 0;
     Held h;
     while (!st->stop.load(std::memory_order_acquire)) {
         if (st->held_count.load(std::memory_order_acquire) == 0) {
@@ -319,11 +319,16 @@ void feeder_main(reef_stream_s* st) {
             continue;
         }
         idle_spins = 0;
-        // `submitted` only changes in this thread while a feeder exists
+        // `submitted` only changes in this thread while a feeder exists.  A full window is the
+        // steady state while a best-effort model runs: its kernels take a few microseconds, far
+        // below what a sleep costs, so the thread polls the completion word -- one host core per
+        // best-effort stream.  Behind a kernel that runs for long it gives the core away.
         if ((int)in_flight(st) >= st->window) {
-            __builtin_ia32_pause();
+            if (++full_spins > 20000) std::this_thread::yield();
+            else __builtin_ia32_pause();
             continue;
         }
+        full_spins = 0;
         std::lock_guard<std::mutex> sub(st->submit_mtx);
         uint32_t seq = 0;
         {

@@ -1,0 +1,207 @@
+"""Importer for the reference's own model directories.
+
+A directory written by the reference's TVM pipeline (`resource/<model>/<model>.json`,
+script/generate_final_schedule.py:109-144) names one generated kernel per call
+(`fused_nn_conv2d_add_nn_relu_3_kernel0`) whose shape is baked into its source; the graph file
+holds the storages, the call order, the argument bindings and nothing about what a kernel
+computes.  This build's kernels are generic, so a graph for them says what every call computes
+(op, shape, epilogue) in the added keys `op` and `attrs`, which the reference's reader ignores
+(src/reef/executor/model.cpp:23-51).
+
+`import_model` rewrites such a graph: same storages (same indices, names, sizes -- including the
+buffers the reference shares between layers), same call order, same parameter keys (a `.param`
+file of the reference loads unchanged), every call replaced by the `reef_*` kernel that computes
+the same thing.  What a kernel name computes comes from a per-model table
+(`legacy_tables/<model>.json`: name -> op, shape, stride, padding, epilogue); the argument roles
+are those of the kernel families (convolution: in, W, out, then the epilogue operands in the
+order the family name lists them; elementwise add and flatten: out first; pooling: in, out).
+While it rewrites, the importer follows the tensor shapes through the graph and refuses a table
+that does not fit the graph.
+"""
+import json
+import os
+
+from .modelgen import builder as MB
+from .modelgen.builder import Tensor
+
+TABLE_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "legacy_tables")
+
+
+class ImportError_(ValueError):
+    pass
+
+
+def load_table(model_name):
+    path = os.path.join(TABLE_DIR, model_name + ".json")
+    if not os.path.exists(path):
+        raise ImportError_("no kernel table for model '%s' (%s)" % (model_name, path))
+    return json.load(open(path))
+
+
+def import_model(ref_json_path, table=None, name=None, input_shape=None):
+    """Reference graph file -> GraphBuilder holding the same graph on this build's kernels.
+    `table`: dict or path (default: the packaged table named after the file).  `input_shape`:
+    (C, H, W) of storage 0 (default: 3 x s x s with s from its size)."""
+    ref = json.load(open(ref_json_path))
+    model_name = name or os.path.splitext(os.path.basename(ref_json_path))[0]
+    if table is None:
+        table = load_table(model_name)
+    elif isinstance(table, str):
+        table = json.load(open(table))
+    g = MB.GraphBuilder(model_name)
+    g.unique_names = True
+    g.fused_reduce = True
+    g.storage = [dict(s) for s in ref["storage"]]
+    g.graph_args = list(ref.get("args", []))
+    n0 = ref["storage"][0]["size"]
+    if input_shape is None:
+        side = int(round((n0 // 3) ** 0.5))
+        if 3 * side * side != n0:
+            raise ImportError_("cannot tell the input shape from %d elements; pass input_shape" % n0)
+        input_shape = (3, side, side)
+    shape = {0: tuple(input_shape)}
+
+    def size(i):
+        return ref["storage"][i]["size"]
+
+    def need(cond, kernel, what):
+        if not cond:
+            raise ImportError_("%s: %s" % (kernel["name"], what))
+
+    def tensor(i, shp, kernel):
+        n = 1
+        for d in shp:
+            n *= d
+        need(n <= size(i), kernel, "storage %d holds %d elements, the table asks for %s" % (i, size(i), shp))
+        return Tensor(i, shp)
+
+    for k in ref["kernels"]:
+        kname, a = k["name"], k["args"]
+        e = table.get(kname)
+        need(e is not None, k, "not in the table")
+        op = e["op"]
+        if op == "conv2d":
+            need(len(a) >= 3 and a[0] in shape, k, "input storage has no shape yet")
+            need(shape[a[0]] == (e["cin"], e["h"], e["w"]), k,
+                 "table says input %s, the graph delivers %s" % ((e["cin"], e["h"], e["w"]), shape[a[0]]))
+            kk, s, p, cout = e["k"], e["stride"], e["pad"], e["cout"]
+            Ho, Wo = (e["h"] + 2 * p - kk) // s + 1, (e["w"] + 2 * p - kk) // s + 1
+            need(size(a[1]) == cout * e["cin"] * kk * kk, k, "weight storage size")
+            ep = e["epilogue"]
+            rest = a[3:]
+            given = {"w": Tensor(a[1], (cout, e["cin"], kk, kk))}
+            kw = dict(bias=False, act=MB.ACT_NONE, residual=None, affine=False)
+            if ep == "bias_relu":
+                need(len(rest) == 1 and size(rest[0]) == cout, k, "bias operand")
+                given["bias"] = Tensor(rest[0], (cout,))
+                kw.update(bias=True, act=MB.ACT_RELU)
+            elif ep == "residual":
+                need(len(rest) == 1 and shape.get(rest[0]) == (cout, Ho, Wo), k, "residual operand")
+                kw.update(residual=Tensor(rest[0], (cout, Ho, Wo)))
+            elif ep == "residual_bias_relu":
+                need(len(rest) == 2 and shape.get(rest[0]) == (cout, Ho, Wo) and size(rest[1]) == cout, k,
+                     "residual / bias operands")
+                given["bias"] = Tensor(rest[1], (cout,))
+                kw.update(residual=Tensor(rest[0], (cout, Ho, Wo)), bias=True, act=MB.ACT_RELU)
+            elif ep == "residual_scale_shift_relu":
+                need(len(rest) == 3 and shape.get(rest[0]) == (cout, Ho, Wo) and size(rest[1]) == cout
+                     and size(rest[2]) == cout, k, "residual / scale / shift operands")
+                given["scale"], given["shift"] = Tensor(rest[1], (cout,)), Tensor(rest[2], (cout,))
+                kw.update(residual=Tensor(rest[0], (cout, Ho, Wo)), affine=True, act=MB.ACT_RELU)
+            else:
+                need(ep == "none" and not rest, k, "unknown epilogue " + ep)
+            # a residual read from the buffer the result goes to would not survive a restart
+            need(kw["residual"] is None or kw["residual"].idx != a[2], k, "in-place residual")
+            g.conv2d(Tensor(a[0], shape[a[0]]), cout, kk, s, p, out=tensor(a[2], (cout, Ho, Wo), k),
+                     given=given, **kw)
+            shape[a[2]] = (cout, Ho, Wo)
+        elif op == "eltwise":                                   # (out, in, per-channel shift)
+            need(len(a) == 3 and a[1] in shape, k, "operands")
+            C, H, W = shape[a[1]]
+            need(C == e["c"] and H * W == e["inner"] and size(a[2]) == C, k, "shape")
+            g.eltwise(Tensor(a[1], shape[a[1]]), shift=True, act=e["act"], out=tensor(a[0], shape[a[1]], k),
+                      shift_t=Tensor(a[2], (C,)))
+            shape[a[0]] = shape[a[1]]
+        elif op == "pool2d":                                    # (in, out[, bias])
+            need(a[0] in shape and shape[a[0]] == (e["c"], e["h"], e["w"]), k, "shape")
+            out = g.pool2d(Tensor(a[0], shape[a[0]]), e["k"], e["stride"], e["pad"], mode=e["mode"],
+                           bias=bool(e.get("bias")), act=e.get("act", 0), out=Tensor(a[1], (1,)),
+                           bias_t=Tensor(a[2], (e["c"],)) if e.get("bias") else None)
+            need(out.size <= size(a[1]), k, "output storage too small")
+            shape[a[1]] = out.shape
+        elif op == "global_avgpool":                            # (in, out)
+            C, H, W = shape[a[0]]
+            need(C == e["c"] and H * W == e["hw"], k, "shape")
+            g.global_avgpool(Tensor(a[0], shape[a[0]]), out=tensor(a[1], (C,), k))
+            shape[a[1]] = (C, 1, 1)
+        elif op == "copy":                                      # flatten: (out, in)
+            n = e["n"]
+            need(shape.get(a[1], (0,))[0] * shape[a[1]][1] * shape[a[1]][2] == n, k, "shape")
+            g.copy_into(Tensor(a[1], (n,)), tensor(a[0], (n,), k), 0)
+            shape[a[0]] = (n, 1, 1)
+        elif op == "dense":                                     # (x, W, out, bias)
+            need(shape[a[0]][0] == e["in"] and size(a[1]) == e["in"] * e["out"], k, "shape")
+            g.dense(Tensor(a[0], (e["in"],)), e["out"], bias=bool(e.get("bias")), out=tensor(a[2], (1, e["out"]), k),
+                    w=Tensor(a[1], (e["out"], e["in"])), bias_t=Tensor(a[3], (e["out"],)) if e.get("bias") else None)
+            shape[a[2]] = (e["out"], 1, 1)
+        elif op == "softmax":                                   # (in, out)
+            need(shape[a[0]][0] == e["cols"], k, "shape")
+            g.softmax(Tensor(a[0], (e["rows"], e["cols"])), e["rows"], e["cols"],
+                      out=tensor(a[1], (e["rows"], e["cols"]), k))
+            shape[a[1]] = shape[a[0]]
+        else:
+            need(False, k, "unknown op " + op)
+    g.imported_from = [k["name"] for k in ref["kernels"]]
+    return g
+
+
+def import_model_dir(ref_dir, model_name, out_dir, table=None, measured_profile=False):
+    """<ref_dir>/<model>.json (+ .param if present) -> a model directory of this build in out_dir.
+    Returns the GraphBuilder.  A `.param` file of the reference is taken over byte for byte (same
+    keys, same storages); the profile is the estimate unless measured_profile (needs a GPU)."""
+    import shutil
+    g = import_model(os.path.join(ref_dir, model_name + ".json"), table=table, name=model_name)
+    g.write(out_dir)
+    src = os.path.join(ref_dir, model_name + ".param")
+    if os.path.exists(src):
+        shutil.copyfile(src, os.path.join(out_dir, model_name + ".param"))
+    if measured_profile:
+        from . import profiler
+        profiler.write_profile(out_dir, model_name)
+    return g
+
+
+def seeded_params(ref_json_path, table=None, seed=0x5EEF):
+    """Seeded parameters for a reference graph that ships without a `.param` file (the checkout's
+    resource/resnet152 does): He-normal weights, small biases / shifts, scales around 1 -- the
+    distributions the generator of this build uses.  Returns [(key, float32 array)] in storage
+    order, ready for modelgen.builder.write_params."""
+    import math
+    from .modelgen import rng
+    ref = json.load(open(ref_json_path))
+    model_name = os.path.splitext(os.path.basename(ref_json_path))[0]
+    if table is None:
+        table = load_table(model_name)
+    elif isinstance(table, str):
+        table = json.load(open(table))
+    std = {}
+    one_plus = set()
+    for k in ref["kernels"]:
+        e, a = table[k["name"]], k["args"]
+        if e["op"] == "conv2d":
+            std[a[1]] = math.sqrt(2.0 / (e["cin"] * e["k"] * e["k"]))
+            if e["epilogue"] == "residual_scale_shift_relu":
+                std[a[4]] = 0.1
+                one_plus.add(a[4])
+        elif e["op"] == "dense":
+            std[a[1]] = math.sqrt(2.0 / e["in"])
+    out = []
+    for i, s in enumerate(ref["storage"]):
+        name = s["name"]
+        if not (name.startswith("p") and name[1:].isdigit()):
+            continue
+        arr = rng.normal_f32(model_name + "/" + name, s["size"], std.get(i, 0.01), seed)
+        if i in one_plus:
+            arr = arr + 1.0
+        out.append((name, arr.astype("float32")))
+    return out

@@ -122,7 +122,7 @@ class GraphBuilder:
 
     def conv2d(self, x, cout, k, stride=1, pad=0, bias=True, act=ACT_RELU, residual=None,
                affine=False, force=None, dual_act=None, fused_reduce=None, out=None, out_channel=0,
-               pre_act=False):
+               pre_act=False, given=None):
         """Fused conv + (residual) + (bias) + (scale, shift) + activation on MFMA.
         pre_act: the layer reads its input through a per-channel scale, shift and ReLU of its own
         (DenseNet pre-activation); folded into the convolution's input loads where a kernel for it
@@ -130,7 +130,10 @@ class GraphBuilder:
         dual_act: also emit out2 = dual_act(out + shift2[c]) and return (out, out2).
         fused_reduce: fold split-K inside the kernel (default: self.fused_reduce).
         out / out_channel: write into channels [out_channel, out_channel + cout) of an existing
-        tensor (a concatenation buffer) instead of a new one."""
+        tensor (a concatenation buffer) instead of a new one.
+        given: operands that exist already (an imported graph): {"w", "bias", "scale", "shift"} ->
+        Tensor; what is not given is created as a seeded parameter."""
+        given = given or {}
         if fused_reduce is None:
             fused_reduce = self.fused_reduce
         kh, kw = (k, k) if isinstance(k, int) else k
@@ -141,21 +144,24 @@ class GraphBuilder:
         Wo = (W + 2 * pw - kw) // sw + 1
         M, N, K = cout, Ho * Wo, cin * kh * kw
         std = self.weight_std if self.weight_std is not None else math.sqrt(2.0 / K)
-        w = self.param((cout, cin, kh, kw), std)
+        w = given.get("w") or self.param((cout, cin, kh, kw), std)
         flags = 0
         opt = []
         if bias:
             flags |= F_BIAS
-            opt.append(self.param((cout,), 0.01).idx)
+            opt.append((given.get("bias") or self.param((cout,), 0.01)).idx)
         if residual is not None:
             flags |= F_RESIDUAL
             assert residual.shape == (cout, Ho, Wo), (residual.shape, (cout, Ho, Wo))
             opt.append(residual.idx)
         if affine:
             flags |= F_AFFINE
-            opt.append(self.param((cout,), 0.1, value=None).idx)   # scale ~ N(0, 0.1) + 1 below
-            self.params[-1] = (self.params[-1][0], self.params[-1][1] + 1.0)
-            opt.append(self.param((cout,), 0.01).idx)
+            if "scale" in given:
+                opt.append(given["scale"].idx)
+            else:
+                opt.append(self.param((cout,), 0.1, value=None).idx)   # scale ~ N(0, 0.1) + 1 below
+                self.params[-1] = (self.params[-1][0], self.params[-1][1] + 1.0)
+            opt.append((given.get("shift") or self.param((cout,), 0.01)).idx)
         dst_off = 0
         if out is None:
             out = self.temp((cout, Ho, Wo))
@@ -257,35 +263,35 @@ class GraphBuilder:
         return out
 
     def pool2d(self, x, k, stride, pad, mode="max", bias=False, act=ACT_NONE, count_include_pad=False,
-               ceil_mode=False):
+               ceil_mode=False, out=None, bias_t=None):
         C, H, W = x.shape
         kh, kw = (k, k) if isinstance(k, int) else k
         rnd = math.ceil if ceil_mode else math.floor
         Ho = int(rnd((H + 2 * pad - kh) / stride)) + 1
         Wo = int(rnd((W + 2 * pad - kw) / stride)) + 1
-        out = self.temp((C, Ho, Wo))
+        out = Tensor(out.idx, (C, Ho, Wo)) if out is not None else self.temp((C, Ho, Wo))
         args = [x.idx, out.idx]
         flags = 0
         if bias:
             flags = 1
-            args.append(self.param((C,), 0.01).idx)
+            args.append((bias_t or self.param((C,), 0.01)).idx)
         self._emit("reef_pool2d", math.ceil(out.size / WG), args,
                    [C, H, W, Ho, Wo, kh, kw, stride, stride, pad, pad, 0 if mode == "max" else 1,
                     1 if count_include_pad else 0, flags, act], "pool2d", 0,
                    4 * (x.size + out.size), 2.0)
         return out
 
-    def global_avgpool(self, x):
+    def global_avgpool(self, x, out=None):
         C = x.shape[0]
-        out = self.temp((C,))
+        out = Tensor(out.idx, (C,)) if out is not None else self.temp((C,))
         self._emit("reef_global_avgpool", math.ceil(C / 4), [x.idx, out.idx], [C, x.size // C],
                    "global_avgpool", 0, 4 * (x.size + C), 2.0)
         return out
 
-    def eltwise(self, a, b=None, scale=False, shift=False, act=ACT_NONE):
+    def eltwise(self, a, b=None, scale=False, shift=False, act=ACT_NONE, out=None, shift_t=None):
         C = a.shape[0]
         inner = a.size // C
-        out = self.temp(a.shape)
+        out = Tensor(out.idx, a.shape) if out is not None else self.temp(a.shape)
         args = [a.idx, out.idx]
         flags = 0
         n_in = 1
@@ -301,28 +307,28 @@ class GraphBuilder:
             args.append(p.idx)
         if shift:
             flags |= 4
-            args.append(self.param((C,), 0.01 if not isinstance(shift, float) else shift).idx)
+            args.append((shift_t or self.param((C,), 0.01 if not isinstance(shift, float) else shift)).idx)
         self._emit("reef_eltwise", math.ceil(a.size / 1024), args, [C, inner, flags, act], "eltwise",
                    0, 4 * (n_in + 1) * a.size, 2.0)
         return out
 
-    def dense(self, x, out_f, bias=True, act=ACT_NONE, rows=1):
+    def dense(self, x, out_f, bias=True, act=ACT_NONE, rows=1, out=None, w=None, bias_t=None):
         in_f = x.size // rows
         std = self.weight_std if self.weight_std is not None else math.sqrt(2.0 / in_f)
-        w = self.param((out_f, in_f), std)
-        out = self.temp((rows, out_f))
+        w = w or self.param((out_f, in_f), std)
+        out = Tensor(out.idx, (rows, out_f)) if out is not None else self.temp((rows, out_f))
         args = [x.idx, w.idx, out.idx]
         flags = 0
         if bias:
             flags = 1
-            args.append(self.param((out_f,), 0.01).idx)
+            args.append((bias_t or self.param((out_f,), 0.01)).idx)
         self.flops += 2 * rows * in_f * out_f
         self._emit("reef_dense", math.ceil(out_f / 4), args, [rows, in_f, out_f, flags, act],
                    "dense", 2 * rows * in_f * out_f, 4 * (x.size + in_f * out_f + rows * out_f), 2.0)
         return out
 
-    def softmax(self, x, rows, cols):
-        out = self.temp((rows, cols))
+    def softmax(self, x, rows, cols, out=None):
+        out = Tensor(out.idx, (rows, cols)) if out is not None else self.temp((rows, cols))
         self._emit("reef_softmax", math.ceil(rows / 4), [x.idx, out.idx], [rows, cols], "softmax", 0,
                    8 * rows * cols, 2.0)
         return out

@@ -206,13 +206,16 @@ def test_dkp_resnet_in_resnet_shadow(dirs):
     s.shutdown()
 
 
-@pytest.mark.parametrize("mode", [B.MODE_RESET, B.MODE_REEF])
+@pytest.mark.parametrize("mode", [B.MODE_RESET, B.MODE_REEF, B.MODE_WAITPREEMPT, B.MODE_NOPREEMPT,
+                                  B.MODE_MULTISTREAM])
 def test_load_generator_preemption_under_load(dirs, mode):
     """One open-loop real-time client (ResNet-18, exponential gaps, mean 3 ms) against three
-    closed-loop best-effort ResNet-50 clients: dozens of preemptions, and afterwards every model
+    closed-loop best-effort ResNet-50 clients, in every schedule mode of the reference
+    (src/reef/server/scheduler.h:22-28): dozens of mode switches, and afterwards every model
     still holds exactly the output of an uninterrupted solo run.  With wait_sync the recorded
-    preemption span covers the drain of every best-effort stream; it has to stay far below a
-    best-effort inference (which is what a scheduler without preemption would wait for)."""
+    span of a reset-based preemption covers the drain of every best-effort stream; it has to
+    stay far below a best-effort inference, which is what the modes that wait for the device
+    (WaitPreempt, NoPreempt) pay instead."""
     x50 = nets.image_input("resnet50", (3, 224, 224))
     x18 = nets.image_input("resnet18", (3, 224, 224))
     ref_be = solo_output(dirs["resnet50"], "resnet50", x50)
@@ -232,13 +235,18 @@ def test_load_generator_preemption_under_load(dirs, mode):
     r = s.run_load(rt_mid, bes, requests=60, warmup=10, mean_interval_us=3000.0, seed=11)
     assert len(r["rt_latency_us"]) == 60 and (r["rt_exec_us"] > 0).all()
     assert r["be_completed"].sum() > 0
-    assert r["be_preempted"].sum() > 0
     ps = s.preempt_samples()
     assert len(ps) >= 30
+    if mode in (B.MODE_RESET, B.MODE_REEF, B.MODE_WAITPREEMPT):
+        assert r["be_preempted"].sum() > 0
     print("mode %d: rt p50 %.0f us, preempt mean %.1f max %d us over %d, BE done %s preempted %s padded %s"
           % (mode, np.percentile(r["rt_latency_us"], 50), ps.mean(), ps.max(), len(ps),
              r["be_completed"], r["be_preempted"], r["be_padded"]))
-    assert ps.mean() < 200 and np.percentile(ps, 95) < 400      # microseconds
+    if mode in (B.MODE_RESET, B.MODE_REEF):
+        assert ps.mean() < 200 and np.percentile(ps, 95) < 400      # microseconds
+    elif mode in (B.MODE_WAITPREEMPT, B.MODE_NOPREEMPT):
+        # these wait until what was launched has run: a good part of a best-effort inference
+        assert ps.mean() > 100
     np.testing.assert_array_equal(s.get_output(rt_mid, 1000), ref_rt)
     # let every best-effort client finish one more uninterrupted inference, then compare
     r2 = s.run_load(rt_mid, bes, requests=0, be_only_ms=30)

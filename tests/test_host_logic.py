@@ -398,6 +398,51 @@ def test_wait_preempt_second_run_restarts_at_the_interrupted_kernel(fake, small_
     s.shutdown()
 
 
+@pytest.mark.parametrize("mode", [B.MODE_NOPREEMPT, B.MODE_MULTISTREAM, B.MODE_WAITPREEMPT])
+def test_real_time_arrival_during_a_best_effort_run_in_the_baseline_modes(fake, small_dirs, mode):
+    """The evaluation baselines of the reference (src/reef/server/scheduler.h:22-28) under contention:
+    a real-time task arrives while a best-effort run is on the device.
+      NoPreempt    waits for everything launched, then runs the real-time task (scheduler.cpp:381-392);
+      MultiStream  switches nothing: the real-time kernels go to their own stream beside the
+                   best-effort ones (scheduler.cpp:402-403);
+      WaitPreempt  raises the flag, waits, restarts at the first incomplete kernel (scheduler.cpp:348-372).
+    Whatever the interleaving, both outputs are those of an undisturbed run, over several runs."""
+    gb, db = small_dirs["tiny18"]
+    gm, dm = small_dirs["mocked_kernel"]
+    x = nets.image_input("t", (3, 32, 32))
+    fake.lib.fake_hal_set_auto_progress(1)
+    s = B.Scheduler(mode)
+    s.run()
+    be_mid = s.load_model(db, gb.name)
+    rt_mid = s.load_model(dm, gm.name)
+    s.bind_model_queue(s.create_queue(B.QUEUE_BE), be_mid)
+    s.bind_model_queue(s.create_queue(B.QUEUE_RT), rt_mid)
+    for n in "abc":
+        s.set_input(rt_mid, THREE, n)
+    overlapped = 0
+    for rep in range(5):
+        xi = (x * (1.0 + 0.5 * rep)).astype(np.float32)
+        want = oracle_output(gb, db, xi)
+        s.set_input(be_mid, xi, "data")
+        done0 = fake.lib.fake_hal_completed()
+        be_tid = s.new_task(be_mid)
+        t0 = time.time()
+        while fake.lib.fake_hal_completed() < done0 + 2 + rep and time.time() - t0 < 10:
+            time.sleep(0.0002)
+        rt_tid = s.new_task(rt_mid)
+        assert s.wait_task(rt_tid) == 0 and s.wait_task(be_tid) == 0
+        np.testing.assert_array_equal(s.get_output(rt_mid, 8192), np.full(8192, 18.0, np.float32))
+        np.testing.assert_array_equal(s.get_output(be_mid, 16), want)
+        be, rt = s.task_info(be_tid), s.task_info(rt_tid)
+        if rt["start"] >= be["start"] and be["end"] >= rt["start"]:
+            overlapped += 1
+            if mode == B.MODE_NOPREEMPT:
+                assert not be["preempted"]
+    assert overlapped > 0, "no real-time task arrived during a best-effort run"
+    assert s.preempt_times() >= overlapped
+    s.shutdown()
+
+
 def test_be_stream_cap_is_fixed_once_a_best_effort_queue_exists(fake, small_dirs):
     s = B.Scheduler(B.MODE_RESET)
     assert s.set_be_stream_cap(3) == 0

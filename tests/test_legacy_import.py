@@ -1,0 +1,147 @@
+"""The importer for the reference's own model directories (reef_amd/legacy.py) on the reference's
+resource/resnet152 graph (tests/golden/resnet152.json, a data fixture): same storages, same call
+order, and the imported graph computes what the reference's kernels compute according to the
+table of shapes that was derived by running those kernels (tests/golden/make_resnet152_shapes.py).
+
+The CPU check interprets the reference graph DIRECTLY from the table with the oracle's ops and
+compares that with the imported model run through the executor (fake backend) -- two code paths
+from the same table, so a wrong role, attribute order or epilogue flag in the importer shows."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from reef_amd import binding as B
+from reef_amd import legacy
+from reef_amd.modelgen import builder as MB
+from reef_amd.modelgen import nets
+from tests.fakehal import FakeHal
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+REF_JSON = os.path.join(HERE, "golden", "resnet152.json")
+TABLE = os.path.join(HERE, "golden", "resnet152_kernel_shapes.json")
+
+
+def interpret_reference_graph(ref, table, params, x, upto=None):
+    """The reference graph evaluated from the table with the oracle's ops.  Returns the storages."""
+    st = {i: np.zeros(s["size"], np.float32) for i, s in enumerate(ref["storage"])}
+    for i, s in enumerate(ref["storage"]):
+        if s["name"] in params:
+            st[i][:] = params[s["name"]]
+    st[0][:] = x.ravel()
+    for n, k in enumerate(ref["kernels"]):
+        if upto is not None and n >= upto:
+            break
+        e, a = table[k["name"]], k["args"]
+        if e["op"] == "conv2d":
+            cin, H, W, cout, kk, s, p = e["cin"], e["h"], e["w"], e["cout"], e["k"], e["stride"], e["pad"]
+            Ho = (H + 2 * p - kk) // s + 1
+            xs = st[a[0]][:cin * H * W].reshape(cin, H, W)
+            ws = st[a[1]].reshape(cout, cin, kk, kk)
+            full = lambda i: st[i][:cout * Ho * Ho].reshape(cout, Ho, Ho)
+            kw = dict(stride=(s, s), pad=(p, p))
+            ep = e["epilogue"]
+            if ep == "none":
+                y = O.conv2d(xs, ws, act=0, **kw)
+            elif ep == "residual":
+                y = O.conv2d(xs, ws, residual=full(a[3]), act=0, **kw)
+            elif ep == "bias_relu":
+                y = O.conv2d(xs, ws, bias=st[a[3]], act=1, **kw)
+            elif ep == "residual_bias_relu":
+                y = O.conv2d(xs, ws, residual=full(a[3]), bias=st[a[4]], act=1, **kw)
+            else:
+                y = O.conv2d(xs, ws, residual=full(a[3]), scale=st[a[4]], shift=st[a[5]], act=1, **kw)
+            st[a[2]][:y.size] = y.ravel()
+        elif e["op"] == "eltwise":
+            C, inner = e["c"], e["inner"]
+            y = O.eltwise(st[a[1]][:C * inner].reshape(C, inner), shift=st[a[2]], act=e["act"])
+            st[a[0]][:y.size] = y.ravel()
+        elif e["op"] == "pool2d":
+            C, H, W = e["c"], e["h"], e["w"]
+            y = O.pool2d(st[a[0]][:C * H * W].reshape(C, H, W), (3, 3), (2, 2), (1, 1), 0, bias=st[a[2]], act=1)
+            st[a[1]][:y.size] = y.ravel()
+        elif e["op"] == "global_avgpool":
+            C, hw = e["c"], e["hw"]
+            st[a[1]][:C] = O.global_avgpool(st[a[0]][:C * hw].reshape(C, hw)).ravel()
+        elif e["op"] == "copy":
+            st[a[0]][:e["n"]] = st[a[1]][:e["n"]]
+        elif e["op"] == "dense":
+            y = O.dense(st[a[0]][:e["in"]].reshape(1, e["in"]), st[a[1]].reshape(e["out"], e["in"]), bias=st[a[3]])
+            st[a[2]][:e["out"]] = y.ravel()
+        elif e["op"] == "softmax":
+            st[a[1]][:e["cols"]] = O.softmax(st[a[0]][:e["cols"]].reshape(1, e["cols"])).ravel()
+        else:
+            raise AssertionError(e["op"])
+    return st
+
+
+@pytest.fixture(scope="module")
+def imported(tmp_path_factory):
+    d = str(tmp_path_factory.mktemp("legacy152"))
+    g = legacy.import_model(REF_JSON, table=TABLE)
+    g.write(d)
+    params = legacy.seeded_params(REF_JSON, table=TABLE)
+    MB.write_params(os.path.join(d, g.name + ".param"), params)
+    return g, d, dict(params)
+
+
+def test_import_keeps_storages_order_and_parameter_keys(imported):
+    g, d, params = imported
+    ref = json.load(open(REF_JSON))
+    out = json.load(open(os.path.join(d, "resnet152.json")))
+    n = len(ref["storage"])
+    assert out["storage"][:n] == ref["storage"]                # same indices, names, sizes
+    assert all(s["name"] in ("temp_arg", "reef_sync") for s in out["storage"][n:])
+    assert out["args"] == ref["args"]
+    assert len(out["kernels"]) == len(ref["kernels"]) == 207   # one launch per reference launch
+    assert g.imported_from == [k["name"] for k in ref["kernels"]]
+    for ko, kr in zip(out["kernels"], ref["kernels"]):
+        assert ko["name"].startswith("reef_") and ko["launch_params"][3:] == [256, 1, 1]
+        # every storage the reference kernel touches is bound to the replacement, and the
+        # replacement binds nothing else of the reference's storages
+        assert sorted(set(x for x in ko["args"] if x < n)) == sorted(set(kr["args"])), (ko, kr)
+    assert len(params) == sum(1 for s in ref["storage"] if s["name"].startswith("p"))
+
+
+def test_imported_graph_equals_the_table_interpretation_through_the_executor(imported):
+    g, d, params = imported
+    ref = json.load(open(REF_JSON))
+    table = json.load(open(TABLE))
+    x = nets.image_input("legacy", (3, 64, 64))
+    want = interpret_reference_graph(ref, table, params, x)
+    fake = FakeHal().install()
+    exe = None
+    try:
+        exe = B.Executor.from_dir(d, "resnet152", B.HYBRID)
+        exe.set_input_checked("data", x)
+        exe.execute()
+        got = exe.get_output()      # the whole `output` storage: a shared buffer, the classes come first
+        out_idx = [i for i, s in enumerate(ref["storage"]) if s["name"] == "output"][0]
+        np.testing.assert_allclose(got, want[out_idx][:got.size], rtol=0, atol=1e-6)
+        assert abs(float(got[:1000].sum()) - 1.0) < 1e-4
+        # every intermediate buffer of the reference graph, as the last writer left it
+        for i, s in enumerate(ref["storage"]):
+            if s["name"] == "null":
+                have = exe.get_data(i, s["size"])
+                scale = max(np.abs(want[i]).max(), 1e-6)
+                assert np.abs(have - want[i]).max() <= 1e-5 * scale, i
+    finally:
+        if exe is not None:
+            exe.close()
+        fake.remove()
+
+
+def test_import_refuses_a_table_that_does_not_fit_the_graph():
+    table = json.load(open(TABLE))
+    bad = json.loads(json.dumps(table))
+    bad["fused_nn_conv2d_add_nn_relu_9_kernel0"]["h"] = 8
+    with pytest.raises(legacy.ImportError_, match="fused_nn_conv2d_add_nn_relu_9_kernel0"):
+        legacy.import_model(REF_JSON, table=bad)
+    del bad["fused_nn_softmax_kernel0"]
+    bad["fused_nn_conv2d_add_nn_relu_9_kernel0"]["h"] = 16
+    with pytest.raises(legacy.ImportError_, match="not in the table"):
+        legacy.import_model(REF_JSON, table=bad)
+    # the packaged table is the fixture
+    assert legacy.load_table("resnet152") == table
