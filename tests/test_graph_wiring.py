@@ -1,0 +1,222 @@
+"""Wiring of the network generators (reef_amd/modelgen/nets.py), pinned independently of the
+generator's own kernel list.
+
+* ResNet: the generator claims to reproduce the graph the reference's TVM pipeline emits
+  (relay.testing.resnet, pre-activation, folded batch norms).  The reference holds that graph for
+  ResNet-152 at 64x64 (resource/resnet152/resnet152.json, fixture tests/golden/resnet152.json):
+  the generator's network, fed the same parameters by key, must compute what the reference graph
+  computes when it is interpreted call by call.
+* MobileNetV2, DenseNet, Inception-v3, BERT: each is written again here as a plain
+  torch.nn.functional program from the architecture's textbook definition, consuming the
+  generator's parameters in order of definition, and compared with the graph run by the oracle.
+  A skipped residual, a wrong channel slice of a concatenation, a swapped branch or a missing
+  activation changes the output by far more than the tolerance (1e-4 of the largest magnitude)."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import oracle as O
+from reef_amd import legacy
+from reef_amd.modelgen import nets
+from tests.helpers import max_rel_err, write_model
+from tests.test_legacy_import import REF_JSON, TABLE, interpret_reference_graph
+
+TOL = 1e-4
+
+
+def oracle_run(g, tmp, key, x):
+    d = write_model(g, tmp)
+    model = json.load(open(os.path.join(d, g.name + ".json")))
+    orc = O.GraphOracle(model, os.path.join(d, g.name + ".param"))
+    orc.set_input(key, x)
+    return np.asarray(orc.run()).copy(), orc, model
+
+
+class Params:
+    def __init__(self, g):
+        self.it = iter(g.params)
+
+    def take(self, *shape):
+        key, arr = next(self.it)
+        assert arr.size == int(np.prod(shape)), (key, arr.size, shape)
+        return torch.from_numpy(np.asarray(arr, np.float32).reshape(shape).copy())
+
+    def done(self):
+        return next(self.it, None) is None
+
+
+def test_resnet_generator_equals_the_reference_graph(tmp_path):
+    g = nets.resnet(152, image=(3, 64, 64), fuse_act=False, fused_reduce=True, name="resnet152_64")
+    ref = json.load(open(REF_JSON))
+    table = json.load(open(TABLE))
+    # the reference also launches a flatten copy between pooling and classifier; a no-op here
+    ref_calls = [k for k in ref["kernels"] if not k["name"].startswith("fused_nn_batch_flatten")]
+    assert len(g.kernels) == len(ref_calls) == 206
+    # Parameters are matched call by call (the reference numbers them in graph order, which
+    # differs from call order where a unit has a projection): the i-th call of both graphs binds
+    # its parameters in the same order -- weights first, then the per-channel operands.
+    mine = dict(g.params)
+    is_param = lambda st, i: st[i]["name"].startswith("p") and st[i]["name"][1:].isdigit()
+    params = {}
+    for ko, kr in zip(g.kernels, ref_calls):
+        po = [g.storage[i]["name"] for i in ko["args"] if is_param(g.storage, i)]
+        pr = [ref["storage"][i]["name"] for i in kr["args"] if is_param(ref["storage"], i)]
+        assert len(po) == len(pr), (ko["name"], kr["name"])
+        for a, b in zip(po, pr):
+            assert mine[a].size == [s_["size"] for s_ in ref["storage"] if s_["name"] == b][0], (ko["name"], a, b)
+            params[b] = mine[a]
+    assert len(params) == sum(1 for s_ in ref["storage"] if is_param(ref["storage"], ref["storage"].index(s_)))
+    x = nets.image_input("wiring", (3, 64, 64))
+    got, orc, model = oracle_run(g, tmp_path, "data", x)
+    st = interpret_reference_graph(ref, table, params, x)
+    out_idx = [i for i, s_ in enumerate(ref["storage"]) if s_["name"] == "output"][0]
+    want = st[out_idx][:1000]
+    assert abs(float(want.sum()) - 1.0) < 1e-4
+    assert max_rel_err(got[:1000], want) <= TOL
+    # and before the saturating softmax: the classifier's logits
+    dense = [k for k in ref["kernels"] if k["name"].startswith("fused_nn_dense")][0]
+    logits_ref = st[dense["args"][2]][:1000]
+    logits = np.asarray(orc.storage[model["kernels"][-1]["args"][0]])[:1000]
+    assert max_rel_err(logits, logits_ref) <= TOL
+
+
+def test_mobilenet_v2_wiring(tmp_path):
+    g = nets.mobilenet_v2(image=(3, 64, 64), classes=40, name="mbv2_64")
+    x = nets.image_input("wiring", (3, 64, 64))
+    _, orc, model = oracle_run(g, tmp_path, "data", x)
+    logits = np.asarray(orc.storage[model["kernels"][-1]["args"][0]])[:40]
+    P = Params(g)
+    relu6 = lambda t: torch.clamp(t, 0.0, 6.0)
+    t = torch.from_numpy(x)[None]
+    t = relu6(F.conv2d(t, P.take(32, 3, 3, 3), P.take(32), stride=2, padding=1))
+    cin = 32
+    for expand, c, n, s in [(1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1),
+                            (6, 160, 3, 2), (6, 320, 1, 1)]:
+        for i in range(n):
+            stride = s if i == 0 else 1
+            y = t
+            if expand != 1:
+                y = relu6(F.conv2d(y, P.take(cin * expand, cin, 1, 1), P.take(cin * expand)))
+            ch = y.shape[1]
+            y = relu6(F.conv2d(y, P.take(ch, 1, 3, 3), P.take(ch), stride=stride, padding=1, groups=ch))
+            y = F.conv2d(y, P.take(c, ch, 1, 1), P.take(c))
+            t = y + t if (stride == 1 and cin == c) else y
+            cin = c
+    t = relu6(F.conv2d(t, P.take(1280, 320, 1, 1), P.take(1280)))
+    t = t.mean(dim=(2, 3))
+    t = F.linear(t, P.take(40, 1280), P.take(40))
+    assert P.done()
+    assert max_rel_err(logits, t.numpy().ravel()) <= TOL
+
+
+def test_densenet_wiring(tmp_path):
+    blocks, growth = (2, 3, 2, 2), 32
+    g = nets.densenet(blocks=blocks, growth=growth, image=(3, 64, 64), classes=24, name="dense_64")
+    x = nets.image_input("wiring", (3, 64, 64))
+    _, orc, model = oracle_run(g, tmp_path, "data", x)
+    logits = np.asarray(orc.storage[model["kernels"][-1]["args"][0]])[:24]
+    P = Params(g)
+    bn_relu = lambda t, sc, sh: F.relu(t * sc[None, :, None, None] + sh[None, :, None, None])
+    t = torch.from_numpy(x)[None]
+    t = F.relu(F.conv2d(t, P.take(64, 3, 7, 7), P.take(64), stride=2, padding=3))
+    t = F.max_pool2d(t, 3, 2, 1)
+    c = 64
+    for bi, n_layers in enumerate(blocks):
+        for _ in range(n_layers):
+            w1, b1 = P.take(128, c, 1, 1), P.take(128)
+            sc, sh = P.take(c), P.take(c)                       # this layer's own BN on the concatenation
+            y = F.relu(F.conv2d(bn_relu(t, sc, sh), w1, b1))
+            y = F.conv2d(y, P.take(growth, 128, 3, 3), None, padding=1)
+            t = torch.cat([t, y], dim=1)
+            c += growth
+        if bi != len(blocks) - 1:
+            wt = P.take(c // 2, c, 1, 1)
+            sc, sh = P.take(c), P.take(c)
+            t = F.avg_pool2d(F.conv2d(bn_relu(t, sc, sh), wt), 2, 2)
+            c //= 2
+    sc, sh = P.take(c), P.take(c)
+    t = bn_relu(t, sc, sh).mean(dim=(2, 3))
+    t = F.linear(t, P.take(24, c), P.take(24))
+    assert P.done()
+    assert max_rel_err(logits, t.numpy().ravel()) <= TOL
+
+
+def test_bert_wiring(tmp_path):
+    layers, hidden, heads, ffn, seq, vocab = 2, 64, 4, 128, 16, 97
+    g = nets.bert(layers=layers, hidden=hidden, heads=heads, ffn=ffn, seq=seq, vocab=vocab, name="bert_s")
+    ids = nets.token_input("wiring", seq, vocab)
+    got, _, _ = oracle_run(g, tmp_path, "input0", ids)
+    P = Params(g)
+    tok, pos, seg = P.take(vocab, hidden), P.take(seq, hidden), P.take(hidden)
+    t = tok[torch.from_numpy(np.asarray(ids, np.int64))] + pos + seg[None, :]
+    ln = lambda v: F.layer_norm(v, (hidden,), P.take(hidden), P.take(hidden), eps=1e-12)
+    t = ln(t)
+    hd = hidden // heads
+    for _ in range(layers):
+        q = F.linear(t, P.take(hidden, hidden), P.take(hidden))
+        k = F.linear(t, P.take(hidden, hidden), P.take(hidden))
+        v = F.linear(t, P.take(hidden, hidden), P.take(hidden))
+        split = lambda m: m.reshape(seq, heads, hd).permute(1, 0, 2)
+        probs = torch.softmax(split(q) @ split(k).transpose(1, 2) / hd ** 0.5, dim=-1)
+        ctx = (probs @ split(v)).permute(1, 0, 2).reshape(seq, hidden)
+        att = F.linear(ctx, P.take(hidden, hidden), P.take(hidden))
+        t = ln(att + t)
+        h = F.gelu(F.linear(t, P.take(ffn, hidden), P.take(ffn)))           # exact erf form
+        y = F.linear(h, P.take(hidden, ffn), P.take(hidden))
+        t = ln(y + t)
+    assert P.done()
+    assert max_rel_err(got[:seq * hidden], t.numpy().ravel()) <= TOL
+
+
+def test_inception_v3_wiring(tmp_path):
+    g = nets.inception_v3(classes=32, name="incv3")
+    x = nets.image_input("wiring", (3, 299, 299))
+    _, orc, model = oracle_run(g, tmp_path, "data", x)
+    logits = np.asarray(orc.storage[model["kernels"][-1]["args"][0]])[:32]
+    P = Params(g)
+
+    def conv(t, cout, k, s=1, p=0):
+        kh, kw = (k, k) if isinstance(k, int) else k
+        return F.relu(F.conv2d(t, P.take(cout, t.shape[1], kh, kw), P.take(cout), stride=s, padding=p))
+
+    avg = lambda t: F.avg_pool2d(t, 3, 1, 1, count_include_pad=True)
+    t = torch.from_numpy(x)[None]
+    t = conv(t, 32, 3, 2); t = conv(t, 32, 3); t = conv(t, 64, 3, 1, 1)
+    t = F.max_pool2d(t, 3, 2)
+    t = conv(t, 80, 1); t = conv(t, 192, 3)
+    t = F.max_pool2d(t, 3, 2)
+    for pool_ch in (32, 64, 64):                                           # 3 x block A
+        b1 = conv(t, 64, 1)
+        b5 = conv(conv(t, 48, 1), 64, 5, 1, 2)
+        b3 = conv(conv(conv(t, 64, 1), 96, 3, 1, 1), 96, 3, 1, 1)
+        bp = conv(avg(t), pool_ch, 1)
+        t = torch.cat([b1, b5, b3, bp], 1)
+    b3 = conv(t, 384, 3, 2)                                                # block B (grid reduction)
+    bd = conv(conv(conv(t, 64, 1), 96, 3, 1, 1), 96, 3, 2)
+    t = torch.cat([b3, bd, F.max_pool2d(t, 3, 2)], 1)
+    for c7 in (128, 160, 160, 192):                                        # 4 x block C
+        b1 = conv(t, 192, 1)
+        b7 = conv(conv(conv(t, c7, 1), c7, (1, 7), 1, (0, 3)), 192, (7, 1), 1, (3, 0))
+        bd = conv(conv(conv(conv(conv(t, c7, 1), c7, (7, 1), 1, (3, 0)), c7, (1, 7), 1, (0, 3)), c7, (7, 1), 1,
+                       (3, 0)), 192, (1, 7), 1, (0, 3))
+        bp = conv(avg(t), 192, 1)
+        t = torch.cat([b1, b7, bd, bp], 1)
+    b3 = conv(conv(t, 192, 1), 320, 3, 2)                                  # block D
+    b7 = conv(conv(conv(conv(t, 192, 1), 192, (1, 7), 1, (0, 3)), 192, (7, 1), 1, (3, 0)), 192, 3, 2)
+    t = torch.cat([b3, b7, F.max_pool2d(t, 3, 2)], 1)
+    for _ in range(2):                                                     # 2 x block E
+        b1 = conv(t, 320, 1)
+        y = conv(t, 384, 1)
+        b3 = torch.cat([conv(y, 384, (1, 3), 1, (0, 1)), conv(y, 384, (3, 1), 1, (1, 0))], 1)
+        y = conv(conv(t, 448, 1), 384, 3, 1, 1)
+        bd = torch.cat([conv(y, 384, (1, 3), 1, (0, 1)), conv(y, 384, (3, 1), 1, (1, 0))], 1)
+        bp = conv(avg(t), 192, 1)
+        t = torch.cat([b1, b3, bd, bp], 1)
+    assert t.shape[1:] == (2048, 8, 8)
+    t = F.linear(t.mean(dim=(2, 3)), P.take(32, 2048), P.take(32))
+    assert P.done()
+    assert max_rel_err(logits, t.numpy().ravel()) <= TOL
