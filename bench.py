@@ -67,6 +67,98 @@ def cpu_baseline(model_dir, name, x, budget_s=30.0):
                       "TVM-llvm build of the model" % len(times)}, orc
 
 
+def torch_cpu_baseline(g, x, budget_s=20.0):
+    """The same ResNet-152 (pre-activation, folded batch norms: the network nets.resnet builds,
+    parameters taken in order of definition) as a torch.nn.functional program on the host cores
+    (oneDNN), fp32.  Returns None where torch is not importable."""
+    try:
+        import torch
+        import torch.nn.functional as F
+    except Exception:
+        return None
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    torch.set_num_threads(threads)
+    params = [torch.from_numpy(np.asarray(a, np.float32)) for _, a in g.params]
+
+    def forward():
+        it = iter(params)
+        take = lambda *shape: next(it).reshape(shape)
+        units, filters = [3, 8, 36, 3], [64, 256, 512, 1024, 2048]
+        t = torch.from_numpy(x)[None] + take(1, 3, 1, 1)
+        t = F.relu(F.conv2d(t, take(64, 3, 7, 7), take(64), stride=2, padding=3))
+        act = F.relu(F.max_pool2d(t, 3, 2, 1) + take(1, 64, 1, 1))
+        raw = None
+        for si, n in enumerate(units):
+            cout, mid = filters[si + 1], filters[si + 1] // 4
+            for ui in range(n):
+                first, last = ui == 0, ui == n - 1
+                stride = (1 if si == 0 else 2) if first else 1
+                cin = act.shape[1]
+                y = F.relu(F.conv2d(act, take(mid, cin, 1, 1), take(mid), stride=stride))
+                y = F.relu(F.conv2d(y, take(mid, mid, 3, 3), take(mid), padding=1))
+                sc = F.conv2d(act, take(cout, cin, 1, 1), None, stride=stride) if first else raw
+                w3 = take(cout, mid, 1, 1)
+                if last and si == 3:
+                    act = F.relu((F.conv2d(y, w3) + sc) * take(1, cout, 1, 1) + take(1, cout, 1, 1))
+                elif last:
+                    act = F.relu(F.conv2d(y, w3, take(cout)) + sc)
+                else:
+                    raw = F.conv2d(y, w3) + sc
+                    act = F.relu(raw + take(1, cout, 1, 1))
+        t = act.mean(dim=(2, 3))
+        return F.linear(t, take(1000, 2048), take(1000))
+
+    with torch.no_grad():
+        logits = forward()
+        times = []
+        t_start = time.time()
+        while len(times) < 10 and (time.time() - t_start) < budget_s:
+            t0 = time.time()
+            forward()
+            times.append(time.time() - t0)
+    return {"value": round(min(times) * 1e3, 2), "unit": "ms", "threads": threads,
+            "sample": "%d whole inferences of the same network as torch.nn.functional calls "
+                      "(torch %s, CPU, fp32), best of them" % (len(times), torch.__version__)}, logits.numpy().ravel()
+
+
+def kernel_sources_sha256():
+    """Fingerprint of the device code the committed counter summaries were taken with."""
+    import hashlib
+    h = hashlib.sha256()
+    base = os.path.join(ROOT, "reef_amd", "csrc", "kernels")
+    for f in sorted(os.listdir(base)) + ["../../../include/reef_kernels.h"]:
+        with open(os.path.join(base, f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()
+
+
+def solo_kernel_table(models, name, iters):
+    """Per kernel symbol of one model run alone: launches, average duration, and the fraction of
+    each roofline (matrix-core FLOPs and HBM bytes, algorithmic)."""
+    from reef_amd import binding as B
+    g, d = models[name]
+    exe = B.Executor.from_dir(d, g.name, B.HYBRID)
+    key, x = model_input(name)
+    exe.set_input_checked(key, x)
+    exe.execute()
+    by = {}
+    for i, k in enumerate(g.kernels):
+        us = exe.time_kernel(i, B.RUN_DEFAULT, 3, iters)
+        e = by.setdefault(k["name"].split("#")[0], {"us": 0.0, "flops": 0.0, "bytes": 0.0, "launches": 0})
+        e["us"] += us
+        e["flops"] += g.kernel_flops[i]
+        e["bytes"] += g.kernel_bytes[i]
+        e["launches"] += 1
+    _, dev_us = exe.time_model(B.RUN_DEFAULT, 10, 50)
+    exe.close()
+    return {"model_device_ms": round(float(dev_us.mean()) / 1e3, 4),
+            "kernels": {k: {"launches": v["launches"], "avg_us": round(v["us"] / v["launches"], 3),
+                            "frac_mfma_peak": round(v["flops"] / v["us"] / 1e6 / FP32_MFMA_PEAK_TFLOPS, 4),
+                            "gbs": round(v["bytes"] / v["us"] / 1e3, 1),
+                            "frac_hbm_peak": round(v["bytes"] / v["us"] / 1e3 / HBM_PEAK_GBS, 4)}
+                        for k, v in sorted(by.items())}}
+
+
 def steady_state_conv(root, iters):
     """The staged convolution tiles on two layers large enough to fill the device (12544 and
     3136 output pixels): what the K loop sustains when a launch is not latency bound."""
@@ -290,10 +382,33 @@ def main():
     conv_us = sum(v["us"] for v in conv.values())
     conv_flops = sum(v["flops"] for v in conv.values())
     best_i = int(np.argmax(np.where(flops > 0, flops / np.maximum(kus, 1e-3), 0)))
+    # HBM bytes per launch from the committed counter runs -- only while the device code is the
+    # code those runs were taken with
     traffic = None
+    traffic_note = "no counter summary committed"
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get(dom)
+        tj = json.load(open(tpath))
+        if tj.get("kernel_sources_sha256") != kernel_sources_sha256():
+            traffic_note = "profiles/traffic.json was taken with other kernel sources: not reported"
+        else:
+            traffic = tj.get("bytes_per_launch", {}).get(dom)
+            traffic_note = "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel)"
+    # every distinct convolution shape of the model
+    shapes = {}
+    for i, nm in enumerate(names_k):
+        if not nm.startswith("reef_conv2d_"):
+            continue
+        a = g.kernels[i]["attrs"]
+        e = shapes.setdefault((tuple(a[:12]), nm), {"us": 0.0, "flops": 0.0, "n": 0})
+        e["us"] += kus[i]
+        e["flops"] += flops[i]
+        e["n"] += 1
+    conv_shapes = [{"cin_h_w": list(sh[:3]), "cout_ho_wo": list(sh[3:6]), "k": list(sh[6:8]), "stride": list(sh[8:10]),
+                    "kernel": nm, "launches": e["n"], "avg_us": round(e["us"] / e["n"], 2),
+                    "tflops": round(e["flops"] / e["us"] / 1e6, 2),
+                    "frac_mfma_peak": round(e["flops"] / e["us"] / 1e6 / FP32_MFMA_PEAK_TFLOPS, 4)}
+                   for (sh, nm), e in sorted(shapes.items(), key=lambda kv: -kv[1]["us"])]
 
     if args.solo_only:
         p99 = pct(lat_us, 99)
@@ -340,6 +455,7 @@ def main():
             "unit": "TFLOP/s",
             "frac": round(dom_tflops / FP32_MFMA_PEAK_TFLOPS, 4),
             "traffic": traffic,
+            "traffic_source": traffic_note,
             "launches_per_inference": dom_e["launches"],
             "avg_launch_us": round(dom_e["us"] / dom_e["launches"], 3),
             "avg_launch_gflop": round(dom_e["flops"] / dom_e["launches"] / 1e9, 4),
@@ -350,6 +466,7 @@ def main():
                            "gbs": round(v["bytes"] / v["us"] / 1e3, 1),
                            "frac_hbm_peak": round(v["bytes"] / v["us"] / 1e3 / HBM_PEAK_GBS, 4)}
                        for k, v in sorted(by.items())},
+        "conv_shapes": conv_shapes,
         "timed_region_wall_s": round(wall_s, 3),
     }
     # the classifier's logits (input of the last kernel, the softmax): a saturated softmax
@@ -377,6 +494,11 @@ def main():
                                    dkp_slack=100, interval_us=2000.0),
             "reset": corun(models, "resnet152", "mobilenetv2", 1, B.MODE_RESET, k, 20, solo=False,
                            interval_us=2000.0)}
+    if not args.solo_only:
+        # the bandwidth-bound families are where they matter: MobileNetV2 (depthwise) and BERT-base
+        for extra in ("mobilenetv2", "bert_base"):
+            if extra in models:
+                out["solo_kernels_" + extra] = solo_kernel_table(models, extra, max(args.kernel_iters // 2, 5))
     if 7 in configs and head is not None:
         # the reference's evaluation baselines (scheduler.h:22-28) on the headline workload
         k = max(args.steps // 4, 50)
@@ -397,6 +519,10 @@ def main():
         out["cpu_baseline"] = cb
         ref = np.asarray(orc.storage[logits_idx], np.float64)
         out["parity_logits_max_rel_err_vs_oracle"] = float(np.abs(got - ref).max() / np.abs(ref).max())
+        tc = torch_cpu_baseline(g, x)
+        if tc is not None:
+            out["cpu_baseline"]["torch_cpu"] = tc[0]
+            out["parity_logits_max_rel_err_vs_torch_cpu"] = float(np.abs(got - tc[1]).max() / np.abs(tc[1]).max())
     print(json.dumps(out))
 
 
