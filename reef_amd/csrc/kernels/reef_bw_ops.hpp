@@ -72,6 +72,29 @@ __device__ __forceinline__ void splitk_reduce_body(const ReefOpDesc& d, int task
     }
 }
 
+// Depthwise convolution, one output per thread.  The taps are read with buffer loads whose
+// offset is moved outside the tensor where the tap falls into the padding (the hardware returns
+// 0 there), so a 3x3 filter is nine loads issued back to back with no branch between them; a tap
+// in the padding then adds 0 * w, which leaves the sum as skipping the tap would.
+template <int KH, int KW>
+__device__ __forceinline__ float dw_taps(rsrc_t rs_in, rsrc_t rs_w, unsigned in_base, unsigned w_base, int y0, int x0,
+                                         int H, int W) {
+    float v[KH * KW], w[KH * KW];
+#pragma unroll
+    for (int ky = 0; ky < KH; ++ky)
+#pragma unroll
+        for (int kx = 0; kx < KW; ++kx) {
+            const int iy = y0 + ky, ix = x0 + kx;
+            const bool ok = (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
+            v[ky * KW + kx] = buf_load(rs_in, ok ? in_base + (unsigned)(iy * W + ix) * 4u : kOutside);
+            w[ky * KW + kx] = buf_load(rs_w, w_base + (unsigned)(ky * KW + kx) * 4u);
+        }
+    float acc = 0.0f;
+#pragma unroll
+    for (int t = 0; t < KH * KW; ++t) acc = fmaf(v[t], w[t], acc);
+    return acc;
+}
+
 __device__ __forceinline__ void dwconv2d_body(const ReefOpDesc& d, int task) {
     const int* a = d.attr;
     const int C = a[REEF_DW_C], H = a[REEF_DW_H], W = a[REEF_DW_W], Ho = a[REEF_DW_HO],
@@ -82,15 +105,23 @@ __device__ __forceinline__ void dwconv2d_body(const ReefOpDesc& d, int task) {
     const int c = idx / (Ho * Wo);
     const int r = idx - c * Ho * Wo;
     const int y = r / Wo, x = r - y * Wo;
-    const float* in = (const float*)d.ptr[0] + (size_t)c * H * W;
-    const float* w = (const float*)d.ptr[1] + (size_t)c * kh * kw;
-    float acc = 0.0f;
-    for (int ky = 0; ky < kh; ++ky) {
-        const int iy = y * sh + ky - ph;
-        if ((unsigned)iy >= (unsigned)H) continue;
-        for (int kx = 0; kx < kw; ++kx) {
-            const int ix = x * sw + kx - pw;
-            if ((unsigned)ix < (unsigned)W) acc = fmaf(in[iy * W + ix], w[ky * kw + kx], acc);
+    float acc;
+    if (kh == 3 && kw == 3) {
+        const rsrc_t rs_in = make_rsrc(d.ptr[0], (unsigned)C * (unsigned)(H * W) * 4u);
+        const rsrc_t rs_w = make_rsrc(d.ptr[1], (unsigned)C * 36u);
+        acc = dw_taps<3, 3>(rs_in, rs_w, (unsigned)c * (unsigned)(H * W) * 4u, (unsigned)c * 36u, y * sh - ph,
+                            x * sw - pw, H, W);
+    } else {
+        const float* in = (const float*)d.ptr[0] + (size_t)c * H * W;
+        const float* w = (const float*)d.ptr[1] + (size_t)c * kh * kw;
+        acc = 0.0f;
+        for (int ky = 0; ky < kh; ++ky) {
+            const int iy = y * sh + ky - ph;
+            if ((unsigned)iy >= (unsigned)H) continue;
+            for (int kx = 0; kx < kw; ++kx) {
+                const int ix = x * sw + kx - pw;
+                if ((unsigned)ix < (unsigned)W) acc = fmaf(in[iy * W + ix], w[ky * kw + kx], acc);
+            }
         }
     }
     if (a[REEF_DW_FLAGS] & 1) acc += ((const float*)d.ptr[3])[c];
@@ -111,6 +142,29 @@ __device__ __forceinline__ void pool2d_body(const ReefOpDesc& d, int task) {
     const float* in = (const float*)d.ptr[0] + (size_t)c * H * W;
     float m = -FLT_MAX, s = 0.0f;
     int cnt = 0;
+    if (kh <= 3 && kw <= 3) {
+        // all loads of the window issued together (a tap outside the image or the window reads
+        // outside the buffer and is ignored), then max / sum in window order
+        const rsrc_t rs_in = make_rsrc(d.ptr[0], (unsigned)C * (unsigned)(H * W) * 4u);
+        const unsigned base = (unsigned)c * (unsigned)(H * W) * 4u;
+        float v[9];
+        bool ok[9];
+#pragma unroll
+        for (int dy = 0; dy < 3; ++dy)
+#pragma unroll
+            for (int dx = 0; dx < 3; ++dx) {
+                const int iy = y * sh + dy - ph, ix = x * sw + dx - pw;
+                ok[dy * 3 + dx] = dy < kh && dx < kw && (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
+                v[dy * 3 + dx] = buf_load(rs_in, ok[dy * 3 + dx] ? base + (unsigned)(iy * W + ix) * 4u : kOutside);
+            }
+#pragma unroll
+        for (int t = 0; t < 9; ++t)
+            if (ok[t]) {
+                m = fmaxf(m, v[t]);
+                s += v[t];
+                ++cnt;
+            }
+    } else
     for (int dy = 0; dy < kh; ++dy) {
         const int iy = y * sh + dy - ph;
         if ((unsigned)iy >= (unsigned)H) continue;
@@ -218,6 +272,31 @@ __device__ __forceinline__ void softmax_body(const ReefOpDesc& d, int task) {
     const int lane = threadIdx.x & 63;
     const float* x = (const float*)d.ptr[0] + (size_t)r * cols;
     float* y = (float*)d.ptr[1] + (size_t)r * cols;
+    // Rows of up to 1024 values stay in registers (16 per lane): one trip to memory instead of
+    // three; same values, same order of the maximum and the sum as the general path below.
+    if (cols <= 16 * 64) {
+        float val[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int i = lane + 64 * j;
+            val[j] = i < cols ? x[i] : -FLT_MAX;
+        }
+        float m = -FLT_MAX;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) m = fmaxf(m, val[j]);
+        m = wave_max(m);
+        float s = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            val[j] = expf(val[j] - m);
+            if (lane + 64 * j < cols) s += val[j];
+        }
+        s = wave_sum(s);
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+            if (lane + 64 * j < cols) y[lane + 64 * j] = val[j] / s;
+        return;
+    }
     float m = -FLT_MAX;
     for (int i = lane; i < cols; i += 64) m = fmaxf(m, x[i]);
     m = wave_max(m);
