@@ -23,8 +23,8 @@ TILES = {
     "32x32k4": (6, 32, 32, 0.50, 2),
     "64x32k2": (7, 64, 32, 0.55, 3),
     "32x64k2": (8, 32, 64, 0.55, 3),
-    # direct family (reef_conv2d_d<taps>_16x16k4): never picked by the analytic model, only
-    # through the measured table or an explicit request
+    # direct family (reef_conv2d_d<taps>_16x16k4): picked through the measured table, an explicit
+    # request, or for a shape outside the table by the cost model direct_cost below
     "16x16k4": (9, 16, 16, 0.40, 2),
     "16x32k4": (10, 16, 32, 0.40, 2),
     "16x64k4": (11, 16, 64, 0.40, 2),
@@ -129,6 +129,12 @@ T_FIXED = 2.0            # prologue + epilogue of a workgroup
 T_REDUCE_LAUNCH = 3.0    # extra launch of the split-K reduce
 T_FUSED_REDUCE = 1.0     # fence + last-arrival fold inside the conv kernel
 HBM_BYTES_PER_US = 4.0e6
+# The constants above describe a workgroup in a long, warm run; in a model (cold operands, one
+# launch per layer) the staged tiles measure about three times that, on small and on
+# device-filling layers alike (sweeps behind tuned.py; bench.py's steady_state_conv).  With the
+# factor the estimate is in the same microseconds as direct_cost, and choosing between the two
+# families by estimate loses 7 % against the measured best over the 181 shapes of the sweeps.
+STAGED_SCALE = 3.0
 
 
 def _steps_time(bm, bn, eff, steps):
@@ -156,6 +162,8 @@ def choose(M, N, K, allow_split=True, tiles=None, max_split=32, fused=True, poin
             t["fused"] = hit[1] < 0
             return t
     best = None
+    if allow_split and tiles is None and direct:
+        best = _choose_direct(M, N, K, taps, fused, rows, image)
     for name in (tiles or [t for t in TILES if t not in DIRECT_TILES and t not in ROW_TILES]):
         tid, bm, bn, eff, occ = TILES[name]
         m_tiles, n_tiles = math.ceil(M / bm), math.ceil(N / bn)
@@ -176,13 +184,71 @@ def choose(M, N, K, allow_split=True, tiles=None, max_split=32, fused=True, poin
             t = rounds * (_steps_time(bm, bn, eff, k_chunk // bk) * share + T_FIXED)
             if s_eff > 1:
                 t += (T_FUSED_REDUCE if fused else T_REDUCE_LAUNCH) + (s_eff + 1) * M * N * 4 / HBM_BYTES_PER_US
+            t *= STAGED_SCALE
             cand = (t, name, s_eff, k_chunk, m_tiles, n_tiles)
             if best is None or cand[0] < best[0] - 1e-9:
                 best = cand
+    if len(best) == 2:          # a direct or row-form geometry, complete already
+        return best[1]
     t, name, s, k_chunk, m_tiles, n_tiles = best
     tid, bm, bn, _, _ = TILES[name]
     return dict(tile=name, tile_id=tid, BM=bm, BN=bn, split_k=s, k_chunk=k_chunk,
                 m_tiles=m_tiles, n_tiles=n_tiles, tasks=s * m_tiles * n_tiles, est_us=t)
+
+
+# Cost of a direct-family launch in microseconds, for shapes the measured table does not cover.
+# Linear in what the batch-1 sweeps showed to matter: the cache lines a workgroup pulls in,
+# (BM + BN) K_chunk / 32, times the rounds of workgroups the device needs; the workgroups per
+# CU; and what a split of K adds (folded inside the launch, or as a launch of its own).  The
+# constants are a least-squares fit over the 4095 direct candidates of the sweeps behind
+# tuned.py (181 shapes of four networks, rms error 12 %); choosing by this model instead of by
+# measurement costs 7 % on average over those shapes (worst case 1.5x), where the staged tiles
+# alone cost 62 % (worst 2.8x).
+DIRECT_COST = dict(fixed=3.57, per_line_round=0.00377, fused_split=2.20, separate_split=2.92,
+                   per_wg_per_cu=0.689, per_split=0.172)
+
+
+def direct_cost(tile, geom, fused):
+    _, bm, bn, _, _ = TILES[tile]
+    c = DIRECT_COST
+    s = geom["split_k"]
+    lines = (bm + bn) * geom["k_chunk"] / 32.0
+    t = c["fixed"] + c["per_line_round"] * lines * math.ceil(geom["tasks"] / NUM_CUS) \
+        + c["per_wg_per_cu"] * geom["tasks"] / NUM_CUS
+    if s > 1:
+        t += (c["fused_split"] if fused else c["separate_split"]) + c["per_split"] * s
+    return t
+
+
+def _choose_direct(M, N, K, taps, fused, rows, image):
+    """Best direct (or row-form) tile and split by direct_cost; (cost, geometry)."""
+    best = None
+    for tile in DIRECT_TILES:
+        if taps not in DIRECT_TAPS[tile]:
+            continue
+        for s in (1, 2, 3, 4, 6, 8, 12, 16):
+            g = forced(tile, M, N, K, s, taps)
+            if g["split_k"] != s:
+                continue
+            t = direct_cost(tile, g, fused)
+            if best is None or t < best[0] - 1e-9:
+                g["est_us"] = t
+                g["fused"] = fused and s > 1
+                best = (t, g)
+    if rows and image is not None and best is not None:
+        # the row form of the same nominal tile loads each input value once instead of once per
+        # tap: measured 5 to 10 % ahead of the tap form on the 3x3 layers of the table
+        for tile in ("g2", "g4"):
+            for s in (1, 2, 3, 4, 6, 8):
+                g = forced_rows(tile, M, image[0], image[1], K, s)
+                if g["split_k"] != s:
+                    continue
+                t = 0.93 * direct_cost(tile, g, fused)
+                if t < best[0] - 1e-9:
+                    g["est_us"] = t
+                    g["fused"] = fused and s > 1
+                    best = (t, g)
+    return best
 
 
 def lds_bytes(tile):

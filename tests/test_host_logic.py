@@ -449,3 +449,26 @@ def test_be_stream_cap_is_fixed_once_a_best_effort_queue_exists(fake, small_dirs
     assert s.set_be_stream_cap(0) == 1           # a window of zero kernels makes no sense
     s.create_queue(B.QUEUE_BE)
     assert s.set_be_stream_cap(1) == 1           # Fail: the stream exists with a window of 3
+
+
+def test_tile_choice_outside_the_measured_table():
+    """A shape the measured table does not hold is scored by two cost models in the same unit:
+    batch-1 layers go to the direct family (or the row form for 3x3 / stride 1 / padding 1), a
+    device-filling layer stays on a staged tile, and a filter the direct family is not compiled
+    for never gets a direct tile."""
+    from reef_amd.modelgen import tiling
+    assert (200, 169, 200 * 9, 0) not in tiling.TUNED
+    t = tiling.choose(200, 169, 1800, fused=True, taps=9, direct=True, rows=True, image=(13, 13))
+    assert (t["tile"] in tiling.ROW_TILES or t["tile"] in tiling.DIRECT_TILES) and t["k_chunk"] % 144 == 0
+    t = tiling.choose(200, 169, 1800, fused=True, taps=9, direct=True)
+    assert t["tile"] in tiling.DIRECT_TILES and t["tasks"] == t["split_k"] * t["m_tiles"] * t["n_tiles"]
+    assert t["split_k"] > 1 and t["fused"]            # 143 tiles alone would leave CUs idle
+    t = tiling.choose(200, 169, 1800, fused=True, taps=9, direct=False)
+    assert t["tile"] not in tiling.DIRECT_TILES and t["tile"] not in tiling.ROW_TILES
+    t = tiling.choose(512, 200 * 200, 4608, fused=True, taps=9, direct=True)
+    assert t["tile"] not in tiling.DIRECT_TILES          # 40000 pixels x 512 channels fill the device
+    t = tiling.choose(96, 500, 25 * 40, fused=True, taps=25, direct=tiling.direct_ok(40, 5, 5))
+    assert t["tile"] not in tiling.DIRECT_TILES
+    # both models answer in microseconds of one launch
+    g = tiling.forced("16x32k4", 256, 196, 1024, 2, 1)
+    assert 4.0 < tiling.direct_cost("16x32k4", g, True) < 12.0
