@@ -279,9 +279,13 @@ enum { REEF_ELT_C = 0, REEF_ELT_INNER, REEF_ELT_FLAGS, REEF_ELT_ACT, REEF_ELT_NA
  * tasks = ceil(out_f / 4) (one wavefront per output neuron). */
 enum { REEF_DENSE_ROWS = 0, REEF_DENSE_IN, REEF_DENSE_OUT, REEF_DENSE_FLAGS, REEF_DENSE_ACT, REEF_DENSE_NATTR };
 
-/* ---- reef_softmax: rows x cols, one wavefront per row.  ptr: in, out.  attr: rows, cols.
- * tasks = ceil(rows / 4). */
-enum { REEF_SM_ROWS = 0, REEF_SM_COLS, REEF_SM_NATTR };
+/* ---- reef_softmax: rows x cols, one wavefront per row.  ptr: in, out, mask(optional).
+ * attr: rows, cols, flags(bit0 = mask).  tasks = ceil(rows / 4).
+ * mask: one byte per column (stype uint1), non-zero = that column counts as -inf in every row:
+ * the attention mask the reference applies with a kernel of its own between the scores and the
+ * softmax (fused_reshape_cast_broadcast_to_like_where, resource/bert/bert.cu:381-388; the mask
+ * itself is resource/bert/bert.json storage[1], zero-filled by fused_full_equal_reshape, :313). */
+enum { REEF_SM_ROWS = 0, REEF_SM_COLS, REEF_SM_FLAGS, REEF_SM_NATTR };
 
 /* ---- reef_layernorm: out = LN(x (+res)) * gamma + beta, one wavefront per row ----
  * ptr: x, gamma, beta, out, res(optional).  attr: rows, cols, flags(bit0 = res), eps (float bits).

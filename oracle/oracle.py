@@ -130,11 +130,17 @@ def eltwise(a, b=None, scale=None, shift=None, act=0, act_max=6.0):
     return out
 
 
-def softmax(x):
+def softmax(x, mask=None):
+    """mask: one byte per column, non-zero = the column counts as -inf (bert.cu:381-388)."""
     x = _f(x)
     rows, cols = x.shape
     out = np.empty_like(x)
-    lib().reef_oracle_softmax(_p(x), _p(out), rows, cols)
+    if mask is None:
+        lib().reef_oracle_softmax(_p(x), _p(out), rows, cols)
+    else:
+        mask = np.ascontiguousarray(mask, dtype=np.uint8)
+        assert mask.size >= cols
+        lib().reef_oracle_softmax_masked(_p(x), mask.ctypes.data_as(ctypes.c_void_p), _p(out), rows, cols)
     return out
 
 
@@ -357,7 +363,8 @@ class GraphOracle:
             P[2][:y.size] = y.reshape(-1)
         elif name == "reef_softmax":
             rows, cols = a[:2]
-            P[1][:rows * cols] = softmax(P[0][:rows * cols].reshape(rows, cols)).reshape(-1)
+            mask = P[2].view(np.uint8)[:cols] if len(a) > 2 and a[2] & 1 else None
+            P[1][:rows * cols] = softmax(P[0][:rows * cols].reshape(rows, cols), mask).reshape(-1)
         elif name == "reef_layernorm":
             rows, cols, flags, eps_bits = a[:4]
             res = P[4][:rows * cols].reshape(rows, cols) if flags & 1 else None

@@ -275,15 +275,28 @@ void reef_oracle_eltwise(const float* a, const float* b, const float* scale, con
  * fused_nn_softmax (resnet152.cu:775-841; bert.cu:3-13,159-166,327-337,389-396):
  * per row: m = max, e = exp(x - m), out = e / sum(e).
  */
+void reef_oracle_softmax_masked(const float* in, const unsigned char* mask, float* out, int rows, int cols);
 void reef_oracle_softmax(const float* in, float* out, int rows, int cols) {
+    reef_oracle_softmax_masked(in, 0, out, rows, cols);
+}
+
+/*
+ * The same with the attention mask of the reference's BERT in front
+ * (fused_reshape_cast_broadcast_to_like_where, bert.cu:381-388): x[r][c] = mask[c] ? -inf : x[r][c],
+ * one mask byte per column, shared by all rows.  mask == NULL: no mask.
+ */
+void reef_oracle_softmax_masked(const float* in, const unsigned char* mask, float* out, int rows, int cols) {
     for (int r = 0; r < rows; ++r) {
         const float* x = in + (size_t)r * cols;
         float* y = out + (size_t)r * cols;
         float m = -FLT_MAX;
-        for (int i = 0; i < cols; ++i) m = x[i] > m ? x[i] : m;
+        for (int i = 0; i < cols; ++i) {
+            const float v = (mask && mask[i]) ? -INFINITY : x[i];
+            m = v > m ? v : m;
+        }
         float s = 0.0f;
         for (int i = 0; i < cols; ++i) {
-            y[i] = expf(x[i] - m);
+            y[i] = expf(((mask && mask[i]) ? -INFINITY : x[i]) - m);
             s += y[i];
         }
         for (int i = 0; i < cols; ++i) y[i] = y[i] / s;

@@ -272,6 +272,7 @@ __device__ __forceinline__ void softmax_body(const ReefOpDesc& d, int task) {
     const int lane = threadIdx.x & 63;
     const float* x = (const float*)d.ptr[0] + (size_t)r * cols;
     float* y = (float*)d.ptr[1] + (size_t)r * cols;
+    const unsigned char* mask = (d.attr[REEF_SM_FLAGS] & 1) ? (const unsigned char*)d.ptr[2] : nullptr;
     // Rows of up to 1024 values stay in registers (16 per lane): one trip to memory instead of
     // three; same values, same order of the maximum and the sum as the general path below.
     if (cols <= 16 * 64) {
@@ -280,6 +281,7 @@ __device__ __forceinline__ void softmax_body(const ReefOpDesc& d, int task) {
         for (int j = 0; j < 16; ++j) {
             const int i = lane + 64 * j;
             val[j] = i < cols ? x[i] : -FLT_MAX;
+            if (mask && i < cols && mask[i]) val[j] = -INFINITY;
         }
         float m = -FLT_MAX;
 #pragma unroll
@@ -297,13 +299,14 @@ __device__ __forceinline__ void softmax_body(const ReefOpDesc& d, int task) {
             if (lane + 64 * j < cols) y[lane + 64 * j] = val[j] / s;
         return;
     }
+    auto at = [&](int i) { return (mask && mask[i]) ? -INFINITY : x[i]; };
     float m = -FLT_MAX;
-    for (int i = lane; i < cols; i += 64) m = fmaxf(m, x[i]);
+    for (int i = lane; i < cols; i += 64) m = fmaxf(m, at(i));
     m = wave_max(m);
     float s = 0.0f;
-    for (int i = lane; i < cols; i += 64) s += expf(x[i] - m);
+    for (int i = lane; i < cols; i += 64) s += expf(at(i) - m);
     s = wave_sum(s);
-    for (int i = lane; i < cols; i += 64) y[i] = expf(x[i] - m) / s;
+    for (int i = lane; i < cols; i += 64) y[i] = expf(at(i) - m) / s;
 }
 
 // one wavefront per row; two-pass mean / variance as the reference splits it

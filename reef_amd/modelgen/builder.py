@@ -327,10 +327,12 @@ class GraphBuilder:
                    "dense", 2 * rows * in_f * out_f, 4 * (x.size + in_f * out_f + rows * out_f), 2.0)
         return out
 
-    def softmax(self, x, rows, cols, out=None):
+    def softmax(self, x, rows, cols, out=None, mask=None):
+        """mask: a uint1 storage of `cols` bytes; a non-zero byte turns its column into -inf."""
         out = Tensor(out.idx, (rows, cols)) if out is not None else self.temp((rows, cols))
-        self._emit("reef_softmax", math.ceil(rows / 4), [x.idx, out.idx], [rows, cols], "softmax", 0,
-                   8 * rows * cols, 2.0)
+        args = [x.idx, out.idx] + ([mask.idx] if mask is not None else [])
+        self._emit("reef_softmax", math.ceil(rows / 4), args, [rows, cols, 1 if mask is not None else 0],
+                   "softmax", 0, 8 * rows * cols, 2.0)
         return out
 
     def layernorm(self, x, rows, cols, res=None, eps=1e-12):

@@ -285,14 +285,20 @@ def inception_v3(image=(3, 299, 299), classes=1000, name="inceptionv3", seed=rng
 
 
 def bert(layers=12, hidden=768, heads=12, ffn=3072, seq=128, vocab=30522, name="bert_base",
-         seed=rng.BASE_SEED):
+         seed=rng.BASE_SEED, attention_mask=False):
     """BERT encoder (base: 12 layers, hidden 768, 12 heads, FFN 3072, sequence 128), fp32,
     weights ~ N(0, 0.02).  Token ids are an int64 input, as in the reference's BERT model
     (resource/bert/bert.json storage[0]).  The per-head views of Q, K, V and of the context
-    are expressed as GEMM strides, so no transpose kernels are needed."""
+    are expressed as GEMM strides, so no transpose kernels are needed.
+    attention_mask: a second input `attention_mask` (uint1, one byte per token, non-zero = padding)
+    that every softmax applies to the key positions.  The reference's BERT derives that mask
+    inside the graph -- as all zeros (fused_full_equal_reshape, bert.cu:313) -- and applies it
+    with a kernel of its own per layer (bert.cu:381-388); here it is an operand of the softmax,
+    and a storage nobody has set is all zeros, as every storage is after loading."""
     g = GraphBuilder(name, seed, weight_std=0.02)
     hd = hidden // heads
     ids = g.input("input0", (seq,), "int64")
+    mask = g.input("attention_mask", (seq,), "uint1") if attention_mask else None
     x = g.embedding(ids, vocab, seq, hidden, pos=True, seg=True)
     x = g.layernorm(x, seq, hidden)
     inv_sqrt = 1.0 / (hd ** 0.5)
@@ -305,7 +311,7 @@ def bert(layers=12, hidden=768, heads=12, ffn=3072, seq=128, vocab=30522, name="
         q, k, v = proj
         scores = g.gemm(q, k, seq, seq, hd, batch=heads, trans_b=True, alpha=inv_sqrt,
                         lda=hidden, ldb=hidden, ldc=seq, stride_a=hd, stride_b=hd, stride_c=seq * seq)
-        probs = g.softmax(scores, heads * seq, seq)
+        probs = g.softmax(scores, heads * seq, seq, mask=mask)
         ctx = g.temp((seq, hidden))
         g.gemm(probs, v, seq, hd, seq, batch=heads, trans_b=False, lda=seq, ldb=hidden, ldc=hidden,
                stride_a=seq * seq, stride_b=hd, stride_c=hd, out=ctx)

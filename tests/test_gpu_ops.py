@@ -296,7 +296,8 @@ def test_transformer_ops(tmp_path):
     qh = g.transpose_102(q, seq, heads, hd)                                   # [heads, seq, hd]
     scores = g.gemm(qh, qh, seq, seq, hd, batch=heads, trans_b=True, alpha=0.25,
                     stride_a=seq * hd, stride_b=seq * hd, stride_c=seq * seq)  # Q.K^T
-    pr = g.softmax(scores, heads * seq, seq)
+    amask = g.input("attention_mask", (seq,), "uint1")
+    pr = g.softmax(scores, heads * seq, seq, mask=amask)      # key positions 19.. are padding
     ctx = g.gemm(pr, qh, seq, hd, seq, batch=heads, trans_b=False,
                  stride_a=seq * seq, stride_b=seq * hd, stride_c=seq * hd)     # P.V
     merged = g.transpose_102(ctx, heads, seq, hd)                              # [seq, heads, hd]
@@ -312,8 +313,12 @@ def test_transformer_ops(tmp_path):
     g.copy_into(ln1, cat, seq * hid)
     g.mark_output(cat)
     token_ids = RNG.integers(0, vocab, seq).astype(np.int64)
-    exe, orc, model = run_both(g, tmp_path, {"input0": token_ids})
+    pad = np.zeros(seq, np.uint8)
+    pad[19:] = 1
+    exe, orc, model = run_both(g, tmp_path, {"input0": token_ids, "attention_mask": pad})
     compare_storages(exe, orc, model, what="transformer ops")
+    probs = exe.get_data(pr.idx, heads * seq * seq).reshape(heads * seq, seq)
+    assert (probs[:, 19:] == 0).all() and np.allclose(probs.sum(1), 1, atol=1e-5)
 
 
 @pytest.mark.parametrize("tile", list(tiling.GEMM_DIRECT_TILES))

@@ -145,11 +145,22 @@ def test_densenet_wiring(tmp_path):
     assert max_rel_err(logits, t.numpy().ravel()) <= TOL
 
 
-def test_bert_wiring(tmp_path):
+@pytest.mark.parametrize("masked", [False, True])
+def test_bert_wiring(tmp_path, masked):
     layers, hidden, heads, ffn, seq, vocab = 2, 64, 4, 128, 16, 97
-    g = nets.bert(layers=layers, hidden=hidden, heads=heads, ffn=ffn, seq=seq, vocab=vocab, name="bert_s")
+    g = nets.bert(layers=layers, hidden=hidden, heads=heads, ffn=ffn, seq=seq, vocab=vocab, name="bert_s",
+                  attention_mask=masked)
     ids = nets.token_input("wiring", seq, vocab)
-    got, _, _ = oracle_run(g, tmp_path, "input0", ids)
+    pad = np.zeros(seq, np.uint8)
+    pad[seq - 5:] = 1                       # the last five tokens are padding
+    d = write_model(g, tmp_path)
+    model = json.load(open(os.path.join(d, g.name + ".json")))
+    orc = O.GraphOracle(model, os.path.join(d, g.name + ".param"))
+    orc.set_input("input0", ids)
+    if masked:
+        orc.set_input("attention_mask", pad)
+    got = np.asarray(orc.run()).copy()
+    key_mask = torch.from_numpy(pad.astype(bool)) if masked else None
     P = Params(g)
     tok, pos, seg = P.take(vocab, hidden), P.take(seq, hidden), P.take(hidden)
     t = tok[torch.from_numpy(np.asarray(ids, np.int64))] + pos + seg[None, :]
@@ -161,7 +172,10 @@ def test_bert_wiring(tmp_path):
         k = F.linear(t, P.take(hidden, hidden), P.take(hidden))
         v = F.linear(t, P.take(hidden, hidden), P.take(hidden))
         split = lambda m: m.reshape(seq, heads, hd).permute(1, 0, 2)
-        probs = torch.softmax(split(q) @ split(k).transpose(1, 2) / hd ** 0.5, dim=-1)
+        scores = split(q) @ split(k).transpose(1, 2) / hd ** 0.5
+        if masked:
+            scores = scores.masked_fill(key_mask[None, None, :], float("-inf"))
+        probs = torch.softmax(scores, dim=-1)
         ctx = (probs @ split(v)).permute(1, 0, 2).reshape(seq, hidden)
         att = F.linear(ctx, P.take(hidden, hidden), P.take(hidden))
         t = ln(att + t)

@@ -180,3 +180,20 @@ def test_eltwise_embedding_transpose_mocked():
     three = np.full(8192, 3.0, np.float32)
     tmp = O.mocked(three, three, False)
     np.testing.assert_array_equal(O.mocked(tmp, three, True), np.full(8192, 18.0, np.float32))
+
+
+def test_masked_softmax_is_the_where_kernel_in_front_of_the_softmax():
+    """The reference's attention mask (resource/bert/bert.cu:381-388): where(mask[col], -inf, x)
+    on the scores, then the softmax.  Against torch; masked columns get probability 0 exactly,
+    an all-zero mask changes nothing, and the unmasked columns renormalise among themselves."""
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((12, 37)).astype(np.float32) * 3
+    mask = (rng.random(37) < 0.3).astype(np.uint8)
+    mask[0] = 0
+    got = O.softmax(x, mask)
+    want = F.softmax(torch.from_numpy(x).double().masked_fill(torch.from_numpy(mask.astype(bool)), -np.inf), 1).numpy()
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-9)
+    assert (got[:, mask != 0] == 0).all() and np.allclose(got.sum(1), 1, atol=1e-5)
+    np.testing.assert_array_equal(O.softmax(x, np.zeros(37, np.uint8)), O.softmax(x))
+    keep = mask == 0
+    np.testing.assert_allclose(got[:, keep], O.softmax(x[:, keep]), rtol=1e-6, atol=1e-9)
