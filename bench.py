@@ -78,7 +78,8 @@ def torch_cpu_baseline(g, x, budget_s=20.0):
         return None
     threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
     torch.set_num_threads(threads)
-    params = [torch.from_numpy(np.asarray(a, np.float32)) for _, a in g.params]
+    params = [torch.from_numpy(np.asarray(a, np.float32)) for k, a in g.params
+              if not k.endswith("k")]       # without the packed copies of the 3x3 weights
 
     def forward():
         it = iter(params)

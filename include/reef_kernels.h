@@ -182,6 +182,9 @@ enum {
     REEF_CONV_SYNC_OFF,  /* first counter of this launch inside the sync storage (ints) */
     REEF_CONV_MODE,      /* REEF_CONV_MODE_*: must match the entry symbol's family */
     REEF_CONV_DST_OFF,   /* element offset added to dst (and out2): channel slice of a concat buffer */
+    REEF_CONV_WPACK,     /* pointer slot of the packed copy of the weights (symbols ...d<R>k_ / r9k_), else 0:
+                            [ceil(Cout/16)][ceil(Cin/4)][ceil(taps/4)][4 channels][16 rows][4 taps] floats,
+                            zero where a row, channel or tap does not exist; the last pointer of the kernel */
     REEF_CONV_NATTR
 };
 #define REEF_F_BIAS 1

@@ -36,14 +36,19 @@ struct OpConv {
         return conv2d_body<T, MODE>(d, task, smem, p);
     }
 };
-template <int R, int TN = 1, int TM = 1, bool PRE = false, bool ROWS = false>
+template <int R, int TN = 1, int TM = 1, bool PRE = false, bool ROWS = false, bool PACKED = false>
 struct OpConvDirect {
     static constexpr int LDS = TileD16<TN, TM>::LDS_BYTES;
     template <class P>
     static __device__ __forceinline__ bool run(const ReefOpDesc& d, int task, char* smem, const P& p) {
-        return conv2d_direct_body<R, TN, TM, PRE, ROWS>(d, task, smem, p);
+        return conv2d_direct_body<R, TN, TM, PRE, ROWS, PACKED>(d, task, smem, p);
     }
 };
+// the same with the weights read from their packed copy
+template <int R, int TN = 1, int TM = 1>
+using OpConvDirectK = OpConvDirect<R, TN, TM, false, false, true>;
+template <int G, int TM = 1>
+using OpConvRowsK = OpConvDirect<9, G, TM, false, true, true>;
 // row form of the 3x3 convolution: G image rows x one 14-column segment per workgroup
 template <int G, int TM = 1>
 using OpConvRows = OpConvDirect<9, G, TM, false, true>;
@@ -256,6 +261,16 @@ REEF_ENTRY(reef_conv2d_r9_g4, OpConvRows<4>)
 REEF_ENTRY(reef_conv2d_r9_g7, OpConvRows<7>)
 REEF_ENTRY(reef_conv2d_r9_g2m2, OpConvRows<2 REEF_COMMA 2>)
 REEF_ENTRY(reef_conv2d_r9_g4m2, OpConvRows<4 REEF_COMMA 2>)
+REEF_ENTRY(reef_conv2d_r9k_g1, OpConvRowsK<1>)
+REEF_ENTRY(reef_conv2d_r9k_g2, OpConvRowsK<2>)
+REEF_ENTRY(reef_conv2d_r9k_g4, OpConvRowsK<4>)
+REEF_ENTRY(reef_conv2d_d9k_16x16k4, OpConvDirectK<9>)
+REEF_ENTRY(reef_conv2d_d9k_16x32k4, OpConvDirectK<9 REEF_COMMA 2>)
+REEF_ENTRY(reef_conv2d_d9k_32x32d4, OpConvDirectK<9 REEF_COMMA 2 REEF_COMMA 2>)
+REEF_ENTRY(reef_conv2d_d3k_16x16k4, OpConvDirectK<3>)
+REEF_ENTRY(reef_conv2d_d3k_16x32k4, OpConvDirectK<3 REEF_COMMA 2>)
+REEF_ENTRY(reef_conv2d_d7k_16x16k4, OpConvDirectK<7>)
+REEF_ENTRY(reef_conv2d_d7k_16x32k4, OpConvDirectK<7 REEF_COMMA 2>)
 REEF_ENTRY(reef_gemm_nt_128x128, OpGemm<Tile128x128 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nt_64x64, OpGemm<Tile64x64 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nt_32x128, OpGemm<Tile32x128 REEF_COMMA true>)

@@ -787,11 +787,21 @@ __device__ __forceinline__ float lane_from_right(float v) {  // lane i <- lane (
 // The eight input values a lane loads per step are eight consecutive channels, so their scales
 // and shifts are two 128-bit loads each; a channel past the split loads scale = shift = 0 and
 // contributes relu(0) = 0.  REEF_F_PRE_ACT; the two vectors follow the optional epilogue operands.
-template <int R, int TN, int TM, bool PRE, bool ROWS, class Poll>
+//
+// PACKED (filters with several taps; symbols reef_conv2d_d<R>k_* / reef_conv2d_r9k_*): the weights
+// are read from a copy laid out for these loads instead of from OIHW, where the R taps of one
+// (row, channel) are R * 4 bytes that start at any multiple of 4 and the 16 rows of a tile lie
+// K * 4 bytes apart (a 128-bit load of a wavefront then touches some forty cache lines and most
+// of its lanes are misaligned).  The copy is [Cout / 16][Cin / 4][taps / 4][k slot][row][4 taps]
+// (zero-padded to whole groups): the 64 lanes of a wavefront read 1 KiB contiguous, aligned, per
+// group of four taps.  Measured on the 3x3 layers of ResNet-152: 1.4 us less per launch.  The
+// model generator writes the copy as a parameter of its own; attr WPACK names its pointer slot.
+template <int R, int TN, int TM, bool PRE, bool ROWS, bool PACKED, class Poll>
 __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int task, char* smem_raw,
                                                    const Poll& poll) {
     static_assert(!PRE || R == 1, "the pre-activation form exists for 1-tap filters only");
     static_assert(!ROWS || R == 9, "the row form exists for 3x3 filters only");
+    static_assert(!PACKED || R > 1, "1-tap filters are read from OIHW as they are");
     typedef DirectGeom<R, TN, TM, PRE, ROWS> G;
     typedef TileD16<TN, TM> TD;
     constexpr int RC = G::RC, NS = G::NS;
@@ -873,10 +883,17 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     const rsrc_t rs_a = make_rsrc(d.ptr[1], (unsigned)M * (unsigned)K * 4u);
     const rsrc_t rs_b = make_rsrc(d.ptr[0], (unsigned)C * HW4);
     const int lane_c = cb + (wave * 4 + kq) * G::CPL;     // first channel of this lane's k slot
+    constexpr int G4 = (R + 3) / 4;                 // groups of four taps in the packed copy
+    const unsigned C4 = (unsigned)(C + 3) / 4u;
+    const rsrc_t rs_ap = make_rsrc(d.ptr[PACKED ? a[REEF_CONV_WPACK] : 1],
+                                   PACKED ? (unsigned)((M + 15) / 16) * C4 * (unsigned)G4 * 1024u
+                                          : (unsigned)M * (unsigned)K * 4u);
     unsigned va[TM];
 #pragma unroll
     for (int h = 0; h < TM; ++h)
-        va[h] = ((unsigned)(m0 + 16 * h + i16) * (unsigned)K + (unsigned)(lane_c * R)) * 4u;
+        va[h] = PACKED ? (((unsigned)(m0 / 16 + h) * C4 + (unsigned)(cb / 4 + wave)) * (unsigned)G4) * 1024u
+                             + (unsigned)lane * 16u
+                       : ((unsigned)(m0 + 16 * h + i16) * (unsigned)K + (unsigned)(lane_c * R)) * 4u;
     unsigned vb[ROWS ? TN + 2 : TN][ROWS ? 1 : R];
     if (ROWS) {
         // one value per input row: column of this lane (lane 15: left of the segment)
@@ -919,8 +936,28 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     auto load_step = [&](int s, int step) {
         // offsets are below kOutside (a power of two), so or-ing it in moves them outside
         const unsigned outm = step < lane_steps ? 0u : kOutside;
-        const unsigned sa = (unsigned)step * (unsigned)(G::STEP_C * R) * 4u;   // uniform
+        const unsigned sa = PACKED ? (unsigned)step * (unsigned)(4 * G4) * 1024u      // uniform
+                                   : (unsigned)step * (unsigned)(G::STEP_C * R) * 4u;
         const unsigned sb = (unsigned)step * (unsigned)G::STEP_C * HW4;         // uniform
+        if (PACKED) {
+#pragma unroll
+            for (int h = 0; h < TM; ++h) {
+                const unsigned oa = va[h] | outm;
+#pragma unroll
+                for (int q = 0; q < G4; ++q) {
+                    if (R - 4 * q == 1) {
+                        ra[s][h][4 * q] = __builtin_bit_cast(
+                            float, __builtin_amdgcn_raw_buffer_load_b32(rs_ap, (int)(oa + 1024u * q), (int)sa, 0));
+                    } else {
+                        const f32x4 v = __builtin_bit_cast(
+                            f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_ap, (int)(oa + 1024u * q), (int)sa, 0));
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (4 * q + e < RC) ra[s][h][4 * q + e] = v[e];
+                    }
+                }
+            }
+        } else
 #pragma unroll
         for (int h = 0; h < TM; ++h) {
             const unsigned oa = va[h] | outm;

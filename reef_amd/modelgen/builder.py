@@ -64,6 +64,9 @@ class GraphBuilder:
         self.unique_names = True
         # split-K folded inside the conv kernel (False: separate reef_splitk_reduce launch)
         self.fused_reduce = False
+        # multi-tap filters on the direct / row tiles also get a copy of their weights in the
+        # layout those kernels load fastest (pack_conv_weights); parameter key = weight key + "k"
+        self.pack_weights = True
 
     # ------------------------------------------------------------ storages
     def _storage(self, name, size, stype="float32"):
@@ -145,6 +148,7 @@ class GraphBuilder:
         M, N, K = cout, Ho * Wo, cin * kh * kw
         std = self.weight_std if self.weight_std is not None else math.sqrt(2.0 / K)
         w = given.get("w") or self.param((cout, cin, kh, kw), std)
+        w_arr = None if "w" in given else self.params[-1][1]
         flags = 0
         opt = []
         if bias:
@@ -211,31 +215,44 @@ class GraphBuilder:
         else:
             mode, fam = 0, ""
         kname = "reef_conv2d_" + fam + t["tile"]
+        packed = []
+        if self.pack_weights and w_arr is not None and (fam, t["tile"]) in PACKED_KERNELS:
+            key = self.storage[w.idx]["name"] + "k"
+            arr = pack_conv_weights(w_arr.reshape(cout, cin, kh * kw))
+            pidx = self._storage(key, arr.size)
+            self.graph_args.append(pidx)
+            self.params.append((key, arr))
+            packed = [pidx]
+            kname = "reef_conv2d_" + fam[:-1] + "k_" + t["tile"]
+            nbytes_pack = 4 * (arr.size - M * K)        # the copy is read instead of the original
+        else:
+            nbytes_pack = 0
         if out2 is not None:
             nbytes += 4 * (M * N + M)
         if pre:
             flags |= F_PRE_ACT
             nbytes += 4 * 2 * cin
         if t["split_k"] == 1:
+            args = [x.idx, w.idx, out.idx] + opt + pre
             attrs = base + [flags, act, t["tile_id"], 1, t["k_chunk"], t["m_tiles"], t["n_tiles"], act2,
-                            0, mode, dst_off]
-            self._emit(kname, t["tasks"], [x.idx, w.idx, out.idx] + opt + pre, attrs, "conv2d", flops,
-                       nbytes, t["est_us"])
+                            0, mode, dst_off, len(args) if packed else 0]
+            self._emit(kname, t["tasks"], args + packed, attrs, "conv2d", flops, nbytes + nbytes_pack, t["est_us"])
         elif fused_reduce:
             # workspace: split_k partial tensors; counters: one int per output tile in
             # the model's single sync storage
             ws = self.workspace(t["split_k"] * M * N)
             sync_idx, sync_off = self._sync_counters(t["m_tiles"] * t["n_tiles"])
+            args = [x.idx, w.idx, out.idx] + opt + pre + [ws.idx, sync_idx]
             attrs = base + [flags | F_FUSED_REDUCE, act, t["tile_id"], t["split_k"], t["k_chunk"],
-                            t["m_tiles"], t["n_tiles"], act2, sync_off, mode, dst_off]
-            self._emit(kname, t["tasks"], [x.idx, w.idx, out.idx] + opt + pre + [ws.idx, sync_idx], attrs,
-                       "conv2d", flops, nbytes, t["est_us"])
+                            t["m_tiles"], t["n_tiles"], act2, sync_off, mode, dst_off, len(args) if packed else 0]
+            self._emit(kname, t["tasks"], args + packed, attrs, "conv2d", flops, nbytes + nbytes_pack, t["est_us"])
         else:
             ws = self.workspace(t["split_k"] * M * N)
+            args = [x.idx, w.idx, ws.idx] + pre
             attrs = base + [F_PRE_ACT if pre else 0, ACT_NONE, t["tile_id"], t["split_k"], t["k_chunk"],
-                            t["m_tiles"], t["n_tiles"], ACT_NONE, 0, mode, 0]
-            self._emit(kname, t["tasks"], [x.idx, w.idx, ws.idx] + pre, attrs, "conv2d", flops,
-                       4 * (x.size + M * K + t["split_k"] * M * N), t["est_us"])
+                            t["m_tiles"], t["n_tiles"], ACT_NONE, 0, mode, 0, len(args) if packed else 0]
+            self._emit(kname, t["tasks"], args + packed, attrs, "conv2d", flops,
+                       4 * (x.size + M * K + t["split_k"] * M * N) + nbytes_pack, t["est_us"])
             self._emit("reef_splitk_reduce", math.ceil(M * N / 1024), [ws.idx, out.idx] + opt,
                        [M, N, t["split_k"], flags & ~F_PRE_ACT, act, act2, dst_off], "splitk_reduce", 0,
                        4 * ((t["split_k"] + 1) * M * N), 2.0)
@@ -474,6 +491,24 @@ class GraphBuilder:
         with open(base + ".meta.json", "w") as f:
             json.dump(meta, f)
         return base
+
+
+# (loader family prefix, tile) of the kernels that exist in a packed-weights form
+PACKED_KERNELS = {("r9_", "g1"), ("r9_", "g2"), ("r9_", "g4"), ("d9_", "16x16k4"), ("d9_", "16x32k4"),
+                  ("d9_", "32x32d4"), ("d3_", "16x16k4"), ("d3_", "16x32k4"), ("d7_", "16x16k4"),
+                  ("d7_", "16x32k4")}
+
+
+def pack_conv_weights(w):
+    """[Cout][Cin][taps] weights -> the layout of attr REEF_CONV_WPACK:
+    [ceil(Cout/16)][ceil(Cin/4)][ceil(taps/4)][4 channels][16 rows][4 taps], zero-padded."""
+    M, C, R = w.shape
+    mt, c4, g4 = -(-M // 16), -(-C // 4), -(-R // 4)
+    pad = np.zeros((mt * 16, c4 * 4, g4 * 4), np.float32)
+    pad[:M, :C, :R] = w
+    # pad[mt*16 + i, c4*4 + kq, g*4 + j] -> out[mt, c4, g, kq, i, j]
+    out = pad.reshape(mt, 16, c4, 4, g4, 4).transpose(0, 2, 4, 3, 1, 5)
+    return np.ascontiguousarray(out).reshape(-1)
 
 
 def write_params(path, params):

@@ -159,6 +159,10 @@ def test_dkp_corun_bit_identical(dirs):
     x18 = nets.image_input("resnet18", (3, 224, 224))
     ref_rt = solo_output(dirs["resnet18"], "resnet18", x18)
     s = B.Scheduler(B.MODE_REEF)
+    # the reference's rule: a best-effort kernel may take as long as the real-time kernel it pads
+    # (scheduler.cpp:565-572); with the default half of that the few-microsecond layers of this
+    # network do not always leave room for both mocked kernels
+    s.set_dkp_slack_percent(100)
     rt_mid = s.load_model(dirs["resnet18"], "resnet18")
     be_mid = s.load_model(dirs["mocked_kernel"], "mocked_kernel")
     rt_q, be_q = s.create_queue(B.QUEUE_RT), s.create_queue(B.QUEUE_BE)
