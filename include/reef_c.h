@@ -70,6 +70,11 @@ int reef_executor_time_kernel(reef_executor_t e, int idx, int flavour, int warmu
  * and the first `task_num` tasks only -- the measurement behind <model>.profile.json
  * (latency[j] = one round of (j+1) x num_cus workgroups; the reference's profiler tool
  * is not in its repository, resource/Makefile:32-36). */
+/* The same with the kernel confined to `cus` virtual CUs (0: all), as the best-effort side of a
+ * padded launch is: `layers` workgroups then really share each of those CUs.  What a profile's
+ * latency[layers - 1] has to describe (scheduler.cpp:565-572,589-590). */
+int reef_executor_time_kernel_dkp_confined(reef_executor_t e, int idx, int layers, int task_num, int cus,
+                                           int warmup, int iters, float* avg_us);
 int reef_executor_time_kernel_dkp(reef_executor_t e, int idx, int layers, int task_num, int warmup,
                                   int iters, float* avg_us);
 int reef_executor_time_model(reef_executor_t e, int flavour, int warmup, int iters, float* lat_us,

@@ -171,6 +171,11 @@ int reef_hal_write_value32(reef_stream_t s, reef_devptr_t ptr, int32_t value);
  * directly from the calling thread and is visible to running kernels about a microsecond later;
  * otherwise the layer falls back to a stream write it waits for.  No ordering against any stream. */
 int reef_hal_host_write32(reef_devptr_t ptr, int32_t value);
+/* The same for a run of 32-bit words: n_words stores of `value` from the calling thread into
+ * REEF_MEM_DEVICE_FINEGRAINED memory, no device work and no stream.  Nothing on the device may
+ * be using the words meanwhile.  Returns 2 where device memory cannot be stored to from the host
+ * (the caller then fills through a stream). */
+int reef_hal_host_fill32(reef_devptr_t ptr, int32_t value, size_t n_words);
 /* Wait until the kernels `s` already has ON THE DEVICE have finished; launches the stream still
  * holds on the host stay there (hipStreamSynchronize after hipStreamClearQueue, scheduler.cpp:339).
  * For a windowed stream this spins on the stream's completion counter instead of sleeping in
@@ -251,6 +256,7 @@ typedef struct reef_hal_backend {
     int (*stream_exit_ticks)(reef_stream_t, uint32_t, uint64_t*);
     int (*clock_sync)(int64_t*, uint64_t*, int64_t*, int*);
     int (*module_kernel_entry)(reef_module_t, const char*, uint64_t*);
+    int (*host_fill32)(reef_devptr_t, int32_t, size_t);
 } reef_hal_backend;
 
 const reef_hal_backend* reef_hal_hip_backend(void);

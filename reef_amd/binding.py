@@ -162,6 +162,12 @@ class Executor:
                                                              ctypes.byref(us)))
         return us.value
 
+    def time_kernel_dkp_confined(self, idx, layers, task_num, cus, warmup=2, iters=10):
+        us = ctypes.c_float()
+        _check("time_kernel_dkp_confined", lib().reef_executor_time_kernel_dkp_confined(
+            self.h, idx, layers, task_num, cus, warmup, iters, ctypes.byref(us)))
+        return us.value
+
     def time_kernel_dkp(self, idx, layers, task_num, warmup=2, iters=10):
         us = ctypes.c_float()
         _check("time_kernel_dkp", lib().reef_executor_time_kernel_dkp(self.h, idx, layers, task_num,

@@ -141,16 +141,21 @@ int reef_executor_time_kernel(reef_executor_t e, int idx, int flavour, int warmu
 
 int reef_executor_time_kernel_dkp(reef_executor_t e, int idx, int layers, int task_num, int warmup,
                                   int iters, float* avg_us) {
+    return reef_executor_time_kernel_dkp_confined(e, idx, layers, task_num, 0, warmup, iters, avg_us);
+}
+int reef_executor_time_kernel_dkp_confined(reef_executor_t e, int idx, int layers, int task_num, int cus,
+                                           int warmup, int iters, float* avg_us) {
     TransExecutor* t = e->trans();
-    if (!t || idx < 0 || idx >= (int)t->num_kernels() || iters <= 0 || layers <= 0) return Status::OutOfRange;
+    if (!t || idx < 0 || idx >= (int)t->num_kernels() || iters <= 0 || layers <= 0 || cus < 0)
+        return Status::OutOfRange;
     GPUStream_t s = t->stream();
-    for (int i = 0; i < warmup; ++i) RETURN_STATUS(t->launch_kernel_dkp(idx, layers, task_num, s));
+    for (int i = 0; i < warmup; ++i) RETURN_STATUS(t->launch_kernel_dkp(idx, layers, task_num, s, cus));
     reef_event_t a, b;
     GPU_RETURN_STATUS(reef_hal_event_create(&a));
     GPU_RETURN_STATUS(reef_hal_event_create(&b));
     GPU_RETURN_STATUS(reef_hal_stream_sync(s));
     GPU_RETURN_STATUS(reef_hal_event_record(a, s));
-    for (int i = 0; i < iters; ++i) RETURN_STATUS(t->launch_kernel_dkp(idx, layers, task_num, s));
+    for (int i = 0; i < iters; ++i) RETURN_STATUS(t->launch_kernel_dkp(idx, layers, task_num, s, cus));
     GPU_RETURN_STATUS(reef_hal_event_record(b, s));
     GPU_RETURN_STATUS(reef_hal_event_sync(b));
     float us = 0.f;

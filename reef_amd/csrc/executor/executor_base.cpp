@@ -8,13 +8,14 @@ namespace reef {
 namespace executor {
 
 ExecutorBase::ExecutorBase()
-    : arena(nullptr), arena_bytes(0), base_mod(nullptr), s(nullptr), owns_stream(false),
+    : arena(nullptr), arena_bytes(0), sync_mem(nullptr), base_mod(nullptr), s(nullptr), owns_stream(false),
       use_graph(std::getenv("REEF_GRAPH") != nullptr), model_graph(nullptr) {}
 
 ExecutorBase::~ExecutorBase() {
     drop_graph();
     if (owns_stream && s) reef_hal_stream_destroy(s);
     if (arena) reef_hal_free(arena, REEF_MEM_DEVICE);
+    if (sync_mem) reef_hal_free(sync_mem, REEF_MEM_DEVICE_FINEGRAINED);
 }
 
 Status ExecutorBase::load_model_from_file(const char* json_file_path, const char* co_file_path) {
@@ -65,8 +66,16 @@ Status ExecutorBase::init_executor_base(const char* json_file_path, GPUModule_t 
     // storages: one zero-filled arena
     std::vector<size_t> offs(model->storage.size());
     size_t total = 0;
+    // The arrival counters of folded split-K launches ("reef_sync") live in fine-grained memory
+    // of their own: the scheduler clears them from the host, without a device operation, before
+    // it pads a kernel of a model whose last run was cut short.
+    size_t sync_idx = model->storage.size();
     for (size_t i = 0; i < model->storage.size(); ++i) {
         if (Model::get_stype_size(model->storage[i].stype) == 0) return Status::Fail;
+        if (model->storage[i].name == "reef_sync" && sync_idx == model->storage.size()) {
+            sync_idx = i;
+            continue;
+        }
         offs[i] = total;
         total += align_up<size_t>(std::max<size_t>(storage_bytes(i), 4), 256);
     }
@@ -75,6 +84,12 @@ Status ExecutorBase::init_executor_base(const char* json_file_path, GPUModule_t 
     GPU_RETURN_STATUS(reef_hal_memset(arena, 0, arena_bytes));
     storage.resize(model->storage.size());
     for (size_t i = 0; i < storage.size(); ++i) storage[i] = (char*)arena + offs[i];
+    if (sync_idx < model->storage.size()) {
+        const size_t bytes = align_up<size_t>(std::max<size_t>(storage_bytes(sync_idx), 4), 256);
+        GPU_RETURN_STATUS(reef_hal_malloc(bytes, REEF_MEM_DEVICE_FINEGRAINED, &sync_mem));
+        GPU_RETURN_STATUS(reef_hal_memset(sync_mem, 0, bytes));
+        storage[sync_idx] = sync_mem;
+    }
 
     // per-call descriptors
     descs.assign(model->kernels.size(), ReefOpDesc());

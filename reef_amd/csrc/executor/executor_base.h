@@ -78,6 +78,7 @@ protected:
     std::vector<ReefOpDesc> descs;                  // per kernel call
     GPUDevicePtr_t arena;
     size_t arena_bytes;
+    GPUDevicePtr_t sync_mem;   // the "reef_sync" storage (fine-grained memory of its own), or null
     GPUModule_t base_mod;
     GPUStream_t s;
     bool owns_stream;

@@ -151,6 +151,16 @@ Status HybridExecutor::reset_sync_storage(GPUStream_t stream) {
     return Status::Succ;
 }
 
+// The same from the host, with no device operation; `fallback` is the stream the fill goes to
+// where the host cannot store into device memory.  No kernel of the model may be running.
+Status HybridExecutor::reset_sync_storage_from_host(GPUStream_t fallback) {
+    if (sync_bytes == 0) return Status::Succ;
+    const int rc = reef_hal_host_fill32(sync_ptr, 0, sync_bytes / 4);
+    if (rc == 0) return Status::Succ;
+    if (rc != 2) RETURN_STATUS(Status::Fail);
+    return reset_sync_storage(fallback);
+}
+
 Status HybridExecutor::launch_preempt_kernel(int i, GPUStream_t stream) {
     const KernelArg& ka = trans_args[i];
     ReefBeArgs arg;

@@ -39,6 +39,7 @@ public:
     // fold split-K internally) in stream order.  Needed before kernels of this model
     // run again after an interrupted run; a no-op for models without that storage.
     Status reset_sync_storage(GPUStream_t stream);
+    Status reset_sync_storage_from_host(GPUStream_t fallback);
     bool has_sync_storage() const { return sync_bytes > 0; }
     const ModelProfile* profile() const { return model_profile.get(); }
 

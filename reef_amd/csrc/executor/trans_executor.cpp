@@ -114,18 +114,27 @@ Status TransExecutor::launch_kernel(int i, GPUStream_t stream) {
     return Status::Succ;
 }
 
-// One single-sided launch with an explicit layer count and task range (profiling).
-Status TransExecutor::launch_kernel_dkp(int i, int layers, int task_num, GPUStream_t stream) {
+// One single-sided launch with an explicit layer count and task range (profiling).  cus > 0:
+// the kernel is confined to that many virtual CUs as the best-effort side of a padded launch is
+// (the right side of a partition with nothing on the left), so `layers` workgroups really share
+// each of those CUs.
+Status TransExecutor::launch_kernel_dkp(int i, int layers, int task_num, GPUStream_t stream, int cus) {
     const KernelArg& ka = trans_args[i];
     const int num_cus = (int)GPUConfig::get_num_cus();
+    const int num_xcds = (int)GPUConfig::get_num_xcds();
     ReefDkpArgs a;
     std::memset(&a, 0, sizeof(a));
     fill_side(a.l, i, layers, std::min(task_num, ka.block_num), 0);
     a.r = a.l;
     a.r.task_num = 0;
     a.cu_partition = num_cus;
+    if (cus > 0 && cus < num_cus) {
+        a.r = a.l;
+        a.l.task_num = 0;
+        a.cu_partition = num_cus - align_up(cus, num_xcds);
+    }
     a.num_cus = num_cus;
-    a.num_xcds = (int)GPUConfig::get_num_xcds();
+    a.num_xcds = num_xcds;
     const uint32_t grid[3] = {(uint32_t)(num_cus * layers), 1, 1};
     const uint32_t block[3] = {ka.thread_dim.count(), 1, 1};
     GPU_RETURN_STATUS(reef_hal_launch(ka.kernel, grid, block, 0, stream, &a, sizeof(a)));

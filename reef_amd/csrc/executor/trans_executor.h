@@ -43,7 +43,7 @@ public:
     static int op_from_name(const std::string& name);
 
     const std::vector<KernelArg>& kernel_args() const { return trans_args; }
-    Status launch_kernel_dkp(int kernel_offset, int layers, int task_num, GPUStream_t stream);
+    Status launch_kernel_dkp(int kernel_offset, int layers, int task_num, GPUStream_t stream, int cus = 0);
     // Waves per SIMD a register count allows on gfx950
     // (trans_executor.cpp:175-199 picks among 10 gfx906 classes the same way).
     static int occupancy_class(const GPUConfig::KernelResource& kr);

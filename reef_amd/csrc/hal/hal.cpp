@@ -68,6 +68,12 @@ int reef_hal_write_value32(reef_stream_t s, reef_devptr_t ptr, int32_t value) {
     return be()->write_value32(s, ptr, value);
 }
 int reef_hal_host_write32(reef_devptr_t ptr, int32_t value) { return be()->host_write32(ptr, value); }
+int reef_hal_host_fill32(reef_devptr_t ptr, int32_t value, size_t n_words) {
+    if (be()->host_fill32) return be()->host_fill32(ptr, value, n_words);
+    for (size_t i = 0; i < n_words; i++)   // a backend without a call of its own: word by word
+        if (int rc = be()->host_write32((char*)ptr + 4 * i, value)) return rc;
+    return 0;
+}
 int reef_hal_stream_wait_device(reef_stream_t s) { return be()->stream_wait_device(s); }
 int reef_hal_graph_begin(reef_stream_t s) { return be()->graph_begin(s); }
 int reef_hal_graph_end(reef_stream_t s, reef_graph_t* out) { return be()->graph_end(s, out); }

@@ -27,6 +27,15 @@ __global__ void clock_probe(volatile uint32_t* mailbox, uint32_t round, uint32_t
                        __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
+// Fills n 32-bit words.  What reef_hal_memset_async launches instead of a runtime fill: the
+// runtime's own fill costs about 20 us on a stream that has kernels ahead of it (it is not an
+// ordinary dispatch of that stream), this one what any small kernel costs; it can also be
+// recorded into a graph, where a memset node cannot be relied on.
+__global__ void fill_words(uint32_t* p, uint32_t value, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = value;
+}
+
 int64_t now_ns() {
     return std::chrono::duration_cast<std::chrono::nanoseconds>(
                std::chrono::steady_clock::now().time_since_epoch()).count();
@@ -36,6 +45,20 @@ volatile uint32_t* g_mailbox = nullptr;
 uint32_t g_round = 0;
 
 }  // namespace
+
+// byte pattern -> n bytes at p (both multiples of 4), as a kernel on `stream`
+int reef_hal_hip_fill(hipStream_t stream, void* p, int byte, size_t n) {
+    const uint32_t b = (uint32_t)(byte & 0xFF);
+    const uint32_t word = b | (b << 8) | (b << 16) | (b << 24);
+    const size_t words = n / 4;
+    if (words == 0) return 0;
+    hipLaunchKernelGGL(fill_words, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream, (uint32_t*)p, word, words);
+    if (hipGetLastError() != hipSuccess) {
+        reef_hal_set_error("reef_hal_memset_async: fill kernel launch failed");
+        return 1;
+    }
+    return 0;
+}
 
 // One correlated (host steady clock, device wall clock) pair: best of `tries` exchanges.
 int reef_hal_hip_clock_probe(hipStream_t stream, int64_t* host_ns, uint64_t* device_ticks, int64_t* err_ns,

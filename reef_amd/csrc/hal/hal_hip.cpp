@@ -17,6 +17,7 @@
 #include "reef_hal.h"
 
 // hal_device.hip
+int reef_hal_hip_fill(hipStream_t stream, void* p, int byte, size_t n);
 int reef_hal_hip_clock_probe(hipStream_t stream, int64_t* host_ns, uint64_t* device_ticks, int64_t* err_ns,
                              int* ticks_per_us);
 
@@ -523,6 +524,13 @@ int h_host_write32(reef_devptr_t p, int32_t v) {
     HIPCHK(hipStreamSynchronize(g_flag_stream));
     return 0;
 }
+int h_host_fill32(reef_devptr_t p, int32_t v, size_t n_words) {
+    if (!g_host_visible) return 2;
+    volatile int32_t* w = (volatile int32_t*)p;
+    for (size_t i = 0; i < n_words; i++) w[i] = v;
+    __atomic_thread_fence(__ATOMIC_SEQ_CST);   // push the write-combined stores out now
+    return 0;
+}
 int h_stream_wait_device(reef_stream_t st) {
     if (st && st->window > 0) {
         // What the device has been given by now.  A launch the feeder has taken out of the ring
@@ -626,16 +634,22 @@ int h_clear_queue(reef_stream_t st, uint64_t* n) {
 }
 int h_reset_cus() { return 0; }
 
+// Word-sized fills go out as a small kernel of this library (see fill_words), anything else
+// through the runtime.
+int fill_async(reef_devptr_t p, int byte, size_t n, hipStream_t s) {
+    if (n % 4 == 0 && ((uintptr_t)p) % 4 == 0 && n <= (size_t)1 << 30) return reef_hal_hip_fill(s, p, byte, n);
+    HIPCHK(hipMemsetAsync(p, byte, n, s));
+    return 0;
+}
+
 int h_memset_async(reef_devptr_t p, int byte, size_t n, reef_stream_t st) {
     // a windowed stream may hold launches on the host: the fill must not overtake them
     if (st && st->window > 0) {
         if (int rc = drain_ring(st)) return rc;
         std::lock_guard<std::mutex> sub(st->submit_mtx);   // behind a launch the feeder has in hand
-        HIPCHK(hipMemsetAsync(p, byte, n, st->s));
-        return 0;
+        return fill_async(p, byte, n, st->s);
     }
-    HIPCHK(hipMemsetAsync(p, byte, n, st ? st->s : nullptr));
-    return 0;
+    return fill_async(p, byte, n, st ? st->s : nullptr);
 }
 
 int h_event_create(reef_event_t* out) {
@@ -666,7 +680,7 @@ const reef_hal_backend kHip = {
     h_memset_async, h_host_write32, h_stream_wait_device,
     h_graph_begin, h_graph_end, h_graph_launch, h_graph_destroy,
     h_stream_set_completion, h_stream_progress, h_stream_exit_ticks, h_clock_sync,
-    h_module_kernel_entry,
+    h_module_kernel_entry, h_host_fill32,
 };
 
 }  // namespace

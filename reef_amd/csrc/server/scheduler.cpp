@@ -615,16 +615,15 @@ void REEFScheduler::dynamic_kernel_padding(std::shared_ptr<Task>& rt_task) {
             if (!cand || cand->state.load() == TaskState::Finish) continue;
             HybridExecutor& be_exe = cand->model->executor;
             if (cand->kernel_offset >= (int)be_exe.num_kernels()) continue;
-            if (cand->sync_dirty) {
-                // an interrupted run left arrival counters behind: pad this task only once
-                // its own stream has drained, and clear the counters first
-                if (be_exe.has_sync_storage()) {
-                    if (!executor::GPUStreamEmpty(be_queues[q]->stream)) continue;
-                    be_exe.reset_sync_storage(rt_queue->stream);
-                }
-                cand->sync_dirty = false;
-            }
             const TransExecutor::KernelArg& ka = be_exe.trans_args[cand->kernel_offset];
+            // Cheapest test first: a kernel that is too long at every occupancy cannot be padded
+            // (decide_padding would find the same).  This loop runs between two real-time
+            // launches, so what it costs per candidate is real-time latency.
+            {
+                const std::vector<int>& lat = ka.profile.latency_ns;
+                const int64_t budget = (int64_t)rt_args.profile.total_latency_ns * dkp_slack_percent / 100;
+                if (lat.empty() || *std::min_element(lat.begin(), lat.end()) > budget) continue;
+            }
             // the proxy whose two register ranges hold both kernels sets the register budget of
             // the launch (scheduler.cpp:613-642 / trans_executor.cpp:175-199)
             const int px = TransExecutor::select_proxy(proxies, rt_args.resource, ka.resource);
@@ -632,6 +631,17 @@ void REEFScheduler::dynamic_kernel_padding(std::shared_ptr<Task>& rt_task) {
             PadDecision d = decide_padding(rt_args, ka, cand->block_offset, proxies[px].resource, num_cus,
                                            num_xcds, dkp_slack_percent);
             if (!d.merge) continue;
+            if (cand->sync_dirty) {
+                // An interrupted run left arrival counters behind: pad this task only once its own
+                // stream has drained, and clear the counters first -- from the host (a fill on
+                // the real-time stream would sit in front of the real-time kernels), and only now
+                // that a kernel of the task is really about to be padded.
+                if (be_exe.has_sync_storage()) {
+                    if (!executor::GPUStreamEmpty(be_queues[q]->stream)) continue;
+                    be_exe.reset_sync_storage_from_host(rt_queue->stream);
+                }
+                cand->sync_dirty = false;
+            }
             dec = d;
             proxy_idx = px;
             be_task = cand;

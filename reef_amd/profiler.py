@@ -29,14 +29,20 @@ def measure_profile(model_dir, name, iters=10, warmup=2, levels=8):
         total = exe.time_kernel_dkp(i, info["min_occupancy"], blocks, warmup, iters)
         max_occ = B.lib().reef_gpuconfig_calculate_occupancy(info["lds"], info["vgprs"], info["sgprs"],
                                                              info["scratch"], 256)
+        # latency[j]: one round at occupancy j + 1, with the kernel confined to a few CUs as the
+        # best-effort side of a padded launch is, so that j + 1 workgroups really share a CU (on
+        # the whole device most kernels do not have the workgroups to reach occupancy 2, and the
+        # cost of sharing a CU -- what a CU can pull from memory -- would not show)
         lat = []
-        for j in range(min(levels, max(max_occ, 1))):
-            us = exe.time_kernel_dkp(i, j + 1, min(blocks, (j + 1) * num_cus), warmup, iters)
-            lat.append(max(1, int(round(us * 1000))))
-            if (j + 1) * num_cus >= blocks:
-                # more layers cannot hold more of this kernel's workgroups
-                lat += [lat[-1]] * (min(levels, max(max_occ, 1)) - len(lat))
+        n_levels = min(levels, max(max_occ, 1))
+        for j in range(n_levels):
+            cus = next((c for c in (32, 16, 8) if (j + 1) * c <= blocks), 0)
+            if cus == 0:
+                # not enough workgroups for this occupancy even on 8 CUs: it cannot occur
+                lat += [lat[-1] if lat else max(1, int(round(total * 1000)))] * (n_levels - len(lat))
                 break
+            us = exe.time_kernel_dkp_confined(i, j + 1, (j + 1) * cus, cus, warmup, iters)
+            lat.append(max(1, int(round(us * 1000))))
         e = kl.setdefault(k["name"], {"total_latency": 0, "latency": [], "total_latency_ns": 0, "latency_ns": lat})
         e["total_latency_ns"] = max(e["total_latency_ns"], max(1, int(round(total * 1000))))
         e["latency_ns"] = [max(a, b) for a, b in zip(e["latency_ns"], lat)]
