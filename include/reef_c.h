@@ -77,6 +77,14 @@ int reef_executor_time_kernel_dkp_confined(reef_executor_t e, int idx, int layer
                                            int warmup, int iters, float* avg_us);
 int reef_executor_time_kernel_dkp(reef_executor_t e, int idx, int layers, int task_num, int warmup,
                                   int iters, float* avg_us);
+/* One launch between two events, `samples` times, median in *single_us.  With evict_bytes > 0 the
+ * `evict` buffer (device memory of the caller, larger than the device's last-level cache) is
+ * overwritten before every sample, so the kernel finds its operands in HBM -- the state a
+ * best-effort kernel is in when several models take turns on the device; with evict_bytes == 0 the
+ * kernel itself runs once before every sample (operands cached).  The two medians carry the same
+ * event overhead, so their difference is what a cold start adds to a back-to-back figure. */
+int reef_executor_time_kernel_dkp_single(reef_executor_t e, int idx, int layers, int task_num, int cus,
+                                         void* evict, size_t evict_bytes, int samples, float* single_us);
 int reef_executor_time_model(reef_executor_t e, int flavour, int warmup, int iters, float* lat_us,
                              float* dev_us);
 

@@ -143,6 +143,11 @@ int reef_hal_stream_destroy(reef_stream_t s);
 int reef_hal_stream_set_completion(reef_stream_t s, int mode);
 /* Launches handed to the device so far on a windowed stream, and how many have signalled. */
 int reef_hal_stream_progress(reef_stream_t s, uint32_t* submitted, uint32_t* done);
+/* *drained = 1 when nothing of a windowed stream is held back and every launch handed to the
+ * device has signalled.  Reads the stream's counters only -- no call into the runtime, whose own
+ * query may put a marker into the hardware queue that the kernels of other streams then queue
+ * behind; for the real-time launch loop.  A stream without a window: reef_hal_stream_query. */
+int reef_hal_stream_drained(reef_stream_t s, int* drained);
 /* Device wall clock at which launch `seq` of a windowed stream in REEF_COMPLETE_IN_KERNEL mode
  * left the device (its last workgroup); kept for the 8 most recent launches.  0 if unknown. */
 int reef_hal_stream_exit_ticks(reef_stream_t s, uint32_t seq, uint64_t* ticks);
@@ -257,6 +262,7 @@ typedef struct reef_hal_backend {
     int (*clock_sync)(int64_t*, uint64_t*, int64_t*, int*);
     int (*module_kernel_entry)(reef_module_t, const char*, uint64_t*);
     int (*host_fill32)(reef_devptr_t, int32_t, size_t);
+    int (*stream_drained)(reef_stream_t, int*);
 } reef_hal_backend;
 
 const reef_hal_backend* reef_hal_hip_backend(void);

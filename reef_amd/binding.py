@@ -168,6 +168,13 @@ class Executor:
             self.h, idx, layers, task_num, cus, warmup, iters, ctypes.byref(us)))
         return us.value
 
+    def time_kernel_dkp_single(self, idx, layers, task_num, cus, evict=None, samples=5):
+        us = ctypes.c_float()
+        _check("time_kernel_dkp_single", lib().reef_executor_time_kernel_dkp_single(
+            self.h, idx, layers, task_num, cus, evict.ptr if evict else None,
+            ctypes.c_size_t(evict.nbytes if evict else 0), samples, ctypes.byref(us)))
+        return us.value
+
     def time_kernel_dkp(self, idx, layers, task_num, warmup=2, iters=10):
         us = ctypes.c_float()
         _check("time_kernel_dkp", lib().reef_executor_time_kernel_dkp(self.h, idx, layers, task_num,

@@ -1,4 +1,5 @@
 // Flat C view of the executors (include/reef_c.h).
+#include <algorithm>
 #include <chrono>
 #include <cstring>
 #include <memory>
@@ -161,6 +162,35 @@ int reef_executor_time_kernel_dkp_confined(reef_executor_t e, int idx, int layer
     float us = 0.f;
     GPU_RETURN_STATUS(reef_hal_event_elapsed_us(a, b, &us));
     *avg_us = us / (float)iters;
+    reef_hal_event_destroy(a);
+    reef_hal_event_destroy(b);
+    return Status::Succ;
+}
+
+int reef_executor_time_kernel_dkp_single(reef_executor_t e, int idx, int layers, int task_num, int cus,
+                                         void* evict, size_t evict_bytes, int samples, float* single_us) {
+    TransExecutor* t = e->trans();
+    if (!t || idx < 0 || idx >= (int)t->num_kernels() || samples <= 0 || layers <= 0 || cus < 0 ||
+        (evict_bytes && !evict))
+        return Status::OutOfRange;
+    GPUStream_t s = t->stream();
+    reef_event_t a, b;
+    GPU_RETURN_STATUS(reef_hal_event_create(&a));
+    GPU_RETURN_STATUS(reef_hal_event_create(&b));
+    std::vector<float> v;
+    for (int i = 0; i < samples; ++i) {
+        if (evict_bytes) GPU_RETURN_STATUS(reef_hal_memset_async(evict, i & 1, evict_bytes, s));
+        else RETURN_STATUS(t->launch_kernel_dkp(idx, layers, task_num, s, cus));
+        GPU_RETURN_STATUS(reef_hal_event_record(a, s));
+        RETURN_STATUS(t->launch_kernel_dkp(idx, layers, task_num, s, cus));
+        GPU_RETURN_STATUS(reef_hal_event_record(b, s));
+        GPU_RETURN_STATUS(reef_hal_event_sync(b));
+        float us = 0.f;
+        GPU_RETURN_STATUS(reef_hal_event_elapsed_us(a, b, &us));
+        v.push_back(us);
+    }
+    std::sort(v.begin(), v.end());
+    *single_us = v[v.size() / 2];
     reef_hal_event_destroy(a);
     reef_hal_event_destroy(b);
     return Status::Succ;

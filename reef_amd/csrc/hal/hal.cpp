@@ -58,6 +58,10 @@ int reef_hal_stream_create(int launch_window, reef_stream_t* out) {
 int reef_hal_stream_destroy(reef_stream_t s) { return be()->stream_destroy(s); }
 int reef_hal_stream_sync(reef_stream_t s) { return be()->stream_sync(s); }
 int reef_hal_stream_query(reef_stream_t s, int* idle) { return be()->stream_query(s, idle); }
+int reef_hal_stream_drained(reef_stream_t s, int* drained) {
+    if (be()->stream_drained) return be()->stream_drained(s, drained);
+    return be()->stream_query(s, drained);
+}
 int reef_hal_device_sync(void) { return be()->device_sync(); }
 int reef_hal_stream_pump(reef_stream_t s) { return be()->stream_pump(s); }
 int reef_hal_launch(reef_function_t fn, const uint32_t grid[3], const uint32_t block[3],

@@ -571,6 +571,12 @@ int h_stream_progress(reef_stream_t st, uint32_t* submitted, uint32_t* done) {
     if (done) *done = *st->done;
     return 0;
 }
+int h_stream_drained(reef_stream_t st, int* drained) {
+    if (!st || st->window <= 0) return h_stream_query(st, drained);
+    std::lock_guard<std::mutex> lock(st->mtx);
+    *drained = st->held.empty() && in_flight(st) == 0 ? 1 : 0;
+    return st->feeder_error.load() ? 1 : 0;
+}
 int h_stream_exit_ticks(reef_stream_t st, uint32_t seq, uint64_t* ticks) {
     if (!ticks) return 1;
     *ticks = 0;
@@ -680,7 +686,7 @@ const reef_hal_backend kHip = {
     h_memset_async, h_host_write32, h_stream_wait_device,
     h_graph_begin, h_graph_end, h_graph_launch, h_graph_destroy,
     h_stream_set_completion, h_stream_progress, h_stream_exit_ticks, h_clock_sync,
-    h_module_kernel_entry, h_host_fill32,
+    h_module_kernel_entry, h_host_fill32, h_stream_drained,
 };
 
 }  // namespace

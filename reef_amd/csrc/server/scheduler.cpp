@@ -637,7 +637,10 @@ void REEFScheduler::dynamic_kernel_padding(std::shared_ptr<Task>& rt_task) {
                 // the real-time stream would sit in front of the real-time kernels), and only now
                 // that a kernel of the task is really about to be padded.
                 if (be_exe.has_sync_storage()) {
-                    if (!executor::GPUStreamEmpty(be_queues[q]->stream)) continue;
+                    // (from the stream's counters: a query of the runtime here would put a
+                    // marker in front of the real-time kernels)
+                    int drained = 0;
+                    if (reef_hal_stream_drained(be_queues[q]->stream, &drained) != 0 || !drained) continue;
                     be_exe.reset_sync_storage_from_host(rt_queue->stream);
                 }
                 cand->sync_dirty = false;

@@ -18,8 +18,18 @@ import os
 from . import binding as B
 
 
-def measure_profile(model_dir, name, iters=10, warmup=2, levels=8):
+# larger than the device's last-level cache (256 MiB): overwriting it leaves no operand cached
+EVICT_BYTES = 768 << 20
+
+
+def measure_profile(model_dir, name, iters=10, warmup=2, levels=8, cold=True):
+    """cold: add to every figure what the kernel loses when its operands come from HBM instead of
+    the caches (one launch between two events after the caches were overwritten, minus the same
+    after a launch of the kernel itself).  Back-to-back repetitions of one kernel -- what the
+    figures are otherwise made of -- find weights and activations cached; a kernel of a model
+    that takes turns with other models does not."""
     exe = B.Executor.from_dir(model_dir, name, B.HYBRID)
+    evict = B.DeviceBuffer(EVICT_BYTES) if cold else None
     num_cus = B.lib().reef_gpuconfig_num_cus()
     model = json.load(open(os.path.join(model_dir, name + ".json")))
     kl = {}
@@ -27,6 +37,11 @@ def measure_profile(model_dir, name, iters=10, warmup=2, levels=8):
         info = exe.kernel_info(i)
         blocks = info["block_num"]
         total = exe.time_kernel_dkp(i, info["min_occupancy"], blocks, warmup, iters)
+        extra = 0.0
+        if cold:
+            extra = max(0.0, exe.time_kernel_dkp_single(i, info["min_occupancy"], blocks, 0, evict, 5)
+                        - exe.time_kernel_dkp_single(i, info["min_occupancy"], blocks, 0, None, 5))
+            total += extra
         max_occ = B.lib().reef_gpuconfig_calculate_occupancy(info["lds"], info["vgprs"], info["sgprs"],
                                                              info["scratch"], 256)
         # latency[j]: one round at occupancy j + 1, with the kernel confined to a few CUs as the
@@ -42,7 +57,7 @@ def measure_profile(model_dir, name, iters=10, warmup=2, levels=8):
                 lat += [lat[-1] if lat else max(1, int(round(total * 1000)))] * (n_levels - len(lat))
                 break
             us = exe.time_kernel_dkp_confined(i, j + 1, (j + 1) * cus, cus, warmup, iters)
-            lat.append(max(1, int(round(us * 1000))))
+            lat.append(max(1, int(round((us + extra) * 1000))))
         e = kl.setdefault(k["name"], {"total_latency": 0, "latency": [], "total_latency_ns": 0, "latency_ns": lat})
         e["total_latency_ns"] = max(e["total_latency_ns"], max(1, int(round(total * 1000))))
         e["latency_ns"] = [max(a, b) for a, b in zip(e["latency_ns"], lat)]
@@ -51,6 +66,8 @@ def measure_profile(model_dir, name, iters=10, warmup=2, levels=8):
     lat_us, _ = exe.time_model(B.RUN_DEFAULT, 3, 10)
     prof = {"model_latency": int(math.ceil(float(lat_us.mean()))), "kernel_latency": kl}
     exe.close()
+    if evict is not None:
+        evict.free()
     return prof
 
 

@@ -472,3 +472,15 @@ def test_tile_choice_outside_the_measured_table():
     # both models answer in microseconds of one launch
     g = tiling.forced("16x32k4", 256, 196, 1024, 2, 1)
     assert 4.0 < tiling.direct_cost("16x32k4", g, True) < 12.0
+
+
+def test_stream_drained_falls_back_to_the_query_of_a_backend_without_counters(fake):
+    """reef_hal_stream_drained is what the padding loop asks between two real-time launches (the
+    reference asks its runtime, scheduler.cpp:655-672 via GPUStreamEmpty); a backend that has no
+    call of its own answers through stream_query."""
+    L = B.lib()
+    s = ctypes.c_void_p()
+    assert L.reef_hal_stream_create(4, ctypes.byref(s)) == 0
+    drained = ctypes.c_int(-1)
+    assert L.reef_hal_stream_drained(s, ctypes.byref(drained)) == 0 and drained.value == 1
+    assert L.reef_hal_stream_destroy(s) == 0
