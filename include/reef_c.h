@@ -66,6 +66,12 @@ int reef_executor_kernel_info(reef_executor_t e, int idx, int out[7]);
  */
 int reef_executor_time_kernel(reef_executor_t e, int idx, int flavour, int warmup, int iters,
                               float* avg_us);
+/* One launch of kernel idx between two events, `samples` times, medians: in the model's own order
+ * (kernels 0..idx-1 before it, the rest after it: operands as cold or warm as a real pass finds
+ * them) and directly after a launch of itself (operands cached).  Both carry the same event
+ * overhead; in_model - after_itself is what the model's order adds to a back-to-back figure. */
+int reef_executor_time_kernel_in_model(reef_executor_t e, int idx, int flavour, int samples,
+                                       float* in_model_us, float* after_itself_us);
 /* time_kernel_dkp: kernel idx through the DKP flavour with `layers` workgroup layers per CU
  * and the first `task_num` tasks only -- the measurement behind <model>.profile.json
  * (latency[j] = one round of (j+1) x num_cus workgroups; the reference's profiler tool

@@ -168,6 +168,13 @@ class Executor:
             self.h, idx, layers, task_num, cus, warmup, iters, ctypes.byref(us)))
         return us.value
 
+    def time_kernel_in_model(self, idx, flavour=RUN_DEFAULT, samples=5):
+        """(in the model's order, directly after itself): one launch between two events, medians."""
+        a, b = ctypes.c_float(), ctypes.c_float()
+        _check("time_kernel_in_model", lib().reef_executor_time_kernel_in_model(
+            self.h, idx, flavour, samples, ctypes.byref(a), ctypes.byref(b)))
+        return a.value, b.value
+
     def time_kernel_dkp_single(self, idx, layers, task_num, cus, evict=None, samples=5):
         us = ctypes.c_float()
         _check("time_kernel_dkp_single", lib().reef_executor_time_kernel_dkp_single(

@@ -140,6 +140,36 @@ int reef_executor_time_kernel(reef_executor_t e, int idx, int flavour, int warmu
     return Status::Succ;
 }
 
+int reef_executor_time_kernel_in_model(reef_executor_t e, int idx, int flavour, int samples,
+                                       float* in_model_us, float* after_itself_us) {
+    const int n = (int)e->exe->num_kernels();
+    if (idx < 0 || idx >= n || samples <= 0 || !in_model_us || !after_itself_us) return Status::OutOfRange;
+    GPUStream_t s = e->exe->stream();
+    reef_event_t a, b;
+    GPU_RETURN_STATUS(reef_hal_event_create(&a));
+    GPU_RETURN_STATUS(reef_hal_event_create(&b));
+    std::vector<float> in_model, warm;
+    for (int i = 0; i < 2 * samples; ++i) {
+        const bool model_order = i < samples;
+        RETURN_STATUS(model_order ? launch_all(e, flavour, 0, idx) : launch_all(e, flavour, idx, idx + 1));
+        GPU_RETURN_STATUS(reef_hal_event_record(a, s));
+        RETURN_STATUS(launch_all(e, flavour, idx, idx + 1));
+        GPU_RETURN_STATUS(reef_hal_event_record(b, s));
+        if (model_order) RETURN_STATUS(launch_all(e, flavour, idx + 1, n));
+        GPU_RETURN_STATUS(reef_hal_stream_sync(s));
+        float us = 0.f;
+        GPU_RETURN_STATUS(reef_hal_event_elapsed_us(a, b, &us));
+        (model_order ? in_model : warm).push_back(us);
+    }
+    std::sort(in_model.begin(), in_model.end());
+    std::sort(warm.begin(), warm.end());
+    *in_model_us = in_model[in_model.size() / 2];
+    *after_itself_us = warm[warm.size() / 2];
+    reef_hal_event_destroy(a);
+    reef_hal_event_destroy(b);
+    return Status::Succ;
+}
+
 int reef_executor_time_kernel_dkp(reef_executor_t e, int idx, int layers, int task_num, int warmup,
                                   int iters, float* avg_us) {
     return reef_executor_time_kernel_dkp_confined(e, idx, layers, task_num, 0, warmup, iters, avg_us);
