@@ -29,6 +29,12 @@
  *     random operands; the oracle reproduces 24 of its 25 convolution kernels
  *     and all of the others named here (tests/test_gpu_reference_kernels.py,
  *     which also says why one convolution kernel and softmax are no witnesses).
+ *   depthwise 3x3 convolution (stride 1 and 2), 11x11 stride 4 / 5x5 / 3x3
+ *   convolutions without bias, unpadded 3x3 stride 2 max-pool, dense+add+relu:
+ *     the generated kernels of resource/mobilenet/mobilenet.cu and
+ *     resource/alexnet/alexnet.cu, the same way (tests/golden/make_chain_shapes.py
+ *     finds each kernel's shape by it; tests/test_gpu_legacy_import.py runs both
+ *     networks from input to classifier beside the reference's kernels).
  *   mocked add/multiply: the reference's closed form (3+3)*3 == 18, also on the
  *     reference's own mocked kernels.
  *   The reference's ResNet-18 ten-float golden vector needs a weight blob that

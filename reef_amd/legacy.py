@@ -14,7 +14,9 @@ file of the reference loads unchanged), every call replaced by the `reef_*` kern
 the same thing.  What a kernel name computes comes from a per-model table
 (`legacy_tables/<model>.json`: name -> op, shape, stride, padding, epilogue); the argument roles
 are those of the kernel families (convolution: in, W, out, then the epilogue operands in the
-order the family name lists them; elementwise add and flatten: out first; pooling: in, out).
+order the family name lists them; depthwise convolution: in, W, out, bias; elementwise add and
+flatten: out first; pooling: in, out; dense: x, W, out, bias).  Tables are packaged for the
+reference's `resnet152`, `mobilenet` and `alexnet` directories.
 While it rewrites, the importer follows the tensor shapes through the graph and refuses a table
 that does not fit the graph.
 """
@@ -108,6 +110,9 @@ def import_model(ref_json_path, table=None, name=None, input_shape=None):
                      and size(rest[2]) == cout, k, "residual / scale / shift operands")
                 given["scale"], given["shift"] = Tensor(rest[1], (cout,)), Tensor(rest[2], (cout,))
                 kw.update(residual=Tensor(rest[0], (cout, Ho, Wo)), affine=True, act=MB.ACT_RELU)
+            elif ep == "relu":
+                need(not rest, k, "operands after the output")
+                kw.update(act=MB.ACT_RELU)
             else:
                 need(ep == "none" and not rest, k, "unknown epilogue " + ep)
             # a residual read from the buffer the result goes to would not survive a restart
@@ -115,6 +120,16 @@ def import_model(ref_json_path, table=None, name=None, input_shape=None):
             g.conv2d(Tensor(a[0], shape[a[0]]), cout, kk, s, p, out=tensor(a[2], (cout, Ho, Wo), k),
                      given=given, **kw)
             shape[a[2]] = (cout, Ho, Wo)
+        elif op == "dwconv2d":                                  # (in, W, out, bias)
+            need(len(a) == 4 and a[0] in shape and shape[a[0]] == (e["c"], e["h"], e["w"]), k, "shape")
+            C, kk = e["c"], e["k"]
+            need(size(a[1]) == C * kk * kk and size(a[3]) == C, k, "weight / bias operand")
+            Ho = (e["h"] + 2 * e["pad"] - kk) // e["stride"] + 1
+            Wo = (e["w"] + 2 * e["pad"] - kk) // e["stride"] + 1
+            g.dwconv2d(Tensor(a[0], shape[a[0]]), kk, e["stride"], e["pad"], bias=True, act=e["act"],
+                       out=tensor(a[2], (C, Ho, Wo), k),
+                       given={"w": Tensor(a[1], (C, 1, kk, kk)), "bias": Tensor(a[3], (C,))})
+            shape[a[2]] = (C, Ho, Wo)
         elif op == "eltwise":                                   # (out, in, per-channel shift)
             need(len(a) == 3 and a[1] in shape, k, "operands")
             C, H, W = shape[a[1]]
@@ -141,7 +156,8 @@ def import_model(ref_json_path, table=None, name=None, input_shape=None):
             shape[a[0]] = (n, 1, 1)
         elif op == "dense":                                     # (x, W, out, bias)
             need(shape[a[0]][0] == e["in"] and size(a[1]) == e["in"] * e["out"], k, "shape")
-            g.dense(Tensor(a[0], (e["in"],)), e["out"], bias=bool(e.get("bias")), out=tensor(a[2], (1, e["out"]), k),
+            g.dense(Tensor(a[0], (e["in"],)), e["out"], bias=bool(e.get("bias")), act=e.get("act", 0),
+                    out=tensor(a[2], (1, e["out"]), k),
                     w=Tensor(a[1], (e["out"], e["in"])), bias_t=Tensor(a[3], (e["out"],)) if e.get("bias") else None)
             shape[a[2]] = (e["out"], 1, 1)
         elif op == "softmax":                                   # (in, out)
@@ -171,6 +187,14 @@ def import_model_dir(ref_dir, model_name, out_dir, table=None, measured_profile=
     return g
 
 
+def param_storages(ref):
+    """{storage name: index} of the parameters of a reference graph: the storages its `args` list
+    names (graph inputs and parameters, generate_final_schedule.py:109-144) other than the
+    input.  TVM calls them p0..pN or by their relay names (conv_1_weight)."""
+    return {ref["storage"][i]["name"]: i for i in ref.get("args", [])
+            if i != 0 and ref["storage"][i]["name"] not in ("data", "null", "output", "temp_arg")}
+
+
 def seeded_params(ref_json_path, table=None, seed=0x5EEF):
     """Seeded parameters for a reference graph that ships without a `.param` file (the checkout's
     resource/resnet152 does): He-normal weights, small biases / shifts, scales around 1 -- the
@@ -193,12 +217,15 @@ def seeded_params(ref_json_path, table=None, seed=0x5EEF):
             if e["epilogue"] == "residual_scale_shift_relu":
                 std[a[4]] = 0.1
                 one_plus.add(a[4])
+        elif e["op"] == "dwconv2d":
+            std[a[1]] = math.sqrt(2.0 / (e["k"] * e["k"]))
         elif e["op"] == "dense":
             std[a[1]] = math.sqrt(2.0 / e["in"])
     out = []
+    params = set(param_storages(ref).values())
     for i, s in enumerate(ref["storage"]):
         name = s["name"]
-        if not (name.startswith("p") and name[1:].isdigit()):
+        if i not in params:
             continue
         arr = rng.normal_f32(model_name + "/" + name, s["size"], std.get(i, 0.01), seed)
         if i in one_plus:

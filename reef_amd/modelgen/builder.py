@@ -258,18 +258,21 @@ class GraphBuilder:
                        4 * ((t["split_k"] + 1) * M * N), 2.0)
         return out if out2 is None else (out, out2)
 
-    def dwconv2d(self, x, k, stride=1, pad=0, bias=True, act=ACT_RELU6):
+    def dwconv2d(self, x, k, stride=1, pad=0, bias=True, act=ACT_RELU6, out=None, given=None):
+        """given: {"w", "bias"} -> existing storages instead of new parameters; out: existing
+        storage for the result (an imported graph brings its own)."""
+        given = given or {}
         C, H, W = x.shape
         Ho = (H + 2 * pad - k) // stride + 1
         Wo = (W + 2 * pad - k) // stride + 1
         std = self.weight_std if self.weight_std is not None else math.sqrt(2.0 / (k * k))
-        w = self.param((C, 1, k, k), std)
+        w = given.get("w") or self.param((C, 1, k, k), std)
         args = [x.idx, w.idx, None]
         flags = 0
         if bias:
             flags |= 1
-            b = self.param((C,), 0.01)
-        out = self.temp((C, Ho, Wo))
+            b = given.get("bias") or self.param((C,), 0.01)
+        out = Tensor(out.idx, (C, Ho, Wo)) if out is not None else self.temp((C, Ho, Wo))
         args[2] = out.idx
         if bias:
             args.append(b.idx)

@@ -1,0 +1,165 @@
+"""Writes <model>_kernel_shapes.json for the reference's chain-shaped model directories
+(resource/mobilenet: MobileNet v1 with depthwise convolutions; resource/alexnet: 11x11 / 5x5 / 3x3
+convolutions without bias, plain max-pools, three dense layers): for every kernel name what it
+computes -- op, shape, filter, stride, padding, epilogue.
+
+As for resnet152 (make_resnet152_shapes.py) the shapes are baked into the generated source and
+the graph JSON only holds shared, maximal buffer sizes, so every entry has a witness: the graph is
+walked from the 3 x 224 x 224 input, each distinct kernel of oracle/_ref/<model>.raw.co (the
+reference's own <model>.cu compiled for gfx950, `make -C oracle ref`) is run once on random
+operands on the GPU, and of the hypotheses that are consistent with its operand sizes and with
+the number of elements it writes (groups 1 or depthwise, filter 1..11, stride 1/2/4, every padding
+up to half the filter) exactly one must make the CPU oracle reproduce its output.  Dense kernels
+are run on small non-negative integers and softmax has no witness, for the reason given in the
+module docstring of tests/test_gpu_reference_kernels.py.
+
+Needs a GPU:  python tests/golden/make_chain_shapes.py mobilenet|alexnet
+The result is committed as tests/golden/<model>_kernel_shapes.json (fixture) and as
+reef_amd/legacy_tables/<model>.json (the importer's table for that model directory)."""
+import json
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+
+from oracle import oracle as O                                   # noqa: E402
+from reef_amd import binding as B                                # noqa: E402
+from tests import test_gpu_reference_kernels as T                # noqa: E402
+
+
+def conv_hypotheses(cin, H, w_size, cout_known, n_written):
+    for groups in (1, cin):
+        for kk in (1, 3, 5, 7, 11):
+            per = (cin // groups) * kk * kk
+            if w_size % per:
+                continue
+            cout = w_size // per
+            if (cout_known and cout != cout_known) or (groups > 1 and cout != cin):
+                continue
+            for s in (1, 2, 4):
+                for p in range(kk // 2 + 1):
+                    Ho = (H + 2 * p - kk) // s + 1
+                    if Ho >= 1 and cout * Ho * Ho == n_written:
+                        yield cout, groups, kk, s, p
+
+
+def derive(name):
+    path = os.path.join(HERE, name + ".json")
+    model = json.load(open(path))
+    roles = json.load(open(os.path.join(HERE, name + "_kernel_roles.json")))
+    exe = B.Executor(B.BASE)
+    exe.load(path, os.path.join(ROOT, "oracle", "_ref", name + ".raw.co"))
+    rng = np.random.default_rng(224)
+    size = lambda i: model["storage"][i]["size"]
+    side = int(round((size(0) // 3) ** 0.5))
+    shape = {0: (3, side, side)}
+    table = {}
+    for kidx, k in enumerate(model["kernels"]):
+        kname, a = k["name"], k["args"]
+        new = kname not in table
+        if kname.startswith("fused_nn_conv2d"):
+            cin, H, W = shape[a[0]]
+            if new:
+                ops, out, n = T.run_reference_kernel(exe, model, roles, kidx, rng)
+                x, w, bias = ops["placeholder"], ops["placeholder1"], ops.get("placeholder2")
+                relu = "nn_relu" in kname
+                hits = []
+                for cout, groups, kk, s, p in conv_hypotheses(cin, H, w.size, bias.size if bias is not None else 0, n):
+                    want = O.conv2d(x[:cin * H * W].reshape(cin, H, W), w.reshape(cout, cin // groups, kk, kk),
+                                    bias=bias, stride=(s, s), pad=(p, p), groups=groups, act=1 if relu else 0,
+                                    acc64=True)
+                    if T.close(out[:n], want):
+                        hits.append((cout, groups, kk, s, p))
+                assert len(hits) == 1, (kname, hits)
+                cout, groups, kk, s, p = hits[0]
+                if groups > 1:
+                    assert bias is not None and relu
+                    table[kname] = {"op": "dwconv2d", "c": cin, "h": H, "w": W, "k": kk, "stride": s, "pad": p,
+                                    "bias": True, "act": 1, "witness": True}
+                else:
+                    ep = ("bias_relu" if relu else "bias") if bias is not None else ("relu" if relu else "none")
+                    assert ep != "bias", kname
+                    table[kname] = {"op": "conv2d", "cin": cin, "h": H, "w": W, "cout": cout, "k": kk, "stride": s,
+                                    "pad": p, "epilogue": ep, "witness": True}
+                print("%-44s %s" % (kname, table[kname]), flush=True)
+            e = table[kname]
+            C = e["c"] if e["op"] == "dwconv2d" else e["cout"]
+            assert (e["h"], e["w"]) == (H, W) and (e.get("cin", e.get("c")) == cin), kname
+            Ho = (H + 2 * e["pad"] - e["k"]) // e["stride"] + 1
+            shape[a[2]] = (C, Ho, Ho)
+        elif kname.startswith("fused_nn_max_pool2d"):               # (in, out)
+            C, H, W = shape[a[0]]
+            if new:
+                ops, out, n = T.run_reference_kernel(exe, model, roles, kidx, rng)
+                x = ops["placeholder"][:C * H * W].reshape(C, H, W)
+                hits = []
+                for kk, s, p in ((3, 2, 0), (3, 2, 1), (2, 2, 0), (3, 1, 1)):
+                    Ho = (H + 2 * p - kk) // s + 1
+                    if C * Ho * Ho == n and T.close(out[:n], O.pool2d(x, (kk, kk), (s, s), (p, p), 0)):
+                        hits.append((kk, s, p))
+                assert len(hits) == 1, (kname, hits)
+                kk, s, p = hits[0]
+                table[kname] = {"op": "pool2d", "c": C, "h": H, "w": W, "k": kk, "stride": s, "pad": p,
+                                "mode": "max", "bias": False, "act": 0, "witness": True}
+                print("%-44s %s" % (kname, table[kname]), flush=True)
+            e = table[kname]
+            Ho = (H + 2 * e["pad"] - e["k"]) // e["stride"] + 1
+            shape[a[1]] = (C, Ho, Ho)
+        elif kname.startswith("fused_nn_global_avg_pool2d"):        # (in, out)
+            C, H, W = shape[a[0]]
+            if new:
+                ops, out, n = T.run_reference_kernel(exe, model, roles, kidx, rng)
+                assert n == C and T.close(out[:n], O.global_avgpool(ops["placeholder"][:C * H * W].reshape(C, H * W)))
+                table[kname] = {"op": "global_avgpool", "c": C, "hw": H * W, "witness": True}
+            shape[a[1]] = (C, 1, 1)
+        elif kname.startswith("fused_nn_batch_flatten"):            # (out, in)
+            C, H, W = shape[a[1]]
+            if new:
+                ops, out, n = T.run_reference_kernel(exe, model, roles, kidx, rng)
+                assert n == C * H * W and np.array_equal(out[:n], ops["placeholder"][:n])
+                table[kname] = {"op": "copy", "n": n, "witness": True}
+            shape[a[0]] = (C * H * W, 1, 1)
+        elif kname.startswith("fused_nn_dense_add"):                # (x, W, out, bias)
+            in_f, out_f = shape[a[0]][0], size(a[3])
+            assert size(a[1]) == in_f * out_f
+            if new:
+                relu = "nn_relu" in kname
+                ints = {}
+                for pn, s_idx in zip(roles[kname], a):
+                    if pn.startswith("placeholder"):
+                        ints[pn] = T._set(exe, model, s_idx, rng.integers(0, 4, size(s_idx)).astype(np.float32))
+                exe.execute_kernel(kidx)
+                got = exe.get_data(a[2], size(a[2]))[:out_f]
+                want = O.dense(ints["placeholder"][:in_f].reshape(1, in_f), ints["placeholder1"].reshape(out_f, in_f),
+                               bias=ints["placeholder2"], act=1 if relu else 0, acc64=True)
+                np.testing.assert_array_equal(got, want.ravel(), err_msg=kname)
+                table[kname] = {"op": "dense", "in": in_f, "out": out_f, "bias": True, "act": 1 if relu else 0,
+                                "witness": True}
+            shape[a[2]] = (out_f, 1, 1)
+        elif kname.startswith("fused_nn_softmax"):                  # (in, out)
+            table.setdefault(kname, {"op": "softmax", "rows": 1, "cols": shape[a[0]][0], "witness": False})
+            shape[a[1]] = shape[a[0]]
+        else:
+            raise AssertionError("unexpected kernel " + kname)
+    assert set(table) == {k["name"] for k in model["kernels"]}
+    exe.close()
+    return table
+
+
+def main():
+    name = sys.argv[1]
+    table = derive(name)
+    for out in (os.path.join(HERE, name + "_kernel_shapes.json"),
+                os.path.join(ROOT, "reef_amd", "legacy_tables", name + ".json"),
+                os.path.join(ROOT, "gpurun_out", name + "_kernel_shapes.json")):
+        os.makedirs(os.path.dirname(out), exist_ok=True)
+        json.dump(table, open(out, "w"), indent=0, sort_keys=True)
+    print(len(table), "kernels; without a witness:", [n for n, e in table.items() if not e["witness"]])
+
+
+if __name__ == "__main__":
+    main()

@@ -1,4 +1,5 @@
-"""The imported reference graph on this build's kernels against the reference's OWN kernels.
+"""The imported reference graphs on this build's kernels against the reference's OWN kernels
+(resource/resnet152 at 64 x 64 below; resource/mobilenet and resource/alexnet at the end).
 
 Two executors hold the reference's resource/resnet152 graph (tests/golden/resnet152.json) with the
 same seeded parameters and the same input: one launches the reference's generated kernels
@@ -52,7 +53,7 @@ def test_imported_resnet152_tracks_the_reference_kernels_call_by_call(tmp_path):
 
     theirs = B.Executor(B.BASE)
     theirs.load(REF_JSON, REF_CO)
-    index = {s["name"]: i for i, s in enumerate(ref["storage"]) if s["name"].startswith("p")}
+    index = legacy.param_storages(ref)
     for key, arr in params:
         _set_idx(theirs, index[key], arr)
     _set_idx(theirs, 0, x.ravel())
@@ -69,7 +70,7 @@ def test_imported_resnet152_tracks_the_reference_kernels_call_by_call(tmp_path):
         if not free_running:
             # identical operands for this call: the reference executor takes over what this build holds
             for a in set(k["args"]):
-                if not ref["storage"][a]["name"].startswith("p"):
+                if a not in index.values():
                     _set_idx(theirs, a, ours.get_data(a, ref["storage"][a]["size"]))
         theirs.execute_kernel(i)
         ours.execute_kernel(i)
@@ -89,5 +90,73 @@ def test_imported_resnet152_tracks_the_reference_kernels_call_by_call(tmp_path):
         compared += 1
     print("compared %d of %d calls, %d without a witness, worst deviation %.2e" % (compared, len(ref["kernels"]), resynced, worst))
     assert compared + resynced == 207 and resynced == 3
+    theirs.close()
+    ours.close()
+
+
+@pytest.mark.parametrize("name,calls,no_witness", [
+    ("mobilenet", 31, ("fused_nn_dense_add_kernel0", "fused_nn_softmax_kernel0")),
+    ("alexnet", 13, ("fused_nn_dense_add_nn_relu_1_kernel0", "fused_nn_dense_add_nn_relu_kernel0",
+                     "fused_nn_dense_add_kernel0", "fused_nn_softmax_kernel0")),
+])
+def test_imported_chain_models_track_the_reference_kernels_call_by_call(name, calls, no_witness, tmp_path):
+    """resource/mobilenet (MobileNet v1: a 3x3 stem, 13 depthwise + 13 pointwise convolutions) and
+    resource/alexnet (11x11 stride 4, 5x5, 3x3 convolutions without bias, plain max-pools, three
+    dense layers) at 224 x 224, the reference's kernels from oracle/_ref/<model>.raw.co.  Both
+    executors run free from the input to the classifier; the dense and softmax kernels of the
+    reference are no witnesses (int shuffle, see tests/test_gpu_reference_kernels.py), there the
+    reference executor takes over this build's result."""
+    co = os.path.join(os.path.dirname(HERE), "oracle", "_ref", name + ".raw.co")
+    _need(co)
+    ref_json = os.path.join(HERE, "golden", name + ".json")
+    ref = json.load(open(ref_json))
+    roles = json.load(open(os.path.join(HERE, "golden", name + "_kernel_roles.json")))
+    g = legacy.import_model(ref_json)
+    d = str(tmp_path)
+    g.write(d)
+    params = legacy.seeded_params(ref_json)
+    MB.write_params(os.path.join(d, name + ".param"), params)
+    x = nets.image_input("legacy", (3, 224, 224))
+
+    theirs = B.Executor(B.BASE)
+    theirs.load(ref_json, co)
+    index = legacy.param_storages(ref)
+    for key, arr in params:
+        _set_idx(theirs, index[key], arr)
+    _set_idx(theirs, 0, x.ravel())
+    ours = B.Executor.from_dir(d, name, B.BASE)
+    ours.set_input_checked("data", x)
+
+    compared = resynced = 0
+    worst = 0.0
+    for i, k in enumerate(ref["kernels"]):
+        names = roles[k["name"]]
+        out_idx = k["args"][[j for j, n in enumerate(names) if not n.startswith("placeholder")][0]]
+        size = ref["storage"][out_idx]["size"]
+        if resynced:
+            for a in set(k["args"]):
+                if a not in index.values():
+                    _set_idx(theirs, a, ours.get_data(a, ref["storage"][a]["size"]))
+        theirs.execute_kernel(i)
+        ours.execute_kernel(i)
+        mine = ours.get_data(out_idx, size)
+        assert np.isfinite(mine).all(), (i, k["name"])
+        if k["name"] in no_witness:
+            resynced += 1
+            continue
+        assert not resynced, "every call before the classifier runs free"
+        want = theirs.get_data(out_idx, size)
+        scale = max(float(np.abs(want).max()), 1e-20)
+        err = float(np.abs(mine - want).max()) / scale
+        worst = max(worst, err)
+        assert err <= TOL, (i, k["name"], err)
+        compared += 1
+    print("%s: %d calls free-running against the reference's kernels, worst deviation %.2e; %d without a witness"
+          % (name, compared, worst, resynced))
+    assert compared + resynced == calls and resynced == len(no_witness)
+    # the classifier: probabilities
+    out_idx = [i for i, s in enumerate(ref["storage"]) if s["name"] == "output"][0]
+    probs = ours.get_data(out_idx, ref["storage"][out_idx]["size"])[:1000]
+    assert abs(float(probs.sum()) - 1.0) < 1e-4
     theirs.close()
     ours.close()

@@ -1,7 +1,9 @@
 """The importer for the reference's own model directories (reef_amd/legacy.py) on the reference's
-resource/resnet152 graph (tests/golden/resnet152.json, a data fixture): same storages, same call
+resource/resnet152, resource/mobilenet and resource/alexnet graphs (tests/golden/<model>.json,
+data fixtures): same storages, same call
 order, and the imported graph computes what the reference's kernels compute according to the
-table of shapes that was derived by running those kernels (tests/golden/make_resnet152_shapes.py).
+table of shapes that was derived by running those kernels (tests/golden/make_resnet152_shapes.py,
+make_chain_shapes.py).
 
 The CPU check interprets the reference graph DIRECTLY from the table with the oracle's ops and
 compares that with the imported model run through the executor (fake backend) -- two code paths
@@ -45,6 +47,8 @@ def interpret_reference_graph(ref, table, params, x, upto=None):
             ep = e["epilogue"]
             if ep == "none":
                 y = O.conv2d(xs, ws, act=0, **kw)
+            elif ep == "relu":
+                y = O.conv2d(xs, ws, act=1, **kw)
             elif ep == "residual":
                 y = O.conv2d(xs, ws, residual=full(a[3]), act=0, **kw)
             elif ep == "bias_relu":
@@ -54,13 +58,19 @@ def interpret_reference_graph(ref, table, params, x, upto=None):
             else:
                 y = O.conv2d(xs, ws, residual=full(a[3]), scale=st[a[4]], shift=st[a[5]], act=1, **kw)
             st[a[2]][:y.size] = y.ravel()
+        elif e["op"] == "dwconv2d":
+            C, H, W, kk, sd, p = e["c"], e["h"], e["w"], e["k"], e["stride"], e["pad"]
+            y = O.conv2d(st[a[0]][:C * H * W].reshape(C, H, W), st[a[1]].reshape(C, 1, kk, kk), bias=st[a[3]],
+                         stride=(sd, sd), pad=(p, p), groups=C, act=e["act"])
+            st[a[2]][:y.size] = y.ravel()
         elif e["op"] == "eltwise":
             C, inner = e["c"], e["inner"]
             y = O.eltwise(st[a[1]][:C * inner].reshape(C, inner), shift=st[a[2]], act=e["act"])
             st[a[0]][:y.size] = y.ravel()
         elif e["op"] == "pool2d":
             C, H, W = e["c"], e["h"], e["w"]
-            y = O.pool2d(st[a[0]][:C * H * W].reshape(C, H, W), (3, 3), (2, 2), (1, 1), 0, bias=st[a[2]], act=1)
+            y = O.pool2d(st[a[0]][:C * H * W].reshape(C, H, W), (e["k"], e["k"]), (e["stride"], e["stride"]),
+                         (e["pad"], e["pad"]), 0, bias=st[a[2]] if e.get("bias") else None, act=e.get("act", 0))
             st[a[1]][:y.size] = y.ravel()
         elif e["op"] == "global_avgpool":
             C, hw = e["c"], e["hw"]
@@ -68,7 +78,8 @@ def interpret_reference_graph(ref, table, params, x, upto=None):
         elif e["op"] == "copy":
             st[a[0]][:e["n"]] = st[a[1]][:e["n"]]
         elif e["op"] == "dense":
-            y = O.dense(st[a[0]][:e["in"]].reshape(1, e["in"]), st[a[1]].reshape(e["out"], e["in"]), bias=st[a[3]])
+            y = O.dense(st[a[0]][:e["in"]].reshape(1, e["in"]), st[a[1]].reshape(e["out"], e["in"]), bias=st[a[3]],
+                        act=e.get("act", 0))
             st[a[2]][:e["out"]] = y.ravel()
         elif e["op"] == "softmax":
             st[a[1]][:e["cols"]] = O.softmax(st[a[0]][:e["cols"]].reshape(1, e["cols"])).ravel()
@@ -145,3 +156,63 @@ def test_import_refuses_a_table_that_does_not_fit_the_graph():
         legacy.import_model(REF_JSON, table=bad)
     # the packaged table is the fixture
     assert legacy.load_table("resnet152") == table
+
+
+# ---- the chain-shaped directories: MobileNet v1 (depthwise convolutions) and AlexNet ----------
+def golden(name, what=""):
+    return os.path.join(HERE, "golden", name + what + ".json")
+
+
+@pytest.mark.parametrize("name,calls,ops", [
+    ("mobilenet", 31, {"reef_dwconv2d": 13, "reef_global_avgpool": 1, "reef_copy": 1, "reef_dense": 1, "reef_softmax": 1}),
+    ("alexnet", 13, {"reef_pool2d": 3, "reef_copy": 1, "reef_dense": 3, "reef_softmax": 1}),
+])
+def test_chain_models_import_with_storages_order_and_keys(name, calls, ops, tmp_path):
+    ref = json.load(open(golden(name)))
+    g = legacy.import_model(golden(name))
+    g.write(str(tmp_path))
+    out = json.load(open(os.path.join(str(tmp_path), name + ".json")))
+    n = len(ref["storage"])
+    assert out["storage"][:n] == ref["storage"] and out["args"] == ref["args"]
+    assert all(s["name"] in ("temp_arg", "reef_sync") for s in out["storage"][n:])
+    assert len(out["kernels"]) == len(ref["kernels"]) == calls
+    count = {}
+    for ko, kr in zip(out["kernels"], ref["kernels"]):
+        sym = ko["name"].split("#")[0]
+        count[sym] = count.get(sym, 0) + 1
+        assert sorted(set(x for x in ko["args"] if x < n)) == sorted(set(kr["args"])), (ko, kr)
+    for sym, c in ops.items():
+        assert count.get(sym) == c, (sym, count)
+    assert sum(c for sym, c in count.items() if sym.startswith("reef_conv2d")) == calls - sum(ops.values())
+    assert legacy.load_table(name) == json.load(open(golden(name, "_kernel_shapes")))
+    # every entry but the softmax was reproduced by the oracle from the reference's own kernel
+    assert [k for k, e in legacy.load_table(name).items() if not e["witness"]] == ["fused_nn_softmax_kernel0"]
+
+
+def test_imported_mobilenet_equals_the_table_interpretation_through_the_executor(tmp_path):
+    name = "mobilenet"
+    d = str(tmp_path)
+    g = legacy.import_model(golden(name))
+    g.write(d)
+    params = legacy.seeded_params(golden(name))
+    MB.write_params(os.path.join(d, name + ".param"), params)
+    ref = json.load(open(golden(name)))
+    x = nets.image_input("legacy", (3, 224, 224))
+    want = interpret_reference_graph(ref, legacy.load_table(name), dict(params), x)
+    fake = FakeHal().install()
+    exe = None
+    try:
+        exe = B.Executor.from_dir(d, name, B.HYBRID)
+        exe.set_input_checked("data", x)
+        exe.execute()
+        for i, s in enumerate(ref["storage"]):
+            if s["name"] in ("null", "output"):
+                have = exe.get_data(i, s["size"])
+                scale = max(np.abs(want[i]).max(), 1e-6)
+                assert np.abs(have - want[i]).max() <= 1e-5 * scale, (i, s)
+        out_idx = [i for i, s in enumerate(ref["storage"]) if s["name"] == "output"][0]
+        assert abs(float(exe.get_data(out_idx, ref["storage"][out_idx]["size"])[:1000].sum()) - 1.0) < 1e-4
+    finally:
+        if exe is not None:
+            exe.close()
+        fake.remove()
