@@ -287,16 +287,27 @@ def corun(models, rt_name, be_name, n_be, mode, requests, warmup, wait_sync=True
                                  "every best-effort stream has no kernel left on the device"
                                  if wait_sync else "host span without waiting for the device to drain"}
     dev = s.preempt_device_samples()
-    dev = dev[-(requests):] if len(dev) > requests else dev
+    late = s.preempt_device_late()
+    late = late[:len(dev)] if len(late) >= len(dev) else np.zeros(len(dev), bool)
+    if len(dev) > requests:
+        dev, late = dev[-requests:], late[-requests:]
+    on_dev = dev[~late]
     out["preempt_us"]["device"] = {
         "n": int(len(dev)), "mean": round(float(dev.mean()), 2) if len(dev) else None,
         "p50": round(float(np.percentile(dev, 50)), 2) if len(dev) else None,
         "p99": round(float(np.percentile(dev, 99)), 2) if len(dev) else None,
         "max": round(float(dev.max()), 2) if len(dev) else None,
         "clock_sync_err_us": round(s.clock_sync_error_us(), 2),
+        "late_launch_samples": int(late.sum()),
+        "without_late_launches": {"n": int(len(on_dev)),
+                                  "mean": round(float(on_dev.mean()), 2) if len(on_dev) else None,
+                                  "p99": round(float(np.percentile(on_dev, 99)), 2) if len(on_dev) else None,
+                                  "max": round(float(on_dev.max()), 2) if len(on_dev) else None},
         "what": "flag store (host clock) -> the last best-effort workgroup that was on the device has left "
-                "(device wall clock written by that workgroup, mapped to the host clock); launches a stream "
-                "was handing to the runtime at that moment are included"}
+                "(device wall clock written by that workgroup, mapped to the host clock).  late_launch_samples: "
+                "preemptions during which a stream was handing a launch to the runtime; that launch reaches the "
+                "device later, finds the flag and leaves, and the sample runs until its exit (without_late_launches "
+                "leaves those samples out)"}
     out["preempt_phase_ns"] = s.preempt_phases()
     out["padded_kernels"] = int(s.padded_kernels())
     out["kernel_select_ns"] = int(s.avg_kernel_sel_latency())

@@ -147,6 +147,10 @@ size_t reef_scheduler_preempt_samples(reef_scheduler_t s, int64_t* out, size_t c
  * mapped to the host clock by a clock exchange whose half-length clock_sync_error_ns returns
  * (-1: this backend has no device clock).  Only with wait_sync on. */
 size_t reef_scheduler_preempt_device_samples(reef_scheduler_t s, int64_t* out_ns, size_t cap);
+/* For the same samples, in the same order: 1 where a best-effort stream was handing a launch to the
+ * runtime when the flag was stored.  That launch reaches the device later (the runtime call may
+ * block), finds the flag and leaves; the sample runs until its exit. */
+size_t reef_scheduler_preempt_device_late(reef_scheduler_t s, uint8_t* out, size_t cap);
 int64_t reef_scheduler_clock_sync_error_ns(reef_scheduler_t s);
 /* Average ns per reset-based preemption in: flag store, host-queue drop + rollback, device drain. */
 void reef_scheduler_preempt_phases(reef_scheduler_t s, int64_t out_ns[3]);

@@ -214,6 +214,7 @@ class Scheduler:
             getattr(L, fn).restype = ctypes.c_uint64
         L.reef_scheduler_preempt_samples.restype = ctypes.c_size_t
         L.reef_scheduler_preempt_device_samples.restype = ctypes.c_size_t
+        L.reef_scheduler_preempt_device_late.restype = ctypes.c_size_t
         L.reef_scheduler_clock_sync_error_ns.restype = ctypes.c_int64
         _check("scheduler_create", L.reef_scheduler_create(mode, ctypes.byref(self.h)))
 
@@ -343,6 +344,12 @@ class Scheduler:
         buf = (ctypes.c_int64 * cap)()
         n = lib().reef_scheduler_preempt_device_samples(self.h, buf, ctypes.c_size_t(cap))
         return np.array(buf[:n], np.float64) / 1e3
+
+    def preempt_device_late(self, cap=100000):
+        """Per device sample: True where a launch reached the device after the flag was raised."""
+        buf = (ctypes.c_uint8 * cap)()
+        n = lib().reef_scheduler_preempt_device_late(self.h, buf, ctypes.c_size_t(cap))
+        return np.array(buf[:n], np.uint8).astype(bool)
 
     def clock_sync_error_us(self):
         return lib().reef_scheduler_clock_sync_error_ns(self.h) / 1e3

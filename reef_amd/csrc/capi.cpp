@@ -339,6 +339,9 @@ int reef_scheduler_padded_by_op(reef_scheduler_t h, uint64_t* out, int n) {
 size_t reef_scheduler_preempt_device_samples(reef_scheduler_t h, int64_t* out_ns, size_t cap) {
     return h->s->preempt_device_samples(out_ns, cap);
 }
+size_t reef_scheduler_preempt_device_late(reef_scheduler_t h, uint8_t* out, size_t cap) {
+    return h->s->preempt_device_late(out, cap);
+}
 int64_t reef_scheduler_clock_sync_error_ns(reef_scheduler_t h) { return h->s->clock_sync_error_ns(); }
 size_t reef_scheduler_preempt_samples(reef_scheduler_t h, int64_t* out, size_t cap) {
     return h->s->preempt_latency_samples(out, cap);

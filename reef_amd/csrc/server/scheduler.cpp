@@ -350,10 +350,12 @@ void REEFScheduler::preempt_reset() {
     auto ns = [](Steady::time_point a, Steady::time_point b) {
         return (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(b - a).count();
     };
-    // the device's own account: when did the last workgroup of each stream's newest launch leave
+    // the device's own account: when did the last workgroup of each stream's newest launch leave.
+    // Only the raw device clock is kept here; it is mapped to the host clock once the real-time
+    // task is done (resolve_late_samples), with a clock exchange that is at most one task old --
+    // the two clocks drift by tens of microseconds per second.
     if (clk_valid && wait_sync) {
         const int64_t t0_ns = std::chrono::duration_cast<std::chrono::nanoseconds>(t1.time_since_epoch()).count();
-        int64_t worst = -1;
         bool any = false, late = false;
         std::lock_guard<std::mutex> lock(stats_mtx);
         const size_t slot = preempt_device_ns.size();
@@ -362,14 +364,14 @@ void REEFScheduler::preempt_reset() {
             any = true;
             uint64_t ticks = 0;
             reef_hal_stream_exit_ticks(be_queues[i]->stream, target[i], &ticks);
-            if (ticks == 0) {   // still inside the runtime call or on the device: completed later
-                late_samples.push_back(LateSample{slot, i, target[i], t0_ns});
-                late = true;
-                continue;
-            }
-            worst = std::max(worst, std::max<int64_t>(device_ticks_to_host_ns(ticks) - t0_ns, 0));
+            // ticks == 0: still inside the runtime call or on the device, read later
+            late_samples.push_back(LateSample{slot, i, target[i], t0_ns, ticks});
+            late = late || ticks == 0;
         }
-        if (any) preempt_device_ns.push_back(late ? -(worst + 2) : worst);   // <= -1: open, holds the worst so far
+        if (any) {
+            preempt_device_ns.push_back(-1);   // open until the task is done
+            preempt_device_late_flag.push_back(late ? 1 : 0);
+        }
     }
     std::lock_guard<std::mutex> lock(stats_mtx);
     preempt_phase_ns[0] += ns(t0, t1);
@@ -397,22 +399,31 @@ int64_t REEFScheduler::device_ticks_to_host_ns(uint64_t ticks) const {
     return clk_host_ns + dt * 1000 / clk_ticks_per_us;
 }
 
-// Samples that waited for a launch which reached the device after the flag was raised: that
-// launch has long left by the time a real-time task is done.
+// Closes the samples of the preemptions since the last call: exit clocks that were not there yet
+// (a launch that reached the device after the flag was raised has long left by the time a
+// real-time task is done) are read now, and every exit clock is mapped to the host clock.
 void REEFScheduler::resolve_late_samples() {
     std::lock_guard<std::mutex> lock(stats_mtx);
     for (const LateSample& l : late_samples) {
-        if (l.slot >= preempt_device_ns.size() || preempt_device_ns[l.slot] > -1) continue;
-        int64_t worst = -(preempt_device_ns[l.slot] + 2);
-        uint64_t ticks = 0;
-        if (l.queue < be_queue_cnt.load()) reef_hal_stream_exit_ticks(be_queues[l.queue]->stream, l.seq, &ticks);
-        if (ticks != 0) worst = std::max(worst, std::max<int64_t>(device_ticks_to_host_ns(ticks) - l.t0_ns, 0));
-        preempt_device_ns[l.slot] = -(worst + 2);
+        if (l.slot >= preempt_device_ns.size()) continue;
+        uint64_t ticks = l.ticks;
+        if (ticks == 0 && l.queue < be_queue_cnt.load())
+            reef_hal_stream_exit_ticks(be_queues[l.queue]->stream, l.seq, &ticks);
+        if (ticks == 0) continue;   // overwritten in the meantime: the other streams' exits stand
+        const int64_t v = std::max<int64_t>(device_ticks_to_host_ns(ticks) - l.t0_ns, 0);
+        preempt_device_ns[l.slot] = std::max(preempt_device_ns[l.slot], v);
     }
     for (const LateSample& l : late_samples)
-        if (l.slot < preempt_device_ns.size() && preempt_device_ns[l.slot] <= -1)
-            preempt_device_ns[l.slot] = std::max<int64_t>(-(preempt_device_ns[l.slot] + 2), 0);
+        if (l.slot < preempt_device_ns.size() && preempt_device_ns[l.slot] < 0) preempt_device_ns[l.slot] = 0;
     late_samples.clear();
+}
+
+size_t REEFScheduler::preempt_device_late(uint8_t* out, size_t cap) const {
+    std::lock_guard<std::mutex> lock(stats_mtx);
+    size_t k = 0;
+    for (size_t i = 0; i < preempt_device_ns.size() && k < cap; i++)
+        if (preempt_device_ns[i] >= 0) out[k++] = preempt_device_late_flag[i];
+    return k;
 }
 
 size_t REEFScheduler::preempt_device_samples(int64_t* out_ns, size_t cap) const {
@@ -535,10 +546,10 @@ void REEFScheduler::execute_rt_task(std::shared_ptr<Task>& task) {
     // off the real-time path: complete preemption samples that waited for a late launch, and
     // renew the clock mapping when it is older than 100 ms (the two clocks drift)
     if (clk_valid) {
-        if (!late_samples.empty()) resolve_late_samples();
         const int64_t now = std::chrono::duration_cast<std::chrono::nanoseconds>(
                                 std::chrono::steady_clock::now().time_since_epoch()).count();
         if (now - clk_synced_at_ns > 100000000) sync_clock();
+        if (!late_samples.empty()) resolve_late_samples();
     }
 }
 

@@ -161,6 +161,8 @@ public:
     // raised is counted too: its sample is completed when it has left the device.  Only
     // preemptions that found best-effort kernels on the device have a sample.
     size_t preempt_device_samples(int64_t* out_ns, size_t cap) const;
+    // 1 where the sample waited for a launch that reached the device after the flag was raised
+    size_t preempt_device_late(uint8_t* out, size_t cap) const;
     // Half the length of the host-device clock exchange the mapping rests on (nanoseconds), -1: no mapping.
     int64_t clock_sync_error_ns() const { return clk_valid ? clk_err_ns : -1; }
     // Average nanoseconds per reset-based preemption spent in: raising the flag, dropping the
@@ -218,8 +220,9 @@ private:
     std::vector<int64_t> preempt_samples;
     uint64_t preempt_phase_ns[3];
     // device-side timing of preemptions
-    struct LateSample { size_t slot; uint32_t queue; uint32_t seq; int64_t t0_ns; };
-    std::vector<int64_t> preempt_device_ns;   // -1: still waiting for a late launch
+    struct LateSample { size_t slot; uint32_t queue; uint32_t seq; int64_t t0_ns; uint64_t ticks; };   // ticks 0: not there yet
+    std::vector<int64_t> preempt_device_ns;   // -1: open until the real-time task that caused it is done
+    std::vector<uint8_t> preempt_device_late_flag;   // same index: a late launch was part of it
     std::vector<LateSample> late_samples;
     bool clk_valid = false;
     int64_t clk_host_ns = 0, clk_err_ns = 0, clk_synced_at_ns = 0;
