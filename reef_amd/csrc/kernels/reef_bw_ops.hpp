@@ -44,7 +44,7 @@ __device__ __forceinline__ void splitk_reduce_body(const ReefOpDesc& d, int task
         if (ep.residual) resv = *(const f32x4*)(ep.residual + i0);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const int ch = (int)((i0 + e) / N);
+            const int ch = div_index(i0 + e, N);
             biasv[e] = ep.bias ? ep.bias[ch] : 0.0f;
             sh2v[e] = ep.shift2 ? ep.shift2[ch] : 0.0f;
         }
@@ -62,12 +62,12 @@ __device__ __forceinline__ void splitk_reduce_body(const ReefOpDesc& d, int task
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-            ep.store_pre(out, acc[e], (int)((i0 + e) / N), i0 + e, resv[e], biasv[e], sh2v[e]);
+            ep.store_pre(out, acc[e], div_index(i0 + e, N), i0 + e, resv[e], biasv[e], sh2v[e]);
     } else {
         for (int e = 0; e < 4 && i0 + e < MN; ++e) {
             float acc = ws[i0 + e];
             for (int s = 1; s < S; ++s) acc += ws[(size_t)s * MN + i0 + e];
-            ep.store(out, acc, (int)((i0 + e) / N), i0 + e);
+            ep.store(out, acc, div_index(i0 + e, N), i0 + e);
         }
     }
 }
@@ -102,9 +102,9 @@ __device__ __forceinline__ void dwconv2d_body(const ReefOpDesc& d, int task) {
               sw = a[REEF_DW_SW], ph = a[REEF_DW_PH], pw = a[REEF_DW_PW];
     const int idx = task * kThreads + threadIdx.x;
     if (idx >= C * Ho * Wo) return;
-    const int c = idx / (Ho * Wo);
+    const int c = div_index((size_t)idx, Ho * Wo);
     const int r = idx - c * Ho * Wo;
-    const int y = r / Wo, x = r - y * Wo;
+    const int y = div_small(r, Wo), x = r - y * Wo;
     float acc;
     if (kh == 3 && kw == 3) {
         const rsrc_t rs_in = make_rsrc(d.ptr[0], (unsigned)C * (unsigned)(H * W) * 4u);
@@ -136,9 +136,9 @@ __device__ __forceinline__ void pool2d_body(const ReefOpDesc& d, int task) {
               pw = a[REEF_POOL_PW], mode = a[REEF_POOL_MODE];
     const int idx = task * kThreads + threadIdx.x;
     if (idx >= C * Ho * Wo) return;
-    const int c = idx / (Ho * Wo);
+    const int c = div_index((size_t)idx, Ho * Wo);
     const int r = idx - c * Ho * Wo;
-    const int y = r / Wo, x = r - y * Wo;
+    const int y = div_small(r, Wo), x = r - y * Wo;
     const float* in = (const float*)d.ptr[0] + (size_t)c * H * W;
     float m = -FLT_MAX, s = 0.0f;
     int cnt = 0;
@@ -210,7 +210,7 @@ __device__ __forceinline__ void eltwise_body(const ReefOpDesc& d, int task) {
     const size_t i0 = ((size_t)task * kThreads + threadIdx.x) * 4;
     if (i0 >= total) return;
     if ((inner & 3) == 0) {
-        const int c = (int)(i0 / inner);
+        const int c = div_index(i0, inner);
         f32x4 v = *(const f32x4*)(a + i0);
         if (b) v += *(const f32x4*)(b + i0);
         if (scale) v *= scale[c];
@@ -220,7 +220,7 @@ __device__ __forceinline__ void eltwise_body(const ReefOpDesc& d, int task) {
         *(f32x4*)(out + i0) = v;
     } else {
         for (int e = 0; e < 4 && i0 + e < total; ++e) {
-            const int c = (int)((i0 + e) / inner);
+            const int c = div_index(i0 + e, inner);
             float v = a[i0 + e];
             if (b) v += b[i0 + e];
             if (scale) v *= scale[c];
@@ -373,7 +373,7 @@ __device__ __forceinline__ void bias_gelu_body(const ReefOpDesc& d, int task) {
     const size_t total = (size_t)rows * cols;
     const size_t i0 = ((size_t)task * kThreads + threadIdx.x) * 4;
     for (int e = 0; e < 4 && i0 + e < total; ++e) {
-        const int c = (int)((i0 + e) % cols);
+        const int c = (int)((i0 + e) - (size_t)div_index(i0 + e, cols) * cols);
         y[i0 + e] = gelu_erf(x[i0 + e] + (bias ? bias[c] : 0.0f));
     }
 }
@@ -390,7 +390,7 @@ __device__ __forceinline__ void embedding_body(const ReefOpDesc& d, int task) {
     const size_t total = (size_t)seq * hidden;
     const size_t i0 = ((size_t)task * kThreads + threadIdx.x) * 4;
     for (int e = 0; e < 4 && i0 + e < total; ++e) {
-        const int s = (int)((i0 + e) / hidden), h = (int)((i0 + e) - (size_t)s * hidden);
+        const int s = div_index(i0 + e, hidden), h = (int)((i0 + e) - (size_t)s * hidden);
         float v = tok[(size_t)ids[s] * hidden + h];
         if (pos) v += pos[i0 + e];
         if (seg) v += seg[h];
@@ -421,9 +421,10 @@ __device__ __forceinline__ void transpose_body(const ReefOpDesc& d, int task) {
     const size_t i0 = ((size_t)task * kThreads + threadIdx.x) * 4;
     for (int e = 0; e < 4 && i0 + e < total; ++e) {
         const size_t i = i0 + e;  // output index (b, a, c)
-        const int c = (int)(i % d2);
-        const int a = (int)((i / d2) % d0);
-        const int b = (int)(i / ((size_t)d2 * d0));
+        const int q = div_index(i, d2);          // (b, a) flattened
+        const int c = (int)(i - (size_t)q * d2);
+        const int b = div_small(q, d0);
+        const int a = q - b * d0;
         float v = in[((size_t)a * d1 + b) * d2 + c];
         if (bias) v += bias[(size_t)b * d2 + c];
         out[i] = v;

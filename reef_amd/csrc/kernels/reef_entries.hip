@@ -126,9 +126,9 @@ struct DkpWalk {
 __device__ __forceinline__ bool dkp_walk(const ReefDkpArgs& a, DkpWalk& w) {
     const int C = a.num_cus, X = a.num_xcds;
     const int b = blockIdx.x;
-    const int layer = b / C, cu = b - layer * C;
-    const int xcd = cu % X, slot = cu / X;
-    const int rt_slots = a.cu_partition / X;
+    const int layer = div_small(b, C), cu = b - layer * C;
+    const int slot = div_small(cu, X), xcd = cu - slot * X;
+    const int rt_slots = div_small(a.cu_partition, X);
     int span, cu_idx, layers, task_num, task_offset;
     if (slot < rt_slots) {
         w.right = false;
@@ -339,8 +339,8 @@ REEF_ENTRY(multiply, OpMocked<true>)
         const unsigned wg = __builtin_amdgcn_workgroup_id_x();                               \
         const unsigned tid = __builtin_amdgcn_workitem_id_x();                               \
         const int C = a.num_cus, X = a.num_xcds;                                             \
-        const int cu = (int)wg % C;                                                          \
-        const bool right = cu / X >= a.cu_partition / X;   /* the side test of dkp_walk */   \
+        const int cu = (int)wg - div_small((int)wg, C) * C;                                  \
+        const bool right = div_small(cu, X) >= div_small(a.cu_partition, X);   /* the side test of dkp_walk */ \
         const void* target = right ? a.entry_r : a.entry_l;                                  \
         asm volatile("s_setpc_b64 %3"                                                        \
                      :                                                                       \

@@ -150,7 +150,7 @@ struct Im2colLoader {
         kw = a[REEF_CONV_KW];
         const int Wo = a[REEF_CONV_WO];
         const int n = n0 + (tid & (T::BN - 1));
-        const int y = n / Wo, x = n - y * Wo;
+        const int y = div_small(n, Wo), x = n - y * Wo;
         const int iy0 = y * a[REEF_CONV_SH] - a[REEF_CONV_PH];
         const int ix0 = x * a[REEF_CONV_SW] - a[REEF_CONV_PW];
         soff = iy0 * W + ix0;
@@ -164,14 +164,14 @@ struct Im2colLoader {
         if (UNIFORM) row0 = __builtin_amdgcn_readfirstlane(row0);
         k = k_begin + row0;
         const int khw = kh * kw;
-        c = k / khw;
+        c = div_small(k, khw);
         const int r = k - c * khw;
-        ky = r / kw;
+        ky = div_small(r, kw);
         kx = r - ky * kw;
-        dkx = RS % kw;
-        const int t = RS / kw;
-        dky = t % kh;
-        dc = t / kh;
+        const int t = div_small(RS, kw);
+        dkx = RS - t * kw;
+        dc = div_small(t, kh);
+        dky = t - dc * kh;
     }
     __device__ __forceinline__ void load(Regs& r) {
 #pragma unroll
@@ -536,9 +536,9 @@ __device__ __forceinline__ bool conv2d_body(const ReefOpDesc& d_in, int task, ch
     const int n_tiles = a[REEF_CONV_N_TILES];
     const int tiles = a[REEF_CONV_M_TILES] * n_tiles;
     task = xcd_chunked(task, tiles * split_k);
-    split = task / tiles;
+    split = div_small(task, tiles);
     rem = task - split * tiles;
-    const int mt = rem / n_tiles, nt = rem - mt * n_tiles;
+    const int mt = div_small(rem, n_tiles), nt = rem - mt * n_tiles;
     m0 = mt * T::BM;
     n0 = nt * T::BN;
     const int k_begin = split * k_chunk;
@@ -824,14 +824,16 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     task = xcd_chunked(task, tiles * split_k);
     // Folded split: the workgroups of one tile are neighbours in the task order, so they run on
     // one XCD and meet in its L2; otherwise split-major like the staged tiles.
-    const int split = fused ? task % split_k : task / tiles;
-    const int rem = fused ? task / split_k : task - split * tiles;
-    const int mt = rem / n_tiles, nt = rem - mt * n_tiles;
+    const int q_split = div_small(task, fused ? split_k : tiles);
+    const int split = fused ? task - q_split * split_k : q_split;
+    const int rem = fused ? q_split : task - split * tiles;
+    const int mt = div_small(rem, n_tiles), nt = rem - mt * n_tiles;
     const int m0 = mt * TD::BM, n0 = nt * TD::BN;
     // row form: spatial tile nt -> (row tile, column segment)
     const int segs = ROWS ? (W + kRowSeg - 1) / kRowSeg : 1;
-    const int y0 = ROWS ? (nt / segs) * TN : 0;
-    const int x0 = ROWS ? (nt % segs) * kRowSeg : 0;
+    const int q_seg = ROWS ? div_small(nt, segs) : 0;
+    const int y0 = ROWS ? q_seg * TN : 0;
+    const int x0 = ROWS ? (nt - q_seg * segs) * kRowSeg : 0;
     const int c_chunk = a[REEF_CONV_K_CHUNK] / R;
     const int cb = split * c_chunk;
     const int ce = min(C, cb + c_chunk);
@@ -909,10 +911,10 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
 #pragma unroll
         for (int g = 0; g < TN; ++g) {
             const int n = n0 + 16 * g + i16;
-            const int oy = n / Wo, ox = n - oy * Wo;
+            const int oy = div_small(n, Wo), ox = n - oy * Wo;
 #pragma unroll
             for (int t = 0; t < R; ++t) {
-                const int ky = t / kw_, kx = t - ky * kw_;
+                const int ky = R == 1 ? 0 : div_small(t, kw_), kx = t - ky * kw_;
                 const int iy = oy * a[REEF_CONV_SH] + ky - a[REEF_CONV_PH];
                 const int ix = ox * a[REEF_CONV_SW] + kx - a[REEF_CONV_PW];
                 const bool ok = n < N && (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
@@ -1187,9 +1189,9 @@ __device__ __forceinline__ bool gemm_body(const ReefOpDesc& d, int task, char* s
     const int M = a[REEF_GEMM_M], N = a[REEF_GEMM_N], K = a[REEF_GEMM_K];
     const int n_tiles = a[REEF_GEMM_N_TILES];
     const int tiles = a[REEF_GEMM_M_TILES] * n_tiles;
-    const int b = task / tiles;
+    const int b = div_small(task, tiles);
     const int rem = task - b * tiles;
-    const int mt = rem / n_tiles, nt = rem - mt * n_tiles;
+    const int mt = div_small(rem, n_tiles), nt = rem - mt * n_tiles;
     const int m0 = mt * T::BM, n0 = nt * T::BN;
     const int lda = a[REEF_GEMM_LDA], ldb = a[REEF_GEMM_LDB], ldc = a[REEF_GEMM_LDC];
     const float* A = (const float*)d.ptr[0] + (size_t)b * a[REEF_GEMM_STRIDE_A];
@@ -1266,9 +1268,9 @@ __device__ __forceinline__ bool gemm_nt_direct_body(const ReefOpDesc& d, int tas
     const int M = a[REEF_GEMM_M], N = a[REEF_GEMM_N], K = a[REEF_GEMM_K];
     const int n_tiles = a[REEF_GEMM_N_TILES];
     const int tiles = a[REEF_GEMM_M_TILES] * n_tiles;
-    const int b = task / tiles;
+    const int b = div_small(task, tiles);
     const int rem = task - b * tiles;
-    const int mt = rem / n_tiles, nt = rem - mt * n_tiles;
+    const int mt = div_small(rem, n_tiles), nt = rem - mt * n_tiles;
     const int m0 = mt * TD::BM, n0 = nt * TD::BN;
     const unsigned lda = (unsigned)a[REEF_GEMM_LDA], ldb = (unsigned)a[REEF_GEMM_LDB],
                    ldc = (unsigned)a[REEF_GEMM_LDC];

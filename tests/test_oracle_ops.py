@@ -197,3 +197,30 @@ def test_masked_softmax_is_the_where_kernel_in_front_of_the_softmax():
     np.testing.assert_array_equal(O.softmax(x, np.zeros(37, np.uint8)), O.softmax(x))
     keep = mask == 0
     np.testing.assert_allclose(got[:, keep], O.softmax(x[:, keep]), rtol=1e-6, atol=1e-9)
+
+
+def test_reciprocal_division_of_the_kernels_is_exact_on_its_stated_range():
+    """reef_common.hpp:div_small computes a / b for 0 <= a < 2^22, 0 < b < 2^22 as
+    trunc(float(a) * rcp(float(b))) corrected by the sign and size of the remainder.  The
+    hardware reciprocal is good to one unit in the last place: the same arithmetic in float32,
+    with the reciprocal pushed one unit either way, must give the exact quotient everywhere it is
+    probed (all small operands, random large ones, and the neighbours of every multiple)."""
+    rng = np.random.default_rng(22)
+
+    def div_small(a, b, nudge):
+        rb = (np.float32(1.0) / b.astype(np.float32)).astype(np.float32)
+        rb = np.nextafter(rb, np.float32(np.inf if nudge > 0 else -np.inf)) if nudge else rb
+        q = (a.astype(np.float32) * rb).astype(np.float32).astype(np.int64)
+        r = a - q * b
+        return q + (r >= b) - (r < 0)
+
+    small = np.arange(0, 2048, dtype=np.int64)
+    a1, b1 = np.meshgrid(small, small[1:], indexing="ij")
+    b2 = rng.integers(1, 1 << 22, 200000)
+    a2 = rng.integers(0, 1 << 22, 200000)
+    b3 = rng.integers(1, 5000, 200000)
+    k3 = rng.integers(0, (1 << 22) // 5000, 200000)
+    a3 = np.clip(b3 * k3 + rng.integers(-1, 2, 200000), 0, (1 << 22) - 1)     # around exact multiples
+    for a, b in ((a1.ravel(), b1.ravel()), (a2, b2), (a3, b3)):
+        for nudge in (-1, 0, 1):
+            np.testing.assert_array_equal(div_small(a, b, nudge), a // b)
