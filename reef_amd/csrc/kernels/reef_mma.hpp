@@ -859,28 +859,12 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
             }
         }
     }
-    ConvEpilogue ep;
-    ep.next = 3;   // plain split-K launches carry no epilogue operands
-    float e_bias[TM], e_sh2[TM], e_res[TM][TN];
-#pragma unroll
-    for (int h = 0; h < TM; ++h) {
-        e_bias[h] = e_sh2[h] = 0.0f;
-#pragma unroll
-        for (int g = 0; g < TN; ++g) e_res[h][g] = 0.0f;
-    }
-    if (!to_ws) {
-        ep.init(d, flags, a[REEF_CONV_ACT], a[REEF_CONV_ACT2], M, MN4, (unsigned)a[REEF_CONV_DST_OFF] * 4u);
-#pragma unroll
-        for (int h = 0; h < TM; ++h) {
-            if (ep.has_bias) e_bias[h] = buf_load(ep.bias, om[h] * 4u);
-            if (ep.has_dual) e_sh2[h] = buf_load(ep.shift2, om[h] * 4u);
-            if (ep.has_res) {
-#pragma unroll
-                for (int g = 0; g < TN; ++g) e_res[h][g] = buf_load(ep.res, ooff[h][g]);
-            }
-        }
-    }
-
+    // Pointer slot behind the optional epilogue operands (known from the flags alone): the
+    // epilogue itself is set up further down, after the first loads of the K loop are on their
+    // way -- its operands are needed last.
+    const int ep_next = to_ws ? 3
+                              : 3 + ((flags & REEF_F_BIAS) ? 1 : 0) + ((flags & REEF_F_RESIDUAL) ? 1 : 0) +
+                                    ((flags & REEF_F_AFFINE) ? 2 : 0) + ((flags & REEF_F_DUAL) ? 2 : 0);
     // per-lane operand offsets
     const rsrc_t rs_a = make_rsrc(d.ptr[1], (unsigned)M * (unsigned)K * 4u);
     const rsrc_t rs_b = make_rsrc(d.ptr[0], (unsigned)C * HW4);
@@ -896,51 +880,17 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
         va[h] = PACKED ? (((unsigned)(m0 / 16 + h) * C4 + (unsigned)(cb / 4 + wave)) * (unsigned)G4) * 1024u
                              + (unsigned)lane * 16u
                        : ((unsigned)(m0 + 16 * h + i16) * (unsigned)K + (unsigned)(lane_c * R)) * 4u;
-    unsigned vb[ROWS ? TN + 2 : TN][ROWS ? 1 : R];
-    if (ROWS) {
-        // one value per input row: column of this lane (lane 15: left of the segment)
-        const int ix = i16 == 15 ? x0 - 1 : x0 + i16;
-#pragma unroll
-        for (int r = 0; r < TN + 2; ++r) {
-            const int iy = y0 - 1 + r;
-            const bool ok = (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
-            vb[ROWS ? r : 0][0] = ok ? (unsigned)(iy * W + ix) * 4u + (unsigned)lane_c * HW4 : kOutside;
-        }
-    } else {
-        const int kw_ = a[REEF_CONV_KW];
-#pragma unroll
-        for (int g = 0; g < TN; ++g) {
-            const int n = n0 + 16 * g + i16;
-            const int oy = div_small(n, Wo), ox = n - oy * Wo;
-#pragma unroll
-            for (int t = 0; t < R; ++t) {
-                const int ky = R == 1 ? 0 : div_small(t, kw_), kx = t - ky * kw_;
-                const int iy = oy * a[REEF_CONV_SH] + ky - a[REEF_CONV_PH];
-                const int ix = ox * a[REEF_CONV_SW] + kx - a[REEF_CONV_PW];
-                const bool ok = n < N && (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
-                vb[ROWS ? 0 : g][ROWS ? 0 : t] = ok ? (unsigned)(iy * W + ix) * 4u + (unsigned)lane_c * HW4 : kOutside;
-            }
-        }
-    }
     // steps this lane's k slot stays inside the channel range of the split
     const int lane_steps = lane_c < ce ? (ce - lane_c + G::STEP_C - 1) / G::STEP_C : 0;
-
-    // operands that follow the optional epilogue operands: (pre-activation scale, shift), then
-    // (workspace, arrival counters) of a folded split
-    const int aux = ep.next + (PRE ? 2 : 0);
-    const rsrc_t rs_ps = make_rsrc(d.ptr[PRE ? ep.next : 0], (unsigned)C * 4u);
-    const rsrc_t rs_pt = make_rsrc(d.ptr[PRE ? ep.next + 1 : 0], (unsigned)C * 4u);
-    const unsigned vpre = (unsigned)lane_c * 4u;
 
     constexpr int NB = G::NB;
     float ra[NS][TM][RC], rb[NS][NB];
     float rps[NS][PRE ? 8 : 1], rpt[NS][PRE ? 8 : 1];
-    auto load_step = [&](int s, int step) {
+    auto load_a = [&](int s, int step) {
         // offsets are below kOutside (a power of two), so or-ing it in moves them outside
         const unsigned outm = step < lane_steps ? 0u : kOutside;
         const unsigned sa = PACKED ? (unsigned)step * (unsigned)(4 * G4) * 1024u      // uniform
                                    : (unsigned)step * (unsigned)(G::STEP_C * R) * 4u;
-        const unsigned sb = (unsigned)step * (unsigned)G::STEP_C * HW4;         // uniform
         if (PACKED) {
 #pragma unroll
             for (int h = 0; h < TM; ++h) {
@@ -975,6 +925,51 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
                 ra[s][h][q] = __builtin_bit_cast(
                     float, __builtin_amdgcn_raw_buffer_load_b32(rs_a, (int)(oa + 4u * q), (int)sa, 0));
         }
+    };
+    // The weights first -- the cold stream, and their offsets need nothing of the pixel
+    // decode -- for all NS steps; the input offsets are worked out while those are on
+    // their way.  (The waits the compiler places count loads in issue order, whatever it is.)
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        load_a(s, s);
+        asm volatile("" ::: "memory");
+    }
+    unsigned vb[ROWS ? TN + 2 : TN][ROWS ? 1 : R];
+    if (ROWS) {
+        // one value per input row: column of this lane (lane 15: left of the segment)
+        const int ix = i16 == 15 ? x0 - 1 : x0 + i16;
+#pragma unroll
+        for (int r = 0; r < TN + 2; ++r) {
+            const int iy = y0 - 1 + r;
+            const bool ok = (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
+            vb[ROWS ? r : 0][0] = ok ? (unsigned)(iy * W + ix) * 4u + (unsigned)lane_c * HW4 : kOutside;
+        }
+    } else {
+        const int kw_ = a[REEF_CONV_KW];
+#pragma unroll
+        for (int g = 0; g < TN; ++g) {
+            const int n = n0 + 16 * g + i16;
+            const int oy = div_small(n, Wo), ox = n - oy * Wo;
+#pragma unroll
+            for (int t = 0; t < R; ++t) {
+                const int ky = R == 1 ? 0 : div_small(t, kw_), kx = t - ky * kw_;
+                const int iy = oy * a[REEF_CONV_SH] + ky - a[REEF_CONV_PH];
+                const int ix = ox * a[REEF_CONV_SW] + kx - a[REEF_CONV_PW];
+                const bool ok = n < N && (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
+                vb[ROWS ? 0 : g][ROWS ? 0 : t] = ok ? (unsigned)(iy * W + ix) * 4u + (unsigned)lane_c * HW4 : kOutside;
+            }
+        }
+    }
+    // operands that follow the optional epilogue operands: (pre-activation scale, shift), then
+    // (workspace, arrival counters) of a folded split
+    const int aux = ep_next + (PRE ? 2 : 0);
+    const rsrc_t rs_ps = make_rsrc(d.ptr[PRE ? ep_next : 0], (unsigned)C * 4u);
+    const rsrc_t rs_pt = make_rsrc(d.ptr[PRE ? ep_next + 1 : 0], (unsigned)C * 4u);
+    const unsigned vpre = (unsigned)lane_c * 4u;
+
+    auto load_b = [&](int s, int step) {
+        const unsigned outm = step < lane_steps ? 0u : kOutside;
+        const unsigned sb = (unsigned)step * (unsigned)G::STEP_C * HW4;         // uniform
         if (PRE) {
             const unsigned op = vpre | outm;
             const unsigned sp = (unsigned)step * (unsigned)G::STEP_C * 4u;   // uniform
@@ -1009,13 +1004,39 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
                 }
         }
     };
-
-    // oldest step first: the wait before a step's MFMAs counts the loads issued after its own
+    auto load_step = [&](int s, int step) {
+        load_a(s, step);
+        load_b(s, step);
+    };
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
-        load_step(s, s);
+        load_b(s, s);
         asm volatile("" ::: "memory");
     }
+
+    // epilogue operands of this thread's output elements, behind the first K steps' loads
+    ConvEpilogue ep;
+    ep.next = 3;   // plain split-K launches carry no epilogue operands
+    float e_bias[TM], e_sh2[TM], e_res[TM][TN];
+#pragma unroll
+    for (int h = 0; h < TM; ++h) {
+        e_bias[h] = e_sh2[h] = 0.0f;
+#pragma unroll
+        for (int g = 0; g < TN; ++g) e_res[h][g] = 0.0f;
+    }
+    if (!to_ws) {
+        ep.init(d, flags, a[REEF_CONV_ACT], a[REEF_CONV_ACT2], M, MN4, (unsigned)a[REEF_CONV_DST_OFF] * 4u);
+#pragma unroll
+        for (int h = 0; h < TM; ++h) {
+            if (ep.has_bias) e_bias[h] = buf_load(ep.bias, om[h] * 4u);
+            if (ep.has_dual) e_sh2[h] = buf_load(ep.shift2, om[h] * 4u);
+            if (ep.has_res) {
+#pragma unroll
+                for (int g = 0; g < TN; ++g) e_res[h][g] = buf_load(ep.res, ooff[h][g]);
+            }
+        }
+    }
+
     if (Poll::enabled) {
         if (threadIdx.x == 0) *sflag = 0;
         __syncthreads();
