@@ -195,6 +195,14 @@ enum {
 #define REEF_F_PRE_ACT 32      /* the input is read through relu(in * pre_scale[c] + pre_shift[c]); the two
                                   vectors follow the optional operands (before workspace and counters);
                                   symbols reef_conv2d_p1_<tile>: 1x1 filters, no padding */
+#define REEF_F_PAIR_FOLD 64    /* with REEF_F_FUSED_REDUCE and split_k == 2, direct family: the workspace has a third
+                                  region of M * N words, zero at rest (the pair slots).  Where every launch on these
+                                  buffers runs to completion (plain launches, the real-time side of a padded launch)
+                                  the two workgroups of a tile meet there with ONE atomic exchange per output element
+                                  instead of partial tile out / count / partial tile in: the first to arrive parks
+                                  its value, the second gets it back, adds in split order, finishes the element and
+                                  empties the slot.  Best-effort launches, which may be cut short, and the
+                                  best-effort side of a padded launch keep the counters. */
 
 /* Loader families of the convolution; the entry symbol carries the family:
  *   reef_conv2d_<tile>      general: im2col gather, needs K % 4 == 0

@@ -24,11 +24,17 @@ constexpr int kThreads = REEF_WG_THREADS;
 // the load is not served from a stale cache line.
 struct NoPoll {
     static constexpr bool enabled = false;
+    // true: every launch of this kernel on this model's buffers runs to completion (a real-time
+    // model: plain launches and the real-time side of a padded launch).  What a folded split of
+    // two may leave between its two workgroups in the pair slots relies on it (REEF_F_PAIR_FOLD).
+    bool completes = false;
     __device__ __forceinline__ int load() const { return 0; }
+    __device__ __forceinline__ bool pair_fold_ok() const { return completes; }
 };
 struct FlagPoll {
     static constexpr bool enabled = true;
     const int* flag;
+    __device__ __forceinline__ bool pair_fold_ok() const { return false; }
     __device__ __forceinline__ int load() const {
         return __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }

@@ -186,7 +186,7 @@ __device__ __forceinline__ bool dkp_walk(const ReefDkpArgs& a, DkpWalk& w) {
     extern "C" __global__ void __launch_bounds__(REEF_WG_THREADS) NAME(ReefOpDesc) {  \
         __shared__ __align__(16) char smem[OP::LDS > 0 ? OP::LDS : 16];               \
         kernarg_warm<sizeof(ReefOpDesc)>();                                           \
-        OP::run(kernarg_at<ReefOpDesc>(0), (int)blockIdx.x, smem, NoPoll{});          \
+        OP::run(kernarg_at<ReefOpDesc>(0), (int)blockIdx.x, smem, NoPoll{true});      \
     }
 #elif REEF_FLAVOUR == 1
 namespace {
@@ -237,7 +237,7 @@ __device__ __forceinline__ void be_signal_exit(const ReefBeArgs& a, int t) {
         if (!dkp_walk(a, w)) return;                                                   \
         const ReefDkpSide& side = w.right ? a.r : a.l;                                 \
         for (int i = w.idx; i < w.end; i += w.step) {                                  \
-            OP::run(side.desc, i, smem, NoPoll{});                                     \
+            OP::run(side.desc, i, smem, NoPoll{!w.right});                             \
             __syncthreads();                                                           \
         }                                                                              \
     }                                                                                  \

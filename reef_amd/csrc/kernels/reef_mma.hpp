@@ -1159,6 +1159,36 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     // split-K folded inside the launch
     const size_t MN = (size_t)M * N;
     float* ws = (float*)d.ptr[aux];
+    if (split_k == 2 && (flags & REEF_F_PAIR_FOLD) && poll.pair_fold_ok()) {
+        // One exchange per output element.  A value is parked with its sign bit flipped: a sum
+        // of products that starts from +0 is never -0, so a parked value is never the empty
+        // slot's 0 (and a -0 is parked as +0, should one ever come).
+        unsigned* slots = (unsigned*)(ws + 2 * MN);
+        unsigned got[TM][TN];
+#pragma unroll
+        for (int h = 0; h < TM; ++h)
+#pragma unroll
+            for (int g = 0; g < TN; ++g) {
+                got[h][g] = 0;
+                if (ooff[h][g] != kOutside && om[h] < (unsigned)M) {
+                    unsigned mine = __float_as_uint(v[h][g]) ^ 0x80000000u;
+                    mine = mine ? mine : 0x80000000u;
+                    got[h][g] = __hip_atomic_exchange(&slots[ooff[h][g] >> 2], mine, __ATOMIC_RELAXED,
+                                                      __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+#pragma unroll
+        for (int h = 0; h < TM; ++h)
+#pragma unroll
+            for (int g = 0; g < TN; ++g)
+                if (got[h][g] != 0) {   // second to arrive: the other half is here
+                    const float other = __uint_as_float(got[h][g] ^ 0x80000000u);
+                    const float sum = split == 0 ? v[h][g] + other : other + v[h][g];   // split order
+                    ep.finish(sum, ooff[h][g], om[h] * 4u, e_res[h][g], e_bias[h], e_sh2[h]);
+                    __hip_atomic_store(&slots[ooff[h][g] >> 2], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+        return true;
+    }
     int* counters = (int*)d.ptr[aux + 1] + a[REEF_CONV_SYNC_OFF];
     int* s_last = sflag + 1;
 #pragma unroll

@@ -24,7 +24,7 @@ from . import rng, tiling
 from ..paths import code_object
 
 ACT_NONE, ACT_RELU, ACT_RELU6, ACT_GELU = 0, 1, 2, 3
-F_BIAS, F_RESIDUAL, F_AFFINE, F_DUAL, F_FUSED_REDUCE, F_PRE_ACT = 1, 2, 4, 8, 16, 32
+F_BIAS, F_RESIDUAL, F_AFFINE, F_DUAL, F_FUSED_REDUCE, F_PRE_ACT, F_PAIR_FOLD = 1, 2, 4, 8, 16, 32, 64
 WG = 256
 
 
@@ -67,6 +67,7 @@ class GraphBuilder:
         # multi-tap filters on the direct / row tiles also get a copy of their weights in the
         # layout those kernels load fastest (pack_conv_weights); parameter key = weight key + "k"
         self.pack_weights = True
+        self.pair_fold = os.environ.get("REEF_PAIR_FOLD", "1") != "0"
 
     # ------------------------------------------------------------ storages
     def _storage(self, name, size, stype="float32"):
@@ -240,9 +241,12 @@ class GraphBuilder:
         elif fused_reduce:
             # workspace: split_k partial tensors; counters: one int per output tile in
             # the model's single sync storage
-            ws = self.workspace(t["split_k"] * M * N)
+            # a split of two in the direct family: a third region, the pair slots (REEF_F_PAIR_FOLD)
+            pair = t["split_k"] == 2 and mode in (3, 4, 5) and self.pair_fold
+            ws = self.workspace((t["split_k"] + (1 if pair else 0)) * M * N)
             sync_idx, sync_off = self._sync_counters(t["m_tiles"] * t["n_tiles"])
             args = [x.idx, w.idx, out.idx] + opt + pre + [ws.idx, sync_idx]
+            flags |= F_PAIR_FOLD if pair else 0
             attrs = base + [flags | F_FUSED_REDUCE, act, t["tile_id"], t["split_k"], t["k_chunk"],
                             t["m_tiles"], t["n_tiles"], act2, sync_off, mode, dst_off, len(args) if packed else 0]
             self._emit(kname, t["tasks"], args + packed, attrs, "conv2d", flops, nbytes + nbytes_pack, t["est_us"])

@@ -44,7 +44,10 @@ def written_float_storages(model):
         s = model["storage"][i]
         if s["name"] in ("data", "input0", "reef_sync") or s["name"].startswith("p"):
             continue
-        if s["stype"] == "float32" or s["name"] == "temp_arg":   # temp_arg: split-K partial tensors, bytes
+        # not the split-K workspaces (temp_arg): scratch whose content depends on how the kernel
+        # was launched (a best-effort launch leaves its partial tiles there, a launch that runs
+        # to completion folds a split of two through the pair slots and leaves nothing)
+        if s["stype"] == "float32":
             out.append(i)
     return out
 
@@ -97,6 +100,15 @@ class Solo:
             if s["name"] == "reef_sync":
                 cnt = sched.get_data(mid, i, s["size"], np.int32)
                 assert not cnt.any(), "%s: split-K arrival counters left non-zero" % what
+        # the pair slots of a split of two (REEF_F_PAIR_FOLD = 64) are empty at rest
+        for k in self.model["kernels"]:
+            a = k.get("attrs", [])
+            if k["name"].startswith("reef_conv2d") and len(a) >= 24 and a[12] & 64:
+                n_args = a[23] if a[23] else len(k["args"])
+                ws = k["args"][n_args - 2]
+                mn = a[3] * a[4] * a[5]
+                slots = sched.get_data(mid, ws, self.n_floats(ws), np.int32)[2 * mn:3 * mn]
+                assert slots.size == mn and not slots.any(), "%s: pair slots of %s left non-zero" % (what, k["name"])
 
 
 @pytest.fixture(scope="module")

@@ -1,6 +1,7 @@
 """End-to-end and per-layer parity of whole models against the CPU oracle,
 through all three kernel flavours (raw / DKP single-sided / preemptible), and
 the bit-identity guarantees between flavours."""
+import ctypes
 import json
 import os
 
@@ -174,3 +175,61 @@ def test_recorded_submission_replays_bit_identical(tmp_path, kind):
         np.testing.assert_array_equal(a, b, err_msg="replay %d" % rep)
         rec.execute_to(7)          # eager partial run between replays
     assert not np.array_equal(a, np.zeros_like(a))
+
+
+def test_split_of_two_meets_in_the_pair_slots_or_on_the_counters_with_the_same_bits(tmp_path):
+    """A split of two folded inside the launch has two protocols (REEF_F_PAIR_FOLD): launches
+    that run to completion (raw flavour, real-time side of the padding flavour) meet in the pair
+    slots with one atomic exchange per element, preemptible launches on the arrival counters.
+    Same sums in the same order: all three flavours hold the same bits, run after run and in any
+    order on ONE executor (shared buffers), the pair slots and the counters are empty at rest,
+    and a preemptible run that was cut short (flag raised) leaves the pair slots alone."""
+    g = nets.resnet(152)          # the benchmark network: 71 of its convolutions are such splits
+    pair = [k for k in g.kernels if k["name"].startswith("reef_conv2d") and k["attrs"][12] & 64]
+    assert len(pair) >= 60, "the network must contain splits of two in the direct family"
+    d = write_model(g, tmp_path)
+    model = json.load(open(os.path.join(d, g.name + ".json")))
+    x = nets.image_input("resnet152", (3, 224, 224))
+    logits = model["kernels"][-1]["args"][0]
+    n_log = model["storage"][logits]["size"]
+
+    def slots_and_counters(exe):
+        for k in model["kernels"]:
+            a = k["attrs"]
+            if k["name"].startswith("reef_conv2d") and a[12] & 64:
+                n_args = a[23] if a[23] else len(k["args"])
+                ws = k["args"][n_args - 2]
+                mn = a[3] * a[4] * a[5]
+                words = exe.get_data(ws, model["storage"][ws]["size"] // 4, np.int32)
+                assert words.size == 3 * mn and not words[2 * mn:].any(), k["name"]
+        for i, s in enumerate(model["storage"]):
+            if s["name"] == "reef_sync":
+                assert not exe.get_data(i, s["size"], np.int32).any()
+
+    exe = B.Executor.from_dir(d, g.name, B.HYBRID)
+    exe.set_input_checked("data", x)
+    exe.execute()
+    want = exe.get_data(logits, n_log)
+    slots_and_counters(exe)
+    for run in ("preemptible", "raw", "cut short", "raw", "preemptible"):
+        zero = np.zeros(n_log, np.float32)
+        assert B.lib().reef_executor_set_input_idx(exe.h, logits, ctypes.c_void_p(zero.ctypes.data),
+                                                   ctypes.c_size_t(zero.nbytes)) == 0
+        if run == "cut short":
+            exe.poke_preempt_flag(1)
+            exe.execute_preemptable()          # every workgroup leaves at once
+            exe.poke_preempt_flag(0)
+            slots_and_counters(exe)
+            continue
+        exe.execute_preemptable() if run == "preemptible" else exe.execute()
+        np.testing.assert_array_equal(exe.get_data(logits, n_log), want, err_msg=run)
+        slots_and_counters(exe)
+    exe.close()
+    # the padding flavour, single-sided (real-time side): pair slots again
+    t = B.Executor.from_dir(d, g.name, B.TRANS)
+    t.set_input_checked("data", x)
+    for _ in range(2):
+        t.execute()
+        np.testing.assert_array_equal(t.get_data(logits, n_log), want)
+        slots_and_counters(t)
+    t.close()
