@@ -39,6 +39,7 @@ struct OpConv {
 template <int R, int TN = 1, int TM = 1, bool PRE = false, bool ROWS = false, bool PACKED = false>
 struct OpConvDirect {
     static constexpr int LDS = TileD16<TN, TM>::LDS_BYTES;
+    static constexpr bool CHECKS_FLAG_ITSELF = true;   // the body makes the wrapper's first flag check
     template <class P>
     static __device__ __forceinline__ bool run(const ReefOpDesc& d, int task, char* smem, const P& p) {
         return conv2d_direct_body<R, TN, TM, PRE, ROWS, PACKED>(d, task, smem, p);
@@ -63,6 +64,7 @@ struct OpGemm {
 template <int TM, int TN>
 struct OpGemmNtDirect {
     static constexpr int LDS = TileD16<TN, TM>::LDS_BYTES;
+    static constexpr bool CHECKS_FLAG_ITSELF = true;
     template <class P>
     static __device__ __forceinline__ bool run(const ReefOpDesc& d, int task, char* smem, const P& p) {
         return gemm_nt_direct_body<TM, TN>(d, task, smem, p);
@@ -208,6 +210,14 @@ __device__ __forceinline__ void be_signal_exit(const ReefBeArgs& a, int t) {
     __hip_atomic_store(a.done_word, a.seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 }  // namespace
+namespace {
+// Ops whose body makes the first flag check of a best-effort workgroup itself, at a point where
+// its loads are already under way (the direct families); for all others the wrapper makes it.
+template <class OP, class = void>
+struct ChecksFlagItself { static constexpr bool value = false; };
+template <class OP>
+struct ChecksFlagItself<OP, decltype((void)OP::CHECKS_FLAG_ITSELF)> { static constexpr bool value = OP::CHECKS_FLAG_ITSELF; };
+}  // namespace
 #define REEF_ENTRY(NAME, OP)                                                              \
     extern "C" __global__ void __launch_bounds__(REEF_WG_THREADS) NAME(ReefBeArgs) {      \
         __shared__ __align__(16) char smem[OP::LDS > 0 ? OP::LDS : 16];                   \
@@ -216,10 +226,14 @@ __device__ __forceinline__ void be_signal_exit(const ReefBeArgs& a, int t) {
         const ReefBeArgs& a = kernarg_at<ReefBeArgs>(0);                                  \
         const int t = threadIdx.x + threadIdx.y * blockDim.x + threadIdx.z * blockDim.x * blockDim.y; \
         FlagPoll poll{a.preempted};                                                       \
-        if (t == 0) s_pre = poll.load();                                                  \
-        __syncthreads();                                                                  \
         bool done = false;                                                                \
-        if (!s_pre) done = OP::run(a.desc, (int)blockIdx.x, smem, poll);                  \
+        if (ChecksFlagItself<OP>::value) {                                                \
+            done = OP::run(a.desc, (int)blockIdx.x, smem, poll);                          \
+        } else {                                                                          \
+            if (t == 0) s_pre = poll.load();                                              \
+            __syncthreads();                                                              \
+            if (!s_pre) done = OP::run(a.desc, (int)blockIdx.x, smem, poll);              \
+        }                                                                                 \
         if (done && t == 0) atomicAdd(a.task_slot, 1);                                    \
         be_signal_exit(a, t);                                                             \
     }

@@ -1038,8 +1038,13 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     }
 
     if (Poll::enabled) {
-        if (threadIdx.x == 0) *sflag = 0;
+        // The flag check every best-effort workgroup makes before it does anything
+        // (script/best_effort_kernel.py:22-29) is made here, with the first loads of the K loop
+        // already on their way: its trip to memory hides behind theirs instead of standing in
+        // front of them.  A workgroup that finds the flag raised has only read.
+        if (threadIdx.x == 0) *sflag = poll.load();
         __syncthreads();
+        if (*sflag) return false;
     }
 
     // Whole groups of NS steps with no condition inside (a loop with per-step conditions gets
@@ -1381,8 +1386,13 @@ __device__ __forceinline__ bool gemm_nt_direct_body(const ReefOpDesc& d, int tas
         asm volatile("" ::: "memory");
     }
     if (Poll::enabled) {
-        if (threadIdx.x == 0) *sflag = 0;
+        // The flag check every best-effort workgroup makes before it does anything
+        // (script/best_effort_kernel.py:22-29) is made here, with the first loads of the K loop
+        // already on their way: its trip to memory hides behind theirs instead of standing in
+        // front of them.  A workgroup that finds the flag raised has only read.
+        if (threadIdx.x == 0) *sflag = poll.load();
         __syncthreads();
+        if (*sflag) return false;
     }
     f32x4 acc[TM][TN][2];
 #pragma unroll
