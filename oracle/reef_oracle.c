@@ -32,9 +32,12 @@
  *   depthwise 3x3 convolution (stride 1 and 2), 11x11 stride 4 / 5x5 / 3x3
  *   convolutions without bias, unpadded 3x3 stride 2 max-pool, dense+add+relu:
  *     the generated kernels of resource/mobilenet/mobilenet.cu and
- *     resource/alexnet/alexnet.cu, the same way (tests/golden/make_chain_shapes.py
+ *     resource/alexnet/alexnet.cu, the same way (tests/golden/make_graph_shapes.py
  *     finds each kernel's shape by it; tests/test_gpu_legacy_import.py runs both
  *     networks from input to classifier beside the reference's kernels).
+ *   the five fused convolution families once more on the 34 kernels of
+ *     resource/vgg/vgg.cu (a pre-activation ResNet-50 at 64 x 64 whose stride-2
+ *     bottleneck kernel is intact): all reproduced, 69 calls free-running.
  *   mocked add/multiply: the reference's closed form (3+3)*3 == 18, also on the
  *     reference's own mocked kernels.
  *   The reference's ResNet-18 ten-float golden vector needs a weight blob that

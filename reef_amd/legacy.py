@@ -16,7 +16,8 @@ the same thing.  What a kernel name computes comes from a per-model table
 are those of the kernel families (convolution: in, W, out, then the epilogue operands in the
 order the family name lists them; depthwise convolution: in, W, out, bias; elementwise add and
 flatten: out first; pooling: in, out; dense: x, W, out, bias).  Tables are packaged for the
-reference's `resnet152`, `mobilenet` and `alexnet` directories.
+reference's `resnet152`, `mobilenet`, `alexnet` and `vgg` directories (the last one holds a
+pre-activation ResNet-50 at 64 x 64 under TVM's `tvmgen_default_` kernel names).
 While it rewrites, the importer follows the tensor shapes through the graph and refuses a table
 that does not fit the graph.
 """

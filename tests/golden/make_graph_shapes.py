@@ -1,19 +1,24 @@
-"""Writes <model>_kernel_shapes.json for the reference's chain-shaped model directories
-(resource/mobilenet: MobileNet v1 with depthwise convolutions; resource/alexnet: 11x11 / 5x5 / 3x3
-convolutions without bias, plain max-pools, three dense layers): for every kernel name what it
-computes -- op, shape, filter, stride, padding, epilogue.
+"""Writes <model>_kernel_shapes.json for model directories of the reference whose graph can be
+walked from the input with every kernel witnessed on the way:
 
-As for resnet152 (make_resnet152_shapes.py) the shapes are baked into the generated source and
-the graph JSON only holds shared, maximal buffer sizes, so every entry has a witness: the graph is
-walked from the 3 x 224 x 224 input, each distinct kernel of oracle/_ref/<model>.raw.co (the
-reference's own <model>.cu compiled for gfx950, `make -C oracle ref`) is run once on random
-operands on the GPU, and of the hypotheses that are consistent with its operand sizes and with
-the number of elements it writes (groups 1 or depthwise, filter 1..11, stride 1/2/4, every padding
-up to half the filter) exactly one must make the CPU oracle reproduce its output.  Dense kernels
+  mobilenet  MobileNet v1 with depthwise convolutions, 224 x 224
+  alexnet    11x11 / 5x5 / 3x3 convolutions without bias, plain max-pools, three dense layers
+  vgg        despite its name a pre-activation ResNet-50 at 64 x 64 (kernel names carry TVM's
+             `tvmgen_default_` prefix): the residual families of resnet152
+
+For every kernel name: what it computes -- op, shape, filter, stride, padding, epilogue.  The
+shapes are baked into the generated source and the graph JSON only holds shared, maximal buffer
+sizes, so every entry has a witness: the graph is walked from the input, each distinct kernel of
+oracle/_ref/<model>.raw.co (the reference's own <model>.cu compiled for gfx950, `make -C oracle
+ref`) is run once on random operands on the GPU, and of the hypotheses that are consistent with
+its operand sizes and with the number of elements it writes (groups 1 or depthwise, filter 1..11,
+stride 1/2/4, every padding up to half the filter) exactly one must make the CPU oracle reproduce
+its output.  The epilogue follows from the family name (resnet152.cu:315-363, 376-713, 2662: add =
+residual when the operand is a tensor of the graph, bias when it is a parameter).  Dense kernels
 are run on small non-negative integers and softmax has no witness, for the reason given in the
 module docstring of tests/test_gpu_reference_kernels.py.
 
-Needs a GPU:  python tests/golden/make_chain_shapes.py mobilenet|alexnet
+Needs a GPU:  python tests/golden/make_graph_shapes.py mobilenet|alexnet|vgg
 The result is committed as tests/golden/<model>_kernel_shapes.json (fixture) and as
 reef_amd/legacy_tables/<model>.json (the importer's table for that model directory)."""
 import json
@@ -28,10 +33,25 @@ sys.path.insert(0, ROOT)
 
 from oracle import oracle as O                                   # noqa: E402
 from reef_amd import binding as B                                # noqa: E402
+from reef_amd import legacy                                      # noqa: E402
 from tests import test_gpu_reference_kernels as T                # noqa: E402
+
+EPILOGUE = {"fused_nn_conv2d": "none", "fused_nn_conv2d_nn_relu": "relu",
+            "fused_nn_conv2d_add": "residual", "fused_nn_conv2d_add_nn_relu": "bias_relu",
+            "fused_nn_conv2d_add_add_nn_relu": "residual_bias_relu",
+            "fused_nn_conv2d_add_multiply_add_nn_relu": "residual_scale_shift_relu"}
+
+
+def plain(name):
+    return name[len("tvmgen_default_"):] if name.startswith("tvmgen_default_") else name
+
+
+def family(name):
+    return plain(name).split("_kernel0")[0].rstrip("0123456789").rstrip("_")
 
 
 def conv_hypotheses(cin, H, w_size, cout_known, n_written):
+    seen = set()
     for groups in (1, cin):
         for kk in (1, 3, 5, 7, 11):
             per = (cin // groups) * kk * kk
@@ -43,7 +63,8 @@ def conv_hypotheses(cin, H, w_size, cout_known, n_written):
             for s in (1, 2, 4):
                 for p in range(kk // 2 + 1):
                     Ho = (H + 2 * p - kk) // s + 1
-                    if Ho >= 1 and cout * Ho * Ho == n_written:
+                    if Ho >= 1 and cout * Ho * Ho == n_written and (cout, groups, kk, s, p) not in seen:
+                        seen.add((cout, groups, kk, s, p))
                         yield cout, groups, kk, s, p
 
 
@@ -51,6 +72,7 @@ def derive(name):
     path = os.path.join(HERE, name + ".json")
     model = json.load(open(path))
     roles = json.load(open(os.path.join(HERE, name + "_kernel_roles.json")))
+    params = set(legacy.param_storages(model).values())
     exe = B.Executor(B.BASE)
     exe.load(path, os.path.join(ROOT, "oracle", "_ref", name + ".raw.co"))
     rng = np.random.default_rng(224)
@@ -60,74 +82,108 @@ def derive(name):
     table = {}
     for kidx, k in enumerate(model["kernels"]):
         kname, a = k["name"], k["args"]
+        pname = plain(kname)
         new = kname not in table
-        if kname.startswith("fused_nn_conv2d"):
+        if pname.startswith("fused_nn_conv2d"):
             cin, H, W = shape[a[0]]
             if new:
+                ep = EPILOGUE[family(kname)]
                 ops, out, n = T.run_reference_kernel(exe, model, roles, kidx, rng)
-                x, w, bias = ops["placeholder"], ops["placeholder1"], ops.get("placeholder2")
-                relu = "nn_relu" in kname
+                x, w = ops["placeholder"], ops["placeholder1"]
+                extra = [(ops[r], s_idx in params) for r, s_idx in zip(roles[kname], a)
+                         if r.startswith("placeholder") and r not in ("placeholder", "placeholder1")]
+                small = [e for e, is_param in extra if is_param]
+                full = [e for e, is_param in extra if not is_param]
+                assert (len(full), len(small)) == {"none": (0, 0), "relu": (0, 0), "residual": (1, 0),
+                                                   "bias_relu": (0, 1), "residual_bias_relu": (1, 1),
+                                                   "residual_scale_shift_relu": (1, 2)}[ep], (kname, ep)
+                relu = ep.endswith("relu")
                 hits = []
-                for cout, groups, kk, s, p in conv_hypotheses(cin, H, w.size, bias.size if bias is not None else 0, n):
-                    want = O.conv2d(x[:cin * H * W].reshape(cin, H, W), w.reshape(cout, cin // groups, kk, kk),
-                                    bias=bias, stride=(s, s), pad=(p, p), groups=groups, act=1 if relu else 0,
-                                    acc64=True)
+                for cout, groups, kk, s, p in conv_hypotheses(cin, H, w.size, small[0].size if small else 0, n):
+                    Ho = (H + 2 * p - kk) // s + 1
+                    kw = dict(stride=(s, s), pad=(p, p), groups=groups, act=1 if relu else 0, acc64=True)
+                    if full:
+                        kw["residual"] = full[0][:cout * Ho * Ho].reshape(cout, Ho, Ho)
+                    if ep == "residual_scale_shift_relu":
+                        kw.update(scale=small[0], shift=small[1])
+                    elif small:
+                        kw["bias"] = small[0]
+                    want = O.conv2d(x[:cin * H * W].reshape(cin, H, W), w.reshape(cout, cin // groups, kk, kk), **kw)
                     if T.close(out[:n], want):
                         hits.append((cout, groups, kk, s, p))
                 assert len(hits) == 1, (kname, hits)
                 cout, groups, kk, s, p = hits[0]
                 if groups > 1:
-                    assert bias is not None and relu
+                    assert ep == "bias_relu", kname
                     table[kname] = {"op": "dwconv2d", "c": cin, "h": H, "w": W, "k": kk, "stride": s, "pad": p,
                                     "bias": True, "act": 1, "witness": True}
                 else:
-                    ep = ("bias_relu" if relu else "bias") if bias is not None else ("relu" if relu else "none")
-                    assert ep != "bias", kname
                     table[kname] = {"op": "conv2d", "cin": cin, "h": H, "w": W, "cout": cout, "k": kk, "stride": s,
                                     "pad": p, "epilogue": ep, "witness": True}
-                print("%-44s %s" % (kname, table[kname]), flush=True)
+                print("%-60s %s" % (kname, table[kname]), flush=True)
             e = table[kname]
             C = e["c"] if e["op"] == "dwconv2d" else e["cout"]
             assert (e["h"], e["w"]) == (H, W) and (e.get("cin", e.get("c")) == cin), kname
             Ho = (H + 2 * e["pad"] - e["k"]) // e["stride"] + 1
             shape[a[2]] = (C, Ho, Ho)
-        elif kname.startswith("fused_nn_max_pool2d"):               # (in, out)
+        elif pname.startswith("fused_add"):                         # (out, in, per-channel shift)
+            C, H, W = shape[a[1]]
+            assert size(a[2]) == C, kname
+            if new:
+                act = 1 if "nn_relu" in pname else 0
+                ops, out, n = T.run_reference_kernel(exe, model, roles, kidx, rng)
+                assert n == C * H * W, kname
+                want = O.eltwise(ops["placeholder"][:n].reshape(C, H * W), shift=ops["placeholder1"], act=act)
+                assert T.close(out[:n], want), kname
+                table[kname] = {"op": "eltwise", "c": C, "inner": H * W, "shift": True, "act": act, "witness": True}
+                print("%-60s %s" % (kname, table[kname]), flush=True)
+            assert table[kname]["c"] == C and table[kname]["inner"] == H * W, kname
+            shape[a[0]] = (C, H, W)
+        elif pname.startswith(("fused_nn_max_pool2d", "fused_nn_avg_pool2d")):   # (in, out[, bias])
             C, H, W = shape[a[0]]
             if new:
+                mode = 0 if "max_pool" in pname else 1
+                with_bias = "_add_nn_relu" in pname
+                assert len(a) == (3 if with_bias else 2) and (not with_bias or size(a[2]) == C), kname
                 ops, out, n = T.run_reference_kernel(exe, model, roles, kidx, rng)
                 x = ops["placeholder"][:C * H * W].reshape(C, H, W)
                 hits = []
-                for kk, s, p in ((3, 2, 0), (3, 2, 1), (2, 2, 0), (3, 1, 1)):
+                for kk, s, p in ((3, 2, 0), (3, 2, 1), (2, 2, 0), (3, 1, 1), (H, 1, 0)):
                     Ho = (H + 2 * p - kk) // s + 1
-                    if C * Ho * Ho == n and T.close(out[:n], O.pool2d(x, (kk, kk), (s, s), (p, p), 0)):
+                    if C * Ho * Ho != n or (kk, s, p) in hits:
+                        continue
+                    want = O.pool2d(x, (kk, kk), (s, s), (p, p), mode,
+                                    bias=ops["placeholder1"] if with_bias else None, act=1 if with_bias else 0)
+                    if T.close(out[:n], want):
                         hits.append((kk, s, p))
                 assert len(hits) == 1, (kname, hits)
                 kk, s, p = hits[0]
                 table[kname] = {"op": "pool2d", "c": C, "h": H, "w": W, "k": kk, "stride": s, "pad": p,
-                                "mode": "max", "bias": False, "act": 0, "witness": True}
-                print("%-44s %s" % (kname, table[kname]), flush=True)
+                                "mode": "max" if mode == 0 else "avg", "bias": with_bias,
+                                "act": 1 if with_bias else 0, "witness": True}
+                print("%-60s %s" % (kname, table[kname]), flush=True)
             e = table[kname]
             Ho = (H + 2 * e["pad"] - e["k"]) // e["stride"] + 1
             shape[a[1]] = (C, Ho, Ho)
-        elif kname.startswith("fused_nn_global_avg_pool2d"):        # (in, out)
+        elif pname.startswith("fused_nn_global_avg_pool2d"):        # (in, out)
             C, H, W = shape[a[0]]
             if new:
                 ops, out, n = T.run_reference_kernel(exe, model, roles, kidx, rng)
                 assert n == C and T.close(out[:n], O.global_avgpool(ops["placeholder"][:C * H * W].reshape(C, H * W)))
                 table[kname] = {"op": "global_avgpool", "c": C, "hw": H * W, "witness": True}
             shape[a[1]] = (C, 1, 1)
-        elif kname.startswith("fused_nn_batch_flatten"):            # (out, in)
+        elif pname.startswith("fused_nn_batch_flatten"):            # (out, in)
             C, H, W = shape[a[1]]
             if new:
                 ops, out, n = T.run_reference_kernel(exe, model, roles, kidx, rng)
                 assert n == C * H * W and np.array_equal(out[:n], ops["placeholder"][:n])
                 table[kname] = {"op": "copy", "n": n, "witness": True}
             shape[a[0]] = (C * H * W, 1, 1)
-        elif kname.startswith("fused_nn_dense_add"):                # (x, W, out, bias)
+        elif pname.startswith("fused_nn_dense_add"):                # (x, W, out, bias)
             in_f, out_f = shape[a[0]][0], size(a[3])
             assert size(a[1]) == in_f * out_f
             if new:
-                relu = "nn_relu" in kname
+                relu = "nn_relu" in pname
                 ints = {}
                 for pn, s_idx in zip(roles[kname], a):
                     if pn.startswith("placeholder"):
@@ -140,7 +196,7 @@ def derive(name):
                 table[kname] = {"op": "dense", "in": in_f, "out": out_f, "bias": True, "act": 1 if relu else 0,
                                 "witness": True}
             shape[a[2]] = (out_f, 1, 1)
-        elif kname.startswith("fused_nn_softmax"):                  # (in, out)
+        elif pname.startswith("fused_nn_softmax"):                  # (in, out)
             table.setdefault(kname, {"op": "softmax", "rows": 1, "cols": shape[a[0]][0], "witness": False})
             shape[a[1]] = shape[a[0]]
         else:

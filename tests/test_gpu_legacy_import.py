@@ -1,5 +1,6 @@
 """The imported reference graphs on this build's kernels against the reference's OWN kernels
-(resource/resnet152 at 64 x 64 below; resource/mobilenet and resource/alexnet at the end).
+(resource/resnet152 at 64 x 64 below; resource/mobilenet, resource/alexnet and resource/vgg at
+the end).
 
 Two executors hold the reference's resource/resnet152 graph (tests/golden/resnet152.json) with the
 same seeded parameters and the same input: one launches the reference's generated kernels
@@ -94,15 +95,18 @@ def test_imported_resnet152_tracks_the_reference_kernels_call_by_call(tmp_path):
     ours.close()
 
 
-@pytest.mark.parametrize("name,calls,no_witness", [
-    ("mobilenet", 31, ("fused_nn_dense_add_kernel0", "fused_nn_softmax_kernel0")),
-    ("alexnet", 13, ("fused_nn_dense_add_nn_relu_1_kernel0", "fused_nn_dense_add_nn_relu_kernel0",
-                     "fused_nn_dense_add_kernel0", "fused_nn_softmax_kernel0")),
+@pytest.mark.parametrize("name,side,calls,no_witness", [
+    ("mobilenet", 224, 31, ("fused_nn_dense_add_kernel0", "fused_nn_softmax_kernel0")),
+    ("alexnet", 224, 13, ("fused_nn_dense_add_nn_relu_1_kernel0", "fused_nn_dense_add_nn_relu_kernel0",
+                          "fused_nn_dense_add_kernel0", "fused_nn_softmax_kernel0")),
+    ("vgg", 64, 71, ("tvmgen_default_fused_nn_dense_add_kernel0", "tvmgen_default_fused_nn_softmax_kernel0")),
 ])
-def test_imported_chain_models_track_the_reference_kernels_call_by_call(name, calls, no_witness, tmp_path):
+def test_imported_walked_models_track_the_reference_kernels_call_by_call(name, side, calls, no_witness, tmp_path):
     """resource/mobilenet (MobileNet v1: a 3x3 stem, 13 depthwise + 13 pointwise convolutions) and
     resource/alexnet (11x11 stride 4, 5x5, 3x3 convolutions without bias, plain max-pools, three
-    dense layers) at 224 x 224, the reference's kernels from oracle/_ref/<model>.raw.co.  Both
+    dense layers) at 224 x 224, resource/vgg (despite the name a pre-activation ResNet-50: all 69
+    calls before the classifier, every residual family, none of them broken) at 64 x 64, the
+    reference's kernels from oracle/_ref/<model>.raw.co.  Both
     executors run free from the input to the classifier; the dense and softmax kernels of the
     reference are no witnesses (int shuffle, see tests/test_gpu_reference_kernels.py), there the
     reference executor takes over this build's result."""
@@ -116,7 +120,7 @@ def test_imported_chain_models_track_the_reference_kernels_call_by_call(name, ca
     g.write(d)
     params = legacy.seeded_params(ref_json)
     MB.write_params(os.path.join(d, name + ".param"), params)
-    x = nets.image_input("legacy", (3, 224, 224))
+    x = nets.image_input("legacy", (3, side, side))
 
     theirs = B.Executor(B.BASE)
     theirs.load(ref_json, co)

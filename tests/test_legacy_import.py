@@ -1,9 +1,9 @@
 """The importer for the reference's own model directories (reef_amd/legacy.py) on the reference's
-resource/resnet152, resource/mobilenet and resource/alexnet graphs (tests/golden/<model>.json,
-data fixtures): same storages, same call
+resource/resnet152, resource/mobilenet, resource/alexnet and resource/vgg graphs
+(tests/golden/<model>.json, data fixtures): same storages, same call
 order, and the imported graph computes what the reference's kernels compute according to the
 table of shapes that was derived by running those kernels (tests/golden/make_resnet152_shapes.py,
-make_chain_shapes.py).
+make_graph_shapes.py).
 
 The CPU check interprets the reference graph DIRECTLY from the table with the oracle's ops and
 compares that with the imported model run through the executor (fake backend) -- two code paths
@@ -158,7 +158,8 @@ def test_import_refuses_a_table_that_does_not_fit_the_graph():
     assert legacy.load_table("resnet152") == table
 
 
-# ---- the chain-shaped directories: MobileNet v1 (depthwise convolutions) and AlexNet ----------
+# ---- the directories whose tables come from a walk of the graph: MobileNet v1 (depthwise
+# ---- convolutions), AlexNet, and `vgg` (in fact a pre-activation ResNet-50 at 64 x 64) ---------
 def golden(name, what=""):
     return os.path.join(HERE, "golden", name + what + ".json")
 
@@ -166,8 +167,10 @@ def golden(name, what=""):
 @pytest.mark.parametrize("name,calls,ops", [
     ("mobilenet", 31, {"reef_dwconv2d": 13, "reef_global_avgpool": 1, "reef_copy": 1, "reef_dense": 1, "reef_softmax": 1}),
     ("alexnet", 13, {"reef_pool2d": 3, "reef_copy": 1, "reef_dense": 3, "reef_softmax": 1}),
+    ("vgg", 71, {"reef_eltwise": 13, "reef_pool2d": 1, "reef_global_avgpool": 1, "reef_copy": 1, "reef_dense": 1,
+                 "reef_softmax": 1}),
 ])
-def test_chain_models_import_with_storages_order_and_keys(name, calls, ops, tmp_path):
+def test_walked_models_import_with_storages_order_and_keys(name, calls, ops, tmp_path):
     ref = json.load(open(golden(name)))
     g = legacy.import_model(golden(name))
     g.write(str(tmp_path))
@@ -186,18 +189,19 @@ def test_chain_models_import_with_storages_order_and_keys(name, calls, ops, tmp_
     assert sum(c for sym, c in count.items() if sym.startswith("reef_conv2d")) == calls - sum(ops.values())
     assert legacy.load_table(name) == json.load(open(golden(name, "_kernel_shapes")))
     # every entry but the softmax was reproduced by the oracle from the reference's own kernel
-    assert [k for k, e in legacy.load_table(name).items() if not e["witness"]] == ["fused_nn_softmax_kernel0"]
+    assert [k.replace("tvmgen_default_", "") for k, e in legacy.load_table(name).items()
+            if not e["witness"]] == ["fused_nn_softmax_kernel0"]
 
 
-def test_imported_mobilenet_equals_the_table_interpretation_through_the_executor(tmp_path):
-    name = "mobilenet"
+@pytest.mark.parametrize("name,side", [("mobilenet", 224), ("vgg", 64)])
+def test_imported_walked_model_equals_the_table_interpretation_through_the_executor(name, side, tmp_path):
     d = str(tmp_path)
     g = legacy.import_model(golden(name))
     g.write(d)
     params = legacy.seeded_params(golden(name))
     MB.write_params(os.path.join(d, name + ".param"), params)
     ref = json.load(open(golden(name)))
-    x = nets.image_input("legacy", (3, 224, 224))
+    x = nets.image_input("legacy", (3, side, side))
     want = interpret_reference_graph(ref, legacy.load_table(name), dict(params), x)
     fake = FakeHal().install()
     exe = None
