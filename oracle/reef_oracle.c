@@ -38,6 +38,11 @@
  *   the five fused convolution families once more on the 34 kernels of
  *     resource/vgg/vgg.cu (a pre-activation ResNet-50 at 64 x 64 whose stride-2
  *     bottleneck kernel is intact): all reproduced, 69 calls free-running.
+ *   3x3 convolution against the reference's Winograd pipeline (input
+ *     transform, GEMMs, inverse transform + epilogue; output tiles 4x4 and
+ *     2x2) on the 13 triples of resource/resnet18/resnet18.cu: the direct
+ *     convolution of a filter g equals the three kernels run on its transform,
+ *     to 1.5e-6; the whole ResNet-18 runs free beside them (29 comparisons).
  *   mocked add/multiply: the reference's closed form (3+3)*3 == 18, also on the
  *     reference's own mocked kernels.
  *   The reference's ResNet-18 ten-float golden vector needs a weight blob that

@@ -16,22 +16,70 @@ the same thing.  What a kernel name computes comes from a per-model table
 are those of the kernel families (convolution: in, W, out, then the epilogue operands in the
 order the family name lists them; depthwise convolution: in, W, out, bias; elementwise add and
 flatten: out first; pooling: in, out; dense: x, W, out, bias).  Tables are packaged for the
-reference's `resnet152`, `mobilenet`, `alexnet` and `vgg` directories (the last one holds a
-pre-activation ResNet-50 at 64 x 64 under TVM's `tvmgen_default_` kernel names).
+reference's `resnet152`, `mobilenet`, `alexnet`, `vgg` (which holds a pre-activation ResNet-50 at
+64 x 64 under TVM's `tvmgen_default_` kernel names) and `resnet18` directories.
 While it rewrites, the importer follows the tensor shapes through the graph and refuses a table
 that does not fit the graph.
+
+Winograd convolutions.  TVM compiles some 3x3 stride-1 convolutions as three calls
+(`fused_nn_contrib_conv2d_winograd_without_weight_transform*_kernel0/1/2`: transform of the input
+tiles, one GEMM per transform point, inverse transform + epilogue) through two scratch storages,
+and stores their weights TRANSFORMED: U[e][n][ci][co] = sum_rs G[e][r] g[co][ci][r][s] G[n][s],
+(t+2)^2 values per filter for output tiles of t x t.  The importer replaces such a triple by one
+direct convolution on the first call's input (the calls 0 and 1 get no counterpart; the scratch
+storages stay, unused), whose weights live in an added storage `<key>_direct`; `convert_params`
+recovers g from a parameter file's U (least squares through G's pseudo-inverse: exact for a U
+that is a transform).  G is the Cook-Toom matrix of TVM's interpolation points, which the
+reference does not vendor; it is pinned by running the reference's three kernels on a U made with
+it against the direct convolution (tests/golden/make_graph_shapes.py).
 """
 import json
 import os
+import struct
+
+import numpy as np
 
 from .modelgen import builder as MB
 from .modelgen.builder import Tensor
 
 TABLE_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "legacy_tables")
 
+# interpolation points of F(t x t, 3 x 3), the point at infinity comes last
+WINOGRAD_POINTS = {2: (0.0, -1.0, 1.0), 4: (0.0, -1.0, 1.0, 0.5, -2.0)}
+
 
 class ImportError_(ValueError):
     pass
+
+
+def winograd_G(tile):
+    """(tile + 2) x 3 filter transform: row i = (1, a_i, a_i^2) / prod_{k != i} (a_i - a_k) for the
+    finite points (the first row's sign made positive), (0, 0, 1) for the point at infinity."""
+    a = WINOGRAD_POINTS[tile]
+    alpha = tile + 2
+    G = np.zeros((alpha, 3))
+    for i in range(alpha - 1):
+        f = 1.0
+        for k in range(alpha - 1):
+            if k != i:
+                f *= a[i] - a[k]
+        if i == 0 and f < 0:
+            f = -f
+        G[i] = [1.0 / f, a[i] / f, a[i] * a[i] / f]
+    G[alpha - 1] = (0.0, 0.0, 1.0)
+    return G
+
+
+def winograd_transform(g, tile):
+    """g [Cout][Cin][3][3] -> U [t+2][t+2][Cin][Cout], float32 (computed in float64)."""
+    G = winograd_G(tile)
+    return np.einsum("er,oirs,ns->enio", G, np.asarray(g, np.float64), G).astype(np.float32)
+
+
+def winograd_untransform(U, tile):
+    """U [t+2][t+2][Cin][Cout] -> g [Cout][Cin][3][3]: the least-squares solution of U = G g G^T."""
+    P = np.linalg.pinv(winograd_G(tile))
+    return np.einsum("re,enio,sn->oirs", P, np.asarray(U, np.float64), P).astype(np.float32)
 
 
 def load_table(model_name):
@@ -63,9 +111,13 @@ def import_model(ref_json_path, table=None, name=None, input_shape=None):
             raise ImportError_("cannot tell the input shape from %d elements; pass input_shape" % n0)
         input_shape = (3, side, side)
     shape = {0: tuple(input_shape)}
+    wino = {}               # scratch storage -> {"in": input storage[, "U": transformed weights]}
+    g.direct_weights = {}   # key of a transformed weight -> (key of its direct copy, tile, Cout, Cin)
+    direct_idx = {}
+    g.imported_calls = []   # per kernel of this graph: the index of the reference call it replaces
 
     def size(i):
-        return ref["storage"][i]["size"]
+        return g.storage[i]["size"]
 
     def need(cond, kernel, what):
         if not cond:
@@ -78,12 +130,32 @@ def import_model(ref_json_path, table=None, name=None, input_shape=None):
         need(n <= size(i), kernel, "storage %d holds %d elements, the table asks for %s" % (i, size(i), shp))
         return Tensor(i, shp)
 
-    for k in ref["kernels"]:
+    for call, k in enumerate(ref["kernels"]):
         kname, a = k["name"], k["args"]
         e = table.get(kname)
         need(e is not None, k, "not in the table")
         op = e["op"]
-        if op == "conv2d":
+        first_new = len(g.kernels)
+        if op == "winograd_data":                               # (in, V)
+            need(len(a) == 2 and a[0] in shape, k, "input storage has no shape yet")
+            wino[a[1]] = {"in": a[0]}
+        elif op == "winograd_gemm":                             # (U, V, M)
+            need(len(a) == 3 and a[1] in wino, k, "no transformed input reaches this call")
+            wino[a[2]] = dict(wino.pop(a[1]), U=a[0])
+        elif op == "conv2d":
+            tile = e.get("winograd_tile")
+            if tile:                                            # (M, out, epilogue operands)
+                need(len(a) >= 2 and "U" in wino.get(a[0], ()), k, "no transformed operands reach this call")
+                need((e["k"], e["stride"], e["pad"]) == (3, 1, 1), k, "a Winograd entry is a 3x3 stride-1 filter")
+                src = wino.pop(a[0])
+                alpha = tile + 2
+                need(size(src["U"]) == alpha * alpha * e["cin"] * e["cout"], k, "transformed weight storage size")
+                if src["U"] not in direct_idx:
+                    key = ref["storage"][src["U"]]["name"]
+                    direct_idx[src["U"]] = g._storage(key + "_direct", e["cout"] * e["cin"] * 9)
+                    g.graph_args.append(direct_idx[src["U"]])
+                    g.direct_weights[key] = (key + "_direct", tile, e["cout"], e["cin"])
+                a = [src["in"], direct_idx[src["U"]], a[1]] + list(a[2:])
             need(len(a) >= 3 and a[0] in shape, k, "input storage has no shape yet")
             need(shape[a[0]] == (e["cin"], e["h"], e["w"]), k,
                  "table says input %s, the graph delivers %s" % ((e["cin"], e["h"], e["w"]), shape[a[0]]))
@@ -168,20 +240,59 @@ def import_model(ref_json_path, table=None, name=None, input_shape=None):
             shape[a[1]] = shape[a[0]]
         else:
             need(False, k, "unknown op " + op)
+        g.imported_calls += [call] * (len(g.kernels) - first_new)
+    need(not wino, ref["kernels"][-1], "a Winograd transform without its last call")
     g.imported_from = [k["name"] for k in ref["kernels"]]
     return g
+
+
+def read_params(path):
+    """[(key, float32 array)] of a `.param` file (reader src/reef/executor/model.cpp:82-121)."""
+    with open(path, "rb") as f:
+        blob = f.read()
+    if blob[:17] != b"TVM_MODEL_PARAMS\0":
+        raise ImportError_("%s is not a parameter file" % path)
+    (count,), pos, out = struct.unpack_from("<Q", blob, 17), 25, []
+    for _ in range(count):
+        end = blob.index(b"\0", pos)
+        key = blob[pos:end].decode("ascii")
+        (n,) = struct.unpack_from("<Q", blob, end + 1)
+        out.append((key, np.frombuffer(blob, "<f4", n, end + 9).copy()))
+        pos = end + 9 + 4 * n
+    return out
+
+
+def convert_params(g, params):
+    """Parameters of the reference graph -> parameters of the imported graph `g`: unchanged, except
+    that a transformed Winograd weight is replaced by the direct weight recovered from it."""
+    out = []
+    for key, arr in params:
+        if key in g.direct_weights:
+            dkey, tile, cout, cin = g.direct_weights[key]
+            alpha = tile + 2
+            if arr.size != alpha * alpha * cin * cout:
+                raise ImportError_("parameter %s holds %d values, the table asks for %d"
+                                   % (key, arr.size, alpha * alpha * cin * cout))
+            out.append((dkey, winograd_untransform(arr.reshape(alpha, alpha, cin, cout), tile).ravel()))
+        else:
+            out.append((key, arr))
+    return out
 
 
 def import_model_dir(ref_dir, model_name, out_dir, table=None, measured_profile=False):
     """<ref_dir>/<model>.json (+ .param if present) -> a model directory of this build in out_dir.
     Returns the GraphBuilder.  A `.param` file of the reference is taken over byte for byte (same
-    keys, same storages); the profile is the estimate unless measured_profile (needs a GPU)."""
+    keys, same storages) unless the graph has Winograd weights, which are converted
+    (convert_params); the profile is the estimate unless measured_profile (needs a GPU)."""
     import shutil
     g = import_model(os.path.join(ref_dir, model_name + ".json"), table=table, name=model_name)
     g.write(out_dir)
     src = os.path.join(ref_dir, model_name + ".param")
     if os.path.exists(src):
-        shutil.copyfile(src, os.path.join(out_dir, model_name + ".param"))
+        if g.direct_weights:
+            MB.write_params(os.path.join(out_dir, model_name + ".param"), convert_params(g, read_params(src)))
+        else:
+            shutil.copyfile(src, os.path.join(out_dir, model_name + ".param"))
     if measured_profile:
         from . import profiler
         profiler.write_profile(out_dir, model_name)
@@ -211,9 +322,18 @@ def seeded_params(ref_json_path, table=None, seed=0x5EEF):
         table = json.load(open(table))
     std = {}
     one_plus = set()
+    transformed = {}                   # storage of a Winograd weight -> (tile, Cout, Cin)
+    gemm_of = {}                       # scratch storage a Winograd GEMM wrote -> its weight storage
     for k in ref["kernels"]:
         e, a = table[k["name"]], k["args"]
-        if e["op"] == "conv2d":
+        if e["op"] == "winograd_gemm":
+            gemm_of[a[2]] = a[0]
+        elif e["op"] == "conv2d" and e.get("winograd_tile"):
+            transformed[gemm_of[a[0]]] = (e["winograd_tile"], e["cout"], e["cin"])
+            if e["epilogue"] == "residual_scale_shift_relu":
+                std[a[3]] = 0.1
+                one_plus.add(a[3])
+        elif e["op"] == "conv2d":
             std[a[1]] = math.sqrt(2.0 / (e["cin"] * e["k"] * e["k"]))
             if e["epilogue"] == "residual_scale_shift_relu":
                 std[a[4]] = 0.1
@@ -227,6 +347,11 @@ def seeded_params(ref_json_path, table=None, seed=0x5EEF):
     for i, s in enumerate(ref["storage"]):
         name = s["name"]
         if i not in params:
+            continue
+        if i in transformed:           # a seeded direct weight, stored the way the reference stores it
+            tile, cout, cin = transformed[i]
+            direct = rng.normal_f32(model_name + "/" + name, cout * cin * 9, math.sqrt(2.0 / (cin * 9)), seed)
+            out.append((name, winograd_transform(direct.reshape(cout, cin, 3, 3), tile).ravel()))
             continue
         arr = rng.normal_f32(model_name + "/" + name, s["size"], std.get(i, 0.01), seed)
         if i in one_plus:

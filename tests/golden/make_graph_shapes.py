@@ -5,6 +5,9 @@ walked from the input with every kernel witnessed on the way:
   alexnet    11x11 / 5x5 / 3x3 convolutions without bias, plain max-pools, three dense layers
   vgg        despite its name a pre-activation ResNet-50 at 64 x 64 (kernel names carry TVM's
              `tvmgen_default_` prefix): the residual families of resnet152
+  resnet18   pre-activation ResNet-18 at 224 x 224 whose 3x3 stride-1 convolutions are Winograd
+             triples (kernel0: input transform, kernel1: GEMMs, kernel2: inverse transform +
+             epilogue) on TRANSFORMED weights
 
 For every kernel name: what it computes -- op, shape, filter, stride, padding, epilogue.  The
 shapes are baked into the generated source and the graph JSON only holds shared, maximal buffer
@@ -18,7 +21,13 @@ residual when the operand is a tensor of the graph, bias when it is a parameter)
 are run on small non-negative integers and softmax has no witness, for the reason given in the
 module docstring of tests/test_gpu_reference_kernels.py.
 
-Needs a GPU:  python tests/golden/make_graph_shapes.py mobilenet|alexnet|vgg
+A Winograd triple is witnessed as one: a random direct filter g is transformed with
+reef_amd.legacy.winograd_transform (output tile 4 or 2, weight layout [e][n][Cin][Cout] or
+[e][n][Cout][Cin]), the reference's three kernels run on it, and exactly one hypothesis must give
+what the oracle's DIRECT convolution of g gives (to 1e-4 of the largest output: two summation
+orders and the transform's own rounding).  That pins the transform matrix the importer inverts.
+
+Needs a GPU:  python tests/golden/make_graph_shapes.py mobilenet|alexnet|vgg|resnet18
 The result is committed as tests/golden/<model>_kernel_shapes.json (fixture) and as
 reef_amd/legacy_tables/<model>.json (the importer's table for that model directory)."""
 import json
@@ -36,6 +45,7 @@ from reef_amd import binding as B                                # noqa: E402
 from reef_amd import legacy                                      # noqa: E402
 from tests import test_gpu_reference_kernels as T                # noqa: E402
 
+WINO = "fused_nn_contrib_conv2d_winograd_without_weight_transform"
 EPILOGUE = {"fused_nn_conv2d": "none", "fused_nn_conv2d_nn_relu": "relu",
             "fused_nn_conv2d_add": "residual", "fused_nn_conv2d_add_nn_relu": "bias_relu",
             "fused_nn_conv2d_add_add_nn_relu": "residual_bias_relu",
@@ -48,6 +58,66 @@ def plain(name):
 
 def family(name):
     return plain(name).split("_kernel0")[0].rstrip("0123456789").rstrip("_")
+
+
+def winograd_family(name):
+    """Epilogue family of a Winograd kernel2 name, as the direct convolutions spell it.  TVM cuts
+    long names and appends a hash (`..._add_multiply_add_nn_re_<digits>__kernel2`)."""
+    rest = plain(name)[len(WINO):].split("_kernel")[0].rstrip("_")
+    if rest.startswith("_add_multiply_add_nn_re"):
+        return "fused_nn_conv2d_add_multiply_add_nn_relu"
+    return "fused_nn_conv2d" + rest.rstrip("0123456789").rstrip("_")
+
+
+def witness_winograd(exe, model, roles, params, src, kidx, cin, H, W, rng):
+    """Runs the triple (src["k0"], src["k1"], kidx) under every hypothesis; returns the table entry."""
+    k = model["kernels"][kidx]
+    kname, a = k["name"], k["args"]
+    size = lambda i: model["storage"][i]["size"]
+    ep = EPILOGUE[winograd_family(kname)]
+    relu = ep.endswith("relu")
+    names = roles[kname]
+    assert names[0] == "bgemm" and names[1].startswith("T_") and all(n.startswith("placeholder") for n in names[2:]), names
+    hits = []
+    for tile in (4, 2):
+        alpha = tile + 2
+        if size(src["U"]) % (alpha * alpha * cin):
+            continue
+        cout = size(src["U"]) // (alpha * alpha * cin)
+        for layout in ("enio", "enoi"):
+            g = (rng.standard_normal((cout, cin, 3, 3)) * np.sqrt(2.0 / (cin * 9))).astype(np.float32)
+            U = legacy.winograd_transform(g, tile)
+            T._set(exe, model, src["U"], U if layout == "enio" else U.transpose(0, 1, 3, 2))
+            x = T._set(exe, model, src["in"], rng.standard_normal(size(src["in"])).astype(np.float32))
+            small, full = [], []
+            for s_idx in a[2:]:
+                v = T._set(exe, model, s_idx, rng.standard_normal(size(s_idx)).astype(np.float32))
+                (small if s_idx in params else full).append(v)
+            T._set(exe, model, a[1], np.full(size(a[1]), T.SENTINEL, np.float32))
+            for i in (src["k0"], src["k1"], kidx):
+                exe.execute_kernel(i)
+            out = exe.get_data(a[1], size(a[1]))
+            written = np.nonzero(out != T.SENTINEL)[0]
+            n = int(written.max()) + 1 if written.size else 0
+            if n != cout * H * W or written.size != n or (small and small[0].size != cout):
+                continue
+            kw = dict(stride=(1, 1), pad=(1, 1), act=1 if relu else 0, acc64=True)
+            if full:
+                kw["residual"] = full[0][:n].reshape(cout, H, W)
+            if ep == "residual_scale_shift_relu":
+                kw.update(scale=small[0], shift=small[1])
+            elif small:
+                kw["bias"] = small[0]
+            want = O.conv2d(x[:cin * H * W].reshape(cin, H, W), g, **kw)
+            dev = float(np.abs(out[:n] - want.ravel()).max()) / max(float(np.abs(want).max()), 1.0)
+            print("    tile %d layout %s: deviation %.2e" % (tile, layout, dev), flush=True)
+            if dev <= 1e-4:
+                hits.append((tile, layout, cout))
+    assert len(hits) == 1, (kname, hits)
+    tile, layout, cout = hits[0]
+    assert layout == "enio", "the importer assumes [e][n][Cin][Cout]"
+    return {"op": "conv2d", "cin": cin, "h": H, "w": W, "cout": cout, "k": 3, "stride": 1, "pad": 1,
+            "epilogue": ep, "winograd_tile": tile, "witness": True}
 
 
 def conv_hypotheses(cin, H, w_size, cout_known, n_written):
@@ -80,11 +150,28 @@ def derive(name):
     side = int(round((size(0) // 3) ** 0.5))
     shape = {0: (3, side, side)}
     table = {}
+    wino = {}
     for kidx, k in enumerate(model["kernels"]):
         kname, a = k["name"], k["args"]
         pname = plain(kname)
         new = kname not in table
-        if pname.startswith("fused_nn_conv2d"):
+        if pname.startswith(WINO) and pname.endswith("_kernel0"):      # (in, V)
+            wino[a[1]] = {"in": a[0], "k0": kidx}
+            table.setdefault(kname, {"op": "winograd_data", "witness": True})
+        elif pname.startswith(WINO) and pname.endswith("_kernel1"):    # (U, V, M)
+            wino[a[2]] = dict(wino.pop(a[1]), U=a[0], k1=kidx)
+            table.setdefault(kname, {"op": "winograd_gemm", "witness": True})
+        elif pname.startswith(WINO):                                    # (M, out, epilogue operands)
+            src = wino.pop(a[0])
+            cin, H, W = shape[src["in"]]
+            if new:
+                print(kname, flush=True)
+                table[kname] = witness_winograd(exe, model, roles, params, src, kidx, cin, H, W, rng)
+                print("%-60s %s" % (kname, table[kname]), flush=True)
+            e = table[kname]
+            assert (e["cin"], e["h"], e["w"]) == (cin, H, W), kname
+            shape[a[1]] = (e["cout"], H, W)
+        elif pname.startswith("fused_nn_conv2d"):
             cin, H, W = shape[a[0]]
             if new:
                 ep = EPILOGUE[family(kname)]

@@ -33,15 +33,27 @@ def interpret_reference_graph(ref, table, params, x, upto=None):
         if s["name"] in params:
             st[i][:] = params[s["name"]]
     st[0][:] = x.ravel()
+    wino = {}
     for n, k in enumerate(ref["kernels"]):
         if upto is not None and n >= upto:
             break
         e, a = table[k["name"]], k["args"]
-        if e["op"] == "conv2d":
+        if e["op"] == "winograd_data":
+            wino[a[1]] = (a[0], None)
+        elif e["op"] == "winograd_gemm":
+            wino[a[2]] = (wino.pop(a[1])[0], a[0])
+        elif e["op"] == "conv2d":
             cin, H, W, cout, kk, s, p = e["cin"], e["h"], e["w"], e["cout"], e["k"], e["stride"], e["pad"]
             Ho = (H + 2 * p - kk) // s + 1
+            if e.get("winograd_tile"):
+                # three calls of the reference = one direct convolution on the un-transformed filter
+                alpha = e["winograd_tile"] + 2
+                src, u = wino.pop(a[0])
+                ws = legacy.winograd_untransform(st[u].reshape(alpha, alpha, cin, cout), e["winograd_tile"])
+                a = [src, u, a[1]] + list(a[2:])
+            else:
+                ws = st[a[1]].reshape(cout, cin, kk, kk)
             xs = st[a[0]][:cin * H * W].reshape(cin, H, W)
-            ws = st[a[1]].reshape(cout, cin, kk, kk)
             full = lambda i: st[i][:cout * Ho * Ho].reshape(cout, Ho, Ho)
             kw = dict(stride=(s, s), pad=(p, p))
             ep = e["epilogue"]
@@ -193,13 +205,67 @@ def test_walked_models_import_with_storages_order_and_keys(name, calls, ops, tmp
             if not e["witness"]] == ["fused_nn_softmax_kernel0"]
 
 
-@pytest.mark.parametrize("name,side", [("mobilenet", 224), ("vgg", 64)])
+def test_winograd_filter_transform():
+    """F(2x2, 3x3) is the textbook transform (Lavin & Gray) up to the order of its points; both
+    tile sizes: transform then least-squares inverse gives the filter back, and the transform of a
+    filter that is 1 at the centre is the outer product of G's middle column with itself."""
+    G2 = legacy.winograd_G(2)
+    textbook = [[1, 0, 0], [0.5, 0.5, 0.5], [0.5, -0.5, 0.5], [0, 0, 1]]
+    assert sorted(map(tuple, G2.tolist())) == sorted(map(tuple, textbook))
+    rs = np.random.default_rng(3)
+    for tile in (2, 4):
+        G = legacy.winograd_G(tile)
+        assert G.shape == (tile + 2, 3) and np.linalg.matrix_rank(G) == 3
+        g = rs.standard_normal((5, 3, 3, 3)).astype(np.float32)
+        U = legacy.winograd_transform(g, tile)
+        assert U.shape == (tile + 2, tile + 2, 3, 5)
+        np.testing.assert_allclose(legacy.winograd_untransform(U, tile), g, rtol=0, atol=1e-6)
+        centre = np.zeros((1, 1, 3, 3), np.float32)
+        centre[0, 0, 1, 1] = 1
+        np.testing.assert_allclose(legacy.winograd_transform(centre, tile)[:, :, 0, 0], np.outer(G[:, 1], G[:, 1]),
+                                   rtol=0, atol=1e-7)
+
+
+def test_resnet18_import_replaces_winograd_triples_by_direct_convolutions(tmp_path):
+    """resource/resnet18: 57 calls, 13 of its convolutions as three calls each on transformed
+    weights (p4: 36 x 64 x 64 values for a 3x3 64 -> 64 filter).  Imported: 31 kernels, a storage
+    `<key>_direct` per transformed weight, the reference's storages untouched."""
+    name = "resnet18"
+    ref = json.load(open(golden(name)))
+    g = legacy.import_model(golden(name))
+    g.write(str(tmp_path))
+    out = json.load(open(os.path.join(str(tmp_path), name + ".json")))
+    n = len(ref["storage"])
+    assert out["storage"][:n] == ref["storage"]
+    added = [s for s in out["storage"][n:] if s["name"] not in ("temp_arg", "reef_sync")]
+    assert len(added) == 13 and all(s["name"].endswith("_direct") for s in added)
+    assert len(ref["kernels"]) == 57 and len(out["kernels"]) == 57 - 2 * 13 == len(g.imported_calls)
+    table = legacy.load_table(name)
+    skipped = [i for i, k in enumerate(ref["kernels"]) if table[k["name"]]["op"].startswith("winograd_")]
+    assert sorted(set(range(57)) - set(skipped)) == g.imported_calls
+    assert g.direct_weights["p4"] == ("p4_direct", 4, 64, 64)
+    assert sum(1 for e in table.values() if e.get("winograd_tile") == 2) == 9       # 28x28 and smaller
+    # parameters: a transformed weight of the reference's file comes back as the filter it was made from
+    params = legacy.seeded_params(golden(name))
+    MB.write_params(os.path.join(str(tmp_path), "ref.param"), params)
+    back = legacy.read_params(os.path.join(str(tmp_path), "ref.param"))
+    assert [k for k, _ in back] == [k for k, _ in params]
+    conv = dict(legacy.convert_params(g, back))
+    assert "p4" not in conv and conv["p4_direct"].size == 64 * 64 * 9 and dict(back)["p4"].size == 36 * 64 * 64
+    np.testing.assert_allclose(legacy.winograd_transform(conv["p4_direct"].reshape(64, 64, 3, 3), 4).ravel(),
+                               dict(back)["p4"], rtol=0, atol=1e-6)
+    with pytest.raises(legacy.ImportError_, match="p4"):
+        legacy.convert_params(g, [("p4", np.zeros(9 * 64 * 64, np.float32))])
+    assert legacy.load_table(name) == json.load(open(golden(name, "_kernel_shapes")))
+
+
+@pytest.mark.parametrize("name,side", [("mobilenet", 224), ("vgg", 64), ("resnet18", 224)])
 def test_imported_walked_model_equals_the_table_interpretation_through_the_executor(name, side, tmp_path):
     d = str(tmp_path)
     g = legacy.import_model(golden(name))
     g.write(d)
     params = legacy.seeded_params(golden(name))
-    MB.write_params(os.path.join(d, name + ".param"), params)
+    MB.write_params(os.path.join(d, name + ".param"), legacy.convert_params(g, params))
     ref = json.load(open(golden(name)))
     x = nets.image_input("legacy", (3, side, side))
     want = interpret_reference_graph(ref, legacy.load_table(name), dict(params), x)
