@@ -43,6 +43,10 @@
  *     2x2) on the 13 triples of resource/resnet18/resnet18.cu: the direct
  *     convolution of a filter g equals the three kernels run on its transform,
  *     to 1.5e-6; the whole ResNet-18 runs free beside them (29 comparisons).
+ *   1x7 / 7x1 / 1x3 / 3x1 / 5x5 convolutions, 3x3 stride-1 average pool that
+ *   counts its padding, unpadded Winograd, channel concatenation: the 75
+ *     kernels of resource/inception/inception.cu (Inception-v3 at 299 x 299),
+ *     the same way; 120 comparisons free-running, worst deviation 3.1e-6.
  *   mocked add/multiply: the reference's closed form (3+3)*3 == 18, also on the
  *     reference's own mocked kernels.
  *   The reference's ResNet-18 ten-float golden vector needs a weight blob that

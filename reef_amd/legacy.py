@@ -14,10 +14,11 @@ file of the reference loads unchanged), every call replaced by the `reef_*` kern
 the same thing.  What a kernel name computes comes from a per-model table
 (`legacy_tables/<model>.json`: name -> op, shape, stride, padding, epilogue); the argument roles
 are those of the kernel families (convolution: in, W, out, then the epilogue operands in the
-order the family name lists them; depthwise convolution: in, W, out, bias; elementwise add and
-flatten: out first; pooling: in, out; dense: x, W, out, bias).  Tables are packaged for the
+order the family name lists them; depthwise convolution: in, W, out, bias; elementwise add,
+flatten and concatenation: out first (TVM lists a concatenation's operands in an order of its own;
+the table says which operand comes first in the result); pooling: in, out; dense: x, W, out, bias).  Tables are packaged for the
 reference's `resnet152`, `mobilenet`, `alexnet`, `vgg` (which holds a pre-activation ResNet-50 at
-64 x 64 under TVM's `tvmgen_default_` kernel names) and `resnet18` directories.
+64 x 64 under TVM's `tvmgen_default_` kernel names), `resnet18` and `inception` directories.
 While it rewrites, the importer follows the tensor shapes through the graph and refuses a table
 that does not fit the graph.
 
@@ -50,6 +51,11 @@ WINOGRAD_POINTS = {2: (0.0, -1.0, 1.0), 4: (0.0, -1.0, 1.0, 0.5, -2.0)}
 
 class ImportError_(ValueError):
     pass
+
+
+def pair(v):
+    """Filter size / padding of a table entry: one number for a square one, [rows, columns] else."""
+    return (v, v) if isinstance(v, int) else (int(v[0]), int(v[1]))
 
 
 def winograd_G(tile):
@@ -146,7 +152,8 @@ def import_model(ref_json_path, table=None, name=None, input_shape=None):
             tile = e.get("winograd_tile")
             if tile:                                            # (M, out, epilogue operands)
                 need(len(a) >= 2 and "U" in wino.get(a[0], ()), k, "no transformed operands reach this call")
-                need((e["k"], e["stride"], e["pad"]) == (3, 1, 1), k, "a Winograd entry is a 3x3 stride-1 filter")
+                need((e["k"], e["stride"]) == (3, 1) and e["pad"] in (0, 1), k,
+                     "a Winograd entry is a 3x3 stride-1 filter")
                 src = wino.pop(a[0])
                 alpha = tile + 2
                 need(size(src["U"]) == alpha * alpha * e["cin"] * e["cout"], k, "transformed weight storage size")
@@ -159,12 +166,12 @@ def import_model(ref_json_path, table=None, name=None, input_shape=None):
             need(len(a) >= 3 and a[0] in shape, k, "input storage has no shape yet")
             need(shape[a[0]] == (e["cin"], e["h"], e["w"]), k,
                  "table says input %s, the graph delivers %s" % ((e["cin"], e["h"], e["w"]), shape[a[0]]))
-            kk, s, p, cout = e["k"], e["stride"], e["pad"], e["cout"]
-            Ho, Wo = (e["h"] + 2 * p - kk) // s + 1, (e["w"] + 2 * p - kk) // s + 1
-            need(size(a[1]) == cout * e["cin"] * kk * kk, k, "weight storage size")
+            (fh, fw), s, (ph, pw), cout = pair(e["k"]), e["stride"], pair(e["pad"]), e["cout"]
+            Ho, Wo = (e["h"] + 2 * ph - fh) // s + 1, (e["w"] + 2 * pw - fw) // s + 1
+            need(size(a[1]) == cout * e["cin"] * fh * fw, k, "weight storage size")
             ep = e["epilogue"]
             rest = a[3:]
-            given = {"w": Tensor(a[1], (cout, e["cin"], kk, kk))}
+            given = {"w": Tensor(a[1], (cout, e["cin"], fh, fw))}
             kw = dict(bias=False, act=MB.ACT_NONE, residual=None, affine=False)
             if ep == "bias_relu":
                 need(len(rest) == 1 and size(rest[0]) == cout, k, "bias operand")
@@ -190,7 +197,7 @@ def import_model(ref_json_path, table=None, name=None, input_shape=None):
                 need(ep == "none" and not rest, k, "unknown epilogue " + ep)
             # a residual read from the buffer the result goes to would not survive a restart
             need(kw["residual"] is None or kw["residual"].idx != a[2], k, "in-place residual")
-            g.conv2d(Tensor(a[0], shape[a[0]]), cout, kk, s, p, out=tensor(a[2], (cout, Ho, Wo), k),
+            g.conv2d(Tensor(a[0], shape[a[0]]), cout, (fh, fw), s, (ph, pw), out=tensor(a[2], (cout, Ho, Wo), k),
                      given=given, **kw)
             shape[a[2]] = (cout, Ho, Wo)
         elif op == "dwconv2d":                                  # (in, W, out, bias)
@@ -214,9 +221,21 @@ def import_model(ref_json_path, table=None, name=None, input_shape=None):
             need(a[0] in shape and shape[a[0]] == (e["c"], e["h"], e["w"]), k, "shape")
             out = g.pool2d(Tensor(a[0], shape[a[0]]), e["k"], e["stride"], e["pad"], mode=e["mode"],
                            bias=bool(e.get("bias")), act=e.get("act", 0), out=Tensor(a[1], (1,)),
+                           count_include_pad=bool(e.get("count_include_pad")),
                            bias_t=Tensor(a[2], (e["c"],)) if e.get("bias") else None)
             need(out.size <= size(a[1]), k, "output storage too small")
             shape[a[1]] = out.shape
+        elif op == "concat":                # (out, operands); `operand`: which of them comes first, second ...
+            H, W, parts = e["h"], e["w"], e["parts"]
+            need(len(a) == 1 + len(parts) and sorted(e["operand"]) == list(range(len(parts))), k,
+                 "as many operands as parts")
+            whole = tensor(a[0], (sum(parts), H, W), k)
+            off = 0
+            for c, i in zip(parts, [a[1 + j] for j in e["operand"]]):
+                need(shape.get(i) == (c, H, W) and i != a[0], k, "part %d: the graph delivers %s" % (i, shape.get(i)))
+                g.copy_into(Tensor(i, (c * H * W,)), whole, off)
+                off += c * H * W
+            shape[a[0]] = (sum(parts), H, W)
         elif op == "global_avgpool":                            # (in, out)
             C, H, W = shape[a[0]]
             need(C == e["c"] and H * W == e["hw"], k, "shape")
@@ -334,7 +353,7 @@ def seeded_params(ref_json_path, table=None, seed=0x5EEF):
                 std[a[3]] = 0.1
                 one_plus.add(a[3])
         elif e["op"] == "conv2d":
-            std[a[1]] = math.sqrt(2.0 / (e["cin"] * e["k"] * e["k"]))
+            std[a[1]] = math.sqrt(2.0 / (e["cin"] * pair(e["k"])[0] * pair(e["k"])[1]))
             if e["epilogue"] == "residual_scale_shift_relu":
                 std[a[4]] = 0.1
                 one_plus.add(a[4])

@@ -8,14 +8,16 @@ walked from the input with every kernel witnessed on the way:
   resnet18   pre-activation ResNet-18 at 224 x 224 whose 3x3 stride-1 convolutions are Winograd
              triples (kernel0: input transform, kernel1: GEMMs, kernel2: inverse transform +
              epilogue) on TRANSFORMED weights
+  inception  Inception-v3 at 299 x 299: 1x7 / 7x1 / 1x3 / 3x1 / 5x5 filters, Winograd triples with
+             and without padding, average pools, channel concatenations
 
 For every kernel name: what it computes -- op, shape, filter, stride, padding, epilogue.  The
 shapes are baked into the generated source and the graph JSON only holds shared, maximal buffer
 sizes, so every entry has a witness: the graph is walked from the input, each distinct kernel of
 oracle/_ref/<model>.raw.co (the reference's own <model>.cu compiled for gfx950, `make -C oracle
 ref`) is run once on random operands on the GPU, and of the hypotheses that are consistent with
-its operand sizes and with the number of elements it writes (groups 1 or depthwise, filter 1..11,
-stride 1/2/4, every padding up to half the filter) exactly one must make the CPU oracle reproduce
+its operand sizes and with the number of elements it writes (groups 1 or depthwise, square
+filters 1..11 and 1xk / kx1, stride 1/2/4, every padding up to half the filter) exactly one must make the CPU oracle reproduce
 its output.  The epilogue follows from the family name (resnet152.cu:315-363, 376-713, 2662: add =
 residual when the operand is a tensor of the graph, bias when it is a parameter).  Dense kernels
 are run on small non-negative integers and softmax has no witness, for the reason given in the
@@ -27,7 +29,7 @@ reef_amd.legacy.winograd_transform (output tile 4 or 2, weight layout [e][n][Cin
 what the oracle's DIRECT convolution of g gives (to 1e-4 of the largest output: two summation
 orders and the transform's own rounding).  That pins the transform matrix the importer inverts.
 
-Needs a GPU:  python tests/golden/make_graph_shapes.py mobilenet|alexnet|vgg|resnet18
+Needs a GPU:  python tests/golden/make_graph_shapes.py mobilenet|alexnet|vgg|resnet18|inception
 The result is committed as tests/golden/<model>_kernel_shapes.json (fixture) and as
 reef_amd/legacy_tables/<model>.json (the importer's table for that model directory)."""
 import json
@@ -84,7 +86,8 @@ def witness_winograd(exe, model, roles, params, src, kidx, cin, H, W, rng):
         if size(src["U"]) % (alpha * alpha * cin):
             continue
         cout = size(src["U"]) // (alpha * alpha * cin)
-        for layout in ("enio", "enoi"):
+        for layout, pad in (("enio", 1), ("enoi", 1), ("enio", 0), ("enoi", 0)):
+            Ho, Wo = H + 2 * pad - 2, W + 2 * pad - 2
             g = (rng.standard_normal((cout, cin, 3, 3)) * np.sqrt(2.0 / (cin * 9))).astype(np.float32)
             U = legacy.winograd_transform(g, tile)
             T._set(exe, model, src["U"], U if layout == "enio" else U.transpose(0, 1, 3, 2))
@@ -99,43 +102,54 @@ def witness_winograd(exe, model, roles, params, src, kidx, cin, H, W, rng):
             out = exe.get_data(a[1], size(a[1]))
             written = np.nonzero(out != T.SENTINEL)[0]
             n = int(written.max()) + 1 if written.size else 0
-            if n != cout * H * W or written.size != n or (small and small[0].size != cout):
+            if n != cout * Ho * Wo or written.size != n or (small and small[0].size != cout):
                 continue
-            kw = dict(stride=(1, 1), pad=(1, 1), act=1 if relu else 0, acc64=True)
+            kw = dict(stride=(1, 1), pad=(pad, pad), act=1 if relu else 0, acc64=True)
             if full:
-                kw["residual"] = full[0][:n].reshape(cout, H, W)
+                kw["residual"] = full[0][:n].reshape(cout, Ho, Wo)
             if ep == "residual_scale_shift_relu":
                 kw.update(scale=small[0], shift=small[1])
             elif small:
                 kw["bias"] = small[0]
             want = O.conv2d(x[:cin * H * W].reshape(cin, H, W), g, **kw)
             dev = float(np.abs(out[:n] - want.ravel()).max()) / max(float(np.abs(want).max()), 1.0)
-            print("    tile %d layout %s: deviation %.2e" % (tile, layout, dev), flush=True)
+            print("    tile %d layout %s pad %d: deviation %.2e" % (tile, layout, pad, dev), flush=True)
             if dev <= 1e-4:
-                hits.append((tile, layout, cout))
+                hits.append((tile, layout, cout, pad))
     assert len(hits) == 1, (kname, hits)
-    tile, layout, cout = hits[0]
+    tile, layout, cout, pad = hits[0]
     assert layout == "enio", "the importer assumes [e][n][Cin][Cout]"
-    return {"op": "conv2d", "cin": cin, "h": H, "w": W, "cout": cout, "k": 3, "stride": 1, "pad": 1,
+    return {"op": "conv2d", "cin": cin, "h": H, "w": W, "cout": cout, "k": 3, "stride": 1, "pad": pad,
             "epilogue": ep, "winograd_tile": tile, "witness": True}
 
 
-def conv_hypotheses(cin, H, w_size, cout_known, n_written):
+FILTERS = [(1, 1), (3, 3), (5, 5), (7, 7), (11, 11), (1, 3), (3, 1), (1, 7), (7, 1)]
+
+
+def conv_hypotheses(cin, H, W, w_size, cout_known, n_written):
     seen = set()
     for groups in (1, cin):
-        for kk in (1, 3, 5, 7, 11):
-            per = (cin // groups) * kk * kk
+        for kh, kw in FILTERS:
+            per = (cin // groups) * kh * kw
             if w_size % per:
                 continue
             cout = w_size // per
             if (cout_known and cout != cout_known) or (groups > 1 and cout != cin):
                 continue
             for s in (1, 2, 4):
-                for p in range(kk // 2 + 1):
-                    Ho = (H + 2 * p - kk) // s + 1
-                    if Ho >= 1 and cout * Ho * Ho == n_written and (cout, groups, kk, s, p) not in seen:
-                        seen.add((cout, groups, kk, s, p))
-                        yield cout, groups, kk, s, p
+                for ph in range(kh // 2 + 1):
+                    for pw in range(kw // 2 + 1):
+                        if kh == kw and ph != pw:
+                            continue
+                        Ho, Wo = (H + 2 * ph - kh) // s + 1, (W + 2 * pw - kw) // s + 1
+                        h = (cout, groups, (kh, kw), s, (ph, pw))
+                        if Ho >= 1 and Wo >= 1 and cout * Ho * Wo == n_written and h not in seen:
+                            seen.add(h)
+                            yield h
+
+
+def one_or_two(v):
+    return v[0] if v[0] == v[1] else list(v)
 
 
 def derive(name):
@@ -170,7 +184,7 @@ def derive(name):
                 print("%-60s %s" % (kname, table[kname]), flush=True)
             e = table[kname]
             assert (e["cin"], e["h"], e["w"]) == (cin, H, W), kname
-            shape[a[1]] = (e["cout"], H, W)
+            shape[a[1]] = (e["cout"], H + 2 * e["pad"] - 2, W + 2 * e["pad"] - 2)
         elif pname.startswith("fused_nn_conv2d"):
             cin, H, W = shape[a[0]]
             if new:
@@ -186,18 +200,19 @@ def derive(name):
                                                    "residual_scale_shift_relu": (1, 2)}[ep], (kname, ep)
                 relu = ep.endswith("relu")
                 hits = []
-                for cout, groups, kk, s, p in conv_hypotheses(cin, H, w.size, small[0].size if small else 0, n):
-                    Ho = (H + 2 * p - kk) // s + 1
-                    kw = dict(stride=(s, s), pad=(p, p), groups=groups, act=1 if relu else 0, acc64=True)
+                for cout, groups, (kh, kwid), s, (ph, pw) in conv_hypotheses(cin, H, W, w.size,
+                                                                             small[0].size if small else 0, n):
+                    Ho, Wo = (H + 2 * ph - kh) // s + 1, (W + 2 * pw - kwid) // s + 1
+                    kw = dict(stride=(s, s), pad=(ph, pw), groups=groups, act=1 if relu else 0, acc64=True)
                     if full:
-                        kw["residual"] = full[0][:cout * Ho * Ho].reshape(cout, Ho, Ho)
+                        kw["residual"] = full[0][:cout * Ho * Wo].reshape(cout, Ho, Wo)
                     if ep == "residual_scale_shift_relu":
                         kw.update(scale=small[0], shift=small[1])
                     elif small:
                         kw["bias"] = small[0]
-                    want = O.conv2d(x[:cin * H * W].reshape(cin, H, W), w.reshape(cout, cin // groups, kk, kk), **kw)
+                    want = O.conv2d(x[:cin * H * W].reshape(cin, H, W), w.reshape(cout, cin // groups, kh, kwid), **kw)
                     if T.close(out[:n], want):
-                        hits.append((cout, groups, kk, s, p))
+                        hits.append((cout, groups, one_or_two((kh, kwid)), s, one_or_two((ph, pw))))
                 assert len(hits) == 1, (kname, hits)
                 cout, groups, kk, s, p = hits[0]
                 if groups > 1:
@@ -211,8 +226,8 @@ def derive(name):
             e = table[kname]
             C = e["c"] if e["op"] == "dwconv2d" else e["cout"]
             assert (e["h"], e["w"]) == (H, W) and (e.get("cin", e.get("c")) == cin), kname
-            Ho = (H + 2 * e["pad"] - e["k"]) // e["stride"] + 1
-            shape[a[2]] = (C, Ho, Ho)
+            (kh, kwid), (ph, pw) = legacy.pair(e["k"]), legacy.pair(e["pad"])
+            shape[a[2]] = (C, (H + 2 * ph - kh) // e["stride"] + 1, (W + 2 * pw - kwid) // e["stride"] + 1)
         elif pname.startswith("fused_add"):                         # (out, in, per-channel shift)
             C, H, W = shape[a[1]]
             assert size(a[2]) == C, kname
@@ -237,21 +252,47 @@ def derive(name):
                 hits = []
                 for kk, s, p in ((3, 2, 0), (3, 2, 1), (2, 2, 0), (3, 1, 1), (H, 1, 0)):
                     Ho = (H + 2 * p - kk) // s + 1
-                    if C * Ho * Ho != n or (kk, s, p) in hits:
-                        continue
-                    want = O.pool2d(x, (kk, kk), (s, s), (p, p), mode,
-                                    bias=ops["placeholder1"] if with_bias else None, act=1 if with_bias else 0)
-                    if T.close(out[:n], want):
-                        hits.append((kk, s, p))
+                    for cip in ((False, True) if mode == 1 and p else (False,)):
+                        if C * Ho * Ho != n or (kk, s, p, cip) in hits:
+                            continue
+                        want = O.pool2d(x, (kk, kk), (s, s), (p, p), mode, count_include_pad=cip,
+                                        bias=ops["placeholder1"] if with_bias else None, act=1 if with_bias else 0)
+                        if T.close(out[:n], want):
+                            hits.append((kk, s, p, cip))
                 assert len(hits) == 1, (kname, hits)
-                kk, s, p = hits[0]
+                kk, s, p, cip = hits[0]
                 table[kname] = {"op": "pool2d", "c": C, "h": H, "w": W, "k": kk, "stride": s, "pad": p,
                                 "mode": "max" if mode == 0 else "avg", "bias": with_bias,
                                 "act": 1 if with_bias else 0, "witness": True}
+                if cip:
+                    table[kname]["count_include_pad"] = True
                 print("%-60s %s" % (kname, table[kname]), flush=True)
             e = table[kname]
             Ho = (H + 2 * e["pad"] - e["k"]) // e["stride"] + 1
             shape[a[1]] = (C, Ho, Ho)
+        elif pname.startswith("fused_concatenate"):                 # (out, parts in SOME order)
+            parts = [shape[i] for i in a[1:]]
+            assert len({p[1:] for p in parts}) == 1 and a[0] not in a[1:], (kname, parts)
+            H, W = parts[0][1:]
+            if new:
+                # which operand lands where is found from the data: at every offset exactly one of
+                # the remaining operands is what the kernel wrote there
+                ops, out, n = T.run_reference_kernel(exe, model, roles, kidx, rng)
+                assert n == sum(p[0] for p in parts) * H * W, kname
+                order, off, left = [], 0, list(range(len(parts)))
+                while left:
+                    fits = [j for j in left if np.array_equal(out[off:off + parts[j][0] * H * W],
+                                                              ops[roles[kname][1 + j]][:parts[j][0] * H * W])]
+                    assert len(fits) == 1, (kname, off, fits)
+                    order.append(fits[0])
+                    left.remove(fits[0])
+                    off += parts[fits[0]][0] * H * W
+                table[kname] = {"op": "concat", "parts": [parts[j][0] for j in order], "operand": order,
+                                "h": H, "w": W, "witness": True}
+                print("%-60s %s" % (kname, table[kname]), flush=True)
+            e = table[kname]
+            assert e["parts"] == [parts[j][0] for j in e["operand"]] and (e["h"], e["w"]) == (H, W), kname
+            shape[a[0]] = (sum(p[0] for p in parts), H, W)
         elif pname.startswith("fused_nn_global_avg_pool2d"):        # (in, out)
             C, H, W = shape[a[0]]
             if new:

@@ -1,6 +1,6 @@
 """The imported reference graphs on this build's kernels against the reference's OWN kernels
-(resource/resnet152 at 64 x 64 below; resource/mobilenet, resource/alexnet, resource/vgg and
-resource/resnet18 at the end).
+(resource/resnet152 at 64 x 64 below; resource/mobilenet, resource/alexnet, resource/vgg,
+resource/resnet18 and resource/inception at the end).
 
 Two executors hold the reference's resource/resnet152 graph (tests/golden/resnet152.json) with the
 same seeded parameters and the same input: one launches the reference's generated kernels
@@ -101,6 +101,7 @@ def test_imported_resnet152_tracks_the_reference_kernels_call_by_call(tmp_path):
                           "fused_nn_dense_add_kernel0", "fused_nn_softmax_kernel0")),
     ("vgg", 64, 71, ("tvmgen_default_fused_nn_dense_add_kernel0", "tvmgen_default_fused_nn_softmax_kernel0")),
     ("resnet18", 224, 57, ("fused_nn_dense_add_kernel0", "fused_nn_softmax_kernel0")),
+    ("inception", 299, 146, ("fused_nn_dense_add_kernel0", "fused_nn_softmax_1_kernel0")),
 ])
 def test_imported_walked_models_track_the_reference_kernels_call_by_call(name, side, calls, no_witness, tmp_path):
     """resource/mobilenet (MobileNet v1: a 3x3 stem, 13 depthwise + 13 pointwise convolutions) and
@@ -109,7 +110,9 @@ def test_imported_walked_models_track_the_reference_kernels_call_by_call(name, s
     calls before the classifier, every residual family, none of them broken) at 64 x 64,
     resource/resnet18 (pre-activation ResNet-18 at 224 x 224: its 13 Winograd convolutions run as
     three reference calls each on transformed weights, here as one direct convolution on the
-    weights recovered from them and compared after the third call), the
+    weights recovered from them and compared after the third call), resource/inception
+    (Inception-v3 at 299 x 299: asymmetric filters, 12 Winograd triples, a concatenation of the
+    reference = one copy per part here), the
     reference's kernels from oracle/_ref/<model>.raw.co.  Both
     executors run free from the input to the classifier; the dense and softmax kernels of the
     reference are no witnesses (int shuffle, see tests/test_gpu_reference_kernels.py), there the
@@ -171,7 +174,7 @@ def test_imported_walked_models_track_the_reference_kernels_call_by_call(name, s
     print("%s: %d calls free-running against the reference's kernels, worst deviation %.2e; %d without a witness"
           % (name, compared, worst, resynced))
     assert compared + resynced + stages == calls and resynced == len(no_witness)
-    assert stages == (26 if name == "resnet18" else 0)
+    assert stages == {"resnet18": 26, "inception": 24}.get(name, 0)
     # the classifier: probabilities
     out_idx = [i for i, s in enumerate(ref["storage"]) if s["name"] == "output"][0]
     probs = ours.get_data(out_idx, ref["storage"][out_idx]["size"])[:1000]

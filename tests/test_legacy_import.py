@@ -1,5 +1,6 @@
 """The importer for the reference's own model directories (reef_amd/legacy.py) on the reference's
-resource/resnet152, resource/mobilenet, resource/alexnet and resource/vgg graphs
+resource/resnet152, resource/mobilenet, resource/alexnet, resource/vgg, resource/resnet18 and
+resource/inception graphs
 (tests/golden/<model>.json, data fixtures): same storages, same call
 order, and the imported graph computes what the reference's kernels compute according to the
 table of shapes that was derived by running those kernels (tests/golden/make_resnet152_shapes.py,
@@ -43,8 +44,9 @@ def interpret_reference_graph(ref, table, params, x, upto=None):
         elif e["op"] == "winograd_gemm":
             wino[a[2]] = (wino.pop(a[1])[0], a[0])
         elif e["op"] == "conv2d":
-            cin, H, W, cout, kk, s, p = e["cin"], e["h"], e["w"], e["cout"], e["k"], e["stride"], e["pad"]
-            Ho = (H + 2 * p - kk) // s + 1
+            cin, H, W, cout, s = e["cin"], e["h"], e["w"], e["cout"], e["stride"]
+            (kh, kwid), (ph, pw) = legacy.pair(e["k"]), legacy.pair(e["pad"])
+            Ho, Wo = (H + 2 * ph - kh) // s + 1, (W + 2 * pw - kwid) // s + 1
             if e.get("winograd_tile"):
                 # three calls of the reference = one direct convolution on the un-transformed filter
                 alpha = e["winograd_tile"] + 2
@@ -52,10 +54,10 @@ def interpret_reference_graph(ref, table, params, x, upto=None):
                 ws = legacy.winograd_untransform(st[u].reshape(alpha, alpha, cin, cout), e["winograd_tile"])
                 a = [src, u, a[1]] + list(a[2:])
             else:
-                ws = st[a[1]].reshape(cout, cin, kk, kk)
+                ws = st[a[1]].reshape(cout, cin, kh, kwid)
             xs = st[a[0]][:cin * H * W].reshape(cin, H, W)
-            full = lambda i: st[i][:cout * Ho * Ho].reshape(cout, Ho, Ho)
-            kw = dict(stride=(s, s), pad=(p, p))
+            full = lambda i: st[i][:cout * Ho * Wo].reshape(cout, Ho, Wo)
+            kw = dict(stride=(s, s), pad=(ph, pw))
             ep = e["epilogue"]
             if ep == "none":
                 y = O.conv2d(xs, ws, act=0, **kw)
@@ -82,8 +84,13 @@ def interpret_reference_graph(ref, table, params, x, upto=None):
         elif e["op"] == "pool2d":
             C, H, W = e["c"], e["h"], e["w"]
             y = O.pool2d(st[a[0]][:C * H * W].reshape(C, H, W), (e["k"], e["k"]), (e["stride"], e["stride"]),
-                         (e["pad"], e["pad"]), 0, bias=st[a[2]] if e.get("bias") else None, act=e.get("act", 0))
+                         (e["pad"], e["pad"]), 0 if e["mode"] == "max" else 1, bias=st[a[2]] if e.get("bias") else None,
+                         act=e.get("act", 0), count_include_pad=bool(e.get("count_include_pad")))
             st[a[1]][:y.size] = y.ravel()
+        elif e["op"] == "concat":
+            hw = e["h"] * e["w"]
+            y = np.concatenate([st[a[1 + j]][:c * hw] for c, j in zip(e["parts"], e["operand"])])
+            st[a[0]][:y.size] = y
         elif e["op"] == "global_avgpool":
             C, hw = e["c"], e["hw"]
             st[a[1]][:C] = O.global_avgpool(st[a[0]][:C * hw].reshape(C, hw)).ravel()
@@ -259,7 +266,39 @@ def test_resnet18_import_replaces_winograd_triples_by_direct_convolutions(tmp_pa
     assert legacy.load_table(name) == json.load(open(golden(name, "_kernel_shapes")))
 
 
-@pytest.mark.parametrize("name,side", [("mobilenet", 224), ("vgg", 64), ("resnet18", 224)])
+def test_inception_import_has_asymmetric_filters_padded_pools_and_concatenations(tmp_path):
+    """resource/inception (Inception-v3 at 299 x 299, 146 calls): 1x7 / 7x1 / 1x3 / 3x1 / 5x5 filters,
+    twelve Winograd triples of six kinds (two of them unpadded), 3x3 stride-1 average pools that count the padding,
+    and concatenations whose operands TVM lists in the REVERSE of their channel order."""
+    name = "inception"
+    ref = json.load(open(golden(name)))
+    table = legacy.load_table(name)
+    assert table == json.load(open(golden(name, "_kernel_shapes")))
+    g = legacy.import_model(golden(name))
+    g.write(str(tmp_path))
+    out = json.load(open(os.path.join(str(tmp_path), name + ".json")))
+    n = len(ref["storage"])
+    assert out["storage"][:n] == ref["storage"] and len(ref["kernels"]) == 146
+    concat_parts = sum(len(table[k["name"]]["parts"]) for k in ref["kernels"] if table[k["name"]]["op"] == "concat")
+    concats = sum(1 for k in ref["kernels"] if table[k["name"]]["op"] == "concat")
+    triples = sum(1 for k in ref["kernels"] if table[k["name"]].get("winograd_tile"))
+    assert (concats, concat_parts, triples) == (11, 46, 12)
+    assert len(out["kernels"]) == 146 - 2 * triples + concat_parts - concats
+    assert sorted(set(g.imported_calls)) == [i for i, k in enumerate(ref["kernels"])
+                                              if not table[k["name"]]["op"].startswith("winograd_")]
+    assert all(e["operand"] == list(range(len(e["parts"])))[::-1] for e in table.values() if e["op"] == "concat")
+    assert {tuple(e["k"]) for e in table.values() if e["op"] == "conv2d" and not isinstance(e["k"], int)} \
+        == {(1, 7), (7, 1), (1, 3), (3, 1)}
+    assert sum(1 for e in table.values() if e.get("winograd_tile") and e["pad"] == 0) == 2
+    assert all(e.get("count_include_pad") for e in table.values() if e["op"] == "pool2d" and e["mode"] == "avg" and e["pad"])
+    assert abs(g.flops / 1e9 - 11.426) < 0.01        # Inception-v3's convolutions + classifier
+    with pytest.raises(legacy.ImportError_, match="fused_concatenate_11_kernel0"):
+        bad = json.loads(json.dumps(table))
+        bad["fused_concatenate_11_kernel0"]["operand"] = [0, 1, 2, 3]
+        legacy.import_model(golden(name), table=bad)
+
+
+@pytest.mark.parametrize("name,side", [("mobilenet", 224), ("vgg", 64), ("resnet18", 224), ("inception", 299)])
 def test_imported_walked_model_equals_the_table_interpretation_through_the_executor(name, side, tmp_path):
     d = str(tmp_path)
     g = legacy.import_model(golden(name))
