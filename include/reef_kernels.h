@@ -329,13 +329,17 @@ enum { REEF_TR_D0 = 0, REEF_TR_D1, REEF_TR_D2, REEF_TR_FLAGS, REEF_TR_NATTR };
  * trans_b = 1: B stored [b][n][k] (dense layers, Q.K^T); 0: [b][k][n] (P.V).
  * ptr: A, B, C, bias(optional).
  * attr: batch, M, N, K, trans_b, flags, act, alpha (float bits), tile, m_tiles, n_tiles,
- *       lda, ldb, ldc, strideA, strideB, strideC (elements).
+ *       lda, ldb, ldc, strideA, strideB, strideC (elements), then offA, offB, offC: where the
+ *       first matrix starts inside its storage, in elements (absent = 0; multiples of 4 like the
+ *       strides) -- several operands can share one storage, e.g. Q, K and V as column blocks of
+ *       one [tokens][3 * hidden] projection.
  * tasks = batch * m_tiles * n_tiles. */
 enum {
     REEF_GEMM_BATCH = 0, REEF_GEMM_M, REEF_GEMM_N, REEF_GEMM_K, REEF_GEMM_TRANS_B,
     REEF_GEMM_FLAGS, REEF_GEMM_ACT, REEF_GEMM_ALPHA_BITS, REEF_GEMM_TILE, REEF_GEMM_M_TILES,
     REEF_GEMM_N_TILES, REEF_GEMM_LDA, REEF_GEMM_LDB, REEF_GEMM_LDC, REEF_GEMM_STRIDE_A,
-    REEF_GEMM_STRIDE_B, REEF_GEMM_STRIDE_C, REEF_GEMM_NATTR
+    REEF_GEMM_STRIDE_B, REEF_GEMM_STRIDE_C, REEF_GEMM_OFF_A, REEF_GEMM_OFF_B, REEF_GEMM_OFF_C,
+    REEF_GEMM_NATTR
 };
 
 /* ---- add / multiply (the reference's mocked model): ptr: a, b, out; no attrs ---- */

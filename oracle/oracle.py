@@ -392,9 +392,10 @@ class GraphOracle:
         elif name.startswith("reef_gemm"):
             (batch, M, N, K, trans_b, flags, act, alpha_bits, _t, _mt, _nt, lda, ldb, ldc, sA, sB,
              sC) = a[:17]
+            oA, oB, oC = (list(a[17:20]) + [0, 0, 0])[:3]     # absent = 0 (include/reef_kernels.h)
             alpha = _bits_to_float(alpha_bits)
             bias = P[3] if flags & 1 else None
-            A, B, C = P[0], P[1], P[2]
+            A, B, C = P[0][oA:], P[1][oB:], P[2][oC:]
             for bi in range(batch):
                 Am = np.lib.stride_tricks.as_strided(A[bi * sA:], (M, K), (lda * 4, 4))
                 if trans_b:

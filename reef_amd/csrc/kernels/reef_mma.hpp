@@ -1250,9 +1250,9 @@ __device__ __forceinline__ bool gemm_body(const ReefOpDesc& d, int task, char* s
     const int mt = div_small(rem, n_tiles), nt = rem - mt * n_tiles;
     const int m0 = mt * T::BM, n0 = nt * T::BN;
     const int lda = a[REEF_GEMM_LDA], ldb = a[REEF_GEMM_LDB], ldc = a[REEF_GEMM_LDC];
-    const float* A = (const float*)d.ptr[0] + (size_t)b * a[REEF_GEMM_STRIDE_A];
-    const float* B = (const float*)d.ptr[1] + (size_t)b * a[REEF_GEMM_STRIDE_B];
-    float* C = (float*)d.ptr[2] + (size_t)b * a[REEF_GEMM_STRIDE_C];
+    const float* A = (const float*)d.ptr[0] + a[REEF_GEMM_OFF_A] + (size_t)b * a[REEF_GEMM_STRIDE_A];
+    const float* B = (const float*)d.ptr[1] + a[REEF_GEMM_OFF_B] + (size_t)b * a[REEF_GEMM_STRIDE_B];
+    float* C = (float*)d.ptr[2] + a[REEF_GEMM_OFF_C] + (size_t)b * a[REEF_GEMM_STRIDE_C];
     const int nk = (K + T::BK - 1) / T::BK;
     float* smem = (float*)smem_raw;
     f32x16 acc[T::TM][T::TN];
@@ -1330,11 +1330,11 @@ __device__ __forceinline__ bool gemm_nt_direct_body(const ReefOpDesc& d, int tas
     const int m0 = mt * TD::BM, n0 = nt * TD::BN;
     const unsigned lda = (unsigned)a[REEF_GEMM_LDA], ldb = (unsigned)a[REEF_GEMM_LDB],
                    ldc = (unsigned)a[REEF_GEMM_LDC];
-    const rsrc_t rs_a = make_rsrc((const float*)d.ptr[0] + (size_t)b * a[REEF_GEMM_STRIDE_A],
+    const rsrc_t rs_a = make_rsrc((const float*)d.ptr[0] + a[REEF_GEMM_OFF_A] + (size_t)b * a[REEF_GEMM_STRIDE_A],
                                   ((unsigned)(M - 1) * lda + (unsigned)K) * 4u);
-    const rsrc_t rs_b = make_rsrc((const float*)d.ptr[1] + (size_t)b * a[REEF_GEMM_STRIDE_B],
+    const rsrc_t rs_b = make_rsrc((const float*)d.ptr[1] + a[REEF_GEMM_OFF_B] + (size_t)b * a[REEF_GEMM_STRIDE_B],
                                   ((unsigned)(N - 1) * ldb + (unsigned)K) * 4u);
-    const rsrc_t rs_c = make_rsrc((const float*)d.ptr[2] + (size_t)b * a[REEF_GEMM_STRIDE_C],
+    const rsrc_t rs_c = make_rsrc((const float*)d.ptr[2] + a[REEF_GEMM_OFF_C] + (size_t)b * a[REEF_GEMM_STRIDE_C],
                                   ((unsigned)(M - 1) * ldc + (unsigned)N) * 4u);
     const bool has_bias = a[REEF_GEMM_FLAGS] & 1;
     const rsrc_t rs_bias = make_rsrc(d.ptr[has_bias ? 3 : 2], (unsigned)N * 4u);

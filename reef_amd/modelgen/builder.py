@@ -413,14 +413,17 @@ class GraphBuilder:
         return out
 
     def gemm(self, a, b, M, N, K, batch=1, trans_b=True, bias=None, act=ACT_NONE, alpha=1.0,
-             lda=None, ldb=None, ldc=None, stride_a=0, stride_b=0, stride_c=0, out=None, force_tile=None):
+             lda=None, ldb=None, ldc=None, stride_a=0, stride_b=0, stride_c=0, out=None, force_tile=None,
+             off_a=0, off_b=0, off_c=0):
         """C[b] = act(alpha * A[b] x B[b] (+bias)); operands are storages with explicit strides.
-        force_tile: a staged tile name or, for trans_b, one of tiling.GEMM_DIRECT_TILES."""
+        force_tile: a staged tile name or, for trans_b, one of tiling.GEMM_DIRECT_TILES.
+        off_a / off_b / off_c: element at which the first matrix starts inside its storage."""
         lda = K if lda is None else lda
         ldb = (K if trans_b else N) if ldb is None else ldb
         ldc = N if ldc is None else ldc
         if out is None:
             out = self.temp((batch, M, N))
+        assert off_a % 4 == 0 and off_b % 4 == 0 and off_c % 4 == 0, "gemm operands must be 16-byte aligned"
         direct_ok = (trans_b and K % 8 == 0 and lda % 4 == 0 and ldb % 4 == 0 and stride_a % 4 == 0
                      and stride_b % 4 == 0)
         if force_tile is not None:
@@ -442,7 +445,8 @@ class GraphBuilder:
         self._emit("reef_gemm_%s_%s" % ("ntd" if direct else "nt" if trans_b else "nn", t["tile"]),
                    batch * t["m_tiles"] * t["n_tiles"], args,
                    [batch, M, N, K, 1 if trans_b else 0, flags, act, float_bits(alpha), t["tile_id"],
-                    t["m_tiles"], t["n_tiles"], lda, ldb, ldc, stride_a, stride_b, stride_c],
+                    t["m_tiles"], t["n_tiles"], lda, ldb, ldc, stride_a, stride_b, stride_c,
+                    off_a, off_b, off_c],
                    "gemm", flops, 4 * batch * (M * K + N * K + M * N), t["est_us"])
         return out
 

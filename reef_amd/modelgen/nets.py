@@ -289,7 +289,11 @@ def bert(layers=12, hidden=768, heads=12, ffn=3072, seq=128, vocab=30522, name="
     """BERT encoder (base: 12 layers, hidden 768, 12 heads, FFN 3072, sequence 128), fp32,
     weights ~ N(0, 0.02).  Token ids are an int64 input, as in the reference's BERT model
     (resource/bert/bert.json storage[0]).  The per-head views of Q, K, V and of the context
-    are expressed as GEMM strides, so no transpose kernels are needed.
+    are expressed as GEMM strides, so no transpose kernels are needed, and the three projections
+    of a layer are ONE product with the stacked weight [3 * hidden][hidden]: Q, K and V are the
+    column blocks of its [seq][3 * hidden] result, which the attention products address by
+    offset and leading dimension (a third of the launches of three separate products, each of
+    which fills only 192 of the 256 CUs' workgroup slots once).
     attention_mask: a second input `attention_mask` (uint1, one byte per token, non-zero = padding)
     that every softmax applies to the key positions.  The reference's BERT derives that mask
     inside the graph -- as all zeros (fused_full_equal_reshape, bert.cu:313) -- and applies it
@@ -303,18 +307,16 @@ def bert(layers=12, hidden=768, heads=12, ffn=3072, seq=128, vocab=30522, name="
     x = g.layernorm(x, seq, hidden)
     inv_sqrt = 1.0 / (hd ** 0.5)
     for _ in range(layers):
-        proj = []
-        for _name in ("q", "k", "v"):
-            w = g.param((hidden, hidden), 0.02)
-            b = g.param((hidden,), 0.02)
-            proj.append(g.gemm(x, w, seq, hidden, hidden, trans_b=True, bias=b))
-        q, k, v = proj
-        scores = g.gemm(q, k, seq, seq, hd, batch=heads, trans_b=True, alpha=inv_sqrt,
-                        lda=hidden, ldb=hidden, ldc=seq, stride_a=hd, stride_b=hd, stride_c=seq * seq)
+        w = g.param((3 * hidden, hidden), 0.02)
+        b = g.param((3 * hidden,), 0.02)
+        qkv = g.gemm(x, w, seq, 3 * hidden, hidden, trans_b=True, bias=b)
+        scores = g.gemm(qkv, qkv, seq, seq, hd, batch=heads, trans_b=True, alpha=inv_sqrt,
+                        lda=3 * hidden, ldb=3 * hidden, ldc=seq, stride_a=hd, stride_b=hd, stride_c=seq * seq,
+                        off_b=hidden)
         probs = g.softmax(scores, heads * seq, seq, mask=mask)
         ctx = g.temp((seq, hidden))
-        g.gemm(probs, v, seq, hd, seq, batch=heads, trans_b=False, lda=seq, ldb=hidden, ldc=hidden,
-               stride_a=seq * seq, stride_b=hd, stride_c=hd, out=ctx)
+        g.gemm(probs, qkv, seq, hd, seq, batch=heads, trans_b=False, lda=seq, ldb=3 * hidden, ldc=hidden,
+               stride_a=seq * seq, stride_b=hd, stride_c=hd, out=ctx, off_b=2 * hidden)
         wo = g.param((hidden, hidden), 0.02)
         bo = g.param((hidden,), 0.02)
         att = g.gemm(ctx, wo, seq, hidden, hidden, trans_b=True, bias=bo)

@@ -343,6 +343,40 @@ def test_gemm_nt_direct_tiles(tmp_path, tile):
     compare_storages(exe, orc, model, what="direct gemm " + tile)
 
 
+def test_gemm_operands_at_offsets_inside_one_storage(tmp_path):
+    """Q, K and V as the column blocks of ONE [seq][3 * hidden] projection (attrs offA/offB/offC):
+    Q K^T on every direct tile and on a staged one, P V reading V at its offset and writing the
+    context into the second half of a larger buffer.  Checked against the oracle and, for the
+    offsets themselves, against numpy on the slices."""
+    seq, hid, heads = 40, 96, 4
+    hd = hid // heads                                     # 24
+    g = MB.GraphBuilder("go", weight_std=0.05)
+    x = g.input("x", (seq, hid))
+    w = g.param((3 * hid, hid), 0.05)
+    bias = g.param((3 * hid,), 0.02)
+    qkv = g.gemm(x, w, seq, 3 * hid, hid, trans_b=True, bias=bias)
+    kw = dict(batch=heads, trans_b=True, alpha=0.25, lda=3 * hid, ldb=3 * hid, stride_a=hd, stride_b=hd,
+              stride_c=seq * seq, off_b=hid)
+    scores = [g.gemm(qkv, qkv, seq, seq, hd, force_tile=t, **kw) for t in list(tiling.GEMM_DIRECT_TILES) + ["32x32k4"]]
+    assert [k["name"].split("_")[2] for k in g.kernels[1:]] == ["ntd"] * len(tiling.GEMM_DIRECT_TILES) + ["nt"]
+    probs = g.softmax(scores[0], heads * seq, seq)
+    both = g.temp((2, seq, hid))
+    g.gemm(probs, qkv, seq, hd, seq, batch=heads, trans_b=False, lda=seq, ldb=3 * hid, ldc=hid,
+           stride_a=seq * seq, stride_b=hd, stride_c=hd, out=both, off_b=2 * hid, off_c=seq * hid)
+    g.mark_output(both)
+    exe, orc, model = run_both(g, tmp_path, {"x": rnd(seq, hid)})
+    compare_storages(exe, orc, model, what="gemm operands at offsets")
+    m = exe.get_data(qkv.idx, seq * 3 * hid).reshape(seq, 3, heads, hd).astype(np.float64)
+    want = 0.25 * np.einsum("shd,thd->hst", m[:, 0], m[:, 1])
+    for s_ in scores:
+        got = exe.get_data(s_.idx, heads * seq * seq).reshape(heads, seq, seq)
+        assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
+    p_ = exe.get_data(probs.idx, heads * seq * seq).reshape(heads, seq, seq).astype(np.float64)
+    ctx = np.einsum("hst,thd->shd", p_, m[:, 2]).reshape(seq, hid)
+    out = exe.get_data(both.idx, 2 * seq * hid).reshape(2, seq, hid)
+    assert (out[0] == 0).all() and np.abs(out[1] - ctx).max() <= 1e-5 * np.abs(ctx).max()
+
+
 def test_mocked_model_closed_form(tmp_path):
     """The reference's executor_base.mocked_kernel test: a = b = c = 3 -> 18 everywhere
     (src/reef/test/test.cpp:102-116)."""

@@ -169,9 +169,8 @@ def test_bert_wiring(tmp_path, masked):
     t = ln(t)
     hd = hidden // heads
     for _ in range(layers):
-        q = F.linear(t, P.take(hidden, hidden), P.take(hidden))
-        k = F.linear(t, P.take(hidden, hidden), P.take(hidden))
-        v = F.linear(t, P.take(hidden, hidden), P.take(hidden))
+        # one stacked projection [3 * hidden][hidden]: rows 0..hidden-1 make Q, then K, then V
+        q, k, v = F.linear(t, P.take(3 * hidden, hidden), P.take(3 * hidden)).split(hidden, dim=1)
         split = lambda m: m.reshape(seq, heads, hd).permute(1, 0, 2)
         scores = split(q) @ split(k).transpose(1, 2) / hd ** 0.5
         if masked:
