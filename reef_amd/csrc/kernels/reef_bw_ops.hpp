@@ -322,13 +322,16 @@ __device__ __forceinline__ void layernorm_body(const ReefOpDesc& d, int task) {
     float* y = (float*)d.ptr[3] + (size_t)r * cols;
     const float* res = (d.attr[REEF_LN_FLAGS] & 1) ? (const float*)d.ptr[4] + (size_t)r * cols : nullptr;
     // Rows of up to 1024 values stay in registers (16 per lane): one trip to memory instead of
-    // three.  The sums run over the same values in the same order as the general path below.
+    // three; gamma and beta come in on that trip too.  The sums run over the same values in the
+    // same order as the general path below.
     if (cols <= 16 * 64) {
-        float val[16];
+        float val[16], gm[16], bt[16];
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
             const int i = lane + 64 * j;
             val[j] = i < cols ? (res ? x[i] + res[i] : x[i]) : 0.0f;
+            gm[j] = i < cols ? gamma[i] : 0.0f;
+            bt[j] = i < cols ? beta[i] : 0.0f;
         }
         float s = 0.0f;
 #pragma unroll
@@ -346,7 +349,7 @@ __device__ __forceinline__ void layernorm_body(const ReefOpDesc& d, int task) {
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
             const int i = lane + 64 * j;
-            if (i < cols) y[i] = (val[j] - mean) * inv * gamma[i] + beta[i];
+            if (i < cols) y[i] = (val[j] - mean) * inv * gm[j] + bt[j];
         }
         return;
     }
