@@ -275,7 +275,10 @@ class GraphOracle:
 
     def run_kernel(self, k, acc64=False):
         name, a = k["name"].split("#")[0], k.get("attrs", [])
-        P = [self.storage[i] for i in k["args"]]
+        # "arg_offsets": the byte at which an operand starts inside its storage (views, so results
+        # land in the storage)
+        offs = k.get("arg_offsets") or [0] * len(k["args"])
+        P = [self.storage[i][o // self.storage[i].itemsize:] for i, o in zip(k["args"], offs)]
         if name.startswith("reef_conv2d"):
             Cin, H, W, Cout, Ho, Wo, kh, kw, sh, sw, ph, pw, flags, act, _tile, split_k = a[:16]
             act2 = a[19] if len(a) > 19 else 0   # a[20]: first sync counter (device detail)

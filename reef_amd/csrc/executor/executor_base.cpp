@@ -97,7 +97,8 @@ Status ExecutorBase::init_executor_base(const char* json_file_path, GPUModule_t 
         const KernelInfo& ki = model->kernels[i];
         ReefOpDesc& d = descs[i];
         std::memset(&d, 0, sizeof(d));
-        for (size_t j = 0; j < ki.args.size(); ++j) d.ptr[j] = storage[ki.args[j]];
+        for (size_t j = 0; j < ki.args.size(); ++j)
+            d.ptr[j] = (char*)storage[ki.args[j]] + (ki.arg_offsets.empty() ? 0 : ki.arg_offsets[j]);
         for (size_t j = 0; j < ki.attrs.size(); ++j) d.attr[j] = ki.attrs[j];
     }
 

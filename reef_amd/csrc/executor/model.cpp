@@ -47,6 +47,18 @@ Model* Model::from_json_text(const std::string& text, std::string* err) {
         }
         if (const JsonValue* at = k->get("attrs"))
             for (const auto& a : at->lval) ki.attrs.push_back((int32_t)a->as_int());
+        if (const JsonValue* ao = k->get("arg_offsets")) {
+            if (ao->lval.size() != ki.args.size())
+                return bad("arg_offsets must have one entry per arg in " + n->sval);
+            for (size_t j = 0; j < ao->lval.size(); ++j) {
+                const int64_t off = ao->lval[j]->as_int();
+                const StorageInfo& st = m->storage[ki.args[j]];
+                const size_t bytes = st.size * get_stype_size(st.stype);
+                if (off < 0 || off % 16 != 0 || (off != 0 && (size_t)off >= bytes))
+                    return bad("arg offset outside its storage or not a multiple of 16 in " + n->sval);
+                ki.arg_offsets.push_back((size_t)off);
+            }
+        }
         m->kernels.push_back(std::move(ki));
     }
     if (const JsonValue* ga = root->get("args"))

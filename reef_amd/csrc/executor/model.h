@@ -27,6 +27,11 @@ public:
     uint32_t launch_params[6];  // grid x,y,z, block x,y,z
     std::vector<size_t> args;   // storage indices, bound positionally
     std::vector<int32_t> attrs; // per-launch shape attributes (may be empty)
+    // Optional "arg_offsets": per argument the byte at which the operand starts inside its
+    // storage (empty = every operand starts at its storage's first byte).  A channel range of a
+    // tensor is one contiguous piece of its storage, so a kernel can read or write a part of a
+    // larger buffer without a variant of its own.  The reference's reader ignores the key.
+    std::vector<size_t> arg_offsets;
 };
 
 class Model {

@@ -33,15 +33,23 @@ def float_bits(x):
 
 
 class Tensor:
-    """A storage index plus its logical shape."""
+    """A storage index plus its logical shape; `off`: the element of the storage at which the
+    tensor starts (a view of a part of a larger buffer, the kernels' `arg_offsets`)."""
 
-    def __init__(self, idx, shape):
+    def __init__(self, idx, shape, off=0):
         self.idx = idx
         self.shape = tuple(int(s) for s in shape)
+        self.off = int(off)
 
     @property
     def size(self):
         return int(np.prod(self.shape))
+
+    def channels(self, first, count):
+        """Channels [first, first + count) of a [C][H][W] tensor: contiguous, so a tensor itself."""
+        C, H, W = self.shape
+        assert 0 <= first and first + count <= C
+        return Tensor(self.idx, (count, H, W), self.off + first * H * W)
 
 
 class GraphBuilder:
@@ -113,13 +121,19 @@ class GraphBuilder:
 
     # ------------------------------------------------------------ kernels
     def _emit(self, name, tasks, args, attrs, op, flops=0, nbytes=0, est_us=1.0, block=(WG, 1, 1)):
+        # an operand is a storage index or a Tensor; a Tensor that starts inside its storage
+        # makes the kernel carry "arg_offsets" (bytes; fp32 operands)
+        offs = [4 * a.off if isinstance(a, Tensor) else 0 for a in args]
+        assert all(o % 16 == 0 for o in offs), "operand views must start on 16 bytes"
         self.kernels.append({
             "name": "%s#%d" % (name, len(self.kernels)) if self.unique_names else name,
             "launch_params": [int(tasks), 1, 1, block[0], block[1], block[2]],
-            "args": [int(a) for a in args],
+            "args": [a.idx if isinstance(a, Tensor) else int(a) for a in args],
             "attrs": [int(a) for a in attrs],
             "op": op,
         })
+        if any(offs):
+            self.kernels[-1]["arg_offsets"] = offs
         self.kernel_flops.append(int(flops))
         self.kernel_bytes.append(int(nbytes))
         self.kernel_est_us.append(float(est_us))
@@ -172,7 +186,7 @@ class GraphBuilder:
             out = self.temp((cout, Ho, Wo))
         else:
             assert out.shape[1:] == (Ho, Wo) and out_channel + cout <= out.shape[0]
-            dst_off = out_channel * Ho * Wo
+            dst_off = out.off + out_channel * Ho * Wo
         out2 = None
         if dual_act is not None:
             assert not affine
@@ -234,7 +248,7 @@ class GraphBuilder:
             flags |= F_PRE_ACT
             nbytes += 4 * 2 * cin
         if t["split_k"] == 1:
-            args = [x.idx, w.idx, out.idx] + opt + pre
+            args = [x, w.idx, out.idx] + opt + pre
             attrs = base + [flags, act, t["tile_id"], 1, t["k_chunk"], t["m_tiles"], t["n_tiles"], act2,
                             0, mode, dst_off, len(args) if packed else 0]
             self._emit(kname, t["tasks"], args + packed, attrs, "conv2d", flops, nbytes + nbytes_pack, t["est_us"])
@@ -245,14 +259,14 @@ class GraphBuilder:
             pair = t["split_k"] == 2 and mode in (3, 4, 5) and self.pair_fold
             ws = self.workspace((t["split_k"] + (1 if pair else 0)) * M * N)
             sync_idx, sync_off = self._sync_counters(t["m_tiles"] * t["n_tiles"])
-            args = [x.idx, w.idx, out.idx] + opt + pre + [ws.idx, sync_idx]
+            args = [x, w.idx, out.idx] + opt + pre + [ws.idx, sync_idx]
             flags |= F_PAIR_FOLD if pair else 0
             attrs = base + [flags | F_FUSED_REDUCE, act, t["tile_id"], t["split_k"], t["k_chunk"],
                             t["m_tiles"], t["n_tiles"], act2, sync_off, mode, dst_off, len(args) if packed else 0]
             self._emit(kname, t["tasks"], args + packed, attrs, "conv2d", flops, nbytes + nbytes_pack, t["est_us"])
         else:
             ws = self.workspace(t["split_k"] * M * N)
-            args = [x.idx, w.idx, ws.idx] + pre
+            args = [x, w.idx, ws.idx] + pre
             attrs = base + [F_PRE_ACT if pre else 0, ACT_NONE, t["tile_id"], t["split_k"], t["k_chunk"],
                             t["m_tiles"], t["n_tiles"], ACT_NONE, 0, mode, 0, len(args) if packed else 0]
             self._emit(kname, t["tasks"], args + packed, attrs, "conv2d", flops,
@@ -293,8 +307,8 @@ class GraphBuilder:
         rnd = math.ceil if ceil_mode else math.floor
         Ho = int(rnd((H + 2 * pad - kh) / stride)) + 1
         Wo = int(rnd((W + 2 * pad - kw) / stride)) + 1
-        out = Tensor(out.idx, (C, Ho, Wo)) if out is not None else self.temp((C, Ho, Wo))
-        args = [x.idx, out.idx]
+        out = Tensor(out.idx, (C, Ho, Wo), out.off) if out is not None else self.temp((C, Ho, Wo))
+        args = [x, out]
         flags = 0
         if bias:
             flags = 1
@@ -308,7 +322,7 @@ class GraphBuilder:
     def global_avgpool(self, x, out=None):
         C = x.shape[0]
         out = Tensor(out.idx, (C,)) if out is not None else self.temp((C,))
-        self._emit("reef_global_avgpool", math.ceil(C / 4), [x.idx, out.idx], [C, x.size // C],
+        self._emit("reef_global_avgpool", math.ceil(C / 4), [x, out.idx], [C, x.size // C],
                    "global_avgpool", 0, 4 * (x.size + C), 2.0)
         return out
 

@@ -172,23 +172,20 @@ def densenet(blocks=(6, 12, 48, 32), growth=32, image=(3, 224, 224), classes=100
 
 
 def inception_v3(image=(3, 299, 299), classes=1000, name="inceptionv3", seed=rng.BASE_SEED):
-    """Inception-v3 (the 299x299 network): every convolution is conv + folded BN + ReLU;
-    branch outputs are written straight into their channel slices of the block output."""
+    """Inception-v3 (the 299x299 network): every convolution is conv + folded BN + ReLU.
+    The 1x1 convolutions of a block that read the block's input (the 1x1 branch and the reductions
+    in front of the 5x5 / 3x3 / 7-tap branches) are ONE convolution with the stacked filter: same
+    input, same epilogue, and each of them alone fills less than the device.  Its result
+    [reductions | 1x1 branch] is written in front of and into the block's output buffer, so the
+    1x1 branch lands where the concatenation wants it and the reductions are read back as channel
+    ranges (operand views); the other branches write straight into their channel slices."""
     g = GraphBuilder(name, seed)
-    T = None
 
     def conv(x, cout, k, s=1, p=0, out=None, ch=0):
         return g.conv2d(x, cout, k, s, p, bias=True, act=ACT_RELU, out=out, out_channel=ch)
 
-    def block(x, branches, H, W):
-        """branches: list of (channels, fn(x, out, ch)); returns the concatenated tensor."""
-        total = sum(c for c, _ in branches)
-        out = g.temp((total, H, W))
-        ch = 0
-        for c, fn in branches:
-            fn(x, out, ch)
-            ch += c
-        return out
+    def avg(x):
+        return g.pool2d(x, 3, 1, 1, "avg", count_include_pad=True)
 
     x = g.input("data", image)
     x = conv(x, 32, 3, 2)            # 149
@@ -201,13 +198,13 @@ def inception_v3(image=(3, 299, 299), classes=1000, name="inceptionv3", seed=rng
 
     def inception_a(x, pool_ch):
         _, H, W = x.shape
-        return block(x, [
-            (64, lambda x, o, c: conv(x, 64, 1, out=o, ch=c)),
-            (64, lambda x, o, c: conv(conv(x, 48, 1), 64, 5, 1, 2, out=o, ch=c)),
-            (96, lambda x, o, c: conv(conv(conv(x, 64, 1), 96, 3, 1, 1), 96, 3, 1, 1, out=o, ch=c)),
-            (pool_ch, lambda x, o, c: conv(g.pool2d(x, 3, 1, 1, "avg", count_include_pad=True), pool_ch, 1,
-                                           out=o, ch=c)),
-        ], H, W)
+        r = 48 + 64                                      # reductions in front of the output
+        S = g.temp((r + 64 + 64 + 96 + pool_ch, H, W))
+        conv(x, 48 + 64 + 64, 1, out=S, ch=0)            # [5x5 reduction | 3x3 reduction | 1x1 branch]
+        conv(S.channels(0, 48), 64, 5, 1, 2, out=S, ch=r + 64)
+        conv(conv(S.channels(48, 64), 96, 3, 1, 1), 96, 3, 1, 1, out=S, ch=r + 128)
+        conv(avg(x), pool_ch, 1, out=S, ch=r + 224)
+        return S.channels(r, 224 + pool_ch)
 
     x = inception_a(x, 32)
     x = inception_a(x, 64)
@@ -219,24 +216,21 @@ def inception_v3(image=(3, 299, 299), classes=1000, name="inceptionv3", seed=rng
         out = g.temp((384 + 96 + cin, Ho, Ho))
         conv(x, 384, 3, 2, out=out, ch=0)
         conv(conv(conv(x, 64, 1), 96, 3, 1, 1), 96, 3, 2, out=out, ch=384)
-        p = g.pool2d(x, 3, 2, 0, "max")
-        g.copy_into(p, out, (384 + 96) * Ho * Ho)
+        g.pool2d(x, 3, 2, 0, "max", out=out.channels(384 + 96, cin))
         return out
 
     x = inception_b(x)               # 768 x 17 x 17
 
     def inception_c(x, c7):
         _, H, W = x.shape
-        return block(x, [
-            (192, lambda x, o, c: conv(x, 192, 1, out=o, ch=c)),
-            (192, lambda x, o, c: conv(conv(conv(x, c7, 1), c7, (1, 7), 1, (0, 3)), 192, (7, 1), 1, (3, 0),
-                                       out=o, ch=c)),
-            (192, lambda x, o, c: conv(conv(conv(conv(conv(x, c7, 1), c7, (7, 1), 1, (3, 0)), c7, (1, 7), 1,
-                                                      (0, 3)), c7, (7, 1), 1, (3, 0)), 192, (1, 7), 1, (0, 3),
-                                       out=o, ch=c)),
-            (192, lambda x, o, c: conv(g.pool2d(x, 3, 1, 1, "avg", count_include_pad=True), 192, 1, out=o,
-                                       ch=c)),
-        ], H, W)
+        r = 2 * c7
+        S = g.temp((r + 768, H, W))
+        conv(x, c7 + c7 + 192, 1, out=S, ch=0)           # [7-tap reduction | double 7-tap reduction | 1x1 branch]
+        conv(conv(S.channels(0, c7), c7, (1, 7), 1, (0, 3)), 192, (7, 1), 1, (3, 0), out=S, ch=r + 192)
+        y = conv(conv(conv(S.channels(c7, c7), c7, (7, 1), 1, (3, 0)), c7, (1, 7), 1, (0, 3)), c7, (7, 1), 1, (3, 0))
+        conv(y, 192, (1, 7), 1, (0, 3), out=S, ch=r + 384)
+        conv(avg(x), 192, 1, out=S, ch=r + 576)
+        return S.channels(r, 768)
 
     for c7 in (128, 160, 160, 192):
         x = inception_c(x, c7)
@@ -245,35 +239,28 @@ def inception_v3(image=(3, 299, 299), classes=1000, name="inceptionv3", seed=rng
         cin, H, W = x.shape
         Ho = (H - 3) // 2 + 1
         out = g.temp((320 + 192 + cin, Ho, Ho))
-        conv(conv(x, 192, 1), 320, 3, 2, out=out, ch=0)
-        y = conv(conv(conv(x, 192, 1), 192, (1, 7), 1, (0, 3)), 192, (7, 1), 1, (3, 0))
+        red = conv(x, 192 + 192, 1)                      # both reductions
+        conv(red.channels(0, 192), 320, 3, 2, out=out, ch=0)
+        y = conv(conv(red.channels(192, 192), 192, (1, 7), 1, (0, 3)), 192, (7, 1), 1, (3, 0))
         conv(y, 192, 3, 2, out=out, ch=320)
-        p = g.pool2d(x, 3, 2, 0, "max")
-        g.copy_into(p, out, (320 + 192) * Ho * Ho)
+        g.pool2d(x, 3, 2, 0, "max", out=out.channels(320 + 192, cin))
         return out
 
     x = inception_d(x)               # 1280 x 8 x 8
 
     def inception_e(x):
         _, H, W = x.shape
-
-        def b3(x, o, c):
-            y = conv(x, 384, 1)
-            conv(y, 384, (1, 3), 1, (0, 1), out=o, ch=c)
-            conv(y, 384, (3, 1), 1, (1, 0), out=o, ch=c + 384)
-
-        def b3dbl(x, o, c):
-            y = conv(conv(x, 448, 1), 384, 3, 1, 1)
-            conv(y, 384, (1, 3), 1, (0, 1), out=o, ch=c)
-            conv(y, 384, (3, 1), 1, (1, 0), out=o, ch=c + 384)
-
-        return block(x, [
-            (320, lambda x, o, c: conv(x, 320, 1, out=o, ch=c)),
-            (768, b3),
-            (768, b3dbl),
-            (192, lambda x, o, c: conv(g.pool2d(x, 3, 1, 1, "avg", count_include_pad=True), 192, 1, out=o,
-                                       ch=c)),
-        ], H, W)
+        r = 384 + 448
+        S = g.temp((r + 2048, H, W))
+        conv(x, 384 + 448 + 320, 1, out=S, ch=0)         # [3-tap reduction | 3x3 reduction | 1x1 branch]
+        y = S.channels(0, 384)
+        conv(y, 384, (1, 3), 1, (0, 1), out=S, ch=r + 320)
+        conv(y, 384, (3, 1), 1, (1, 0), out=S, ch=r + 704)
+        y = conv(S.channels(384, 448), 384, 3, 1, 1)
+        conv(y, 384, (1, 3), 1, (0, 1), out=S, ch=r + 1088)
+        conv(y, 384, (3, 1), 1, (1, 0), out=S, ch=r + 1472)
+        conv(avg(x), 192, 1, out=S, ch=r + 1856)
+        return S.channels(r, 2048)
 
     x = inception_e(x)
     x = inception_e(x)               # 2048 x 8 x 8

@@ -143,6 +143,23 @@ def test_json_subset_and_superset(tmp_path):
     assert model_summary(str(tmp_path / "missing.json"))[0] == 2
 
 
+def test_arg_offsets_are_checked_against_their_storages(tmp_path):
+    """The added key `arg_offsets` (bytes into each operand's storage): one entry per argument,
+    multiples of 16, inside the storage; the reference's reader never looks at the key."""
+    p = tmp_path / "m.json"
+    body = ("{\"storage\": [{\"name\": \"a\", \"size\": 64, \"stype\": \"float32\"}, {\"name\": \"b\", \"size\": 8, "
+            "\"stype\": \"float32\"}], \"kernels\": [{\"name\": \"add\", \"launch_params\": [1,1,1,4,8,4], "
+            "\"args\": [0, 0, 1], \"arg_offsets\": %s}], \"args\": [0], \"shared_memory\": {}}")
+    for offs, ok in (("[0, 128, 16]", True), ("[0, 240, 0]", True), ("[0, 0, 0]", True),
+                     ("[0, 128]", False),          # one entry per argument
+                     ("[0, 8, 0]", False),         # 16-byte steps
+                     ("[0, 256, 0]", False),       # a holds 256 bytes
+                     ("[0, 0, 32]", False),        # b holds 32 bytes
+                     ("[0, -16, 0]", False)):
+        p.write_text(body % offs)
+        assert (model_summary(str(p))[0] == 0) == ok, offs
+
+
 def test_generated_model_is_reference_parsable_subset(tmp_path):
     """Generated graph JSON holds only ints, strings, lists and dicts (what the reference's
     parser accepts) and keeps its four top-level keys."""

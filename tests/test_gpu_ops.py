@@ -377,6 +377,43 @@ def test_gemm_operands_at_offsets_inside_one_storage(tmp_path):
     assert (out[0] == 0).all() and np.abs(out[1] - ctx).max() <= 1e-5 * np.abs(ctx).max()
 
 
+def test_operands_as_channel_ranges_of_a_larger_buffer(tmp_path):
+    """Kernels read and write parts of a storage through `arg_offsets`: one 1x1 convolution with a
+    stacked filter writes [reduction | branch] into a block buffer, a 5x5 and a 3x3 row-form
+    convolution read the reduction as a channel range and write their slices, a max-pool writes
+    its slice directly, the next layers (convolution, average pool, global average pool) read the
+    concatenation as a range that starts inside the storage.  Against the oracle, and the
+    concatenation against numpy slices of the oracle-independent pieces."""
+    C, H, W = 24, 19, 19
+    g = MB.GraphBuilder("views", weight_std=None)
+    x = g.input("data", (C, H, W))
+    # [16 unused | reduction 16 | b1 32 | b5 16 | b3 16 | pool C]
+    S = g.temp((16 + 16 + 32 + 16 + 16 + C, H, W))
+    g.conv2d(x, 16 + 32, 1, out=S, out_channel=16)               # reduction and 1x1 branch at once
+    red = S.channels(16, 16)
+    g.conv2d(red, 16, 5, 1, 2, out=S, out_channel=64)            # staged tile, input at an offset
+    g.conv2d(red, 16, 3, 1, 1, out=S, out_channel=80)            # row form, input at an offset
+    g.pool2d(x, 3, 1, 1, "max", out=S.channels(96, C))
+    cat = S.channels(32, 32 + 16 + 16 + C)                        # the block's output
+    g.conv2d(cat, 40, 1)
+    g.pool2d(cat, 3, 1, 1, "avg", count_include_pad=True)
+    gp = g.global_avgpool(cat)
+    z = g.conv2d(cat, 8, 3, 2, 0)
+    g.mark_output(z)
+    assert sum(1 for k in g.kernels if "arg_offsets" in k) == 7
+    xin = rnd(C, H, W)
+    exe, orc, model = run_both(g, tmp_path, {"data": xin})
+    compare_storages(exe, orc, model, what="operand views")
+    whole = exe.get_data(S.idx, S.size).reshape(-1, H, W)
+    assert (whole[:16] == 0).all()                                # nobody writes in front of its slice
+    pooled = np.pad(xin, ((0, 0), (1, 1), (1, 1)), constant_values=-np.inf)
+    want = np.max([pooled[:, i:i + H, j:j + W] for i in range(3) for j in range(3)], axis=0)
+    np.testing.assert_array_equal(whole[96:], want)              # the pool wrote its slice
+    got_gp = exe.get_data(gp.idx, 88)
+    np.testing.assert_allclose(got_gp, whole[32:].reshape(88, -1).mean(1), rtol=1e-5, atol=1e-6)
+    assert np.isfinite(whole).all()
+
+
 def test_mocked_model_closed_form(tmp_path):
     """The reference's executor_base.mocked_kernel test: a = b = c = 3 -> 18 everywhere
     (src/reef/test/test.cpp:102-116)."""
