@@ -95,9 +95,14 @@ def torch_cpu_baseline(g, x, budget_s=20.0):
                 first, last = ui == 0, ui == n - 1
                 stride = (1 if si == 0 else 2) if first else 1
                 cin = act.shape[1]
-                y = F.relu(F.conv2d(act, take(mid, cin, 1, 1), take(mid), stride=stride))
+                if first:   # conv1 and the projection shortcut: one stacked filter [conv1 | shortcut]
+                    both = F.conv2d(act, take(mid + cout, cin, 1, 1), None, stride=stride)
+                    y = F.relu(both + take(1, mid + cout, 1, 1))[:, :mid]
+                    sc = both[:, mid:]
+                else:
+                    y = F.relu(F.conv2d(act, take(mid, cin, 1, 1), take(mid)))
+                    sc = raw
                 y = F.relu(F.conv2d(y, take(mid, mid, 3, 3), take(mid), padding=1))
-                sc = F.conv2d(act, take(cout, cin, 1, 1), None, stride=stride) if first else raw
                 w3 = take(cout, mid, 1, 1)
                 if last and si == 3:
                     act = F.relu((F.conv2d(y, w3) + sc) * take(1, cout, 1, 1) + take(1, cout, 1, 1))

@@ -172,7 +172,7 @@ class GraphBuilder:
         if residual is not None:
             flags |= F_RESIDUAL
             assert residual.shape == (cout, Ho, Wo), (residual.shape, (cout, Ho, Wo))
-            opt.append(residual.idx)
+            opt.append(residual)
         if affine:
             flags |= F_AFFINE
             if "scale" in given:

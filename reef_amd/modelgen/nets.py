@@ -35,9 +35,15 @@ def image_input(name, shape, seed=rng.BASE_SEED):
 
 
 def resnet(num_layers=152, image=(3, 224, 224), classes=1000, name=None, seed=rng.BASE_SEED,
-           fused_reduce=False, fuse_act=True):
+           fused_reduce=False, fuse_act=True, stack_first=True):
     """fused_reduce: fold split-K inside the conv kernels.  fuse_act: let the unit's last
-    conv also write the next unit's activated input (one kernel instead of conv + add/relu)."""
+    conv also write the next unit's activated input (one kernel instead of conv + add/relu).
+    The first unit of a bottleneck stage has two 1x1 convolutions on the same input with the same
+    stride: conv1 (+bias, ReLU) and the projection shortcut (bare).  They are one convolution
+    with the stacked filter and two outputs: the bare result, whose shortcut rows are the
+    residual of the unit's last convolution, and relu(result + shift), whose conv1 rows feed the
+    3x3 convolution (channel ranges of the two outputs, operand views).  stack_first=False keeps
+    them two launches, as the reference's graph has them."""
     if num_layers >= 50:
         bottleneck = True
         filters = [64, 256, 512, 1024, 2048]
@@ -62,14 +68,20 @@ def resnet(num_layers=152, image=(3, 224, 224), classes=1000, name=None, seed=rn
             last_of_net = last_of_stage and si == n_stages - 1
             stride = (1 if si == 0 else 2) if first else 1
             mid = cout // 4 if bottleneck else cout
-            if bottleneck:
+            if bottleneck and first and stack_first:
+                both, both_act = g.conv2d(act, mid + cout, 1, stride, 0, bias=False, act=ACT_NONE, dual_act=ACT_RELU)
+                y = g.conv2d(both_act.channels(0, mid), mid, 3, 1, 1, bias=True, act=ACT_RELU)
+                shortcut = both.channels(mid, cout)
+                last_k, last_p = 1, 0
+            elif bottleneck:
                 y = g.conv2d(act, mid, 1, stride, 0, bias=True, act=ACT_RELU)
                 y = g.conv2d(y, mid, 3, 1, 1, bias=True, act=ACT_RELU)
+                shortcut = g.conv2d(act, cout, 1, stride, 0, bias=False, act=ACT_NONE) if first else raw
                 last_k, last_p = 1, 0
             else:
                 y = g.conv2d(act, mid, 3, stride, 1, bias=True, act=ACT_RELU)
+                shortcut = g.conv2d(act, cout, 1, stride, 0, bias=False, act=ACT_NONE) if first else raw
                 last_k, last_p = 3, 1
-            shortcut = g.conv2d(act, cout, 1, stride, 0, bias=False, act=ACT_NONE) if first else raw
             if last_of_net:
                 act = g.conv2d(y, cout, last_k, 1, last_p, bias=False, act=ACT_RELU,
                                residual=shortcut, affine=True)

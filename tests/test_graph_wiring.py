@@ -51,7 +51,8 @@ class Params:
 
 
 def test_resnet_generator_equals_the_reference_graph(tmp_path):
-    g = nets.resnet(152, image=(3, 64, 64), fuse_act=False, fused_reduce=True, name="resnet152_64")
+    g = nets.resnet(152, image=(3, 64, 64), fuse_act=False, fused_reduce=True, stack_first=False,
+                    name="resnet152_64")
     ref = json.load(open(REF_JSON))
     table = json.load(open(TABLE))
     # the reference also launches a flatten copy between pooling and classifier; a no-op here
@@ -83,6 +84,54 @@ def test_resnet_generator_equals_the_reference_graph(tmp_path):
     logits_ref = st[dense["args"][2]][:1000]
     logits = np.asarray(orc.storage[model["kernels"][-1]["args"][0]])[:1000]
     assert max_rel_err(logits, logits_ref) <= TOL
+
+
+def test_resnet_bottleneck_wiring_with_stacked_projection(tmp_path):
+    """The generator's default form of a bottleneck ResNet (ResNet-50 at 64 x 64 here): the last
+    convolution of a unit also writes the next unit's activated input, and in the first unit of a
+    stage conv1 and the projection shortcut are one convolution with the stacked filter
+    [conv1 | shortcut] whose two outputs are read back as channel ranges.  Built again from torch
+    functional calls on the generator's parameters."""
+    classes = 24
+    g = nets.resnet(50, image=(3, 64, 64), classes=classes, name="r50s")
+    # conv0 + 3 convolutions per unit (without the stacking the 4 first units would have 4)
+    assert sum(1 for k in g.kernels if k["op"] == "conv2d") == 1 + 3 * 16
+    assert sum(1 for k in g.kernels if "arg_offsets" in k) == 4
+    x = nets.image_input("wiring", (3, 64, 64))
+    _, orc, model = oracle_run(g, tmp_path, "data", x)
+    logits = np.asarray(orc.storage[model["kernels"][-1]["args"][0]])[:classes]
+    P = Params(g)
+    ch = lambda v: v[None, :, None, None]
+    t = torch.from_numpy(x)[None] + ch(P.take(3))
+    t = F.relu(F.conv2d(t, P.take(64, 3, 7, 7), P.take(64), stride=2, padding=3))
+    act = F.relu(F.max_pool2d(t, 3, 2, 1) + ch(P.take(64)))
+    filters, units = [64, 256, 512, 1024, 2048], [3, 4, 6, 3]
+    raw, cin = None, 64
+    for si, n in enumerate(units):
+        cout = filters[si + 1]
+        mid = cout // 4
+        for ui in range(n):
+            stride = (1 if si == 0 else 2) if ui == 0 else 1
+            if ui == 0:
+                both = F.conv2d(act, P.take(mid + cout, cin, 1, 1), None, stride=stride)
+                y = F.relu(both + ch(P.take(mid + cout)))[:, :mid]
+                shortcut = both[:, mid:]
+            else:
+                y = F.relu(F.conv2d(act, P.take(mid, cin, 1, 1), P.take(mid)))
+                shortcut = raw
+            y = F.relu(F.conv2d(y, P.take(mid, mid, 3, 3), P.take(mid), padding=1))
+            z = F.conv2d(y, P.take(cout, mid, 1, 1), None) + shortcut
+            if ui == n - 1 and si == len(units) - 1:
+                act = F.relu(z * ch(P.take(cout)) + ch(P.take(cout)))
+            elif ui == n - 1:
+                act = F.relu(z + ch(P.take(cout)))
+            else:
+                raw = z
+                act = F.relu(raw + ch(P.take(cout)))
+            cin = cout
+    t = F.linear(act.mean(dim=(2, 3)), P.take(classes, 2048), P.take(classes))
+    assert P.done()
+    assert max_rel_err(logits, t.numpy().ravel()) <= TOL
 
 
 def test_mobilenet_v2_wiring(tmp_path):
