@@ -1,7 +1,7 @@
 """The CPU oracle against the reference's OWN device code.
 
 `oracle/_ref/*.raw.co` are the reference's generated kernels (resource/resnet152/resnet152.cu,
-resource/mocked_kernel/mocked_kernel.cu) compiled for gfx950 from where they lie in the reference
+resource/mocked_kernel/mocked_kernel.cu, resource/bert/bert.cu) compiled for gfx950 from where they lie in the reference
 tree (`make -C oracle ref`); `tests/golden/*.json` are the reference's graph files for them.  The
 executor of this build loads that pair like any model directory (kernel names resolve in the code
 object, arguments are the storages in JSON order) and runs ONE reference kernel at a time on
@@ -242,6 +242,140 @@ def test_reference_bandwidth_kernels_match_oracle(ref152):
             raise AssertionError("unexpected kernel " + name)
         print("%-44s wrote %6d elements: oracle agrees" % (name, n))
     assert len(done) == 10
+
+
+def _set_typed(exe, model, idx, values):
+    """A storage of any element type (int64 ids, one-byte masks, float tensors), zero-extended."""
+    st = model["storage"][idx]
+    dt = {"int64": np.int64, "uint1": np.uint8, "byte": np.uint8}.get(st["stype"], np.float32)
+    buf = np.zeros(st["size"], dt)
+    v = np.asarray(values).astype(dt).ravel()
+    buf[:v.size] = v
+    assert lib_ok(B.lib().reef_executor_set_input_idx(exe.h, idx, ctypes.c_void_p(buf.ctypes.data),
+                                                      ctypes.c_size_t(buf.nbytes)))
+    return buf
+
+
+def test_reference_bert_kernels_match_oracle():
+    """The transformer kernels of the reference's BERT (resource/bert/bert.cu: hidden 480, 12 heads of
+    40, sequence 480), each on random operands against the oracle's op: the five calls of a
+    LayerNorm (mean, variance, normalise: bert.cu fused_mean_1 / fused_variance_1 /
+    fused_subtract_add_sqrt_divide_multiply_add_1, eps 1e-12), the mask kernel + the four calls
+    of a softmax (fused_reshape_cast_broadcast_to_like_where, fused_nn_softmax_1_kernel0-3), exact
+    GELU with its bias, the embedding sum, the three batched products, the head split / merge
+    transposes with their bias and scale, and the residual add.  These kernels reduce through
+    shared memory, not through the shuffle that spoils the CNN directories' dense and softmax
+    kernels, so all of them are witnesses.  (The reference lays activations out [feature][token]
+    in places, hence the transposes around the oracle calls below.)"""
+    co = os.path.join(ROOT, "oracle", "_ref", "bert.raw.co")
+    _need(co)
+    path = os.path.join(HERE, "golden", "bert.json")
+    model = json.load(open(path))
+    exe = B.Executor(B.BASE)
+    exe.load(path, co)
+    rng = np.random.default_rng(480)
+    S = Hd = 480
+    heads, hd = 12, 40
+    calls = model["kernels"]
+    first = {}
+    for i, k in enumerate(calls):
+        first.setdefault(k["name"], i)
+    size = lambda i: model["storage"][i]["size"]
+    rnd_into = lambda idx, n=None: _set_typed(exe, model, idx, rng.standard_normal(n or size(idx)))
+    get = lambda idx, n: exe.get_data(idx, size(idx))[:n]
+
+    # LayerNorm: calls mean k0, k1, variance k0, k1, normalise, as the graph wires them
+    i0 = first["fused_mean_1_kernel0"]
+    assert [c["name"] for c in calls[i0:i0 + 5]] == ["fused_mean_1_kernel0", "fused_mean_1_kernel1",
+                                                      "fused_variance_1_kernel0", "fused_variance_1_kernel1",
+                                                      "fused_subtract_add_sqrt_divide_multiply_add_1_kernel0"]
+    a = calls[i0 + 4]["args"]                      # (out, x, mean, variance, gamma, beta)
+    assert a[1] == calls[i0]["args"][0] and a[2] == calls[i0 + 1]["args"][0] and a[3] == calls[i0 + 3]["args"][0]
+    x = rnd_into(a[1])[:S * Hd].reshape(S, Hd) * 3 + 0.5
+    _set_typed(exe, model, a[1], x)
+    gamma, beta = rnd_into(a[4])[:Hd], rnd_into(a[5])[:Hd]
+    for i in range(i0, i0 + 5):
+        exe.execute_kernel(i)
+    assert close(get(a[0], S * Hd), O.layernorm(x, gamma, beta, None, 1e-12)), "layernorm"
+    assert close(get(a[2], S), x.mean(1)) and close(get(a[3], S), x.var(1)), "mean / variance"
+
+    # attention mask + softmax: where(mask, -inf, x), then max, exp, sum, divide
+    i0 = first["fused_reshape_cast_broadcast_to_like_where_kernel0"]
+    assert [c["name"][-20:] for c in calls[i0 + 1:i0 + 5]] == ["nn_softmax_1_kernel%d" % j for j in range(4)]
+    w = calls[i0]["args"]                          # (out, mask, x)
+    mask = (rng.random(S) < 0.3).astype(np.uint8)
+    mask[:4] = 0
+    _set_typed(exe, model, w[1], mask)
+    x = rnd_into(w[2])[:heads * S * S].reshape(heads * S, S) * 4
+    _set_typed(exe, model, w[2], x)
+    for i in range(i0, i0 + 5):
+        exe.execute_kernel(i)
+    out = get(calls[i0 + 4]["args"][0], heads * S * S).reshape(heads * S, S)
+    assert (out[:, mask != 0] == 0).all() and close(out, O.softmax(x, mask)), "masked softmax"
+
+    # exact GELU of (x + bias[feature]) on a [feature][token] tensor
+    i0 = first["fused_reshape_add_multiply_erf_multiply_add_multiply_reshape_kernel0"]
+    a = calls[i0]["args"]                          # (out, x, bias)
+    x, bias = rnd_into(a[1])[:Hd * S].reshape(Hd, S) * 2, rnd_into(a[2])[:Hd]
+    _set_typed(exe, model, a[1], x)
+    exe.execute_kernel(i0)
+    assert close(get(a[0], Hd * S).reshape(Hd, S), O.bias_gelu(np.ascontiguousarray(x.T), bias).T), "gelu"
+
+    # embedding: tok[ids] + pos[position ids]
+    i0 = first["fused_cast_take_broadcast_to_like_cast_take_add_1_kernel0"]
+    a = calls[i0]["args"]                          # (out, tok, ids, pos, position ids)
+    vocab = size(a[1]) // Hd
+    tok = rnd_into(a[1]).reshape(vocab, Hd)
+    pos = rnd_into(a[3]).reshape(-1, Hd)
+    ids = rng.integers(0, vocab, S)
+    _set_typed(exe, model, a[2], ids)
+    _set_typed(exe, model, a[4], np.arange(S))
+    exe.execute_kernel(i0)
+    np.testing.assert_array_equal(get(a[0], S * Hd).reshape(S, Hd), O.embedding(ids, tok, pos[:S]))
+
+    # batched products (B stored [n][k] in all three)
+    for name, (bt, M, N, K) in (("fused_nn_batch_matmul_3_kernel0", (1, S, Hd, Hd)),
+                                 ("fused_nn_batch_matmul_5_kernel0", (heads, S, S, hd)),
+                                 ("fused_nn_batch_matmul_4_kernel0", (heads, S, hd, S))):
+        i0 = first[name]
+        a = calls[i0]["args"]                      # (A, B, C)
+        A = rnd_into(a[0])[:bt * M * K].reshape(bt, M, K)
+        Bm = rnd_into(a[1])[:bt * N * K].reshape(bt, N, K)
+        _set(exe, model, a[2], np.full(size(a[2]), SENTINEL, np.float32))
+        exe.execute_kernel(i0)
+        out = exe.get_data(a[2], size(a[2]))
+        assert (out[:bt * M * N] != SENTINEL).all() and (out[bt * M * N:] == SENTINEL).all(), name
+        assert close(out[:bt * M * N], O.batch_matmul(A, Bm, True, 1.0, True)), name
+
+    # head split [row][head][d] -> [head][row][d] of (x + bias[row]) (and the 1/sqrt(d) of the queries)
+    for name, scale in (("fused_reshape_add_reshape_transpose_divide_reshape_kernel0", 1.0 / np.sqrt(np.float32(hd))),
+                        ("fused_reshape_add_reshape_transpose_transpose_reshape_transpose_kernel0", 1.0)):
+        i0 = first[name]
+        a = calls[i0]["args"]                      # (out, x, bias)
+        x, bias = rnd_into(a[1])[:S * Hd].reshape(S, Hd), rnd_into(a[2])[:S]
+        exe.execute_kernel(i0)
+        want = O.transpose_102(O.eltwise(x, shift=bias).reshape(S, heads, hd)) * np.float32(scale)
+        assert close(get(a[0], S * Hd), want), name
+    # values: (x + bias[feature]) transposed, x stored [feature][token]
+    i0 = first["fused_reshape_add_reshape_transpose_reshape_transpose_kernel0"]
+    a = calls[i0]["args"]
+    x, bias = rnd_into(a[1])[:Hd * S].reshape(Hd, S), rnd_into(a[2])[:Hd]
+    exe.execute_kernel(i0)
+    want = O.transpose_102(O.eltwise(x, shift=bias).reshape(Hd, S, 1))
+    np.testing.assert_array_equal(get(a[0], S * Hd), want.ravel())
+    # head merge [head][token][d] -> [token][head][d]
+    i0 = first["fused_reshape_transpose_copy_reshape_1_kernel0"]
+    a = calls[i0]["args"]
+    x = rnd_into(a[1])[:S * Hd].reshape(heads, S, hd)
+    exe.execute_kernel(i0)
+    np.testing.assert_array_equal(get(a[0], S * Hd), O.transpose_102(x).ravel())
+    # residual: (x + bias[feature]) + res
+    i0 = first["fused_reshape_add_add_kernel0"]
+    a = calls[i0]["args"]                          # (out, x, bias, res)
+    x, bias, res = rnd_into(a[1])[:Hd * S].reshape(Hd, S), rnd_into(a[2])[:Hd], rnd_into(a[3])[:Hd * S].reshape(Hd, S)
+    exe.execute_kernel(i0)
+    assert close(get(a[0], Hd * S), O.eltwise(x, b=res, shift=bias)), "residual add"
+    exe.close()
 
 
 def test_reference_mocked_kernels_closed_form():
