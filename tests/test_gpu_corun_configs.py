@@ -10,6 +10,8 @@ preemption), MobileNetV2 under ResNet-152 (dynamic kernel padding, measured prof
 2 x BERT-base under Inception-v3.  After each co-run EVERY float storage a kernel writes (all
 activations, the logits, split-K partial tensors) is compared with the solo run bit for bit,
 and the logits with the CPU oracle within 1e-4 of the tensor's largest magnitude.
+The last test does the same with two of the reference's OWN model directories, imported
+(reef_amd/legacy.py): resource/resnet18 real-time over two resource/mobilenet best-effort clients.
 """
 import json
 import os
@@ -19,7 +21,9 @@ import pytest
 
 from oracle import oracle as O
 from reef_amd import binding as B
+from reef_amd import legacy
 from reef_amd import profiler
+from reef_amd.modelgen import builder as MB
 from reef_amd.modelgen import nets
 from tests.helpers import max_rel_err, write_model, REL_TOL
 
@@ -28,7 +32,24 @@ pytestmark = pytest.mark.gpu
 NAMES = ("resnet152", "densenet201", "mobilenetv2", "inceptionv3", "bert_base")
 
 
+IMPORTED = {"resnet18": 224, "mobilenet": 224}      # reference model directory -> image side
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def write_imported(name, root):
+    """tests/golden/<name>.json (the reference's graph file) imported onto this build's kernels,
+    with seeded parameters in the reference's own format converted the way a `.param` file is."""
+    ref_json = os.path.join(GOLDEN, name + ".json")
+    g = legacy.import_model(ref_json)
+    d = str(root)
+    g.write(d)
+    MB.write_params(os.path.join(d, name + ".param"), legacy.convert_params(g, legacy.seeded_params(ref_json)))
+    return g, d
+
+
 def model_input(name):
+    if name in IMPORTED:
+        return "data", nets.image_input(name, (3, IMPORTED[name], IMPORTED[name]))
     if name == "bert_base":
         return "input0", nets.token_input(name, 128, 30522)
     side = 299 if name == "inceptionv3" else 224
@@ -58,8 +79,11 @@ class Solo:
 
     def __init__(self, name, root):
         self.name = name
-        self.g = nets.BUILDERS[name]()
-        self.dir = write_model(self.g, root)
+        if name in IMPORTED:
+            self.g, self.dir = write_imported(name, root)
+        else:
+            self.g = nets.BUILDERS[name]()
+            self.dir = write_model(self.g, root)
         profiler.write_profile(self.dir, name, iters=5, warmup=1)
         self.model = json.load(open(os.path.join(self.dir, name + ".json")))
         self.key, self.x = model_input(name)
@@ -186,3 +210,13 @@ def test_cfg5_two_bert_base_under_inceptionv3(solos):
     print("cfg5:", {k: (v.tolist() if hasattr(v, "tolist") else v) for k, v in st.items() if k != "preempt_us"})
     assert st["preempt_times"] >= 10
     assert st["be_preempted"].sum() >= 5 and st["be_completed"].sum() > 0
+
+
+def test_imported_reference_directories_corun(solos):
+    """The reference's resource/resnet18 (its Winograd triples as direct convolutions) as the
+    real-time model over two clients of its resource/mobilenet (depthwise kernels), both imported:
+    preemptions and padded kernels happen, and all three models end with solo bits."""
+    st = corun(solos, "resnet18", "mobilenet", 2, B.MODE_REEF, requests=60, interval_us=1500.0, slack=100)
+    print("imported:", {k: (v.tolist() if hasattr(v, "tolist") else v) for k, v in st.items() if k != "preempt_us"})
+    assert st["preempt_times"] >= 10 and st["be_completed"].sum() > 0
+    assert st["padded_kernels"] > 0
