@@ -18,7 +18,7 @@ order the family name lists them; depthwise convolution: in, W, out, bias; eleme
 flatten and concatenation: out first (TVM lists a concatenation's operands in an order of its own;
 the table says which operand comes first in the result); pooling: in, out; dense: x, W, out, bias).  Tables are packaged for the
 reference's `resnet152`, `mobilenet`, `alexnet`, `vgg` (which holds a pre-activation ResNet-50 at
-64 x 64 under TVM's `tvmgen_default_` kernel names), `resnet18` and `inception` directories.
+64 x 64 under TVM's `tvmgen_default_` kernel names), `resnet18`, `inception` and `bert` directories.
 While it rewrites, the importer follows the tensor shapes through the graph and refuses a table
 that does not fit the graph.
 
@@ -33,6 +33,16 @@ recovers g from a parameter file's U (least squares through G's pseudo-inverse: 
 that is a transform).  G is the Cook-Toom matrix of TVM's interpolation points, which the
 reference does not vendor; it is pinned by running the reference's three kernels on a U made with
 it against the direct convolution (tests/golden/make_graph_shapes.py).
+
+The transformer directory (`bert`: hidden 480, 12 heads, sequence 480).  TVM splits a LayerNorm
+into five calls (two for the mean, two for the variance, one that normalises) and a softmax into
+four behind a call that applies the attention mask; this build has one kernel for each, so the
+leading calls of such a chain get no counterpart and the last one becomes the whole operation on
+the chain's input.  The calls that add a bias along the ROWS of a [480][480] tensor before they
+split heads, transpose or apply GELU become a per-row add followed by the transpose / GELU
+kernel through an added scratch storage.  The 1/sqrt(d) that the query's head split applies is
+moved into the product of queries and keys that follows it (alpha of that GEMM): the query buffer
+holds unscaled values here, every other storage holds what the reference's call leaves there.
 """
 import json
 import os
@@ -111,16 +121,21 @@ def import_model(ref_json_path, table=None, name=None, input_shape=None):
     g.storage = [dict(s) for s in ref["storage"]]
     g.graph_args = list(ref.get("args", []))
     n0 = ref["storage"][0]["size"]
+    if ref["storage"][0]["stype"] != "float32":
+        input_shape = ()                                # token ids: the table says every shape
     if input_shape is None:
         side = int(round((n0 // 3) ** 0.5))
         if 3 * side * side != n0:
             raise ImportError_("cannot tell the input shape from %d elements; pass input_shape" % n0)
         input_shape = (3, side, side)
     shape = {0: tuple(input_shape)}
+    cnn = len(shape[0]) == 3
     wino = {}               # scratch storage -> {"in": input storage[, "U": transformed weights]}
     g.direct_weights = {}   # key of a transformed weight -> (key of its direct copy, tile, Cout, Cin)
     direct_idx = {}
     g.imported_calls = []   # per kernel of this graph: the index of the reference call it replaces
+    chain = {}              # storage a skipped call of a LayerNorm / softmax chain wrote -> what it stands for
+    alpha_of = {}           # storage holding unscaled queries -> the factor its consumer applies
 
     def size(i):
         return g.storage[i]["size"]
@@ -243,7 +258,9 @@ def import_model(ref_json_path, table=None, name=None, input_shape=None):
             shape[a[1]] = (C, 1, 1)
         elif op == "copy":                                      # flatten: (out, in)
             n = e["n"]
-            need(shape.get(a[1], (0,))[0] * shape[a[1]][1] * shape[a[1]][2] == n, k, "shape")
+            if cnn:         # the input's shape is known and must fit
+                need(a[1] in shape and shape[a[1]][0] * shape[a[1]][1] * shape[a[1]][2] == n, k, "shape")
+            need(len(a) == 2 and size(a[1]) >= n and a[0] != a[1], k, "operands")
             g.copy_into(Tensor(a[1], (n,)), tensor(a[0], (n,), k), 0)
             shape[a[0]] = (n, 1, 1)
         elif op == "dense":                                     # (x, W, out, bias)
@@ -252,6 +269,74 @@ def import_model(ref_json_path, table=None, name=None, input_shape=None):
                     out=tensor(a[2], (1, e["out"]), k),
                     w=Tensor(a[1], (e["out"], e["in"])), bias_t=Tensor(a[3], (e["out"],)) if e.get("bias") else None)
             shape[a[2]] = (e["out"], 1, 1)
+        elif op == "chain_stage":
+            # a call of a LayerNorm / softmax chain that has no counterpart: remember what its
+            # result stands for.  `input`: position of the chain's input among the call's operands
+            # (taken over from the stage before it when the call does not see the input itself),
+            # `mask`: position of the attention mask; the call that applies the mask becomes a
+            # copy of the scores (`copy`: elements), so that the softmax kernel, which applies the
+            # mask itself, does not work in place and a restarted launch finds its input intact.
+            src = None
+            for j, i in enumerate(a):
+                if j != e["result"] and i in chain:
+                    src = dict(chain[i])
+            if "input" in e:
+                src = {"x": a[e["input"]]}
+            need(src is not None, k, "a chain stage without its chain")
+            if "mask" in e:
+                src["mask"] = a[e["mask"]]
+            if "copy" in e:
+                need(src["x"] != a[e["result"]], k, "in-place mask")
+                g.copy_into(Tensor(src["x"], (e["copy"],)), tensor(a[e["result"]], (e["copy"],), k), 0)
+                src["x"] = a[e["result"]]
+            chain[a[e["result"]]] = src
+        elif op == "mask_fill":                                 # writes the all-zero mask: storages start as zeros
+            pass
+        elif op == "layernorm":                                 # (out, x, mean, variance, gamma, beta)
+            need(len(a) == 6 and chain.get(a[2], {}).get("x") == a[1] and a[3] in chain, k, "not the end of a LayerNorm chain")
+            g.layernorm(Tensor(a[1], (e["rows"], e["cols"])), e["rows"], e["cols"], eps=e["eps"],
+                        out=tensor(a[0], (e["rows"], e["cols"]), k), gamma=Tensor(a[4], (e["cols"],)),
+                        beta=Tensor(a[5], (e["cols"],)))
+        elif op == "masked_softmax":                            # last call of the chain: (out, exp, sum)
+            src = chain.get(a[1])
+            need(src is not None and "mask" in src and src["x"] != a[0], k, "not the end of a softmax chain")
+            g.softmax(Tensor(src["x"], (e["rows"], e["cols"])), e["rows"], e["cols"],
+                      out=tensor(a[0], (e["rows"], e["cols"]), k), mask=Tensor(src["mask"], (e["cols"],)))
+        elif op == "embedding":                                 # (out, table, ids, position table, position ids)
+            seq, hid = e["seq"], e["hidden"]
+            need(size(a[1]) == e["vocab"] * hid and size(a[3]) == e["positions"] * hid, k, "table sizes")
+            t1 = g.embedding(Tensor(a[2], (seq,)), e["vocab"], seq, hid, pos=False, seg=False, tok=Tensor(a[1], (e["vocab"], hid)))
+            t2 = g.embedding(Tensor(a[4], (seq,)), e["positions"], seq, hid, pos=False, seg=False,
+                             tok=Tensor(a[3], (e["positions"], hid)))
+            g.eltwise(t1, b=t2, out=tensor(a[0], (seq, hid), k))
+        elif op == "gemm_nt":                                   # (A, B, C): C[b] = alpha A[b] B[b]^T
+            bt, M, N, K = e["batch"], e["m"], e["n"], e["k"]
+            need(size(a[0]) >= bt * M * K and size(a[1]) >= bt * N * K, k, "operand sizes")
+            g.gemm(Tensor(a[0], (bt, M, K)), Tensor(a[1], (bt, N, K)), M, N, K, batch=bt, trans_b=True,
+                   alpha=alpha_of.pop(a[0], 1.0), stride_a=M * K if bt > 1 else 0, stride_b=N * K if bt > 1 else 0,
+                   stride_c=M * N if bt > 1 else 0, out=tensor(a[2], (bt, M, N), k))
+        elif op == "rowbias_heads":                             # (out, x, bias): [row][head][d] -> [head][row][d] of x + bias[row]
+            R, H, D = e["rows"], e["heads"], e["d"]
+            t = g.eltwise(Tensor(a[1], (R, H * D)), shift=True, shift_t=Tensor(a[2], (R,)))
+            g.transpose_102(t, R, H, D, out=tensor(a[0], (H, R, D), k))
+            if e.get("scale", 1.0) != 1.0:
+                alpha_of[a[0]] = e["scale"]
+        elif op == "rowbias_transpose":                         # (out, x, bias): out[c][r] = x[r][c] + bias[r]
+            R, C = e["rows"], e["cols"]
+            t = g.eltwise(Tensor(a[1], (R, C)), shift=True, shift_t=Tensor(a[2], (R,)))
+            g.transpose_102(t, R, C, 1, out=tensor(a[0], (C, R, 1), k))
+        elif op == "heads_merge":                               # (out, x): [head][row][d] -> [row][head][d]
+            H, R, D = e["heads"], e["rows"], e["d"]
+            g.transpose_102(Tensor(a[1], (H, R, D)), H, R, D, out=tensor(a[0], (R, H, D), k))
+        elif op == "rowbias_add":                               # (out, x, bias, res): (x + bias[row]) + res
+            R, C = e["rows"], e["cols"]
+            need(a[0] not in (a[1], a[3]), k, "in-place add")
+            g.eltwise(Tensor(a[1], (R, C)), b=Tensor(a[3], (R, C)), shift=True, shift_t=Tensor(a[2], (R,)),
+                      out=tensor(a[0], (R, C), k))
+        elif op == "rowbias_gelu":                              # (out, x, bias): gelu(x + bias[row])
+            R, C = e["rows"], e["cols"]
+            t = g.eltwise(Tensor(a[1], (R, C)), shift=True, shift_t=Tensor(a[2], (R,)))
+            g.bias_gelu(t, R, C, bias=False, out=tensor(a[0], (R, C), k))
         elif op == "softmax":                                   # (in, out)
             need(shape[a[0]][0] == e["cols"], k, "shape")
             g.softmax(Tensor(a[0], (e["rows"], e["cols"])), e["rows"], e["cols"],
@@ -341,6 +426,7 @@ def seeded_params(ref_json_path, table=None, seed=0x5EEF):
         table = json.load(open(table))
     std = {}
     one_plus = set()
+    params = set(param_storages(ref).values())
     transformed = {}                   # storage of a Winograd weight -> (tile, Cout, Cin)
     gemm_of = {}                       # scratch storage a Winograd GEMM wrote -> its weight storage
     for k in ref["kernels"]:
@@ -361,11 +447,17 @@ def seeded_params(ref_json_path, table=None, seed=0x5EEF):
             std[a[1]] = math.sqrt(2.0 / (e["k"] * e["k"]))
         elif e["op"] == "dense":
             std[a[1]] = math.sqrt(2.0 / e["in"])
+        elif e["op"] == "gemm_nt" and a[1] in params:
+            std[a[1]] = math.sqrt(1.0 / e["k"])
+        elif e["op"] == "layernorm":
+            std[a[4]] = 0.1
+            one_plus.add(a[4])
+        elif e["op"] == "embedding":
+            std[a[1]] = std[a[3]] = 0.5
     out = []
-    params = set(param_storages(ref).values())
     for i, s in enumerate(ref["storage"]):
         name = s["name"]
-        if i not in params:
+        if i not in params or s["stype"] != "float32":      # a parameter file holds floats only
             continue
         if i in transformed:           # a seeded direct weight, stored the way the reference stores it
             tile, cout, cin = transformed[i]

@@ -373,11 +373,13 @@ class GraphBuilder:
                    "softmax", 0, 8 * rows * cols, 2.0)
         return out
 
-    def layernorm(self, x, rows, cols, res=None, eps=1e-12):
-        gamma = self.param((cols,), 0.1)
-        self.params[-1] = (self.params[-1][0], self.params[-1][1] + 1.0)
-        beta = self.param((cols,), 0.01)
-        out = self.temp((rows, cols))
+    def layernorm(self, x, rows, cols, res=None, eps=1e-12, out=None, gamma=None, beta=None):
+        if gamma is None:
+            gamma = self.param((cols,), 0.1)
+            self.params[-1] = (self.params[-1][0], self.params[-1][1] + 1.0)
+        if beta is None:
+            beta = self.param((cols,), 0.01)
+        out = Tensor(out.idx, (rows, cols)) if out is not None else self.temp((rows, cols))
         args = [x.idx, gamma.idx, beta.idx, out.idx]
         flags = 0
         if res is not None:
@@ -387,8 +389,8 @@ class GraphBuilder:
                    "layernorm", 0, 4 * rows * cols * (3 if res is not None else 2), 2.0)
         return out
 
-    def bias_gelu(self, x, rows, cols, bias=True):
-        out = self.temp((rows, cols))
+    def bias_gelu(self, x, rows, cols, bias=True, out=None):
+        out = Tensor(out.idx, (rows, cols)) if out is not None else self.temp((rows, cols))
         args = [x.idx, out.idx]
         if bias:
             args.append(self.param((cols,), 0.01).idx)
@@ -396,9 +398,9 @@ class GraphBuilder:
                    "bias_gelu", 0, 8 * rows * cols, 2.0)
         return out
 
-    def embedding(self, ids, vocab, seq, hidden, pos=True, seg=True):
-        tok = self.param((vocab, hidden), self.weight_std or 0.02)
-        out = self.temp((seq, hidden))
+    def embedding(self, ids, vocab, seq, hidden, pos=True, seg=True, tok=None, out=None):
+        tok = tok or self.param((vocab, hidden), self.weight_std or 0.02)
+        out = Tensor(out.idx, (seq, hidden)) if out is not None else self.temp((seq, hidden))
         args = [ids.idx, tok.idx, out.idx]
         flags = 0
         if pos:
@@ -415,8 +417,8 @@ class GraphBuilder:
         self._emit("reef_copy", math.ceil(src.size / 1024), [src.idx, dst.idx], [src.size, dst_off],
                    "copy", 0, 8 * src.size, 2.0)
 
-    def transpose_102(self, x, d0, d1, d2, bias=None):
-        out = self.temp((d1, d0, d2))
+    def transpose_102(self, x, d0, d1, d2, bias=None, out=None):
+        out = Tensor(out.idx, (d1, d0, d2)) if out is not None else self.temp((d1, d0, d2))
         args = [x.idx, out.idx]
         flags = 0
         if bias is not None:

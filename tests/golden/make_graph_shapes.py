@@ -10,6 +10,11 @@ walked from the input with every kernel witnessed on the way:
              epilogue) on TRANSFORMED weights
   inception  Inception-v3 at 299 x 299: 1x7 / 7x1 / 1x3 / 3x1 / 5x5 filters, Winograd triples with
              and without padding, average pools, channel concatenations
+  bert       a 6-layer transformer encoder (hidden 480, 12 heads of 40, sequence 480).  Its shapes
+             follow from the storage sizes; what each kernel computes is witnessed by
+             tests/test_gpu_reference_kernels.py::test_reference_bert_kernels_match_oracle, which
+             this script runs before it writes the table (LayerNorm and softmax are chains of
+             five calls each there; the table marks the calls that only carry a chain forward)
 
 For every kernel name: what it computes -- op, shape, filter, stride, padding, epilogue.  The
 shapes are baked into the generated source and the graph JSON only holds shared, maximal buffer
@@ -29,7 +34,7 @@ reef_amd.legacy.winograd_transform (output tile 4 or 2, weight layout [e][n][Cin
 what the oracle's DIRECT convolution of g gives (to 1e-4 of the largest output: two summation
 orders and the transform's own rounding).  That pins the transform matrix the importer inverts.
 
-Needs a GPU:  python tests/golden/make_graph_shapes.py mobilenet|alexnet|vgg|resnet18|inception
+Needs a GPU:  python tests/golden/make_graph_shapes.py mobilenet|alexnet|vgg|resnet18|inception|bert
 The result is committed as tests/golden/<model>_kernel_shapes.json (fixture) and as
 reef_amd/legacy_tables/<model>.json (the importer's table for that model directory)."""
 import json
@@ -334,9 +339,58 @@ def derive(name):
     return table
 
 
+def derive_bert():
+    model = json.load(open(os.path.join(HERE, "bert.json")))
+    size = lambda i: model["storage"][i]["size"]
+    first = {}
+    for k in model["kernels"]:
+        first.setdefault(k["name"], k["args"])
+    emb = first["fused_cast_take_broadcast_to_like_cast_take_add_1_kernel0"]      # (out, table, ids, positions, position ids)
+    S = size(emb[2])
+    H = size(first["fused_subtract_add_sqrt_divide_multiply_add_1_kernel0"][4])     # gamma
+    assert size(first["fused_nn_batch_matmul_3_kernel0"][1]) == H * H
+    heads, d = 12, 40           # grid z of fused_nn_batch_matmul_5 and the `% 40` of the head split (bert.cu)
+    assert heads * d == H and size(first["fused_nn_softmax_1_kernel3"][0]) == heads * S * S
+    T.test_reference_bert_kernels_match_oracle()         # every family below, on random operands
+    scale = float(np.float32(1.0) / np.sqrt(np.float32(d)))
+    table = {
+        "fused_full_equal_reshape_kernel0": {"op": "mask_fill", "n": S},
+        "fused_cast_take_broadcast_to_like_cast_take_add_1_kernel0":
+            {"op": "embedding", "vocab": size(emb[1]) // H, "positions": size(emb[3]) // H, "seq": S, "hidden": H},
+        "fused_mean_1_kernel0": {"op": "chain_stage", "input": 0, "result": 1},
+        "fused_mean_1_kernel1": {"op": "chain_stage", "result": 0},
+        "fused_variance_1_kernel0": {"op": "chain_stage", "input": 0, "result": 2},
+        "fused_variance_1_kernel1": {"op": "chain_stage", "result": 0},
+        "fused_subtract_add_sqrt_divide_multiply_add_1_kernel0": {"op": "layernorm", "rows": S, "cols": H, "eps": 1e-12},
+        "fused_reshape_4_kernel0": {"op": "copy", "n": S * H},
+        "fused_reshape_5_kernel0": {"op": "copy", "n": heads * S * S},
+        "fused_nn_batch_matmul_3_kernel0": {"op": "gemm_nt", "batch": 1, "m": S, "n": H, "k": H},
+        "fused_nn_batch_matmul_5_kernel0": {"op": "gemm_nt", "batch": heads, "m": S, "n": S, "k": d},
+        "fused_nn_batch_matmul_4_kernel0": {"op": "gemm_nt", "batch": heads, "m": S, "n": d, "k": S},
+        "fused_reshape_add_reshape_transpose_divide_reshape_kernel0":
+            {"op": "rowbias_heads", "rows": S, "heads": heads, "d": d, "scale": scale},
+        "fused_reshape_add_reshape_transpose_transpose_reshape_transpose_kernel0":
+            {"op": "rowbias_heads", "rows": S, "heads": heads, "d": d},
+        "fused_reshape_add_reshape_transpose_reshape_transpose_kernel0": {"op": "rowbias_transpose", "rows": H, "cols": S},
+        "fused_reshape_transpose_copy_reshape_1_kernel0": {"op": "heads_merge", "heads": heads, "rows": S, "d": d},
+        "fused_reshape_cast_broadcast_to_like_where_kernel0":
+            {"op": "chain_stage", "input": 2, "mask": 1, "result": 0, "copy": heads * S * S},
+        "fused_nn_softmax_1_kernel0": {"op": "chain_stage", "result": 0},
+        "fused_nn_softmax_1_kernel1": {"op": "chain_stage", "result": 0},
+        "fused_nn_softmax_1_kernel2": {"op": "chain_stage", "result": 0},
+        "fused_nn_softmax_1_kernel3": {"op": "masked_softmax", "rows": heads * S, "cols": S},
+        "fused_reshape_add_add_kernel0": {"op": "rowbias_add", "rows": H, "cols": S},
+        "fused_reshape_add_multiply_erf_multiply_add_multiply_reshape_kernel0": {"op": "rowbias_gelu", "rows": H, "cols": S},
+    }
+    assert set(table) == {k["name"] for k in model["kernels"]}
+    for e in table.values():
+        e["witness"] = True
+    return table
+
+
 def main():
     name = sys.argv[1]
-    table = derive(name)
+    table = derive_bert() if name == "bert" else derive(name)
     for out in (os.path.join(HERE, name + "_kernel_shapes.json"),
                 os.path.join(ROOT, "reef_amd", "legacy_tables", name + ".json"),
                 os.path.join(ROOT, "gpurun_out", name + "_kernel_shapes.json")):

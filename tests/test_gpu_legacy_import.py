@@ -181,3 +181,80 @@ def test_imported_walked_models_track_the_reference_kernels_call_by_call(name, s
     assert abs(float(probs.sum()) - 1.0) < 1e-4
     theirs.close()
     ours.close()
+
+
+def test_imported_bert_tracks_the_reference_kernels_call_by_call(tmp_path):
+    """resource/bert (6 layers, hidden 480, 12 heads, sequence 480; 205 calls): every call that has
+    a counterpart here is compared with what the reference's own kernel left in the same storage,
+    both executors running free from the token ids to the last LayerNorm.  The calls inside a
+    LayerNorm or softmax chain have none (one kernel does the chain); the query head split holds
+    unscaled values here (its 1/sqrt(d) is the alpha of the product that follows) and is compared
+    after scaling; the mask call is a copy here, identical under the all-zero mask the graph makes."""
+    name = "bert"
+    co = os.path.join(os.path.dirname(HERE), "oracle", "_ref", name + ".raw.co")
+    _need(co)
+    ref_json = os.path.join(HERE, "golden", name + ".json")
+    ref = json.load(open(ref_json))
+    roles = json.load(open(os.path.join(HERE, "golden", name + "_kernel_roles.json")))
+    table = legacy.load_table(name)
+    g = legacy.import_model(ref_json)
+    d = str(tmp_path)
+    g.write(d)
+    params = legacy.seeded_params(ref_json)
+    MB.write_params(os.path.join(d, name + ".param"), legacy.convert_params(g, params))
+    mine_of = {}
+    for j, call in enumerate(g.imported_calls):
+        mine_of.setdefault(call, []).append(j)
+    ids = nets.token_input("legacy", 480, 30522)
+    position_ids = np.arange(480, dtype=np.int64)        # parameter p2: int64, not in a float parameter file
+    pos_idx = ref["kernels"][1]["args"][4]
+    assert ref["storage"][pos_idx]["stype"] == "int64"
+
+    def set_raw(exe, idx, arr):
+        arr = np.ascontiguousarray(arr)
+        st = B.lib().reef_executor_set_input_idx(exe.h, idx, ctypes.c_void_p(arr.ctypes.data), ctypes.c_size_t(arr.nbytes))
+        assert st == 0, B.last_error()
+
+    theirs = B.Executor(B.BASE)
+    theirs.load(ref_json, co)
+    index = legacy.param_storages(ref)
+    for key, arr in params:
+        _set_idx(theirs, index[key], arr)
+    ours = B.Executor.from_dir(d, name, B.BASE)
+    for exe in (theirs, ours):
+        set_raw(exe, 0, ids)
+        set_raw(exe, pos_idx, position_ids)
+
+    compared = stages = 0
+    worst = 0.0
+    for i, k in enumerate(ref["kernels"]):
+        theirs.execute_kernel(i)
+        e = table[k["name"]]
+        if i not in mine_of:
+            assert e["op"] in ("chain_stage", "mask_fill"), k["name"]
+            stages += 1
+            continue
+        for j in mine_of[i]:
+            ours.execute_kernel(j)
+        if e["op"] == "chain_stage":                 # the mask call: a copy here
+            stages += 1
+            continue
+        names = roles[k["name"]]
+        out_idx = k["args"][[j for j, n in enumerate(names) if n.startswith(("T_", "compute"))][0]]
+        size = ref["storage"][out_idx]["size"]
+        n = {"gemm_nt": e.get("batch", 0) * e.get("m", 0) * e.get("n", 0)}.get(e["op"], 0) or \
+            e.get("n") or e.get("rows", 0) * e.get("cols", 0) or e.get("rows", 0) * e.get("heads", 0) * e.get("d", 0) \
+            or e.get("seq", 0) * e.get("hidden", 0)
+        assert 0 < n <= size, (k["name"], n)
+        mine = ours.get_data(out_idx, size)[:n] * np.float32(e.get("scale", 1.0))
+        want = theirs.get_data(out_idx, size)[:n]
+        scale = max(float(np.abs(want).max()), 1e-20)
+        err = float(np.abs(mine - want).max()) / scale
+        worst = max(worst, err)
+        assert np.isfinite(mine).all() and err <= TOL, (i, k["name"], err)
+        compared += 1
+    print("bert: %d calls free-running against the reference's kernels, worst deviation %.2e; %d chain stages"
+          % (compared, worst, stages))
+    assert compared + stages == 205 and stages == 1 + 13 * 4 + 6 * 4
+    theirs.close()
+    ours.close()

@@ -9,6 +9,7 @@ make_graph_shapes.py).
 The CPU check interprets the reference graph DIRECTLY from the table with the oracle's ops and
 compares that with the imported model run through the executor (fake backend) -- two code paths
 from the same table, so a wrong role, attribute order or epilogue flag in the importer shows."""
+import ctypes
 import json
 import os
 
@@ -321,6 +322,128 @@ def test_imported_walked_model_equals_the_table_interpretation_through_the_execu
                 assert np.abs(have - want[i]).max() <= 1e-5 * scale, (i, s)
         out_idx = [i for i, s in enumerate(ref["storage"]) if s["name"] == "output"][0]
         assert abs(float(exe.get_data(out_idx, ref["storage"][out_idx]["size"])[:1000].sum()) - 1.0) < 1e-4
+    finally:
+        if exe is not None:
+            exe.close()
+        fake.remove()
+
+
+# ---- the transformer directory --------------------------------------------------------------
+def interpret_bert_graph(ref, table, params, ids, position_ids):
+    """resource/bert evaluated call by call from the table with the oracle's ops: every call of a
+    LayerNorm / softmax chain is computed as its own step (mean, variance, ...), the way the
+    reference runs it.  Returns the storages."""
+    dt = {"int64": np.int64, "uint1": np.uint8, "byte": np.uint8}
+    st = {i: np.zeros(s["size"], dt.get(s["stype"], np.float32)) for i, s in enumerate(ref["storage"])}
+    for i, s in enumerate(ref["storage"]):
+        if s["name"] in params:
+            st[i][:] = params[s["name"]]
+    st[0][:] = ids
+    st[ref["kernels"][1]["args"][4]][:] = position_ids
+    f32 = lambda i: st[i].view(np.float32) if st[i].dtype != np.float32 else st[i]   # byte scratch holds floats
+    for k in ref["kernels"]:
+        name, a = k["name"], k["args"]
+        e = table[name]
+        if name.startswith("fused_full_equal"):
+            st[a[0]][:e["n"]] = 0
+        elif e["op"] == "embedding":
+            S, H = e["seq"], e["hidden"]
+            y = st[a[1]].reshape(-1, H)[st[a[2]][:S]] + st[a[3]].reshape(-1, H)[st[a[4]][:S]]
+            st[a[0]][:S * H] = y.ravel()
+        elif name.startswith("fused_mean_1_kernel0"):
+            f32(a[1])[:480] = st[a[0]][:480 * 480].reshape(480, 480).sum(1, dtype=np.float64)
+        elif name.startswith("fused_mean_1_kernel1"):
+            st[a[0]][:480] = f32(a[1])[:480] / 480
+        elif name.startswith("fused_variance_1_kernel0"):
+            x = st[a[0]][:480 * 480].reshape(480, 480).astype(np.float64)
+            f32(a[2])[:480] = ((x - st[a[1]][:480, None]) ** 2).sum(1)
+        elif name.startswith("fused_variance_1_kernel1"):
+            st[a[0]][:480] = f32(a[1])[:480] / 480
+        elif e["op"] == "layernorm":
+            R, C = e["rows"], e["cols"]
+            x = st[a[1]][:R * C].reshape(R, C).astype(np.float64)
+            y = (x - st[a[2]][:R, None]) / np.sqrt(st[a[3]][:R, None].astype(np.float64) + e["eps"]) * st[a[4]][:C] + st[a[5]][:C]
+            st[a[0]][:R * C] = y.ravel()
+        elif e["op"] == "copy":
+            st[a[0]][:e["n"]] = st[a[1]][:e["n"]]
+        elif e["op"] == "gemm_nt":
+            bt, M, N, K = e["batch"], e["m"], e["n"], e["k"]
+            y = O.batch_matmul(st[a[0]][:bt * M * K].reshape(bt, M, K), st[a[1]][:bt * N * K].reshape(bt, N, K), True, 1.0)
+            st[a[2]][:y.size] = y.ravel()
+        elif e["op"] == "rowbias_heads":
+            R, Hh, D = e["rows"], e["heads"], e["d"]
+            x = st[a[1]][:R * Hh * D].reshape(R, Hh, D) + st[a[2]][:R, None, None]
+            st[a[0]][:x.size] = (x.transpose(1, 0, 2) * np.float32(e.get("scale", 1.0))).ravel()
+        elif e["op"] == "rowbias_transpose":
+            R, C = e["rows"], e["cols"]
+            st[a[0]][:R * C] = (st[a[1]][:R * C].reshape(R, C) + st[a[2]][:R, None]).T.ravel()
+        elif e["op"] == "heads_merge":
+            Hh, R, D = e["heads"], e["rows"], e["d"]
+            st[a[0]][:Hh * R * D] = st[a[1]][:Hh * R * D].reshape(Hh, R, D).transpose(1, 0, 2).ravel()
+        elif name.startswith("fused_reshape_cast_broadcast_to_like_where"):
+            n = e["copy"]
+            x = st[a[2]][:n].reshape(-1, 480)
+            st[a[0]][:n] = np.where(st[a[1]][:480][None, :] != 0, -np.inf, x).ravel()
+        elif name.startswith("fused_nn_softmax_1_kernel0"):              # row maxima
+            f32(a[0])[:12 * 480] = st[a[1]][:12 * 480 * 480].reshape(-1, 480).max(1)
+        elif name.startswith("fused_nn_softmax_1_kernel1"):              # exp(x - max)
+            x = st[a[1]][:12 * 480 * 480].reshape(-1, 480)
+            f32(a[0])[:x.size] = np.exp(x - f32(a[2])[:12 * 480, None]).ravel()
+        elif name.startswith("fused_nn_softmax_1_kernel2"):              # row sums
+            f32(a[0])[:12 * 480] = f32(a[1])[:12 * 480 * 480].reshape(-1, 480).sum(1, dtype=np.float64)
+        elif e["op"] == "masked_softmax":
+            R, C = e["rows"], e["cols"]
+            st[a[0]][:R * C] = (f32(a[1])[:R * C].reshape(R, C) / f32(a[2])[:R, None]).ravel()
+        elif e["op"] == "rowbias_add":
+            R, C = e["rows"], e["cols"]
+            st[a[0]][:R * C] = ((st[a[1]][:R * C].reshape(R, C) + st[a[2]][:R, None]) + st[a[3]][:R * C].reshape(R, C)).ravel()
+        elif e["op"] == "rowbias_gelu":
+            R, C = e["rows"], e["cols"]
+            st[a[0]][:R * C] = O.bias_gelu((st[a[1]][:R * C].reshape(R, C) + st[a[2]][:R, None]).astype(np.float32)).ravel()
+        else:
+            raise AssertionError(name)
+    return st
+
+
+def test_imported_bert_equals_the_call_by_call_interpretation(tmp_path):
+    """resource/bert: 205 calls -> 160 kernels (a LayerNorm's five calls and a softmax's five become
+    one kernel each, a row-bias call two); the imported graph through the executor (recording
+    backend) gives what the reference's call sequence gives when every call is evaluated as its
+    own step."""
+    name = "bert"
+    ref = json.load(open(golden(name)))
+    table = legacy.load_table(name)
+    assert table == json.load(open(golden(name, "_kernel_shapes"))) and all(e["witness"] for e in table.values())
+    g = legacy.import_model(golden(name))
+    d = str(tmp_path)
+    g.write(d)
+    out = json.load(open(os.path.join(d, name + ".json")))
+    n = len(ref["storage"])
+    assert out["storage"][:n] == ref["storage"] and len(ref["kernels"]) == 205 and len(out["kernels"]) == 160
+    skipped = [i for i, k in enumerate(ref["kernels"]) if i not in g.imported_calls]
+    assert len(skipped) == 1 + 13 * 4 + 6 * 3 and all(table[ref["kernels"][i]["name"]]["op"] in ("chain_stage", "mask_fill")
+                                                      for i in skipped)
+    params = legacy.seeded_params(golden(name))
+    assert len(params) == 100 and "p2" not in dict(params)      # the int64 position ids are not a float parameter
+    MB.write_params(os.path.join(d, name + ".param"), legacy.convert_params(g, params))
+    ids = nets.token_input("legacy", 480, 30522)
+    pos = np.arange(480, dtype=np.int64)
+    want = interpret_bert_graph(ref, table, dict(params), ids, pos)
+    fake = FakeHal().install()
+    exe = None
+    try:
+        exe = B.Executor.from_dir(d, name, B.HYBRID)
+        for idx, arr in ((0, ids), (ref["kernels"][1]["args"][4], pos)):
+            arr = np.ascontiguousarray(arr, np.int64)
+            assert B.lib().reef_executor_set_input_idx(exe.h, idx, ctypes.c_void_p(arr.ctypes.data),
+                                                       ctypes.c_size_t(arr.nbytes)) == 0
+        exe.execute()
+        out_idx = [i for i, s in enumerate(ref["storage"]) if s["name"] == "output"][0]
+        got = exe.get_data(out_idx, 480 * 480)
+        assert np.isfinite(got).all()
+        assert np.abs(got - want[out_idx][:got.size]).max() <= 1e-4 * np.abs(want[out_idx]).max()
+        rows = got.reshape(480, 480)
+        assert np.abs(rows.mean(1)).max() < 0.2     # the last call is a LayerNorm with gamma ~ 1, beta ~ 0
     finally:
         if exe is not None:
             exe.close()
