@@ -156,24 +156,24 @@ def densenet(blocks=(6, 12, 48, 32), growth=32, image=(3, 224, 224), classes=100
     of the concatenation buffer."""
     g = GraphBuilder(name, seed)
     x = g.input("data", image)
-    x = g.conv2d(x, 2 * growth, 7, 2, 3, bias=True, act=ACT_RELU)
-    x = g.pool2d(x, 3, 2, 1, "max")
+    y = g.conv2d(x, 2 * growth, 7, 2, 3, bias=True, act=ACT_RELU)
     c = 2 * growth
     for bi, n_layers in enumerate(blocks):
-        _, H, W = x.shape
+        # the pool in front of a block writes the first channels of the block's buffer itself
+        pool = (3, 2, 1, "max") if bi == 0 else (2, 2, 0, "avg")
+        H = (y.shape[1] + 2 * pool[2] - pool[0]) // pool[1] + 1
+        W = (y.shape[2] + 2 * pool[2] - pool[0]) // pool[1] + 1
         total = c + n_layers * growth
         buf = g.temp((total, H, W))
-        g.copy_into(x, buf, 0)
+        g.pool2d(y, *pool, out=buf.channels(0, c))
         for li in range(n_layers):
             cur = c + li * growth
-            view = type(x)(buf.idx, (cur, H, W))          # first `cur` channels of the buffer
-            y = g.conv2d(view, 4 * growth, 1, 1, 0, bias=True, act=ACT_RELU, pre_act=True)
+            y = g.conv2d(buf.channels(0, cur), 4 * growth, 1, 1, 0, bias=True, act=ACT_RELU, pre_act=True)
             g.conv2d(y, growth, 3, 1, 1, bias=False, act=ACT_NONE, out=buf, out_channel=cur)
         c = total
         x = buf
         if bi != len(blocks) - 1:
             y = g.conv2d(x, c // 2, 1, 1, 0, bias=False, act=ACT_NONE, pre_act=True)
-            x = g.pool2d(y, 2, 2, 0, "avg")
             c = c // 2
     a = g.eltwise(x, scale=True, shift=True, act=ACT_RELU)
     pooled = g.global_avgpool(a)
