@@ -299,6 +299,33 @@ def test_inception_import_has_asymmetric_filters_padded_pools_and_concatenations
         legacy.import_model(golden(name), table=bad)
 
 
+def test_import_model_dir_converts_a_parameter_file_with_transformed_weights(tmp_path):
+    """A directory laid out like the reference's (resnet18.json + resnet18.param holding the
+    Winograd weights transformed) -> a directory of this build: graph, profile, code objects, and
+    a parameter file in which every transformed weight has become its direct filter; a directory
+    without Winograd kernels keeps its parameter file byte for byte."""
+    import shutil
+    for name in ("resnet18", "alexnet"):
+        src, dst = tmp_path / (name + "_ref"), tmp_path / (name + "_out")
+        src.mkdir()
+        shutil.copyfile(golden(name), src / (name + ".json"))
+        params = legacy.seeded_params(golden(name))
+        MB.write_params(str(src / (name + ".param")), params)
+        g = legacy.import_model_dir(str(src), name, str(dst))
+        for ext in (".json", ".profile.json", ".param", ".raw.co", ".be.co", ".trans.co"):
+            assert (dst / (name + ext)).exists(), ext
+        got = legacy.read_params(str(dst / (name + ".param")))
+        if name == "alexnet":
+            assert not g.direct_weights
+            assert (dst / (name + ".param")).read_bytes() == (src / (name + ".param")).read_bytes()
+            continue
+        keys = [k for k, _ in got]
+        assert len(g.direct_weights) == 13 and all(k + "_direct" in keys and k not in keys for k in g.direct_weights)
+        assert len(keys) == len(params)
+        storages = {s_["name"]: s_["size"] for s_ in json.load(open(dst / (name + ".json")))["storage"]}
+        assert all(storages[k] == a.size for k, a in got)          # every parameter fits the storage of its name
+
+
 @pytest.mark.parametrize("name,side", [("mobilenet", 224), ("vgg", 64), ("resnet18", 224), ("inception", 299)])
 def test_imported_walked_model_equals_the_table_interpretation_through_the_executor(name, side, tmp_path):
     d = str(tmp_path)
