@@ -24,9 +24,12 @@ Also here: REEFClient / ModelHandle, the Python mirror of src/reef/client/client
 the three command lines of src/example (`python -m reef_amd.rpc server|client|client_cont ...`).
 """
 import ctypes
+import json
 import mmap
 import os
+import shutil
 import sys
+import tempfile
 import threading
 import time
 from concurrent import futures
@@ -120,9 +123,12 @@ class SharedMemory:
 class REEFServer:
     """server/server.{h,cpp}: owns one scheduler (REEF mode, server.cpp:11) and the blobs."""
 
-    def __init__(self, addr=DEFAULT_REEF_ADDR, mode=B.MODE_REEF, max_workers=16):
+    def __init__(self, addr=DEFAULT_REEF_ADDR, mode=B.MODE_REEF, max_workers=16, measure_imported=True):
         self.addr = addr
         self.scheduler = B.Scheduler(mode)
+        self.measure_imported = measure_imported   # profile an imported directory on the device (else: estimates)
+        self.import_root = None                    # where directories of the reference are imported to
+        self.import_mtx = threading.Lock()
         self.shms = {}                       # key -> (mid, name, SharedMemory)
         self.shm_mtx = threading.Lock()
         self.server = grpc.server(futures.ThreadPoolExecutor(max_workers=max_workers))
@@ -152,6 +158,9 @@ class REEFServer:
             for _, _, shm in self.shms.values():
                 shm.close()
             self.shms.clear()
+        if self.import_root is not None:
+            shutil.rmtree(self.import_root, ignore_errors=True)
+            self.import_root = None
 
     # ---- handlers ----
     def SetPriority(self, request, context):
@@ -162,9 +171,34 @@ class REEFServer:
             reply.qid = qid
         return reply
 
+    def _model_dir(self, model_dir, name):
+        """A directory written by the reference's own pipeline (generated kernel names, no `op`
+        keys; scheduler.cpp:62-65 names its files) cannot be loaded as it is: its code objects are
+        for another GPU.  Where a kernel table is packaged for it (reef_amd/legacy.py), it is
+        imported once into a directory of this server and loaded from there, so a client of the
+        reference can keep sending the paths it always sent."""
+        from . import legacy
+        try:
+            with open(os.path.join(model_dir, name + ".json")) as f:
+                kernels = json.load(f).get("kernels") or []
+        except (OSError, ValueError):
+            return model_dir
+        if not kernels or "op" in kernels[0] or not os.path.exists(os.path.join(legacy.TABLE_DIR, name + ".json")):
+            return model_dir
+        with self.import_mtx:
+            if self.import_root is None:
+                self.import_root = tempfile.mkdtemp(prefix="reef_imported_")
+            out = os.path.join(self.import_root, name)
+            if not os.path.exists(os.path.join(out, name + ".json")):
+                try:
+                    legacy.import_model_dir(model_dir, name, out, measured_profile=self.measure_imported)
+                except (legacy.ImportError_, OSError, RuntimeError):
+                    return model_dir
+        return out
+
     def LoadModel(self, request, context):
         reply = MSG["LoadModelReply"]()
-        prefix = request.dir + "/" + request.name
+        prefix = self._model_dir(request.dir, request.name) + "/" + request.name
         param = prefix + ".param"
         if not os.access(param, os.F_OK):
             param = ""

@@ -70,3 +70,43 @@ def test_rpc_round_trip_on_the_device(tmp_path_factory):
         c.close()
     finally:
         server.shutdown()
+
+
+def test_rpc_load_model_takes_a_directory_of_the_reference(tmp_path):
+    """The reference's resource/resnet18 as its pipeline wrote it (graph with TVM's kernel names, a
+    parameter file holding the Winograd weights transformed) sent to LoadModel as it is: the
+    server imports it, times its kernels for the profile, and the client's inference through
+    shared memory gives the probabilities the oracle gives for the imported graph."""
+    import shutil
+    from reef_amd import legacy
+    from reef_amd.modelgen import builder as MB
+    name = "resnet18"
+    golden = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", name + ".json")
+    ref_dir = tmp_path / "resource" / name
+    ref_dir.mkdir(parents=True)
+    shutil.copyfile(golden, ref_dir / (name + ".json"))
+    MB.write_params(str(ref_dir / (name + ".param")), legacy.seeded_params(golden))
+    x = nets.image_input("rpc", (3, 224, 224))
+    server = rpc.REEFServer("127.0.0.1:0")
+    server.run()
+    try:
+        c = rpc.REEFClient("127.0.0.1:%d" % server.port)
+        c.init(True)
+        m = c.load_model(str(ref_dir), name)
+        imported = os.path.join(server.import_root, name)
+        prof = json.load(open(os.path.join(imported, name + ".profile.json")))
+        assert prof["model_latency"] > 0 and len(prof["kernel_latency"]) == 31
+        orc = O.GraphOracle(json.load(open(os.path.join(imported, name + ".json"))), os.path.join(imported, name + ".param"))
+        orc.set_input("data", x)
+        want = orc.run().copy()
+        m.get_input_blob("data").array()[:] = x.ravel()
+        m.load_input()
+        _, lat = m.infer()
+        out = m.get_output_blob("output")
+        m.get_output()
+        got = out.array()[:1000]
+        assert abs(float(got.sum()) - 1.0) < 1e-4 and max_rel_err(got, want[:1000]) <= REL_TOL
+        print("imported resnet18 over rpc: %.2f ms" % (lat * 1e3))
+        c.close()
+    finally:
+        server.shutdown()

@@ -21,7 +21,7 @@ from tests.helpers import write_model
 def served(tmp_path_factory):
     fake = FakeHal().install()
     fake.lib.fake_hal_set_auto_progress(4)
-    server = rpc.REEFServer("127.0.0.1:0")
+    server = rpc.REEFServer("127.0.0.1:0", measure_imported=False)    # no device to time kernels on here
     server.run()
     dirs = {}
     for g in (nets.mocked_kernel(), nets.resnet(18, image=(3, 32, 32), classes=16, name="tiny18")):
@@ -109,3 +109,47 @@ def test_failures_answer_succ_false_with_status_ok(served):
     r = call("SetPriority", b"")                                                     # rt = false
     assert r.succ and r.qid == 0
     ch.close()
+
+
+def test_load_model_imports_a_directory_of_the_reference(served, tmp_path):
+    """A client sends the path of a directory as the reference's pipeline wrote it (alexnet.json with
+    TVM's kernel names, alexnet.param with its keys; the code objects there are for another GPU and
+    are never opened): LoadModel imports it and the inference gives what the table's
+    interpretation of the reference graph gives."""
+    import shutil
+    from reef_amd import legacy
+    from reef_amd.modelgen import builder as MB
+    from tests.test_legacy_import import golden, interpret_reference_graph
+    server, addr, _ = served
+    name = "alexnet"
+    ref_dir = tmp_path / "resource" / name
+    ref_dir.mkdir(parents=True)
+    shutil.copyfile(golden(name), ref_dir / (name + ".json"))
+    params = legacy.seeded_params(golden(name))
+    MB.write_params(str(ref_dir / (name + ".param")), params)
+    (ref_dir / (name + ".trans.co")).write_bytes(b"not for this GPU")
+    x = nets.image_input("rpc", (3, 224, 224))
+    ref = json.load(open(golden(name)))
+    want = interpret_reference_graph(ref, legacy.load_table(name), dict(params), x)
+    out_idx = [i for i, s in enumerate(ref["storage"]) if s["name"] == "output"][0]
+
+    client = rpc.REEFClient(addr)
+    client.init(True)
+    m = client.load_model(str(ref_dir), name)
+    assert server.import_root and os.path.exists(os.path.join(server.import_root, name, name + ".be.co"))
+    inp = m.get_input_blob("data")
+    inp.array()[:] = x.ravel()
+    m.load_input()
+    m.infer()
+    out = m.get_output_blob("output")
+    m.get_output()
+    got = out.array()[:1000]
+    assert abs(float(got.sum()) - 1.0) < 1e-4
+    np.testing.assert_allclose(got, want[out_idx][:1000], rtol=0, atol=1e-6)
+    # a directory of the reference without a packaged table is answered like any other failure
+    other = tmp_path / "resource" / "nonet"
+    other.mkdir()
+    shutil.copyfile(golden(name), other / "nonet.json")
+    reply = client.calls["LoadModel"](rpc.MSG["LoadModelRequest"](dir=str(other), name="nonet", qid=client.qid))
+    assert reply.succ is False
+    client.close()
