@@ -305,7 +305,7 @@ def test_import_model_dir_converts_a_parameter_file_with_transformed_weights(tmp
     a parameter file in which every transformed weight has become its direct filter; a directory
     without Winograd kernels keeps its parameter file byte for byte."""
     import shutil
-    for name in ("resnet18", "alexnet"):
+    for name in ("resnet18", "mobilenet"):
         src, dst = tmp_path / (name + "_ref"), tmp_path / (name + "_out")
         src.mkdir()
         shutil.copyfile(golden(name), src / (name + ".json"))
@@ -315,7 +315,7 @@ def test_import_model_dir_converts_a_parameter_file_with_transformed_weights(tmp
         for ext in (".json", ".profile.json", ".param", ".raw.co", ".be.co", ".trans.co"):
             assert (dst / (name + ext)).exists(), ext
         got = legacy.read_params(str(dst / (name + ".param")))
-        if name == "alexnet":
+        if name == "mobilenet":
             assert not g.direct_weights
             assert (dst / (name + ".param")).read_bytes() == (src / (name + ".param")).read_bytes()
             continue

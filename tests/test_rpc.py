@@ -112,8 +112,8 @@ def test_failures_answer_succ_false_with_status_ok(served):
 
 
 def test_load_model_imports_a_directory_of_the_reference(served, tmp_path):
-    """A client sends the path of a directory as the reference's pipeline wrote it (alexnet.json with
-    TVM's kernel names, alexnet.param with its keys; the code objects there are for another GPU and
+    """A client sends the path of a directory as the reference's pipeline wrote it (mobilenet.json with
+    TVM's kernel names, mobilenet.param with its keys; the code objects there are for another GPU and
     are never opened): LoadModel imports it and the inference gives what the table's
     interpretation of the reference graph gives."""
     import shutil
@@ -121,7 +121,7 @@ def test_load_model_imports_a_directory_of_the_reference(served, tmp_path):
     from reef_amd.modelgen import builder as MB
     from tests.test_legacy_import import golden, interpret_reference_graph
     server, addr, _ = served
-    name = "alexnet"
+    name = "mobilenet"
     ref_dir = tmp_path / "resource" / name
     ref_dir.mkdir(parents=True)
     shutil.copyfile(golden(name), ref_dir / (name + ".json"))
