@@ -140,7 +140,7 @@ class GraphBuilder:
 
     def conv2d(self, x, cout, k, stride=1, pad=0, bias=True, act=ACT_RELU, residual=None,
                affine=False, force=None, dual_act=None, fused_reduce=None, out=None, out_channel=0,
-               pre_act=False, given=None):
+               pre_act=False, given=None, out2=None):
         """Fused conv + (residual) + (bias) + (scale, shift) + activation on MFMA.
         pre_act: the layer reads its input through a per-channel scale, shift and ReLU of its own
         (DenseNet pre-activation); folded into the convolution's input loads where a kernel for it
@@ -150,7 +150,10 @@ class GraphBuilder:
         out / out_channel: write into channels [out_channel, out_channel + cout) of an existing
         tensor (a concatenation buffer) instead of a new one.
         given: operands that exist already (an imported graph): {"w", "bias", "scale", "shift"} ->
-        Tensor; what is not given is created as a seeded parameter."""
+        Tensor; what is not given is created as a seeded parameter.
+        out2: with dual_act, an existing tensor whose first `cout` channels take the second output
+        (the two outputs share one destination offset, so both start at their tensors' first
+        element here)."""
         given = given or {}
         if fused_reduce is None:
             fused_reduce = self.fused_reduce
@@ -187,11 +190,13 @@ class GraphBuilder:
         else:
             assert out.shape[1:] == (Ho, Wo) and out_channel + cout <= out.shape[0]
             dst_off = out.off + out_channel * Ho * Wo
-        out2 = None
         if dual_act is not None:
             assert not affine
             flags |= F_DUAL
-            out2 = self.temp((cout, Ho, Wo))
+            if out2 is None:
+                out2 = self.temp((cout, Ho, Wo))
+            else:
+                assert dst_off == 0 and out2.off == 0 and out2.shape[1:] == (Ho, Wo) and cout <= out2.shape[0]
             opt.append(out2.idx)
             opt.append(self.param((cout,), 0.01).idx)
         act2 = dual_act or ACT_NONE

@@ -190,14 +190,26 @@ def inception_v3(image=(3, 299, 299), classes=1000, name="inceptionv3", seed=rng
     input, same epilogue, and each of them alone fills less than the device.  Its result
     [reductions | 1x1 branch] is written in front of and into the block's output buffer, so the
     1x1 branch lands where the concatenation wants it and the reductions are read back as channel
-    ranges (operand views); the other branches write straight into their channel slices."""
+    ranges (operand views); the other branches write straight into their channel slices.
+    The pool branch (3x3 average pool, then a 1x1 convolution + bias + ReLU) joins the stacked
+    filter too: averaging and a 1x1 filter commute, so the filter is applied first, as more rows
+    of the stacked convolution, and the pool then averages the few result channels instead of
+    all input channels and adds the bias and the ReLU.  Those rows must leave the convolution
+    bare, so the stacked convolution uses its two-output epilogue: out = the bare result (the
+    pool reads its rows of it), out2 = relu(out + shift) in the block buffer (everything else)."""
     g = GraphBuilder(name, seed)
 
     def conv(x, cout, k, s=1, p=0, out=None, ch=0):
         return g.conv2d(x, cout, k, s, p, bias=True, act=ACT_RELU, out=out, out_channel=ch)
 
-    def avg(x):
-        return g.pool2d(x, 3, 1, 1, "avg", count_include_pad=True)
+    def stacked(x, pool_ch, rest, S):
+        """[pool branch | rest] 1x1 filters on x at once.  relu(result + shift) goes to the first
+        channels of S (the pool branch's rows of it are never read); returns the bare result."""
+        bare, _ = g.conv2d(x, pool_ch + rest, 1, 1, 0, bias=False, act=ACT_NONE, dual_act=ACT_RELU, out2=S)
+        return bare
+
+    def pool_branch(bare, pool_ch, out):
+        g.pool2d(bare.channels(0, pool_ch), 3, 1, 1, "avg", count_include_pad=True, bias=True, act=ACT_RELU, out=out)
 
     x = g.input("data", image)
     x = conv(x, 32, 3, 2)            # 149
@@ -210,12 +222,12 @@ def inception_v3(image=(3, 299, 299), classes=1000, name="inceptionv3", seed=rng
 
     def inception_a(x, pool_ch):
         _, H, W = x.shape
-        r = 48 + 64                                      # reductions in front of the output
+        r = pool_ch + 48 + 64                            # what lies in front of the output
         S = g.temp((r + 64 + 64 + 96 + pool_ch, H, W))
-        conv(x, 48 + 64 + 64, 1, out=S, ch=0)            # [5x5 reduction | 3x3 reduction | 1x1 branch]
-        conv(S.channels(0, 48), 64, 5, 1, 2, out=S, ch=r + 64)
-        conv(conv(S.channels(48, 64), 96, 3, 1, 1), 96, 3, 1, 1, out=S, ch=r + 128)
-        conv(avg(x), pool_ch, 1, out=S, ch=r + 224)
+        bare = stacked(x, pool_ch, 48 + 64 + 64, S)      # [pool branch | 5x5 reduction | 3x3 reduction | 1x1 branch]
+        conv(S.channels(pool_ch, 48), 64, 5, 1, 2, out=S, ch=r + 64)
+        conv(conv(S.channels(pool_ch + 48, 64), 96, 3, 1, 1), 96, 3, 1, 1, out=S, ch=r + 128)
+        pool_branch(bare, pool_ch, S.channels(r + 224, pool_ch))
         return S.channels(r, 224 + pool_ch)
 
     x = inception_a(x, 32)
@@ -235,13 +247,13 @@ def inception_v3(image=(3, 299, 299), classes=1000, name="inceptionv3", seed=rng
 
     def inception_c(x, c7):
         _, H, W = x.shape
-        r = 2 * c7
+        r = 192 + 2 * c7
         S = g.temp((r + 768, H, W))
-        conv(x, c7 + c7 + 192, 1, out=S, ch=0)           # [7-tap reduction | double 7-tap reduction | 1x1 branch]
-        conv(conv(S.channels(0, c7), c7, (1, 7), 1, (0, 3)), 192, (7, 1), 1, (3, 0), out=S, ch=r + 192)
-        y = conv(conv(conv(S.channels(c7, c7), c7, (7, 1), 1, (3, 0)), c7, (1, 7), 1, (0, 3)), c7, (7, 1), 1, (3, 0))
+        bare = stacked(x, 192, c7 + c7 + 192, S)         # [pool branch | 7-tap reduction | double 7-tap reduction | 1x1 branch]
+        conv(conv(S.channels(192, c7), c7, (1, 7), 1, (0, 3)), 192, (7, 1), 1, (3, 0), out=S, ch=r + 192)
+        y = conv(conv(conv(S.channels(192 + c7, c7), c7, (7, 1), 1, (3, 0)), c7, (1, 7), 1, (0, 3)), c7, (7, 1), 1, (3, 0))
         conv(y, 192, (1, 7), 1, (0, 3), out=S, ch=r + 384)
-        conv(avg(x), 192, 1, out=S, ch=r + 576)
+        pool_branch(bare, 192, S.channels(r + 576, 192))
         return S.channels(r, 768)
 
     for c7 in (128, 160, 160, 192):
@@ -262,16 +274,16 @@ def inception_v3(image=(3, 299, 299), classes=1000, name="inceptionv3", seed=rng
 
     def inception_e(x):
         _, H, W = x.shape
-        r = 384 + 448
+        r = 192 + 384 + 448
         S = g.temp((r + 2048, H, W))
-        conv(x, 384 + 448 + 320, 1, out=S, ch=0)         # [3-tap reduction | 3x3 reduction | 1x1 branch]
-        y = S.channels(0, 384)
+        bare = stacked(x, 192, 384 + 448 + 320, S)       # [pool branch | 3-tap reduction | 3x3 reduction | 1x1 branch]
+        y = S.channels(192, 384)
         conv(y, 384, (1, 3), 1, (0, 1), out=S, ch=r + 320)
         conv(y, 384, (3, 1), 1, (1, 0), out=S, ch=r + 704)
-        y = conv(S.channels(384, 448), 384, 3, 1, 1)
+        y = conv(S.channels(192 + 384, 448), 384, 3, 1, 1)
         conv(y, 384, (1, 3), 1, (0, 1), out=S, ch=r + 1088)
         conv(y, 384, (3, 1), 1, (1, 0), out=S, ch=r + 1472)
-        conv(avg(x), 192, 1, out=S, ch=r + 1856)
+        pool_branch(bare, 192, S.channels(r + 1856, 192))
         return S.channels(r, 2048)
 
     x = inception_e(x)

@@ -253,33 +253,41 @@ def test_inception_v3_wiring(tmp_path):
     t = conv(t, 80, 1); t = conv(t, 192, 3)
     t = F.max_pool2d(t, 3, 2)
     # The 1x1 convolutions that read a block's input are one convolution with the stacked filter
-    # [reductions..., 1x1 branch]; torch splits its result, the graph reads channel ranges of it.
+    # [pool branch, reductions..., 1x1 branch]; torch splits its result, the graph reads channel
+    # ranges of it.  The pool branch's filter runs BEFORE its average pool there (they commute);
+    # torch keeps the textbook order pool -> 1x1 -> bias -> ReLU with the same weights.
+    def stacked(t, pool_ch, parts):
+        w, shift = P.take(pool_ch + sum(parts), t.shape[1], 1, 1), P.take(pool_ch + sum(parts))
+        act = F.relu(F.conv2d(t, w[pool_ch:], shift[pool_ch:]))
+        return w[:pool_ch], act.split(parts, 1)
+
+    pooled = lambda t, w: F.relu(F.conv2d(avg(t), w, P.take(w.shape[0])))
     for pool_ch in (32, 64, 64):                                           # 3 x block A
-        r5, r3, b1 = conv(t, 48 + 64 + 64, 1).split([48, 64, 64], 1)
+        wp, (r5, r3, b1) = stacked(t, pool_ch, [48, 64, 64])
         b5 = conv(r5, 64, 5, 1, 2)
         b3 = conv(conv(r3, 96, 3, 1, 1), 96, 3, 1, 1)
-        bp = conv(avg(t), pool_ch, 1)
+        bp = pooled(t, wp)
         t = torch.cat([b1, b5, b3, bp], 1)
     b3 = conv(t, 384, 3, 2)                                                # block B (grid reduction)
     bd = conv(conv(conv(t, 64, 1), 96, 3, 1, 1), 96, 3, 2)
     t = torch.cat([b3, bd, F.max_pool2d(t, 3, 2)], 1)
     for c7 in (128, 160, 160, 192):                                        # 4 x block C
-        r7, rd, b1 = conv(t, c7 + c7 + 192, 1).split([c7, c7, 192], 1)
+        wp, (r7, rd, b1) = stacked(t, 192, [c7, c7, 192])
         b7 = conv(conv(r7, c7, (1, 7), 1, (0, 3)), 192, (7, 1), 1, (3, 0))
         bd = conv(conv(conv(conv(rd, c7, (7, 1), 1, (3, 0)), c7, (1, 7), 1, (0, 3)), c7, (7, 1), 1,
                        (3, 0)), 192, (1, 7), 1, (0, 3))
-        bp = conv(avg(t), 192, 1)
+        bp = pooled(t, wp)
         t = torch.cat([b1, b7, bd, bp], 1)
     r3, r7 = conv(t, 192 + 192, 1).split([192, 192], 1)                    # block D
     b3 = conv(r3, 320, 3, 2)
     b7 = conv(conv(conv(r7, 192, (1, 7), 1, (0, 3)), 192, (7, 1), 1, (3, 0)), 192, 3, 2)
     t = torch.cat([b3, b7, F.max_pool2d(t, 3, 2)], 1)
     for _ in range(2):                                                     # 2 x block E
-        y, rd, b1 = conv(t, 384 + 448 + 320, 1).split([384, 448, 320], 1)
+        wp, (y, rd, b1) = stacked(t, 192, [384, 448, 320])
         b3 = torch.cat([conv(y, 384, (1, 3), 1, (0, 1)), conv(y, 384, (3, 1), 1, (1, 0))], 1)
         y = conv(rd, 384, 3, 1, 1)
         bd = torch.cat([conv(y, 384, (1, 3), 1, (0, 1)), conv(y, 384, (3, 1), 1, (1, 0))], 1)
-        bp = conv(avg(t), 192, 1)
+        bp = pooled(t, wp)
         t = torch.cat([b1, b3, bd, bp], 1)
     assert t.shape[1:] == (2048, 8, 8)
     t = F.linear(t.mean(dim=(2, 3)), P.take(32, 2048), P.take(32))
