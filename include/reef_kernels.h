@@ -117,6 +117,7 @@ enum {
     REEF_OP_GEMM = 14,
     REEF_OP_MOCK_ADD = 15,
     REEF_OP_MOCK_MULTIPLY = 16,
+    REEF_OP_ATTENTION = 17,
     REEF_OP_COUNT
 };
 
@@ -135,6 +136,7 @@ enum {
 #define REEF_K_COPY "reef_copy"
 #define REEF_K_TRANSPOSE "reef_transpose"
 #define REEF_K_GEMM "reef_gemm"
+#define REEF_K_ATTENTION "reef_attention"
 /* The reference's mocked model (resource/mocked_kernel/mocked_kernel.json)
  * keeps its own names and its (64,1,1)x(4,8,4) launch. */
 #define REEF_K_MOCK_ADD "add"
@@ -302,6 +304,27 @@ enum { REEF_SM_ROWS = 0, REEF_SM_COLS, REEF_SM_FLAGS, REEF_SM_NATTR };
  * ptr: x, gamma, beta, out, res(optional).  attr: rows, cols, flags(bit0 = res), eps (float bits).
  * tasks = ceil(rows / 4). */
 enum { REEF_LN_ROWS = 0, REEF_LN_COLS, REEF_LN_FLAGS, REEF_LN_EPS_BITS, REEF_LN_NATTR };
+
+/* ---- reef_attention: softmax(alpha Q K^T (masked)) V for every head, one launch ----
+ * The three launches of an attention layer (scores, softmax, context: bert.cu:22-271, 3-13,
+ * 159-166, 327-337, 381-396) for sequences whose scores fit a workgroup: seq <= 128,
+ * head_dim <= 64 and a multiple of 4 (as ld, ldo and the offsets: 128-bit loads).  Q, K and V are column blocks of one [seq][ld] storage
+ * (head h at columns off + h * head_dim), the context goes to out[seq][ldo] at columns
+ * h * head_dim.  A workgroup takes REEF_AT_ROWS query rows of one head: it holds them, all keys and then
+ * all values of the head in LDS, the scores never leave the chip.
+ * ptr: qkv, out, mask(optional: one byte per key position, non-zero = -inf).
+ * attr: seq, head_dim, heads, ld, ldo, offQ, offK, offV (elements), alpha (float bits), flags
+ * (bit0 = mask).  tasks = heads * ceil(seq / REEF_AT_ROWS). */
+enum {
+    REEF_AT_SEQ = 0, REEF_AT_HEAD_DIM, REEF_AT_HEADS, REEF_AT_LD, REEF_AT_LDO, REEF_AT_OFF_Q,
+    REEF_AT_OFF_K, REEF_AT_OFF_V, REEF_AT_ALPHA_BITS, REEF_AT_FLAGS, REEF_AT_NATTR
+};
+#define REEF_AT_ROWS 8 /* query rows per workgroup: 16 leave too few workgroups, 4 stage the keys and values too often */
+#define REEF_AT_MAX_SEQ 128
+#define REEF_AT_MAX_HEAD_DIM 64
+#define REEF_AT_KV_STRIDE 68 /* floats per staged key / value row: 64 + 4, rows 16-byte aligned */
+#define REEF_AT_LDS_BYTES \
+    (4 * (REEF_AT_ROWS * REEF_AT_MAX_HEAD_DIM + REEF_AT_MAX_SEQ * REEF_AT_KV_STRIDE + REEF_AT_ROWS * (REEF_AT_MAX_SEQ + 4)))
 
 /* ---- reef_bias_gelu: out = gelu_erf(x + bias[col]).  ptr: x, out, bias(optional).
  * attr: rows, cols, flags.  tasks = ceil(rows*cols / 1024). */

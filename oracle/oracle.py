@@ -415,6 +415,18 @@ class GraphOracle:
                     c = bias_gelu(c)
                 Cm = np.lib.stride_tricks.as_strided(C[bi * sC:], (M, N), (ldc * 4, 4))
                 Cm[:, :] = c
+        elif name == "reef_attention":
+            # softmax(alpha Q K^T (masked)) V per head; Q, K, V column blocks of one [seq][ld] tensor
+            S, HD, heads, ld, ldo, oq, ok, ov, alpha_bits, flags = a[:10]
+            alpha = _bits_to_float(alpha_bits)
+            qkv = P[0][:S * ld].reshape(S, ld)
+            mask = P[2].view(np.uint8)[:S] if flags & 1 else None
+            out = P[1][:S * ldo].reshape(S, ldo)
+            for h in range(heads):
+                q, kk, v = (np.ascontiguousarray(qkv[:, o + h * HD:o + (h + 1) * HD]) for o in (oq, ok, ov))
+                sc = batch_matmul(q[None], kk[None], True, alpha, acc64)[0]
+                pr = softmax(sc, mask)
+                out[:, h * HD:(h + 1) * HD] = batch_matmul(pr[None], v[None], False, 1.0, acc64)[0]
         elif name in ("add", "multiply"):
             lp = k["launch_params"]
             blocks, threads = lp[0] * lp[1] * lp[2], lp[3] * lp[4] * lp[5]

@@ -38,6 +38,7 @@ int TransExecutor::op_from_name(const std::string& n) {
         {REEF_K_BIAS_GELU, REEF_OP_BIAS_GELU}, {REEF_K_EMBEDDING, REEF_OP_EMBEDDING},
         {REEF_K_COPY, REEF_OP_COPY}, {REEF_K_TRANSPOSE, REEF_OP_TRANSPOSE},
         {REEF_K_MOCK_ADD, REEF_OP_MOCK_ADD}, {REEF_K_MOCK_MULTIPLY, REEF_OP_MOCK_MULTIPLY},
+        {REEF_K_ATTENTION, REEF_OP_ATTENTION},
     };
     for (auto& e : table) {
         const size_t len = std::strlen(e.prefix);

@@ -309,6 +309,128 @@ __device__ __forceinline__ void softmax_body(const ReefOpDesc& d, int task) {
     for (int i = lane; i < cols; i += 64) y[i] = expf(at(i) - m) / s;
 }
 
+// Attention of one head for REEF_AT_ROWS query rows: scores, masked softmax and context without a
+// trip to memory in between.  256 threads as ROWS rows x LANES column lanes: a thread owns the
+// scores of its row at columns c, c + LANES, ... and later the context values at columns
+// c, c + LANES, ....  The lanes of a row are neighbours in a wavefront, so the row's maximum
+// and sum are a few exchanges.  The values are fetched into registers while
+// the scores are computed and take the keys' place in LDS afterwards.  Every thread reaches
+// every barrier (rows and columns outside the tensor compute on zeros and are not stored).
+__device__ __forceinline__ void attention_body(const ReefOpDesc& d, int task, char* smem_raw) {
+    const int* a = d.attr;
+    const int S = a[REEF_AT_SEQ], HD = a[REEF_AT_HEAD_DIM];
+    const int ld = a[REEF_AT_LD], ldo = a[REEF_AT_LDO];
+    const int row_blocks = (S + REEF_AT_ROWS - 1) / REEF_AT_ROWS;
+    const int h = div_small(task, row_blocks);
+    const int m0 = (task - h * row_blocks) * REEF_AT_ROWS;
+    const float alpha = __int_as_float(a[REEF_AT_ALPHA_BITS]);
+    const float* base = (const float*)d.ptr[0];
+    const float* Q = base + a[REEF_AT_OFF_Q] + h * HD;
+    const float* K = base + a[REEF_AT_OFF_K] + h * HD;
+    const float* V = base + a[REEF_AT_OFF_V] + h * HD;
+    const unsigned char* mask = (a[REEF_AT_FLAGS] & 1) ? (const unsigned char*)d.ptr[2] : nullptr;
+    float* Qs = (float*)smem_raw;                                  // [8][64]
+    float* KV = Qs + REEF_AT_ROWS * REEF_AT_MAX_HEAD_DIM;          // [128][68]: keys, later values
+    float* Ps = KV + REEF_AT_MAX_SEQ * REEF_AT_KV_STRIDE;          // [8][132]
+    constexpr int PST = REEF_AT_MAX_SEQ + 4;
+    constexpr int KV4 = REEF_AT_MAX_SEQ * REEF_AT_MAX_HEAD_DIM / 4 / REEF_WG_THREADS;   // 8 float4 per thread
+    constexpr int LANES = REEF_WG_THREADS / REEF_AT_ROWS;            // column lanes per row
+    constexpr int SC = REEF_AT_MAX_SEQ / LANES;                      // scores per thread
+    constexpr int OC = (REEF_AT_MAX_HEAD_DIM + LANES - 1) / LANES;   // context values per thread
+    static_assert(LANES <= 64 && (LANES & (LANES - 1)) == 0, "a row's lanes share a wavefront");
+    const int t = threadIdx.x, r = t / LANES, c = t % LANES;
+    const int hd4 = HD >> 2;
+
+    // stage the query rows and all key rows (128-bit loads; rows outside the tensor as zeros)
+    for (int i = t; i < REEF_AT_ROWS * hd4; i += REEF_WG_THREADS) {
+        const int row = div_small(i, hd4), c4 = i - row * hd4;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (m0 + row < S) v = *(const float4*)(Q + (size_t)(m0 + row) * ld + 4 * c4);
+        *(float4*)(Qs + row * REEF_AT_MAX_HEAD_DIM + 4 * c4) = v;
+    }
+    float4 vreg[KV4];
+#pragma unroll
+    for (int u = 0; u < KV4; ++u) {
+        const int i = t + REEF_WG_THREADS * u;
+        const int row = div_small(i, hd4), c4 = i - row * hd4;
+        float4 kv = make_float4(0.f, 0.f, 0.f, 0.f);
+        vreg[u] = kv;
+        if (row < S) {
+            kv = *(const float4*)(K + (size_t)row * ld + 4 * c4);
+            vreg[u] = *(const float4*)(V + (size_t)row * ld + 4 * c4);
+        }
+        if (row < REEF_AT_MAX_SEQ) *(float4*)(KV + row * REEF_AT_KV_STRIDE + 4 * c4) = kv;
+    }
+    __syncthreads();
+
+    float s[SC];
+#pragma unroll
+    for (int j = 0; j < SC; ++j) s[j] = 0.0f;
+#pragma unroll 2
+    for (int k4 = 0; k4 < hd4; ++k4) {
+        const float4 q = *(const float4*)(Qs + r * REEF_AT_MAX_HEAD_DIM + 4 * k4);
+#pragma unroll
+        for (int j = 0; j < SC; ++j) {
+            const float4 kv = *(const float4*)(KV + (c + LANES * j) * REEF_AT_KV_STRIDE + 4 * k4);
+            s[j] = fmaf(q.x, kv.x, s[j]);
+            s[j] = fmaf(q.y, kv.y, s[j]);
+            s[j] = fmaf(q.z, kv.z, s[j]);
+            s[j] = fmaf(q.w, kv.w, s[j]);
+        }
+    }
+    float m = -FLT_MAX;
+#pragma unroll
+    for (int j = 0; j < SC; ++j) {
+        const int col = c + LANES * j;
+        s[j] = (col < S && !(mask && mask[col])) ? s[j] * alpha : -INFINITY;
+        m = fmaxf(m, s[j]);
+    }
+#pragma unroll
+    for (int o = LANES / 2; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, LANES));
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < SC; ++j) {
+        s[j] = expf(s[j] - m);          // -inf - m -> 0 for masked and missing columns
+        sum += s[j];
+    }
+#pragma unroll
+    for (int o = LANES / 2; o > 0; o >>= 1) sum += __shfl_xor(sum, o, LANES);
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int j = 0; j < SC; ++j) Ps[r * PST + c + LANES * j] = s[j] * inv;
+    __syncthreads();                     // nobody reads keys any more: the values take their place
+#pragma unroll
+    for (int u = 0; u < KV4; ++u) {
+        const int i = t + REEF_WG_THREADS * u;
+        const int row = div_small(i, hd4), c4 = i - row * hd4;
+        if (row < REEF_AT_MAX_SEQ) *(float4*)(KV + row * REEF_AT_KV_STRIDE + 4 * c4) = vreg[u];
+    }
+    __syncthreads();
+
+    float o2[OC];
+#pragma unroll
+    for (int j = 0; j < OC; ++j) o2[j] = 0.0f;
+    const int k_end = (S + 3) & ~3;      // probabilities and value rows beyond S are zeros
+#pragma unroll 2
+    for (int k = 0; k < k_end; k += 4) {
+        const float4 p = *(const float4*)(Ps + r * PST + k);
+#pragma unroll
+        for (int j = 0; j < OC; ++j) {
+            const float* col = KV + k * REEF_AT_KV_STRIDE + c + LANES * j;
+            o2[j] = fmaf(p.x, col[0], o2[j]);
+            o2[j] = fmaf(p.y, col[REEF_AT_KV_STRIDE], o2[j]);
+            o2[j] = fmaf(p.z, col[2 * REEF_AT_KV_STRIDE], o2[j]);
+            o2[j] = fmaf(p.w, col[3 * REEF_AT_KV_STRIDE], o2[j]);
+        }
+    }
+    if (m0 + r < S) {
+        float* out = (float*)d.ptr[1] + (size_t)(m0 + r) * ldo + h * HD;
+#pragma unroll
+        for (int j = 0; j < OC; ++j)
+            if (c + LANES * j < HD) out[c + LANES * j] = o2[j];
+    }
+}
+
 // one wavefront per row; two-pass mean / variance as the reference splits it
 __device__ __forceinline__ void layernorm_body(const ReefOpDesc& d, int task) {
     const int rows = d.attr[REEF_LN_ROWS], cols = d.attr[REEF_LN_COLS];

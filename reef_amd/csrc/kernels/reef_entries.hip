@@ -79,6 +79,14 @@ struct OpGemmNtDirect {
             return true;                                                                        \
         }                                                                                       \
     };
+struct OpAttention {
+    static constexpr int LDS = REEF_AT_LDS_BYTES;
+    template <class P>
+    static __device__ __forceinline__ bool run(const ReefOpDesc& d, int task, char* smem, const P&) {
+        attention_body(d, task, smem);
+        return true;
+    }
+};
 REEF_SIMPLE_OP(OpSplitKReduce, splitk_reduce_body<8>)
 REEF_SIMPLE_OP(OpDwConv, dwconv2d_body)
 REEF_SIMPLE_OP(OpPool, pool2d_body)
@@ -338,6 +346,7 @@ REEF_ENTRY(reef_dense, OpDense)
 REEF_ENTRY(reef_softmax, OpSoftmax)
 REEF_ENTRY(reef_layernorm, OpLayerNorm)
 REEF_ENTRY(reef_bias_gelu, OpBiasGelu)
+REEF_ENTRY(reef_attention, OpAttention)
 REEF_ENTRY(reef_embedding, OpEmbedding)
 REEF_ENTRY(reef_copy, OpCopy)
 REEF_ENTRY(reef_transpose, OpTranspose)

@@ -418,6 +418,29 @@ class GraphBuilder:
                    "embedding", 0, 4 * seq * hidden * 3, 2.0)
         return out
 
+    ATTENTION_MAX_SEQ, ATTENTION_MAX_HEAD_DIM, ATTENTION_ROWS = 128, 64, 8    # REEF_AT_* of include/reef_kernels.h
+
+    @classmethod
+    def attention_ok(cls, seq, head_dim, ld, ldo, offs):
+        """Whether reef_attention takes this shape (all keys of a head fit a workgroup's LDS)."""
+        return (seq <= cls.ATTENTION_MAX_SEQ and head_dim <= cls.ATTENTION_MAX_HEAD_DIM
+                and all(v % 4 == 0 for v in (head_dim, ld, ldo) + tuple(offs)))
+
+    def attention(self, qkv, seq, heads, head_dim, ld, off_q, off_k, off_v, alpha, mask=None, out=None, ldo=None):
+        """softmax(alpha Q K^T (masked)) V for every head in one launch; Q, K, V are column blocks
+        of qkv [seq][ld] (head h at columns off + h * head_dim), the context goes to
+        out [seq][ldo] at columns h * head_dim."""
+        ldo = heads * head_dim if ldo is None else ldo
+        assert self.attention_ok(seq, head_dim, ld, ldo, (off_q, off_k, off_v))
+        out = Tensor(out.idx, (seq, ldo)) if out is not None else self.temp((seq, ldo))
+        args = [qkv.idx, out.idx] + ([mask.idx] if mask is not None else [])
+        flops = 4 * heads * seq * seq * head_dim
+        self.flops += flops
+        self._emit("reef_attention", heads * math.ceil(seq / self.ATTENTION_ROWS), args,
+                   [seq, head_dim, heads, ld, ldo, off_q, off_k, off_v, float_bits(alpha), 1 if mask is not None else 0],
+                   "attention", flops, 4 * (3 * seq * heads * head_dim + seq * ldo), 4.0)
+        return out
+
     def copy_into(self, src, dst, dst_off):
         self._emit("reef_copy", math.ceil(src.size / 1024), [src.idx, dst.idx], [src.size, dst_off],
                    "copy", 0, 8 * src.size, 2.0)

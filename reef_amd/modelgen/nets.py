@@ -296,7 +296,7 @@ def inception_v3(image=(3, 299, 299), classes=1000, name="inceptionv3", seed=rng
 
 
 def bert(layers=12, hidden=768, heads=12, ffn=3072, seq=128, vocab=30522, name="bert_base",
-         seed=rng.BASE_SEED, attention_mask=False):
+         seed=rng.BASE_SEED, attention_mask=False, fused_attention=True):
     """BERT encoder (base: 12 layers, hidden 768, 12 heads, FFN 3072, sequence 128), fp32,
     weights ~ N(0, 0.02).  Token ids are an int64 input, as in the reference's BERT model
     (resource/bert/bert.json storage[0]).  The per-head views of Q, K, V and of the context
@@ -321,13 +321,18 @@ def bert(layers=12, hidden=768, heads=12, ffn=3072, seq=128, vocab=30522, name="
         w = g.param((3 * hidden, hidden), 0.02)
         b = g.param((3 * hidden,), 0.02)
         qkv = g.gemm(x, w, seq, 3 * hidden, hidden, trans_b=True, bias=b)
-        scores = g.gemm(qkv, qkv, seq, seq, hd, batch=heads, trans_b=True, alpha=inv_sqrt,
-                        lda=3 * hidden, ldb=3 * hidden, ldc=seq, stride_a=hd, stride_b=hd, stride_c=seq * seq,
-                        off_b=hidden)
-        probs = g.softmax(scores, heads * seq, seq, mask=mask)
-        ctx = g.temp((seq, hidden))
-        g.gemm(probs, qkv, seq, hd, seq, batch=heads, trans_b=False, lda=seq, ldb=3 * hidden, ldc=hidden,
-               stride_a=seq * seq, stride_b=hd, stride_c=hd, out=ctx, off_b=2 * hidden)
+        if fused_attention and g.attention_ok(seq, hd, 3 * hidden, hidden, (0, hidden, 2 * hidden)):
+            # scores, masked softmax and context of all heads in one launch: the scores of a
+            # workgroup's query rows stay in its registers and LDS
+            ctx = g.attention(qkv, seq, heads, hd, 3 * hidden, 0, hidden, 2 * hidden, inv_sqrt, mask=mask)
+        else:
+            scores = g.gemm(qkv, qkv, seq, seq, hd, batch=heads, trans_b=True, alpha=inv_sqrt,
+                            lda=3 * hidden, ldb=3 * hidden, ldc=seq, stride_a=hd, stride_b=hd, stride_c=seq * seq,
+                            off_b=hidden)
+            probs = g.softmax(scores, heads * seq, seq, mask=mask)
+            ctx = g.temp((seq, hidden))
+            g.gemm(probs, qkv, seq, hd, seq, batch=heads, trans_b=False, lda=seq, ldb=3 * hidden, ldc=hidden,
+                   stride_a=seq * seq, stride_b=hd, stride_c=hd, out=ctx, off_b=2 * hidden)
         wo = g.param((hidden, hidden), 0.02)
         bo = g.param((hidden,), 0.02)
         att = g.gemm(ctx, wo, seq, hidden, hidden, trans_b=True, bias=bo)

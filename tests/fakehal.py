@@ -48,7 +48,7 @@ class DeviceInfo(ctypes.Structure):
 OP_SYMBOL = {1: "reef_conv2d", 2: "reef_splitk_reduce", 3: "reef_dwconv2d", 4: "reef_pool2d",
              5: "reef_global_avgpool", 6: "reef_eltwise", 7: "reef_dense", 8: "reef_softmax",
              9: "reef_layernorm", 10: "reef_bias_gelu", 11: "reef_embedding", 12: "reef_copy",
-             13: "reef_transpose", 14: "reef_gemm", 15: "add", 16: "multiply"}
+             13: "reef_transpose", 14: "reef_gemm", 15: "add", 16: "multiply", 17: "reef_attention"}
 
 CB_TYPE = ctypes.CFUNCTYPE(None, ctypes.c_char_p, ctypes.c_char_p, ctypes.c_void_p, ctypes.c_size_t,
                            ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32),

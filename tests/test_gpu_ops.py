@@ -414,6 +414,39 @@ def test_operands_as_channel_ranges_of_a_larger_buffer(tmp_path):
     assert np.isfinite(whole).all()
 
 
+@pytest.mark.parametrize("seq,heads,hd,masked", [(128, 12, 64, False), (40, 4, 24, True), (77, 3, 64, True),
+                                                 (16, 2, 16, False), (5, 1, 8, True)])
+def test_attention_in_one_launch(tmp_path, seq, heads, hd, masked):
+    """reef_attention against the oracle's three steps (scores, masked softmax, context) and against
+    numpy on the projected tensor: the full BERT-base shape, ragged sequence lengths (not a multiple
+    of the rows a workgroup takes), head sizes below 64, padding positions at the end."""
+    hid = heads * hd
+    g = MB.GraphBuilder("att", weight_std=0.05)
+    x = g.input("x", (seq, hid))
+    w = g.param((3 * hid, hid), 0.2)
+    bias = g.param((3 * hid,), 0.1)
+    qkv = g.gemm(x, w, seq, 3 * hid, hid, trans_b=True, bias=bias)
+    mask = g.input("attention_mask", (seq,), "uint1") if masked else None
+    ctx = g.attention(qkv, seq, heads, hd, 3 * hid, 0, hid, 2 * hid, 1.0 / np.sqrt(hd), mask=mask)
+    g.mark_output(ctx)
+    pad = np.zeros(seq, np.uint8)
+    pad[seq - max(1, seq // 4):] = 1
+    inputs = {"x": rnd(seq, hid)}
+    if masked:
+        inputs["attention_mask"] = pad
+    exe, orc, model = run_both(g, tmp_path, inputs)
+    compare_storages(exe, orc, model, what="attention")
+    m = exe.get_data(qkv.idx, seq * 3 * hid).reshape(seq, 3, heads, hd).astype(np.float64)
+    sc = np.einsum("shd,thd->hst", m[:, 0], m[:, 1]) / np.sqrt(hd)
+    if masked:
+        sc[:, :, pad != 0] = -np.inf
+    pr = np.exp(sc - sc.max(-1, keepdims=True))
+    pr /= pr.sum(-1, keepdims=True)
+    want = np.einsum("hst,thd->shd", pr, m[:, 2]).reshape(seq, hid)
+    got = exe.get_data(ctx.idx, seq * hid).reshape(seq, hid)
+    assert np.isfinite(got).all() and np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
+
+
 def test_mocked_model_closed_form(tmp_path):
     """The reference's executor_base.mocked_kernel test: a = b = c = 3 -> 18 everywhere
     (src/reef/test/test.cpp:102-116)."""
