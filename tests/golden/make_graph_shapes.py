@@ -391,9 +391,11 @@ def derive_bert():
 def main():
     name = sys.argv[1]
     table = derive_bert() if name == "bert" else derive(name)
-    for out in (os.path.join(HERE, name + "_kernel_shapes.json"),
-                os.path.join(ROOT, "reef_amd", "legacy_tables", name + ".json"),
-                os.path.join(ROOT, "gpurun_out", name + "_kernel_shapes.json")):
+    outs = [os.path.join(HERE, name + "_kernel_shapes.json"),
+            os.path.join(ROOT, "reef_amd", "legacy_tables", name + ".json")]
+    if os.environ.get("REEF_SHAPES_COPY_DIR"):      # a third copy, e.g. where results of a remote run are collected
+        outs.append(os.path.join(os.environ["REEF_SHAPES_COPY_DIR"], name + "_kernel_shapes.json"))
+    for out in outs:
         os.makedirs(os.path.dirname(out), exist_ok=True)
         json.dump(table, open(out, "w"), indent=0, sort_keys=True)
     print(len(table), "kernels; without a witness:", [n for n, e in table.items() if not e["witness"]])
