@@ -208,7 +208,10 @@ int reef_ops_conv2d(const reef_conv2d_desc* c, const float* in, const float* w, 
         hipError_t e = hipMalloc(&ws, p.ws_floats * 4);
         if (e != hipSuccess) return hip_fail(e, "hipMalloc(workspace)");
         e = hipMalloc(&cnt, (size_t)p.tiles * 4);
-        if (e != hipSuccess) { hipFree(ws); return hip_fail(e, "hipMalloc(counters)"); }
+        if (e != hipSuccess) {
+            (void)hipFree(ws);
+            return hip_fail(e, "hipMalloc(counters)");
+        }
         hipLaunchKernelGGL(fill_words, dim3((p.tiles + 255) / 256), dim3(256), 0, s, (uint32_t*)cnt, 0u, (size_t)p.tiles);
         p.desc.ptr[p.ws_slot] = ws;
         p.desc.ptr[p.sync_slot] = cnt;
@@ -217,9 +220,9 @@ int reef_ops_conv2d(const reef_conv2d_desc* c, const float* in, const float* w, 
     if (p.split_k > 1) {
         // the buffers live until the kernel is done with them
         hipError_t e = hipStreamSynchronize(s);
-        hipFree(ws);
-        hipFree(cnt);
+        const hipError_t f1 = hipFree(ws), f2 = hipFree(cnt);
         if (rc == 0 && e != hipSuccess) rc = hip_fail(e, "hipStreamSynchronize");
+        if (rc == 0 && (f1 != hipSuccess || f2 != hipSuccess)) rc = hip_fail(f1 != hipSuccess ? f1 : f2, "hipFree");
     }
     return rc;
 }
