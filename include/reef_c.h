@@ -241,6 +241,13 @@ int reef_dkp_walk(int block_idx, int num_cus, int num_xcds, int cu_partition, in
 /* Parsers (src/reef/executor/model.cpp), exposed for format tests. */
 int reef_model_parse_summary(const char* json_path, int* n_storage, int* n_kernels, int* n_args,
                              int* n_shared);
+/* The check every executor makes when it loads a graph file, before anything is launched: each
+ * kernel's shape attributes must fit the storages it is given (operand count, bytes behind each
+ * operand's start) and the number of workgroups it is launched with.  0 = every kernel fits;
+ * otherwise `why` (when given) names the first kernel that does not, the operand and the sizes.
+ * No counterpart in the reference: its generated kernels have their shapes compiled in
+ * (resource/resnet152/resnet152.cu:315-338), the shape-generic kernels here trust their attributes. */
+int reef_model_check_kernels(const char* json_path, char* why, int why_len);
 int reef_profile_parse_summary(const char* json_path, int* model_latency, int* n_kernels,
                                int* min_latency, int* n_latency_values);
 int reef_profile_roundtrip(const char* json_path, char* out, size_t cap);

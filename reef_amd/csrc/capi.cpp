@@ -8,6 +8,7 @@
 
 #include "client/loadgen.h"
 #include "executor/hybrid_executor.h"
+#include "executor/op_extents.h"
 #include "hal/code_object.h"
 #include "reef_c.h"
 #include "server/scheduler.h"
@@ -468,6 +469,22 @@ int reef_model_parse_summary(const char* json_path, int* n_storage, int* n_kerne
     *n_kernels = (int)m->kernels.size();
     *n_args = (int)m->args.size();
     *n_shared = (int)m->shared_memory.size();
+    return Status::Succ;
+}
+int reef_model_check_kernels(const char* json_path, char* why, int why_len) {
+    std::unique_ptr<Model> m(Model::from_json(json_path));
+    if (why && why_len > 0) why[0] = 0;
+    if (!m) return Status::NotFound;
+    for (size_t i = 0; i < m->kernels.size(); ++i) {
+        std::string reason;
+        if (!reef::executor::kernel_fits_storages(*m, i, &reason)) {
+            if (why && why_len > 0) {
+                std::strncpy(why, reason.c_str(), (size_t)why_len - 1);
+                why[why_len - 1] = 0;
+            }
+            return Status::OutOfRange;
+        }
+    }
     return Status::Succ;
 }
 int reef_profile_parse_summary(const char* json_path, int* model_latency, int* n_kernels,

@@ -1,4 +1,5 @@
 #include "executor/executor_base.h"
+#include "executor/op_extents.h"
 
 #include <cstdlib>
 
@@ -59,6 +60,15 @@ Status ExecutorBase::init_executor_base(const char* json_file_path, GPUModule_t 
         kernel_funcs.push_back(it->second);
         if (ki.args.size() > REEF_MAX_PTRS || ki.attrs.size() > REEF_MAX_ATTRS) {
             REEF_LOG_ERROR("kernel %s: too many args/attrs", ki.name.c_str());
+            return Status::OutOfRange;
+        }
+    }
+
+    // every kernel must fit the storages it is given and the grid it is launched with
+    for (size_t i = 0; i < model->kernels.size(); ++i) {
+        std::string why;
+        if (!kernel_fits_storages(*model, i, &why)) {
+            REEF_LOG_ERROR("%s: %s", json_file_path, why.c_str());
             return Status::OutOfRange;
         }
     }

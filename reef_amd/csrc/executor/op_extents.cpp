@@ -1,0 +1,330 @@
+#include "executor/op_extents.h"
+
+#include <cstdio>
+#include <cstring>
+
+#include "reef_kernels.h"
+
+namespace reef {
+namespace executor {
+
+int op_from_symbol(const std::string& n) {
+    struct { const char* prefix; int op; } table[] = {
+        {"reef_conv2d_", REEF_OP_CONV2D}, {"reef_gemm_", REEF_OP_GEMM},
+        {REEF_K_SPLITK_REDUCE, REEF_OP_SPLITK_REDUCE}, {REEF_K_DWCONV2D, REEF_OP_DWCONV2D},
+        {REEF_K_POOL2D, REEF_OP_POOL2D}, {REEF_K_GLOBAL_AVGPOOL, REEF_OP_GLOBAL_AVGPOOL},
+        {REEF_K_ELTWISE, REEF_OP_ELTWISE}, {REEF_K_DENSE, REEF_OP_DENSE},
+        {REEF_K_SOFTMAX, REEF_OP_SOFTMAX}, {REEF_K_LAYERNORM, REEF_OP_LAYERNORM},
+        {REEF_K_BIAS_GELU, REEF_OP_BIAS_GELU}, {REEF_K_EMBEDDING, REEF_OP_EMBEDDING},
+        {REEF_K_COPY, REEF_OP_COPY}, {REEF_K_TRANSPOSE, REEF_OP_TRANSPOSE},
+        {REEF_K_MOCK_ADD, REEF_OP_MOCK_ADD}, {REEF_K_MOCK_MULTIPLY, REEF_OP_MOCK_MULTIPLY},
+        {REEF_K_ATTENTION, REEF_OP_ATTENTION},
+    };
+    for (auto& e : table) {
+        const size_t len = std::strlen(e.prefix);
+        const bool is_prefix = e.prefix[len - 1] == '_';
+        if (is_prefix ? n.compare(0, len, e.prefix) == 0 : n == e.prefix) return e.op;
+    }
+    return REEF_OP_NONE;
+}
+
+namespace {
+
+typedef long long i64;
+
+i64 cdiv(i64 a, i64 b) { return (a + b - 1) / b; }
+
+// The operands of one launch in pointer-slot order, each with the bytes it needs.
+struct Needs {
+    struct Slot { const char* role; i64 bytes; };
+    std::vector<Slot> slots;
+    i64 tasks = -1;  // workgroups the launch must have; -1 = whatever the graph file says
+    std::string bad; // non-empty: the attributes contradict themselves
+    void f32(const char* role, i64 elements) { slots.push_back({role, 4 * elements}); }
+    void raw(const char* role, i64 bytes) { slots.push_back({role, bytes}); }
+};
+
+struct Attrs {
+    const std::vector<int32_t>& v;
+    i64 operator[](int i) const { return (size_t)i < v.size() ? v[(size_t)i] : 0; }
+};
+
+bool all_positive(const Attrs& a, std::initializer_list<int> idx) {
+    for (int i : idx)
+        if (a[i] <= 0) return false;
+    return true;
+}
+
+void conv2d(const Attrs& a, Needs& n) {
+    if (a.v.size() <= (size_t)REEF_CONV_N_TILES) { n.bad = "too few attributes for a convolution"; return; }
+    if (!all_positive(a, {REEF_CONV_CIN, REEF_CONV_H, REEF_CONV_W, REEF_CONV_COUT, REEF_CONV_HO, REEF_CONV_WO,
+                          REEF_CONV_KH, REEF_CONV_KW, REEF_CONV_SH, REEF_CONV_SW, REEF_CONV_SPLIT_K,
+                          REEF_CONV_M_TILES, REEF_CONV_N_TILES}) ||
+        a[REEF_CONV_PH] < 0 || a[REEF_CONV_PW] < 0 || a[REEF_CONV_DST_OFF] < 0 || a[REEF_CONV_SYNC_OFF] < 0) {
+        n.bad = "a dimension of the convolution is not positive";
+        return;
+    }
+    const i64 cin = a[REEF_CONV_CIN], H = a[REEF_CONV_H], W = a[REEF_CONV_W], M = a[REEF_CONV_COUT];
+    const i64 Ho = a[REEF_CONV_HO], Wo = a[REEF_CONV_WO], kh = a[REEF_CONV_KH], kw = a[REEF_CONV_KW];
+    if (Ho != (H + 2 * a[REEF_CONV_PH] - kh) / a[REEF_CONV_SH] + 1 ||
+        Wo != (W + 2 * a[REEF_CONV_PW] - kw) / a[REEF_CONV_SW] + 1 || H + 2 * a[REEF_CONV_PH] < kh ||
+        W + 2 * a[REEF_CONV_PW] < kw) {
+        n.bad = "the output size does not follow from input, filter, stride and padding";
+        return;
+    }
+    const i64 N = Ho * Wo, split = a[REEF_CONV_SPLIT_K], flags = a[REEF_CONV_FLAGS], off = a[REEF_CONV_DST_OFF];
+    const bool fused = flags & REEF_F_FUSED_REDUCE;
+    n.f32("input", cin * H * W);
+    n.f32("weights", M * cin * kh * kw);
+    if (split > 1 && !fused) n.f32("partial sums", split * M * N);
+    else n.f32("output", off + M * N);
+    if (flags & REEF_F_BIAS) n.f32("bias", M);
+    if (flags & REEF_F_RESIDUAL) n.f32("residual", M * N);
+    if (flags & REEF_F_AFFINE) { n.f32("scale", M); n.f32("shift", M); }
+    if (flags & REEF_F_DUAL) { n.f32("second output", off + M * N); n.f32("second shift", M); }
+    if (flags & REEF_F_PRE_ACT) { n.f32("input scale", cin); n.f32("input shift", cin); }
+    if (fused) {
+        n.f32("partial sums", (split + ((flags & REEF_F_PAIR_FOLD) ? 1 : 0)) * M * N);
+        n.raw("tile counters", 4 * (a[REEF_CONV_SYNC_OFF] + a[REEF_CONV_M_TILES] * a[REEF_CONV_N_TILES]));
+    }
+    if (a[REEF_CONV_WPACK] != 0) {
+        if (a[REEF_CONV_WPACK] != (i64)n.slots.size()) { n.bad = "the packed weights are not the last operand"; return; }
+        n.f32("packed weights", cdiv(M, 16) * cdiv(cin, 4) * cdiv(kh * kw, 4) * 4 * 16 * 4);
+    }
+    n.tasks = split * a[REEF_CONV_M_TILES] * a[REEF_CONV_N_TILES];
+}
+
+void splitk_reduce(const Attrs& a, Needs& n) {
+    if (!all_positive(a, {REEF_RED_M, REEF_RED_N, REEF_RED_SPLIT_K}) || a[REEF_RED_DST_OFF] < 0) {
+        n.bad = "a dimension of the reduction is not positive";
+        return;
+    }
+    const i64 M = a[REEF_RED_M], MN = M * a[REEF_RED_N], flags = a[REEF_RED_FLAGS], off = a[REEF_RED_DST_OFF];
+    n.f32("partial sums", a[REEF_RED_SPLIT_K] * MN);
+    n.f32("output", off + MN);
+    if (flags & REEF_F_BIAS) n.f32("bias", M);
+    if (flags & REEF_F_RESIDUAL) n.f32("residual", MN);
+    if (flags & REEF_F_AFFINE) { n.f32("scale", M); n.f32("shift", M); }
+    if (flags & REEF_F_DUAL) { n.f32("second output", off + MN); n.f32("second shift", M); }
+    n.tasks = cdiv(MN, 1024);
+}
+
+void gemm(const Attrs& a, Needs& n) {
+    if (a.v.size() <= (size_t)REEF_GEMM_STRIDE_C) { n.bad = "too few attributes for a matrix product"; return; }
+    if (!all_positive(a, {REEF_GEMM_BATCH, REEF_GEMM_M, REEF_GEMM_N, REEF_GEMM_K, REEF_GEMM_M_TILES,
+                          REEF_GEMM_N_TILES, REEF_GEMM_LDA, REEF_GEMM_LDB, REEF_GEMM_LDC})) {
+        n.bad = "a dimension of the matrix product is not positive";
+        return;
+    }
+    for (int i : {REEF_GEMM_STRIDE_A, REEF_GEMM_STRIDE_B, REEF_GEMM_STRIDE_C, REEF_GEMM_OFF_A, REEF_GEMM_OFF_B,
+                  REEF_GEMM_OFF_C})
+        if (a[i] < 0) { n.bad = "a stride or an offset of the matrix product is negative"; return; }
+    const i64 b1 = a[REEF_GEMM_BATCH] - 1, M = a[REEF_GEMM_M], N = a[REEF_GEMM_N], K = a[REEF_GEMM_K];
+    const bool trans_b = a[REEF_GEMM_TRANS_B] != 0;
+    if ((K | a[REEF_GEMM_LDA] | a[REEF_GEMM_STRIDE_A] | a[REEF_GEMM_OFF_A] | a[REEF_GEMM_OFF_B] | a[REEF_GEMM_OFF_C]) & 3 ||
+        (trans_b && ((a[REEF_GEMM_LDB] | a[REEF_GEMM_STRIDE_B]) & 3))) {
+        n.bad = "K, a leading dimension, a stride or an offset is not a multiple of 4 (128-bit loads)";
+        return;
+    }
+    n.f32("A", a[REEF_GEMM_OFF_A] + b1 * a[REEF_GEMM_STRIDE_A] + (M - 1) * a[REEF_GEMM_LDA] + K);
+    if (trans_b) n.f32("B", a[REEF_GEMM_OFF_B] + b1 * a[REEF_GEMM_STRIDE_B] + (N - 1) * a[REEF_GEMM_LDB] + K);
+    else n.f32("B", a[REEF_GEMM_OFF_B] + b1 * a[REEF_GEMM_STRIDE_B] + (K - 1) * a[REEF_GEMM_LDB] + N);
+    n.f32("C", a[REEF_GEMM_OFF_C] + b1 * a[REEF_GEMM_STRIDE_C] + (M - 1) * a[REEF_GEMM_LDC] + N);
+    if (a[REEF_GEMM_FLAGS] & 1) n.f32("bias", N);
+    n.tasks = a[REEF_GEMM_BATCH] * a[REEF_GEMM_M_TILES] * a[REEF_GEMM_N_TILES];
+}
+
+void attention(const Attrs& a, Needs& n) {
+    if (!all_positive(a, {REEF_AT_SEQ, REEF_AT_HEAD_DIM, REEF_AT_HEADS, REEF_AT_LD, REEF_AT_LDO}) ||
+        a[REEF_AT_OFF_Q] < 0 || a[REEF_AT_OFF_K] < 0 || a[REEF_AT_OFF_V] < 0) {
+        n.bad = "a dimension of the attention is not positive";
+        return;
+    }
+    if (a[REEF_AT_SEQ] > REEF_AT_MAX_SEQ || a[REEF_AT_HEAD_DIM] > REEF_AT_MAX_HEAD_DIM) {
+        n.bad = "the sequence or the head is larger than the kernel's staging area";
+        return;
+    }
+    if ((a[REEF_AT_HEAD_DIM] | a[REEF_AT_LD] | a[REEF_AT_LDO] | a[REEF_AT_OFF_Q] | a[REEF_AT_OFF_K] | a[REEF_AT_OFF_V]) & 3) {
+        n.bad = "head size, a leading dimension or an offset is not a multiple of 4 (128-bit loads)";
+        return;
+    }
+    const i64 seq = a[REEF_AT_SEQ], width = a[REEF_AT_HEADS] * a[REEF_AT_HEAD_DIM];
+    i64 last = a[REEF_AT_OFF_Q];
+    if (a[REEF_AT_OFF_K] > last) last = a[REEF_AT_OFF_K];
+    if (a[REEF_AT_OFF_V] > last) last = a[REEF_AT_OFF_V];
+    n.f32("queries, keys and values", last + (seq - 1) * a[REEF_AT_LD] + width);
+    n.f32("context", (seq - 1) * a[REEF_AT_LDO] + width);
+    if (a[REEF_AT_FLAGS] & 1) n.raw("mask", seq);
+    n.tasks = a[REEF_AT_HEADS] * cdiv(seq, REEF_AT_ROWS);
+}
+
+// Fills `n` for the ops that are a few lines each; false for an op that is not judged.
+bool small_op(int op, const Attrs& a, i64 grid, Needs& n) {
+    switch (op) {
+    case REEF_OP_DWCONV2D: {
+        if (!all_positive(a, {REEF_DW_C, REEF_DW_H, REEF_DW_W, REEF_DW_HO, REEF_DW_WO, REEF_DW_KH, REEF_DW_KW,
+                              REEF_DW_SH, REEF_DW_SW}) || a[REEF_DW_PH] < 0 || a[REEF_DW_PW] < 0 ||
+            a[REEF_DW_HO] != (a[REEF_DW_H] + 2 * a[REEF_DW_PH] - a[REEF_DW_KH]) / a[REEF_DW_SH] + 1 ||
+            a[REEF_DW_WO] != (a[REEF_DW_W] + 2 * a[REEF_DW_PW] - a[REEF_DW_KW]) / a[REEF_DW_SW] + 1) {
+            n.bad = "the sizes of the depthwise convolution do not fit each other";
+            return true;
+        }
+        const i64 C = a[REEF_DW_C], out = C * a[REEF_DW_HO] * a[REEF_DW_WO];
+        n.f32("input", C * a[REEF_DW_H] * a[REEF_DW_W]);
+        n.f32("weights", C * a[REEF_DW_KH] * a[REEF_DW_KW]);
+        n.f32("output", out);
+        if (a[REEF_DW_FLAGS] & 1) n.f32("bias", C);
+        n.tasks = cdiv(out, 256);
+        return true;
+    }
+    case REEF_OP_POOL2D: {
+        if (!all_positive(a, {REEF_POOL_C, REEF_POOL_H, REEF_POOL_W, REEF_POOL_HO, REEF_POOL_WO, REEF_POOL_KH,
+                              REEF_POOL_KW, REEF_POOL_SH, REEF_POOL_SW}) || a[REEF_POOL_PH] < 0 || a[REEF_POOL_PW] < 0) {
+            n.bad = "a dimension of the pooling is not positive";
+            return true;
+        }
+        const i64 C = a[REEF_POOL_C], out = C * a[REEF_POOL_HO] * a[REEF_POOL_WO];
+        n.f32("input", C * a[REEF_POOL_H] * a[REEF_POOL_W]);
+        n.f32("output", out);
+        if (a[REEF_POOL_FLAGS] & 1) n.f32("bias", C);
+        n.tasks = cdiv(out, 256);
+        return true;
+    }
+    case REEF_OP_GLOBAL_AVGPOOL:
+        if (!all_positive(a, {REEF_GAP_C, REEF_GAP_HW})) { n.bad = "a dimension of the pooling is not positive"; return true; }
+        n.f32("input", a[REEF_GAP_C] * a[REEF_GAP_HW]);
+        n.f32("output", a[REEF_GAP_C]);
+        n.tasks = cdiv(a[REEF_GAP_C], 4);
+        return true;
+    case REEF_OP_ELTWISE: {
+        if (!all_positive(a, {REEF_ELT_C, REEF_ELT_INNER})) { n.bad = "a dimension is not positive"; return true; }
+        const i64 C = a[REEF_ELT_C], total = C * a[REEF_ELT_INNER];
+        n.f32("input", total);
+        n.f32("output", total);
+        if (a[REEF_ELT_FLAGS] & REEF_ELT_F_B) n.f32("second input", total);
+        if (a[REEF_ELT_FLAGS] & REEF_ELT_F_SCALE) n.f32("scale", C);
+        if (a[REEF_ELT_FLAGS] & REEF_ELT_F_SHIFT) n.f32("shift", C);
+        n.tasks = cdiv(total, 1024);
+        return true;
+    }
+    case REEF_OP_DENSE:
+        if (!all_positive(a, {REEF_DENSE_ROWS, REEF_DENSE_IN, REEF_DENSE_OUT})) { n.bad = "a dimension is not positive"; return true; }
+        n.f32("input", a[REEF_DENSE_ROWS] * a[REEF_DENSE_IN]);
+        n.f32("weights", a[REEF_DENSE_OUT] * a[REEF_DENSE_IN]);
+        n.f32("output", a[REEF_DENSE_ROWS] * a[REEF_DENSE_OUT]);
+        if (a[REEF_DENSE_FLAGS] & 1) n.f32("bias", a[REEF_DENSE_OUT]);
+        n.tasks = cdiv(a[REEF_DENSE_OUT], 4);
+        return true;
+    case REEF_OP_SOFTMAX:
+        if (!all_positive(a, {REEF_SM_ROWS, REEF_SM_COLS})) { n.bad = "a dimension is not positive"; return true; }
+        n.f32("input", a[REEF_SM_ROWS] * a[REEF_SM_COLS]);
+        n.f32("output", a[REEF_SM_ROWS] * a[REEF_SM_COLS]);
+        if (a[REEF_SM_FLAGS] & 1) n.raw("mask", a[REEF_SM_COLS]);
+        n.tasks = cdiv(a[REEF_SM_ROWS], 4);
+        return true;
+    case REEF_OP_LAYERNORM: {
+        if (!all_positive(a, {REEF_LN_ROWS, REEF_LN_COLS})) { n.bad = "a dimension is not positive"; return true; }
+        const i64 total = a[REEF_LN_ROWS] * a[REEF_LN_COLS];
+        n.f32("input", total);
+        n.f32("gamma", a[REEF_LN_COLS]);
+        n.f32("beta", a[REEF_LN_COLS]);
+        n.f32("output", total);
+        if (a[REEF_LN_FLAGS] & 1) n.f32("residual", total);
+        n.tasks = cdiv(a[REEF_LN_ROWS], 4);
+        return true;
+    }
+    case REEF_OP_BIAS_GELU: {
+        if (!all_positive(a, {REEF_GELU_ROWS, REEF_GELU_COLS})) { n.bad = "a dimension is not positive"; return true; }
+        const i64 total = a[REEF_GELU_ROWS] * a[REEF_GELU_COLS];
+        n.f32("input", total);
+        n.f32("output", total);
+        if (a[REEF_GELU_FLAGS] & 1) n.f32("bias", a[REEF_GELU_COLS]);
+        n.tasks = cdiv(total, 1024);
+        return true;
+    }
+    case REEF_OP_EMBEDDING: {
+        if (!all_positive(a, {REEF_EMB_SEQ, REEF_EMB_HIDDEN, REEF_EMB_VOCAB})) { n.bad = "a dimension is not positive"; return true; }
+        const i64 total = a[REEF_EMB_SEQ] * a[REEF_EMB_HIDDEN];
+        n.raw("token ids", 8 * a[REEF_EMB_SEQ]);
+        n.f32("token table", a[REEF_EMB_VOCAB] * a[REEF_EMB_HIDDEN]);
+        n.f32("output", total);
+        if (a[REEF_EMB_FLAGS] & 1) n.f32("position table", total);
+        if (a[REEF_EMB_FLAGS] & 2) n.f32("segment row", a[REEF_EMB_HIDDEN]);
+        n.tasks = cdiv(total, 1024);
+        return true;
+    }
+    case REEF_OP_COPY:
+        if (a[REEF_COPY_COUNT] <= 0 || a[REEF_COPY_DST_OFF] < 0) { n.bad = "count or offset of the copy is out of range"; return true; }
+        n.f32("input", a[REEF_COPY_COUNT]);
+        n.f32("output", a[REEF_COPY_DST_OFF] + a[REEF_COPY_COUNT]);
+        n.tasks = cdiv(a[REEF_COPY_COUNT], 1024);
+        return true;
+    case REEF_OP_TRANSPOSE: {
+        if (!all_positive(a, {REEF_TR_D0, REEF_TR_D1, REEF_TR_D2})) { n.bad = "a dimension is not positive"; return true; }
+        const i64 total = a[REEF_TR_D0] * a[REEF_TR_D1] * a[REEF_TR_D2];
+        n.f32("input", total);
+        n.f32("output", total);
+        if (a[REEF_TR_FLAGS] & 1) n.f32("bias", a[REEF_TR_D1] * a[REEF_TR_D2]);
+        n.tasks = cdiv(total, 1024);
+        return true;
+    }
+    case REEF_OP_MOCK_ADD:
+    case REEF_OP_MOCK_MULTIPLY:
+        // out[task * 128 + t] = a[t] (+|*) b[task * 128 + t]  (resource/mocked_kernel/mocked_kernel.cu:9-27)
+        n.f32("a", 128);
+        n.f32("b", grid * 128);
+        n.f32("out", grid * 128);
+        return true;
+    default:
+        return false;
+    }
+}
+
+}  // namespace
+
+bool kernel_fits_storages(const Model& m, size_t index, std::string* why) {
+    const KernelInfo& ki = m.kernels[index];
+    const std::string symbol = ki.name.substr(0, ki.name.find('#'));
+    const int op = op_from_symbol(symbol);
+    if (op == REEF_OP_NONE) return true;
+    const Attrs a{ki.attrs};
+    const i64 grid = (i64)ki.launch_params[0] * ki.launch_params[1] * ki.launch_params[2];
+    Needs n;
+    switch (op) {
+    case REEF_OP_CONV2D: conv2d(a, n); break;
+    case REEF_OP_SPLITK_REDUCE: splitk_reduce(a, n); break;
+    case REEF_OP_GEMM: gemm(a, n); break;
+    case REEF_OP_ATTENTION: attention(a, n); break;
+    default:
+        if (!small_op(op, a, grid, n)) return true;
+    }
+    char buf[512];
+    auto fail = [&](const char* msg) {
+        if (why) *why = "kernel " + std::to_string(index) + " (" + ki.name + "): " + msg;
+        return false;
+    };
+    if (!n.bad.empty()) return fail(n.bad.c_str());
+    if (n.slots.size() != ki.args.size()) {
+        std::snprintf(buf, sizeof buf, "its attributes ask for %zu operands, the graph file lists %zu", n.slots.size(),
+                      ki.args.size());
+        return fail(buf);
+    }
+    if (n.tasks >= 0 && grid != n.tasks) {
+        std::snprintf(buf, sizeof buf, "its attributes ask for %lld workgroups, the graph file launches %lld", n.tasks, grid);
+        return fail(buf);
+    }
+    for (size_t j = 0; j < n.slots.size(); ++j) {
+        if (ki.args[j] >= m.storage.size()) return fail("an operand names a storage that does not exist");
+        const StorageInfo& s = m.storage[ki.args[j]];
+        const i64 have = (i64)(s.size * Model::get_stype_size(s.stype)) - (i64)(ki.arg_offsets.empty() ? 0 : ki.arg_offsets[j]);
+        if (n.slots[j].bytes > have) {
+            std::snprintf(buf, sizeof buf, "operand %zu (%s) needs %lld bytes, storage %zu (%s) has %lld behind the operand's start",
+                          j, n.slots[j].role, n.slots[j].bytes, ki.args[j], s.name.c_str(), have);
+            return fail(buf);
+        }
+    }
+    return true;
+}
+
+}  // namespace executor
+}  // namespace reef

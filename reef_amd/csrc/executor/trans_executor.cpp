@@ -1,4 +1,5 @@
 #include "executor/trans_executor.h"
+#include "executor/op_extents.h"
 
 #include <cstring>
 
@@ -28,25 +29,7 @@ int TransExecutor::cu_partition_for(int block_num, int num_cus, int num_xcds) {
     return std::min(part, num_cus);
 }
 
-int TransExecutor::op_from_name(const std::string& n) {
-    struct { const char* prefix; int op; } table[] = {
-        {"reef_conv2d_", REEF_OP_CONV2D}, {"reef_gemm_", REEF_OP_GEMM},
-        {REEF_K_SPLITK_REDUCE, REEF_OP_SPLITK_REDUCE}, {REEF_K_DWCONV2D, REEF_OP_DWCONV2D},
-        {REEF_K_POOL2D, REEF_OP_POOL2D}, {REEF_K_GLOBAL_AVGPOOL, REEF_OP_GLOBAL_AVGPOOL},
-        {REEF_K_ELTWISE, REEF_OP_ELTWISE}, {REEF_K_DENSE, REEF_OP_DENSE},
-        {REEF_K_SOFTMAX, REEF_OP_SOFTMAX}, {REEF_K_LAYERNORM, REEF_OP_LAYERNORM},
-        {REEF_K_BIAS_GELU, REEF_OP_BIAS_GELU}, {REEF_K_EMBEDDING, REEF_OP_EMBEDDING},
-        {REEF_K_COPY, REEF_OP_COPY}, {REEF_K_TRANSPOSE, REEF_OP_TRANSPOSE},
-        {REEF_K_MOCK_ADD, REEF_OP_MOCK_ADD}, {REEF_K_MOCK_MULTIPLY, REEF_OP_MOCK_MULTIPLY},
-        {REEF_K_ATTENTION, REEF_OP_ATTENTION},
-    };
-    for (auto& e : table) {
-        const size_t len = std::strlen(e.prefix);
-        const bool is_prefix = e.prefix[len - 1] == '_';
-        if (is_prefix ? n.compare(0, len, e.prefix) == 0 : n == e.prefix) return e.op;
-    }
-    return REEF_OP_NONE;
-}
+int TransExecutor::op_from_name(const std::string& n) { return op_from_symbol(n); }
 
 Status TransExecutor::init_rt_executor(const char* json_file_path, GPUModule_t module) {
     const size_t n = model->kernels.size();

@@ -376,3 +376,88 @@ def test_every_padding_kernel_starts_its_wavefronts_in_the_same_state():
         assert state == ref, (name, state, ref)
         if name.startswith("merge_framework_"):
             assert group_seg == 0, name     # LDS of a merged launch is all dynamic, from offset 0
+
+
+def check_kernels(path):
+    why = ctypes.create_string_buffer(512)
+    st = L.reef_model_check_kernels(str(path).encode(), why, 512)
+    return st, why.value.decode()
+
+
+def test_every_generated_kernel_fits_its_storages(tmp_path):
+    """What the executors check at load time: the shape attributes of each kernel against the
+    storages it is given and its grid.  Every network of the generator passes, views included."""
+    from reef_amd.modelgen import nets
+    graphs = [nets.resnet(50, image=(3, 64, 64), classes=16, name="r50"),
+              nets.densenet(image=(3, 64, 64), classes=16, name="d"),
+              nets.mobilenet_v2(image=(3, 64, 64), classes=16, name="mb"),
+              nets.inception_v3(image=(3, 107, 107), classes=16, name="inc"),
+              nets.bert(layers=2, hidden=128, heads=2, seq=48, ffn=256, vocab=100, name="bert", attention_mask=True),
+              nets.bert(layers=1, hidden=128, heads=2, seq=48, ffn=256, vocab=100, name="bert3",
+                        fused_attention=False),
+              nets.mocked_kernel(name="mock")]
+    for g in graphs:
+        g.write(str(tmp_path), link_code_objects=False)
+        st, why = check_kernels(tmp_path / (g.name + ".json"))
+        assert st == 0, (g.name, why)
+
+
+def test_kernels_that_do_not_fit_are_refused(tmp_path):
+    """A graph file whose attributes ask for more than its storages hold, for another number of
+    operands or for another grid is refused with a reason, by the check and by an executor that
+    loads it (no launch is ever made from it)."""
+    from reef_amd.modelgen import nets
+    from tests.fakehal import FakeHal
+    g = nets.bert(layers=1, hidden=128, heads=2, seq=48, ffn=256, vocab=100, name="b", attention_mask=True)
+    g.write(str(tmp_path))
+    good = json.load(open(tmp_path / "b.json"))
+    by_symbol = {}
+    for i, k in enumerate(good["kernels"]):
+        by_symbol.setdefault(k["name"].split("#")[0].rsplit("_", 1)[0] if k["name"].startswith("reef_gemm") else
+                             k["name"].split("#")[0], i)
+    at, ln, gm = by_symbol["reef_attention"], by_symbol["reef_layernorm"], by_symbol["reef_gemm_ntd"]
+
+    def broken(edit):
+        m = json.loads(json.dumps(good))
+        edit(m)
+        p = tmp_path / "x.json"
+        p.write_text(json.dumps(m))
+        return p
+
+    def shrink(m):       # the output of the attention loses its last element
+        m["storage"][m["kernels"][at]["args"][1]]["size"] -= 1
+
+    def longer(m):       # more key positions than the kernel can stage
+        m["kernels"][at]["attrs"][0] = 129
+
+    def grid(m):         # one workgroup too many
+        m["kernels"][ln]["launch_params"][0] += 1
+
+    def operand(m):      # the residual flag without a residual operand
+        k = m["kernels"][ln]
+        k["attrs"][2] ^= 1
+        if not k["attrs"][2] & 1:
+            k["args"].append(k["args"][0])
+
+    def offset(m):       # a matrix that starts so late that its last row leaves the storage
+        m["kernels"][gm]["attrs"][17] += 4
+
+    def view(m):         # the same through an operand view
+        k = m["kernels"][ln]
+        k["arg_offsets"] = [16] + [0] * (len(k["args"]) - 1)
+
+    for edit, word in ((shrink, "context"), (longer, "staging"), (grid, "workgroups"), (operand, "operands"),
+                       (offset, "needs"), (view, "input")):
+        p = broken(edit)
+        st, why = check_kernels(p)
+        assert st != 0 and word in why, (edit.__name__, st, why)
+    # and the executor refuses the file
+    fake = FakeHal().install()
+    try:
+        exe = B.Executor(B.BASE)
+        exe.load(str(tmp_path / "b.json"), str(tmp_path / "b.raw.co"))      # the file as generated loads
+        del exe
+        with pytest.raises(B.ReefError, match="OutOfRange"):
+            B.Executor(B.BASE).load(str(broken(shrink)), str(tmp_path / "b.raw.co"))
+    finally:
+        fake.remove()
