@@ -1,6 +1,7 @@
 #include "executor/op_extents.h"
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "reef_kernels.h"
@@ -55,7 +56,7 @@ bool all_positive(const Attrs& a, std::initializer_list<int> idx) {
     return true;
 }
 
-void conv2d(const Attrs& a, Needs& n) {
+void conv2d(const std::string& symbol, const Attrs& a, Needs& n) {
     if (a.v.size() <= (size_t)REEF_CONV_N_TILES) { n.bad = "too few attributes for a convolution"; return; }
     if (!all_positive(a, {REEF_CONV_CIN, REEF_CONV_H, REEF_CONV_W, REEF_CONV_COUT, REEF_CONV_HO, REEF_CONV_WO,
                           REEF_CONV_KH, REEF_CONV_KW, REEF_CONV_SH, REEF_CONV_SW, REEF_CONV_SPLIT_K,
@@ -74,6 +75,43 @@ void conv2d(const Attrs& a, Needs& n) {
     }
     const i64 N = Ho * Wo, split = a[REEF_CONV_SPLIT_K], flags = a[REEF_CONV_FLAGS], off = a[REEF_CONV_DST_OFF];
     const bool fused = flags & REEF_F_FUSED_REDUCE;
+    // the loader family is part of the symbol: what it was compiled for must be what the layer is
+    const i64 K = cin * kh * kw, taps = kh * kw;
+    const bool unit = kh == 1 && kw == 1 && a[REEF_CONV_PH] == 0 && a[REEF_CONV_PW] == 0;
+    const std::string fam = symbol.substr(std::strlen("reef_conv2d_"));
+    const std::string head = fam.substr(0, fam.find('_'));  // "d9", "d9k", "r9k", "pw", a tile for the general family
+    if (head.empty()) { n.bad = "not a convolution symbol"; return; }
+    i64 mode = REEF_CONV_MODE_GENERAL;
+    bool fits = K % 4 == 0, packed = false;
+    if (fam.compare(0, 3, "pw_") == 0) {
+        mode = REEF_CONV_MODE_POINTWISE;
+        fits = unit && a[REEF_CONV_SH] == 1 && a[REEF_CONV_SW] == 1 && N % 4 == 0 && K % 4 == 0;
+    } else if (fam.compare(0, 2, "u_") == 0) {
+        mode = REEF_CONV_MODE_UNALIGNED;
+        fits = true;
+    } else if (fam.compare(0, 3, "p1_") == 0) {
+        mode = REEF_CONV_MODE_DIRECT_PRE;
+        fits = unit && cin % 8 == 0 && (flags & REEF_F_PRE_ACT);
+    } else if (fam.compare(0, 2, "r9") == 0) {
+        mode = REEF_CONV_MODE_ROWS;
+        packed = head.back() == 'k';
+        fits = kh == 3 && kw == 3 && a[REEF_CONV_SH] == 1 && a[REEF_CONV_SW] == 1 && a[REEF_CONV_PH] == 1 &&
+               a[REEF_CONV_PW] == 1;
+    } else if (fam[0] == 'd') {
+        mode = REEF_CONV_MODE_DIRECT;
+        const i64 compiled = std::atoi(fam.c_str() + 1);
+        packed = head.back() == 'k';
+        fits = compiled == taps && (taps > 1 || cin % 8 == 0);
+    }
+    if (!fits || mode != a[REEF_CONV_MODE] || ((flags & REEF_F_PRE_ACT) != 0) != (mode == REEF_CONV_MODE_DIRECT_PRE)) {
+        n.bad = "the layer is not one that this symbol's loader family was compiled for";
+        return;
+    }
+    if (packed != (a[REEF_CONV_WPACK] != 0)) { n.bad = "packed weights and symbol do not go together"; return; }
+    if (a[REEF_CONV_K_CHUNK] <= 0 || split * a[REEF_CONV_K_CHUNK] < K) {
+        n.bad = "the splits do not cover the reduction";
+        return;
+    }
     n.f32("input", cin * H * W);
     n.f32("weights", M * cin * kh * kw);
     if (split > 1 && !fused) n.f32("partial sums", split * M * N);
@@ -291,7 +329,7 @@ bool kernel_fits_storages(const Model& m, size_t index, std::string* why) {
     const i64 grid = (i64)ki.launch_params[0] * ki.launch_params[1] * ki.launch_params[2];
     Needs n;
     switch (op) {
-    case REEF_OP_CONV2D: conv2d(a, n); break;
+    case REEF_OP_CONV2D: conv2d(symbol, a, n); break;
     case REEF_OP_SPLITK_REDUCE: splitk_reduce(a, n); break;
     case REEF_OP_GEMM: gemm(a, n); break;
     case REEF_OP_ATTENTION: attention(a, n); break;

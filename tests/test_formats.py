@@ -451,6 +451,24 @@ def test_kernels_that_do_not_fit_are_refused(tmp_path):
         p = broken(edit)
         st, why = check_kernels(p)
         assert st != 0 and word in why, (edit.__name__, st, why)
+    # a convolution under a symbol that was compiled for another filter, and splits that stop short
+    r = nets.resnet(18, image=(3, 32, 32), classes=8, name="r")
+    r.write(str(tmp_path), link_code_objects=False)
+    good_b, good = good, json.load(open(tmp_path / "r.json"))
+    ci = next(i for i, k in enumerate(good["kernels"]) if k["name"].startswith("reef_conv2d_d1_"))
+
+    def family(m):
+        k = m["kernels"][ci]
+        k["name"] = k["name"].replace("reef_conv2d_d1_", "reef_conv2d_d9_")
+
+    def chunk(m):
+        a = m["kernels"][ci]["attrs"]
+        a[16] = a[0] * a[6] * a[7] // (2 * a[15])       # each split takes half of its share of K
+
+    for edit, word in ((family, "loader family"), (chunk, "cover")):
+        st, why = check_kernels(broken(edit))
+        assert st != 0 and word in why, (edit.__name__, st, why)
+    good = good_b
     # and the executor refuses the file
     fake = FakeHal().install()
     try:
