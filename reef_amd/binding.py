@@ -50,6 +50,14 @@ def _check(what, st):
         raise ReefError(what, st)
 
 
+def check_model(json_path):
+    """(ok, reason): whether every kernel of a graph file fits the storages it names, its operand
+    count and its grid -- the check an executor makes when it loads the file, without a device."""
+    why = ctypes.create_string_buffer(512)
+    st = lib().reef_model_check_kernels(str(json_path).encode(), why, 512)
+    return st == 0, why.value.decode()
+
+
 class Executor:
     """ExecutorBase / TransExecutor / HybridExecutor behind one Python class."""
 

@@ -379,9 +379,8 @@ def test_every_padding_kernel_starts_its_wavefronts_in_the_same_state():
 
 
 def check_kernels(path):
-    why = ctypes.create_string_buffer(512)
-    st = L.reef_model_check_kernels(str(path).encode(), why, 512)
-    return st, why.value.decode()
+    ok, why = B.check_model(path)
+    return (0 if ok else 1), why
 
 
 def test_every_generated_kernel_fits_its_storages(tmp_path):
