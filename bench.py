@@ -24,6 +24,13 @@ The same JSON line carries
   * two further co-location scenarios (dynamic kernel padding with a
     MobileNetV2 best-effort client; Inception-v3 real-time with two BERT-base
     best-effort clients), shorter runs.
+
+Standard output is ONE compact JSON line (a few KB: the contract fields, `roofline`,
+`cpu_baseline` and a handful of scalars to read beside `value`).  Everything else -- every
+co-location leg in full, the per-kernel and per-shape tables, the schedule modes -- goes to
+the file named by --detail-out.  After every co-location leg the real-time model's and every
+best-effort model's storages are compared bit for bit with a solo run of the same model
+(`corun_outputs_bit_identical`); a difference makes the run exit non-zero.
 """
 import argparse
 import json
@@ -234,6 +241,56 @@ def model_input(name):
     return "data", nets.image_input(name, (3, side, side))
 
 
+class SoloBits:
+    """Every float storage a model's kernels write, after one uninterrupted run of the model
+    alone: what the same model must hold, bit for bit, after a co-location leg -- preempted and
+    restarted, padded into real-time launches or sharing its launches with best-effort work
+    (the two guarantees of src/reef/test/test.cpp:448-536)."""
+
+    def __init__(self, models, name):
+        from reef_amd import binding as B
+        g, d = models[name]
+        self.name = name
+        self.model = json.load(open(os.path.join(d, g.name + ".json")))
+        written = set()
+        for k in self.model["kernels"]:
+            written.update(k["args"])
+        # not inputs, parameters, arrival counters or the split-K workspaces (scratch whose
+        # content depends on how the kernel was launched)
+        self.idx = [i for i in sorted(written)
+                    if self.model["storage"][i]["stype"] == "float32"
+                    and self.model["storage"][i]["name"] not in ("data", "input0", "reef_sync")
+                    and not self.model["storage"][i]["name"].startswith("p")]
+        key, x = model_input(name)
+        exe = B.Executor.from_dir(d, g.name, B.HYBRID)
+        exe.set_input_checked(key, x)
+        exe.execute()
+        self.state = {i: exe.get_data(i, self.model["storage"][i]["size"]) for i in self.idx}
+        exe.close()
+
+    def differs(self, sched, mid):
+        """None, or a description of the first storage of model `mid` that differs."""
+        for i in self.idx:
+            got = sched.get_data(mid, i, self.model["storage"][i]["size"])
+            if not np.array_equal(got, self.state[i]):
+                bad = int(np.flatnonzero(got != self.state[i])[0])
+                return "%s storage %d element %d: %r vs solo %r" % (self.name, i, bad, float(got[bad]),
+                                                                    float(self.state[i][bad]))
+        for i, st in enumerate(self.model["storage"]):
+            if st["name"] == "reef_sync" and sched.get_data(mid, i, st["size"], np.int32).any():
+                return "%s: split-K arrival counters left non-zero" % self.name
+        return None
+
+
+_SOLO_BITS = {}
+
+
+def solo_bits(models, name):
+    if name not in _SOLO_BITS:
+        _SOLO_BITS[name] = SoloBits(models, name)
+    return _SOLO_BITS[name]
+
+
 def summarize(r, sched, n_be):
     lat = r["rt_latency_us"]
     return {"rt_ms": {"p50": pct(lat, 50), "p99": pct(lat, 99), "mean": round(float(lat.mean()) / 1e3, 4),
@@ -316,9 +373,116 @@ def corun(models, rt_name, be_name, n_be, mode, requests, warmup, wait_sync=True
     out["preempt_phase_ns"] = s.preempt_phases()
     out["padded_kernels"] = int(s.padded_kernels())
     out["kernel_select_ns"] = int(s.avg_kernel_sel_latency())
+    # the clients stopped after their current task; every best-effort model completes one more
+    # uninterrupted inference so that its final state is that of a whole run, then every model
+    # of this scheduler must hold the bits of its solo run
+    if n_be:
+        s.run_load(rt, bes, 0, be_only_ms=40)
+    why = solo_bits(models, rt_name).differs(s, rt)
+    for m in bes:
+        why = why or solo_bits(models, be_name).differs(s, m)
+    out["outputs_bit_identical_to_solo"] = why is None
+    if why is not None:
+        out["outputs_differ"] = why
+        print("bench: co-run outputs differ from the solo run: %s" % why, file=sys.stderr)
     s.shutdown()
     s.close()
     return out
+
+
+def corun_legs(detail):
+    """Every co-location leg (a dict with a `loaded` summary) anywhere in the full result."""
+    legs = []
+
+    def walk(v):
+        if isinstance(v, dict):
+            if "loaded" in v and "outputs_bit_identical_to_solo" in v:
+                legs.append(v)
+            for k, w in v.items():
+                if k != "schedule_modes":
+                    walk(w)
+    walk(detail)
+    return legs
+
+
+COMPACT_LIMIT = 6144
+
+
+def compact_line(detail):
+    """The one line of standard output: the contract fields, `roofline`, `cpu_baseline` and the few
+    scalars needed to read `value` (with --steps 20 the p99 is the largest of 20 Poisson-queued
+    requests: `rt_p50_ms` and the execution-only percentiles say what a request costs without
+    the queueing).  Kept below COMPACT_LIMIT bytes whatever the full result holds."""
+    keep = ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better",
+            "scaling", "vs_baseline", "dtype", "data", "config")
+    line = {k: detail.get(k) for k in keep}
+    rf = detail.get("roofline") or {}
+    line["roofline"] = {k: rf.get(k) for k in ("bound", "kernel", "achieved", "peak", "unit", "frac", "traffic",
+                                                "launches_per_inference", "avg_launch_us", "avg_launch_gflop")}
+    cb = detail.get("cpu_baseline")
+    if cb is not None:
+        line["cpu_baseline"] = {k: cb.get(k) for k in ("value", "unit", "cores", "kind", "sample")}
+        line["cpu_baseline"]["sample"] = str(line["cpu_baseline"]["sample"])[:300]
+        if "oracle" in cb:
+            line["cpu_baseline"]["oracle_ms"] = cb["oracle"]["value"]
+    head = detail.get("corun_resnet152_4x_densenet201") or {}
+    loaded, solo = head.get("loaded") or {}, head.get("solo") or {}
+    pre = head.get("preempt_us") or {}
+    dev = pre.get("device") or {}
+
+    def at(dct, *path):
+        for k in path:
+            dct = dct.get(k) if isinstance(dct, dict) else None
+        return dct
+    line.update({
+        "rt_p50_ms": at(loaded, "rt_ms", "p50"),
+        "rt_exec_p50_ms": at(loaded, "rt_exec_ms", "p50"),
+        "rt_exec_p99_ms": at(loaded, "rt_exec_ms", "p99"),
+        "rt_solo_p50_ms": at(solo, "rt_ms", "p50"),
+        "rt_solo_p99_ms": at(solo, "rt_ms", "p99"),
+        "rt_p99_vs_solo": detail.get("rt_p99_vs_solo"),
+        "rt_p50_vs_solo": detail.get("rt_p50_vs_solo"),
+        "rt_exec_p99_vs_solo": detail.get("rt_exec_p99_vs_solo"),
+        "preempt_host_us": {k: pre.get(k) for k in ("mean", "p99", "max")} if pre else None,
+        "preempt_device_us": {k: dev.get(k) for k in ("mean", "p99", "max")} if dev else None,
+        "be_inferences_per_s": loaded.get("be_inferences_per_s"),
+        "be_only_inferences_per_s": head.get("be_only_inferences_per_s"),
+        "solo_device_ms": at(detail, "solo_back_to_back_ms", "mean_device"),
+        "rt_launches_per_inference": at(detail, "config", "rt_kernels_per_inference"),
+        "model_tflops": detail.get("model_tflops"),
+        "conv_tflops_all_layers": detail.get("conv_tflops_all_layers"),
+        "corun_outputs_bit_identical": detail.get("corun_outputs_bit_identical"),
+        "parity_logits_max_rel_err_vs_oracle": detail.get("parity_logits_max_rel_err_vs_oracle"),
+    })
+    other = {}
+    for key, label in (("corun_dkp_mobilenetv2", "cfg4_rt_resnet152_be_mobilenetv2"),
+                       ("corun_inceptionv3_2x_bert", "cfg5_rt_inceptionv3_be_2x_bert_base")):
+        leg = detail.get(key)
+        if leg is None:
+            continue
+        reset = None
+        if "reef" in leg:
+            leg, reset = leg["reef"], leg.get("reset")
+        other[label] = {"rt_exec_p50_ms": at(leg, "loaded", "rt_exec_ms", "p50"),
+                        "rt_solo_exec_p50_ms": at(leg, "solo", "rt_exec_ms", "p50"),
+                        "be_inferences_per_s": at(leg, "loaded", "be_inferences_per_s"),
+                        "padded_kernels": leg.get("padded_kernels"),
+                        "preempt_device_us_p99": at(leg, "preempt_us", "device", "p99")}
+        if reset is not None:
+            other[label]["be_inferences_per_s_reset_mode"] = at(reset, "loaded", "be_inferences_per_s")
+    if other:
+        line["other_configs"] = other
+    for nm in ("mobilenetv2", "bert_base"):
+        v = at(detail, "solo_kernels_" + nm, "model_device_ms")
+        if v is not None:
+            line.setdefault("solo_device_ms_other_models", {})[nm] = v
+    text = json.dumps(line, separators=(",", ":"))
+    for drop in ("solo_device_ms_other_models", "other_configs"):   # never reached at today's sizes
+        if len(text) <= COMPACT_LIMIT:
+            break
+        line.pop(drop, None)
+        text = json.dumps(line, separators=(",", ":"))
+    return text
 
 
 def main():
@@ -339,6 +503,9 @@ def main():
                     help="also run a plain copy kernel over this many MiB 20 times (scale for the "
                          "FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--workdir", default=None)
+    ap.add_argument("--detail-out", default=None, metavar="FILE",
+                    help="where the full result goes (every co-location leg, per-kernel and per-shape tables); "
+                         "default gpurun_out/bench_detail.json beside this file")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (replicas per GPU share nothing); "
@@ -472,6 +639,8 @@ def main():
         "rt_p99_vs_solo": round(p99 / solo_p99, 4),
         "rt_p50_vs_solo": None if args.solo_only
         else round(head["loaded"]["rt_ms"]["p50"] / head["solo"]["rt_ms"]["p50"], 4),
+        "rt_exec_p99_vs_solo": None if args.solo_only
+        else round(head["loaded"]["rt_exec_ms"]["p99"] / head["solo"]["rt_exec_ms"]["p99"], 4),
         "preempt_us": None if args.solo_only else head["preempt_us"],
         "corun_resnet152_4x_densenet201": head,
         "corun_reset_mode": reset_only,
@@ -555,18 +724,45 @@ def main():
                     "rt_exec_ms_p99": r["loaded"]["rt_exec_ms"]["p99"],
                     "be_inferences_per_s": r["loaded"]["be_inferences_per_s"],
                     "switch_us_mean": r["preempt_us"]["mean"], "switch_us_p99": r["preempt_us"]["p99"],
-                    "rt_requests": r["preempt_us"]["n"]}
+                    "rt_requests": r["preempt_us"]["n"],
+                    "outputs_bit_identical_to_solo": r.get("outputs_bit_identical_to_solo")}
             for label, r in runs.items()}
     if not args.no_cpu:
+        # two stand-ins for "the model compiled by TVM for llvm" (TVM is not installed): the CPU
+        # oracle and the same network as torch.nn.functional calls.  The stated baseline is the
+        # faster of the two; the other is kept beside it.
         cb, orc = cpu_baseline(d, g.name, x)
-        out["cpu_baseline"] = cb
         ref = np.asarray(orc.storage[logits_idx], np.float64)
         out["parity_logits_max_rel_err_vs_oracle"] = float(np.abs(got - ref).max() / np.abs(ref).max())
         tc = torch_cpu_baseline(g, x)
         if tc is not None:
-            out["cpu_baseline"]["torch_cpu"] = tc[0]
             out["parity_logits_max_rel_err_vs_torch_cpu"] = float(np.abs(got - tc[1]).max() / np.abs(tc[1]).max())
-    print(json.dumps(out))
+        if tc is not None and tc[0]["value"] < cb["value"]:
+            out["cpu_baseline"] = {"value": tc[0]["value"], "unit": "ms", "cores": tc[0]["threads"], "kind": "port",
+                                   "sample": tc[0]["sample"] + "; stands in for the TVM-llvm build of the model "
+                                             "(TVM is not installed)",
+                                   "oracle": {"value": cb["value"], "unit": "ms", "cores": cb["cores"],
+                                              "sample": cb["sample"]}}
+        else:
+            out["cpu_baseline"] = cb
+            if tc is not None:
+                out["cpu_baseline"]["torch_cpu"] = tc[0]
+    identical = [leg.get("outputs_bit_identical_to_solo") for leg in corun_legs(out)]
+    identical += [m.get("outputs_bit_identical_to_solo") for m in out.get("schedule_modes", {}).values()]
+    out["corun_outputs_bit_identical"] = all(identical) if identical else None
+    line = compact_line(out)
+    detail_path = args.detail_out or os.path.join(ROOT, "gpurun_out", "bench_detail.json")
+    try:
+        os.makedirs(os.path.dirname(os.path.abspath(detail_path)), exist_ok=True)
+        with open(detail_path, "w") as f:
+            json.dump(out, f)
+        print("bench: full tables and every co-location leg in %s" % detail_path, file=sys.stderr)
+    except OSError as e:
+        print("bench: could not write %s (%s)" % (detail_path, e), file=sys.stderr)
+    sys.stdout.flush()
+    print(line)
+    if out["corun_outputs_bit_identical"] is False:
+        sys.exit(1)
 
 
 if __name__ == "__main__":

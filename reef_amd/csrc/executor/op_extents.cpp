@@ -35,6 +35,12 @@ typedef long long i64;
 
 i64 cdiv(i64 a, i64 b) { return (a + b - 1) / b; }
 
+// The kernels divide task, tile and pixel numbers through a float reciprocal with a remainder
+// correction (div_small), which is exact for operands below 2^22; and a tensor must stay below
+// 1 GiB, the byte offset that stands for "outside" in their buffer loads.
+constexpr i64 kDivSmallLimit = 1ll << 22;
+constexpr i64 kTensorLimit = 1ll << 30;
+
 // The operands of one launch in pointer-slot order, each with the bytes it needs.
 struct Needs {
     struct Slot { const char* role; i64 bytes; };
@@ -74,6 +80,15 @@ void conv2d(const std::string& symbol, const Attrs& a, Needs& n) {
         return;
     }
     const i64 N = Ho * Wo, split = a[REEF_CONV_SPLIT_K], flags = a[REEF_CONV_FLAGS], off = a[REEF_CONV_DST_OFF];
+    if (N >= kDivSmallLimit || H * W >= kDivSmallLimit ||
+        split * a[REEF_CONV_M_TILES] * a[REEF_CONV_N_TILES] >= kDivSmallLimit) {
+        n.bad = "an image or the task count is 4 Mi or more (the kernels' index arithmetic is exact below that)";
+        return;
+    }
+    if (4 * cin * H * W >= kTensorLimit || 4 * M * cin * kh * kw >= kTensorLimit || 4 * (off + M * N) >= kTensorLimit) {
+        n.bad = "a tensor of the convolution is 1 GiB or more";
+        return;
+    }
     const bool fused = flags & REEF_F_FUSED_REDUCE;
     // the loader family is part of the symbol: what it was compiled for must be what the layer is
     const i64 K = cin * kh * kw, taps = kh * kw;
@@ -170,6 +185,7 @@ void gemm(const Attrs& a, Needs& n) {
     n.f32("C", a[REEF_GEMM_OFF_C] + b1 * a[REEF_GEMM_STRIDE_C] + (M - 1) * a[REEF_GEMM_LDC] + N);
     if (a[REEF_GEMM_FLAGS] & 1) n.f32("bias", N);
     n.tasks = a[REEF_GEMM_BATCH] * a[REEF_GEMM_M_TILES] * a[REEF_GEMM_N_TILES];
+    if (n.tasks >= kDivSmallLimit) n.bad = "4 Mi workgroups or more (the kernels' index arithmetic is exact below that)";
 }
 
 void attention(const Attrs& a, Needs& n) {
@@ -208,6 +224,10 @@ bool small_op(int op, const Attrs& a, i64 grid, Needs& n) {
             return true;
         }
         const i64 C = a[REEF_DW_C], out = C * a[REEF_DW_HO] * a[REEF_DW_WO];
+        if (a[REEF_DW_HO] * a[REEF_DW_WO] >= kDivSmallLimit || 4 * C * a[REEF_DW_H] * a[REEF_DW_W] >= kTensorLimit) {
+            n.bad = "an image of 4 Mi pixels or a tensor of 1 GiB or more";
+            return true;
+        }
         n.f32("input", C * a[REEF_DW_H] * a[REEF_DW_W]);
         n.f32("weights", C * a[REEF_DW_KH] * a[REEF_DW_KW]);
         n.f32("output", out);
@@ -222,6 +242,10 @@ bool small_op(int op, const Attrs& a, i64 grid, Needs& n) {
             return true;
         }
         const i64 C = a[REEF_POOL_C], out = C * a[REEF_POOL_HO] * a[REEF_POOL_WO];
+        if (a[REEF_POOL_HO] * a[REEF_POOL_WO] >= kDivSmallLimit || 4 * C * a[REEF_POOL_H] * a[REEF_POOL_W] >= kTensorLimit) {
+            n.bad = "an image of 4 Mi pixels or a tensor of 1 GiB or more";
+            return true;
+        }
         n.f32("input", C * a[REEF_POOL_H] * a[REEF_POOL_W]);
         n.f32("output", out);
         if (a[REEF_POOL_FLAGS] & 1) n.f32("bias", C);
@@ -300,6 +324,7 @@ bool small_op(int op, const Attrs& a, i64 grid, Needs& n) {
     case REEF_OP_TRANSPOSE: {
         if (!all_positive(a, {REEF_TR_D0, REEF_TR_D1, REEF_TR_D2})) { n.bad = "a dimension is not positive"; return true; }
         const i64 total = a[REEF_TR_D0] * a[REEF_TR_D1] * a[REEF_TR_D2];
+        if (a[REEF_TR_D0] * a[REEF_TR_D1] >= kDivSmallLimit) { n.bad = "4 Mi rows or more"; return true; }
         n.f32("input", total);
         n.f32("output", total);
         if (a[REEF_TR_FLAGS] & 1) n.f32("bias", a[REEF_TR_D1] * a[REEF_TR_D2]);

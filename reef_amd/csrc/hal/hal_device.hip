@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <chrono>
+#include <mutex>
 #include <cstdint>
 
 #include "reef_hal.h"
@@ -41,6 +42,8 @@ int64_t now_ns() {
                std::chrono::steady_clock::now().time_since_epoch()).count();
 }
 
+// the mailbox of the clock exchange and its round number: one exchange at a time per process
+std::mutex g_probe_mtx;
 volatile uint32_t* g_mailbox = nullptr;
 uint32_t g_round = 0;
 
@@ -63,6 +66,7 @@ int reef_hal_hip_fill(hipStream_t stream, void* p, int byte, size_t n) {
 // One correlated (host steady clock, device wall clock) pair: best of `tries` exchanges.
 int reef_hal_hip_clock_probe(hipStream_t stream, int64_t* host_ns, uint64_t* device_ticks, int64_t* err_ns,
                              int* ticks_per_us) {
+    std::lock_guard<std::mutex> probe_lock(g_probe_mtx);
     if (!g_mailbox) {
         void* p = nullptr;
         if (hipHostMalloc(&p, 64, hipHostMallocDefault) != hipSuccess) {

@@ -134,24 +134,35 @@ __device__ __forceinline__ const T& kernarg_at(int byte_offset) {
 // lines are in the scalar cache and those reads cost a cache hit.  The loaded words themselves
 // are not used; the wait is part of the statement, so no register is written behind the
 // compiler's back.
+// Only words of the block itself are read: one every 64 bytes from its start, and its last
+// word (the block need not start on a line boundary, so its tail may lie on a line of its
+// own).  An offset that would fall behind the block is moved onto the last word.
+template <int BYTES, int I>
+struct KernargWord {
+    static constexpr int value = I * 64 + 4 <= BYTES ? I * 64 : BYTES - 4;
+    static_assert(value >= 0 && value + 4 <= BYTES && value % 4 == 0, "reads inside the argument block only");
+};
 template <int BYTES>
 __device__ __forceinline__ void kernarg_warm() {
     const char* base = (const char*)__builtin_amdgcn_kernarg_segment_ptr();
-    static_assert(BYTES <= 512, "argument blocks are at most 512 bytes");
-    int t0, t1, t2, t3, t4, t5, t6, t7;
-    if (BYTES <= 128)
-        asm volatile("s_load_dword %0, %2, 0x0\n\ts_load_dword %1, %2, 0x40\n\ts_waitcnt lgkmcnt(0)"
-                     : "=&s"(t0), "=&s"(t1) : "s"(base) : "memory");
-    else if (BYTES <= 256)
-        asm volatile("s_load_dword %0, %4, 0x0\n\ts_load_dword %1, %4, 0x40\n\ts_load_dword %2, %4, 0x80\n\t"
-                     "s_load_dword %3, %4, 0xc0\n\ts_waitcnt lgkmcnt(0)"
-                     : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3) : "s"(base) : "memory");
+    static_assert(BYTES >= 4 && BYTES % 4 == 0 && BYTES <= 512, "argument blocks are whole words, at most 512 bytes");
+    int t0, t1, t2, t3, t4, t5, t6, t7, t8;
+#define REEF_KW(I) "n"(KernargWord<BYTES, I>::value)
+    if (BYTES <= 256)
+        asm volatile("s_load_dword %0, %5, %6\n\ts_load_dword %1, %5, %7\n\ts_load_dword %2, %5, %8\n\t"
+                     "s_load_dword %3, %5, %9\n\ts_load_dword %4, %5, %10\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4)
+                     : "s"(base), REEF_KW(0), REEF_KW(1), REEF_KW(2), REEF_KW(3), "n"(BYTES - 4) : "memory");
     else
-        asm volatile("s_load_dword %0, %8, 0x0\n\ts_load_dword %1, %8, 0x40\n\ts_load_dword %2, %8, 0x80\n\t"
-                     "s_load_dword %3, %8, 0xc0\n\ts_load_dword %4, %8, 0x100\n\ts_load_dword %5, %8, 0x140\n\t"
-                     "s_load_dword %6, %8, 0x180\n\ts_load_dword %7, %8, 0x1c0\n\ts_waitcnt lgkmcnt(0)"
-                     : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7)
-                     : "s"(base) : "memory");
+        asm volatile("s_load_dword %0, %9, %10\n\ts_load_dword %1, %9, %11\n\ts_load_dword %2, %9, %12\n\t"
+                     "s_load_dword %3, %9, %13\n\ts_load_dword %4, %9, %14\n\ts_load_dword %5, %9, %15\n\t"
+                     "s_load_dword %6, %9, %16\n\ts_load_dword %7, %9, %17\n\ts_load_dword %8, %9, %18\n\t"
+                     "s_waitcnt lgkmcnt(0)"
+                     : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7),
+                       "=&s"(t8)
+                     : "s"(base), REEF_KW(0), REEF_KW(1), REEF_KW(2), REEF_KW(3), REEF_KW(4), REEF_KW(5),
+                       REEF_KW(6), REEF_KW(7), "n"(BYTES - 4) : "memory");
+#undef REEF_KW
 }
 
 #if REEF_FLAVOUR == 2

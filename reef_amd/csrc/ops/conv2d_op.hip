@@ -118,6 +118,9 @@ int make_plan(const DeviceState& dv, const reef_conv2d_desc* c, const float* in,
     const long long K = (long long)c->cin * taps;
     if ((long long)M * N >= (1ll << 28) || K * M >= (1ll << 28) || (long long)c->cin * c->h * c->w >= (1ll << 28))
         return fail("reef_ops_conv2d: tensor of 1 GiB or more");
+    // the kernels decode pixel, tile and task numbers with a float reciprocal that is exact below 2^22
+    if (N >= (1 << 22) || (long long)c->h * c->w >= (1 << 22))
+        return fail("reef_ops_conv2d: image of 4 Mi pixels or more");
     int mode, tile, bm, bk, n_tiles;
     const bool rows = c->kh == 3 && c->kw == 3 && c->stride_h == 1 && c->stride_w == 1 && c->pad_h == 1 && c->pad_w == 1;
     if (rows) {
@@ -213,6 +216,13 @@ int reef_ops_conv2d(const reef_conv2d_desc* c, const float* in, const float* w, 
             return hip_fail(e, "hipMalloc(counters)");
         }
         hipLaunchKernelGGL(fill_words, dim3((p.tiles + 255) / 256), dim3(256), 0, s, (uint32_t*)cnt, 0u, (size_t)p.tiles);
+        e = hipGetLastError();
+        if (e != hipSuccess) {
+            // the convolution would count on whatever the fresh allocation holds
+            (void)hipFree(ws);
+            (void)hipFree(cnt);
+            return hip_fail(e, "fill_words(counters)");
+        }
         p.desc.ptr[p.ws_slot] = ws;
         p.desc.ptr[p.sync_slot] = cnt;
     }
@@ -247,6 +257,9 @@ int reef_ops_conv2d_noalloc(const reef_conv2d_desc* c, const float* in, const fl
         float* ws = (float*)(d->scratch_ptr + kCounterBytes);
         // the array keeps what the last call left: the counters of this launch start at zero
         hipLaunchKernelGGL(fill_words, dim3((p.tiles + 255) / 256), dim3(256), 0, s, cnt, 0u, (size_t)p.tiles);
+        // a fill that was not launched would leave the last call's counts in place: wrong sums, no error
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return hip_fail(e, "fill_words(counters)");
         p.desc.ptr[p.ws_slot] = ws;
         p.desc.ptr[p.sync_slot] = cnt;
     }

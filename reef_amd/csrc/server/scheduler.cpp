@@ -543,13 +543,16 @@ void REEFScheduler::execute_rt_task(std::shared_ptr<Task>& task) {
     }
     finish_task(task, Clock::now());
     REEF_LOG_INFO("rt task finish");
-    // off the real-time path: complete preemption samples that waited for a late launch, and
-    // renew the clock mapping when it is older than 100 ms (the two clocks drift)
-    if (clk_valid) {
+    // Off the real-time path, and only when this task preempted something whose device-side
+    // sample is still open: complete the samples, with a clock mapping that is renewed first
+    // when it is older than 100 ms (the two clocks drift by tens of microseconds per second).
+    // The exchange keeps this thread for some tens of microseconds, so a task that has no
+    // sample to convert does not pay for it.
+    if (clk_valid && !late_samples.empty()) {
         const int64_t now = std::chrono::duration_cast<std::chrono::nanoseconds>(
                                 std::chrono::steady_clock::now().time_since_epoch()).count();
         if (now - clk_synced_at_ns > 100000000) sync_clock();
-        if (!late_samples.empty()) resolve_late_samples();
+        resolve_late_samples();
     }
 }
 

@@ -24,6 +24,7 @@ Also here: REEFClient / ModelHandle, the Python mirror of src/reef/client/client
 the three command lines of src/example (`python -m reef_amd.rpc server|client|client_cont ...`).
 """
 import ctypes
+import hashlib
 import json
 import mmap
 import os
@@ -188,7 +189,18 @@ class REEFServer:
         with self.import_mtx:
             if self.import_root is None:
                 self.import_root = tempfile.mkdtemp(prefix="reef_imported_")
-            out = os.path.join(self.import_root, name)
+            # one import per source: the directory it lies in and the state of its graph and
+            # parameter files, so that another directory holding a model of the same name, or the
+            # same directory after its files changed, is imported again instead of served stale
+            ident = [os.path.realpath(model_dir)]
+            for ext in (".json", ".param"):
+                try:
+                    st = os.stat(os.path.join(model_dir, name + ext))
+                    ident.append("%s:%d:%d" % (ext, st.st_size, st.st_mtime_ns))
+                except OSError:
+                    ident.append(ext + ":absent")
+            tag = hashlib.sha256("|".join(ident).encode()).hexdigest()[:16]
+            out = os.path.join(self.import_root, tag, name)
             if not os.path.exists(os.path.join(out, name + ".json")):
                 try:
                     legacy.import_model_dir(model_dir, name, out, measured_profile=self.measure_imported)

@@ -136,7 +136,10 @@ def test_load_model_imports_a_directory_of_the_reference(served, tmp_path):
     client = rpc.REEFClient(addr)
     client.init(True)
     m = client.load_model(str(ref_dir), name)
-    assert server.import_root and os.path.exists(os.path.join(server.import_root, name, name + ".be.co"))
+    # imported once, into a directory keyed by where the source lies and the state of its files
+    import glob
+    first = glob.glob(os.path.join(server.import_root, "*", name, name + ".be.co"))
+    assert server.import_root and len(first) == 1
     inp = m.get_input_blob("data")
     inp.array()[:] = x.ravel()
     m.load_input()
@@ -152,4 +155,14 @@ def test_load_model_imports_a_directory_of_the_reference(served, tmp_path):
     shutil.copyfile(golden(name), other / "nonet.json")
     reply = client.calls["LoadModel"](rpc.MSG["LoadModelRequest"](dir=str(other), name="nonet", qid=client.qid))
     assert reply.succ is False
+    # the same directory again is served from the first import; a model of the same name in ANOTHER
+    # directory (other parameters) is imported on its own instead of being answered with the first
+    client.load_model(str(ref_dir), name)
+    assert len(glob.glob(os.path.join(server.import_root, "*", name, name + ".json"))) == 1
+    second = tmp_path / "elsewhere" / name
+    second.mkdir(parents=True)
+    shutil.copyfile(golden(name), second / (name + ".json"))
+    MB.write_params(str(second / (name + ".param")), [(k, np.asarray(v) * 0.5) for k, v in params])
+    client.load_model(str(second), name)
+    assert len(glob.glob(os.path.join(server.import_root, "*", name, name + ".json"))) == 2
     client.close()

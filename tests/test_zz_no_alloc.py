@@ -37,3 +37,25 @@ def test_no_alloc_needs_init_and_states_its_limit():
     L = B.lib()
     L.reef_ops_scratch_bytes.restype = __import__("ctypes").c_size_t
     assert L.reef_ops_scratch_bytes() == 4 << 20
+    # A call in a process where reef_ops_init has not run is refused before anything is launched
+    # (set-up -- loading the kernels, finding this GPU's copy of the array -- is never done by
+    # the entry point that must not allocate).  In a process of its own: this one has run init.
+    import subprocess
+    import sys
+    code = (
+        "import ctypes, sys\n"
+        "from reef_amd import binding as B\n"
+        "d = B.Conv2dDesc(256, 14, 14, 256, 3, 3, 1, 1, 1, 1, 1)\n"
+        "p = ctypes.c_void_p(4096)\n"      # never dereferenced: the refusal comes first
+        "st = B.lib().reef_ops_conv2d_noalloc(ctypes.byref(d), p, p, None, None, p, None)\n"
+        "print(st, B.last_error())\n"
+        "sys.exit(0 if st == 1 and 'reef_ops_init has not run' in B.last_error() else 3)\n")
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300,
+                       cwd=__import__("os").path.dirname(__import__("os").path.dirname(__import__("os").path.abspath(__file__))))
+    assert r.returncode == 0, (r.stdout, r.stderr)
+    # The size check of the entry point is a guard that no shape reaches today: its plan puts at most
+    # 256 workgroups on a split layer and a workgroup's tile has at most 64 x 64 outputs, so the
+    # partial tiles never exceed 256 x 4096 floats = the 4 MiB array, and a split layer has at most
+    # 128 tiles against 16384 counters.  The largest such layer goes through and matches:
+    B.ops_init()
+    both((2048, 7, 7, 2048, 1, 1, 0, 0, False, False))
