@@ -93,7 +93,8 @@ def test_rpc_load_model_takes_a_directory_of_the_reference(tmp_path):
         c = rpc.REEFClient("127.0.0.1:%d" % server.port)
         c.init(True)
         m = c.load_model(str(ref_dir), name)
-        imported = os.path.join(server.import_root, name)
+        import glob
+        (imported,) = glob.glob(os.path.join(server.import_root, "*", name))   # keyed by its source
         prof = json.load(open(os.path.join(imported, name + ".profile.json")))
         assert prof["model_latency"] > 0 and len(prof["kernel_latency"]) == 31
         orc = O.GraphOracle(json.load(open(os.path.join(imported, name + ".json"))), os.path.join(imported, name + ".param"))
