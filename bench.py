@@ -470,6 +470,12 @@ def compact_line(detail):
                         "preempt_device_us_p99": at(leg, "preempt_us", "device", "p99")}
         if reset is not None:
             other[label]["be_inferences_per_s_reset_mode"] = at(reset, "loaded", "be_inferences_per_s")
+    leg16 = detail.get("corun_16_be_queues")
+    if leg16 is not None:
+        other["headline_with_16_be_queues"] = {"rt_p50_ms": at(leg16, "loaded", "rt_ms", "p50"),
+                                               "rt_exec_p99_ms": at(leg16, "loaded", "rt_exec_ms", "p99"),
+                                               "be_inferences_per_s": at(leg16, "loaded", "be_inferences_per_s"),
+                                               "preempt_device_us_p99": at(leg16, "preempt_us", "device", "p99")}
     if other:
         line["other_configs"] = other
     for nm in ("mobilenetv2", "bert_base"):
@@ -491,9 +497,10 @@ def main():
     ap.add_argument("--steps", type=int, default=400, help="recorded real-time requests")
     ap.add_argument("--warmup", type=int, default=40, help="real-time requests before recording")
     ap.add_argument("--kernel-iters", type=int, default=20)
-    ap.add_argument("--configs", default="3,4,5,6,7",
+    ap.add_argument("--configs", default="3,4,5,6,7,8",
                     help="co-location scenarios to run (3 is the headline; 6 = dynamic kernel padding under "
-                         "a real-time request every 2 ms; 7 = the headline workload in every schedule mode)")
+                         "a real-time request every 2 ms; 7 = the headline workload in every schedule mode; "
+                         "8 = the headline workload with 16 best-effort queues)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--solo-only", action="store_true",
                     help="only the solo ResNet-152 executor part (whole-model and per-kernel timing); "
@@ -706,6 +713,11 @@ def main():
                                    dkp_slack=100, interval_us=2000.0),
             "reset": corun(models, "resnet152", "mobilenetv2", 1, B.MODE_RESET, k, 20, solo=False,
                            interval_us=2000.0)}
+    if 8 in configs and head is not None:
+        # the headline pair with 16 best-effort queues instead of 4: the launch windows of the 16
+        # streams share the pool of feeder threads (four host threads, not sixteen)
+        k = max(args.steps // 2, 50)
+        out["corun_16_be_queues"] = corun(models, "resnet152", "densenet201", 16, B.MODE_REEF, k, 20, solo=False)
     if not args.solo_only:
         # the bandwidth-bound families are where they matter: MobileNetV2 (depthwise) and BERT-base
         for extra in ("mobilenetv2", "bert_base"):

@@ -1,6 +1,7 @@
 // HIP backend of the C-ABI layer (stock ROCm, no patched runtime).
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 #include <chrono>
 #include <condition_variable>
@@ -71,17 +72,22 @@ struct HeldRing {
 // device writes after every kernel of a windowed stream; submitted - *done is
 // the number of kernels still on the device.
 //
-// A windowed stream has a feeder thread of its own that moves held launches to the
+// A windowed stream is served by a feeder thread that moves held launches to the
 // device as the window frees up.  The caller of reef_hal_launch (the scheduler
-// thread) then only copies the launch into the ring; the two runtime calls per
-// kernel (launch + completion write, 5-6 us together) are paid by the feeder, one
-// per stream, so several best-effort streams are fed in parallel instead of one
-// after the other from the scheduler's loop.  `mtx` guards the ring and `submitted`
-// and is only held for copies; `submit_mtx` is held around the runtime calls on the
-// HIP stream.  A launch counts as in flight from the moment the feeder takes it out
+// thread) then only copies the launch into the ring; the runtime call per kernel
+// (3 us of host time) is paid by the feeder, so several best-effort streams are fed in
+// parallel instead of one after the other from the scheduler's loop.  Feeders are a
+// small pool (Feeder below): the first streams get a thread each, further streams
+// share them, so the host cores this costs do not grow with the number of queues.
+// `mtx` guards the ring and `submitted` and is only held for copies; `submit_mtx` is
+// held around the runtime calls on the HIP stream.  A launch counts as in flight from the moment the feeder takes it out
 // of the ring, so "ring dropped + at most `window` kernels not known complete" -- what
 // the rollback after a preemption relies on -- holds at every instant.
 constexpr int kExitRing = 8;   // launches whose exit clock is kept
+
+namespace {
+struct Feeder;
+}
 
 struct reef_stream_s {
     hipStream_t s;
@@ -94,9 +100,7 @@ struct reef_stream_s {
     HeldRing held;
     std::mutex mtx;
     std::mutex submit_mtx;
-    std::condition_variable cv;
-    std::thread feeder;
-    std::atomic<bool> stop{false};
+    Feeder* feeder = nullptr;            // the pool thread that serves this stream
     std::atomic<int> feeder_error{0};
     std::atomic<size_t> held_count{0};   // mirror of held.size(), readable without mtx
     std::atomic<uint32_t> enqueued{0};   // highest seq whose runtime calls have returned
@@ -298,51 +302,138 @@ int pump_locked(reef_stream_t st) {
     return 0;
 }
 
-// The feeder looks at the ring size and the window through lock-free mirrors and only
-// takes the locks when there is a launch to move: a thread that re-takes a mutex in a
-// tight loop starves whoever else wants it (here the scheduler thread in the middle of
-// a preemption) for milliseconds.
-void feeder_main(reef_stream_s* st) {
+// One thread of the feeder pool and the windowed streams it serves.
+//
+// While a best-effort model runs, its stream's window is full most of the time and its kernels
+// take a few microseconds -- far below what a sleep costs -- so a feeder polls the completion
+// words of its streams: one busy host core per feeder while any of its streams has launches
+// held.  With a thread per stream that was one core per best-effort queue (32 at the
+// reference's queue limit).  The pool has kMaxFeeders threads (REEF_HAL_FEEDERS, default 4: the
+// number of hardware queues a process gets, i.e. of best-effort streams that can really run
+// side by side); stream k is served by feeder k mod n.  Streams that share a feeder also share
+// the device, so each needs its window refilled proportionally less often.
+//
+// A feeder looks at the ring sizes and the windows through lock-free mirrors and only takes a
+// stream's locks when there is a launch to move: a thread that re-takes a mutex in a tight loop
+// starves whoever else wants it (here the scheduler thread in the middle of a preemption) for
+// milliseconds.
+struct Feeder {
+    std::thread th;
+    std::mutex mtx;                        // guards `streams`; the condition variable's mutex
+    std::condition_variable cv;            // a launch was held on one of the streams, or the list changed
+    std::vector<reef_stream_s*> streams;
+    std::atomic<uint32_t> version{0};      // bumped whenever `streams` changes
+    std::atomic<uint32_t> seen{0};         // the version the thread is working with
+};
+constexpr int kMaxFeeders = 16;
+Feeder* g_feeders[kMaxFeeders] = {};
+int g_n_feeders = 0;                       // pool size, fixed when the first windowed stream is made
+unsigned g_next_feeder = 0;
+std::mutex g_feeders_mtx;
+
+// Moves one held launch of `st` to the device if its window has room.  Returns true when it did.
+bool feed_one(reef_stream_s* st, Held& h) {
+    // `submitted` only changes in the stream's feeder thread
+    if ((int)in_flight(st) >= st->window) return false;
+    std::lock_guard<std::mutex> sub(st->submit_mtx);
+    uint32_t seq = 0;
+    {
+        std::lock_guard<std::mutex> lock(st->mtx);
+        if (st->held.empty()) return false;   // dropped in the meantime
+        h = st->held.front();
+        st->held.pop_front();
+        st->held_count.store(st->held.size(), std::memory_order_release);
+        seq = ++st->submitted;   // in flight from now on
+    }
+    if (submit(st, h.fn, h.grid, h.block, h.lds, h.kernarg, h.bytes, seq) != 0) st->feeder_error.store(1);
+    return true;
+}
+
+void feeder_main(Feeder* f) {
     hipSetDevice(g_device);
+    std::vector<reef_stream_s*> mine;
+    uint32_t ver = ~0u;
     int idle_spins = 0, full_spins = 0;
     Held h;
-    while (!st->stop.load(std::memory_order_acquire)) {
-        if (st->held_count.load(std::memory_order_acquire) == 0) {
+    for (;;) {   // pool threads live as long as the process
+        const uint32_t v = f->version.load(std::memory_order_acquire);
+        if (v != ver) {
+            std::lock_guard<std::mutex> lock(f->mtx);
+            mine = f->streams;
+            ver = f->version.load(std::memory_order_acquire);
+            f->seen.store(ver, std::memory_order_release);   // a stream taken off the list is not touched again
+        }
+        bool any_held = false, fed = false;
+        for (reef_stream_s* st : mine) {
+            if (st->held_count.load(std::memory_order_acquire) == 0) continue;
+            any_held = true;
+            fed = feed_one(st, h) || fed;
+        }
+        if (fed) {
+            idle_spins = full_spins = 0;
+            continue;
+        }
+        if (!any_held) {
             // nothing to feed: after a while sleep until a launch is held (bounded, so that a
             // missed wake-up costs little)
+            full_spins = 0;
             if (++idle_spins > 2000) {
-                std::unique_lock<std::mutex> lock(st->mtx);
-                if (st->held.empty()) st->cv.wait_for(lock, std::chrono::microseconds(200));
+                std::unique_lock<std::mutex> lock(f->mtx);
+                if (f->version.load(std::memory_order_acquire) == ver)
+                    f->cv.wait_for(lock, std::chrono::microseconds(mine.empty() ? 20000 : 200));
                 idle_spins = 0;
             } else {
                 __builtin_ia32_pause();
             }
             continue;
         }
+        // every stream with held launches has a full window: the steady state while best-effort
+        // models run.  Behind kernels that run for long the core is given away.
         idle_spins = 0;
-        // `submitted` only changes in this thread while a feeder exists.  A full window is the
-        // steady state while a best-effort model runs: its kernels take a few microseconds, far
-        // below what a sleep costs, so the thread polls the completion word -- one host core per
-        // best-effort stream.  Behind a kernel that runs for long it gives the core away.
-        if ((int)in_flight(st) >= st->window) {
-            if (++full_spins > 20000) std::this_thread::yield();
-            else __builtin_ia32_pause();
-            continue;
-        }
-        full_spins = 0;
-        std::lock_guard<std::mutex> sub(st->submit_mtx);
-        uint32_t seq = 0;
-        {
-            std::lock_guard<std::mutex> lock(st->mtx);
-            if (st->held.empty()) continue;   // dropped in the meantime
-            h = st->held.front();
-            st->held.pop_front();
-            st->held_count.store(st->held.size(), std::memory_order_release);
-            seq = ++st->submitted;   // in flight from now on
-        }
-        if (submit(st, h.fn, h.grid, h.block, h.lds, h.kernarg, h.bytes, seq) != 0)
-            st->feeder_error.store(1);
+        if (++full_spins > 20000) std::this_thread::yield();
+        else __builtin_ia32_pause();
     }
+}
+
+// The feeder a new windowed stream is served by; starts the pool on first use.
+Feeder* attach_feeder(reef_stream_s* st) {
+    std::lock_guard<std::mutex> pool(g_feeders_mtx);
+    if (g_n_feeders == 0) {
+        int n = 4;
+        if (const char* v = std::getenv("REEF_HAL_FEEDERS")) n = std::atoi(v);
+        g_n_feeders = std::max(1, std::min(n, kMaxFeeders));
+    }
+    Feeder*& f = g_feeders[g_next_feeder++ % (unsigned)g_n_feeders];
+    if (!f) {
+        f = new Feeder;                    // never deleted: its thread runs until the process ends
+        f->th = std::thread(feeder_main, f);
+        f->th.detach();
+    }
+    {
+        std::lock_guard<std::mutex> lock(f->mtx);
+        f->streams.push_back(st);
+        f->version.fetch_add(1, std::memory_order_release);
+    }
+    f->cv.notify_all();
+    return f;
+}
+
+// Takes a stream off its feeder's list and waits until the thread has let go of it.
+void detach_feeder(reef_stream_s* st) {
+    Feeder* f = st->feeder;
+    uint32_t want;
+    {
+        std::lock_guard<std::mutex> lock(f->mtx);
+        for (size_t i = 0; i < f->streams.size(); ++i)
+            if (f->streams[i] == st) {
+                f->streams.erase(f->streams.begin() + (long)i);
+                break;
+            }
+        want = f->version.fetch_add(1, std::memory_order_release) + 1;
+    }
+    f->cv.notify_all();
+    while ((int32_t)(f->seen.load(std::memory_order_acquire) - want) < 0) std::this_thread::sleep_for(std::chrono::microseconds(50));
+    st->feeder = nullptr;
 }
 
 bool g_use_feeder = true;
@@ -371,7 +462,7 @@ int h_stream_create(int window, reef_stream_t* out) {
         if (const char* v = std::getenv("REEF_HAL_FEEDER")) g_use_feeder = std::atoi(v) != 0;
         if (g_use_feeder) {
             st->has_feeder = true;
-            st->feeder = std::thread(feeder_main, st);
+            st->feeder = attach_feeder(st);
         }
     }
     *out = st;
@@ -379,11 +470,7 @@ int h_stream_create(int window, reef_stream_t* out) {
 }
 int h_stream_destroy(reef_stream_t st) {
     if (!st) return 0;
-    if (st->has_feeder) {
-        st->stop.store(true, std::memory_order_release);
-        st->cv.notify_all();
-        st->feeder.join();
-    }
+    if (st->has_feeder) detach_feeder(st);
     hipStreamSynchronize(st->s);
     hipStreamDestroy(st->s);
     if (st->done) hipHostFree((void*)st->done);
@@ -456,7 +543,7 @@ int h_launch(reef_function_t f, const uint32_t* g, const uint32_t* b, uint32_t l
         std::memcpy(h.kernarg, kernarg, bytes);
         st->held_count.store(st->held.size(), std::memory_order_release);
         lock.unlock();
-        if (st->has_feeder && was_empty) st->cv.notify_one();
+        if (st->has_feeder && was_empty) st->feeder->cv.notify_one();
         return st->feeder_error.load() ? 1 : 0;
     }
     return submit(st, f->fn, g, b, lds, kernarg, bytes, 0);

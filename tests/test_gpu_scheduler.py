@@ -310,3 +310,40 @@ def test_pre_activation_and_folded_split_survive_preemption(tmp_path_factory):
         np.testing.assert_array_equal(s.get_output(m, 1000), refs["densenet_s"])
     np.testing.assert_array_equal(s.get_output(bert, n_out), bert_ref)
     s.shutdown()
+
+
+def test_more_best_effort_queues_than_feeder_threads(dirs):
+    """Ten best-effort clients (ResNet-18) under a real-time ResNet-18: the launch windows of the
+    ten streams are served by the pool of feeder threads (four unless REEF_HAL_FEEDERS says
+    otherwise), so two or three streams share a thread.  Every client makes progress, is
+    preempted and restarted, and ends with the bits of a solo run; a scheduler that is torn down
+    and built again in the same process finds the pool working (streams leave and join it)."""
+    x = nets.image_input("resnet18", (3, 224, 224))
+    ref = solo_output(dirs["resnet18"], "resnet18", x)
+    for round_ in range(2):
+        s = B.Scheduler(B.MODE_REEF)
+        s.set_wait_sync(True)
+        rt = s.load_model(dirs["resnet18"], "resnet18")
+        s.bind_model_queue(s.create_queue(B.QUEUE_RT), rt)
+        s.set_input(rt, x, "data")
+        bes = []
+        for _ in range(10 if round_ == 0 else 3):
+            m = s.load_model(dirs["resnet18"], "resnet18")
+            s.bind_model_queue(s.create_queue(B.QUEUE_BE), m)
+            s.set_input(m, x, "data")
+            bes.append(m)
+        s.run()
+        r = s.run_load(rt, bes, requests=40, warmup=5, mean_interval_us=3000.0, seed=5)
+        assert (r["be_completed"] > 0).all(), r["be_completed"]
+        assert r["be_preempted"].sum() > 0
+        ps = s.preempt_samples()
+        print("round %d: %d best-effort queues, BE done %s, preempt mean %.1f max %d us, rt p50 %.0f us"
+              % (round_, len(bes), r["be_completed"], ps.mean(), ps.max(), np.percentile(r["rt_latency_us"], 50)))
+        assert ps.mean() < 300
+        np.testing.assert_array_equal(s.get_output(rt, 1000), ref)
+        r2 = s.run_load(rt, bes, requests=0, be_only_ms=60)
+        assert (r2["be_completed"] > 0).all()
+        for m in bes:
+            np.testing.assert_array_equal(s.get_output(m, 1000), ref)
+        s.shutdown()
+        s.close()
