@@ -206,6 +206,13 @@ enum {
                                   empties the slot.  Best-effort launches, which may be cut short, and the
                                   best-effort side of a padded launch keep the counters. */
 
+#define REEF_F_DW_OUTPUT 128   /* symbols reef_conv2d_xdw_g<G> (G = 2, 4 image rows per tile): a 1x1 filter (stride 1, +
+                                  bias, activation ACT) followed by a depthwise 3x3 filter (stride 1, padding 1, + bias,
+                                  activation ACT2) in one launch; the 1x1 result never leaves the chip.  ptr: in, W,
+                                  out, bias, depthwise weights [Cout][9], depthwise bias [Cout].  Spatial tiles as in
+                                  the row form: G output rows x one 14-column segment; M_TILES = ceil(Cout / 16),
+                                  N_TILES = ceil(H / G) * ceil(W / 14), TILE = REEF_TILE_R9G2 / R9G4, no split */
+
 /* Loader families of the convolution; the entry symbol carries the family:
  *   reef_conv2d_<tile>      general: im2col gather, needs K % 4 == 0
  *   reef_conv2d_pw_<tile>   pointwise: 1x1, stride 1, no padding, N % 4 == 0, K % 4 == 0
@@ -221,6 +228,7 @@ enum {
 #define REEF_CONV_MODE_UNALIGNED 2
 #define REEF_CONV_MODE_DIRECT 3
 #define REEF_CONV_MODE_DIRECT_PRE 4   /* direct, 1 tap, with REEF_F_PRE_ACT (reef_conv2d_p1_<tile>) */
+#define REEF_CONV_MODE_XDW 6          /* 1x1 filter + depthwise 3x3 behind it (reef_conv2d_xdw_g<G>, REEF_F_DW_OUTPUT) */
 #define REEF_CONV_MODE_ROWS 5         /* direct, row form: 3x3 / stride 1 / padding 1 (reef_conv2d_r9_g<G>[m2]).
                                          The output tile is 16 (m2: 32) channels x G image rows x one 14-column
                                          segment; N_TILES = ceil(Ho / G) * ceil(Wo / 14), spatial tile index =

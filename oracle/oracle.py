@@ -308,6 +308,12 @@ class GraphOracle:
             out = conv2d(xin, wgt, bias,
                          None if res is None else res[:Cout * Ho * Wo].reshape(Cout, Ho, Wo),
                          scale, shift, (sh, sw), (ph, pw), 1, act, 6.0, acc64)
+            if flags & 128:
+                # a depthwise 3x3 stage (stride 1, padding 1, + bias, activation act2) behind the 1x1
+                # filter, in the same launch; its weights and bias follow the optional operands
+                pos = 3 + bool(flags & 1) + bool(flags & 2) + 2 * bool(flags & 4) + 2 * bool(flags & 8)
+                out = conv2d(out, P[pos][:Cout * 9].reshape(Cout, 1, 3, 3), P[pos + 1][:Cout], stride=(1, 1),
+                             pad=(1, 1), groups=Cout, act=act2, acc64=acc64)
             P[2][dst_off:dst_off + out.size] = out.reshape(-1)
             if out2 is not None:
                 out2[dst_off:dst_off + out.size] = eltwise(out.reshape(Cout, -1), shift=shift2[:Cout],

@@ -104,6 +104,15 @@ void conv2d(const std::string& symbol, const Attrs& a, Needs& n) {
     } else if (fam.compare(0, 2, "u_") == 0) {
         mode = REEF_CONV_MODE_UNALIGNED;
         fits = true;
+    } else if (fam.compare(0, 5, "xdw_g") == 0) {
+        // a 1x1 filter and the depthwise 3x3 filter behind it (stride 1, padding 1) in one launch
+        mode = REEF_CONV_MODE_XDW;
+        const i64 G = a[REEF_CONV_TILE] == REEF_TILE_R9G2 ? 2 : a[REEF_CONV_TILE] == REEF_TILE_R9G4 ? 4 : 0;
+        fits = unit && a[REEF_CONV_SH] == 1 && a[REEF_CONV_SW] == 1 && cin % 8 == 0 && G > 0 &&
+               fam == std::string("xdw_g") + (char)('0' + G) && split == 1 &&
+               flags == (REEF_F_BIAS | REEF_F_DW_OUTPUT) && off == 0 && a[REEF_CONV_M_TILES] == cdiv(M, 16) &&
+               a[REEF_CONV_N_TILES] == cdiv(Ho, G) * cdiv(Wo, 14) && a[REEF_CONV_ACT] <= REEF_ACT_RELU6 &&
+               a[REEF_CONV_ACT2] <= REEF_ACT_RELU6;
     } else if (fam.compare(0, 3, "p1_") == 0) {
         mode = REEF_CONV_MODE_DIRECT_PRE;
         fits = unit && cin % 8 == 0 && (flags & REEF_F_PRE_ACT);
@@ -118,7 +127,8 @@ void conv2d(const std::string& symbol, const Attrs& a, Needs& n) {
         packed = head.back() == 'k';
         fits = compiled == taps && (taps > 1 || cin % 8 == 0);
     }
-    if (!fits || mode != a[REEF_CONV_MODE] || ((flags & REEF_F_PRE_ACT) != 0) != (mode == REEF_CONV_MODE_DIRECT_PRE)) {
+    if (!fits || mode != a[REEF_CONV_MODE] || ((flags & REEF_F_PRE_ACT) != 0) != (mode == REEF_CONV_MODE_DIRECT_PRE) ||
+        ((flags & REEF_F_DW_OUTPUT) != 0) != (mode == REEF_CONV_MODE_XDW)) {
         n.bad = "the layer is not one that this symbol's loader family was compiled for";
         return;
     }
@@ -136,6 +146,7 @@ void conv2d(const std::string& symbol, const Attrs& a, Needs& n) {
     if (flags & REEF_F_AFFINE) { n.f32("scale", M); n.f32("shift", M); }
     if (flags & REEF_F_DUAL) { n.f32("second output", off + M * N); n.f32("second shift", M); }
     if (flags & REEF_F_PRE_ACT) { n.f32("input scale", cin); n.f32("input shift", cin); }
+    if (flags & REEF_F_DW_OUTPUT) { n.f32("depthwise weights", M * 9); n.f32("depthwise bias", M); }
     if (fused) {
         n.f32("partial sums", (split + ((flags & REEF_F_PAIR_FOLD) ? 1 : 0)) * M * N);
         n.raw("tile counters", 4 * (a[REEF_CONV_SYNC_OFF] + a[REEF_CONV_M_TILES] * a[REEF_CONV_N_TILES]));

@@ -24,7 +24,7 @@ from . import rng, tiling
 from ..paths import code_object
 
 ACT_NONE, ACT_RELU, ACT_RELU6, ACT_GELU = 0, 1, 2, 3
-F_BIAS, F_RESIDUAL, F_AFFINE, F_DUAL, F_FUSED_REDUCE, F_PRE_ACT, F_PAIR_FOLD = 1, 2, 4, 8, 16, 32, 64
+F_BIAS, F_RESIDUAL, F_AFFINE, F_DUAL, F_FUSED_REDUCE, F_PRE_ACT, F_PAIR_FOLD, F_DW_OUTPUT = 1, 2, 4, 8, 16, 32, 64, 128
 WG = 256
 
 
@@ -281,6 +281,35 @@ class GraphBuilder:
                        4 * ((t["split_k"] + 1) * M * N), 2.0)
         return out if out2 is None else (out, out2)
 
+    XDW_TILES = {"g2": 2, "g4": 4}     # reef_conv2d_xdw_<tile>: image rows per tile
+
+    def conv2d_dw(self, x, cout, act=ACT_RELU6, dw_act=ACT_RELU6, tile=None):
+        """1x1 convolution (+ bias, act) followed by a depthwise 3x3 convolution (stride 1, padding
+        1, + bias, dw_act) as ONE launch (reef_conv2d_xdw_<tile>): the front half of a MobileNetV2
+        block without the expanded tensor in memory.  Parameters are created in the order the two
+        separate layers would create them."""
+        cin, H, W = x.shape
+        assert cin % 8 == 0
+        w = self.param((cout, cin, 1, 1), self.weight_std if self.weight_std is not None else math.sqrt(2.0 / cin))
+        b = self.param((cout,), 0.01)
+        wd = self.param((cout, 1, 3, 3), self.weight_std if self.weight_std is not None else math.sqrt(2.0 / 9))
+        bd = self.param((cout,), 0.01)
+        out = self.temp((cout, H, W))
+        if tile is None:
+            # two image rows per tile; four on large images, where four still leave every CU several
+            # workgroups and the rows computed twice by neighbouring tiles weigh more (measured on
+            # the shapes of MobileNetV2: 56 x 56 10.7 against 11.9 us, 28 x 28 and below two rows)
+            tile = "g4" if H * W >= 3136 else "g2"
+        G = self.XDW_TILES[tile]
+        mt, nt = math.ceil(cout / 16), math.ceil(H / G) * math.ceil(W / tiling.ROW_SEG)
+        flops = 2 * cout * H * W * (cin + 9)
+        self.flops += flops
+        attrs = [cin, H, W, cout, H, W, 1, 1, 1, 1, 0, 0, F_BIAS | F_DW_OUTPUT, act, tiling.TILES[tile][0], 1,
+                 math.ceil(cin / 128) * 128, mt, nt, dw_act, 0, 6, 0, 0]
+        self._emit("reef_conv2d_xdw_" + tile, mt * nt, [x, w.idx, out.idx, b.idx, wd.idx, bd.idx], attrs, "conv2d",
+                   flops, 4 * (x.size + cout * cin + 11 * cout + out.size), 6.0)
+        return out
+
     def dwconv2d(self, x, k, stride=1, pad=0, bias=True, act=ACT_RELU6, out=None, given=None):
         """given: {"w", "bias"} -> existing storages instead of new parameters; out: existing
         storage for the result (an imported graph brings its own)."""
@@ -504,7 +533,10 @@ class GraphBuilder:
         for k in self.kernels:
             n = k["name"]
             sym = n.split("#")[0]
-            if sym.startswith("reef_conv2d_") or sym.startswith("reef_gemm_"):
+            if sym.startswith("reef_conv2d_xdw_"):
+                R = self.XDW_TILES[sym.split("_")[-1]] + 2
+                shared[n] = (4 * R * 320 + 16 * (R + 1) * 16) * 4 + 16
+            elif sym.startswith("reef_conv2d_") or sym.startswith("reef_gemm_"):
                 shared[n] = tiling.lds_bytes(sym.split("_")[-1])
             else:
                 shared[n] = 4   # the reference's floor (generate_final_schedule.py:117-143)

@@ -117,11 +117,14 @@ def mocked_kernel(name="mocked_kernel"):
     return g
 
 
-def mobilenet_v2(image=(3, 224, 224), classes=1000, name="mobilenetv2", seed=rng.BASE_SEED):
+def mobilenet_v2(image=(3, 224, 224), classes=1000, name="mobilenetv2", seed=rng.BASE_SEED, fuse_expand_dw=True):
     """MobileNetV2, width 1.0: 3x3/2 stem, 17 inverted-residual blocks (1x1 expand + ReLU6,
     depthwise 3x3 + ReLU6, linear 1x1 projection, residual add when stride 1 and equal
     channels), 1x1 to 1280, global average pool, classifier.  Batch norms are folded
-    into the convolutions as biases; the residual add is the projection's epilogue."""
+    into the convolutions as biases; the residual add is the projection's epilogue.
+    fuse_expand_dw: where the depthwise convolution has stride 1, the 1x1 expansion in front of it
+    and the depthwise convolution are one launch and the expanded tensor is never written
+    (GraphBuilder.conv2d_dw); False keeps the two launches."""
     g = GraphBuilder(name, seed)
     x = g.input("data", image)
     x = g.conv2d(x, 32, 3, 2, 1, bias=True, act=ACT_RELU6)
@@ -132,9 +135,12 @@ def mobilenet_v2(image=(3, 224, 224), classes=1000, name="mobilenetv2", seed=rng
         for i in range(n):
             stride = s if i == 0 else 1
             y = x
-            if t != 1:
-                y = g.conv2d(y, cin * t, 1, 1, 0, bias=True, act=ACT_RELU6)
-            y = g.dwconv2d(y, 3, stride, 1, bias=True, act=ACT_RELU6)
+            if t != 1 and stride == 1 and fuse_expand_dw and cin % 8 == 0:
+                y = g.conv2d_dw(y, cin * t, act=ACT_RELU6, dw_act=ACT_RELU6)
+            else:
+                if t != 1:
+                    y = g.conv2d(y, cin * t, 1, 1, 0, bias=True, act=ACT_RELU6)
+                y = g.dwconv2d(y, 3, stride, 1, bias=True, act=ACT_RELU6)
             res = x if (stride == 1 and cin == c) else None
             x = g.conv2d(y, c, 1, 1, 0, bias=True, act=ACT_NONE, residual=res)
             cin = c

@@ -478,3 +478,31 @@ def test_kernels_that_do_not_fit_are_refused(tmp_path):
             B.Executor(B.BASE).load(str(broken(shrink)), str(tmp_path / "b.raw.co"))
     finally:
         fake.remove()
+
+
+def test_a_pointwise_plus_depthwise_kernel_is_checked_against_its_storages(tmp_path):
+    """reef_conv2d_xdw_<tile>: operand list, sizes and tile counts follow from the attributes; a graph
+    file that disagrees is refused with the reason."""
+    from reef_amd import binding as B
+    g = MB.GraphBuilder("xdwfmt")
+    x = g.input("data", (24, 20, 30))
+    g.mark_output(g.conv2d_dw(x, 48))
+    base = g.write(str(tmp_path / "ok"), link_code_objects=False)
+    assert B.check_model(base + ".json") == (True, "")
+    model = json.load(open(base + ".json"))
+    k = model["kernels"][0]
+    assert k["name"].startswith("reef_conv2d_xdw_g2") and len(k["args"]) == 6
+
+    def broken(change, reason):
+        m = json.loads(json.dumps(model))
+        change(m)
+        p = str(tmp_path / "broken.json")
+        json.dump(m, open(p, "w"))
+        ok, why = B.check_model(p)
+        assert not ok and reason in why, why
+
+    broken(lambda m: m["kernels"][0]["args"].pop(), "operands")                         # no depthwise bias
+    broken(lambda m: m["kernels"][0]["attrs"].__setitem__(18, 7), "loader family")      # wrong tile count
+    broken(lambda m: m["kernels"][0]["attrs"].__setitem__(12, 1), "loader family")      # flag missing
+    broken(lambda m: m["storage"][m["kernels"][0]["args"][4]].__setitem__("size", 48 * 8), "depthwise weights")
+    broken(lambda m: m["kernels"][0]["launch_params"].__setitem__(0, 5), "workgroups")

@@ -458,3 +458,63 @@ def test_mocked_model_closed_form(tmp_path):
     assert out.shape == (8192,)
     np.testing.assert_array_equal(out, np.full(8192, 18.0, np.float32))
     np.testing.assert_array_equal(orc.get("output"), out)
+
+
+XDW_CASES = [
+    # cin, H, W, cout: 1x1 (+bias, ReLU6), then depthwise 3x3 / stride 1 / padding 1 (+bias, ReLU6)
+    (24, 56, 56, 144),        # MobileNetV2, four segments per row
+    (64, 14, 14, 384),
+    (160, 7, 7, 960),         # two K steps, half a segment wide
+    (16, 9, 30, 40),          # ragged everywhere: three segments (the last two columns wide), odd rows,
+                              # output channels not a multiple of 16
+    (8, 1, 1, 16),            # one pixel: every neighbour is padding
+    (392, 5, 17, 32),         # four K steps
+]
+
+
+@pytest.mark.parametrize("tile", ["g2", "g4"])
+@pytest.mark.parametrize("case", XDW_CASES)
+def test_pointwise_then_depthwise_in_one_launch(tmp_path, tile, case):
+    """reef_conv2d_xdw_<tile> against the oracle's two layers, in all three flavours: the raw and the
+    padding flavour on one executor each, the preemptible flavour on the hybrid one; same bits in
+    all of them (a task's arithmetic does not depend on the flavour)."""
+    import ctypes
+    import json
+    from reef_amd import binding as B
+    from tests.helpers import write_model
+    cin, H, W, cout = case
+    g = MB.GraphBuilder("x")
+    x = g.input("data", (cin, H, W))
+    y = g.conv2d_dw(x, cout, act=MB.ACT_RELU6, dw_act=MB.ACT_RELU6, tile=tile)
+    z = g.conv2d_dw(y, 24, act=MB.ACT_NONE, dw_act=MB.ACT_RELU, tile=tile) if cout % 8 == 0 else y
+    g.mark_output(z)
+    data = rnd(cin, H, W)
+    exe, orc, model = run_both(g, tmp_path, {"data": data})
+    worst = compare_storages(exe, orc, model, what="xdw %s %s" % (tile, case))
+    want = exe.get_output()
+    d = write_model(g, tmp_path)
+    for kind, pre in ((B.TRANS, False), (B.HYBRID, True), (B.HYBRID, False)):
+        e = B.Executor.from_dir(d, g.name, kind)
+        e.set_input_checked("data", data)
+        e.execute_preemptable() if pre else e.execute()
+        np.testing.assert_array_equal(e.get_output(), want, err_msg="flavour %s %s" % (kind, pre))
+        e.close()
+    print("xdw %s %s: worst rel err %.2e" % (tile, case, worst[0]))
+
+
+def test_mobilenetv2_with_and_without_the_fused_front_half(tmp_path):
+    """The network with expansion + depthwise in one launch holds, in every tensor both variants
+    have (block outputs, logits), what the variant with two launches holds, to 1e-4: the fused
+    kernel sums the 1x1 filter in another order than the tiles the separate layer uses."""
+    from reef_amd.modelgen import nets
+    x = nets.image_input("mobilenetv2", (3, 224, 224))
+    outs = []
+    for fuse in (False, True):
+        g = nets.mobilenet_v2(fuse_expand_dw=fuse)
+        exe, orc, model = run_both(g, tmp_path / str(fuse), {"data": x})
+        compare_storages(exe, orc, model, what="mobilenetv2 fuse=%s" % fuse)
+        li = model["kernels"][-1]["args"][0]
+        outs.append((len(g.kernels), exe.get_data(li, model["storage"][li]["size"])))
+    assert outs[0][0] == 55 and outs[1][0] == 43
+    from tests.helpers import max_rel_err, REL_TOL
+    assert max_rel_err(outs[1][1], outs[0][1]) <= REL_TOL
