@@ -206,12 +206,14 @@ enum {
                                   empties the slot.  Best-effort launches, which may be cut short, and the
                                   best-effort side of a padded launch keep the counters. */
 
-#define REEF_F_DW_OUTPUT 128   /* symbols reef_conv2d_xdw_g<G> (G = 2, 4 image rows per tile): a 1x1 filter (stride 1, +
-                                  bias, activation ACT) followed by a depthwise 3x3 filter (stride 1, padding 1, + bias,
-                                  activation ACT2) in one launch; the 1x1 result never leaves the chip.  ptr: in, W,
-                                  out, bias, depthwise weights [Cout][9], depthwise bias [Cout].  Spatial tiles as in
-                                  the row form: G output rows x one 14-column segment; M_TILES = ceil(Cout / 16),
-                                  N_TILES = ceil(H / G) * ceil(W / 14), TILE = REEF_TILE_R9G2 / R9G4, no split */
+#define REEF_F_DW_OUTPUT 128   /* symbols reef_conv2d_xdw_g<G> (G = 2, 4 image rows per tile) and reef_conv2d_xdw2_g2: a 1x1
+                                  filter (+ bias, activation ACT) followed by a depthwise 3x3 filter (padding 1, stride
+                                  1 resp. 2, + bias, activation ACT2) in one launch; the 1x1 result never leaves the
+                                  chip.  ptr: in, W, out, bias, depthwise weights [Cout][9], depthwise bias [Cout].
+                                  H, W: the input; HO, WO: the output; SH = SW = the depthwise stride (the 1x1 filter
+                                  itself has stride 1).  Spatial tiles as in the row form: G output rows x one
+                                  14-column segment; M_TILES = ceil(Cout / 16), N_TILES = ceil(HO / G) * ceil(WO / 14),
+                                  TILE = REEF_TILE_R9G2 / R9G4, no split */
 
 /* Loader families of the convolution; the entry symbol carries the family:
  *   reef_conv2d_<tile>      general: im2col gather, needs K % 4 == 0

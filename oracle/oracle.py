@@ -305,15 +305,19 @@ class GraphOracle:
                 return
             # single pass, or split-K folded inside the kernel (workspace untouched here)
             bias, res, scale, shift, out2, shift2 = self._conv_opt(P, 3, flags)
-            out = conv2d(xin, wgt, bias,
-                         None if res is None else res[:Cout * Ho * Wo].reshape(Cout, Ho, Wo),
-                         scale, shift, (sh, sw), (ph, pw), 1, act, 6.0, acc64)
             if flags & 128:
-                # a depthwise 3x3 stage (stride 1, padding 1, + bias, activation act2) behind the 1x1
-                # filter, in the same launch; its weights and bias follow the optional operands
+                # a depthwise 3x3 stage (padding 1, + bias, activation act2) behind the 1x1 filter, in
+                # the same launch; its weights and bias follow the optional operands.  The stride
+                # attributes are the depthwise stage's; the 1x1 filter itself has stride 1.
                 pos = 3 + bool(flags & 1) + bool(flags & 2) + 2 * bool(flags & 4) + 2 * bool(flags & 8)
-                out = conv2d(out, P[pos][:Cout * 9].reshape(Cout, 1, 3, 3), P[pos + 1][:Cout], stride=(1, 1),
+                mid = conv2d(xin, wgt, bias, None, None, None, (1, 1), (ph, pw), 1, act, 6.0, acc64)
+                out = conv2d(mid, P[pos][:Cout * 9].reshape(Cout, 1, 3, 3), P[pos + 1][:Cout], stride=(sh, sw),
                              pad=(1, 1), groups=Cout, act=act2, acc64=acc64)
+                assert out.shape == (Cout, Ho, Wo)
+            else:
+                out = conv2d(xin, wgt, bias,
+                             None if res is None else res[:Cout * Ho * Wo].reshape(Cout, Ho, Wo),
+                             scale, shift, (sh, sw), (ph, pw), 1, act, 6.0, acc64)
             P[2][dst_off:dst_off + out.size] = out.reshape(-1)
             if out2 is not None:
                 out2[dst_off:dst_off + out.size] = eltwise(out.reshape(Cout, -1), shift=shift2[:Cout],

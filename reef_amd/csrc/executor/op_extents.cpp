@@ -104,12 +104,15 @@ void conv2d(const std::string& symbol, const Attrs& a, Needs& n) {
     } else if (fam.compare(0, 2, "u_") == 0) {
         mode = REEF_CONV_MODE_UNALIGNED;
         fits = true;
-    } else if (fam.compare(0, 5, "xdw_g") == 0) {
-        // a 1x1 filter and the depthwise 3x3 filter behind it (stride 1, padding 1) in one launch
+    } else if (fam.compare(0, 3, "xdw") == 0) {
+        // a 1x1 filter and the depthwise 3x3 filter behind it (padding 1, stride 1: xdw_g<G>, stride 2:
+        // xdw2_g2) in one launch; SH = SW carry the depthwise stride
         mode = REEF_CONV_MODE_XDW;
         const i64 G = a[REEF_CONV_TILE] == REEF_TILE_R9G2 ? 2 : a[REEF_CONV_TILE] == REEF_TILE_R9G4 ? 4 : 0;
-        fits = unit && a[REEF_CONV_SH] == 1 && a[REEF_CONV_SW] == 1 && cin % 8 == 0 && G > 0 &&
-               fam == std::string("xdw_g") + (char)('0' + G) && split == 1 &&
+        const i64 ds = a[REEF_CONV_SH];
+        const std::string want = ds == 1 ? std::string("xdw_g") + (char)('0' + G) : std::string("xdw2_g2");
+        fits = kh == 1 && kw == 1 && a[REEF_CONV_PH] == 0 && a[REEF_CONV_PW] == 0 && a[REEF_CONV_SW] == ds &&
+               (ds == 1 || (ds == 2 && G == 2)) && cin % 8 == 0 && G > 0 && fam == want && split == 1 &&
                flags == (REEF_F_BIAS | REEF_F_DW_OUTPUT) && off == 0 && a[REEF_CONV_M_TILES] == cdiv(M, 16) &&
                a[REEF_CONV_N_TILES] == cdiv(Ho, G) * cdiv(Wo, 14) && a[REEF_CONV_ACT] <= REEF_ACT_RELU6 &&
                a[REEF_CONV_ACT2] <= REEF_ACT_RELU6;

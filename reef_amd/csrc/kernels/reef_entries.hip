@@ -53,13 +53,13 @@ using OpConvRowsK = OpConvDirect<9, G, TM, false, true, true>;
 // row form of the 3x3 convolution: G image rows x one 14-column segment per workgroup
 template <int G, int TM = 1>
 using OpConvRows = OpConvDirect<9, G, TM, false, true>;
-// 1x1 convolution and the depthwise 3x3 convolution behind it in one launch
-template <int G>
+// 1x1 convolution and the depthwise 3x3 convolution (stride S) behind it in one launch
+template <int G, int S = 1>
 struct OpConvXdw {
-    static constexpr int LDS = TileXdw<G>::LDS_BYTES;
+    static constexpr int LDS = TileXdw<G, S>::LDS_BYTES;
     template <class P>
     static __device__ __forceinline__ bool run(const ReefOpDesc& d, int task, char* smem, const P& p) {
-        return conv2d_xdw_body<G>(d, task, smem, p);
+        return conv2d_xdw_body<G, S>(d, task, smem, p);
     }
 };
 template <class T, bool TRANS_B>
@@ -346,6 +346,7 @@ REEF_ENTRY(reef_conv2d_d7k_16x16k4, OpConvDirectK<7>)
 REEF_ENTRY(reef_conv2d_d7k_16x32k4, OpConvDirectK<7 REEF_COMMA 2>)
 REEF_ENTRY(reef_conv2d_xdw_g2, OpConvXdw<2>)
 REEF_ENTRY(reef_conv2d_xdw_g4, OpConvXdw<4>)
+REEF_ENTRY(reef_conv2d_xdw2_g2, OpConvXdw<2 REEF_COMMA 2>)
 REEF_ENTRY(reef_gemm_nt_128x128, OpGemm<Tile128x128 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nt_64x64, OpGemm<Tile64x64 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nt_32x128, OpGemm<Tile32x128 REEF_COMMA true>)

@@ -1234,53 +1234,62 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     return true;
 }
 
-// ---- reef_conv2d_xdw_g<G>: 1x1 convolution, then depthwise 3x3, in one launch ------------------
+// ---- reef_conv2d_xdw[2]_g<G>: 1x1 convolution, then depthwise 3x3, in one launch --------------
 // The front half of a MobileNetV2 block: expand (1x1 filter, + bias, activation) and the depthwise
-// 3x3 filter (stride 1, padding 1, + bias, activation) that follows it.  As two launches the
-// expanded tensor -- six times the block's input, the largest tensor of the network -- is written
-// and read back; here it never leaves the chip.  The depthwise stage is channel-local, so a
-// workgroup owns 16 channels x G image rows x one 14-column segment of the OUTPUT and needs the
-// 1x1 result of the same 16 channels on G + 2 rows x 16 columns (one row above and below, one
-// column left and right): it forms that itself.  The input has few channels (K = 16..160 for 96
-// ..960 expanded channels), so what is computed twice by neighbouring tiles is (G + 2) / G x
-// 16 / 14 of a small product, and no workgroup waits for another.
-//   phase 1  the 1x1 result on the matrix cores, direct form: pixel group r is image row
-//            y0 - 1 + r, lanes 0..13 of a k slot are the segment's columns, lane 14 the column
-//            right of it, lane 15 the column left of it; the four wavefronts split the input
-//            channels; partial tiles meet in LDS; + bias, activation; positions outside the
-//            image become 0 (the depthwise stage's padding) -> E[16][G + 2][16] in LDS
+// 3x3 filter (padding 1, stride S = 1 or 2, + bias, activation) that follows it.  As two launches
+// the expanded tensor -- six times the block's input, the largest tensor of the network -- is
+// written and read back; here it never leaves the chip.  The depthwise stage is channel-local, so
+// a workgroup owns 16 channels x G image rows x one 14-column segment of the OUTPUT and needs the
+// 1x1 result of the same 16 channels on the rows and columns its taps touch: it forms that
+// itself.  The input has few channels (K = 16..160 for 96..960 expanded channels), so what
+// neighbouring tiles compute twice is a fraction of a small product, and no workgroup waits for
+// another.
+//   phase 1  the 1x1 result on the matrix cores, direct form; the four wavefronts split the input
+//            channels, partial tiles meet in LDS; + bias, activation; positions outside the image
+//            become 0 (the depthwise stage's padding) -> E in LDS.
+//            S = 1: pixel group r is image row y0 - 1 + r (G + 2 of them); lanes 0..13 of a k slot
+//            are the segment's columns, lane 14 the column right of it, lane 15 the column left.
+//            S = 2: input rows 2 y0 - 1 + r (2 G + 1 of them), each as two groups: the even
+//            columns 2 x (lanes 0..13 = the segment's x) and the odd columns 2 x + 1 (lane 15:
+//            column 2 x0 - 1, left of the segment).
 //   phase 2  thread t = (channel t / 16, column t % 16) forms its G outputs from E: taps in filter
-//            order, then the bias, then the activation, as the depthwise kernel does
-// ptr: in [Cin][H][W], W [Cout][Cin], out [Cout][H][W], bias [Cout], depthwise weights [Cout][9],
-// depthwise bias [Cout].  attr: the 1x1 layer's (ACT its activation, ACT2 the depthwise stage's),
-// flags REEF_F_BIAS | REEF_F_DW_OUTPUT, M_TILES = ceil(Cout / 16), N_TILES = ceil(H / G) *
-// ceil(W / 14), no split.  tasks = M_TILES * N_TILES.
-template <int G>
+//            order, then the bias, then the activation, as the depthwise kernel does.  The left
+//            neighbour of column c is lane (c - 1) mod 16, the right one lane c + 1 (S = 1) or the
+//            odd group's lane c (S = 2).
+// ptr: in [Cin][H][W], W [Cout][Cin], out [Cout][Ho][Wo], bias [Cout], depthwise weights [Cout][9],
+// depthwise bias [Cout].  attr: H, W the input (and the 1x1 result), HO, WO the output, SH = SW =
+// S (the 1x1 filter itself has stride 1), ACT the 1x1 layer's activation, ACT2 the depthwise
+// stage's, flags REEF_F_BIAS | REEF_F_DW_OUTPUT, M_TILES = ceil(Cout / 16), N_TILES = ceil(Ho / G)
+// * ceil(Wo / 14), no split.  tasks = M_TILES * N_TILES.
+template <int G, int S = 1>
 struct TileXdw {
-    static constexpr int R = G + 2;                    // rows of the 1x1 result a tile needs
-    static constexpr int PART = 320;                   // floats per 16 x 16 partial tile (skewed rows)
-    static constexpr int ESTRIDE = (R + 1) * 16;       // floats per channel of E (one spare row: no bank conflicts)
-    static constexpr int LDS_BYTES = (4 * R * PART + 16 * ESTRIDE) * 4 + 16;
+    static constexpr int R = S == 1 ? G + 2 : 2 * G + 1;    // rows of the 1x1 result a tile needs
+    static constexpr int NG = R * S;                         // pixel groups of 16 lanes: S per row
+    static constexpr int PART = 320;                         // floats per 16 x 16 partial tile (skewed rows)
+    static constexpr int ESTRIDE = (NG + 1) * 16;            // floats per channel of E (+ one group: no bank conflicts)
+    static constexpr int LDS_BYTES = (4 * NG * PART + 16 * ESTRIDE) * 4 + 16;
 };
 
-template <int G, class Poll>
+template <int G, int S, class Poll>
 __device__ __forceinline__ bool conv2d_xdw_body(const ReefOpDesc& d, int task, char* smem_raw, const Poll&) {
-    typedef TileXdw<G> T;
-    constexpr int R = T::R;
+    typedef TileXdw<G, S> T;
+    constexpr int R = T::R, NG = T::NG;
+    constexpr int NSTAGE = S == 1 ? 2 : 1;      // K steps whose loads are in flight
     float* smem = (float*)smem_raw;
-    float* E = smem + 4 * R * T::PART;
+    float* E = smem + 4 * NG * T::PART;
     const int* a = d.attr;
     const int lane = threadIdx.x & 63, i16 = lane & 15, kq = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int C = a[REEF_CONV_CIN], H = a[REEF_CONV_H], W = a[REEF_CONV_W], M = a[REEF_CONV_COUT];
+    const int Ho = a[REEF_CONV_HO], Wo = a[REEF_CONV_WO];
     const int m_tiles = a[REEF_CONV_M_TILES], n_tiles = a[REEF_CONV_N_TILES];
     // the tiles of one pixel tile (all channel tiles) are neighbours in the order: they read the
     // same input, and a contiguous piece of the order runs on one XCD
     task = xcd_chunked(task, m_tiles * n_tiles);
     const int nt = div_small(task, m_tiles), mt = task - nt * m_tiles;
-    const int segs = (W + kRowSeg - 1) / kRowSeg;
+    const int segs = (Wo + kRowSeg - 1) / kRowSeg;
     const int q_seg = div_small(nt, segs);
-    const int y0 = q_seg * G, x0 = (nt - q_seg * segs) * kRowSeg;
+    const int y0 = q_seg * G, x0 = (nt - q_seg * segs) * kRowSeg;     // first output row and column
     const int m0 = mt * 16;
     const unsigned HW4 = (unsigned)(H * W) * 4u;
 
@@ -1293,21 +1302,31 @@ __device__ __forceinline__ bool conv2d_xdw_body(const ReefOpDesc& d, int task, c
     const rsrc_t rs_dw = make_rsrc(d.ptr[4], (unsigned)M * 36u);
     const rsrc_t rs_db = make_rsrc(d.ptr[5], (unsigned)M * 4u);
 
+    // Image column that lane / column c of pixel group (r, p) stands for.  S = 1: the segment's
+    // columns, lane 14 right of it, lane 15 left of it.  S = 2, p = 0: even columns 2 x; p = 1:
+    // odd columns 2 x + 1, lane 15 the odd column left of the segment; lanes nobody reads: none.
+    auto image_col = [&](int c, int p) -> int {
+        if (S == 1) return c == 15 ? x0 - 1 : x0 + c;
+        if (p == 0) return c < kRowSeg ? 2 * (x0 + c) : -1;
+        return c == 15 ? 2 * x0 - 1 : c < kRowSeg ? 2 * (x0 + c) + 1 : -1;
+    };
+
     // phase-1 operands: weights W[m0 + i16][8 channels of the k slot], input values of the lane's
-    // column on the R rows; both steps' loads go out at once
+    // column in every pixel group
     const int lane_c = (wave * 4 + kq) * 8;
     const int nsteps = (C + 127) / 128;
     const int lane_steps = lane_c < C ? (C - lane_c + 127) / 128 : 0;
     const unsigned va = ((unsigned)(m0 + i16) * (unsigned)C + (unsigned)lane_c) * 4u;
-    const int ix = i16 == 15 ? x0 - 1 : x0 + i16;
-    unsigned vb[R];
+    unsigned vb[NG];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const int iy = y0 - 1 + r;
-        const bool ok = (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
-        vb[r] = ok ? (unsigned)(iy * W + ix) * 4u + (unsigned)lane_c * HW4 : kOutside;
-    }
-    float ra[2][8], rb[2][R][8];
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int p = 0; p < S; ++p) {
+            const int iy = y0 * S - 1 + r, ix = image_col(i16, p);
+            const bool ok = (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
+            vb[r * S + p] = ok ? (unsigned)(iy * W + ix) * 4u + (unsigned)lane_c * HW4 : kOutside;
+        }
+    float ra[NSTAGE][8], rb[NSTAGE][NG][8];
     auto load_step = [&](int s, int step) {
         const unsigned outm = step < lane_steps ? 0u : kOutside;
         const unsigned sa = (unsigned)step * 512u;
@@ -1318,69 +1337,85 @@ __device__ __forceinline__ bool conv2d_xdw_body(const ReefOpDesc& d, int task, c
             ra[s][4 * e] = v[0]; ra[s][4 * e + 1] = v[1]; ra[s][4 * e + 2] = v[2]; ra[s][4 * e + 3] = v[3];
         }
 #pragma unroll
-        for (int r = 0; r < R; ++r)
+        for (int g = 0; g < NG; ++g)
 #pragma unroll
             for (int q = 0; q < 8; ++q)
-                rb[s][r][q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                    rs_b, (int)(vb[r] | outm), (int)((unsigned)(step * 128 + q) * HW4), 0));
+                rb[s][g][q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                    rs_b, (int)(vb[g] | outm), (int)((unsigned)(step * 128 + q) * HW4), 0));
     };
     load_step(0, 0);
-    if (nsteps > 1) load_step(1, 1);
+    if (NSTAGE > 1 && nsteps > 1) load_step(NSTAGE - 1, 1);
     float wdw[9];
 #pragma unroll
     for (int t = 0; t < 9; ++t) wdw[t] = buf_load(rs_dw, ch * 36u + 4u * t);
     const float bdw = buf_load(rs_db, ch * 4u), bex = buf_load(rs_bias, ch * 4u);
 
-    f32x4 acc[R][2];
+    f32x4 acc[NG][2];
 #pragma unroll
-    for (int r = 0; r < R; ++r) acc[r][0] = acc[r][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int g = 0; g < NG; ++g) acc[g][0] = acc[g][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     auto mma_stage = [&](int s) {
 #pragma unroll
         for (int q = 0; q < 8; ++q)
 #pragma unroll
-            for (int r = 0; r < R; ++r)
-                acc[r][q & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[s][q], rb[s][r][q], acc[r][q & 1], 0, 0, 0);
+            for (int g = 0; g < NG; ++g)
+                acc[g][q & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[s][q], rb[s][g][q], acc[g][q & 1], 0, 0, 0);
     };
-    for (int it = 0; it < nsteps; it += 2) {
-        mma_stage(0);
-        if (it + 2 < nsteps) load_step(0, it + 2);
-        if (it + 1 < nsteps) {
-            mma_stage(1);
-            if (it + 3 < nsteps) load_step(1, it + 3);
+    if (NSTAGE == 1) {
+        for (int it = 0; it < nsteps; ++it) {
+            mma_stage(0);
+            if (it + 1 < nsteps) load_step(0, it + 1);
+        }
+    } else {
+        for (int it = 0; it < nsteps; it += 2) {
+            mma_stage(0);
+            if (it + 2 < nsteps) load_step(0, it + 2);
+            if (it + 1 < nsteps) {
+                mma_stage(NSTAGE - 1);
+                if (it + 3 < nsteps) load_step(NSTAGE - 1, it + 3);
+            }
         }
     }
 
     // the four wavefronts' partial tiles meet in LDS (row groups skewed: no bank conflicts)
-    float* part = smem + wave * (R * T::PART);
+    float* part = smem + wave * (NG * T::PART);
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) part[g * T::PART + (5 * kq + j) * 16 + i16] = acc[g][0][j] + acc[g][1][j];
+    __syncthreads();
+    const float* mine = smem + threadIdx.x + (threadIdx.x >> 6) * 16;
+    constexpr int WSTRIDE = NG * T::PART;
+    const int act = a[REEF_CONV_ACT], act2 = a[REEF_CONV_ACT2];
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) part[r * T::PART + (5 * kq + j) * 16 + i16] = acc[r][0][j] + acc[r][1][j];
-    __syncthreads();
-    const float* mine = smem + threadIdx.x + (threadIdx.x >> 6) * 16;
-    constexpr int WSTRIDE = R * T::PART;
-    const int act = a[REEF_CONV_ACT], act2 = a[REEF_CONV_ACT2];
-    const int cx = col == 15 ? x0 - 1 : x0 + col;      // image column of this thread's E column
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const float* e = mine + r * T::PART;
-        const float v = ((e[0] + e[WSTRIDE]) + e[2 * WSTRIDE]) + e[3 * WSTRIDE];
-        const bool inside = (unsigned)(y0 - 1 + r) < (unsigned)H && (unsigned)cx < (unsigned)W;
-        E[row * T::ESTRIDE + r * 16 + col] = inside ? act_apply(v + bex, act) : 0.0f;
-    }
+        for (int p = 0; p < S; ++p) {
+            const float* e = mine + (r * S + p) * T::PART;
+            const float v = ((e[0] + e[WSTRIDE]) + e[2 * WSTRIDE]) + e[3 * WSTRIDE];
+            const bool inside = (unsigned)(y0 * S - 1 + r) < (unsigned)H && (unsigned)image_col(col, p) < (unsigned)W;
+            E[row * T::ESTRIDE + (r * S + p) * 16 + col] = inside ? act_apply(v + bex, act) : 0.0f;
+        }
     __syncthreads();
 
-    // depthwise stage from E: the neighbours of column c are columns (c - 1) and (c + 1) mod 16
-    // (column 15 holds what lies left of column 0, column 14 what lies right of column 13)
-    const rsrc_t rs_o = make_rsrc(d.ptr[2], (unsigned)M * HW4);
+    // depthwise stage from E
+    const rsrc_t rs_o = make_rsrc(d.ptr[2], (unsigned)M * (unsigned)(Ho * Wo) * 4u);
     const float* Ec = E + row * T::ESTRIDE;
 #pragma unroll
     for (int g = 0; g < G; ++g) {
         float s = 0.0f;
 #pragma unroll
-        for (int t = 0; t < 9; ++t) s = fmaf(Ec[(g + t / 3) * 16 + ((col + t % 3 - 1) & 15)], wdw[t], s);
-        const bool ok = col < kRowSeg && x0 + col < W && y0 + g < H && ch < (unsigned)M;
-        buf_store(rs_o, ok ? ch * HW4 + (unsigned)((y0 + g) * W + x0 + col) * 4u : kOutside, act_apply(s + bdw, act2));
+        for (int t = 0; t < 9; ++t) {
+            const int ky = t / 3, kx = t % 3;
+            float tap;
+            if (S == 1) tap = Ec[(g + ky) * 16 + ((col + kx - 1) & 15)];
+            else tap = kx == 0 ? Ec[((2 * g + ky) * 2 + 1) * 16 + ((col - 1) & 15)]       // odd column left of 2 x
+                     : kx == 1 ? Ec[((2 * g + ky) * 2 + 0) * 16 + col]                    // 2 x
+                               : Ec[((2 * g + ky) * 2 + 1) * 16 + col];                   // 2 x + 1
+            s = fmaf(tap, wdw[t], s);
+        }
+        const bool ok = col < kRowSeg && x0 + col < Wo && y0 + g < Ho && ch < (unsigned)M;
+        buf_store(rs_o, ok ? (ch * (unsigned)(Ho * Wo) + (unsigned)((y0 + g) * Wo + x0 + col)) * 4u : kOutside,
+                  act_apply(s + bdw, act2));
     }
     return true;
 }

@@ -283,30 +283,34 @@ class GraphBuilder:
 
     XDW_TILES = {"g2": 2, "g4": 4}     # reef_conv2d_xdw_<tile>: image rows per tile
 
-    def conv2d_dw(self, x, cout, act=ACT_RELU6, dw_act=ACT_RELU6, tile=None):
-        """1x1 convolution (+ bias, act) followed by a depthwise 3x3 convolution (stride 1, padding
-        1, + bias, dw_act) as ONE launch (reef_conv2d_xdw_<tile>): the front half of a MobileNetV2
-        block without the expanded tensor in memory.  Parameters are created in the order the two
-        separate layers would create them."""
+    def conv2d_dw(self, x, cout, act=ACT_RELU6, dw_act=ACT_RELU6, tile=None, stride=1):
+        """1x1 convolution (+ bias, act) followed by a depthwise 3x3 convolution (padding 1, stride 1
+        or 2, + bias, dw_act) as ONE launch (reef_conv2d_xdw_<tile>, reef_conv2d_xdw2_g2): the front
+        half of a MobileNetV2 block without the expanded tensor in memory.  Parameters are created in
+        the order the two separate layers would create them."""
         cin, H, W = x.shape
-        assert cin % 8 == 0
+        assert cin % 8 == 0 and stride in (1, 2)
         w = self.param((cout, cin, 1, 1), self.weight_std if self.weight_std is not None else math.sqrt(2.0 / cin))
         b = self.param((cout,), 0.01)
         wd = self.param((cout, 1, 3, 3), self.weight_std if self.weight_std is not None else math.sqrt(2.0 / 9))
         bd = self.param((cout,), 0.01)
-        out = self.temp((cout, H, W))
-        if tile is None:
+        Ho, Wo = (H - 1) // stride + 1, (W - 1) // stride + 1
+        out = self.temp((cout, Ho, Wo))
+        if stride == 2:
+            tile = "g2"
+        elif tile is None:
             # two image rows per tile; four on large images, where four still leave every CU several
             # workgroups and the rows computed twice by neighbouring tiles weigh more (measured on
             # the shapes of MobileNetV2: 56 x 56 10.7 against 11.9 us, 28 x 28 and below two rows)
             tile = "g4" if H * W >= 3136 else "g2"
         G = self.XDW_TILES[tile]
-        mt, nt = math.ceil(cout / 16), math.ceil(H / G) * math.ceil(W / tiling.ROW_SEG)
-        flops = 2 * cout * H * W * (cin + 9)
+        mt, nt = math.ceil(cout / 16), math.ceil(Ho / G) * math.ceil(Wo / tiling.ROW_SEG)
+        flops = 2 * cout * (H * W * cin + Ho * Wo * 9)
         self.flops += flops
-        attrs = [cin, H, W, cout, H, W, 1, 1, 1, 1, 0, 0, F_BIAS | F_DW_OUTPUT, act, tiling.TILES[tile][0], 1,
-                 math.ceil(cin / 128) * 128, mt, nt, dw_act, 0, 6, 0, 0]
-        self._emit("reef_conv2d_xdw_" + tile, mt * nt, [x, w.idx, out.idx, b.idx, wd.idx, bd.idx], attrs, "conv2d",
+        attrs = [cin, H, W, cout, Ho, Wo, 1, 1, stride, stride, 0, 0, F_BIAS | F_DW_OUTPUT, act, tiling.TILES[tile][0],
+                 1, math.ceil(cin / 128) * 128, mt, nt, dw_act, 0, 6, 0, 0]
+        self._emit("reef_conv2d_xdw%s_%s" % ("2" if stride == 2 else "", tile), mt * nt,
+                   [x, w.idx, out.idx, b.idx, wd.idx, bd.idx], attrs, "conv2d",
                    flops, 4 * (x.size + cout * cin + 11 * cout + out.size), 6.0)
         return out
 
@@ -533,9 +537,10 @@ class GraphBuilder:
         for k in self.kernels:
             n = k["name"]
             sym = n.split("#")[0]
-            if sym.startswith("reef_conv2d_xdw_"):
-                R = self.XDW_TILES[sym.split("_")[-1]] + 2
-                shared[n] = (4 * R * 320 + 16 * (R + 1) * 16) * 4 + 16
+            if sym.startswith("reef_conv2d_xdw"):
+                G, S = self.XDW_TILES[sym.split("_")[-1]], 2 if sym.startswith("reef_conv2d_xdw2_") else 1
+                NG = (G + 2) if S == 1 else (2 * G + 1) * 2      # TileXdw: pixel groups of the 1x1 result
+                shared[n] = (4 * NG * 320 + 16 * (NG + 1) * 16) * 4 + 16
             elif sym.startswith("reef_conv2d_") or sym.startswith("reef_gemm_"):
                 shared[n] = tiling.lds_bytes(sym.split("_")[-1])
             else:
