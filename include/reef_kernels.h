@@ -358,21 +358,36 @@ enum { REEF_TR_D0 = 0, REEF_TR_D1, REEF_TR_D2, REEF_TR_FLAGS, REEF_TR_NATTR };
  * ntd: trans_b = 1, operands straight from memory into 16x16x4 MFMAs (tiles 16x16k4, 16x32k4,
  *      32x32d4; K a multiple of 8, lda, ldb and the batch strides multiples of 4);
  * nn: trans_b = 0 (K and lda multiples of 4).
- * C[b][m][n] = act(alpha * sum_k A[b][m][k] * B(b,k,n) (+bias[n]))
+ * C[b][m][n] = act(alpha * sum_k A[b][m][k] * B(b,k,n) (+bias[n])) (+R[b][m][n])
  * trans_b = 1: B stored [b][n][k] (dense layers, Q.K^T); 0: [b][k][n] (P.V).
- * ptr: A, B, C, bias(optional).
+ * R (REEF_GEMM_F_RES): a residual laid out as C is (ldc, offC, strideC), added after the activation.
+ * ptr: A, B, C, bias (optional), R (optional).
  * attr: batch, M, N, K, trans_b, flags, act, alpha (float bits), tile, m_tiles, n_tiles,
  *       lda, ldb, ldc, strideA, strideB, strideC (elements), then offA, offB, offC: where the
  *       first matrix starts inside its storage, in elements (absent = 0; multiples of 4 like the
  *       strides) -- several operands can share one storage, e.g. Q, K and V as column blocks of
  *       one [tokens][3 * hidden] projection.
- * tasks = batch * m_tiles * n_tiles. */
+ * tasks = batch * m_tiles * n_tiles.
+ *
+ * reef_gemm_ntl_<tile> (staged tiles, trans_b = 1, batch 1, flags has REEF_GEMM_F_LN): A is read
+ * through a LayerNorm of its rows,
+ *   A'[m][k] = (A[m][k] - mean[m]) / sqrt(var[m] + eps) * gamma[k] + beta[k]
+ * (mean and variance over the K columns of the row), and C = act(alpha * A' x B^T (+bias)) (+R).
+ * A and A' are [M][K] with leading dimension lda and no offset.
+ * ptr: A, B, C, bias (optional), R (optional), gamma, beta, A' (REEF_GEMM_F_LN_OUT: the
+ * normalised rows are written as well, a share by every workgroup of a row block).
+ * attr: as above, then eps (float bits). */
+#define REEF_GEMM_F_BIAS 1
+#define REEF_GEMM_F_LN 2
+#define REEF_GEMM_F_LN_OUT 4
+#define REEF_GEMM_F_RES 8
 enum {
     REEF_GEMM_BATCH = 0, REEF_GEMM_M, REEF_GEMM_N, REEF_GEMM_K, REEF_GEMM_TRANS_B,
     REEF_GEMM_FLAGS, REEF_GEMM_ACT, REEF_GEMM_ALPHA_BITS, REEF_GEMM_TILE, REEF_GEMM_M_TILES,
     REEF_GEMM_N_TILES, REEF_GEMM_LDA, REEF_GEMM_LDB, REEF_GEMM_LDC, REEF_GEMM_STRIDE_A,
     REEF_GEMM_STRIDE_B, REEF_GEMM_STRIDE_C, REEF_GEMM_OFF_A, REEF_GEMM_OFF_B, REEF_GEMM_OFF_C,
-    REEF_GEMM_NATTR
+    REEF_GEMM_NATTR,
+    REEF_GEMM_LN_EPS_BITS = REEF_GEMM_NATTR      /* reef_gemm_ntl_* only */
 };
 
 /* ---- add / multiply (the reference's mocked model): ptr: a, b, out; no attrs ---- */

@@ -409,6 +409,19 @@ class GraphOracle:
             alpha = _bits_to_float(alpha_bits)
             bias = P[3] if flags & 1 else None
             A, B, C = P[0][oA:], P[1][oB:], P[2][oC:]
+            p = 3 + (flags & 1)
+            R = None
+            if flags & 8:                                     # residual, laid out as C is
+                R = P[p][oC:]
+                p += 1
+            if flags & 2:
+                # reef_gemm_ntl_*: A goes through a LayerNorm of its rows first (include/reef_kernels.h)
+                gamma, beta = P[p][:K], P[p + 1][:K]
+                rows = np.ascontiguousarray(np.lib.stride_tricks.as_strided(A, (M, K), (lda * 4, 4)))
+                normed = layernorm(rows, gamma, beta, None, _bits_to_float(a[20]))
+                if flags & 4:
+                    np.lib.stride_tricks.as_strided(P[p + 2], (M, K), (lda * 4, 4))[:, :] = normed
+                A, lda = normed.reshape(-1), K
             for bi in range(batch):
                 Am = np.lib.stride_tricks.as_strided(A[bi * sA:], (M, K), (lda * 4, 4))
                 if trans_b:
@@ -423,6 +436,8 @@ class GraphOracle:
                     c = np.maximum(c, 0)
                 elif act == 3:
                     c = bias_gelu(c)
+                if R is not None:
+                    c = c + np.lib.stride_tricks.as_strided(R[bi * sC:], (M, N), (ldc * 4, 4))
                 Cm = np.lib.stride_tricks.as_strided(C[bi * sC:], (M, N), (ldc * 4, 4))
                 Cm[:, :] = c
         elif name == "reef_attention":

@@ -176,7 +176,7 @@ void splitk_reduce(const Attrs& a, Needs& n) {
     n.tasks = cdiv(MN, 1024);
 }
 
-void gemm(const Attrs& a, Needs& n) {
+void gemm(const std::string& symbol, const Attrs& a, Needs& n) {
     if (a.v.size() <= (size_t)REEF_GEMM_STRIDE_C) { n.bad = "too few attributes for a matrix product"; return; }
     if (!all_positive(a, {REEF_GEMM_BATCH, REEF_GEMM_M, REEF_GEMM_N, REEF_GEMM_K, REEF_GEMM_M_TILES,
                           REEF_GEMM_N_TILES, REEF_GEMM_LDA, REEF_GEMM_LDB, REEF_GEMM_LDC})) {
@@ -197,7 +197,21 @@ void gemm(const Attrs& a, Needs& n) {
     if (trans_b) n.f32("B", a[REEF_GEMM_OFF_B] + b1 * a[REEF_GEMM_STRIDE_B] + (N - 1) * a[REEF_GEMM_LDB] + K);
     else n.f32("B", a[REEF_GEMM_OFF_B] + b1 * a[REEF_GEMM_STRIDE_B] + (K - 1) * a[REEF_GEMM_LDB] + N);
     n.f32("C", a[REEF_GEMM_OFF_C] + b1 * a[REEF_GEMM_STRIDE_C] + (M - 1) * a[REEF_GEMM_LDC] + N);
-    if (a[REEF_GEMM_FLAGS] & 1) n.f32("bias", N);
+    const i64 fl = a[REEF_GEMM_FLAGS];
+    const i64 c_elems = a[REEF_GEMM_OFF_C] + b1 * a[REEF_GEMM_STRIDE_C] + (M - 1) * a[REEF_GEMM_LDC] + N;
+    if (fl & REEF_GEMM_F_BIAS) n.f32("bias", N);
+    if (fl & REEF_GEMM_F_RES) n.f32("residual", c_elems);
+    // A read through a LayerNorm of its rows: only the kernels named ntl do that, and they do nothing else
+    const bool ln_kernel = symbol.compare(0, 14, "reef_gemm_ntl_") == 0;
+    if (ln_kernel != ((fl & REEF_GEMM_F_LN) != 0)) { n.bad = "the LayerNorm flag and the kernel's name contradict each other"; return; }
+    if (!ln_kernel && (fl & REEF_GEMM_F_LN_OUT)) { n.bad = "LayerNorm operands on a plain matrix product"; return; }
+    if (ln_kernel) {
+        if (!trans_b || b1 != 0 || a[REEF_GEMM_OFF_A] != 0) { n.bad = "the LayerNorm form takes one K-contiguous B and A without offset"; return; }
+        if (a.v.size() <= (size_t)REEF_GEMM_LN_EPS_BITS) { n.bad = "the LayerNorm form needs its epsilon"; return; }
+        n.f32("gamma", K);
+        n.f32("beta", K);
+        if (fl & REEF_GEMM_F_LN_OUT) n.f32("normalised A", (M - 1) * a[REEF_GEMM_LDA] + K);
+    }
     n.tasks = a[REEF_GEMM_BATCH] * a[REEF_GEMM_M_TILES] * a[REEF_GEMM_N_TILES];
     if (n.tasks >= kDivSmallLimit) n.bad = "4 Mi workgroups or more (the kernels' index arithmetic is exact below that)";
 }
@@ -370,7 +384,7 @@ bool kernel_fits_storages(const Model& m, size_t index, std::string* why) {
     switch (op) {
     case REEF_OP_CONV2D: conv2d(symbol, a, n); break;
     case REEF_OP_SPLITK_REDUCE: splitk_reduce(a, n); break;
-    case REEF_OP_GEMM: gemm(a, n); break;
+    case REEF_OP_GEMM: gemm(symbol, a, n); break;
     case REEF_OP_ATTENTION: attention(a, n); break;
     default:
         if (!small_op(op, a, grid, n)) return true;

@@ -101,6 +101,10 @@ __device__ __forceinline__ f32x4 buf_load4(rsrc_t r, unsigned byte_off) {
 __device__ __forceinline__ void buf_store(rsrc_t r, unsigned byte_off, float v) {
     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, (int)byte_off, 0, 0);
 }
+__device__ __forceinline__ void buf_store4(rsrc_t r, unsigned byte_off, f32x4 v) {
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, (int)byte_off, 0, 0);
+}
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

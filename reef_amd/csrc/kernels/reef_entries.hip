@@ -62,12 +62,12 @@ struct OpConvXdw {
         return conv2d_xdw_body<G, S>(d, task, smem, p);
     }
 };
-template <class T, bool TRANS_B>
+template <class T, bool TRANS_B, bool LN_A = false>
 struct OpGemm {
-    static constexpr int LDS = T::LDS_BYTES;
+    static constexpr int LDS = T::LDS_BYTES + (LN_A ? 2 * T::BM * 4 : 0);   // + mean, rstd of the tile's rows
     template <class P>
     static __device__ __forceinline__ bool run(const ReefOpDesc& d, int task, char* smem, const P& p) {
-        return gemm_body<T, TRANS_B>(d, task, smem, p);
+        return gemm_body<T, TRANS_B, LN_A>(d, task, smem, p);
     }
 };
 template <int TM, int TN>
@@ -352,6 +352,8 @@ REEF_ENTRY(reef_gemm_nt_64x64, OpGemm<Tile64x64 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nt_32x128, OpGemm<Tile32x128 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nt_32x32k4, OpGemm<Tile32x32k4 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nt_64x32k2, OpGemm<Tile64x32k2 REEF_COMMA true>)
+REEF_ENTRY(reef_gemm_ntl_32x32k4, OpGemm<Tile32x32k4 REEF_COMMA true REEF_COMMA true>)
+REEF_ENTRY(reef_gemm_ntl_64x32k2, OpGemm<Tile64x32k2 REEF_COMMA true REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_ntd_16x16k4, OpGemmNtDirect<1 REEF_COMMA 1>)
 REEF_ENTRY(reef_gemm_ntd_16x32k4, OpGemmNtDirect<1 REEF_COMMA 2>)
 REEF_ENTRY(reef_gemm_ntd_32x32d4, OpGemmNtDirect<2 REEF_COMMA 2>)

@@ -71,17 +71,37 @@ typedef Tile<1, 2, 1, 1, 2, 2> Tile32x64k2;
 
 // ---- A tile: rows of a K-contiguous matrix -------------------------------
 // VEC: rows are 16-byte aligned at every k that is a multiple of 4 (K % 4 == 0).
-template <class T, bool VEC>
+// LN (reef_gemm_ntl_*): the matrix is read through a LayerNorm of its rows -- what goes into LDS
+// is (a - mean[row]) * rstd[row] * gamma[k] + beta[k], with the row statistics worked out
+// by the workgroup beforehand (gemm_body).  gamma and beta ride along with every load; the
+// arithmetic happens on the way into LDS, so the loads stay asynchronous.  (No store to memory in
+// here: loads and stores share one counter of outstanding operations, and a store in the K loop
+// makes every wait for a tile a wait for everything.)
+template <class T, bool VEC, bool LN = false>
 struct ALoader {
     static constexpr int TPR = T::BK / 4;          // threads (float4s) per tile row
     static constexpr int RPP = kThreads / TPR;     // rows per pass
     static constexpr int NV = T::BM / RPP;         // float4 per thread per tile
     static_assert(NV >= 1, "tile shorter than one pass");
-    struct Regs { f32x4 v[NV]; };
+    static_assert(!LN || VEC, "the LayerNorm form loads whole float4s");
+    struct Regs { f32x4 v[NV]; f32x4 g, b; };
     rsrc_t rs;
     unsigned rowoff[NV];    // byte offset of the row (kOutside when the row is outside M)
     int k;                  // k of this thread's float4 in the next tile
     int k_end;
+    // LN only
+    rsrc_t rs_g, rs_b;
+    float mean[LN ? NV : 1], rstd[LN ? NV : 1];
+    __device__ __forceinline__ void init_ln(const float* gamma, const float* beta, int K, const float* stats) {
+        rs_g = make_rsrc(gamma, (unsigned)K * 4u);
+        rs_b = make_rsrc(beta, (unsigned)K * 4u);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int r = threadIdx.x / TPR + RPP * i;     // row inside the tile
+            mean[LN ? i : 0] = stats[2 * r];
+            rstd[LN ? i : 0] = stats[2 * r + 1];
+        }
+    }
 
     // `bytes`: size of the matrix from `a` on
     __device__ __forceinline__ void init(const float* a, unsigned bytes, int lda, int m0, int M,
@@ -102,6 +122,10 @@ struct ALoader {
             const unsigned koff = k < k_end ? (unsigned)k * 4u : kOutside;
 #pragma unroll
             for (int i = 0; i < NV; ++i) r.v[i] = buf_load4(rs, rowoff[i] + koff);
+            if (LN) {
+                r.g = buf_load4(rs_g, koff);     // outside K: gamma = beta = 0, the value becomes 0
+                r.b = buf_load4(rs_b, koff);
+            }
         } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -115,8 +139,15 @@ struct ALoader {
     __device__ __forceinline__ void store(const Regs& r, float* As) const {
         const int tid = threadIdx.x;
 #pragma unroll
-        for (int i = 0; i < NV; ++i)
-            *(f32x4*)(As + (tid / TPR + RPP * i) * T::LDA + (tid % TPR) * 4) = r.v[i];
+        for (int i = 0; i < NV; ++i) {
+            f32x4 v = r.v[i];
+            if (LN) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    v[e] = (v[e] - mean[LN ? i : 0]) * rstd[LN ? i : 0] * r.g[e] + r.b[e];
+            }
+            *(f32x4*)(As + (tid / TPR + RPP * i) * T::LDA + (tid % TPR) * 4) = v;
+        }
     }
 };
 
@@ -1424,7 +1455,21 @@ __device__ __forceinline__ bool conv2d_xdw_body(const ReefOpDesc& d, int task, c
 // TRANS_B: B stored [N][K] (dense layers, Q.K^T) -- both operands take 128-bit row
 // loads, so K, lda, ldb and the batch strides must be multiples of 4 floats.
 // !TRANS_B: B stored [K][N] (P.V) -- element-wise B loads, 128-bit A loads.
-template <class T, bool TRANS_B, class Poll>
+// LN_A (symbols reef_gemm_ntl_<tile>, REEF_GEMM_F_LN): A is read through a LayerNorm of its rows,
+// A' = LayerNorm(A) * gamma + beta (row statistics over all K columns).  A transformer layer
+// normalises and then multiplies: as two launches the normalised matrix makes a round trip
+// through memory behind a launch that only reads and writes 128 rows.  Here every workgroup works
+// out mean and 1 / sqrt(var + eps) of its own BM rows before its K loop -- all column tiles of a
+// row block do the same, on rows that are cache hits after the first -- and normalises on the
+// way into LDS.  The statistics are made in ONE pass over the row (a second pass would be a
+// second trip to memory, and a row held in registers between two passes takes the registers that
+// let two workgroups share a CU): every thread sums x - p and (x - p)^2 around a pivot p, the first
+// value it meets, which gives its own count, mean and sum of squared deviations; the threads of
+// a row merge these pairwise (Chan, Golub, LeVeque 1979), which is as stable as two passes.
+// The workgroups of a row block also write A', a share each (REEF_GEMM_F_LN_OUT: the operand of
+// the next residual).  A and A' are [M][K] with leading dimension lda and no offset; no batch.
+// ptr: A, B, C, bias (optional), residual (optional), then gamma, beta, A' (optional).
+template <class T, bool TRANS_B, bool LN_A, class Poll>
 __device__ __forceinline__ bool gemm_body(const ReefOpDesc& d, int task, char* smem_raw,
                                           const Poll& poll) {
     const int* a = d.attr;
@@ -1444,8 +1489,97 @@ __device__ __forceinline__ bool gemm_body(const ReefOpDesc& d, int task, char* s
     f32x16 acc[T::TM][T::TN];
 
     bool ok;
-    ALoader<T, true> la;
+    ALoader<T, true, LN_A> la;
     la.init(A, ((unsigned)(M - 1) * (unsigned)lda + (unsigned)K) * 4u, lda, m0, M, 0, K);
+    if (LN_A) {
+        static_assert(!LN_A || TRANS_B, "the LayerNorm form exists for K-contiguous B");
+        const int fl = a[REEF_GEMM_FLAGS];
+        int p = 3 + (fl & REEF_GEMM_F_BIAS ? 1 : 0) + (fl & REEF_GEMM_F_RES ? 1 : 0);
+        const float* gamma = (const float*)d.ptr[p++];
+        const float* beta = (const float*)d.ptr[p++];
+        float* Aout = (fl & REEF_GEMM_F_LN_OUT) ? (float*)d.ptr[p] : nullptr;
+        const unsigned bytes = ((unsigned)(M - 1) * (unsigned)lda + (unsigned)K) * 4u;
+        // kThreads / BM threads per row (neighbouring lanes), thread `spart` of a row on float4s
+        // spart, spart + TPRS, ..; UB of them per batch, the next batch in flight behind the current.
+        constexpr int TPRS = kThreads / T::BM, UB = 8;
+        static_assert(TPRS >= 1 && TPRS <= 64 && (TPRS & (TPRS - 1)) == 0, "threads per row: a power of two within a wavefront");
+        float* stats = smem + (T::LDS_BYTES / 4);          // behind the staging buffers: mean, rstd per row
+        const int srow = threadIdx.x / TPRS, spart = threadIdx.x % TPRS;
+        const rsrc_t rs1 = make_rsrc(A, bytes);
+        const unsigned roff = m0 + srow < M ? (unsigned)(m0 + srow) * (unsigned)lda * 4u : kOutside;
+        const int per_thread = (K / 4 + TPRS - 1) / TPRS;      // float4s of the busiest thread of a row
+        auto load_batch = [&](f32x4 (&v)[UB], int j0) {
+#pragma unroll
+            for (int u = 0; u < UB; ++u) {
+                const int k4 = (spart + (j0 + u) * TPRS) * 4;
+                v[u] = buf_load4(rs1, k4 < K ? roff + (unsigned)k4 * 4u : kOutside);
+            }
+        };
+        f32x4 cur[UB], nxt[UB];
+        load_batch(cur, 0);
+        const float pivot = cur[0][0];
+        float s1 = 0.0f, s2 = 0.0f, cnt = 0.0f;
+        for (int j0 = 0; j0 < per_thread; j0 += UB) {
+            if (j0 + UB < per_thread) load_batch(nxt, j0 + UB);
+#pragma unroll
+            for (int u = 0; u < UB; ++u) {
+                const bool in = (spart + (j0 + u) * TPRS) * 4 < K;
+                cnt += in ? 4.0f : 0.0f;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float dl = in ? cur[u][e] - pivot : 0.0f;
+                    s1 += dl;
+                    s2 = fmaf(dl, dl, s2);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < UB; ++u) cur[u] = nxt[u];
+        }
+        // this thread's part of the row: count, mean, sum of squared deviations from that mean
+        float mean = cnt > 0.0f ? pivot + s1 / cnt : 0.0f;
+        float m2 = cnt > 0.0f ? s2 - s1 * (s1 / cnt) : 0.0f;
+#pragma unroll
+        for (int o = 1; o < TPRS; o <<= 1) {
+            const float cnt_o = __shfl_xor(cnt, o, 64), mean_o = __shfl_xor(mean, o, 64), m2_o = __shfl_xor(m2, o, 64);
+            const float tot = cnt + cnt_o, dm = mean_o - mean;
+            // symmetric in the two partners, so both hold the same bits afterwards
+            const float w_o = tot > 0.0f ? cnt_o / tot : 0.0f, w_s = tot > 0.0f ? cnt / tot : 0.0f;
+            mean = mean * w_s + mean_o * w_o;
+            m2 = (m2 + m2_o) + dm * dm * (tot > 0.0f ? (cnt * cnt_o) / tot : 0.0f);
+            cnt = tot;
+        }
+        const float rstd = 1.0f / sqrtf(fmaxf(m2, 0.0f) / (float)K + __int_as_float(a[REEF_GEMM_LN_EPS_BITS]));
+        if (spart == 0) {
+            stats[2 * srow] = mean;
+            stats[2 * srow + 1] = rstd;
+        }
+        __syncthreads();
+        if (Aout) {
+            // The normalised rows go to memory as well, a share per column tile: the BM * K / 4
+            // float4s of the row block in n_tiles contiguous runs (one or two per thread, in flight
+            // beside the first loads of the K loop; one workgroup writing it all would be the
+            // launch's straggler).
+            const rsrc_t rs_g = make_rsrc(gamma, (unsigned)K * 4u), rs_b = make_rsrc(beta, (unsigned)K * 4u);
+            const rsrc_t rs_o = make_rsrc(Aout, bytes);
+            const int row4 = K / 4, total = T::BM * row4;
+            const int share = (total + n_tiles - 1) / n_tiles;
+            const int end = (nt + 1) * share < total ? (nt + 1) * share : total;
+            for (int id = nt * share + (int)threadIdx.x; id < end; id += kThreads) {
+                const int r = div_small(id, row4), k4 = (id - r * row4) * 4;
+                if (m0 + r < M) {
+                    const unsigned off = ((unsigned)(m0 + r) * (unsigned)lda + (unsigned)k4) * 4u;
+                    const f32x4 v = buf_load4(rs1, off);
+                    const f32x4 gm = buf_load4(rs_g, (unsigned)k4 * 4u), bt = buf_load4(rs_b, (unsigned)k4 * 4u);
+                    const float mu = stats[2 * r], rs = stats[2 * r + 1];
+                    f32x4 y;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) y[e] = (v[e] - mu) * rs * gm[e] + bt[e];
+                    buf_store4(rs_o, off, y);
+                }
+            }
+        }
+        la.init_ln(gamma, beta, K, stats);
+    }
     if (TRANS_B) {
         // B is [N][K]: stage it exactly like A (rows = n).
         typedef Tile<T::WGN, T::WGM, T::TN, T::TM, T::DEPTH, T::KW> TB;  // BM of TB == BN of T
@@ -1464,7 +1598,11 @@ __device__ __forceinline__ bool gemm_body(const ReefOpDesc& d, int task, char* s
     const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
     const WaveGeom<T> wg;
     const int wm0 = wg.wm0, wn0 = wg.wn0;
-    const float* bias = (a[REEF_GEMM_FLAGS] & 1) ? (const float*)d.ptr[3] : nullptr;
+    const float* bias = (a[REEF_GEMM_FLAGS] & REEF_GEMM_F_BIAS) ? (const float*)d.ptr[3] : nullptr;
+    // the residual: laid out as C is (same leading dimension, offset and batch stride)
+    const float* R = (a[REEF_GEMM_FLAGS] & REEF_GEMM_F_RES)
+                         ? (const float*)d.ptr[bias ? 4 : 3] + a[REEF_GEMM_OFF_C] + (size_t)b * a[REEF_GEMM_STRIDE_C]
+                         : nullptr;
     const float alpha = __int_as_float(a[REEF_GEMM_ALPHA_BITS]);
     const int act = a[REEF_GEMM_ACT];
 #pragma unroll
@@ -1481,6 +1619,7 @@ __device__ __forceinline__ bool gemm_body(const ReefOpDesc& d, int task, char* s
                     float v = res[tm][tn][rr] * alpha + bv;
                     if (act == REEF_ACT_RELU) v = fmaxf(v, 0.0f);
                     else if (act == REEF_ACT_GELU) v = gelu_erf(v);
+                    if (R) v += R[(size_t)m * ldc + n];
                     C[(size_t)m * ldc + n] = v;
                 }
             }
@@ -1522,13 +1661,17 @@ __device__ __forceinline__ bool gemm_nt_direct_body(const ReefOpDesc& d, int tas
                                   ((unsigned)(N - 1) * ldb + (unsigned)K) * 4u);
     const rsrc_t rs_c = make_rsrc((const float*)d.ptr[2] + a[REEF_GEMM_OFF_C] + (size_t)b * a[REEF_GEMM_STRIDE_C],
                                   ((unsigned)(M - 1) * ldc + (unsigned)N) * 4u);
-    const bool has_bias = a[REEF_GEMM_FLAGS] & 1;
+    const bool has_bias = a[REEF_GEMM_FLAGS] & REEF_GEMM_F_BIAS, has_res = a[REEF_GEMM_FLAGS] & REEF_GEMM_F_RES;
     const rsrc_t rs_bias = make_rsrc(d.ptr[has_bias ? 3 : 2], (unsigned)N * 4u);
+    // the residual is laid out as C is; without one an empty buffer, whose loads give 0
+    const rsrc_t rs_res = make_rsrc((const float*)d.ptr[has_res ? (has_bias ? 4 : 3) : 2] + a[REEF_GEMM_OFF_C] +
+                                        (size_t)b * a[REEF_GEMM_STRIDE_C],
+                                    has_res ? ((unsigned)(M - 1) * ldc + (unsigned)N) * 4u : 0u);
 
     // the outputs of this thread and their bias, ahead of the K loop
     const int orow = threadIdx.x >> 4, ocol = threadIdx.x & 15;
     unsigned ooff[TM][TN];
-    float e_bias[TN];
+    float e_bias[TN], e_res[TM][TN];
 #pragma unroll
     for (int g = 0; g < TN; ++g) {
         const unsigned n = (unsigned)(n0 + 16 * g + ocol);
@@ -1537,6 +1680,7 @@ __device__ __forceinline__ bool gemm_nt_direct_body(const ReefOpDesc& d, int tas
         for (int h = 0; h < TM; ++h) {
             const unsigned m = (unsigned)(m0 + 16 * h + orow);
             ooff[h][g] = n < (unsigned)N ? (m * ldc + n) * 4u : kOutside;
+            e_res[h][g] = buf_load(rs_res, ooff[h][g]);
         }
     }
 
@@ -1644,7 +1788,7 @@ __device__ __forceinline__ bool gemm_nt_direct_body(const ReefOpDesc& d, int tas
             float v = (((e[0] + e[WSTRIDE]) + e[2 * WSTRIDE]) + e[3 * WSTRIDE]) * alpha + e_bias[g];
             if (act == REEF_ACT_RELU) v = fmaxf(v, 0.0f);
             else if (act == REEF_ACT_GELU) v = gelu_erf(v);
-            buf_store(rs_c, ooff[h][g], v);
+            buf_store(rs_c, ooff[h][g], v + e_res[h][g]);
         }
     return true;
 }

@@ -411,10 +411,16 @@ class GraphBuilder:
                    "softmax", 0, 8 * rows * cols, 2.0)
         return out
 
+    def layernorm_params(self, cols):
+        """gamma ~ 1 + N(0, 0.1), beta ~ N(0, 0.01): the parameters layernorm() makes for itself."""
+        gamma = self.param((cols,), 0.1)
+        self.params[-1] = (self.params[-1][0], self.params[-1][1] + 1.0)
+        return gamma, self.param((cols,), 0.01)
+
     def layernorm(self, x, rows, cols, res=None, eps=1e-12, out=None, gamma=None, beta=None):
         if gamma is None:
-            gamma = self.param((cols,), 0.1)
-            self.params[-1] = (self.params[-1][0], self.params[-1][1] + 1.0)
+            gamma, b = self.layernorm_params(cols)
+            beta = b if beta is None else beta
         if beta is None:
             beta = self.param((cols,), 0.01)
         out = Tensor(out.idx, (rows, cols)) if out is not None else self.temp((rows, cols))
@@ -491,10 +497,14 @@ class GraphBuilder:
 
     def gemm(self, a, b, M, N, K, batch=1, trans_b=True, bias=None, act=ACT_NONE, alpha=1.0,
              lda=None, ldb=None, ldc=None, stride_a=0, stride_b=0, stride_c=0, out=None, force_tile=None,
-             off_a=0, off_b=0, off_c=0):
-        """C[b] = act(alpha * A[b] x B[b] (+bias)); operands are storages with explicit strides.
+             off_a=0, off_b=0, off_c=0, ln=None, res=None):
+        """C[b] = act(alpha * A[b] x B[b] (+bias)) (+res[b]); operands are storages with explicit strides.
+        res: a residual laid out as C is.
         force_tile: a staged tile name or, for trans_b, one of tiling.GEMM_DIRECT_TILES.
-        off_a / off_b / off_c: element at which the first matrix starts inside its storage."""
+        off_a / off_b / off_c: element at which the first matrix starts inside its storage.
+        ln: dict(gamma=, beta=, eps=1e-12, out=None) -- A is read through a LayerNorm of its rows,
+        and `out`, if given, receives the normalised rows (kernels reef_gemm_ntl_<tile>: staged
+        tiles, one K-contiguous B)."""
         lda = K if lda is None else lda
         ldb = (K if trans_b else N) if ldb is None else ldb
         ldc = N if ldc is None else ldc
@@ -503,6 +513,12 @@ class GraphBuilder:
         assert off_a % 4 == 0 and off_b % 4 == 0 and off_c % 4 == 0, "gemm operands must be 16-byte aligned"
         direct_ok = (trans_b and K % 8 == 0 and lda % 4 == 0 and ldb % 4 == 0 and stride_a % 4 == 0
                      and stride_b % 4 == 0)
+        if ln is not None:
+            assert trans_b and batch == 1 and off_a == 0, "the LayerNorm form: one K-contiguous B, A without offset"
+            direct_ok = False
+            if force_tile is None:
+                force_tile = self.LN_GEMM_TILE
+            assert force_tile in self.LN_GEMM_TILES, "no LayerNorm form of this tile"
         if force_tile is not None:
             t = tiling.forced(force_tile, M, N, K, 1)
         else:
@@ -514,18 +530,32 @@ class GraphBuilder:
         if bias is not None:
             flags = 1
             args.append(bias.idx)
+        if res is not None:
+            flags |= 8
+            args.append(res.idx)
+        attrs_ln = []
+        if ln is not None:
+            flags |= 2
+            args += [ln["gamma"].idx, ln["beta"].idx]
+            if ln.get("out") is not None:
+                flags |= 4
+                args.append(ln["out"].idx)
+            attrs_ln = [float_bits(ln.get("eps", 1e-12))]
         flops = 2 * batch * M * N * K
         self.flops += flops
         assert K % 4 == 0 and lda % 4 == 0 and stride_a % 4 == 0, "gemm operands must be 16-byte aligned"
         if trans_b:
             assert ldb % 4 == 0 and stride_b % 4 == 0, "gemm operands must be 16-byte aligned"
-        self._emit("reef_gemm_%s_%s" % ("ntd" if direct else "nt" if trans_b else "nn", t["tile"]),
+        self._emit("reef_gemm_%s_%s" % ("ntl" if ln is not None else "ntd" if direct else "nt" if trans_b else "nn", t["tile"]),
                    batch * t["m_tiles"] * t["n_tiles"], args,
                    [batch, M, N, K, 1 if trans_b else 0, flags, act, float_bits(alpha), t["tile_id"],
                     t["m_tiles"], t["n_tiles"], lda, ldb, ldc, stride_a, stride_b, stride_c,
-                    off_a, off_b, off_c],
+                    off_a, off_b, off_c] + attrs_ln,
                    "gemm", flops, 4 * batch * (M * K + N * K + M * N), t["est_us"])
         return out
+
+    LN_GEMM_TILES = ("32x32k4", "64x32k2")     # tiles that exist as reef_gemm_ntl_<tile>
+    LN_GEMM_TILE = "32x32k4"
 
     def mocked(self, name, a, b, out):
         self._emit(name, 64, [a.idx, b.idx, out.idx], [], "mocked", 0, 3 * 8192 * 4, 14.0,
@@ -543,6 +573,8 @@ class GraphBuilder:
                 shared[n] = (4 * NG * 320 + 16 * (NG + 1) * 16) * 4 + 16
             elif sym.startswith("reef_conv2d_") or sym.startswith("reef_gemm_"):
                 shared[n] = tiling.lds_bytes(sym.split("_")[-1])
+                if sym.startswith("reef_gemm_ntl_"):
+                    shared[n] += 2 * tiling.TILES[sym.split("_")[-1]][1] * 4    # mean, 1/std of the tile's rows
             else:
                 shared[n] = 4   # the reference's floor (generate_final_schedule.py:117-143)
         return {"storage": self.storage, "kernels": self.kernels, "args": self.graph_args,

@@ -305,7 +305,7 @@ def inception_v3(image=(3, 299, 299), classes=1000, name="inceptionv3", seed=rng
 
 
 def bert(layers=12, hidden=768, heads=12, ffn=3072, seq=128, vocab=30522, name="bert_base",
-         seed=rng.BASE_SEED, attention_mask=False, fused_attention=True):
+         seed=rng.BASE_SEED, attention_mask=False, fused_attention=True, fuse_layernorm=True):
     """BERT encoder (base: 12 layers, hidden 768, 12 heads, FFN 3072, sequence 128), fp32,
     weights ~ N(0, 0.02).  Token ids are an int64 input, as in the reference's BERT model
     (resource/bert/bert.json storage[0]).  The per-head views of Q, K, V and of the context
@@ -318,18 +318,46 @@ def bert(layers=12, hidden=768, heads=12, ffn=3072, seq=128, vocab=30522, name="
     that every softmax applies to the key positions.  The reference's BERT derives that mask
     inside the graph -- as all zeros (fused_full_equal_reshape, bert.cu:313) -- and applies it
     with a kernel of its own per layer (bert.cu:381-388); here it is an operand of the softmax,
-    and a storage nobody has set is all zeros, as every storage is after loading."""
+    and a storage nobody has set is all zeros, as every storage is after loading.
+    fuse_layernorm: a LayerNorm whose result feeds a projection (the one before Q/K/V and the one
+    before the FFN) is not a launch of its own: the projection normalises the rows on the way into
+    its tiles and writes them out for the next residual (reef_gemm_ntl_*); only the last
+    LayerNorm of the network remains a kernel, and the residual sums are made by the epilogues
+    of the products in front -- 24 launches fewer, same parameters in the same order."""
     g = GraphBuilder(name, seed, weight_std=0.02)
     hd = hidden // heads
     ids = g.input("input0", (seq,), "int64")
     mask = g.input("attention_mask", (seq,), "uint1") if attention_mask else None
     x = g.embedding(ids, vocab, seq, hidden, pos=True, seg=True)
-    x = g.layernorm(x, seq, hidden)
+
+    # fuse_layernorm: the residual sum is made by the product in front of the LayerNorm (its
+    # epilogue adds the residual), the LayerNorm by the product behind it
+    def norm_then_project(pre, res, wt, bias, n, act=0):
+        """LayerNorm(pre (+ res)) and its projection: (normalised rows, product)."""
+        gamma, beta = g.layernorm_params(hidden)
+        w_, b_ = wt(), bias()
+        if fuse_layernorm:
+            assert res is None
+            normed = g.temp((seq, hidden))
+            out = g.gemm(pre, w_, seq, n, hidden, trans_b=True, bias=b_, act=act,
+                         ln=dict(gamma=gamma, beta=beta, out=normed))
+            return normed, out
+        normed = g.layernorm(pre, seq, hidden, res=res, gamma=gamma, beta=beta)
+        return normed, g.gemm(normed, w_, seq, n, hidden, trans_b=True, bias=b_, act=act)
+
+    def project_back(a, wt, k, res):
+        """a x wt^T + bias and the residual: the sum itself (fused) or (product, residual) for the LayerNorm kernel."""
+        w_ = g.param((hidden, k), 0.02)
+        b_ = g.param((hidden,), 0.02)
+        if fuse_layernorm:
+            return g.gemm(a, w_, seq, hidden, k, trans_b=True, bias=b_, res=res), None
+        return g.gemm(a, w_, seq, hidden, k, trans_b=True, bias=b_), res
+
+    pre, res = x, None
     inv_sqrt = 1.0 / (hd ** 0.5)
     for _ in range(layers):
-        w = g.param((3 * hidden, hidden), 0.02)
-        b = g.param((3 * hidden,), 0.02)
-        qkv = g.gemm(x, w, seq, 3 * hidden, hidden, trans_b=True, bias=b)
+        x, qkv = norm_then_project(pre, res, lambda: g.param((3 * hidden, hidden), 0.02),
+                                   lambda: g.param((3 * hidden,), 0.02), 3 * hidden)
         if fused_attention and g.attention_ok(seq, hd, 3 * hidden, hidden, (0, hidden, 2 * hidden)):
             # scores, masked softmax and context of all heads in one launch: the scores of a
             # workgroup's query rows stay in its registers and LDS
@@ -342,18 +370,11 @@ def bert(layers=12, hidden=768, heads=12, ffn=3072, seq=128, vocab=30522, name="
             ctx = g.temp((seq, hidden))
             g.gemm(probs, qkv, seq, hd, seq, batch=heads, trans_b=False, lda=seq, ldb=3 * hidden, ldc=hidden,
                    stride_a=seq * seq, stride_b=hd, stride_c=hd, out=ctx, off_b=2 * hidden)
-        wo = g.param((hidden, hidden), 0.02)
-        bo = g.param((hidden,), 0.02)
-        att = g.gemm(ctx, wo, seq, hidden, hidden, trans_b=True, bias=bo)
-        x = g.layernorm(att, seq, hidden, res=x)
-        w1 = g.param((ffn, hidden), 0.02)
-        b1 = g.param((ffn,), 0.02)
-        h = g.gemm(x, w1, seq, ffn, hidden, trans_b=True, bias=b1, act=ACT_GELU)
-        w2 = g.param((hidden, ffn), 0.02)
-        b2 = g.param((hidden,), 0.02)
-        y = g.gemm(h, w2, seq, hidden, ffn, trans_b=True, bias=b2)
-        x = g.layernorm(y, seq, hidden, res=x)
-    g.mark_output(x)
+        pre, res = project_back(ctx, None, hidden, x)
+        x, h = norm_then_project(pre, res, lambda: g.param((ffn, hidden), 0.02), lambda: g.param((ffn,), 0.02),
+                                 ffn, ACT_GELU)
+        pre, res = project_back(h, None, ffn, x)
+    g.mark_output(g.layernorm(pre, seq, hidden, res=res))
     return g
 
 

@@ -506,3 +506,40 @@ def test_a_pointwise_plus_depthwise_kernel_is_checked_against_its_storages(tmp_p
     broken(lambda m: m["kernels"][0]["attrs"].__setitem__(12, 1), "loader family")      # flag missing
     broken(lambda m: m["storage"][m["kernels"][0]["args"][4]].__setitem__("size", 48 * 8), "depthwise weights")
     broken(lambda m: m["kernels"][0]["launch_params"].__setitem__(0, 5), "workgroups")
+
+
+def test_a_product_behind_a_layernorm_is_checked_against_its_storages(tmp_path):
+    """reef_gemm_ntl_<tile> and the residual of a matrix product: operand list and sizes follow from
+    the flags; the LayerNorm flag belongs to the kernels named ntl and to no other."""
+    from reef_amd import binding as B
+    g = MB.GraphBuilder("ntlfmt")
+    x = g.input("x", (40, 200))
+    r = g.input("r", (40, 96))
+    w = g.param((96, 200), 0.05)
+    b = g.param((96,), 0.05)
+    gamma, beta = g.layernorm_params(200)
+    normed = g.temp((40, 200))
+    y = g.gemm(x, w, 40, 96, 200, trans_b=True, bias=b, res=r, ln=dict(gamma=gamma, beta=beta, out=normed))
+    g.mark_output(y)
+    base = g.write(str(tmp_path / "ok"), link_code_objects=False)
+    assert B.check_model(base + ".json") == (True, "")
+    model = json.load(open(base + ".json"))
+    k = model["kernels"][0]
+    assert k["name"].startswith("reef_gemm_ntl_32x32k4") and len(k["args"]) == 8 and k["attrs"][5] == 1 | 2 | 4 | 8
+
+    def broken(change, reason):
+        m = json.loads(json.dumps(model))
+        change(m)
+        p = str(tmp_path / "broken.json")
+        json.dump(m, open(p, "w"))
+        ok, why = B.check_model(p)
+        assert not ok and reason in why, why
+
+    broken(lambda m: m["kernels"][0]["args"].pop(), "operands")                               # no A'
+    broken(lambda m: m["kernels"][0]["attrs"].pop(), "epsilon")
+    broken(lambda m: m["kernels"][0]["attrs"].__setitem__(5, 1 | 8), "contradict")            # ntl without the flag
+    broken(lambda m: m["kernels"][0].__setitem__("name", "reef_gemm_nt_32x32k4#0"), "contradict")
+    broken(lambda m: m["kernels"][0]["attrs"].__setitem__(17, 4), "without offset")           # offA
+    broken(lambda m: m["storage"][m["kernels"][0]["args"][4]].__setitem__("size", 40 * 95), "residual")
+    broken(lambda m: m["storage"][m["kernels"][0]["args"][5]].__setitem__("size", 199), "gamma")
+    broken(lambda m: m["storage"][m["kernels"][0]["args"][7]].__setitem__("size", 39 * 200), "normalised A")

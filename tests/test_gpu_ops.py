@@ -523,3 +523,73 @@ def test_mobilenetv2_with_and_without_the_fused_front_half(tmp_path):
     assert outs[0][0] == 55 and outs[1][0] == 40
     from tests.helpers import max_rel_err, REL_TOL
     assert max_rel_err(outs[1][1], outs[0][1]) <= REL_TOL
+
+
+@pytest.mark.parametrize("tile", list(MB.GraphBuilder.LN_GEMM_TILES))
+def test_gemm_reading_its_rows_through_a_layernorm(tmp_path, tile):
+    """reef_gemm_ntl_<tile>: C = act(LayerNorm(A) B^T + bias) (+ residual) and the normalised rows
+    written beside it -- ragged M, N and K (K = 200: one full 128-wide step and a partial one; 50
+    float4s per row do not divide among the threads of a row), rows far from zero mean; against
+    the oracle's two-pass LayerNorm followed by its product, and the written rows against the
+    LayerNorm kernel's own output."""
+    seq, hid, n = 45, 200, 3 * 200 + 8
+    g = MB.GraphBuilder("gl", weight_std=0.05)
+    x = g.input("x", (seq, hid))
+    r = g.input("r", (seq, n))
+    w = g.param((n, hid), 0.05)
+    bias = g.param((n,), 0.02)
+    gamma, beta = g.layernorm_params(hid)
+    n1 = g.temp((seq, hid))
+    g.gemm(x, w, seq, n, hid, trans_b=True, bias=bias, act=MB.ACT_GELU, force_tile=tile, res=r,
+           ln=dict(gamma=gamma, beta=beta, out=n1))
+    g.gemm(x, w, seq, n, hid, trans_b=True, alpha=0.5, force_tile=tile, ln=dict(gamma=gamma, beta=beta, eps=1e-5))
+    g.gemm(x, w, seq, n, hid, trans_b=True, force_tile=tile, res=r, ln=dict(gamma=gamma, beta=beta))
+    sep = g.layernorm(x, seq, hid, gamma=gamma, beta=beta)
+    g.mark_output(sep)
+    assert [k["name"].split("#")[0] for k in g.kernels[:3]] == ["reef_gemm_ntl_" + tile] * 3
+    exe, orc, model = run_both(g, tmp_path, {"x": 30.0 + 2.0 * rnd(seq, hid), "r": rnd(seq, n)})
+    compare_storages(exe, orc, model, what="layernorm gemm " + tile)
+    from tests.helpers import max_rel_err, REL_TOL
+    got = exe.get_data(n1.idx, seq * hid)
+    assert max_rel_err(got, exe.get_data(sep.idx, seq * hid)) <= REL_TOL
+
+
+@pytest.mark.parametrize("tile,trans_b", [("16x32k4", True), ("32x32d4", True), ("32x32k4", True), ("64x64", True),
+                                          ("64x64", False), ("32x128", False)])
+def test_gemm_adds_a_residual_behind_the_activation(tmp_path, tile, trans_b):
+    """C = act(A B + bias) + R, with R laid out as C is: a column block of a wider tensor, batched."""
+    seq, hid, heads = 40, 200, 5
+    hd = hid // heads
+    g = MB.GraphBuilder("gr", weight_std=0.05)
+    x = g.input("x", (seq, hid))
+    r = g.input("r", (seq, 2 * hid))
+    w = g.param((hid, hid), 0.05)
+    bias = g.param((hid,), 0.02)
+    out = g.temp((seq, 2 * hid))
+    # the right half of `out` = gelu(x w + bias) + the right half of r
+    g.gemm(x, w, seq, hid, hid, trans_b=trans_b, bias=bias, act=MB.ACT_GELU, ldc=2 * hid, off_c=hid, out=out,
+           res=r, force_tile=tile)
+    # per head: C[b] = x_b (w_b)^T or x_b w_b + r_b, heads as column blocks of the left half
+    g.gemm(x, w, seq, hd, hd, batch=heads, trans_b=trans_b, lda=hid, ldb=hid, ldc=2 * hid, stride_a=hd,
+           stride_b=hd, stride_c=hd, out=out, res=r, force_tile=tile)
+    g.mark_output(out)
+    exe, orc, model = run_both(g, tmp_path, {"x": rnd(seq, hid), "r": rnd(seq, 2 * hid)})
+    compare_storages(exe, orc, model, what="gemm with residual " + tile)
+
+
+def test_bert_with_and_without_the_layernorm_inside_the_projection(tmp_path):
+    """Three BERT layers with the LayerNorms folded into the projections behind them hold, in the
+    encoder output, what the network with a LayerNorm launch each holds, to 1e-4; both against
+    the oracle in every storage."""
+    from reef_amd.modelgen import nets
+    from tests.helpers import max_rel_err, REL_TOL
+    ids = nets.token_input("bert3", 128, 30522)
+    outs = []
+    for fuse in (False, True):
+        g = nets.bert(layers=3, name="bert3", fuse_layernorm=fuse)
+        exe, orc, model = run_both(g, tmp_path / str(fuse), {"input0": ids})
+        compare_storages(exe, orc, model, what="bert3 fuse=%s" % fuse)
+        oi = model["kernels"][-1]["args"][3]
+        outs.append((len(g.kernels), exe.get_data(oi, 128 * 768)))
+    assert outs[0][0] == 2 + 3 * 7 and outs[1][0] == 2 + 3 * 5
+    assert max_rel_err(outs[1][1], outs[0][1]) <= REL_TOL
