@@ -381,13 +381,22 @@ enum { REEF_TR_D0 = 0, REEF_TR_D1, REEF_TR_D2, REEF_TR_FLAGS, REEF_TR_NATTR };
 #define REEF_GEMM_F_LN 2
 #define REEF_GEMM_F_LN_OUT 4
 #define REEF_GEMM_F_RES 8
+#define REEF_GEMM_F_PAIR_FOLD 16
+/* K split across workgroups (reef_gemm_ntd_<tile>, batch 1; attrs split_k > 1, k_chunk a multiple
+ * of 128): tasks = split_k * m_tiles * n_tiles, the split_k workgroups of a tile neighbours in
+ * the task order.  The partial tiles meet inside the launch as those of the direct convolutions
+ * do: ptr gets two more operands behind the optional ones, a workspace of split_k regions of
+ * M x N floats and the model's arrival counters (sync_off: first counter of this launch, one per
+ * output tile); with REEF_GEMM_F_PAIR_FOLD (split_k = 2) the workspace has a third region, the
+ * pair slots, zero at rest, and launches that always run to completion exchange through them. */
 enum {
     REEF_GEMM_BATCH = 0, REEF_GEMM_M, REEF_GEMM_N, REEF_GEMM_K, REEF_GEMM_TRANS_B,
     REEF_GEMM_FLAGS, REEF_GEMM_ACT, REEF_GEMM_ALPHA_BITS, REEF_GEMM_TILE, REEF_GEMM_M_TILES,
     REEF_GEMM_N_TILES, REEF_GEMM_LDA, REEF_GEMM_LDB, REEF_GEMM_LDC, REEF_GEMM_STRIDE_A,
     REEF_GEMM_STRIDE_B, REEF_GEMM_STRIDE_C, REEF_GEMM_OFF_A, REEF_GEMM_OFF_B, REEF_GEMM_OFF_C,
     REEF_GEMM_NATTR,
-    REEF_GEMM_LN_EPS_BITS = REEF_GEMM_NATTR      /* reef_gemm_ntl_* only */
+    REEF_GEMM_LN_EPS_BITS = REEF_GEMM_NATTR,     /* reef_gemm_ntl_* only */
+    REEF_GEMM_SPLIT_K, REEF_GEMM_K_CHUNK, REEF_GEMM_SYNC_OFF      /* absent or 0: no split */
 };
 
 /* ---- add / multiply (the reference's mocked model): ptr: a, b, out; no attrs ---- */

@@ -213,6 +213,22 @@ void gemm(const std::string& symbol, const Attrs& a, Needs& n) {
         if (fl & REEF_GEMM_F_LN_OUT) n.f32("normalised A", (M - 1) * a[REEF_GEMM_LDA] + K);
     }
     n.tasks = a[REEF_GEMM_BATCH] * a[REEF_GEMM_M_TILES] * a[REEF_GEMM_N_TILES];
+    // K split across workgroups, folded inside the launch: the direct kernels only
+    const i64 split = a[REEF_GEMM_SPLIT_K];
+    if (split < 0 || split == 1) { n.bad = "a split of K is 0 (none) or at least 2"; return; }
+    if ((fl & REEF_GEMM_F_PAIR_FOLD) && split != 2) { n.bad = "the pair fold is for a split of two"; return; }
+    if (split > 1) {
+        const i64 chunk = a[REEF_GEMM_K_CHUNK];
+        if (symbol.compare(0, 14, "reef_gemm_ntd_") != 0 || b1 != 0) { n.bad = "only the direct kernels split K, and only without a batch"; return; }
+        if (chunk <= 0 || chunk % 128 != 0 || chunk * split < K || chunk * (split - 1) >= K) {
+            n.bad = "the K chunks are not multiples of 128 that cover K without an empty one";
+            return;
+        }
+        if (a[REEF_GEMM_SYNC_OFF] < 0) { n.bad = "negative counter offset"; return; }
+        n.f32("split-K workspace", (split + ((fl & REEF_GEMM_F_PAIR_FOLD) ? 1 : 0)) * M * N);
+        n.raw("arrival counters", 4 * (a[REEF_GEMM_SYNC_OFF] + a[REEF_GEMM_M_TILES] * a[REEF_GEMM_N_TILES]));
+        n.tasks *= split;
+    }
     if (n.tasks >= kDivSmallLimit) n.bad = "4 Mi workgroups or more (the kernels' index arithmetic is exact below that)";
 }
 

@@ -1649,8 +1649,12 @@ __device__ __forceinline__ bool gemm_nt_direct_body(const ReefOpDesc& d, int tas
     const int M = a[REEF_GEMM_M], N = a[REEF_GEMM_N], K = a[REEF_GEMM_K];
     const int n_tiles = a[REEF_GEMM_N_TILES];
     const int tiles = a[REEF_GEMM_M_TILES] * n_tiles;
-    const int b = div_small(task, tiles);
-    const int rem = task - b * tiles;
+    // K split across workgroups (batch 1): the split_k workgroups of a tile are neighbours in the task order
+    const int split_k = a[REEF_GEMM_SPLIT_K] > 1 ? a[REEF_GEMM_SPLIT_K] : 1;
+    const int tile_task = split_k > 1 ? div_small(task, split_k) : task;
+    const int split = task - tile_task * split_k;
+    const int b = div_small(tile_task, tiles);
+    const int rem = tile_task - b * tiles;
     const int mt = div_small(rem, n_tiles), nt = rem - mt * n_tiles;
     const int m0 = mt * TD::BM, n0 = nt * TD::BN;
     const unsigned lda = (unsigned)a[REEF_GEMM_LDA], ldb = (unsigned)a[REEF_GEMM_LDB],
@@ -1684,9 +1688,11 @@ __device__ __forceinline__ bool gemm_nt_direct_body(const ReefOpDesc& d, int tas
         }
     }
 
-    const int lane_k = (wave * 4 + kq) * 8;          // first k of this lane's slot
-    const int nsteps = (K + 127) / 128;
-    const int lane_steps = lane_k < K ? (K - lane_k + 127) / 128 : 0;
+    const int k_lo = split_k > 1 ? split * a[REEF_GEMM_K_CHUNK] : 0;        // this workgroup's part of K
+    const int k_hi = split_k > 1 ? min(K, k_lo + a[REEF_GEMM_K_CHUNK]) : K;
+    const int lane_k = k_lo + (wave * 4 + kq) * 8;   // first k of this lane's slot
+    const int nsteps = (k_hi - k_lo + 127) / 128;
+    const int lane_steps = lane_k < k_hi ? (k_hi - lane_k + 127) / 128 : 0;
     unsigned va[TM], vb[TN];
 #pragma unroll
     for (int h = 0; h < TM; ++h) va[h] = ((unsigned)(m0 + 16 * h + i16) * lda + (unsigned)lane_k) * 4u;
@@ -1780,16 +1786,105 @@ __device__ __forceinline__ bool gemm_nt_direct_body(const ReefOpDesc& d, int tas
     constexpr int WSTRIDE = TD::SUBS * TD::PART;
     const float alpha = __int_as_float(a[REEF_GEMM_ALPHA_BITS]);
     const int act = a[REEF_GEMM_ACT];
+    auto finish = [&](float sum, int h, int g) {
+        float v = sum * alpha + e_bias[g];
+        if (act == REEF_ACT_RELU) v = fmaxf(v, 0.0f);
+        else if (act == REEF_ACT_GELU) v = gelu_erf(v);
+        buf_store(rs_c, ooff[h][g], v + e_res[h][g]);
+    };
+    float v[TM][TN];
 #pragma unroll
     for (int h = 0; h < TM; ++h)
 #pragma unroll
         for (int g = 0; g < TN; ++g) {
             const float* e = mine + (h * TN + g) * TD::PART;
-            float v = (((e[0] + e[WSTRIDE]) + e[2 * WSTRIDE]) + e[3 * WSTRIDE]) * alpha + e_bias[g];
-            if (act == REEF_ACT_RELU) v = fmaxf(v, 0.0f);
-            else if (act == REEF_ACT_GELU) v = gelu_erf(v);
-            buf_store(rs_c, ooff[h][g], v + e_res[h][g]);
+            v[h][g] = ((e[0] + e[WSTRIDE]) + e[2 * WSTRIDE]) + e[3 * WSTRIDE];
         }
+    if (split_k == 1) {
+#pragma unroll
+        for (int h = 0; h < TM; ++h)
+#pragma unroll
+            for (int g = 0; g < TN; ++g) finish(v[h][g], h, g);
+        return true;
+    }
+
+    // The split_k partial tiles of an output tile meet inside the launch, as those of the direct
+    // convolutions do: a split of two through one exchange per element where every launch on the
+    // buffers runs to completion, otherwise partial tiles to the workspace, a count per tile,
+    // and the last arrival sums them in split order.  The sums and their order are the same.
+    // ptr: .., workspace (split_k [+1] regions of M x N), arrival counters.
+    const int aux = 3 + (has_bias ? 1 : 0) + (has_res ? 1 : 0);
+    const size_t MN = (size_t)M * N;
+    float* ws = (float*)d.ptr[aux];
+    unsigned widx[TM][TN];         // element m * N + n of a dense M x N region, ~0u outside the matrix
+#pragma unroll
+    for (int h = 0; h < TM; ++h)
+#pragma unroll
+        for (int g = 0; g < TN; ++g) {
+            const unsigned m = (unsigned)(m0 + 16 * h + orow), n = (unsigned)(n0 + 16 * g + ocol);
+            widx[h][g] = (m < (unsigned)M && n < (unsigned)N) ? m * (unsigned)N + n : ~0u;
+        }
+    if (split_k == 2 && (a[REEF_GEMM_FLAGS] & REEF_GEMM_F_PAIR_FOLD) && poll.pair_fold_ok()) {
+        // a value is parked with its sign bit flipped, so a parked value is never the empty slot's 0
+        unsigned* slots = (unsigned*)(ws + 2 * MN);
+        unsigned got[TM][TN];
+#pragma unroll
+        for (int h = 0; h < TM; ++h)
+#pragma unroll
+            for (int g = 0; g < TN; ++g) {
+                got[h][g] = 0;
+                if (widx[h][g] != ~0u) {
+                    unsigned parked = __float_as_uint(v[h][g]) ^ 0x80000000u;
+                    parked = parked ? parked : 0x80000000u;
+                    got[h][g] = __hip_atomic_exchange(&slots[widx[h][g]], parked, __ATOMIC_RELAXED,
+                                                      __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+#pragma unroll
+        for (int h = 0; h < TM; ++h)
+#pragma unroll
+            for (int g = 0; g < TN; ++g)
+                if (got[h][g] != 0) {   // second to arrive: the other half is here
+                    const float other = __uint_as_float(got[h][g] ^ 0x80000000u);
+                    finish(split == 0 ? v[h][g] + other : other + v[h][g], h, g);   // split order
+                    __hip_atomic_store(&slots[widx[h][g]], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+        return true;
+    }
+    int* counters = (int*)d.ptr[aux + 1] + a[REEF_GEMM_SYNC_OFF];
+    int* s_last = sflag + 1;
+#pragma unroll
+    for (int h = 0; h < TM; ++h)
+#pragma unroll
+        for (int g = 0; g < TN; ++g)
+            if (widx[h][g] != ~0u) store_agent(ws + (size_t)split * MN + widx[h][g], v[h][g]);
+    partial_stores_done();   // every store of this workgroup is acknowledged before it counts in
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int old = __hip_atomic_fetch_add(&counters[rem], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *s_last = (old == split_k - 1);
+    }
+    __syncthreads();
+    if (!*s_last) return true;
+#pragma unroll
+    for (int h = 0; h < TM; ++h)
+#pragma unroll
+        for (int g = 0; g < TN; ++g)
+            if (widx[h][g] != ~0u) {
+                const float* src = ws + widx[h][g];
+                float sum = 0.0f;
+                for (int s0 = 0; s0 < split_k; s0 += 4) {
+                    float p[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) p[j] = load_agent(src + (size_t)min(s0 + j, split_k - 1) * MN);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (s0 + j < split_k) sum = (s0 + j == 0) ? p[j] : sum + p[j];
+                }
+                finish(sum, h, g);
+            }
+    if (threadIdx.x == 0)  // ready for the next run
+        __hip_atomic_store(&counters[rem], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return true;
 }
 

@@ -497,9 +497,11 @@ class GraphBuilder:
 
     def gemm(self, a, b, M, N, K, batch=1, trans_b=True, bias=None, act=ACT_NONE, alpha=1.0,
              lda=None, ldb=None, ldc=None, stride_a=0, stride_b=0, stride_c=0, out=None, force_tile=None,
-             off_a=0, off_b=0, off_c=0, ln=None, res=None):
+             off_a=0, off_b=0, off_c=0, ln=None, res=None, split_k=None):
         """C[b] = act(alpha * A[b] x B[b] (+bias)) (+res[b]); operands are storages with explicit strides.
         res: a residual laid out as C is.
+        split_k: K split across workgroups and folded inside the launch (direct tiles, batch 1);
+        None = what tiling.choose_gemm finds (1 or 2).
         force_tile: a staged tile name or, for trans_b, one of tiling.GEMM_DIRECT_TILES.
         off_a / off_b / off_c: element at which the first matrix starts inside its storage.
         ln: dict(gamma=, beta=, eps=1e-12, out=None) -- A is read through a LayerNorm of its rows,
@@ -533,6 +535,22 @@ class GraphBuilder:
         if res is not None:
             flags |= 8
             args.append(res.idx)
+        attrs_split = []
+        tasks = batch * t["m_tiles"] * t["n_tiles"]
+        if split_k is None:
+            split_k = t.get("gemm_split", 1)
+        if split_k > 1:
+            assert direct and batch == 1, "only the direct tiles split K, and only without a batch"
+            k_chunk = math.ceil(math.ceil(K / split_k) / 128) * 128
+            split_k = math.ceil(K / k_chunk)
+        if split_k > 1:
+            pair = split_k == 2 and self.pair_fold
+            ws = self.workspace((split_k + (1 if pair else 0)) * M * N)
+            sync_idx, sync_off = self._sync_counters(t["m_tiles"] * t["n_tiles"])
+            args += [ws.idx, sync_idx]
+            flags |= 16 if pair else 0
+            attrs_split = [split_k, k_chunk, sync_off]
+            tasks *= split_k
         attrs_ln = []
         if ln is not None:
             flags |= 2
@@ -547,10 +565,10 @@ class GraphBuilder:
         if trans_b:
             assert ldb % 4 == 0 and stride_b % 4 == 0, "gemm operands must be 16-byte aligned"
         self._emit("reef_gemm_%s_%s" % ("ntl" if ln is not None else "ntd" if direct else "nt" if trans_b else "nn", t["tile"]),
-                   batch * t["m_tiles"] * t["n_tiles"], args,
+                   tasks, args,
                    [batch, M, N, K, 1 if trans_b else 0, flags, act, float_bits(alpha), t["tile_id"],
                     t["m_tiles"], t["n_tiles"], lda, ldb, ldc, stride_a, stride_b, stride_c,
-                    off_a, off_b, off_c] + attrs_ln,
+                    off_a, off_b, off_c] + ((attrs_ln or [0]) + attrs_split if attrs_split else attrs_ln),
                    "gemm", flops, 4 * batch * (M * K + N * K + M * N), t["est_us"])
         return out
 

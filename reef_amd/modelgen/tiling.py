@@ -55,24 +55,36 @@ GEMM_DIRECT_TILES = ("16x16k4", "16x32k4", "32x32d4")   # reef_gemm_ntd_<tile>
 
 
 def choose_gemm(M, N, K, batch=1, direct_ok=False):
-    """Tile of a GEMM.  Without a measured table: the staged choice of the analytic model,
-    against the direct tiles (both operands K-contiguous) scored by the rule the batch-1
-    convolutions were found to follow -- a workgroup's time grows with the cache lines it has to
-    pull in, (BM + BN) K / 32 of them, and workgroups beyond one per CU queue up."""
+    """Tile of a GEMM, and for a direct tile whether K is split in two across workgroups.
+    Without a measured table: the staged choice of the analytic model, against the direct tiles
+    (both operands K-contiguous) scored by the rule the batch-1 convolutions were found to
+    follow -- a workgroup's time grows with the cache lines it has to pull in, (BM + BN) K / 32
+    of them, and workgroups beyond one per CU queue up.  A split of two (folded inside the
+    launch through the pair slots) halves a workgroup's lines and doubles the workgroups, at a
+    price measured on BERT-base's 128 x 768 x 3072 product (32x32d4: 25.8 us whole, 16.8 us
+    split in two, against 19.4 us for 16x32k4 whole; splits of three and more meet on counters
+    and were slower throughout)."""
     staged = choose(M, N, K, allow_split=False, tiles=GEMM_TILES)
     if not direct_ok:
         return staged
 
-    def cost(bm, bn):
-        wgs = batch * math.ceil(M / bm) * math.ceil(N / bn)
-        return math.ceil(wgs / NUM_CUS) * (bm + bn) * K / 32.0
-    best = min(GEMM_DIRECT_TILES, key=lambda t: (cost(TILES[t][1], TILES[t][2]), -TILES[t][1] * TILES[t][2]))
+    def cost(bm, bn, split=1):
+        wgs = batch * math.ceil(M / bm) * math.ceil(N / bn) * split
+        return math.ceil(wgs / NUM_CUS) * (bm + bn) * (K / split) / 32.0 + (GEMM_PAIR_FOLD_LINES if split == 2 else 0)
+    cands = [(t, 1) for t in GEMM_DIRECT_TILES]
+    if batch == 1 and K >= 1024:
+        cands += [(t, 2) for t in GEMM_DIRECT_TILES]
+    best, split = min(cands, key=lambda c: (cost(TILES[c[0]][1], TILES[c[0]][2], c[1]), c[1],
+                                            -TILES[c[0]][1] * TILES[c[0]][2]))
     _, bm, bn, _, _ = TILES[staged["tile"]]
-    if cost(bm, bn) * GEMM_STAGED_BONUS <= cost(TILES[best][1], TILES[best][2]):
+    if cost(bm, bn) * GEMM_STAGED_BONUS <= cost(TILES[best][1], TILES[best][2], split):
         return staged
-    return forced(best, M, N, K, 1)
+    t = forced(best, M, N, K, 1)
+    t["gemm_split"] = split
+    return t
 
 
+GEMM_PAIR_FOLD_LINES = 900.0    # what a split of two costs, in the cost rule's cache lines
 GEMM_STAGED_BONUS = 1.0
 
 

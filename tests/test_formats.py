@@ -296,8 +296,11 @@ def test_gemm_tile_choice_follows_the_line_rule():
     cache lines, (BM + BN) K / 32 times the workgroups queued per CU, is shorter than the staged
     tile's, and never without K-contiguous, 16-byte aligned operands."""
     from reef_amd.modelgen import tiling
-    assert tiling.choose_gemm(128, 768, 768, 1, True)["tile"] == "16x32k4"       # projections
-    assert tiling.choose_gemm(128, 768, 3072, 1, True)["tile"] == "16x32k4"      # FFN down
+    t = tiling.choose_gemm(128, 768, 768, 1, True)                               # projections
+    assert (t["tile"], t["gemm_split"]) == ("16x32k4", 1)
+    t = tiling.choose_gemm(128, 768, 3072, 1, True)              # FFN down: the long K split in two
+    assert (t["tile"], t["gemm_split"]) == ("32x32d4", 2)
+    assert tiling.choose_gemm(12 * 128, 128, 3072, 12, True).get("gemm_split", 1) == 1    # a batch never splits
     assert tiling.choose_gemm(128, 3072, 768, 1, True)["tile"] == "32x32k4"      # FFN up: staged
     assert tiling.choose_gemm(128, 768, 768, 1, False)["tile"] in tiling.GEMM_TILES
     for t in tiling.GEMM_DIRECT_TILES:
@@ -543,3 +546,35 @@ def test_a_product_behind_a_layernorm_is_checked_against_its_storages(tmp_path):
     broken(lambda m: m["storage"][m["kernels"][0]["args"][4]].__setitem__("size", 40 * 95), "residual")
     broken(lambda m: m["storage"][m["kernels"][0]["args"][5]].__setitem__("size", 199), "gamma")
     broken(lambda m: m["storage"][m["kernels"][0]["args"][7]].__setitem__("size", 39 * 200), "normalised A")
+
+
+def test_a_matrix_product_with_k_split_across_workgroups_is_checked(tmp_path):
+    """reef_gemm_ntd_<tile> with split_k: two more operands (workspace, counters), split_k times
+    the workgroups, chunks that are multiples of 128 and cover K."""
+    from reef_amd import binding as B
+    g = MB.GraphBuilder("splitfmt")
+    x = g.input("x", (40, 520))
+    w = g.param((96, 520), 0.05)
+    g.mark_output(g.gemm(x, w, 40, 96, 520, trans_b=True, force_tile="16x32k4", split_k=2))
+    base = g.write(str(tmp_path / "ok"), link_code_objects=False)
+    assert B.check_model(base + ".json") == (True, "")
+    model = json.load(open(base + ".json"))
+    k = model["kernels"][0]
+    assert k["attrs"][20:] == [0, 2, 384, 0] and k["attrs"][5] == 16 and len(k["args"]) == 5
+    assert k["launch_params"][0] == 2 * 3 * 3
+
+    def broken(change, reason):
+        m = json.loads(json.dumps(model))
+        change(m)
+        p = str(tmp_path / "broken.json")
+        json.dump(m, open(p, "w"))
+        ok, why = B.check_model(p)
+        assert not ok and reason in why, why
+
+    broken(lambda m: m["kernels"][0]["args"].pop(), "operands")
+    broken(lambda m: m["kernels"][0]["attrs"].__setitem__(22, 256), "cover K")
+    broken(lambda m: m["kernels"][0]["attrs"].__setitem__(22, 300), "multiples of 128")
+    broken(lambda m: m["kernels"][0]["attrs"].__setitem__(21, 3), "pair fold")
+    broken(lambda m: m["kernels"][0].__setitem__("name", "reef_gemm_nt_32x32k4#0"), "only the direct kernels")
+    broken(lambda m: m["kernels"][0]["launch_params"].__setitem__(0, 9), "workgroups")
+    broken(lambda m: m["storage"][m["kernels"][0]["args"][3]].__setitem__("size", 2 * 40 * 96 * 4), "workspace")

@@ -593,3 +593,51 @@ def test_bert_with_and_without_the_layernorm_inside_the_projection(tmp_path):
         outs.append((len(g.kernels), exe.get_data(oi, 128 * 768)))
     assert outs[0][0] == 2 + 3 * 7 and outs[1][0] == 2 + 3 * 5
     assert max_rel_err(outs[1][1], outs[0][1]) <= REL_TOL
+
+
+@pytest.mark.parametrize("split", [2, 3])
+@pytest.mark.parametrize("tile", list(tiling.GEMM_DIRECT_TILES))
+def test_gemm_direct_splits_k_across_workgroups(tmp_path, tile, split):
+    """reef_gemm_ntd_<tile> with K split over 2 or 3 workgroups per tile and folded inside the
+    launch (pair slots for a split of two where launches run to completion, arrival counters
+    otherwise): ragged M and N, K = 520 (chunks of 384 + 136 or 256 + 256 + 8), bias + GELU +
+    residual; against the oracle, the three flavours bit for bit, twice on one executor, pair
+    slots and counters empty afterwards."""
+    import json
+    import os
+    from reef_amd import binding as B
+    from tests.helpers import write_model
+    seq, hid, n = 40, 520, 200
+    g = MB.GraphBuilder("gs", weight_std=0.05)
+    x = g.input("x", (seq, hid))
+    r = g.input("r", (seq, n))
+    w = g.param((n, hid), 0.05)
+    bias = g.param((n,), 0.02)
+    y = g.gemm(x, w, seq, n, hid, trans_b=True, bias=bias, act=MB.ACT_GELU, res=r, force_tile=tile, split_k=split)
+    one = g.gemm(x, w, seq, n, hid, trans_b=True, bias=bias, act=MB.ACT_GELU, res=r, force_tile=tile, split_k=1)
+    g.mark_output(y)
+    k0 = g.kernels[0]
+    assert k0["attrs"][21] == split and k0["launch_params"][0] == split * g.kernels[1]["launch_params"][0]
+    assert bool(k0["attrs"][5] & 16) == (split == 2)
+    inputs = {"x": rnd(seq, hid), "r": rnd(seq, n)}
+    exe, orc, model = run_both(g, tmp_path, inputs)
+    compare_storages(exe, orc, model, what="split gemm %s x%d" % (tile, split))
+    want = exe.get_output()
+    from tests.helpers import max_rel_err, REL_TOL
+    assert max_rel_err(want, exe.get_data(one.idx, seq * n)) <= REL_TOL
+    d = write_model(g, tmp_path)
+    ws = model["kernels"][0]["args"][-2]
+    for kind, pre in ((B.TRANS, False), (B.HYBRID, True), (B.HYBRID, False), (B.HYBRID, True)):
+        e = B.Executor.from_dir(d, g.name, kind)
+        for name, arr in inputs.items():
+            e.set_input_checked(name, arr)
+        for _ in range(2):
+            e.execute_preemptable() if pre else e.execute()
+            np.testing.assert_array_equal(e.get_output(), want, err_msg="flavour %s %s" % (kind, pre))
+        words = e.get_data(ws, model["storage"][ws]["size"] // 4, np.int32)
+        if split == 2:
+            assert words.size == 3 * seq * n and not words[2 * seq * n:].any()
+        for i, s in enumerate(model["storage"]):
+            if s["name"] == "reef_sync":
+                assert not e.get_data(i, s["size"], np.int32).any()
+        e.close()
