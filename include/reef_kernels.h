@@ -373,7 +373,7 @@ enum { REEF_TR_D0 = 0, REEF_TR_D1, REEF_TR_D2, REEF_TR_FLAGS, REEF_TR_NATTR };
  * through a LayerNorm of its rows,
  *   A'[m][k] = (A[m][k] - mean[m]) / sqrt(var[m] + eps) * gamma[k] + beta[k]
  * (mean and variance over the K columns of the row), and C = act(alpha * A' x B^T (+bias)) (+R).
- * A and A' are [M][K] with leading dimension lda and no offset.
+ * A and A' are [M][K] with leading dimension lda and no offset; K <= 65536.
  * ptr: A, B, C, bias (optional), R (optional), gamma, beta, A' (REEF_GEMM_F_LN_OUT: the
  * normalised rows are written as well, a share by every workgroup of a row block).
  * attr: as above, then eps (float bits). */

@@ -208,6 +208,8 @@ void gemm(const std::string& symbol, const Attrs& a, Needs& n) {
     if (ln_kernel) {
         if (!trans_b || b1 != 0 || a[REEF_GEMM_OFF_A] != 0) { n.bad = "the LayerNorm form takes one K-contiguous B and A without offset"; return; }
         if (a.v.size() <= (size_t)REEF_GEMM_LN_EPS_BITS) { n.bad = "the LayerNorm form needs its epsilon"; return; }
+        // the kernel numbers the float4s of a row block (at most 128 rows) and divides those numbers
+        if (K > (1 << 16)) { n.bad = "the LayerNorm form takes rows of at most 65536 columns"; return; }
         n.f32("gamma", K);
         n.f32("beta", K);
         if (fl & REEF_GEMM_F_LN_OUT) n.f32("normalised A", (M - 1) * a[REEF_GEMM_LDA] + K);

@@ -543,6 +543,7 @@ def test_a_product_behind_a_layernorm_is_checked_against_its_storages(tmp_path):
     broken(lambda m: m["kernels"][0]["attrs"].__setitem__(5, 1 | 8), "contradict")            # ntl without the flag
     broken(lambda m: m["kernels"][0].__setitem__("name", "reef_gemm_nt_32x32k4#0"), "contradict")
     broken(lambda m: m["kernels"][0]["attrs"].__setitem__(17, 4), "without offset")           # offA
+    broken(lambda m: m["kernels"][0]["attrs"].__setitem__(3, 1 << 17), "65536")               # K
     broken(lambda m: m["storage"][m["kernels"][0]["args"][4]].__setitem__("size", 40 * 95), "residual")
     broken(lambda m: m["storage"][m["kernels"][0]["args"][5]].__setitem__("size", 199), "gamma")
     broken(lambda m: m["storage"][m["kernels"][0]["args"][7]].__setitem__("size", 39 * 200), "normalised A")
