@@ -369,13 +369,16 @@ enum { REEF_TR_D0 = 0, REEF_TR_D1, REEF_TR_D2, REEF_TR_FLAGS, REEF_TR_NATTR };
  *       one [tokens][3 * hidden] projection.
  * tasks = batch * m_tiles * n_tiles.
  *
- * reef_gemm_ntl_<tile> (staged tiles, trans_b = 1, batch 1, flags has REEF_GEMM_F_LN): A is read
- * through a LayerNorm of its rows,
+ * reef_gemm_ntl_<tile> (staged tiles, trans_b = 1, batch 1, flags has REEF_GEMM_F_LN): the product
+ * behind a LayerNorm of the rows of A,
  *   A'[m][k] = (A[m][k] - mean[m]) / sqrt(var[m] + eps) * gamma[k] + beta[k]
- * (mean and variance over the K columns of the row), and C = act(alpha * A' x B^T (+bias)) (+R).
+ * (mean and variance over the K columns of the row), C = act(alpha * A' x W^T (+bias)) (+R), computed
+ * as  alpha * (rstd[m] * (sum_k A[m][k] Wg[n][k] - mean[m] c1[n]) + c2[n])  from three tensors derived
+ * from the parameters: Wg[n][k] = gamma[k] W[n][k], c1[n] = sum_k Wg[n][k], c2[n] = sum_k beta[k] W[n][k].
  * A and A' are [M][K] with leading dimension lda and no offset; K <= 65536.
- * ptr: A, B, C, bias (optional), R (optional), gamma, beta, A' (REEF_GEMM_F_LN_OUT: the
- * normalised rows are written as well, a share by every workgroup of a row block).
+ * ptr: A, Wg, C, bias (optional), R (optional), c1, c2, gamma, beta, A' (REEF_GEMM_F_LN_OUT: the
+ * normalised rows are written as well, a share by every workgroup of a row block).  The storage
+ * of Wg is named <name of W's storage>gk; W itself stays a storage of the model.
  * attr: as above, then eps (float bits). */
 #define REEF_GEMM_F_BIAS 1
 #define REEF_GEMM_F_LN 2

@@ -415,13 +415,19 @@ class GraphOracle:
                 R = P[p][oC:]
                 p += 1
             if flags & 2:
-                # reef_gemm_ntl_*: A goes through a LayerNorm of its rows first (include/reef_kernels.h)
-                gamma, beta = P[p][:K], P[p + 1][:K]
+                # reef_gemm_ntl_*: LayerNorm of the rows of A, then the product with W -- the weights as
+                # the reference has them, which the model keeps under the name of the scaled copy
+                # without its "gk"; the scaled copy and the two vectors the kernel works from
+                # (include/reef_kernels.h) are not used here
+                gamma, beta = P[p + 2][:K], P[p + 3][:K]
                 rows = np.ascontiguousarray(np.lib.stride_tricks.as_strided(A, (M, K), (lda * 4, 4)))
                 normed = layernorm(rows, gamma, beta, None, _bits_to_float(a[20]))
                 if flags & 4:
-                    np.lib.stride_tricks.as_strided(P[p + 2], (M, K), (lda * 4, 4))[:, :] = normed
+                    np.lib.stride_tricks.as_strided(P[p + 4], (M, K), (lda * 4, 4))[:, :] = normed
                 A, lda = normed.reshape(-1), K
+                wname = self.model["storage"][k["args"][1]]["name"]
+                assert wname.endswith("gk"), wname
+                B = self.storage[[t["name"] for t in self.model["storage"]].index(wname[:-2])]
             for bi in range(batch):
                 Am = np.lib.stride_tricks.as_strided(A[bi * sA:], (M, K), (lda * 4, 4))
                 if trans_b:

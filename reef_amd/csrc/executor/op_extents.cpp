@@ -210,6 +210,8 @@ void gemm(const std::string& symbol, const Attrs& a, Needs& n) {
         if (a.v.size() <= (size_t)REEF_GEMM_LN_EPS_BITS) { n.bad = "the LayerNorm form needs its epsilon"; return; }
         // the kernel numbers the float4s of a row block (at most 128 rows) and divides those numbers
         if (K > (1 << 16)) { n.bad = "the LayerNorm form takes rows of at most 65536 columns"; return; }
+        n.f32("column sums of the scaled weights", N);
+        n.f32("weights times beta", N);
         n.f32("gamma", K);
         n.f32("beta", K);
         if (fl & REEF_GEMM_F_LN_OUT) n.f32("normalised A", (M - 1) * a[REEF_GEMM_LDA] + K);

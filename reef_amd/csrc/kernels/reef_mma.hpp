@@ -71,12 +71,9 @@ typedef Tile<1, 2, 1, 1, 2, 2> Tile32x64k2;
 
 // ---- A tile: rows of a K-contiguous matrix -------------------------------
 // VEC: rows are 16-byte aligned at every k that is a multiple of 4 (K % 4 == 0).
-// LN (reef_gemm_ntl_*): the matrix is read through a LayerNorm of its rows -- what goes into LDS
-// is (a - mean[row]) * rstd[row] * gamma[k] + beta[k], with the row statistics worked out
-// by the workgroup beforehand (gemm_body).  gamma and beta ride along with every load; the
-// arithmetic happens on the way into LDS, so the loads stay asynchronous.  (No store to memory in
-// here: loads and stores share one counter of outstanding operations, and a store in the K loop
-// makes every wait for a tile a wait for everything.)
+// LN (reef_gemm_ntl_*): the rows go into LDS as they are; on the way every thread adds what it
+// loads to per-row sums of (a - p) and (a - p)^2 around a pivot p (element 0 of the row), from
+// which gemm_body makes the row's mean and variance once the K loop has seen the whole row.
 template <class T, bool VEC, bool LN = false>
 struct ALoader {
     static constexpr int TPR = T::BK / 4;          // threads (float4s) per tile row
@@ -84,22 +81,18 @@ struct ALoader {
     static constexpr int NV = T::BM / RPP;         // float4 per thread per tile
     static_assert(NV >= 1, "tile shorter than one pass");
     static_assert(!LN || VEC, "the LayerNorm form loads whole float4s");
-    struct Regs { f32x4 v[NV]; f32x4 g, b; };
+    struct Regs { f32x4 v[NV]; float in; };     // in (LN): 1 for a float4 inside K, 0 for one outside
     rsrc_t rs;
     unsigned rowoff[NV];    // byte offset of the row (kOutside when the row is outside M)
     int k;                  // k of this thread's float4 in the next tile
     int k_end;
     // LN only
-    rsrc_t rs_g, rs_b;
-    float mean[LN ? NV : 1], rstd[LN ? NV : 1];
-    __device__ __forceinline__ void init_ln(const float* gamma, const float* beta, int K, const float* stats) {
-        rs_g = make_rsrc(gamma, (unsigned)K * 4u);
-        rs_b = make_rsrc(beta, (unsigned)K * 4u);
+    float pivot[LN ? NV : 1], s1[LN ? NV : 1], s2[LN ? NV : 1];
+    __device__ __forceinline__ void init_ln() {
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            const int r = threadIdx.x / TPR + RPP * i;     // row inside the tile
-            mean[LN ? i : 0] = stats[2 * r];
-            rstd[LN ? i : 0] = stats[2 * r + 1];
+            pivot[LN ? i : 0] = buf_load(rs, rowoff[i]);
+            s1[LN ? i : 0] = s2[LN ? i : 0] = 0.0f;
         }
     }
 
@@ -122,10 +115,7 @@ struct ALoader {
             const unsigned koff = k < k_end ? (unsigned)k * 4u : kOutside;
 #pragma unroll
             for (int i = 0; i < NV; ++i) r.v[i] = buf_load4(rs, rowoff[i] + koff);
-            if (LN) {
-                r.g = buf_load4(rs_g, koff);     // outside K: gamma = beta = 0, the value becomes 0
-                r.b = buf_load4(rs_b, koff);
-            }
+            if (LN) r.in = k < k_end ? 1.0f : 0.0f;
         } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -136,17 +126,22 @@ struct ALoader {
         }
         k += T::BK;
     }
-    __device__ __forceinline__ void store(const Regs& r, float* As) const {
+    __device__ __forceinline__ void store(const Regs& r, float* As) {
         const int tid = threadIdx.x;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            f32x4 v = r.v[i];
             if (LN) {
+                // no branch in here: a branch between a stage's loads and its LDS stores makes the wait
+                // for that stage a wait for every outstanding load, the next stage's included
+                const float pv = pivot[LN ? i : 0] * r.in;     // a float4 outside K was loaded as zeros: 0 - 0
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    v[e] = (v[e] - mean[LN ? i : 0]) * rstd[LN ? i : 0] * r.g[e] + r.b[e];
+                for (int e = 0; e < 4; ++e) {
+                    const float dl = r.v[i][e] - pv;
+                    s1[LN ? i : 0] += dl;
+                    s2[LN ? i : 0] = fmaf(dl, dl, s2[LN ? i : 0]);
+                }
             }
-            *(f32x4*)(As + (tid / TPR + RPP * i) * T::LDA + (tid % TPR) * 4) = v;
+            *(f32x4*)(As + (tid / TPR + RPP * i) * T::LDA + (tid % TPR) * 4) = r.v[i];
         }
     }
 };
@@ -1455,20 +1450,24 @@ __device__ __forceinline__ bool conv2d_xdw_body(const ReefOpDesc& d, int task, c
 // TRANS_B: B stored [N][K] (dense layers, Q.K^T) -- both operands take 128-bit row
 // loads, so K, lda, ldb and the batch strides must be multiples of 4 floats.
 // !TRANS_B: B stored [K][N] (P.V) -- element-wise B loads, 128-bit A loads.
-// LN_A (symbols reef_gemm_ntl_<tile>, REEF_GEMM_F_LN): A is read through a LayerNorm of its rows,
-// A' = LayerNorm(A) * gamma + beta (row statistics over all K columns).  A transformer layer
-// normalises and then multiplies: as two launches the normalised matrix makes a round trip
-// through memory behind a launch that only reads and writes 128 rows.  Here every workgroup works
-// out mean and 1 / sqrt(var + eps) of its own BM rows before its K loop -- all column tiles of a
-// row block do the same, on rows that are cache hits after the first -- and normalises on the
-// way into LDS.  The statistics are made in ONE pass over the row (a second pass would be a
-// second trip to memory, and a row held in registers between two passes takes the registers that
-// let two workgroups share a CU): every thread sums x - p and (x - p)^2 around a pivot p, the first
-// value it meets, which gives its own count, mean and sum of squared deviations; the threads of
-// a row merge these pairwise (Chan, Golub, LeVeque 1979), which is as stable as two passes.
-// The workgroups of a row block also write A', a share each (REEF_GEMM_F_LN_OUT: the operand of
-// the next residual).  A and A' are [M][K] with leading dimension lda and no offset; no batch.
-// ptr: A, B, C, bias (optional), residual (optional), then gamma, beta, A' (optional).
+// LN_A (symbols reef_gemm_ntl_<tile>, REEF_GEMM_F_LN): C = act(alpha LayerNorm(A) W^T + bias) (+ R),
+// LayerNorm(A)[m][k] = (A[m][k] - mean[m]) rstd[m] gamma[k] + beta[k].  A transformer layer
+// normalises and then multiplies; as two launches the normalised matrix makes a round trip
+// through memory behind a launch that only reads and writes 128 rows.  Normalising the rows on
+// the way into the tiles needs their statistics BEFORE the K loop -- a pass over the rows that
+// every column tile of a row block repeats (measured: 2.4 us of a 17 us kernel, plus 1.3 us
+// for gamma and beta riding along with every load).  The product is linear in the row, so the
+// normalisation moves behind the K loop instead:
+//     sum_k LN(A)[m][k] W[n][k] = rstd[m] (sum_k A[m][k] Wg[n][k] - mean[m] c1[n]) + c2[n]
+// with Wg[n][k] = gamma[k] W[n][k], c1[n] = sum_k Wg[n][k], c2[n] = sum_k beta[k] W[n][k], three
+// tensors the model generator derives from the parameters once.  The K loop is the plain
+// product A Wg^T; the A loader adds every value it moves to per-row sums around a pivot (the
+// workgroup sees each of its rows completely), the threads of a row merge them after the loop,
+// and the epilogue applies mean, rstd, c1 and c2.  The normalised rows themselves (the operand
+// of the next residual, REEF_GEMM_F_LN_OUT) are written by the workgroups of a row block, a
+// share each, from the statistics and a second look at their share of A.
+// A and A' are [M][K] with leading dimension lda and no offset; no batch.
+// ptr: A, Wg, C, bias (optional), residual (optional), c1, c2, gamma, beta, A' (optional).
 template <class T, bool TRANS_B, bool LN_A, class Poll>
 __device__ __forceinline__ bool gemm_body(const ReefOpDesc& d, int task, char* smem_raw,
                                           const Poll& poll) {
@@ -1491,94 +1490,59 @@ __device__ __forceinline__ bool gemm_body(const ReefOpDesc& d, int task, char* s
     bool ok;
     ALoader<T, true, LN_A> la;
     la.init(A, ((unsigned)(M - 1) * (unsigned)lda + (unsigned)K) * 4u, lda, m0, M, 0, K);
+    static_assert(!LN_A || TRANS_B, "the LayerNorm form exists for K-contiguous B");
+    const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
+    const WaveGeom<T> wg;
+    const int wm0 = wg.wm0, wn0 = wg.wn0;
+    const int fl = a[REEF_GEMM_FLAGS];
+    const float* bias = (fl & REEF_GEMM_F_BIAS) ? (const float*)d.ptr[3] : nullptr;
+    // the residual: laid out as C is (same leading dimension, offset and batch stride)
+    const float* R = (fl & REEF_GEMM_F_RES)
+                         ? (const float*)d.ptr[bias ? 4 : 3] + a[REEF_GEMM_OFF_C] + (size_t)b * a[REEF_GEMM_STRIDE_C]
+                         : nullptr;
+    const int lnp = 3 + (bias ? 1 : 0) + (R ? 1 : 0);      // LN_A: first of c1, c2, gamma, beta, A'
+    float e_c1[T::TN], e_c2[T::TN];
+    // LN_A with REEF_GEMM_F_LN_OUT: the normalised rows go to memory as well, a share per column
+    // tile -- the BM * K / 4 float4s of the row block in n_tiles contiguous runs (one workgroup
+    // writing it all would be the launch's straggler).  What a thread needs for the first float4
+    // of its share (the only one for rows of up to 256 n_tiles / BM float4s) is loaded here, ahead
+    // of the K loop, so that after the loop only arithmetic and a store are left.
+    float* Aout = nullptr;
+    int o_share = 0, o_end = 0, o_row4 = 1, o_r = 0;
+    unsigned o_off = kOutside, o_koff = kOutside;
+    f32x4 o_v, o_g, o_b;
+    rsrc_t rs_oa, rs_og, rs_ob;
     if (LN_A) {
-        static_assert(!LN_A || TRANS_B, "the LayerNorm form exists for K-contiguous B");
-        const int fl = a[REEF_GEMM_FLAGS];
-        int p = 3 + (fl & REEF_GEMM_F_BIAS ? 1 : 0) + (fl & REEF_GEMM_F_RES ? 1 : 0);
-        const float* gamma = (const float*)d.ptr[p++];
-        const float* beta = (const float*)d.ptr[p++];
-        float* Aout = (fl & REEF_GEMM_F_LN_OUT) ? (float*)d.ptr[p] : nullptr;
+        la.init_ln();
+        if (fl & REEF_GEMM_F_LN_OUT) Aout = (float*)d.ptr[lnp + 4];
         const unsigned bytes = ((unsigned)(M - 1) * (unsigned)lda + (unsigned)K) * 4u;
-        // kThreads / BM threads per row (neighbouring lanes), thread `spart` of a row on float4s
-        // spart, spart + TPRS, ..; UB of them per batch, the next batch in flight behind the current.
-        constexpr int TPRS = kThreads / T::BM, UB = 8;
-        static_assert(TPRS >= 1 && TPRS <= 64 && (TPRS & (TPRS - 1)) == 0, "threads per row: a power of two within a wavefront");
-        float* stats = smem + (T::LDS_BYTES / 4);          // behind the staging buffers: mean, rstd per row
-        const int srow = threadIdx.x / TPRS, spart = threadIdx.x % TPRS;
-        const rsrc_t rs1 = make_rsrc(A, bytes);
-        const unsigned roff = m0 + srow < M ? (unsigned)(m0 + srow) * (unsigned)lda * 4u : kOutside;
-        const int per_thread = (K / 4 + TPRS - 1) / TPRS;      // float4s of the busiest thread of a row
-        auto load_batch = [&](f32x4 (&v)[UB], int j0) {
-#pragma unroll
-            for (int u = 0; u < UB; ++u) {
-                const int k4 = (spart + (j0 + u) * TPRS) * 4;
-                v[u] = buf_load4(rs1, k4 < K ? roff + (unsigned)k4 * 4u : kOutside);
-            }
-        };
-        f32x4 cur[UB], nxt[UB];
-        load_batch(cur, 0);
-        const float pivot = cur[0][0];
-        float s1 = 0.0f, s2 = 0.0f, cnt = 0.0f;
-        for (int j0 = 0; j0 < per_thread; j0 += UB) {
-            if (j0 + UB < per_thread) load_batch(nxt, j0 + UB);
-#pragma unroll
-            for (int u = 0; u < UB; ++u) {
-                const bool in = (spart + (j0 + u) * TPRS) * 4 < K;
-                cnt += in ? 4.0f : 0.0f;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float dl = in ? cur[u][e] - pivot : 0.0f;
-                    s1 += dl;
-                    s2 = fmaf(dl, dl, s2);
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < UB; ++u) cur[u] = nxt[u];
-        }
-        // this thread's part of the row: count, mean, sum of squared deviations from that mean
-        float mean = cnt > 0.0f ? pivot + s1 / cnt : 0.0f;
-        float m2 = cnt > 0.0f ? s2 - s1 * (s1 / cnt) : 0.0f;
-#pragma unroll
-        for (int o = 1; o < TPRS; o <<= 1) {
-            const float cnt_o = __shfl_xor(cnt, o, 64), mean_o = __shfl_xor(mean, o, 64), m2_o = __shfl_xor(m2, o, 64);
-            const float tot = cnt + cnt_o, dm = mean_o - mean;
-            // symmetric in the two partners, so both hold the same bits afterwards
-            const float w_o = tot > 0.0f ? cnt_o / tot : 0.0f, w_s = tot > 0.0f ? cnt / tot : 0.0f;
-            mean = mean * w_s + mean_o * w_o;
-            m2 = (m2 + m2_o) + dm * dm * (tot > 0.0f ? (cnt * cnt_o) / tot : 0.0f);
-            cnt = tot;
-        }
-        const float rstd = 1.0f / sqrtf(fmaxf(m2, 0.0f) / (float)K + __int_as_float(a[REEF_GEMM_LN_EPS_BITS]));
-        if (spart == 0) {
-            stats[2 * srow] = mean;
-            stats[2 * srow + 1] = rstd;
-        }
-        __syncthreads();
-        if (Aout) {
-            // The normalised rows go to memory as well, a share per column tile: the BM * K / 4
-            // float4s of the row block in n_tiles contiguous runs (one or two per thread, in flight
-            // beside the first loads of the K loop; one workgroup writing it all would be the
-            // launch's straggler).
-            const rsrc_t rs_g = make_rsrc(gamma, (unsigned)K * 4u), rs_b = make_rsrc(beta, (unsigned)K * 4u);
-            const rsrc_t rs_o = make_rsrc(Aout, bytes);
-            const int row4 = K / 4, total = T::BM * row4;
-            const int share = (total + n_tiles - 1) / n_tiles;
-            const int end = (nt + 1) * share < total ? (nt + 1) * share : total;
-            for (int id = nt * share + (int)threadIdx.x; id < end; id += kThreads) {
-                const int r = div_small(id, row4), k4 = (id - r * row4) * 4;
-                if (m0 + r < M) {
-                    const unsigned off = ((unsigned)(m0 + r) * (unsigned)lda + (unsigned)k4) * 4u;
-                    const f32x4 v = buf_load4(rs1, off);
-                    const f32x4 gm = buf_load4(rs_g, (unsigned)k4 * 4u), bt = buf_load4(rs_b, (unsigned)k4 * 4u);
-                    const float mu = stats[2 * r], rs = stats[2 * r + 1];
-                    f32x4 y;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) y[e] = (v[e] - mu) * rs * gm[e] + bt[e];
-                    buf_store4(rs_o, off, y);
-                }
+        rs_oa = make_rsrc(A, Aout ? bytes : 0u);
+        rs_og = make_rsrc(d.ptr[lnp + 2], Aout ? (unsigned)K * 4u : 0u);
+        rs_ob = make_rsrc(d.ptr[lnp + 3], Aout ? (unsigned)K * 4u : 0u);
+        o_row4 = K / 4;
+        const int total = T::BM * o_row4;
+        o_share = (total + n_tiles - 1) / n_tiles;
+        o_end = (nt + 1) * o_share < total ? (nt + 1) * o_share : total;
+        const int id = nt * o_share + (int)threadIdx.x;
+        if (Aout && id < o_end) {
+            o_r = div_small(id, o_row4);
+            if (m0 + o_r < M) {
+                o_koff = (unsigned)(id - o_r * o_row4) * 16u;
+                o_off = (unsigned)(m0 + o_r) * (unsigned)lda * 4u + o_koff;
             }
         }
-        la.init_ln(gamma, beta, K, stats);
+        o_v = buf_load4(rs_oa, o_off);
+        o_g = buf_load4(rs_og, o_koff);
+        o_b = buf_load4(rs_ob, o_koff);
+        // c1 and c2 of this thread's output columns, on their way before the K loop
+        const float* c1 = (const float*)d.ptr[lnp];
+        const float* c2 = (const float*)d.ptr[lnp + 1];
+#pragma unroll
+        for (int tn = 0; tn < T::TN; ++tn) {
+            const int n = n0 + wn0 + tn * 32 + l32;
+            e_c1[tn] = n < N ? c1[n] : 0.0f;
+            e_c2[tn] = n < N ? c2[n] : 0.0f;
+        }
     }
     if (TRANS_B) {
         // B is [N][K]: stage it exactly like A (rows = n).
@@ -1592,17 +1556,55 @@ __device__ __forceinline__ bool gemm_body(const ReefOpDesc& d, int task, char* s
         ok = k_loop<T, false>(la, lb, nk, smem, acc, poll);
     }
     if (!ok) return false;
+    float* stats = smem + (T::LDS_BYTES / 4);      // LN_A: mean, rstd per row, behind the staging buffers
+    if (LN_A) {
+        // a row's sums: the TPR threads that loaded its float4s are neighbouring lanes
+        typedef ALoader<T, true, LN_A> LA;
+        const float eps = __int_as_float(a[REEF_GEMM_LN_EPS_BITS]);
+#pragma unroll
+        for (int i = 0; i < LA::NV; ++i) {
+            float t1 = la.s1[LN_A ? i : 0], t2 = la.s2[LN_A ? i : 0];
+#pragma unroll
+            for (int o = 1; o < LA::TPR; o <<= 1) {
+                t1 += __shfl_xor(t1, o, 64);
+                t2 += __shfl_xor(t2, o, 64);
+            }
+            if (threadIdx.x % LA::TPR == 0) {
+                const int r = threadIdx.x / LA::TPR + LA::RPP * i;
+                const float m1 = t1 / (float)K;                        // mean of a - pivot
+                const float var = fmaxf(t2 / (float)K - m1 * m1, 0.0f);
+                stats[2 * r] = la.pivot[LN_A ? i : 0] + m1;
+                stats[2 * r + 1] = 1.0f / sqrtf(var + eps);
+            }
+        }
+        __syncthreads();
+        if (Aout) {
+            const rsrc_t rs_o = make_rsrc(Aout, ((unsigned)(M - 1) * (unsigned)lda + (unsigned)K) * 4u);
+            {   // the float4 whose operands have been waiting since before the K loop
+                const float mu = stats[2 * o_r], rs = stats[2 * o_r + 1];
+                f32x4 y;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) y[e] = (o_v[e] - mu) * rs * o_g[e] + o_b[e];
+                buf_store4(rs_o, o_off, y);      // no share, or a row outside M: an offset outside the buffer
+            }
+            for (int id = nt * o_share + (int)threadIdx.x + kThreads; id < o_end; id += kThreads) {
+                const int r = div_small(id, o_row4), k4 = (id - r * o_row4) * 4;
+                if (m0 + r < M) {
+                    const unsigned off = ((unsigned)(m0 + r) * (unsigned)lda + (unsigned)k4) * 4u;
+                    const f32x4 v = buf_load4(rs_oa, off);
+                    const f32x4 gm = buf_load4(rs_og, (unsigned)k4 * 4u), bt = buf_load4(rs_ob, (unsigned)k4 * 4u);
+                    const float mu = stats[2 * r], rs = stats[2 * r + 1];
+                    f32x4 y;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) y[e] = (v[e] - mu) * rs * gm[e] + bt[e];
+                    buf_store4(rs_o, off, y);
+                }
+            }
+        }
+    }
     float res[T::TM][T::TN][T::RPW];
     const int r0 = finish_tile<T>(acc, res, smem);
 
-    const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
-    const WaveGeom<T> wg;
-    const int wm0 = wg.wm0, wn0 = wg.wn0;
-    const float* bias = (a[REEF_GEMM_FLAGS] & REEF_GEMM_F_BIAS) ? (const float*)d.ptr[3] : nullptr;
-    // the residual: laid out as C is (same leading dimension, offset and batch stride)
-    const float* R = (a[REEF_GEMM_FLAGS] & REEF_GEMM_F_RES)
-                         ? (const float*)d.ptr[bias ? 4 : 3] + a[REEF_GEMM_OFF_C] + (size_t)b * a[REEF_GEMM_STRIDE_C]
-                         : nullptr;
     const float alpha = __int_as_float(a[REEF_GEMM_ALPHA_BITS]);
     const int act = a[REEF_GEMM_ACT];
 #pragma unroll
@@ -1614,9 +1616,12 @@ __device__ __forceinline__ bool gemm_body(const ReefOpDesc& d, int task, char* s
 #pragma unroll
             for (int rr = 0; rr < T::RPW; ++rr) {
                 const int r = r0 + rr;
-                const int m = m0 + wm0 + tm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                const int ml = wm0 + tm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);     // row inside the tile
+                const int m = m0 + ml;
                 if (m < M && n < N) {
-                    float v = res[tm][tn][rr] * alpha + bv;
+                    float v = res[tm][tn][rr];
+                    if (LN_A) v = stats[2 * ml + 1] * (v - stats[2 * ml] * e_c1[tn]) + e_c2[tn];
+                    v = v * alpha + bv;
                     if (act == REEF_ACT_RELU) v = fmaxf(v, 0.0f);
                     else if (act == REEF_ACT_GELU) v = gelu_erf(v);
                     if (R) v += R[(size_t)m * ldc + n];

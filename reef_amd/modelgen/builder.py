@@ -61,6 +61,7 @@ class GraphBuilder:
         self.kernels = []
         self.graph_args = []
         self.params = []               # (key, float32 array)
+        self._param_pos = {}           # storage index of a parameter -> its place in params
         self.flops = 0                 # algorithmic FLOPs of contractions
         self.kernel_flops = []         # per kernel call
         self.kernel_bytes = []         # algorithmic bytes per kernel call
@@ -106,7 +107,22 @@ class GraphBuilder:
         idx = self._storage(key, n)
         self.graph_args.append(idx)
         self.params.append((key, arr))
+        self._param_pos[idx] = len(self.params) - 1
         return Tensor(idx, shape)
+
+    def param_array(self, t):
+        """The values of a parameter made by param() (as they stand now)."""
+        return self.params[self._param_pos[t.idx]][1]
+
+    def derived_param(self, key, arr):
+        """A tensor computed from parameters when the model is generated (its key ends in "k", as the
+        packed weight copies' do: readers that want the network's own parameters skip those)."""
+        assert key.endswith("k")
+        arr = np.ascontiguousarray(arr, np.float32).reshape(-1)
+        idx = self._storage(key, arr.size)
+        self.graph_args.append(idx)
+        self.params.append((key, arr))
+        return Tensor(idx, (arr.size,))
 
     def _sync_counters(self, n):
         """Reserves n counters in the model's sync storage; returns (storage idx, first counter)."""
@@ -504,9 +520,10 @@ class GraphBuilder:
         None = what tiling.choose_gemm finds (1 or 2).
         force_tile: a staged tile name or, for trans_b, one of tiling.GEMM_DIRECT_TILES.
         off_a / off_b / off_c: element at which the first matrix starts inside its storage.
-        ln: dict(gamma=, beta=, eps=1e-12, out=None) -- A is read through a LayerNorm of its rows,
-        and `out`, if given, receives the normalised rows (kernels reef_gemm_ntl_<tile>: staged
-        tiles, one K-contiguous B)."""
+        ln: dict(gamma=, beta=, eps=1e-12, out=None) -- the product behind a LayerNorm of the rows
+        of A; `out`, if given, receives the normalised rows (kernels reef_gemm_ntl_<tile>: staged
+        tiles, one K-contiguous B).  b, gamma and beta must be parameters: the kernel works from
+        b scaled by gamma and two vectors derived from them (include/reef_kernels.h)."""
         lda = K if lda is None else lda
         ldb = (K if trans_b else N) if ldb is None else ldb
         ldc = N if ldc is None else ldc
@@ -528,6 +545,17 @@ class GraphBuilder:
         direct = t["tile"] in tiling.GEMM_DIRECT_TILES
         assert direct_ok or not direct, "this GEMM has no direct form"
         args = [a.idx, b.idx, out.idx]
+        if ln is not None:
+            # Wg = W gamma (column k scaled by gamma[k]); c1 = its row sums; c2 = W beta
+            assert ldb == K and off_b == 0, "the LayerNorm form takes the weight matrix whole"
+            W = self.param_array(b).reshape(N, K).astype(np.float64)
+            gm = self.param_array(ln["gamma"]).astype(np.float64)
+            bt = self.param_array(ln["beta"]).astype(np.float64)
+            wkey = self.storage[b.idx]["name"]
+            Wg = (W * gm[None, :]).astype(np.float32)
+            args[1] = self.derived_param(wkey + "gk", Wg).idx      # the storage named wkey keeps W itself
+            ln = dict(ln, c1=self.derived_param(wkey + "sk", Wg.astype(np.float64).sum(axis=1)),
+                      c2=self.derived_param(wkey + "tk", W @ bt))
         flags = 0
         if bias is not None:
             flags = 1
@@ -554,7 +582,7 @@ class GraphBuilder:
         attrs_ln = []
         if ln is not None:
             flags |= 2
-            args += [ln["gamma"].idx, ln["beta"].idx]
+            args += [ln["c1"].idx, ln["c2"].idx, ln["gamma"].idx, ln["beta"].idx]
             if ln.get("out") is not None:
                 flags |= 4
                 args.append(ln["out"].idx)

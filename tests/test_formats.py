@@ -528,7 +528,17 @@ def test_a_product_behind_a_layernorm_is_checked_against_its_storages(tmp_path):
     assert B.check_model(base + ".json") == (True, "")
     model = json.load(open(base + ".json"))
     k = model["kernels"][0]
-    assert k["name"].startswith("reef_gemm_ntl_32x32k4") and len(k["args"]) == 8 and k["attrs"][5] == 1 | 2 | 4 | 8
+    # A, W gamma, C, bias, residual, c1, c2, gamma, beta, A'
+    assert k["name"].startswith("reef_gemm_ntl_32x32k4") and len(k["args"]) == 10 and k["attrs"][5] == 1 | 2 | 4 | 8
+    # the three derived tensors are what their definitions say
+    par = dict(g.params)
+    gm, bt = (par[model["storage"][k["args"][i]]["name"]].astype(np.float64) for i in (7, 8))
+    W = par[model["storage"][k["args"][1]]["name"][:-2]].astype(np.float64).reshape(96, 200)
+    Wg, c1, c2 = (par[model["storage"][k["args"][i]]["name"]] for i in (1, 5, 6))
+    np.testing.assert_array_equal(Wg.reshape(96, 200), (W * gm[None, :]).astype(np.float32))
+    np.testing.assert_allclose(c1, (W * gm[None, :]).sum(1), rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(c2, W @ bt, rtol=1e-6, atol=1e-7)
+    assert all(model["storage"][k["args"][i]]["name"].endswith("k") for i in (1, 5, 6))
 
     def broken(change, reason):
         m = json.loads(json.dumps(model))
@@ -545,8 +555,10 @@ def test_a_product_behind_a_layernorm_is_checked_against_its_storages(tmp_path):
     broken(lambda m: m["kernels"][0]["attrs"].__setitem__(17, 4), "without offset")           # offA
     broken(lambda m: m["kernels"][0]["attrs"].__setitem__(3, 1 << 17), "65536")               # K
     broken(lambda m: m["storage"][m["kernels"][0]["args"][4]].__setitem__("size", 40 * 95), "residual")
-    broken(lambda m: m["storage"][m["kernels"][0]["args"][5]].__setitem__("size", 199), "gamma")
-    broken(lambda m: m["storage"][m["kernels"][0]["args"][7]].__setitem__("size", 39 * 200), "normalised A")
+    broken(lambda m: m["storage"][m["kernels"][0]["args"][5]].__setitem__("size", 95), "column sums")
+    broken(lambda m: m["storage"][m["kernels"][0]["args"][7]].__setitem__("size", 199), "gamma")
+    broken(lambda m: m["storage"][m["kernels"][0]["args"][9]].__setitem__("size", 39 * 200), "normalised A")
+
 
 
 def test_a_matrix_product_with_k_split_across_workgroups_is_checked(tmp_path):

@@ -270,11 +270,11 @@ def test_load_generator_counts_and_outputs(fake, small_dirs):
         s.set_input(m, x, "data")
         bes.append(m)
     s.run()
-    r = s.run_load(rt_mid, bes, requests=12, warmup=3, mean_interval_us=25000.0, seed=7)
-    assert len(r["rt_latency_us"]) == 12
+    r = s.run_load(rt_mid, bes, requests=24, warmup=3, mean_interval_us=25000.0, seed=7)
+    assert len(r["rt_latency_us"]) == 24
     assert (r["rt_queue_us"] >= 0).all() and (r["rt_exec_us"] >= 0).all()
     np.testing.assert_allclose(r["rt_latency_us"], r["rt_queue_us"] + r["rt_exec_us"], atol=1e-3)
-    assert r["span_s"] > 12 * 0.005
+    assert r["span_s"] > 24 * 0.005
     assert r["be_completed"].sum() > 0 and (r["be_preempted"] <= r["be_completed"]).all()
     assert s.preempt_times() > 0
     ph = s.preempt_phases()
