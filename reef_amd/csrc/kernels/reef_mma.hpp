@@ -439,6 +439,11 @@ __device__ __forceinline__ bool k_loop(LA& la, LB& lb, int nk, float* smem, f32x
     for (int s = 0; s < D; ++s) {
         la.load(ra[s]);
         lb.load(rb[s]);
+        // Keep the stages' loads in this order: loads come back in the order they were issued, and the
+        // wait in front of a stage's LDS stores counts the loads issued after it.  If the compiler moves
+        // stage 1's loads in front of stage 0's here, the loop's first wait has to be a wait for
+        // everything, and since the loop has one wait for both ways into it, so has every later one.
+        asm volatile("" ::: "memory");
     }
     int pf = 0;
     int it = 0;
