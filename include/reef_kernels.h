@@ -225,11 +225,21 @@ enum {
  *                           of R (R > 1) or 8 (d1) and splits K on channel boundaries.
  *   reef_conv2d_r9_g<G>[m2] row form of the direct 3x3 / stride 1 / padding 1 convolution: every input value
  *                           is loaded once per tile and the horizontal taps come from neighbouring lanes. */
+#define REEF_F_POOL_OUTPUT 256  /* symbol reef_conv2d_sp7_g2: a 7x7 convolution (stride 2, padding 3, Cin <= 3; + bias,
+                                  activation ACT) and the 3x3 max-pool (stride 2, padding 1; + pool shift, activation
+                                  ACT2) behind it in one launch.  ptr: in, W, out, bias, then the input shift
+                                  (REEF_F_IN_SHIFT) and the pool's shift (REEF_F_POOL_SHIFT).  H, W: the input; HO, WO:
+                                  the POOLED output; KH = KW = 7, SH = SW = 2, PH = PW = 3; TILE = REEF_TILE_R9G2;
+                                  M_TILES = ceil(Cout / 16), N_TILES = ceil(HO / 2) * ceil(WO / 14); no split. */
+#define REEF_F_IN_SHIFT 512    /* with REEF_F_POOL_OUTPUT: the input is read as in + shift[c] inside the image (the
+                                  convolution's padding stays 0) */
+#define REEF_F_POOL_SHIFT 1024 /* with REEF_F_POOL_OUTPUT: out = act2(maxpool(..) + shift[channel]) */
 #define REEF_CONV_MODE_GENERAL 0
 #define REEF_CONV_MODE_POINTWISE 1
 #define REEF_CONV_MODE_UNALIGNED 2
 #define REEF_CONV_MODE_DIRECT 3
 #define REEF_CONV_MODE_DIRECT_PRE 4   /* direct, 1 tap, with REEF_F_PRE_ACT (reef_conv2d_p1_<tile>) */
+#define REEF_CONV_MODE_SP7 7          /* 7x7 stride-2 convolution + 3x3 stride-2 max-pool (reef_conv2d_sp7_g2, REEF_F_POOL_OUTPUT) */
 #define REEF_CONV_MODE_XDW 6          /* 1x1 filter + depthwise 3x3 behind it (reef_conv2d_xdw_g<G>, REEF_F_DW_OUTPUT) */
 #define REEF_CONV_MODE_ROWS 5         /* direct, row form: 3x3 / stride 1 / padding 1 (reef_conv2d_r9_g<G>[m2]).
                                          The output tile is 16 (m2: 32) channels x G image rows x one 14-column

@@ -314,6 +314,18 @@ class GraphOracle:
                 out = conv2d(mid, P[pos][:Cout * 9].reshape(Cout, 1, 3, 3), P[pos + 1][:Cout], stride=(sh, sw),
                              pad=(1, 1), groups=Cout, act=act2, acc64=acc64)
                 assert out.shape == (Cout, Ho, Wo)
+            elif flags & 256:
+                # a 3x3 / stride 2 / padding 1 max-pool behind the convolution in the same launch (Ho, Wo
+                # are the pooled sizes); optionally a per-channel shift on the input -- inside the image,
+                # the convolution's padding stays zero, as when the shift is a launch of its own -- and
+                # one behind the pool, with the pool's activation act2
+                pos = 3 + bool(flags & 1)
+                if flags & 512:
+                    xin = eltwise(xin.reshape(Cin, -1), shift=P[pos][:Cin]).reshape(Cin, H, W)
+                    pos += 1
+                mid = conv2d(xin, wgt, bias, None, None, None, (sh, sw), (ph, pw), 1, act, 6.0, acc64)
+                out = pool2d(mid, (3, 3), (2, 2), (1, 1), 0, P[pos][:Cout] if flags & 1024 else None, act2)
+                assert out.shape == (Cout, Ho, Wo)
             else:
                 out = conv2d(xin, wgt, bias,
                              None if res is None else res[:Cout * Ho * Wo].reshape(Cout, Ho, Wo),

@@ -73,9 +73,14 @@ void conv2d(const std::string& symbol, const Attrs& a, Needs& n) {
     }
     const i64 cin = a[REEF_CONV_CIN], H = a[REEF_CONV_H], W = a[REEF_CONV_W], M = a[REEF_CONV_COUT];
     const i64 Ho = a[REEF_CONV_HO], Wo = a[REEF_CONV_WO], kh = a[REEF_CONV_KH], kw = a[REEF_CONV_KW];
-    if (Ho != (H + 2 * a[REEF_CONV_PH] - kh) / a[REEF_CONV_SH] + 1 ||
-        Wo != (W + 2 * a[REEF_CONV_PW] - kw) / a[REEF_CONV_SW] + 1 || H + 2 * a[REEF_CONV_PH] < kh ||
-        W + 2 * a[REEF_CONV_PW] < kw) {
+    // the sizes a convolution gives; behind a fused 3x3 / stride 2 / padding 1 max-pool (sp7) the pooled ones
+    i64 want_ho = (H + 2 * a[REEF_CONV_PH] - kh) / a[REEF_CONV_SH] + 1;
+    i64 want_wo = (W + 2 * a[REEF_CONV_PW] - kw) / a[REEF_CONV_SW] + 1;
+    if (a[REEF_CONV_FLAGS] & REEF_F_POOL_OUTPUT) {
+        want_ho = (want_ho + 2 - 3) / 2 + 1;
+        want_wo = (want_wo + 2 - 3) / 2 + 1;
+    }
+    if (Ho != want_ho || Wo != want_wo || H + 2 * a[REEF_CONV_PH] < kh || W + 2 * a[REEF_CONV_PW] < kw) {
         n.bad = "the output size does not follow from input, filter, stride and padding";
         return;
     }
@@ -116,6 +121,17 @@ void conv2d(const std::string& symbol, const Attrs& a, Needs& n) {
                flags == (REEF_F_BIAS | REEF_F_DW_OUTPUT) && off == 0 && a[REEF_CONV_M_TILES] == cdiv(M, 16) &&
                a[REEF_CONV_N_TILES] == cdiv(Ho, G) * cdiv(Wo, 14) && a[REEF_CONV_ACT] <= REEF_ACT_RELU6 &&
                a[REEF_CONV_ACT2] <= REEF_ACT_RELU6;
+    } else if (fam == "sp7_g2") {
+        // 7x7 / stride 2 / padding 3 convolution of at most 3 channels and the 3x3 / stride 2 / padding 1
+        // max-pool behind it in one launch; HO, WO are the pooled sizes
+        mode = REEF_CONV_MODE_SP7;
+        fits = kh == 7 && kw == 7 && a[REEF_CONV_SH] == 2 && a[REEF_CONV_SW] == 2 && a[REEF_CONV_PH] == 3 &&
+               a[REEF_CONV_PW] == 3 && cin <= 3 && split == 1 && off == 0 && (flags & REEF_F_BIAS) &&
+               (flags & REEF_F_POOL_OUTPUT) &&
+               (flags & ~(i64)(REEF_F_BIAS | REEF_F_POOL_OUTPUT | REEF_F_IN_SHIFT | REEF_F_POOL_SHIFT)) == 0 &&
+               a[REEF_CONV_TILE] == REEF_TILE_R9G2 && a[REEF_CONV_M_TILES] == cdiv(M, 16) &&
+               a[REEF_CONV_N_TILES] == cdiv(Ho, 2) * cdiv(Wo, 14) && a[REEF_CONV_ACT] <= REEF_ACT_RELU6 &&
+               a[REEF_CONV_ACT2] <= REEF_ACT_RELU6;
     } else if (fam.compare(0, 3, "p1_") == 0) {
         mode = REEF_CONV_MODE_DIRECT_PRE;
         fits = unit && cin % 8 == 0 && (flags & REEF_F_PRE_ACT);
@@ -131,7 +147,9 @@ void conv2d(const std::string& symbol, const Attrs& a, Needs& n) {
         fits = compiled == taps && (taps > 1 || cin % 8 == 0);
     }
     if (!fits || mode != a[REEF_CONV_MODE] || ((flags & REEF_F_PRE_ACT) != 0) != (mode == REEF_CONV_MODE_DIRECT_PRE) ||
-        ((flags & REEF_F_DW_OUTPUT) != 0) != (mode == REEF_CONV_MODE_XDW)) {
+        ((flags & REEF_F_DW_OUTPUT) != 0) != (mode == REEF_CONV_MODE_XDW) ||
+        ((flags & REEF_F_POOL_OUTPUT) != 0) != (mode == REEF_CONV_MODE_SP7) ||
+        ((flags & (REEF_F_IN_SHIFT | REEF_F_POOL_SHIFT)) != 0 && mode != REEF_CONV_MODE_SP7)) {
         n.bad = "the layer is not one that this symbol's loader family was compiled for";
         return;
     }
@@ -150,6 +168,8 @@ void conv2d(const std::string& symbol, const Attrs& a, Needs& n) {
     if (flags & REEF_F_DUAL) { n.f32("second output", off + M * N); n.f32("second shift", M); }
     if (flags & REEF_F_PRE_ACT) { n.f32("input scale", cin); n.f32("input shift", cin); }
     if (flags & REEF_F_DW_OUTPUT) { n.f32("depthwise weights", M * 9); n.f32("depthwise bias", M); }
+    if (flags & REEF_F_IN_SHIFT) n.f32("input shift", cin);
+    if (flags & REEF_F_POOL_SHIFT) n.f32("pool shift", M);
     if (fused) {
         n.f32("partial sums", (split + ((flags & REEF_F_PAIR_FOLD) ? 1 : 0)) * M * N);
         n.raw("tile counters", 4 * (a[REEF_CONV_SYNC_OFF] + a[REEF_CONV_M_TILES] * a[REEF_CONV_N_TILES]));

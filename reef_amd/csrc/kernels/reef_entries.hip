@@ -62,6 +62,14 @@ struct OpConvXdw {
         return conv2d_xdw_body<G, S>(d, task, smem, p);
     }
 };
+// 7x7 stride-2 convolution and the 3x3 stride-2 max-pool behind it in one launch
+struct OpConvStemPool {
+    static constexpr int LDS = TileSp7::LDS_BYTES;
+    template <class P>
+    static __device__ __forceinline__ bool run(const ReefOpDesc& d, int task, char* smem, const P& p) {
+        return conv2d_stem_pool_body(d, task, smem, p);
+    }
+};
 template <class T, bool TRANS_B, bool LN_A = false>
 struct OpGemm {
     static constexpr int LDS = T::LDS_BYTES + (LN_A ? 2 * T::BM * 4 : 0);   // + mean, rstd of the tile's rows
@@ -346,6 +354,7 @@ REEF_ENTRY(reef_conv2d_d7k_16x16k4, OpConvDirectK<7>)
 REEF_ENTRY(reef_conv2d_d7k_16x32k4, OpConvDirectK<7 REEF_COMMA 2>)
 REEF_ENTRY(reef_conv2d_xdw_g2, OpConvXdw<2>)
 REEF_ENTRY(reef_conv2d_xdw_g4, OpConvXdw<4>)
+REEF_ENTRY(reef_conv2d_sp7_g2, OpConvStemPool)
 REEF_ENTRY(reef_conv2d_xdw2_g2, OpConvXdw<2 REEF_COMMA 2>)
 REEF_ENTRY(reef_gemm_nt_128x128, OpGemm<Tile128x128 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nt_64x64, OpGemm<Tile64x64 REEF_COMMA true>)

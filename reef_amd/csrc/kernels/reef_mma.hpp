@@ -1451,6 +1451,164 @@ __device__ __forceinline__ bool conv2d_xdw_body(const ReefOpDesc& d, int task, c
     return true;
 }
 
+// ---- reef_conv2d_sp7_g2: the stem of a ResNet / DenseNet in one launch ------------------------
+// in (+ a per-channel shift) -> 7x7 convolution, stride 2, padding 3, + bias, activation ->
+// 3x3 max-pool, stride 2, padding 1 (+ a per-channel shift, activation).  As launches of their own
+// the three are 3.5 + 16.6 + 4.3 us on a 224 x 224 image, and the 64 x 112 x 112 tensor between
+// convolution and pool (3.2 MB) is written to be read once.  The convolution has K = 147: cheap to
+// compute again, and the pool is local to a channel -- the case of reef_conv2d_xdw: a workgroup
+// owns 16 channels x 2 pooled rows x 14 pooled columns and forms the 5 x 29 convolution results
+// its windows touch itself (1.3 x the convolution's work in total); no workgroup waits for another.
+//   phase 0  the 15 x 63 input patch of every channel into LDS (zero outside the image: the
+//            convolution's padding; the input shift applies inside the image only, as it does
+//            when the shift is a launch of its own in front of a zero-padding convolution).
+//   phase 1  the convolution on the matrix cores: pixel group (r, c) is convolution row
+//            2 py0 - 1 + r and columns 2 px0 - 1 + 16 c + lane.  The taps are taken in the order
+//            (channel, ky, kx) with kx counted to 8 (the eighth weight is 0): MFMA s of a group
+//            covers filter row s / 2 and taps kx = 4 (s % 2) + lane / 16, so the weight's and the
+//            patch value's addresses are the lane's base plus a constant of s -- no index
+//            arithmetic, nothing to keep in registers.
+//            The wavefronts split the ten groups, so nobody adds partial sums.  + bias,
+//            activation; a position outside the convolution's output counts as -FLT_MAX (the
+//            pool's padding) -> E in LDS.
+//   phase 2  thread (channel, pooled column) takes the maximum of its 3 x 3 windows for the two
+//            pooled rows, adds the pool's shift, applies its activation, stores.
+// ptr: in [Cin][H][W] (Cin <= 3), W [Cout][Cin][7][7], out [Cout][Ho][Wo] (pooled), bias [Cout],
+// then the input shift [Cin] (REEF_F_IN_SHIFT) and the pool's shift [Cout] (REEF_F_POOL_SHIFT).
+// attr: H, W of the input; Ho, Wo of the POOLED output; M_TILES = ceil(Cout / 16),
+// N_TILES = ceil(Ho / 2) * ceil(Wo / 14); ACT the convolution's, ACT2 the pool's activation.
+struct TileSp7 {
+    static constexpr int G = 2, CR = 2 * G + 1, NG = 2 * CR;       // pooled rows; convolution rows; pixel groups
+    static constexpr int PR = 2 * CR + 5, PC = 64, CMAX = 3;       // patch rows, row stride, channels
+    static constexpr int STEPS = CMAX * 7 * 2;                     // 42 MFMAs per group: two per filter row
+    static constexpr int ESTRIDE = CR * 32 + 1;                    // floats per channel of E
+    static constexpr int PATCH = CMAX * PR * PC, EFLOATS = 16 * ESTRIDE + 32;
+    static constexpr int LDS_BYTES = (PATCH + EFLOATS) * 4 + 16;
+};
+
+template <class Poll>
+__device__ __forceinline__ bool conv2d_stem_pool_body(const ReefOpDesc& d, int task, char* smem_raw, const Poll&) {
+    typedef TileSp7 T;
+    float* patch = (float*)smem_raw;
+    float* E = patch + T::PATCH;
+    const int* a = d.attr;
+    const int lane = threadIdx.x & 63, i16 = lane & 15, kq = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int C = a[REEF_CONV_CIN], H = a[REEF_CONV_H], W = a[REEF_CONV_W], M = a[REEF_CONV_COUT];
+    const int Ho = a[REEF_CONV_HO], Wo = a[REEF_CONV_WO];
+    const int Hc = (H - 1) / 2 + 1, Wc = (W - 1) / 2 + 1;          // the convolution's output: (H + 6 - 7) / 2 + 1
+    const int flags = a[REEF_CONV_FLAGS];
+    const int m_tiles = a[REEF_CONV_M_TILES], n_tiles = a[REEF_CONV_N_TILES];
+    task = xcd_chunked(task, m_tiles * n_tiles);
+    const int nt = div_small(task, m_tiles), mt = task - nt * m_tiles;
+    const int segs = (Wo + kRowSeg - 1) / kRowSeg;
+    const int q_seg = div_small(nt, segs);
+    const int py0 = q_seg * T::G, px0 = (nt - q_seg * segs) * kRowSeg;
+    const int m0 = mt * 16;
+    const int K = C * 49;
+    int p = 4;
+    const float* in_shift = (flags & REEF_F_IN_SHIFT) ? (const float*)d.ptr[p++] : nullptr;
+    const float* pool_shift = (flags & REEF_F_POOL_SHIFT) ? (const float*)d.ptr[p++] : nullptr;
+
+    // the weights of this lane's channel row: step s = filter row s / 2 (of channel s / 14), tap
+    // kx = 4 (s % 2) + kq; kx = 7 does not exist (weight 0).  All on their way at once.
+    const rsrc_t rs_w = make_rsrc(d.ptr[1], (unsigned)M * (unsigned)K * 4u);
+    float ra[T::STEPS];
+    const unsigned wrow = ((unsigned)(m0 + i16) * (unsigned)K + (unsigned)kq) * 4u;      // a row outside M: outside the buffer
+#pragma unroll
+    for (int s = 0; s < T::STEPS; ++s) {
+        const int c = s / 14, ky = (s % 14) / 2, kx0 = 4 * (s & 1);
+        const bool real = c < C && kx0 + kq < 7;
+        ra[s] = buf_load(rs_w, real ? wrow + (unsigned)(c * 49 + ky * 7 + kx0) * 4u : kOutside);
+    }
+    const rsrc_t rs_bias = make_rsrc(d.ptr[3], (unsigned)M * 4u);
+    float bias[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) bias[j] = buf_load(rs_bias, (unsigned)(m0 + 4 * kq + j) * 4u);
+
+    // phase 0: the patch.  Origin: input row 4 py0 - 5, column 4 px0 - 5.
+    const rsrc_t rs_in = make_rsrc(d.ptr[0], (unsigned)C * (unsigned)(H * W) * 4u);
+    const int iy0 = 4 * py0 - 5, ix0 = 4 * px0 - 5;
+    {
+        // every load of the thread's share on its way before the first value is stored
+        constexpr int SHARE = (T::PATCH + kThreads - 1) / kThreads;
+        float sh[T::CMAX];
+#pragma unroll
+        for (int c = 0; c < T::CMAX; ++c) sh[c] = (in_shift && c < C) ? in_shift[c] : 0.0f;
+        float v[SHARE];
+        int cc[SHARE];
+        bool inside[SHARE];
+#pragma unroll
+        for (int i = 0; i < SHARE; ++i) {
+            const int idx = (int)threadIdx.x + kThreads * i;
+            const int c = idx / (T::PR * T::PC), rem = idx - c * (T::PR * T::PC);     // constants: shifts and a multiply
+            const int iy = iy0 + (rem >> 6), ix = ix0 + (rem & 63);
+            inside[i] = c < C && (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
+            cc[i] = c;
+            v[i] = buf_load(rs_in, inside[i] ? (unsigned)(c * H * W + iy * W + ix) * 4u : kOutside);
+        }
+#pragma unroll
+        for (int i = 0; i < SHARE; ++i) {
+            const int idx = (int)threadIdx.x + kThreads * i;
+            const float s = cc[i] == 0 ? sh[0] : cc[i] == 1 ? sh[1] : sh[2];
+            if (idx < T::PATCH) patch[idx] = inside[i] ? v[i] + s : 0.0f;
+        }
+    }
+    __syncthreads();
+
+    // phase 1
+    const int act = a[REEF_CONV_ACT], act2 = a[REEF_CONV_ACT2];
+    for (int g = wave; g < T::NG; g += 4) {
+        const int r = g >> 1, gc = g & 1;
+        const int j = min(16 * gc + i16, 28);          // columns past the 29 a tile needs: computed, never read
+        const float* base = patch + (2 * r) * T::PC + 2 * j + kq;
+        f32x4 acc0 = f32x4{0.0f, 0.0f, 0.0f, 0.0f}, acc1 = acc0;
+        // a channel at a time: its fourteen patch values into registers, then fourteen MFMAs (a channel
+        // the image does not have: weights 0 against a patch of zeros)
+#pragma unroll
+        for (int c = 0; c < T::CMAX; ++c) {
+            float b[14];
+#pragma unroll
+            for (int i = 0; i < 14; ++i) b[i] = base[(c * T::PR + i / 2) * T::PC + 4 * (i & 1)];
+            __builtin_amdgcn_sched_barrier(0);      // all fourteen reads issued before the first MFMA waits for one
+#pragma unroll
+            for (int i = 0; i < 14; ++i) {
+                // the tap that does not exist (kx = 7): 0 x 0, whatever the patch holds there
+                const float bv = (i & 1) ? (kq == 3 ? 0.0f : b[i]) : b[i];
+                if (i & 1) acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[14 * c + i], bv, acc1, 0, 0, 0);
+                else acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[14 * c + i], bv, acc0, 0, 0, 0);
+            }
+        }
+        const int cy = 2 * py0 - 1 + r, cx = 2 * px0 - 1 + 16 * gc + i16;
+        const bool inside = (unsigned)cy < (unsigned)Hc && (unsigned)cx < (unsigned)Wc;
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            const float v = act_apply((acc0[jj] + acc1[jj]) + bias[jj], act);
+            E[(4 * kq + jj) * T::ESTRIDE + r * 32 + 16 * gc + i16] = inside ? v : -FLT_MAX;
+        }
+    }
+    __syncthreads();
+
+    // phase 2
+    const int row = threadIdx.x >> 4, col = threadIdx.x & 15;
+    const unsigned ch = (unsigned)(m0 + row);
+    const rsrc_t rs_o = make_rsrc(d.ptr[2], (unsigned)M * (unsigned)(Ho * Wo) * 4u);
+    const float sh2 = (pool_shift && ch < (unsigned)M) ? pool_shift[ch] : 0.0f;
+    const float* Ec = E + row * T::ESTRIDE + 2 * col;
+#pragma unroll
+    for (int g = 0; g < T::G; ++g) {
+        float m = -FLT_MAX;
+#pragma unroll
+        for (int ky = 0; ky < 3; ++ky)
+#pragma unroll
+            for (int kx = 0; kx < 3; ++kx) m = fmaxf(m, Ec[(2 * g + ky) * 32 + kx]);
+        const bool ok = col < kRowSeg && px0 + col < Wo && py0 + g < Ho && ch < (unsigned)M;
+        buf_store(rs_o, ok ? (ch * (unsigned)(Ho * Wo) + (unsigned)((py0 + g) * Wo + px0 + col)) * 4u : kOutside,
+                  act_apply(m + sh2, act2));
+    }
+    return true;
+}
+
 // ---- reef_gemm ----------------------------------------------------------------
 // TRANS_B: B stored [N][K] (dense layers, Q.K^T) -- both operands take 128-bit row
 // loads, so K, lda, ldb and the batch strides must be multiples of 4 floats.

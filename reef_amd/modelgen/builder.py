@@ -25,6 +25,7 @@ from ..paths import code_object
 
 ACT_NONE, ACT_RELU, ACT_RELU6, ACT_GELU = 0, 1, 2, 3
 F_BIAS, F_RESIDUAL, F_AFFINE, F_DUAL, F_FUSED_REDUCE, F_PRE_ACT, F_PAIR_FOLD, F_DW_OUTPUT = 1, 2, 4, 8, 16, 32, 64, 128
+F_POOL_OUTPUT, F_IN_SHIFT, F_POOL_SHIFT = 256, 512, 1024
 WG = 256
 
 
@@ -296,6 +297,31 @@ class GraphBuilder:
                        [M, N, t["split_k"], flags & ~F_PRE_ACT, act, act2, dst_off], "splitk_reduce", 0,
                        4 * ((t["split_k"] + 1) * M * N), 2.0)
         return out if out2 is None else (out, out2)
+
+    def conv2d_pool(self, x, cout, act=ACT_RELU, in_shift=False, pool_shift=False, pool_act=ACT_NONE, out=None):
+        """7x7 / stride 2 / padding 3 convolution (+ bias, act) of an image of at most 3 channels and the
+        3x3 / stride 2 / padding 1 max-pool (+ shift, pool_act) behind it in one launch
+        (reef_conv2d_sp7_g2).  in_shift: a per-channel shift on the input, inside the image.
+        Parameters are made in the order: input shift, weights, bias, pool shift."""
+        cin, H, W = x.shape
+        assert cin <= 3, "the fused stem takes at most 3 input channels"
+        sh_in = self.param((cin,), 0.01) if in_shift else None
+        w = self.param((cout, cin, 7, 7), self.weight_std if self.weight_std is not None else math.sqrt(2.0 / (cin * 49)))
+        b = self.param((cout,), 0.01)
+        sh_pool = self.param((cout,), 0.01) if pool_shift else None
+        Hc, Wc = (H + 6 - 7) // 2 + 1, (W + 6 - 7) // 2 + 1
+        Ho, Wo = (Hc + 2 - 3) // 2 + 1, (Wc + 2 - 3) // 2 + 1
+        out = Tensor(out.idx, (cout, Ho, Wo), out.off) if out is not None else self.temp((cout, Ho, Wo))
+        mt, nt = math.ceil(cout / 16), math.ceil(Ho / 2) * math.ceil(Wo / 14)
+        flags = F_BIAS | F_POOL_OUTPUT | (F_IN_SHIFT if in_shift else 0) | (F_POOL_SHIFT if pool_shift else 0)
+        args = [x, w.idx, out, b.idx] + ([sh_in.idx] if in_shift else []) + ([sh_pool.idx] if pool_shift else [])
+        flops = 2 * cout * cin * 49 * Hc * Wc
+        self.flops += flops
+        self._emit("reef_conv2d_sp7_g2", mt * nt, args,
+                   [cin, H, W, cout, Ho, Wo, 7, 7, 2, 2, 3, 3, flags, act, tiling.TILES["g2"][0], 1,
+                    math.ceil(cin * 49 / 4) * 4, mt, nt, pool_act, 0, 7, 0, 0],
+                   "conv2d", flops, 4 * (x.size + w.size + cout + out.size), 8.0)
+        return out
 
     XDW_TILES = {"g2": 2, "g4": 4}     # reef_conv2d_xdw_<tile>: image rows per tile
 
@@ -613,7 +639,9 @@ class GraphBuilder:
         for k in self.kernels:
             n = k["name"]
             sym = n.split("#")[0]
-            if sym.startswith("reef_conv2d_xdw"):
+            if sym == "reef_conv2d_sp7_g2":
+                shared[n] = (3 * 15 * 64 + 16 * (5 * 32 + 1) + 32) * 4 + 16     # TileSp7: input patch + pooled-from block
+            elif sym.startswith("reef_conv2d_xdw"):
                 G, S = self.XDW_TILES[sym.split("_")[-1]], 2 if sym.startswith("reef_conv2d_xdw2_") else 1
                 NG = (G + 2) if S == 1 else (2 * G + 1) * 2      # TileXdw: pixel groups of the 1x1 result
                 shared[n] = (4 * NG * 320 + 16 * (NG + 1) * 16) * 4 + 16

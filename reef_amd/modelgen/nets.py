@@ -35,7 +35,7 @@ def image_input(name, shape, seed=rng.BASE_SEED):
 
 
 def resnet(num_layers=152, image=(3, 224, 224), classes=1000, name=None, seed=rng.BASE_SEED,
-           fused_reduce=False, fuse_act=True, stack_first=True):
+           fused_reduce=False, fuse_act=True, stack_first=True, fuse_stem=True):
     """fused_reduce: fold split-K inside the conv kernels.  fuse_act: let the unit's last
     conv also write the next unit's activated input (one kernel instead of conv + add/relu).
     The first unit of a bottleneck stage has two 1x1 convolutions on the same input with the same
@@ -43,7 +43,9 @@ def resnet(num_layers=152, image=(3, 224, 224), classes=1000, name=None, seed=rn
     with the stacked filter and two outputs: the bare result, whose shortcut rows are the
     residual of the unit's last convolution, and relu(result + shift), whose conv1 rows feed the
     3x3 convolution (channel ranges of the two outputs, operand views).  stack_first=False keeps
-    them two launches, as the reference's graph has them."""
+    them two launches, as the reference's graph has them.
+    fuse_stem: the shift on the input, the 7x7 convolution and the max-pool behind it are one launch
+    (reef_conv2d_sp7_g2) instead of three; same parameters in the same order."""
     if num_layers >= 50:
         bottleneck = True
         filters = [64, 256, 512, 1024, 2048]
@@ -55,9 +57,12 @@ def resnet(num_layers=152, image=(3, 224, 224), classes=1000, name=None, seed=rn
     g = GraphBuilder(name or "resnet%d" % num_layers, seed)
     g.fused_reduce = fused_reduce
     data = g.input("data", image)
-    x = g.eltwise(data, shift=True)                                  # bn_data (shift only)
-    x = g.conv2d(x, filters[0], 7, 2, 3, bias=True, act=ACT_RELU)    # conv0 + bn0 + relu
-    act = g.pool2d(x, 3, 2, 1, "max", bias=True, act=ACT_RELU)       # pool + first bn1 + relu
+    if fuse_stem and image[0] <= 3:
+        act = g.conv2d_pool(data, filters[0], act=ACT_RELU, in_shift=True, pool_shift=True, pool_act=ACT_RELU)
+    else:
+        x = g.eltwise(data, shift=True)                                  # bn_data (shift only)
+        x = g.conv2d(x, filters[0], 7, 2, 3, bias=True, act=ACT_RELU)    # conv0 + bn0 + relu
+        act = g.pool2d(x, 3, 2, 1, "max", bias=True, act=ACT_RELU)       # pool + first bn1 + relu
     raw = None
     n_stages = len(units)
     for si in range(n_stages):
@@ -156,25 +161,32 @@ def mobilenet_v2(image=(3, 224, 224), classes=1000, name="mobilenetv2", seed=rng
 
 
 def densenet(blocks=(6, 12, 48, 32), growth=32, image=(3, 224, 224), classes=1000, name="densenet201",
-             seed=rng.BASE_SEED):
+             seed=rng.BASE_SEED, fuse_stem=True):
     """DenseNet-BC (201: blocks 6/12/48/32, growth 32): every layer reads the running
     concatenation through its own BN + ReLU (it cannot be folded into the producing
     convolution because each consumer has its own statistics; it is folded into the input
     loads of the consuming 1x1 convolution where a kernel for that exists), then
     1x1 -> 128 (+bias, ReLU) and 3x3 -> 32, which writes straight into its channel slice
-    of the concatenation buffer."""
+    of the concatenation buffer.
+    fuse_stem: the 7x7 convolution and the max-pool behind it are one launch (reef_conv2d_sp7_g2)."""
     g = GraphBuilder(name, seed)
     x = g.input("data", image)
-    y = g.conv2d(x, 2 * growth, 7, 2, 3, bias=True, act=ACT_RELU)
+    fuse_stem = fuse_stem and image[0] <= 3
+    y = None if fuse_stem else g.conv2d(x, 2 * growth, 7, 2, 3, bias=True, act=ACT_RELU)
+    stem_hw = ((image[1] - 1) // 2 + 1, (image[2] - 1) // 2 + 1)       # the 7x7 / 2 convolution's output
     c = 2 * growth
     for bi, n_layers in enumerate(blocks):
         # the pool in front of a block writes the first channels of the block's buffer itself
         pool = (3, 2, 1, "max") if bi == 0 else (2, 2, 0, "avg")
-        H = (y.shape[1] + 2 * pool[2] - pool[0]) // pool[1] + 1
-        W = (y.shape[2] + 2 * pool[2] - pool[0]) // pool[1] + 1
+        yh, yw = stem_hw if y is None else y.shape[1:]
+        H = (yh + 2 * pool[2] - pool[0]) // pool[1] + 1
+        W = (yw + 2 * pool[2] - pool[0]) // pool[1] + 1
         total = c + n_layers * growth
         buf = g.temp((total, H, W))
-        g.pool2d(y, *pool, out=buf.channels(0, c))
+        if y is None:
+            g.conv2d_pool(x, c, act=ACT_RELU, out=buf.channels(0, c))
+        else:
+            g.pool2d(y, *pool, out=buf.channels(0, c))
         for li in range(n_layers):
             cur = c + li * growth
             y = g.conv2d(buf.channels(0, cur), 4 * growth, 1, 1, 0, bias=True, act=ACT_RELU, pre_act=True)

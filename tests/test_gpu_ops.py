@@ -641,3 +641,50 @@ def test_gemm_direct_splits_k_across_workgroups(tmp_path, tile, split):
             if s["name"] == "reef_sync":
                 assert not e.get_data(i, s["size"], np.int32).any()
         e.close()
+
+
+SP7_CASES = [
+    # cin, H, W, cout, input shift, pool shift, conv act, pool act
+    (3, 224, 224, 64, True, True, MB.ACT_RELU, MB.ACT_RELU),      # the ResNet stem
+    (3, 37, 45, 24, False, False, MB.ACT_RELU, MB.ACT_NONE),      # odd sizes, a partial channel tile
+    (1, 64, 64, 16, True, False, MB.ACT_NONE, MB.ACT_RELU),       # one channel: K = 49
+    (2, 30, 57, 40, False, True, MB.ACT_RELU6, MB.ACT_NONE),
+    (3, 9, 9, 16, True, True, MB.ACT_RELU, MB.ACT_RELU),          # image smaller than one tile
+]
+
+
+@pytest.mark.parametrize("case", SP7_CASES)
+def test_stem_convolution_and_pool_in_one_launch(tmp_path, case):
+    """reef_conv2d_sp7_g2: input shift, 7x7 / 2 convolution + bias + activation and the 3x3 / 2
+    max-pool + shift + activation behind it against the oracle's three steps, against the three
+    launches on the device (1e-4: the fused kernel sums the taps in another order), and bit for
+    bit in the three flavours."""
+    from reef_amd import binding as B
+    from tests.helpers import write_model, max_rel_err, REL_TOL
+    cin, H, W, cout, in_shift, pool_shift, act, pool_act = case
+    g = MB.GraphBuilder("sp7")
+    x = g.input("data", (cin, H, W))
+    y = g.conv2d_pool(x, cout, act=act, in_shift=in_shift, pool_shift=pool_shift, pool_act=pool_act)
+    g.mark_output(y)
+    assert g.kernels[0]["name"].startswith("reef_conv2d_sp7_g2") and len(g.kernels) == 1
+    # the same parameters through launches of their own
+    g3 = MB.GraphBuilder("sp7")
+    x3 = g3.input("data", (cin, H, W))
+    t = g3.eltwise(x3, shift=True) if in_shift else x3
+    t = g3.conv2d(t, cout, 7, 2, 3, bias=True, act=act)
+    g3.mark_output(g3.pool2d(t, 3, 2, 1, "max", bias=pool_shift, act=pool_act))
+    assert [k for k, _ in g3.params if not k.endswith("k")] == [k for k, _ in g.params]
+    data = 2.0 * rnd(cin, H, W) - 0.5
+    exe, orc, model = run_both(g, tmp_path / "one", {"data": data})
+    worst = compare_storages(exe, orc, model, what="sp7 %s" % (case,))
+    want = exe.get_output()
+    exe3, orc3, model3 = run_both(g3, tmp_path / "three", {"data": data})
+    assert max_rel_err(want, exe3.get_output()) <= REL_TOL
+    d = write_model(g, tmp_path / "one")
+    for kind, pre in ((B.TRANS, False), (B.HYBRID, True), (B.HYBRID, False)):
+        e = B.Executor.from_dir(d, g.name, kind)
+        e.set_input_checked("data", data)
+        e.execute_preemptable() if pre else e.execute()
+        np.testing.assert_array_equal(e.get_output(), want, err_msg="flavour %s %s" % (kind, pre))
+        e.close()
+    print("sp7 %s: worst rel err %.2e" % (case, worst[0]))

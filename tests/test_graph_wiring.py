@@ -51,7 +51,7 @@ class Params:
 
 
 def test_resnet_generator_equals_the_reference_graph(tmp_path):
-    g = nets.resnet(152, image=(3, 64, 64), fuse_act=False, fused_reduce=True, stack_first=False,
+    g = nets.resnet(152, image=(3, 64, 64), fuse_act=False, fused_reduce=True, stack_first=False, fuse_stem=False,
                     name="resnet152_64")
     ref = json.load(open(REF_JSON))
     table = json.load(open(TABLE))
