@@ -591,3 +591,36 @@ def test_a_matrix_product_with_k_split_across_workgroups_is_checked(tmp_path):
     broken(lambda m: m["kernels"][0].__setitem__("name", "reef_gemm_nt_32x32k4#0"), "only the direct kernels")
     broken(lambda m: m["kernels"][0]["launch_params"].__setitem__(0, 9), "workgroups")
     broken(lambda m: m["storage"][m["kernels"][0]["args"][3]].__setitem__("size", 2 * 40 * 96 * 4), "workspace")
+
+
+def test_a_stem_kernel_is_checked_against_its_storages(tmp_path):
+    """reef_conv2d_sp7_g2: the output sizes are the pooled ones, the operand list follows the flags,
+    and the kernel is only for 7x7 / stride 2 / padding 3 filters on at most three channels."""
+    from reef_amd import binding as B
+    g = MB.GraphBuilder("sp7fmt")
+    x = g.input("data", (3, 37, 45))
+    g.mark_output(g.conv2d_pool(x, 24, in_shift=True, pool_shift=True, pool_act=MB.ACT_RELU))
+    base = g.write(str(tmp_path / "ok"), link_code_objects=False)
+    assert B.check_model(base + ".json") == (True, "")
+    model = json.load(open(base + ".json"))
+    k = model["kernels"][0]
+    a = k["attrs"]
+    assert k["name"].startswith("reef_conv2d_sp7_g2") and len(k["args"]) == 6
+    assert a[4:6] == [10, 12] and a[12] == 1 | 256 | 512 | 1024 and a[17:19] == [2, 5] and k["launch_params"][0] == 10
+
+    def broken(change, reason):
+        m = json.loads(json.dumps(model))
+        change(m)
+        p = str(tmp_path / "broken.json")
+        json.dump(m, open(p, "w"))
+        ok, why = B.check_model(p)
+        assert not ok and reason in why, why
+
+    broken(lambda m: m["kernels"][0]["args"].pop(), "operands")                              # no pool shift
+    broken(lambda m: m["kernels"][0]["attrs"].__setitem__(4, 19), "output size")             # the convolution's rows, not the pooled
+    broken(lambda m: m["kernels"][0]["attrs"].__setitem__(8, 1), "output size")              # stride 1
+    broken(lambda m: m["kernels"][0]["attrs"].__setitem__(12, 1 | 256 | 2), "loader family") # a residual is not supported
+    broken(lambda m: m["kernels"][0]["attrs"].__setitem__(18, 4), "loader family")           # wrong tile count
+    broken(lambda m: m["kernels"][0].__setitem__("name", "reef_conv2d_u_64x32k2#0"), "loader family")
+    broken(lambda m: m["storage"][m["kernels"][0]["args"][2]].__setitem__("size", 24 * 10 * 11), "output")
+    broken(lambda m: m["storage"][m["kernels"][0]["args"][4]].__setitem__("size", 2), "input shift")
