@@ -287,8 +287,10 @@ enum {
 };
 
 /* ---- reef_pool2d: max / average pooling (+bias +relu) ----
- * ptr: in, out, bias(optional).  mode 0 max (pads with -FLT_MAX), 1 average.
+ * ptr: in, out, bias (flags & 1), then pre-scale and pre-shift (flags & REEF_POOL_F_PRE: the input is
+ * read as relu(in * scale[c] + shift[c])).  mode 0 max (pads with -FLT_MAX), 1 average.
  * tasks = ceil(C*Ho*Wo / 256). */
+#define REEF_POOL_F_PRE 2
 enum {
     REEF_POOL_C = 0, REEF_POOL_H, REEF_POOL_W, REEF_POOL_HO, REEF_POOL_WO, REEF_POOL_KH,
     REEF_POOL_KW, REEF_POOL_SH, REEF_POOL_SW, REEF_POOL_PH, REEF_POOL_PW, REEF_POOL_MODE,

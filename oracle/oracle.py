@@ -367,7 +367,11 @@ class GraphOracle:
         elif name == "reef_pool2d":
             C, H, W, Ho, Wo, kh, kw, sh, sw, ph, pw, mode, cpad, flags, act = a[:15]
             bias = P[2] if flags & 1 else None
-            out = pool2d(P[0][:C * H * W].reshape(C, H, W), (kh, kw), (sh, sw), (ph, pw), mode, bias,
+            xin = P[0][:C * H * W].reshape(C, H, W)
+            if flags & 2:       # read through relu(in * scale[c] + shift[c])
+                pp = 2 + (flags & 1)
+                xin = eltwise(xin.reshape(C, -1), scale=P[pp][:C], shift=P[pp + 1][:C], act=1).reshape(C, H, W)
+            out = pool2d(xin, (kh, kw), (sh, sw), (ph, pw), mode, bias,
                          act, bool(cpad), (Ho, Wo))
             P[1][:out.size] = out.reshape(-1)
         elif name == "reef_global_avgpool":

@@ -317,6 +317,7 @@ bool small_op(int op, const Attrs& a, i64 grid, Needs& n) {
         n.f32("input", C * a[REEF_POOL_H] * a[REEF_POOL_W]);
         n.f32("output", out);
         if (a[REEF_POOL_FLAGS] & 1) n.f32("bias", C);
+        if (a[REEF_POOL_FLAGS] & REEF_POOL_F_PRE) { n.f32("input scale", C); n.f32("input shift", C); }
         n.tasks = cdiv(out, 256);
         return true;
     }

@@ -142,6 +142,12 @@ __device__ __forceinline__ void pool2d_body(const ReefOpDesc& d, int task) {
     const float* in = (const float*)d.ptr[0] + (size_t)c * H * W;
     float m = -FLT_MAX, s = 0.0f;
     int cnt = 0;
+    // REEF_POOL_F_PRE: the input is read through relu(in * scale[c] + shift[c]) (a DenseNet transition
+    // pools what its pre-activation produced; the 1x1 filter that commutes with the average runs behind)
+    const int pflags = a[REEF_POOL_FLAGS];
+    const bool pre = pflags & REEF_POOL_F_PRE;
+    const int pp = 2 + (pflags & 1);
+    const float psc = pre ? ((const float*)d.ptr[pp])[c] : 1.0f, psh = pre ? ((const float*)d.ptr[pp + 1])[c] : 0.0f;
     if (kh <= 3 && kw <= 3) {
         // all loads of the window issued together (a tap outside the image or the window reads
         // outside the buffer and is ignored), then max / sum in window order
@@ -160,8 +166,9 @@ __device__ __forceinline__ void pool2d_body(const ReefOpDesc& d, int task) {
 #pragma unroll
         for (int t = 0; t < 9; ++t)
             if (ok[t]) {
-                m = fmaxf(m, v[t]);
-                s += v[t];
+                const float x_ = pre ? fmaxf(fmaf(v[t], psc, psh), 0.0f) : v[t];
+                m = fmaxf(m, x_);
+                s += x_;
                 ++cnt;
             }
     } else
@@ -171,7 +178,7 @@ __device__ __forceinline__ void pool2d_body(const ReefOpDesc& d, int task) {
         for (int dx = 0; dx < kw; ++dx) {
             const int ix = x * sw + dx - pw;
             if ((unsigned)ix >= (unsigned)W) continue;
-            const float v = in[iy * W + ix];
+            const float v = pre ? fmaxf(fmaf(in[iy * W + ix], psc, psh), 0.0f) : in[iy * W + ix];
             m = fmaxf(m, v);
             s += v;
             ++cnt;

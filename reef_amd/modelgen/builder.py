@@ -381,7 +381,8 @@ class GraphBuilder:
         return out
 
     def pool2d(self, x, k, stride, pad, mode="max", bias=False, act=ACT_NONE, count_include_pad=False,
-               ceil_mode=False, out=None, bias_t=None):
+               ceil_mode=False, out=None, bias_t=None, pre=None):
+        """pre: (scale, shift) parameters -- the input is read through relu(x * scale[c] + shift[c])."""
         C, H, W = x.shape
         kh, kw = (k, k) if isinstance(k, int) else k
         rnd = math.ceil if ceil_mode else math.floor
@@ -393,6 +394,9 @@ class GraphBuilder:
         if bias:
             flags = 1
             args.append((bias_t or self.param((C,), 0.01)).idx)
+        if pre is not None:
+            flags |= 2
+            args += [pre[0].idx, pre[1].idx]
         self._emit("reef_pool2d", math.ceil(out.size / WG), args,
                    [C, H, W, Ho, Wo, kh, kw, stride, stride, pad, pad, 0 if mode == "max" else 1,
                     1 if count_include_pad else 0, flags, act], "pool2d", 0,
@@ -452,6 +456,12 @@ class GraphBuilder:
         self._emit("reef_softmax", math.ceil(rows / 4), args, [rows, cols, 1 if mask is not None else 0],
                    "softmax", 0, 8 * rows * cols, 2.0)
         return out
+
+    def pre_act_params(self, c):
+        """scale ~ 1 + N(0, 0.1), shift ~ N(0, 0.01): what conv2d(pre_act=True) makes for itself."""
+        ps = self.param((c,), 0.1)
+        self.params[-1] = (self.params[-1][0], self.params[-1][1] + 1.0)
+        return ps, self.param((c,), 0.01)
 
     def layernorm_params(self, cols):
         """gamma ~ 1 + N(0, 0.1), beta ~ N(0, 0.01): the parameters layernorm() makes for itself."""

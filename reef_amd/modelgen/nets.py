@@ -16,6 +16,7 @@ off resource/resnet152/resnet152.json kernels[0..18]:
   last unit of the net : conv3 + residual, * scale + shift, relu
   global average pool -> dense (+bias) -> softmax
 """
+import math
 import numpy as np
 
 from . import rng
@@ -161,14 +162,19 @@ def mobilenet_v2(image=(3, 224, 224), classes=1000, name="mobilenetv2", seed=rng
 
 
 def densenet(blocks=(6, 12, 48, 32), growth=32, image=(3, 224, 224), classes=1000, name="densenet201",
-             seed=rng.BASE_SEED, fuse_stem=True):
+             seed=rng.BASE_SEED, fuse_stem=True, pool_first=True):
     """DenseNet-BC (201: blocks 6/12/48/32, growth 32): every layer reads the running
     concatenation through its own BN + ReLU (it cannot be folded into the producing
     convolution because each consumer has its own statistics; it is folded into the input
     loads of the consuming 1x1 convolution where a kernel for that exists), then
     1x1 -> 128 (+bias, ReLU) and 3x3 -> 32, which writes straight into its channel slice
     of the concatenation buffer.
-    fuse_stem: the 7x7 convolution and the max-pool behind it are one launch (reef_conv2d_sp7_g2)."""
+    fuse_stem: the 7x7 convolution and the max-pool behind it are one launch (reef_conv2d_sp7_g2).
+    pool_first: a transition is BN + ReLU, a 1x1 filter (no bias) and a 2x2 average pool.  Filter
+    and average are both linear and the filter is pointwise, so they commute: the pool reads the
+    concatenation through the BN + ReLU and the filter runs on a quarter of the pixels, writing
+    straight into the next block's buffer -- a quarter of the transition's multiplications, same
+    parameters in the same order.  False keeps the textbook order."""
     g = GraphBuilder(name, seed)
     x = g.input("data", image)
     fuse_stem = fuse_stem and image[0] <= 3
@@ -178,13 +184,19 @@ def densenet(blocks=(6, 12, 48, 32), growth=32, image=(3, 224, 224), classes=100
     for bi, n_layers in enumerate(blocks):
         # the pool in front of a block writes the first channels of the block's buffer itself
         pool = (3, 2, 1, "max") if bi == 0 else (2, 2, 0, "avg")
-        yh, yw = stem_hw if y is None else y.shape[1:]
-        H = (yh + 2 * pool[2] - pool[0]) // pool[1] + 1
-        W = (yw + 2 * pool[2] - pool[0]) // pool[1] + 1
+        if isinstance(y, tuple):
+            H, W = y[0].shape[1:]          # already pooled
+        else:
+            yh, yw = stem_hw if y is None else y.shape[1:]
+            H = (yh + 2 * pool[2] - pool[0]) // pool[1] + 1
+            W = (yw + 2 * pool[2] - pool[0]) // pool[1] + 1
         total = c + n_layers * growth
         buf = g.temp((total, H, W))
         if y is None:
             g.conv2d_pool(x, c, act=ACT_RELU, out=buf.channels(0, c))
+        elif isinstance(y, tuple):
+            # transition with the pool in front: y = (pooled pre-activated input, weights of the 1x1 filter)
+            g.conv2d(y[0], c, 1, 1, 0, bias=False, act=ACT_NONE, out=buf, out_channel=0, given={"w": y[1]})
         else:
             g.pool2d(y, *pool, out=buf.channels(0, c))
         for li in range(n_layers):
@@ -194,7 +206,13 @@ def densenet(blocks=(6, 12, 48, 32), growth=32, image=(3, 224, 224), classes=100
         c = total
         x = buf
         if bi != len(blocks) - 1:
-            y = g.conv2d(x, c // 2, 1, 1, 0, bias=False, act=ACT_NONE, pre_act=True)
+            if pool_first:
+                # parameters in the order the textbook form makes them: weights, pre-scale, pre-shift
+                w = g.param((c // 2, c, 1, 1), math.sqrt(2.0 / c))
+                ps, pt = g.pre_act_params(c)
+                y = (g.pool2d(x, 2, 2, 0, "avg", pre=(ps, pt)), w)
+            else:
+                y = g.conv2d(x, c // 2, 1, 1, 0, bias=False, act=ACT_NONE, pre_act=True)
             c = c // 2
     a = g.eltwise(x, scale=True, shift=True, act=ACT_RELU)
     pooled = g.global_avgpool(a)
