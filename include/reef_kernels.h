@@ -297,9 +297,11 @@ enum {
     REEF_POOL_COUNT_PAD, REEF_POOL_FLAGS, REEF_POOL_ACT, REEF_POOL_NATTR
 };
 
-/* ---- reef_global_avgpool: out[c] = sum(in[c][:]) * (1/HW).  ptr: in, out.
- * attr: C, HW.  tasks = ceil(C / 4) (one wavefront per channel). */
-enum { REEF_GAP_C = 0, REEF_GAP_HW, REEF_GAP_NATTR };
+/* ---- reef_global_avgpool: out[c] = sum(in[c][:]) * (1/HW).  ptr: in, out, then scale and shift
+ * (flags & REEF_GAP_F_PRE: the input is read as relu(in * scale[c] + shift[c])).
+ * attr: C, HW, flags (absent = 0).  tasks = ceil(C / 4) (one wavefront per channel). */
+#define REEF_GAP_F_PRE 1
+enum { REEF_GAP_C = 0, REEF_GAP_HW, REEF_GAP_FLAGS, REEF_GAP_NATTR };
 
 /* ---- reef_eltwise: out = act(a (+b) (*scale[c]) (+shift[c])), c = i / inner ----
  * ptr: a, out, then optional b, scale, shift by flag.  attr: C, inner, flags, act.

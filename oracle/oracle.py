@@ -376,7 +376,10 @@ class GraphOracle:
             P[1][:out.size] = out.reshape(-1)
         elif name == "reef_global_avgpool":
             C, HW = a[:2]
-            P[1][:C] = global_avgpool(P[0][:C * HW].reshape(C, HW))
+            xin = P[0][:C * HW].reshape(C, HW)
+            if len(a) > 2 and a[2] & 1:       # read through relu(in * scale[c] + shift[c])
+                xin = eltwise(xin, scale=P[2][:C], shift=P[3][:C], act=1)
+            P[1][:C] = global_avgpool(xin)
         elif name == "reef_eltwise":
             C, inner, flags, act = a[:4]
             b, scale, shift = _opt(P, 2, flags, (1, 2, 4))

@@ -325,6 +325,7 @@ bool small_op(int op, const Attrs& a, i64 grid, Needs& n) {
         if (!all_positive(a, {REEF_GAP_C, REEF_GAP_HW})) { n.bad = "a dimension of the pooling is not positive"; return true; }
         n.f32("input", a[REEF_GAP_C] * a[REEF_GAP_HW]);
         n.f32("output", a[REEF_GAP_C]);
+        if (a[REEF_GAP_FLAGS] & REEF_GAP_F_PRE) { n.f32("input scale", a[REEF_GAP_C]); n.f32("input shift", a[REEF_GAP_C]); }
         n.tasks = cdiv(a[REEF_GAP_C], 4);
         return true;
     case REEF_OP_ELTWISE: {

@@ -198,7 +198,13 @@ __device__ __forceinline__ void global_avgpool_body(const ReefOpDesc& d, int tas
     if (c >= C) return;
     const float* in = (const float*)d.ptr[0] + (size_t)c * HW;
     float s = 0.0f;
-    for (int i = threadIdx.x & 63; i < HW; i += 64) s += in[i];
+    if (d.attr[REEF_GAP_FLAGS] & REEF_GAP_F_PRE) {
+        // the input is read through relu(in * scale[c] + shift[c]) (the last BN + ReLU of a DenseNet)
+        const float sc = ((const float*)d.ptr[2])[c], sh = ((const float*)d.ptr[3])[c];
+        for (int i = threadIdx.x & 63; i < HW; i += 64) s += fmaxf(fmaf(in[i], sc, sh), 0.0f);
+    } else {
+        for (int i = threadIdx.x & 63; i < HW; i += 64) s += in[i];
+    }
     s = wave_sum(s);
     if ((threadIdx.x & 63) == 0) ((float*)d.ptr[1])[c] = s * (1.0f / (float)HW);
 }

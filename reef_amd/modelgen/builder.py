@@ -403,10 +403,13 @@ class GraphBuilder:
                    4 * (x.size + out.size), 2.0)
         return out
 
-    def global_avgpool(self, x, out=None):
+    def global_avgpool(self, x, out=None, pre=None):
+        """pre: (scale, shift) parameters -- the input is read through relu(x * scale[c] + shift[c])."""
         C = x.shape[0]
         out = Tensor(out.idx, (C,)) if out is not None else self.temp((C,))
-        self._emit("reef_global_avgpool", math.ceil(C / 4), [x, out.idx], [C, x.size // C],
+        self._emit("reef_global_avgpool", math.ceil(C / 4),
+                   [x, out.idx] + ([pre[0].idx, pre[1].idx] if pre is not None else []),
+                   [C, x.size // C, 1 if pre is not None else 0],
                    "global_avgpool", 0, 4 * (x.size + C), 2.0)
         return out
 

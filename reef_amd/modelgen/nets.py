@@ -174,7 +174,8 @@ def densenet(blocks=(6, 12, 48, 32), growth=32, image=(3, 224, 224), classes=100
     and average are both linear and the filter is pointwise, so they commute: the pool reads the
     concatenation through the BN + ReLU and the filter runs on a quarter of the pixels, writing
     straight into the next block's buffer -- a quarter of the transition's multiplications, same
-    parameters in the same order.  False keeps the textbook order."""
+    parameters in the same order; the network's last BN + ReLU is applied by the global average
+    pool as it reads.  False keeps the textbook order and a launch for that BN + ReLU."""
     g = GraphBuilder(name, seed)
     x = g.input("data", image)
     fuse_stem = fuse_stem and image[0] <= 3
@@ -214,8 +215,11 @@ def densenet(blocks=(6, 12, 48, 32), growth=32, image=(3, 224, 224), classes=100
             else:
                 y = g.conv2d(x, c // 2, 1, 1, 0, bias=False, act=ACT_NONE, pre_act=True)
             c = c // 2
-    a = g.eltwise(x, scale=True, shift=True, act=ACT_RELU)
-    pooled = g.global_avgpool(a)
+    if pool_first:
+        pooled = g.global_avgpool(x, pre=g.pre_act_params(c))     # the last BN + ReLU on the way into the pool
+    else:
+        a = g.eltwise(x, scale=True, shift=True, act=ACT_RELU)
+        pooled = g.global_avgpool(a)
     logits = g.dense(pooled, classes, bias=True)
     out = g.softmax(logits, 1, classes)
     g.mark_output(out)

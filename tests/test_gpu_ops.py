@@ -693,12 +693,13 @@ def test_stem_convolution_and_pool_in_one_launch(tmp_path, case):
 def test_average_pool_reading_through_a_pre_activation(tmp_path):
     """reef_pool2d with REEF_POOL_F_PRE: relu(in * scale[c] + shift[c]) then a 2x2 average (what a
     DenseNet transition pools), and a 3x3 / stride 2 / padding 1 max-pool of the same with a bias
-    and ReLU behind it; odd sizes, against the oracle."""
+    and ReLU behind it, and the global average of the same (REEF_GAP_F_PRE); odd sizes, against the oracle."""
     g = MB.GraphBuilder("prepool")
     x = g.input("data", (37, 19, 23))
     ps, pt = g.pre_act_params(37)
     a = g.pool2d(x, 2, 2, 0, "avg", pre=(ps, pt))
     b = g.pool2d(x, 3, 2, 1, "max", bias=True, act=MB.ACT_RELU, pre=(ps, pt))
+    g.global_avgpool(x, pre=(ps, pt))
     g.mark_output(a)
     assert a.shape == (37, 9, 11) and b.shape == (37, 10, 12)
     exe, orc, model = run_both(g, tmp_path, {"data": rnd(37, 19, 23)})
