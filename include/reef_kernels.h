@@ -234,6 +234,9 @@ enum {
 #define REEF_F_IN_SHIFT 512    /* with REEF_F_POOL_OUTPUT: the input is read as in + shift[c] inside the image (the
                                   convolution's padding stays 0) */
 #define REEF_F_POOL_SHIFT 1024 /* with REEF_F_POOL_OUTPUT: out = act2(maxpool(..) + shift[channel]) */
+#define REEF_F_GAP_OUTPUT 2048 /* direct family, 1-tap or multi-tap, no split, N_TILES = 1 (the tile's pixel groups cover
+                                  the image): out is [Cout], the global average of what the layer would have written
+                                  (bias, residual, scale / shift and activation applied per element first) */
 #define REEF_CONV_MODE_GENERAL 0
 #define REEF_CONV_MODE_POINTWISE 1
 #define REEF_CONV_MODE_UNALIGNED 2

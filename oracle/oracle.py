@@ -330,6 +330,9 @@ class GraphOracle:
                 out = conv2d(xin, wgt, bias,
                              None if res is None else res[:Cout * Ho * Wo].reshape(Cout, Ho, Wo),
                              scale, shift, (sh, sw), (ph, pw), 1, act, 6.0, acc64)
+            if flags & 2048:      # the global average of the layer's output instead of the output
+                P[2][:Cout] = global_avgpool(out.reshape(Cout, -1))
+                return
             P[2][dst_off:dst_off + out.size] = out.reshape(-1)
             if out2 is not None:
                 out2[dst_off:dst_off + out.size] = eltwise(out.reshape(Cout, -1), shift=shift2[:Cout],

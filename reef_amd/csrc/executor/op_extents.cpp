@@ -160,7 +160,13 @@ void conv2d(const std::string& symbol, const Attrs& a, Needs& n) {
     }
     n.f32("input", cin * H * W);
     n.f32("weights", M * cin * kh * kw);
-    if (split > 1 && !fused) n.f32("partial sums", split * M * N);
+    if (flags & REEF_F_GAP_OUTPUT) {
+        if (mode != REEF_CONV_MODE_DIRECT || split != 1 || a[REEF_CONV_N_TILES] != 1 || off != 0 || (flags & REEF_F_DUAL)) {
+            n.bad = "the averaged output needs a direct kernel, no split, one pixel tile and a single output";
+            return;
+        }
+        n.f32("averaged output", M);
+    } else if (split > 1 && !fused) n.f32("partial sums", split * M * N);
     else n.f32("output", off + M * N);
     if (flags & REEF_F_BIAS) n.f32("bias", M);
     if (flags & REEF_F_RESIDUAL) n.f32("residual", M * N);

@@ -531,12 +531,16 @@ struct ConvEpilogue {
     }
     // off = (m * N + n) * 4 or outside; m4 = m * 4.  v = acc; v += residual; v += bias;
     // v = fma(v, scale, shift); act  -- then out2 = act2(out + shift2).
-    __device__ __forceinline__ void finish(float v, unsigned off, unsigned m4, float resv, float biasv,
-                                           float sh2v) const {
+    // the layer's value for one output element
+    __device__ __forceinline__ float value(float v, unsigned m4, float resv, float biasv) const {
         if (has_res) v = v + resv;
         if (has_bias) v = v + biasv;
         if (has_affine) v = fmaf(v, buf_load(scale, m4), buf_load(shift, m4));
-        const float o = act_apply(v, act);
+        return act_apply(v, act);
+    }
+    __device__ __forceinline__ void finish(float v, unsigned off, unsigned m4, float resv, float biasv,
+                                           float sh2v) const {
+        const float o = value(v, m4, resv, biasv);
         buf_store(out, off + doff4, o);
         if (has_dual) buf_store(out2, off + doff4, act_apply(o + sh2v, act2));
     }
@@ -1184,6 +1188,23 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
         return true;
     }
     if (!fused) {
+        if (flags & REEF_F_GAP_OUTPUT) {
+            // The global average of the layer's output instead of the output (a classifier's last
+            // convolution): one pixel tile covers the image, so the 16 lanes of an output row hold
+            // the whole row between them.  out[m] = sum over the pixels / N, pixels in ascending order
+            // within a lane, lanes folded pairwise.
+#pragma unroll
+            for (int h = 0; h < TM; ++h) {
+                float s = 0.0f;
+#pragma unroll
+                for (int g = 0; g < TN; ++g)
+                    if (ooff[h][g] != kOutside) s += ep.value(v[h][g], om[h] * 4u, e_res[h][g], e_bias[h]);
+#pragma unroll
+                for (int o = 1; o < 16; o <<= 1) s += __shfl_xor(s, o, 64);
+                if ((threadIdx.x & 15) == 0 && om[h] < (unsigned)M) buf_store(ep.out, om[h] * 4u, s * (1.0f / (float)N));
+            }
+            return true;
+        }
 #pragma unroll
         for (int h = 0; h < TM; ++h)
 #pragma unroll

@@ -25,7 +25,7 @@ from ..paths import code_object
 
 ACT_NONE, ACT_RELU, ACT_RELU6, ACT_GELU = 0, 1, 2, 3
 F_BIAS, F_RESIDUAL, F_AFFINE, F_DUAL, F_FUSED_REDUCE, F_PRE_ACT, F_PAIR_FOLD, F_DW_OUTPUT = 1, 2, 4, 8, 16, 32, 64, 128
-F_POOL_OUTPUT, F_IN_SHIFT, F_POOL_SHIFT = 256, 512, 1024
+F_POOL_OUTPUT, F_IN_SHIFT, F_POOL_SHIFT, F_GAP_OUTPUT = 256, 512, 1024, 2048
 WG = 256
 
 
@@ -157,8 +157,10 @@ class GraphBuilder:
 
     def conv2d(self, x, cout, k, stride=1, pad=0, bias=True, act=ACT_RELU, residual=None,
                affine=False, force=None, dual_act=None, fused_reduce=None, out=None, out_channel=0,
-               pre_act=False, given=None, out2=None):
+               pre_act=False, given=None, out2=None, gap=False):
         """Fused conv + (residual) + (bias) + (scale, shift) + activation on MFMA.
+        gap: return the global average of the layer's output, a (cout,) tensor, instead of the
+        output (direct tiles whose pixel groups cover the image: Ho * Wo <= 64; no split).
         pre_act: the layer reads its input through a per-channel scale, shift and ReLU of its own
         (DenseNet pre-activation); folded into the convolution's input loads where a kernel for it
         exists (1x1 filters on the direct tiles), a separate elementwise launch otherwise.
@@ -217,6 +219,14 @@ class GraphBuilder:
             opt.append(out2.idx)
             opt.append(self.param((cout,), 0.01).idx)
         act2 = dual_act or ACT_NONE
+        if gap:
+            assert out.idx is not None and dual_act is None and not pre_act and dst_off == 0
+            tile = self.gap_tile(cin, kh, kw, N)
+            assert tile is not None, "no direct tile covers this image"
+            force = tiling.forced(tile, M, N, K, 1, kh * kw)
+            flags |= F_GAP_OUTPUT
+            self.storage[out.idx]["size"] = cout            # the storage holds the averages only
+            out = Tensor(out.idx, (cout,))
         t = force or tiling.choose(M, N, K, fused=fused_reduce, pointwise=(kh, kw) == (1, 1),
                                    taps=kh * kw, direct=tiling.direct_ok(cin, kh, kw),
                                    rows=tiling.rows_ok(kh, kw, sh, sw, ph, pw), image=(Ho, Wo))
@@ -297,6 +307,14 @@ class GraphBuilder:
                        [M, N, t["split_k"], flags & ~F_PRE_ACT, act, act2, dst_off], "splitk_reduce", 0,
                        4 * ((t["split_k"] + 1) * M * N), 2.0)
         return out if out2 is None else (out, out2)
+
+    @staticmethod
+    def gap_tile(cin, kh, kw, n_pixels):
+        """The narrowest direct tile whose pixel groups cover an image of n_pixels, or None."""
+        for tile in ("16x16k4", "16x32k4", "16x64k4"):
+            if tiling.TILES[tile][2] >= n_pixels and tiling.direct_ok(cin, kh, kw, tile):
+                return tile
+        return None
 
     def conv2d_pool(self, x, cout, act=ACT_RELU, in_shift=False, pool_shift=False, pool_act=ACT_NONE, out=None):
         """7x7 / stride 2 / padding 3 convolution (+ bias, act) of an image of at most 3 channels and the

@@ -36,7 +36,7 @@ def image_input(name, shape, seed=rng.BASE_SEED):
 
 
 def resnet(num_layers=152, image=(3, 224, 224), classes=1000, name=None, seed=rng.BASE_SEED,
-           fused_reduce=False, fuse_act=True, stack_first=True, fuse_stem=True):
+           fused_reduce=False, fuse_act=True, stack_first=True, fuse_stem=True, fuse_gap=False):
     """fused_reduce: fold split-K inside the conv kernels.  fuse_act: let the unit's last
     conv also write the next unit's activated input (one kernel instead of conv + add/relu).
     The first unit of a bottleneck stage has two 1x1 convolutions on the same input with the same
@@ -64,7 +64,7 @@ def resnet(num_layers=152, image=(3, 224, 224), classes=1000, name=None, seed=rn
         x = g.eltwise(data, shift=True)                                  # bn_data (shift only)
         x = g.conv2d(x, filters[0], 7, 2, 3, bias=True, act=ACT_RELU)    # conv0 + bn0 + relu
         act = g.pool2d(x, 3, 2, 1, "max", bias=True, act=ACT_RELU)       # pool + first bn1 + relu
-    raw = None
+    raw = pooled = None
     n_stages = len(units)
     for si in range(n_stages):
         cout = filters[si + 1]
@@ -89,8 +89,11 @@ def resnet(num_layers=152, image=(3, 224, 224), classes=1000, name=None, seed=rn
                 shortcut = g.conv2d(act, cout, 1, stride, 0, bias=False, act=ACT_NONE) if first else raw
                 last_k, last_p = 3, 1
             if last_of_net:
+                # fuse_gap: the network's last convolution averages its own output (one pixel tile covers 7 x 7)
+                gap = fuse_gap and GraphBuilder.gap_tile(y.shape[0], last_k, last_k, y.shape[1] * y.shape[2]) is not None
                 act = g.conv2d(y, cout, last_k, 1, last_p, bias=False, act=ACT_RELU,
-                               residual=shortcut, affine=True)
+                               residual=shortcut, affine=True, gap=gap)
+                pooled = act if gap else None
             elif last_of_stage:
                 act = g.conv2d(y, cout, last_k, 1, last_p, bias=True, act=ACT_RELU,
                                residual=shortcut)
@@ -101,7 +104,8 @@ def resnet(num_layers=152, image=(3, 224, 224), classes=1000, name=None, seed=rn
                 raw = g.conv2d(y, cout, last_k, 1, last_p, bias=False, act=ACT_NONE,
                                residual=shortcut)
                 act = g.eltwise(raw, shift=True, act=ACT_RELU)
-    pooled = g.global_avgpool(act)
+    if pooled is None:
+        pooled = g.global_avgpool(act)
     logits = g.dense(pooled, classes, bias=True)
     out = g.softmax(logits, 1, classes)
     g.mark_output(out)
@@ -123,7 +127,8 @@ def mocked_kernel(name="mocked_kernel"):
     return g
 
 
-def mobilenet_v2(image=(3, 224, 224), classes=1000, name="mobilenetv2", seed=rng.BASE_SEED, fuse_expand_dw=True):
+def mobilenet_v2(image=(3, 224, 224), classes=1000, name="mobilenetv2", seed=rng.BASE_SEED, fuse_expand_dw=True,
+                 fuse_gap=True):
     """MobileNetV2, width 1.0: 3x3/2 stem, 17 inverted-residual blocks (1x1 expand + ReLU6,
     depthwise 3x3 + ReLU6, linear 1x1 projection, residual add when stride 1 and equal
     channels), 1x1 to 1280, global average pool, classifier.  Batch norms are folded
@@ -153,8 +158,12 @@ def mobilenet_v2(image=(3, 224, 224), classes=1000, name="mobilenetv2", seed=rng
             res = x if (stride == 1 and cin == c) else None
             x = g.conv2d(y, c, 1, 1, 0, bias=True, act=ACT_NONE, residual=res)
             cin = c
-    x = g.conv2d(x, 1280, 1, 1, 0, bias=True, act=ACT_RELU6)
-    pooled = g.global_avgpool(x)
+    # fuse_gap: the last convolution averages its own output where one pixel tile covers the image
+    if fuse_gap and GraphBuilder.gap_tile(cin, 1, 1, x.shape[1] * x.shape[2]) is not None:
+        pooled = g.conv2d(x, 1280, 1, 1, 0, bias=True, act=ACT_RELU6, gap=True)
+    else:
+        x = g.conv2d(x, 1280, 1, 1, 0, bias=True, act=ACT_RELU6)
+        pooled = g.global_avgpool(x)
     logits = g.dense(pooled, classes, bias=True)
     out = g.softmax(logits, 1, classes)
     g.mark_output(out)

@@ -515,12 +515,12 @@ def test_mobilenetv2_with_and_without_the_fused_front_half(tmp_path):
     x = nets.image_input("mobilenetv2", (3, 224, 224))
     outs = []
     for fuse in (False, True):
-        g = nets.mobilenet_v2(fuse_expand_dw=fuse)
+        g = nets.mobilenet_v2(fuse_expand_dw=fuse, fuse_gap=fuse)
         exe, orc, model = run_both(g, tmp_path / str(fuse), {"data": x})
         compare_storages(exe, orc, model, what="mobilenetv2 fuse=%s" % fuse)
         li = model["kernels"][-1]["args"][0]
         outs.append((len(g.kernels), exe.get_data(li, model["storage"][li]["size"])))
-    assert outs[0][0] == 55 and outs[1][0] == 40
+    assert outs[0][0] == 55 and outs[1][0] == 39      # fused: expansion + depthwise, and the last convolution averages
     from tests.helpers import max_rel_err, REL_TOL
     assert max_rel_err(outs[1][1], outs[0][1]) <= REL_TOL
 
@@ -704,3 +704,41 @@ def test_average_pool_reading_through_a_pre_activation(tmp_path):
     assert a.shape == (37, 9, 11) and b.shape == (37, 10, 12)
     exe, orc, model = run_both(g, tmp_path, {"data": rnd(37, 19, 23)})
     compare_storages(exe, orc, model, what="pool with pre-activation")
+
+
+@pytest.mark.parametrize("case", [(320, 7, 7, 1280, 1, 0, False, False), (64, 5, 6, 40, 1, 0, True, True),
+                                  (48, 4, 4, 24, 3, 1, True, False), (32, 3, 5, 16, 1, 0, False, False)])
+def test_convolution_that_averages_its_own_output(tmp_path, case):
+    """REEF_F_GAP_OUTPUT: a direct kernel whose pixel groups cover the image writes the global
+    average of what it would have written (bias, residual, scale / shift, activation first);
+    against the oracle and against convolution + average pool as two launches; the three flavours
+    bit for bit."""
+    from reef_amd import binding as B
+    from tests.helpers import write_model, max_rel_err, REL_TOL
+    cin, H, W, cout, k, pad, residual, affine = case
+
+    def build(gap):
+        g = MB.GraphBuilder("gapconv")
+        x = g.input("data", (cin, H, W))
+        r = g.input("res", (cout, H, W)) if residual else None
+        y = g.conv2d(x, cout, k, 1, pad, bias=not affine, act=MB.ACT_RELU6, residual=r, affine=affine, gap=gap)
+        g.mark_output(y if gap else g.global_avgpool(y))
+        return g
+    g, g2 = build(True), build(False)
+    assert len(g.kernels) == 1 and len(g2.kernels) == 2 and g.kernels[0]["attrs"][12] & 2048
+    inputs = {"data": rnd(cin, H, W)}
+    if residual:
+        inputs["res"] = rnd(cout, H, W)
+    exe, orc, model = run_both(g, tmp_path / "one", inputs)
+    compare_storages(exe, orc, model, what="gap conv %s" % (case,))
+    want = exe.get_output()[:cout].copy()
+    exe2, _, _ = run_both(g2, tmp_path / "two", inputs)
+    assert max_rel_err(want, exe2.get_output()[:cout]) <= REL_TOL
+    d = write_model(g, tmp_path / "one")
+    for kind, pre in ((B.TRANS, False), (B.HYBRID, True), (B.HYBRID, False)):
+        e = B.Executor.from_dir(d, g.name, kind)
+        for name, arr in inputs.items():
+            e.set_input_checked(name, arr)
+        e.execute_preemptable() if pre else e.execute()
+        np.testing.assert_array_equal(e.get_output()[:cout], want, err_msg="flavour %s %s" % (kind, pre))
+        e.close()
