@@ -350,6 +350,10 @@ REEF_ENTRY(reef_conv2d_d9k_16x32k4, OpConvDirectK<9 REEF_COMMA 2>)
 REEF_ENTRY(reef_conv2d_d9k_32x32d4, OpConvDirectK<9 REEF_COMMA 2 REEF_COMMA 2>)
 REEF_ENTRY(reef_conv2d_d3k_16x16k4, OpConvDirectK<3>)
 REEF_ENTRY(reef_conv2d_d3k_16x32k4, OpConvDirectK<3 REEF_COMMA 2>)
+REEF_ENTRY(reef_conv2d_d25_16x16k4, OpConvDirect<25>)
+REEF_ENTRY(reef_conv2d_d25_16x32k4, OpConvDirect<25 REEF_COMMA 2>)
+REEF_ENTRY(reef_conv2d_d25k_16x16k4, OpConvDirectK<25>)
+REEF_ENTRY(reef_conv2d_d25k_16x32k4, OpConvDirectK<25 REEF_COMMA 2>)
 REEF_ENTRY(reef_conv2d_d7k_16x16k4, OpConvDirectK<7>)
 REEF_ENTRY(reef_conv2d_d7k_16x32k4, OpConvDirectK<7 REEF_COMMA 2>)
 REEF_ENTRY(reef_conv2d_xdw_g2, OpConvXdw<2>)

@@ -725,7 +725,7 @@ class GraphBuilder:
 # (loader family prefix, tile) of the kernels that exist in a packed-weights form
 PACKED_KERNELS = {("r9_", "g1"), ("r9_", "g2"), ("r9_", "g4"), ("d9_", "16x16k4"), ("d9_", "16x32k4"),
                   ("d9_", "32x32d4"), ("d3_", "16x16k4"), ("d3_", "16x32k4"), ("d7_", "16x16k4"),
-                  ("d7_", "16x32k4")}
+                  ("d7_", "16x32k4"), ("d25_", "16x16k4"), ("d25_", "16x32k4")}
 
 
 def pack_conv_weights(w):

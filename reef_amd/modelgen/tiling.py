@@ -45,7 +45,7 @@ DIRECT_TILE = "16x16k4"
 DIRECT_TILES = ("16x16k4", "16x32k4", "16x64k4", "32x32d4")
 # filter sizes kh*kw each direct tile is compiled for
 PRE_ACT_TILES = ("16x16k4", "16x32k4", "32x32d4")   # tiles with a pre-activation 1x1 kernel (reef_conv2d_p1_*)
-DIRECT_TAPS = {"16x16k4": (1, 3, 7, 9), "16x32k4": (1, 3, 7, 9), "16x64k4": (1, 9), "32x32d4": (1, 9)}
+DIRECT_TAPS = {"16x16k4": (1, 3, 7, 9, 25), "16x32k4": (1, 3, 7, 9, 25), "16x64k4": (1, 9), "32x32d4": (1, 9)}
 # wavefronts that share one output block and split K inside the workgroup
 KW = {"32x32k4": 4, "64x32k2": 2, "32x64k2": 2}
 GEMM_TILES = ("128x128", "64x64", "32x128", "32x32k4", "64x32k2")

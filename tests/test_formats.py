@@ -283,7 +283,8 @@ def test_direct_tile_geometry():
     f = tiling.forced("32x32d4", 256, 196, 2304, 4, 9)
     assert (f["m_tiles"], f["n_tiles"], f["split_k"], f["tasks"]) == (8, 7, 4, 224)
     assert tiling.lds_bytes("32x32d4") == 4 * 4 * 320 * 4 + 16
-    assert not tiling.direct_ok(3, 7, 7) and not tiling.direct_ok(20, 1, 1) and not tiling.direct_ok(16, 5, 5)
+    assert not tiling.direct_ok(3, 7, 7) and not tiling.direct_ok(20, 1, 1) and not tiling.direct_ok(16, 4, 4)
+    assert tiling.direct_ok(48, 5, 5) and tiling.direct_ok(48, 5, 5, "16x32k4") and not tiling.direct_ok(48, 5, 5, "32x32d4")
     # the analytic model never picks the direct tile; only the measured table may, and only
     # when the caller vouches for the filter
     t = tiling.choose(256, 196, 2304, fused=False, pointwise=False, taps=9, direct=False)

@@ -444,7 +444,9 @@ def test_attention_in_one_launch(tmp_path, seq, heads, hd, masked):
     pr /= pr.sum(-1, keepdims=True)
     want = np.einsum("hst,thd->shd", pr, m[:, 2]).reshape(seq, hid)
     got = exe.get_data(ctx.idx, seq * hid).reshape(seq, hid)
-    assert np.isfinite(got).all() and np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
+    # scores of magnitude 100 (weights of deviation 0.2 on 768 inputs) carry 1e-5 of absolute error in
+    # fp32, which the exponential turns into that much relative error: the suite's 1e-4, not less
+    assert np.isfinite(got).all() and np.abs(got - want).max() <= 1e-4 * np.abs(want).max()
 
 
 def test_mocked_model_closed_form(tmp_path):

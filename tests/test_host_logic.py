@@ -467,7 +467,7 @@ def test_tile_choice_outside_the_measured_table():
     assert t["tile"] not in tiling.DIRECT_TILES and t["tile"] not in tiling.ROW_TILES
     t = tiling.choose(512, 200 * 200, 4608, fused=True, taps=9, direct=True)
     assert t["tile"] not in tiling.DIRECT_TILES          # 40000 pixels x 512 channels fill the device
-    t = tiling.choose(96, 500, 25 * 40, fused=True, taps=25, direct=tiling.direct_ok(40, 5, 5))
+    t = tiling.choose(96, 500, 16 * 40, fused=True, taps=16, direct=tiling.direct_ok(40, 4, 4))
     assert t["tile"] not in tiling.DIRECT_TILES
     # both models answer in microseconds of one launch
     g = tiling.forced("16x32k4", 256, 196, 1024, 2, 1)
