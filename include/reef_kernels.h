@@ -182,6 +182,8 @@ enum {
     REEF_CONV_M_TILES, REEF_CONV_N_TILES,
     REEF_CONV_ACT2,      /* activation of the second output (REEF_F_DUAL) */
     REEF_CONV_SYNC_OFF,  /* first counter of this launch inside the sync storage (ints) */
+#define REEF_CONV_PROJ REEF_CONV_SYNC_OFF /* REEF_F_PROJ_OUTPUT (a launch without counters): the slot carries the
+                                             output channels of the projection behind the depthwise stage */
     REEF_CONV_MODE,      /* REEF_CONV_MODE_*: must match the entry symbol's family */
     REEF_CONV_DST_OFF,   /* element offset added to dst (and out2): channel slice of a concat buffer */
     REEF_CONV_WPACK,     /* pointer slot of the packed copy of the weights (symbols ...d<R>k_ / r9k_), else 0:
@@ -237,6 +239,18 @@ enum {
 #define REEF_F_GAP_OUTPUT 2048 /* direct family, 1-tap or multi-tap, no split, N_TILES = 1 (the tile's pixel groups cover
                                   the image): out is [Cout], the global average of what the layer would have written
                                   (bias, residual, scale / shift and activation applied per element first) */
+#define REEF_F_PROJ_OUTPUT 4096 /* with REEF_F_DW_OUTPUT, symbols reef_conv2d_sdp_g<G> and reef_conv2d_xdp2_g<G>: a 1x1
+                                  projection (+ bias, no activation) behind the depthwise stage in the same launch -- a
+                                  whole MobileNetV2 block, for blocks of few channels (COUT = the middle channels <= 32
+                                  resp. 96, REEF_CONV_PROJ = P <= 32 output channels; out is [P][HO][WO]).  The front
+                                  filter is either the network's 3x3 / stride 2 / padding 1 stem on at most 3 channels
+                                  (sdp: KH = KW = 3, SH = SW = 2, PH = PW = 1, depthwise stride 1) or a 1x1 expansion
+                                  of at most 16 channels (xdp2: KH = KW = 1, SH = SW = 2 = the depthwise stride; CIN a
+                                  multiple of 4, W even).  COUT is a multiple of 4.  ptr:
+                                  in, W, out, bias, depthwise weights [COUT][9], depthwise bias [COUT], projection
+                                  weights [P][COUT], projection bias [P].  A workgroup holds every channel of its G
+                                  output rows x 14 columns: M_TILES = 1, N_TILES = ceil(HO / G) * ceil(WO / 14),
+                                  TILE = REEF_TILE_R9G<G>, no split. */
 #define REEF_CONV_MODE_GENERAL 0
 #define REEF_CONV_MODE_POINTWISE 1
 #define REEF_CONV_MODE_UNALIGNED 2
@@ -244,6 +258,8 @@ enum {
 #define REEF_CONV_MODE_DIRECT_PRE 4   /* direct, 1 tap, with REEF_F_PRE_ACT (reef_conv2d_p1_<tile>) */
 #define REEF_CONV_MODE_SP7 7          /* 7x7 stride-2 convolution + 3x3 stride-2 max-pool (reef_conv2d_sp7_g2, REEF_F_POOL_OUTPUT) */
 #define REEF_CONV_MODE_XDW 6          /* 1x1 filter + depthwise 3x3 behind it (reef_conv2d_xdw_g<G>, REEF_F_DW_OUTPUT) */
+#define REEF_CONV_MODE_BLOCK 8        /* front filter + depthwise 3x3 + 1x1 projection (reef_conv2d_sdp_g<G>, reef_conv2d_xdp2_g<G>,
+                                         REEF_F_DW_OUTPUT | REEF_F_PROJ_OUTPUT) */
 #define REEF_CONV_MODE_ROWS 5         /* direct, row form: 3x3 / stride 1 / padding 1 (reef_conv2d_r9_g<G>[m2]).
                                          The output tile is 16 (m2: 32) channels x G image rows x one 14-column
                                          segment; N_TILES = ceil(Ho / G) * ceil(Wo / 14), spatial tile index =

@@ -306,14 +306,21 @@ class GraphOracle:
             # single pass, or split-K folded inside the kernel (workspace untouched here)
             bias, res, scale, shift, out2, shift2 = self._conv_opt(P, 3, flags)
             if flags & 128:
-                # a depthwise 3x3 stage (padding 1, + bias, activation act2) behind the 1x1 filter, in
-                # the same launch; its weights and bias follow the optional operands.  The stride
-                # attributes are the depthwise stage's; the 1x1 filter itself has stride 1.
+                # a depthwise 3x3 stage (padding 1, + bias, activation act2) behind the front filter, in
+                # the same launch; its weights and bias follow the optional operands.  Behind a 1x1 front
+                # filter the stride attributes are the depthwise stage's and the filter has stride 1;
+                # behind a larger one they are the filter's and the depthwise stage has stride 1.
                 pos = 3 + bool(flags & 1) + bool(flags & 2) + 2 * bool(flags & 4) + 2 * bool(flags & 8)
-                mid = conv2d(xin, wgt, bias, None, None, None, (1, 1), (ph, pw), 1, act, 6.0, acc64)
-                out = conv2d(mid, P[pos][:Cout * 9].reshape(Cout, 1, 3, 3), P[pos + 1][:Cout], stride=(sh, sw),
+                front, behind = ((1, 1), (sh, sw)) if kh == 1 and kw == 1 else ((sh, sw), (1, 1))
+                mid = conv2d(xin, wgt, bias, None, None, None, front, (ph, pw), 1, act, 6.0, acc64)
+                out = conv2d(mid, P[pos][:Cout * 9].reshape(Cout, 1, 3, 3), P[pos + 1][:Cout], stride=behind,
                              pad=(1, 1), groups=Cout, act=act2, acc64=acc64)
                 assert out.shape == (Cout, Ho, Wo)
+                if flags & 4096:
+                    # and a linear 1x1 projection (+ bias) behind that; such a launch has no counters and
+                    # the slot of the first counter carries the projection's output channels
+                    Pn = a[20]
+                    out = conv2d(out, P[pos + 2][:Pn * Cout].reshape(Pn, Cout, 1, 1), P[pos + 3][:Pn], acc64=acc64)
             elif flags & 256:
                 # a 3x3 / stride 2 / padding 1 max-pool behind the convolution in the same launch (Ho, Wo
                 # are the pooled sizes); optionally a per-channel shift on the input -- inside the image,

@@ -121,6 +121,26 @@ void conv2d(const std::string& symbol, const Attrs& a, Needs& n) {
                flags == (REEF_F_BIAS | REEF_F_DW_OUTPUT) && off == 0 && a[REEF_CONV_M_TILES] == cdiv(M, 16) &&
                a[REEF_CONV_N_TILES] == cdiv(Ho, G) * cdiv(Wo, 14) && a[REEF_CONV_ACT] <= REEF_ACT_RELU6 &&
                a[REEF_CONV_ACT2] <= REEF_ACT_RELU6;
+    } else if (fam.compare(0, 4, "sdp_") == 0 || fam.compare(0, 5, "xdp2_") == 0) {
+        // a whole block in one launch, every channel in one workgroup: front filter (sdp: the 3x3 / stride 2 /
+        // padding 1 stem on at most 3 channels, depthwise stride 1; xdp2: a 1x1 expansion of at most 16
+        // channels, SH = SW = 2 the depthwise stride), depthwise 3x3, projection to REEF_CONV_PROJ channels.
+        // The kernels move the middle channels in fours, xdp2 also its input channels, and its input
+        // columns in pairs.
+        mode = REEF_CONV_MODE_BLOCK;
+        const bool stem = fam[0] == 's';
+        const i64 G = a[REEF_CONV_TILE] == REEF_TILE_R9G1 ? 1 : a[REEF_CONV_TILE] == REEF_TILE_R9G2 ? 2
+                    : a[REEF_CONV_TILE] == REEF_TILE_R9G4 ? 4 : 0;
+        const std::string want = std::string(stem ? "sdp_g" : "xdp2_g") + (char)('0' + G);
+        const bool front = stem ? kh == 3 && kw == 3 && a[REEF_CONV_PH] == 1 && a[REEF_CONV_PW] == 1 && cin <= 3 &&
+                                      M <= 32 && (G == 2 || G == 4)
+                                : kh == 1 && kw == 1 && a[REEF_CONV_PH] == 0 && a[REEF_CONV_PW] == 0 && cin <= 16 &&
+                                      cin % 4 == 0 && W % 2 == 0 && M <= 96 && (G == 1 || G == 2);
+        fits = front && M % 4 == 0 && a[REEF_CONV_SH] == 2 && a[REEF_CONV_SW] == 2 && fam == want && split == 1 && off == 0 &&
+               flags == (REEF_F_BIAS | REEF_F_DW_OUTPUT | REEF_F_PROJ_OUTPUT) && a[REEF_CONV_PROJ] >= 1 &&
+               a[REEF_CONV_PROJ] <= 32 && a[REEF_CONV_M_TILES] == 1 &&
+               a[REEF_CONV_N_TILES] == cdiv(Ho, G) * cdiv(Wo, 14) && a[REEF_CONV_ACT] <= REEF_ACT_RELU6 &&
+               a[REEF_CONV_ACT2] <= REEF_ACT_RELU6;
     } else if (fam == "sp7_g2") {
         // 7x7 / stride 2 / padding 3 convolution of at most 3 channels and the 3x3 / stride 2 / padding 1
         // max-pool behind it in one launch; HO, WO are the pooled sizes
@@ -147,7 +167,8 @@ void conv2d(const std::string& symbol, const Attrs& a, Needs& n) {
         fits = compiled == taps && (taps > 1 || cin % 8 == 0);
     }
     if (!fits || mode != a[REEF_CONV_MODE] || ((flags & REEF_F_PRE_ACT) != 0) != (mode == REEF_CONV_MODE_DIRECT_PRE) ||
-        ((flags & REEF_F_DW_OUTPUT) != 0) != (mode == REEF_CONV_MODE_XDW) ||
+        ((flags & REEF_F_DW_OUTPUT) != 0) != (mode == REEF_CONV_MODE_XDW || mode == REEF_CONV_MODE_BLOCK) ||
+        ((flags & REEF_F_PROJ_OUTPUT) != 0) != (mode == REEF_CONV_MODE_BLOCK) ||
         ((flags & REEF_F_POOL_OUTPUT) != 0) != (mode == REEF_CONV_MODE_SP7) ||
         ((flags & (REEF_F_IN_SHIFT | REEF_F_POOL_SHIFT)) != 0 && mode != REEF_CONV_MODE_SP7)) {
         n.bad = "the layer is not one that this symbol's loader family was compiled for";
@@ -167,6 +188,7 @@ void conv2d(const std::string& symbol, const Attrs& a, Needs& n) {
         }
         n.f32("averaged output", M);
     } else if (split > 1 && !fused) n.f32("partial sums", split * M * N);
+    else if (mode == REEF_CONV_MODE_BLOCK) n.f32("output", a[REEF_CONV_PROJ] * N);
     else n.f32("output", off + M * N);
     if (flags & REEF_F_BIAS) n.f32("bias", M);
     if (flags & REEF_F_RESIDUAL) n.f32("residual", M * N);
@@ -174,6 +196,7 @@ void conv2d(const std::string& symbol, const Attrs& a, Needs& n) {
     if (flags & REEF_F_DUAL) { n.f32("second output", off + M * N); n.f32("second shift", M); }
     if (flags & REEF_F_PRE_ACT) { n.f32("input scale", cin); n.f32("input shift", cin); }
     if (flags & REEF_F_DW_OUTPUT) { n.f32("depthwise weights", M * 9); n.f32("depthwise bias", M); }
+    if (flags & REEF_F_PROJ_OUTPUT) { n.f32("projection weights", a[REEF_CONV_PROJ] * M); n.f32("projection bias", a[REEF_CONV_PROJ]); }
     if (flags & REEF_F_IN_SHIFT) n.f32("input shift", cin);
     if (flags & REEF_F_POOL_SHIFT) n.f32("pool shift", M);
     if (fused) {

@@ -62,6 +62,16 @@ struct OpConvXdw {
         return conv2d_xdw_body<G, S>(d, task, smem, p);
     }
 };
+// front filter (STEM: 3x3 / stride 2 on the image, else a 1x1 expansion), depthwise 3x3 (stride S) and 1x1
+// projection in one launch, every channel in one workgroup
+template <int G, int S, bool STEM, int MT, int KC>
+struct OpConvBlock {
+    static constexpr int LDS = TileBlk<G, S, STEM, MT, KC>::LDS_BYTES;
+    template <class P>
+    static __device__ __forceinline__ bool run(const ReefOpDesc& d, int task, char* smem, const P& p) {
+        return conv2d_block_body<G, S, STEM, MT, KC>(d, task, smem, p);
+    }
+};
 // 7x7 stride-2 convolution and the 3x3 stride-2 max-pool behind it in one launch
 struct OpConvStemPool {
     static constexpr int LDS = TileSp7::LDS_BYTES;
@@ -359,6 +369,10 @@ REEF_ENTRY(reef_conv2d_d7k_16x32k4, OpConvDirectK<7 REEF_COMMA 2>)
 REEF_ENTRY(reef_conv2d_xdw_g2, OpConvXdw<2>)
 REEF_ENTRY(reef_conv2d_xdw_g4, OpConvXdw<4>)
 REEF_ENTRY(reef_conv2d_sp7_g2, OpConvStemPool)
+REEF_ENTRY(reef_conv2d_sdp_g2, OpConvBlock<2 REEF_COMMA 1 REEF_COMMA true REEF_COMMA 2 REEF_COMMA 1>)
+REEF_ENTRY(reef_conv2d_sdp_g4, OpConvBlock<4 REEF_COMMA 1 REEF_COMMA true REEF_COMMA 2 REEF_COMMA 1>)
+REEF_ENTRY(reef_conv2d_xdp2_g1, OpConvBlock<1 REEF_COMMA 2 REEF_COMMA false REEF_COMMA 6 REEF_COMMA 4>)
+REEF_ENTRY(reef_conv2d_xdp2_g2, OpConvBlock<2 REEF_COMMA 2 REEF_COMMA false REEF_COMMA 6 REEF_COMMA 4>)
 REEF_ENTRY(reef_conv2d_xdw2_g2, OpConvXdw<2 REEF_COMMA 2>)
 REEF_ENTRY(reef_gemm_nt_128x128, OpGemm<Tile128x128 REEF_COMMA true>)
 REEF_ENTRY(reef_gemm_nt_64x64, OpGemm<Tile64x64 REEF_COMMA true>)

@@ -1472,6 +1472,360 @@ __device__ __forceinline__ bool conv2d_xdw_body(const ReefOpDesc& d, int task, c
     return true;
 }
 
+// ---- reef_conv2d_sdp_g<G> / reef_conv2d_xdp2_g<G>: a whole MobileNetV2 block in one launch -------
+// front filter (+ bias, activation) -> depthwise 3x3 filter (padding 1, + bias, activation) -> 1x1
+// projection (+ bias, linear), for the blocks at the head of the network, whose images are large
+// and whose channels are few: every tensor between the three layers is several times the block's
+// input or output (32 and 96 channels at 112 x 112 against 3 in and 16 or 24 out), and with so
+// few channels a workgroup can hold ALL of them for its pixels.  A workgroup owns G output rows x
+// one 14-column segment x every channel; nothing is split, nobody waits for anybody.
+//   STEM   the front filter is the network's first layer: 3x3, stride 2, padding 1 on at most 3
+//          channels (K = 27: what neighbouring tiles compute twice costs nothing); the depthwise
+//          stage has stride 1.
+//   !STEM  the front filter is a 1x1 expansion of at most 4 KC channels; the depthwise stage has
+//          stride S.
+//   phase 0  the input patch and the parameters of the first two layers into LDS, all loads of a
+//            thread on their way before its first store (zero where the image or a channel ends).
+//   phase 1  the front filter on the matrix cores, operands from LDS; pixel groups as in
+//            reef_conv2d_xdw (S = 1: group r = row y0 - 1 + r of the front filter's result, lanes
+//            0..13 the segment's columns, lane 14 the column right of it, lane 15 the one left;
+//            S = 2: rows 2 y0 - 1 + r as an even-column and an odd-column group).  + bias,
+//            activation, 0 outside the image (the depthwise padding) -> E in LDS.  The wavefronts
+//            share the (channel tile, pixel group) pairs.
+//   phase 2  thread (channel, column) forms the depthwise outputs of its G rows, a channel tile
+//            at a time, taps in filter order, then bias and activation -> D in LDS.
+//   phase 3  the projection on the matrix cores from D, its weights waiting in registers since the
+//            kernel's start, + bias, store.
+// ptr: in [Cin][H][W], front weights [Cmid][Cin][KH][KW], out [P][Ho][Wo], front bias [Cmid],
+// depthwise weights [Cmid][9], depthwise bias [Cmid], projection weights [P][Cmid], projection
+// bias [P].  attr: COUT = Cmid (<= 16 MT), REEF_CONV_PROJ = P (<= 32); H, W the input; HO, WO the
+// output; KH = KW = 3, SH = SW = 2, PH = PW = 1 (STEM: the front filter's) or KH = KW = 1, SH = SW
+// = S, PH = PW = 0 (the depthwise stride, as for reef_conv2d_xdw); ACT, ACT2 the front filter's
+// and the depthwise stage's activation; flags REEF_F_BIAS | REEF_F_DW_OUTPUT | REEF_F_PROJ_OUTPUT;
+// M_TILES = 1, N_TILES = ceil(Ho / G) * ceil(Wo / 14) = tasks.
+template <int G, int S, bool STEM, int MT, int KC>
+struct TileBlk {
+    static constexpr int R = S == 1 ? G + 2 : 2 * G + 1;    // rows of the front filter's result a tile needs
+    static constexpr int NG = R * S;                         // pixel groups of 16 lanes: S per row
+    static constexpr int CM = MT * 16, CP = 32;              // most middle channels, most output channels
+    // k slot (s, lane / 16) of an MFMA stands for tap resp. channel (lane / 16) * KF + s in phase 1 and
+    // for channel (lane / 16) * KP + s in phase 3: what a lane multiplies is contiguous in memory
+    static constexpr int KF = STEM ? 7 : KC, KP = MT * 4;
+    static constexpr int WFS = STEM ? 36 : 4 * KC + 4;       // floats per channel of the front weights ([lane / 16][KF], 4 mod 32: banks)
+    static constexpr int PR = 2 * R + 1, PCS = 36;           // STEM: patch rows per channel, row stride (33 columns)
+    static constexpr int PS = 4 * KC + 4;                    // !STEM: floats per pixel of the input patch [pixel][channel]
+    static constexpr int PATCH = STEM ? 3 * PR * PCS : NG * 16 * PS;
+    // floats per channel of E [channel][pixel]: 20 mod 32, so that the 4 x 16 values a wavefront writes
+    // (channels 4 apart) and the 4 x 16 it reads (consecutive channels) each meet every bank twice
+    static constexpr int ESTRIDE = NG * 16 + (NG % 2 == 0 ? 20 : 4);
+    static constexpr int DPS = CM + 4;                       // floats per pixel of D [pixel][channel]
+    static constexpr int MH = MT / 2, GH = NG / 2;           // phase 1: a wavefront's channel tiles x pixel groups
+    // LDS map (floats; every block starts on 16 bytes)
+    static constexpr int O_WF = PATCH, O_BF = O_WF + CM * WFS, O_WD = O_BF + CM, O_BD = O_WD + CM * 9;
+    static constexpr int O_BP = O_BD + CM, O_E = O_BP + CP, O_D = O_E + CM * ESTRIDE;
+    static constexpr int FLOATS = O_D + G * 16 * DPS;
+    static constexpr int LDS_BYTES = FLOATS * 4 + 16;
+    static_assert(MT % 2 == 0 && NG % 2 == 0, "the wavefronts share phase 1 as 2 x 2 rectangles");
+    static_assert(STEM || (KC == 4 && S == 2), "the expansion form: sixteen input channels, depthwise stride 2");
+    static_assert(MT % 2 == 0 && CM * 9 / 4 <= kThreads && CM <= kThreads, "phase 0 and 2 take the channels in these steps");
+};
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ f32x2 buf_load2(rsrc_t r, unsigned byte_off) {
+    return __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(r, (int)byte_off, 0, 0));
+}
+
+// One segment of phase 0: COUNT floats of LDS at dst, float i from byte offset src(i) of the
+// buffer (kOutside: 0).  Loads first, stores second.
+template <int COUNT, class F>
+__device__ __forceinline__ void blk_stage_load(float (&v)[(COUNT + kThreads - 1) / kThreads], const rsrc_t& rs, F src) {
+#pragma unroll
+    for (int i = 0; i < (COUNT + kThreads - 1) / kThreads; ++i) {
+        const int idx = (int)threadIdx.x + kThreads * i;
+        v[i] = buf_load(rs, idx < COUNT ? src(idx) : kOutside);
+    }
+}
+template <int COUNT>
+__device__ __forceinline__ void blk_stage_store(const float (&v)[(COUNT + kThreads - 1) / kThreads], float* dst) {
+#pragma unroll
+    for (int i = 0; i < (COUNT + kThreads - 1) / kThreads; ++i) {
+        const int idx = (int)threadIdx.x + kThreads * i;
+        if (idx < COUNT) dst[idx] = v[i];
+    }
+}
+
+template <int G, int S, bool STEM, int MT, int KC, class Poll>
+__device__ __forceinline__ bool conv2d_block_body(const ReefOpDesc& d, int task, char* smem_raw, const Poll&) {
+    typedef TileBlk<G, S, STEM, MT, KC> T;
+    constexpr int R = T::R, NG = T::NG, KF = T::KF, KP = T::KP;
+    static_assert(!STEM || S == 1, "the stem form has a stride-1 depthwise stage");
+    float* smem = (float*)smem_raw;
+    const int* a = d.attr;
+    const int lane = threadIdx.x & 63, i16 = lane & 15, kq = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int C = a[REEF_CONV_CIN], H = a[REEF_CONV_H], W = a[REEF_CONV_W], M = a[REEF_CONV_COUT];
+    const int Ho = a[REEF_CONV_HO], Wo = a[REEF_CONV_WO], P = a[REEF_CONV_PROJ];
+    const int Hm = STEM ? Ho : H, Wm = STEM ? Wo : W;            // the front filter's result
+    task = xcd_chunked(task, a[REEF_CONV_N_TILES]);
+    const int segs = (Wo + kRowSeg - 1) / kRowSeg;
+    const int q_seg = div_small(task, segs);
+    const int y0 = q_seg * G, x0 = (task - q_seg * segs) * kRowSeg;     // first output row and column
+
+    // column of the front filter's result that lane / column c of pixel group (r, p) stands for
+    auto image_col = [&](int c, int p) -> int {
+        if (S == 1) return c == 15 ? x0 - 1 : x0 + c;
+        if (p == 0) return c < kRowSeg ? 2 * (x0 + c) : -1;
+        return c == 15 ? 2 * x0 - 1 : c < kRowSeg ? 2 * (x0 + c) + 1 : -1;
+    };
+    // activation without a branch per element: clamp to [0, hi], or the value itself
+    auto activate = [](float v, int act) -> float {
+        const float hi = act == REEF_ACT_RELU6 ? 6.0f : __builtin_inff();
+        const float c = fminf(fmaxf(v, 0.0f), hi);
+        return act == REEF_ACT_NONE ? v : c;
+    };
+
+    // The projection's weights go from memory straight into the registers of the wavefront that
+    // multiplies with them (row i16 of output tile pt, channels kq KP .. + KP - 1: 128-bit loads; the
+    // channel count is a multiple of 4), on their way from the first instruction on: phase 3 is the
+    // last to need anything.
+    const int npairs3 = ((P + 15) >> 4) * G;
+    const rsrc_t rs_wp = make_rsrc(d.ptr[6], (unsigned)P * (unsigned)M * 4u);
+    f32x4 wp[KP / 4];
+    auto load_wp = [&](int pr) {
+        const unsigned prow = (unsigned)((pr / G) * 16 + i16);
+#pragma unroll
+        for (int q = 0; q < KP / 4; ++q) {
+            const int ch0 = kq * KP + 4 * q;
+            wp[q] = buf_load4(rs_wp, (prow < (unsigned)P && ch0 < M) ? (prow * (unsigned)M + (unsigned)ch0) * 4u : kOutside);
+        }
+    };
+    if (wave < npairs3) load_wp(wave);
+
+    // ---- phase 0.  Channels, rows and columns that do not exist are staged as zeros, so the phases
+    // below run over the compiled sizes whatever the layer's.
+    {
+        const rsrc_t rs_in = make_rsrc(d.ptr[0], (unsigned)C * (unsigned)(H * W) * 4u);
+        const rsrc_t rs_wf = make_rsrc(d.ptr[1], (unsigned)M * (unsigned)C * (STEM ? 36u : 4u));
+        const rsrc_t rs_bf = make_rsrc(d.ptr[3], (unsigned)M * 4u);
+        const rsrc_t rs_wd = make_rsrc(d.ptr[4], (unsigned)M * 36u);
+        const rsrc_t rs_bd = make_rsrc(d.ptr[5], (unsigned)M * 4u);
+        const rsrc_t rs_bp = make_rsrc(d.ptr[7], (unsigned)P * 4u);
+        const int t = (int)threadIdx.x;
+        // depthwise weights: a copy, four floats a thread; the three bias vectors
+        const f32x4 v_wd = buf_load4(rs_wd, t < T::CM * 9 / 4 ? (unsigned)t * 16u : kOutside);
+        const float v_bf = buf_load(rs_bf, t < T::CM ? (unsigned)t * 4u : kOutside);
+        const float v_bd = buf_load(rs_bd, t < T::CM ? (unsigned)t * 4u : kOutside);
+        const float v_bp = buf_load(rs_bp, t < T::CP ? (unsigned)t * 4u : kOutside);
+        if constexpr (STEM) {
+            constexpr int N_WF = T::CM * T::WFS;
+            float v_in[(T::PATCH + kThreads - 1) / kThreads], v_wf[(N_WF + kThreads - 1) / kThreads];
+            const int iy0 = 2 * y0 - 3, ix0 = 2 * x0 - 3;            // the patch's first input row and column
+            const int K = 9 * C;
+            blk_stage_load<T::PATCH>(v_in, rs_in, [&](int idx) -> unsigned {
+                const int c = idx / (T::PR * T::PCS), rem = idx - c * (T::PR * T::PCS);
+                const int row = rem / T::PCS, colp = rem - row * T::PCS;
+                const int iy = iy0 + row, ix = ix0 + colp;
+                const bool ok = c < C && colp < 33 && (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
+                return ok ? (unsigned)(c * H * W + iy * W + ix) * 4u : kOutside;
+            });
+            blk_stage_load<N_WF>(v_wf, rs_wf, [&](int idx) -> unsigned {
+                // [middle channel][lane / 16][8]: tap (lane / 16) * 7 + s of the 9 Cin, s < 7
+                const int m = idx / T::WFS, q = idx - m * T::WFS;
+                const int k = (q >> 3) * KF + (q & 7);
+                const bool ok = m < M && q < 32 && (q & 7) < KF && k < K;
+                return ok ? (unsigned)(m * K + k) * 4u : kOutside;
+            });
+            blk_stage_store<T::PATCH>(v_in, smem);
+            blk_stage_store<N_WF>(v_wf, smem + T::O_WF);
+        } else {
+            // the patch: thread = (input channel, column); a 64-bit load brings an even column and
+            // the odd one right of it (W is even).  Lane 15 fetches the pair left of the segment
+            // for its odd column; lane 14 has nothing to fetch.
+            const int c = t >> 4, l = t & 15;
+            f32x2 v_in[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int iy = y0 * S - 1 + r, ix = l == 15 ? 2 * x0 - 2 : 2 * (x0 + l);
+                const bool ok = c < C && l != 14 && (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
+                v_in[r] = buf_load2(rs_in, ok ? (unsigned)(c * H * W + iy * W + ix) * 4u : kOutside);
+            }
+            // the front weights: thread = (middle channel of 64, four input channels), 128-bit loads
+            constexpr int NWF = (T::CM + 63) / 64;
+            f32x4 v_wf[NWF];
+#pragma unroll
+            for (int i = 0; i < NWF; ++i) {
+                const int m = (t >> 2) + 64 * i, k0 = 4 * (t & 3);
+                v_wf[i] = buf_load4(rs_wf, (m < M && k0 < C) ? (unsigned)(m * C + k0) * 4u : kOutside);
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                smem[((2 * r) * 16 + l) * T::PS + c] = l < kRowSeg ? v_in[r][0] : 0.0f;
+                smem[((2 * r + 1) * 16 + l) * T::PS + c] = v_in[r][1];
+            }
+#pragma unroll
+            for (int i = 0; i < NWF; ++i) {
+                const int m = (t >> 2) + 64 * i;
+                if (m < T::CM) *(f32x4*)(smem + T::O_WF + m * T::WFS + 4 * (t & 3)) = v_wf[i];
+            }
+        }
+        if (t < T::CM * 9 / 4) *(f32x4*)(smem + T::O_WD + 4 * t) = v_wd;
+        if (t < T::CM) { smem[T::O_BF + t] = v_bf; smem[T::O_BD + t] = v_bd; }
+        if (t < T::CP) smem[T::O_BP + t] = v_bp;
+    }
+    __syncthreads();
+
+    // ---- phase 1: E = act(front filter + bias), 0 outside the image
+    const int act = a[REEF_CONV_ACT], act2 = a[REEF_CONV_ACT2];
+    float* E = smem + T::O_E;
+    int poff[STEM ? KF : 1];       // STEM: where tap kq * 7 + s sits in the patch, relative to tap 0
+    if constexpr (STEM) {
+#pragma unroll
+        for (int s = 0; s < KF; ++s) {
+            const int k = min(kq * KF + s, 26);      // (the 28th tap does not exist: its weight is 0)
+            const int c = k / 9, ky = (k - 9 * c) / 3, kx = k - 9 * c - 3 * ky;
+            poff[s] = (c * T::PR + ky) * T::PCS + kx;
+        }
+    }
+    {
+        // a wavefront takes MH channel tiles x GH pixel groups: every operand read once, then per
+        // channel tile the MFMAs of its GH groups (2 GH independent sums) and their results
+        const int mtb = (wave & 1) * T::MH, gb = (wave >> 1) * T::GH;
+        float ra[T::MH][STEM ? 8 : KF], rb[T::GH][KF];
+        f32x4 bias[T::MH];
+#pragma unroll
+        for (int m = 0; m < T::MH; ++m) {
+            const float* wa = smem + T::O_WF + ((mtb + m) * 16 + i16) * T::WFS + kq * (STEM ? 8 : KF);
+            const f32x4 w0 = *(const f32x4*)wa;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) ra[m][e] = w0[e];
+            if constexpr (STEM) {
+                const f32x4 w1 = *(const f32x4*)(wa + 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) ra[m][4 + e] = w1[e];
+            }
+            bias[m] = *(const f32x4*)(smem + T::O_BF + (mtb + m) * 16 + 4 * kq);
+        }
+#pragma unroll
+        for (int b = 0; b < T::GH; ++b) {
+            const int g = gb + b;
+            if constexpr (STEM) {
+                // the lane's column of the result is patch column 2 ((i16 + 1) mod 16) of filter column 0
+                const float* pb = smem + 2 * g * T::PCS + 2 * ((i16 + 1) & 15);
+#pragma unroll
+                for (int s = 0; s < KF; ++s) rb[b][s] = pb[poff[s]];
+            } else {
+                const f32x4 b0 = *(const f32x4*)(smem + (g * 16 + i16) * T::PS + 4 * kq);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) rb[b][e] = b0[e];
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int m = 0; m < T::MH; ++m) {
+            f32x4 acc[T::GH][2];
+#pragma unroll
+            for (int b = 0; b < T::GH; ++b) acc[b][0] = acc[b][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int s = 0; s < KF; ++s)
+#pragma unroll
+                for (int b = 0; b < T::GH; ++b)
+                    acc[b][s & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[m][s], rb[b][s], acc[b][s & 1], 0, 0, 0);
+#pragma unroll
+            for (int b = 0; b < T::GH; ++b) {
+                const int g = gb + b, r = g / S, p = g - r * S;
+                const int my = y0 * S - 1 + r, mx = image_col(i16, p);
+                const bool inside = (unsigned)my < (unsigned)Hm && (unsigned)mx < (unsigned)Wm;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float v = activate((acc[b][0][j] + acc[b][1][j]) + bias[m][j], act);
+                    E[((mtb + m) * 16 + 4 * kq + j) * T::ESTRIDE + g * 16 + i16] = inside ? v : 0.0f;
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- phase 2: D = act2(depthwise(E) + bias), two channel tiles at a time: every value a thread
+    // needs read once, then its outputs formed, then stored
+    float* D = smem + T::O_D;
+    {
+        const int row = threadIdx.x >> 4, col = threadIdx.x & 15;
+#pragma unroll
+        for (int mt0 = 0; mt0 < MT; mt0 += 2) {
+            float wdw[2][9], bdw[2], e[2][R][3];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int ch = (mt0 + h) * 16 + row;
+#pragma unroll
+                for (int tp = 0; tp < 9; ++tp) wdw[h][tp] = smem[T::O_WD + ch * 9 + tp];
+                bdw[h] = smem[T::O_BD + ch];
+                const float* Ec = E + ch * T::ESTRIDE;
+#pragma unroll
+                for (int rr = 0; rr < R; ++rr) {
+                    // the sixteen threads of a channel are one row of lanes: neighbours come from there
+                    if (S == 1) {
+                        e[h][rr][1] = Ec[rr * 16 + col];
+                    } else {
+                        e[h][rr][1] = Ec[(2 * rr) * 16 + col];         // 2 x
+                        e[h][rr][2] = Ec[(2 * rr + 1) * 16 + col];     // 2 x + 1
+                    }
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int rr = 0; rr < R; ++rr) {
+                    if (S == 1) {
+                        e[h][rr][0] = lane_from_left(e[h][rr][1]);
+                        e[h][rr][2] = lane_from_right(e[h][rr][1]);
+                    } else {
+                        e[h][rr][0] = lane_from_left(e[h][rr][2]);     // the odd column left of 2 x
+                    }
+                }
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int ch = (mt0 + h) * 16 + row;
+#pragma unroll
+                for (int g = 0; g < G; ++g) {
+                    float s = 0.0f;
+#pragma unroll
+                    for (int tp = 0; tp < 9; ++tp) s = fmaf(e[h][S * g + tp / 3][tp % 3], wdw[h][tp], s);
+                    D[(g * 16 + col) * T::DPS + ch] = activate(s + bdw[h], act2);
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- phase 3: out = projection(D) + bias
+    const rsrc_t rs_o = make_rsrc(d.ptr[2], (unsigned)P * (unsigned)(Ho * Wo) * 4u);
+    for (int pr = wave; pr < npairs3; pr += 4) {
+        if (pr != wave) load_wp(pr);
+        const int pt = pr / G, g = pr - pt * G;
+        const float* db = D + (g * 16 + i16) * T::DPS + kq * KP;
+        f32x4 rb[KP / 4];
+#pragma unroll
+        for (int q = 0; q < KP / 4; ++q) rb[q] = *(const f32x4*)(db + 4 * q);
+        const f32x4 bias = *(const f32x4*)(smem + T::O_BP + pt * 16 + 4 * kq);
+        __builtin_amdgcn_sched_barrier(0);
+        f32x4 acc[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[q] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int q = 0; q < KP / 4; ++q)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(wp[q][e], rb[q][e], acc[e], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int ch = pt * 16 + 4 * kq + j;
+            const bool ok = i16 < kRowSeg && x0 + i16 < Wo && y0 + g < Ho && ch < P;
+            buf_store(rs_o, ok ? ((unsigned)ch * (unsigned)(Ho * Wo) + (unsigned)((y0 + g) * Wo + x0 + i16)) * 4u : kOutside,
+                      ((acc[0][j] + acc[1][j]) + (acc[2][j] + acc[3][j])) + bias[j]);
+        }
+    }
+    return true;
+}
+
 // ---- reef_conv2d_sp7_g2: the stem of a ResNet / DenseNet in one launch ------------------------
 // in (+ a per-channel shift) -> 7x7 convolution, stride 2, padding 3, + bias, activation ->
 // 3x3 max-pool, stride 2, padding 1 (+ a per-channel shift, activation).  As launches of their own

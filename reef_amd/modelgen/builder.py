@@ -25,6 +25,7 @@ from ..paths import code_object
 
 ACT_NONE, ACT_RELU, ACT_RELU6, ACT_GELU = 0, 1, 2, 3
 F_BIAS, F_RESIDUAL, F_AFFINE, F_DUAL, F_FUSED_REDUCE, F_PRE_ACT, F_PAIR_FOLD, F_DW_OUTPUT = 1, 2, 4, 8, 16, 32, 64, 128
+F_PROJ_OUTPUT = 4096
 F_POOL_OUTPUT, F_IN_SHIFT, F_POOL_SHIFT, F_GAP_OUTPUT = 256, 512, 1024, 2048
 WG = 256
 
@@ -374,6 +375,56 @@ class GraphBuilder:
                    flops, 4 * (x.size + cout * cin + 11 * cout + out.size), 6.0)
         return out
 
+    BLOCK_TILES = {"sdp": ("g2", "g4"), "xdp2": ("g1", "g2")}      # reef_conv2d_<family>_<tile> that exist
+
+    @staticmethod
+    def block_fits(front, cin, cmid, cout, width):
+        """Whether a front filter + depthwise 3x3 + projection go into one launch of the block family:
+        few enough channels for one workgroup to hold all of them (the kernels move the middle
+        channels, and the expansion form its input channels and columns, in fours resp. pairs)."""
+        if cmid % 4 != 0 or cout > 32:
+            return False
+        if front == "stem":
+            return cin <= 3 and cmid <= 32
+        return cin <= 16 and cin % 4 == 0 and cmid <= 96 and width % 2 == 0
+
+    def conv2d_block(self, x, cmid, cout, front="expand", act=ACT_RELU6, dw_act=ACT_RELU6, tile=None):
+        """A whole MobileNetV2 block as ONE launch: the front filter (+ bias, act) -- front="stem": the
+        network's 3x3 / stride 2 / padding 1 first layer, then a stride-1 depthwise stage
+        (reef_conv2d_sdp_<tile>); front="expand": a 1x1 expansion, then a stride-2 depthwise stage
+        (reef_conv2d_xdp2_<tile>) --, the depthwise 3x3 filter (padding 1, + bias, dw_act) and the linear
+        1x1 projection (+ bias) to cout channels.  For the blocks at the head of the network: a workgroup
+        holds every channel of its pixels, and neither the front filter's result nor the depthwise
+        stage's is written.  Parameters are created in the order the three layers would create them."""
+        cin, H, W = x.shape
+        stem = front == "stem"
+        assert self.block_fits(front, cin, cmid, cout, W)
+        kf = 3 if stem else 1
+        std = lambda fan: self.weight_std if self.weight_std is not None else math.sqrt(2.0 / fan)
+        w = self.param((cmid, cin, kf, kf), std(cin * kf * kf))
+        b = self.param((cmid,), 0.01)
+        wd = self.param((cmid, 1, 3, 3), std(9))
+        bd = self.param((cmid,), 0.01)
+        wp = self.param((cout, cmid, 1, 1), std(cmid))
+        bp = self.param((cout,), 0.01)
+        Ho, Wo = (H - 1) // 2 + 1, (W - 1) // 2 + 1
+        out = self.temp((cout, Ho, Wo))
+        family = "sdp" if stem else "xdp2"
+        if tile is None:
+            tile = "g4" if stem else "g1"
+        assert tile in self.BLOCK_TILES[family]
+        G = tiling.ROW_TILES[tile]
+        nt = math.ceil(Ho / G) * math.ceil(Wo / tiling.ROW_SEG)
+        mid_px = Ho * Wo if stem else H * W
+        flops = 2 * (cmid * cin * kf * kf * mid_px + cmid * 9 * Ho * Wo + cout * cmid * Ho * Wo)
+        self.flops += flops
+        attrs = [cin, H, W, cmid, Ho, Wo, kf, kf, 2, 2, kf // 2, kf // 2, F_BIAS | F_DW_OUTPUT | F_PROJ_OUTPUT, act,
+                 tiling.TILES[tile][0], 1, math.ceil(cin * kf * kf / 4) * 4, 1, nt, dw_act, cout, 8, 0, 0]
+        self._emit("reef_conv2d_%s_%s" % (family, tile), nt,
+                   [x, w.idx, out.idx, b.idx, wd.idx, bd.idx, wp.idx, bp.idx], attrs, "conv2d",
+                   flops, 4 * (x.size + w.size + 11 * cmid + wp.size + cout + out.size), 7.0)
+        return out
+
     def dwconv2d(self, x, k, stride=1, pad=0, bias=True, act=ACT_RELU6, out=None, given=None):
         """given: {"w", "bias"} -> existing storages instead of new parameters; out: existing
         storage for the result (an imported graph brings its own)."""
@@ -672,6 +723,16 @@ class GraphBuilder:
             sym = n.split("#")[0]
             if sym == "reef_conv2d_sp7_g2":
                 shared[n] = (3 * 15 * 64 + 16 * (5 * 32 + 1) + 32) * 4 + 16     # TileSp7: input patch + pooled-from block
+            elif sym.startswith("reef_conv2d_sdp_") or sym.startswith("reef_conv2d_xdp2_"):
+                # TileBlk: patch, the three layers' parameters, the front filter's result, the depthwise stage's
+                stem, G = sym.startswith("reef_conv2d_sdp_"), tiling.ROW_TILES[sym.split("_")[-1]]
+                R, S, CM, KC = (G + 2, 1, 32, 1) if stem else (2 * G + 1, 2, 96, 4)
+                NG = R * S
+                patch = 3 * (2 * R + 1) * 36 if stem else NG * 16 * (4 * KC + 4)
+                wfs = 36 if stem else 4 * KC + 4
+                floats = (patch + CM * wfs + CM + CM * 9 + CM + 32 + CM * (NG * 16 + (20 if NG % 2 == 0 else 4))
+                          + G * 16 * (CM + 4))
+                shared[n] = floats * 4 + 16
             elif sym.startswith("reef_conv2d_xdw"):
                 G, S = self.XDW_TILES[sym.split("_")[-1]], 2 if sym.startswith("reef_conv2d_xdw2_") else 1
                 NG = (G + 2) if S == 1 else (2 * G + 1) * 2      # TileXdw: pixel groups of the 1x1 result

@@ -128,24 +128,39 @@ def mocked_kernel(name="mocked_kernel"):
 
 
 def mobilenet_v2(image=(3, 224, 224), classes=1000, name="mobilenetv2", seed=rng.BASE_SEED, fuse_expand_dw=True,
-                 fuse_gap=True):
+                 fuse_gap=True, fuse_head=True):
     """MobileNetV2, width 1.0: 3x3/2 stem, 17 inverted-residual blocks (1x1 expand + ReLU6,
     depthwise 3x3 + ReLU6, linear 1x1 projection, residual add when stride 1 and equal
     channels), 1x1 to 1280, global average pool, classifier.  Batch norms are folded
     into the convolutions as biases; the residual add is the projection's epilogue.
     fuse_expand_dw: the 1x1 expansion of a block and the depthwise convolution behind it are one
     launch and the expanded tensor is never written
-    (GraphBuilder.conv2d_dw); False keeps the two launches."""
+    (GraphBuilder.conv2d_dw); False keeps the two launches.
+    fuse_head: the layers on the 112 x 112 image are two launches instead of six: stem + first
+    block (no expansion: depthwise filter and projection to 16 channels), and the second block
+    (16 -> 96 -> 24 channels, stride 2) -- GraphBuilder.conv2d_block, every channel of a pixel tile
+    in one workgroup; same parameters in the same order."""
     g = GraphBuilder(name, seed)
     x = g.input("data", image)
-    x = g.conv2d(x, 32, 3, 2, 1, bias=True, act=ACT_RELU6)
     cfg = [(1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1), (6, 160, 3, 2),
            (6, 320, 1, 1)]
     cin = 32
-    for t, c, n, s in cfg:
+    stem_done = False
+    if fuse_head and image[0] <= 3 and cfg[0][0] == 1 and cfg[0][3] == 1 and GraphBuilder.block_fits("stem", image[0], 32, cfg[0][1], image[2]):
+        x = g.conv2d_block(x, 32, cfg[0][1], front="stem")
+        cin, stem_done = cfg[0][1], True
+    else:
+        x = g.conv2d(x, 32, 3, 2, 1, bias=True, act=ACT_RELU6)
+    for bi, (t, c, n, s) in enumerate(cfg):
         for i in range(n):
+            if bi == 0 and stem_done:
+                continue
             stride = s if i == 0 else 1
             y = x
+            if fuse_head and t != 1 and stride == 2 and GraphBuilder.block_fits("expand", cin, cin * t, c, x.shape[2]):
+                x = g.conv2d_block(x, cin * t, c, front="expand")
+                cin = c
+                continue
             # (not the stride-2 block at 112 x 112: its 1x1 result is 96 x 112 x 112, and forming it
             # tile by tile with the rows and columns neighbours share costs more than the launch and
             # the round trip saved: 14.9 against 13.1 us)

@@ -512,6 +512,43 @@ def test_a_pointwise_plus_depthwise_kernel_is_checked_against_its_storages(tmp_p
     broken(lambda m: m["kernels"][0]["launch_params"].__setitem__(0, 5), "workgroups")
 
 
+def test_a_whole_block_kernel_is_checked_against_its_storages(tmp_path):
+    """reef_conv2d_sdp_<tile> / reef_conv2d_xdp2_<tile>: eight operands, the output sized by the
+    projection's channels (carried in the counter slot, which such a launch does not use), the
+    limits of the two forms; a graph file that disagrees is refused with the reason."""
+    from reef_amd import binding as B
+    g = MB.GraphBuilder("blkfmt")
+    x = g.input("data", (3, 30, 44))
+    y = g.conv2d_block(x, 32, 16, front="stem")
+    g.mark_output(g.conv2d_block(y, 96, 24, front="expand"))
+    base = g.write(str(tmp_path / "ok"), link_code_objects=False)
+    assert B.check_model(base + ".json") == (True, "")
+    model = json.load(open(base + ".json"))
+    k0, k1 = model["kernels"]
+    assert k0["name"].startswith("reef_conv2d_sdp_g4") and k1["name"].startswith("reef_conv2d_xdp2_g1")
+    assert len(k0["args"]) == 8 and k0["attrs"][20] == 16 and k1["attrs"][20] == 24
+    assert model["storage"][k1["args"][2]]["size"] == 24 * 8 * 11
+    assert not MB.GraphBuilder.block_fits("expand", 16, 96, 24, 45)         # odd width
+    assert not MB.GraphBuilder.block_fits("expand", 24, 144, 32, 56)        # too many channels for one workgroup
+    assert not MB.GraphBuilder.block_fits("stem", 3, 30, 16, 224)           # middle channels not in fours
+
+    def broken(change, reason):
+        m = json.loads(json.dumps(model))
+        change(m)
+        p = str(tmp_path / "broken.json")
+        json.dump(m, open(p, "w"))
+        ok, why = B.check_model(p)
+        assert not ok and reason in why, why
+
+    broken(lambda m: m["kernels"][0]["args"].pop(), "operands")                         # no projection bias
+    broken(lambda m: m["kernels"][0]["attrs"].__setitem__(20, 40), "loader family")     # more than 32 output channels
+    broken(lambda m: m["kernels"][0]["attrs"].__setitem__(12, 1 | 128), "loader family")  # projection flag missing
+    broken(lambda m: m["kernels"][1]["attrs"].__setitem__(17, 6), "loader family")      # a workgroup holds every channel
+    broken(lambda m: m["storage"][m["kernels"][1]["args"][6]].__setitem__("size", 24 * 90), "projection weights")
+    broken(lambda m: m["storage"][m["kernels"][0]["args"][2]].__setitem__("size", 15 * 15 * 22), "output")
+    broken(lambda m: m["kernels"][1]["launch_params"].__setitem__(0, 5), "workgroups")
+
+
 def test_a_product_behind_a_layernorm_is_checked_against_its_storages(tmp_path):
     """reef_gemm_ntl_<tile> and the residual of a matrix product: operand list and sizes follow from
     the flags; the LayerNorm flag belongs to the kernels named ntl and to no other."""

@@ -509,6 +509,47 @@ def test_pointwise_then_depthwise_in_one_launch(tmp_path, tile, case):
     print("xdw %s %s: worst rel err %.2e" % (tile, case, worst[0]))
 
 
+BLOCK_CASES = [
+    # front, cin, H, W, middle channels, output channels
+    ("stem", 3, 224, 224, 32, 16),      # MobileNetV2: stem + first block
+    ("stem", 3, 61, 45, 32, 16),        # ragged: odd sizes, the last segment three columns wide
+    ("stem", 1, 9, 9, 20, 7),           # one channel in, channel counts that fill no tile
+    ("stem", 3, 2, 2, 32, 32),          # one output pixel: every neighbour is padding
+    ("expand", 16, 112, 112, 96, 24),   # MobileNetV2: second block
+    ("expand", 16, 33, 58, 96, 24),     # ragged
+    ("expand", 4, 7, 30, 40, 9),        # channel counts that fill no tile
+    ("expand", 8, 1, 2, 16, 32),        # one output pixel
+]
+
+
+@pytest.mark.parametrize("case", BLOCK_CASES)
+def test_front_filter_depthwise_and_projection_in_one_launch(tmp_path, case):
+    """reef_conv2d_sdp_<tile> / reef_conv2d_xdp2_<tile> against the oracle's three layers, each compiled
+    tile, in all three flavours (same bits in all of them)."""
+    from reef_amd import binding as B
+    from tests.helpers import write_model
+    front, cin, H, W, cmid, cout = case
+    g = MB.GraphBuilder("blk")
+    x = g.input("data", (cin, H, W))
+    family = "sdp" if front == "stem" else "xdp2"
+    outs = [g.conv2d_block(x, cmid, cout, front=front, tile=t) for t in MB.GraphBuilder.BLOCK_TILES[family]]
+    other = g.conv2d_block(x, cmid, cout, front=front, act=MB.ACT_NONE, dw_act=MB.ACT_RELU)
+    g.mark_output(other)
+    assert [k["name"].split("_")[2] for k in g.kernels] == [family] * 3
+    data = rnd(cin, H, W)
+    exe, orc, model = run_both(g, tmp_path, {"data": data})
+    worst = compare_storages(exe, orc, model, what="block %s" % (case,))
+    want = exe.get_output()
+    d = write_model(g, tmp_path)
+    for kind, pre in ((B.TRANS, False), (B.HYBRID, True), (B.HYBRID, False)):
+        e = B.Executor.from_dir(d, g.name, kind)
+        e.set_input_checked("data", data)
+        e.execute_preemptable() if pre else e.execute()
+        np.testing.assert_array_equal(e.get_output(), want, err_msg="flavour %s %s" % (kind, pre))
+        e.close()
+    print("block %s: worst rel err %.2e" % (case, worst[0]))
+
+
 def test_mobilenetv2_with_and_without_the_fused_front_half(tmp_path):
     """The network with expansion + depthwise in one launch holds, in every tensor both variants
     have (block outputs, logits), what the variant with two launches holds, to 1e-4: the fused
@@ -517,12 +558,13 @@ def test_mobilenetv2_with_and_without_the_fused_front_half(tmp_path):
     x = nets.image_input("mobilenetv2", (3, 224, 224))
     outs = []
     for fuse in (False, True):
-        g = nets.mobilenet_v2(fuse_expand_dw=fuse, fuse_gap=fuse)
+        g = nets.mobilenet_v2(fuse_expand_dw=fuse, fuse_gap=fuse, fuse_head=fuse)
         exe, orc, model = run_both(g, tmp_path / str(fuse), {"data": x})
         compare_storages(exe, orc, model, what="mobilenetv2 fuse=%s" % fuse)
         li = model["kernels"][-1]["args"][0]
         outs.append((len(g.kernels), exe.get_data(li, model["storage"][li]["size"])))
-    assert outs[0][0] == 55 and outs[1][0] == 39      # fused: expansion + depthwise, and the last convolution averages
+    # fused: expansion + depthwise, the last convolution averages, the layers at 112 x 112 are two launches
+    assert outs[0][0] == 55 and outs[1][0] == 35
     from tests.helpers import max_rel_err, REL_TOL
     assert max_rel_err(outs[1][1], outs[0][1]) <= REL_TOL
 
