@@ -1287,6 +1287,11 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
 }
 
 // ---- reef_conv2d_xdw[2]_g<G>: 1x1 convolution, then depthwise 3x3, in one launch --------------
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ f32x2 buf_load2(rsrc_t r, unsigned byte_off) {
+    return __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(r, (int)byte_off, 0, 0));
+}
+
 // The front half of a MobileNetV2 block: expand (1x1 filter, + bias, activation) and the depthwise
 // 3x3 filter (padding 1, stride S = 1 or 2, + bias, activation) that follows it.  As two launches
 // the expanded tensor -- six times the block's input, the largest tensor of the network -- is
@@ -1296,18 +1301,23 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
 // itself.  The input has few channels (K = 16..160 for 96..960 expanded channels), so what
 // neighbouring tiles compute twice is a fraction of a small product, and no workgroup waits for
 // another.
-//   phase 1  the 1x1 result on the matrix cores, direct form; the four wavefronts split the input
-//            channels, partial tiles meet in LDS; + bias, activation; positions outside the image
-//            become 0 (the depthwise stage's padding) -> E in LDS.
-//            S = 1: pixel group r is image row y0 - 1 + r (G + 2 of them); lanes 0..13 of a k slot
+//   phase 0  CK input channels at a time: the input patch into LDS as [pixel][channel] (every
+//            value loaded once, by one thread), the tile's weight rows as [row][channel] (128-bit
+//            loads), all loads of a thread on their way before its first store.
+//            S = 1: pixel group r is image row y0 - 1 + r (G + 2 of them); lanes 0..13 of a group
 //            are the segment's columns, lane 14 the column right of it, lane 15 the column left.
 //            S = 2: input rows 2 y0 - 1 + r (2 G + 1 of them), each as two groups: the even
 //            columns 2 x (lanes 0..13 = the segment's x) and the odd columns 2 x + 1 (lane 15:
 //            column 2 x0 - 1, left of the segment).
-//   phase 2  thread t = (channel t / 16, column t % 16) forms its G outputs from E: taps in filter
-//            order, then the bias, then the activation, as the depthwise kernel does.  The left
-//            neighbour of column c is lane (c - 1) mod 16, the right one lane c + 1 (S = 1) or the
-//            odd group's lane c (S = 2).
+//   phase 1  the 1x1 result on the matrix cores, both operands 128-bit LDS reads: k slot
+//            (s, lane / 16) of a chunk's MFMAs stands for channel (lane / 16) * (chunk / 4) + s, so
+//            what a lane multiplies is contiguous.  The wavefronts split the pixel groups, each
+//            sums over all channels: nobody adds partial sums.  + bias, activation; positions
+//            outside the image become 0 (the depthwise stage's padding) -> E in LDS.
+//   phase 2  thread t = (channel t / 16, column t % 16) forms its G outputs from E: a value per
+//            row (two for S = 2) from LDS, the neighbouring columns from the neighbouring lanes
+//            (the sixteen threads of a channel are one row of lanes); taps in filter order, then
+//            the bias, then the activation, as the depthwise kernel does.
 // ptr: in [Cin][H][W], W [Cout][Cin], out [Cout][Ho][Wo], bias [Cout], depthwise weights [Cout][9],
 // depthwise bias [Cout].  attr: H, W the input (and the 1x1 result), HO, WO the output, SH = SW =
 // S (the 1x1 filter itself has stride 1), ACT the 1x1 layer's activation, ACT2 the depthwise
@@ -1317,18 +1327,25 @@ template <int G, int S = 1>
 struct TileXdw {
     static constexpr int R = S == 1 ? G + 2 : 2 * G + 1;    // rows of the 1x1 result a tile needs
     static constexpr int NG = R * S;                         // pixel groups of 16 lanes: S per row
-    static constexpr int PART = 320;                         // floats per 16 x 16 partial tile (skewed rows)
-    static constexpr int ESTRIDE = (NG + 1) * 16;            // floats per channel of E (+ one group: no bank conflicts)
-    static constexpr int LDS_BYTES = (4 * NG * PART + 16 * ESTRIDE) * 4 + 16;
+    static constexpr int GW = (NG + 3) / 4;                  // pixel groups per wavefront at most
+    // input channels staged at a time: what the network's layers of the tile's kind have
+    static constexpr int CK = S == 2 ? 96 : G == 4 ? 64 : 160;
+    static constexpr int PS = CK + 4;                        // floats per pixel of the patch and per weight row (4 mod 32: banks)
+    // floats per channel of E [channel][pixel]: 20 mod 32, so that the 4 x 16 values a wavefront writes
+    // (channels 4 apart) and the 4 x 16 it reads (consecutive channels) each meet every bank twice
+    static constexpr int ESTRIDE = NG * 16 + (NG % 2 == 0 ? 20 : 4);
+    static constexpr int O_W = NG * 16 * PS, O_E = O_W + 16 * PS;
+    static constexpr int LDS_BYTES = (O_E + 16 * ESTRIDE) * 4 + 16;
+    static_assert(CK % 16 == 0 && PS % 32 == 4, "chunks are whole 16-channel steps");
 };
 
 template <int G, int S, class Poll>
 __device__ __forceinline__ bool conv2d_xdw_body(const ReefOpDesc& d, int task, char* smem_raw, const Poll&) {
     typedef TileXdw<G, S> T;
-    constexpr int R = T::R, NG = T::NG;
-    constexpr int NSTAGE = S == 1 ? 2 : 1;      // K steps whose loads are in flight
+    constexpr int R = T::R, NG = T::NG, GW = T::GW, JM = T::CK / 16;
     float* smem = (float*)smem_raw;
-    float* E = smem + 4 * NG * T::PART;
+    float* Wl = smem + T::O_W;
+    float* E = smem + T::O_E;
     const int* a = d.attr;
     const int lane = threadIdx.x & 63, i16 = lane & 15, kq = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1343,13 +1360,13 @@ __device__ __forceinline__ bool conv2d_xdw_body(const ReefOpDesc& d, int task, c
     const int q_seg = div_small(nt, segs);
     const int y0 = q_seg * G, x0 = (nt - q_seg * segs) * kRowSeg;     // first output row and column
     const int m0 = mt * 16;
-    const unsigned HW4 = (unsigned)(H * W) * 4u;
+    const int HW = H * W;
 
-    // phase-2 role of this thread: channel and column; its depthwise weights, biases
+    // roles: phase 0 thread = (channel or weight row t / 16, column t % 16); phase 2 the same
     const int row = threadIdx.x >> 4, col = threadIdx.x & 15;
     const unsigned ch = (unsigned)(m0 + row);
     const rsrc_t rs_a = make_rsrc(d.ptr[1], (unsigned)M * (unsigned)C * 4u);
-    const rsrc_t rs_b = make_rsrc(d.ptr[0], (unsigned)C * HW4);
+    const rsrc_t rs_b = make_rsrc(d.ptr[0], (unsigned)C * (unsigned)HW * 4u);
     const rsrc_t rs_bias = make_rsrc(d.ptr[3], (unsigned)M * 4u);
     const rsrc_t rs_dw = make_rsrc(d.ptr[4], (unsigned)M * 36u);
     const rsrc_t rs_db = make_rsrc(d.ptr[5], (unsigned)M * 4u);
@@ -1362,112 +1379,161 @@ __device__ __forceinline__ bool conv2d_xdw_body(const ReefOpDesc& d, int task, c
         if (p == 0) return c < kRowSeg ? 2 * (x0 + c) : -1;
         return c == 15 ? 2 * x0 - 1 : c < kRowSeg ? 2 * (x0 + c) + 1 : -1;
     };
-
-    // phase-1 operands: weights W[m0 + i16][8 channels of the k slot], input values of the lane's
-    // column in every pixel group
-    const int lane_c = (wave * 4 + kq) * 8;
-    const int nsteps = (C + 127) / 128;
-    const int lane_steps = lane_c < C ? (C - lane_c + 127) / 128 : 0;
-    const unsigned va = ((unsigned)(m0 + i16) * (unsigned)C + (unsigned)lane_c) * 4u;
-    unsigned vb[NG];
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int p = 0; p < S; ++p) {
-            const int iy = y0 * S - 1 + r, ix = image_col(i16, p);
-            const bool ok = (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
-            vb[r * S + p] = ok ? (unsigned)(iy * W + ix) * 4u + (unsigned)lane_c * HW4 : kOutside;
-        }
-    float ra[NSTAGE][8], rb[NSTAGE][NG][8];
-    auto load_step = [&](int s, int step) {
-        const unsigned outm = step < lane_steps ? 0u : kOutside;
-        const unsigned sa = (unsigned)step * 512u;
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            const f32x4 v = __builtin_bit_cast(
-                f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, (int)((va | outm) + 16u * e), (int)sa, 0));
-            ra[s][4 * e] = v[0]; ra[s][4 * e + 1] = v[1]; ra[s][4 * e + 2] = v[2]; ra[s][4 * e + 3] = v[3];
-        }
-#pragma unroll
-        for (int g = 0; g < NG; ++g)
-#pragma unroll
-            for (int q = 0; q < 8; ++q)
-                rb[s][g][q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                    rs_b, (int)(vb[g] | outm), (int)((unsigned)(step * 128 + q) * HW4), 0));
+    // activation without a branch per element: clamp to [0, hi], or the value itself
+    auto activate = [](float v, int act) -> float {
+        const float hi = act == REEF_ACT_RELU6 ? 6.0f : __builtin_inff();
+        const float c = fminf(fmaxf(v, 0.0f), hi);
+        return act == REEF_ACT_NONE ? v : c;
     };
-    load_step(0, 0);
-    if (NSTAGE > 1 && nsteps > 1) load_step(NSTAGE - 1, 1);
+
+    // what the later phases need from memory, on its way from the start
     float wdw[9];
 #pragma unroll
     for (int t = 0; t < 9; ++t) wdw[t] = buf_load(rs_dw, ch * 36u + 4u * t);
-    const float bdw = buf_load(rs_db, ch * 4u), bex = buf_load(rs_bias, ch * 4u);
+    const float bdw = buf_load(rs_db, ch * 4u);
+    float bexs[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) bexs[j] = buf_load(rs_bias, (unsigned)(m0 + 4 * kq + j) * 4u);
 
-    f32x4 acc[NG][2];
+    // the wavefront's pixel groups (one that does not exist: the last one again, result dropped)
+    int gcl[GW];
 #pragma unroll
-    for (int g = 0; g < NG; ++g) acc[g][0] = acc[g][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    auto mma_stage = [&](int s) {
+    for (int u = 0; u < GW; ++u) gcl[u] = min(wave + 4 * u, NG - 1);
+    f32x4 acc[GW][4];
 #pragma unroll
-        for (int q = 0; q < 8; ++q)
+    for (int u = 0; u < GW; ++u)
 #pragma unroll
-            for (int g = 0; g < NG; ++g)
-                acc[g][q & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[s][q], rb[s][g][q], acc[g][q & 1], 0, 0, 0);
-    };
-    if (NSTAGE == 1) {
-        for (int it = 0; it < nsteps; ++it) {
-            mma_stage(0);
-            if (it + 1 < nsteps) load_step(0, it + 1);
+        for (int e = 0; e < 4; ++e) acc[u][e] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    for (int c0 = 0; c0 < C; c0 += T::CK) {
+        const int nq = (min(C - c0, T::CK) + 15) >> 4;          // 16-channel steps of this chunk
+        if (c0 > 0) __syncthreads();                            // the previous chunk has been multiplied
+        // ---- phase 0
+        {
+            float v[JM][NG];
+            f32x4 vw[(JM + 3) / 4];
+#pragma unroll
+            for (int i = 0; i < (JM + 3) / 4; ++i) {
+                const int c = c0 + 4 * col + 64 * i;
+                const bool ok = 4 * col + 64 * i < 16 * nq && c < C && ch < (unsigned)M;
+                vw[i] = buf_load4(rs_a, ok ? (ch * (unsigned)C + (unsigned)c) * 4u : kOutside);
+            }
+#pragma unroll
+            for (int j = 0; j < JM; ++j) {
+                if (j < nq) {
+                    const int c = c0 + row + 16 * j;
+                    const bool c_ok = c < C;
+                    const unsigned cbase = (unsigned)(c * HW) * 4u;
+                    if (S == 2 && !(W & 1)) {
+                        // an even column and the odd one right of it in one 64-bit load; lane 15 fetches
+                        // the pair left of the segment for its odd column, lane 14 has nothing to fetch
+#pragma unroll
+                        for (int r = 0; r < R; ++r) {
+                            const int iy = y0 * S - 1 + r, ix = col == 15 ? 2 * x0 - 2 : 2 * (x0 + col);
+                            const bool ok = c_ok && col != 14 && (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
+                            const f32x2 p2 = buf_load2(rs_b, ok ? cbase + (unsigned)(iy * W + ix) * 4u : kOutside);
+                            v[j][2 * r] = col < kRowSeg ? p2[0] : 0.0f;
+                            v[j][2 * r + 1] = p2[1];
+                        }
+                    } else {
+#pragma unroll
+                        for (int g = 0; g < NG; ++g) {
+                            const int r = g / S, p = g % S;
+                            const int iy = y0 * S - 1 + r, ix = image_col(col, p);
+                            const bool ok = c_ok && (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
+                            v[j][g] = buf_load(rs_b, ok ? cbase + (unsigned)(iy * W + ix) * 4u : kOutside);
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < (JM + 3) / 4; ++i)
+                if (4 * col + 64 * i < 16 * nq) *(f32x4*)(Wl + row * T::PS + 4 * col + 64 * i) = vw[i];
+#pragma unroll
+            for (int j = 0; j < JM; ++j) {
+                if (j < nq) {
+#pragma unroll
+                    for (int g = 0; g < NG; ++g) smem[(g * 16 + col) * T::PS + row + 16 * j] = v[j][g];
+                }
+            }
         }
-    } else {
-        for (int it = 0; it < nsteps; it += 2) {
-            mma_stage(0);
-            if (it + 2 < nsteps) load_step(0, it + 2);
-            if (it + 1 < nsteps) {
-                mma_stage(NSTAGE - 1);
-                if (it + 3 < nsteps) load_step(NSTAGE - 1, it + 3);
+        __syncthreads();
+
+        // ---- phase 1: the chunk's MFMAs, the operands of step q + 1 read while step q multiplies
+        {
+            const float* wa = Wl + i16 * T::PS + kq * 4 * nq;
+            const float* pb[GW];
+#pragma unroll
+            for (int u = 0; u < GW; ++u) pb[u] = smem + (gcl[u] * 16 + i16) * T::PS + kq * 4 * nq;
+            f32x4 a_cur = *(const f32x4*)wa, b_cur[GW];
+#pragma unroll
+            for (int u = 0; u < GW; ++u) b_cur[u] = *(const f32x4*)pb[u];
+            for (int q = 0; q < nq; ++q) {
+                const int qn = min(q + 1, nq - 1);
+                const f32x4 a_nxt = *(const f32x4*)(wa + 4 * qn);
+                f32x4 b_nxt[GW];
+#pragma unroll
+                for (int u = 0; u < GW; ++u) b_nxt[u] = *(const f32x4*)(pb[u] + 4 * qn);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int u = 0; u < GW; ++u)
+                        acc[u][e] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_cur[e], b_cur[u][e], acc[u][e], 0, 0, 0);
+                a_cur = a_nxt;
+#pragma unroll
+                for (int u = 0; u < GW; ++u) b_cur[u] = b_nxt[u];
             }
         }
     }
 
-    // the four wavefronts' partial tiles meet in LDS (row groups skewed: no bank conflicts)
-    float* part = smem + wave * (NG * T::PART);
-#pragma unroll
-    for (int g = 0; g < NG; ++g)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) part[g * T::PART + (5 * kq + j) * 16 + i16] = acc[g][0][j] + acc[g][1][j];
-    __syncthreads();
-    const float* mine = smem + threadIdx.x + (threadIdx.x >> 6) * 16;
-    constexpr int WSTRIDE = NG * T::PART;
+    // + bias, activation, 0 outside the image -> E
     const int act = a[REEF_CONV_ACT], act2 = a[REEF_CONV_ACT2];
 #pragma unroll
-    for (int r = 0; r < R; ++r)
+    for (int u = 0; u < GW; ++u) {
+        const int g = wave + 4 * u;
+        if (g < NG) {
+            const int r = g / S, p = g - r * S;
+            const int my = y0 * S - 1 + r, mx = image_col(i16, p);
+            const bool inside = (unsigned)my < (unsigned)H && (unsigned)mx < (unsigned)W;
 #pragma unroll
-        for (int p = 0; p < S; ++p) {
-            const float* e = mine + (r * S + p) * T::PART;
-            const float v = ((e[0] + e[WSTRIDE]) + e[2 * WSTRIDE]) + e[3 * WSTRIDE];
-            const bool inside = (unsigned)(y0 * S - 1 + r) < (unsigned)H && (unsigned)image_col(col, p) < (unsigned)W;
-            E[row * T::ESTRIDE + (r * S + p) * 16 + col] = inside ? act_apply(v + bex, act) : 0.0f;
+            for (int j = 0; j < 4; ++j) {
+                const float v = activate(((acc[u][0][j] + acc[u][1][j]) + (acc[u][2][j] + acc[u][3][j])) + bexs[j], act);
+                E[(4 * kq + j) * T::ESTRIDE + g * 16 + i16] = inside ? v : 0.0f;
+            }
         }
+    }
     __syncthreads();
 
-    // depthwise stage from E
+    // ---- phase 2: the depthwise stage from E
     const rsrc_t rs_o = make_rsrc(d.ptr[2], (unsigned)M * (unsigned)(Ho * Wo) * 4u);
     const float* Ec = E + row * T::ESTRIDE;
+    float e[R][3];
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr) {
+        if (S == 1) {
+            e[rr][1] = Ec[rr * 16 + col];
+        } else {
+            e[rr][1] = Ec[(2 * rr) * 16 + col];         // 2 x
+            e[rr][2] = Ec[(2 * rr + 1) * 16 + col];     // 2 x + 1
+        }
+    }
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr) {
+        if (S == 1) {
+            e[rr][0] = lane_from_left(e[rr][1]);
+            e[rr][2] = lane_from_right(e[rr][1]);
+        } else {
+            e[rr][0] = lane_from_left(e[rr][2]);        // the odd column left of 2 x
+        }
+    }
 #pragma unroll
     for (int g = 0; g < G; ++g) {
         float s = 0.0f;
 #pragma unroll
-        for (int t = 0; t < 9; ++t) {
-            const int ky = t / 3, kx = t % 3;
-            float tap;
-            if (S == 1) tap = Ec[(g + ky) * 16 + ((col + kx - 1) & 15)];
-            else tap = kx == 0 ? Ec[((2 * g + ky) * 2 + 1) * 16 + ((col - 1) & 15)]       // odd column left of 2 x
-                     : kx == 1 ? Ec[((2 * g + ky) * 2 + 0) * 16 + col]                    // 2 x
-                               : Ec[((2 * g + ky) * 2 + 1) * 16 + col];                   // 2 x + 1
-            s = fmaf(tap, wdw[t], s);
-        }
+        for (int t = 0; t < 9; ++t) s = fmaf(e[S * g + t / 3][t % 3], wdw[t], s);
         const bool ok = col < kRowSeg && x0 + col < Wo && y0 + g < Ho && ch < (unsigned)M;
         buf_store(rs_o, ok ? (ch * (unsigned)(Ho * Wo) + (unsigned)((y0 + g) * Wo + x0 + col)) * 4u : kOutside,
-                  act_apply(s + bdw, act2));
+                  activate(s + bdw, act2));
     }
     return true;
 }
@@ -1529,11 +1595,6 @@ struct TileBlk {
     static_assert(STEM || (KC == 4 && S == 2), "the expansion form: sixteen input channels, depthwise stride 2");
     static_assert(MT % 2 == 0 && CM * 9 / 4 <= kThreads && CM <= kThreads, "phase 0 and 2 take the channels in these steps");
 };
-
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ f32x2 buf_load2(rsrc_t r, unsigned byte_off) {
-    return __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(r, (int)byte_off, 0, 0));
-}
 
 // One segment of phase 0: COUNT floats of LDS at dst, float i from byte offset src(i) of the
 // buffer (kOutside: 0).  Loads first, stores second.

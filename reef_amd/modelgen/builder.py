@@ -736,7 +736,8 @@ class GraphBuilder:
             elif sym.startswith("reef_conv2d_xdw"):
                 G, S = self.XDW_TILES[sym.split("_")[-1]], 2 if sym.startswith("reef_conv2d_xdw2_") else 1
                 NG = (G + 2) if S == 1 else (2 * G + 1) * 2      # TileXdw: pixel groups of the 1x1 result
-                shared[n] = (4 * NG * 320 + 16 * (NG + 1) * 16) * 4 + 16
+                PS = (96 if S == 2 else 64 if G == 4 else 160) + 4     # a chunk of input channels per pixel / weight row
+                shared[n] = (NG * 16 * PS + 16 * PS + 16 * (NG * 16 + 20)) * 4 + 16
             elif sym.startswith("reef_conv2d_") or sym.startswith("reef_gemm_"):
                 shared[n] = tiling.lds_bytes(sym.split("_")[-1])
                 if sym.startswith("reef_gemm_ntl_"):
