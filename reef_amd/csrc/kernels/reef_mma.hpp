@@ -1919,7 +1919,8 @@ struct TileSp7 {
     static constexpr int STEPS = CMAX * 7 * 2;                     // 42 MFMAs per group: two per filter row
     static constexpr int ESTRIDE = CR * 32 + 1;                    // floats per channel of E
     static constexpr int PATCH = CMAX * PR * PC, EFLOATS = 16 * ESTRIDE + 32;
-    static constexpr int LDS_BYTES = (PATCH + EFLOATS) * 4 + 16;
+    static constexpr int WFLOATS = 16 * CMAX * 49;                 // the tile's weight rows
+    static constexpr int LDS_BYTES = (PATCH + EFLOATS + WFLOATS) * 4 + 16;
 };
 
 template <class Poll>
@@ -1946,16 +1947,17 @@ __device__ __forceinline__ bool conv2d_stem_pool_body(const ReefOpDesc& d, int t
     const float* in_shift = (flags & REEF_F_IN_SHIFT) ? (const float*)d.ptr[p++] : nullptr;
     const float* pool_shift = (flags & REEF_F_POOL_SHIFT) ? (const float*)d.ptr[p++] : nullptr;
 
-    // the weights of this lane's channel row: step s = filter row s / 2 (of channel s / 14), tap
-    // kx = 4 (s % 2) + kq; kx = 7 does not exist (weight 0).  All on their way at once.
+    // the tile's sixteen weight rows into LDS as they are (contiguous in memory; every value loaded
+    // once by one thread -- as 42 loads per lane in each of the four wavefronts they took longer than
+    // the convolution itself)
     const rsrc_t rs_w = make_rsrc(d.ptr[1], (unsigned)M * (unsigned)K * 4u);
-    float ra[T::STEPS];
-    const unsigned wrow = ((unsigned)(m0 + i16) * (unsigned)K + (unsigned)kq) * 4u;      // a row outside M: outside the buffer
+    float* WL = E + T::EFLOATS;
+    constexpr int WSHARE = (T::WFLOATS + kThreads - 1) / kThreads;
+    float wv[WSHARE];
 #pragma unroll
-    for (int s = 0; s < T::STEPS; ++s) {
-        const int c = s / 14, ky = (s % 14) / 2, kx0 = 4 * (s & 1);
-        const bool real = c < C && kx0 + kq < 7;
-        ra[s] = buf_load(rs_w, real ? wrow + (unsigned)(c * 49 + ky * 7 + kx0) * 4u : kOutside);
+    for (int i = 0; i < WSHARE; ++i) {
+        const int idx = (int)threadIdx.x + kThreads * i;
+        wv[i] = buf_load(rs_w, idx < 16 * K ? ((unsigned)(m0 * K) + (unsigned)idx) * 4u : kOutside);
     }
     const rsrc_t rs_bias = make_rsrc(d.ptr[3], (unsigned)M * 4u);
     float bias[4];
@@ -1990,10 +1992,24 @@ __device__ __forceinline__ bool conv2d_stem_pool_body(const ReefOpDesc& d, int t
             if (idx < T::PATCH) patch[idx] = inside[i] ? v[i] + s : 0.0f;
         }
     }
+#pragma unroll
+    for (int i = 0; i < WSHARE; ++i) {
+        const int idx = (int)threadIdx.x + kThreads * i;
+        if (idx < T::WFLOATS) WL[idx] = wv[i];
+    }
     __syncthreads();
 
-    // phase 1
+    // phase 1.  The weights of this lane's channel row: step s = filter row s / 2 (of channel s / 14),
+    // tap kx = 4 (s % 2) + kq; kx = 7 does not exist (weight 0).
     const int act = a[REEF_CONV_ACT], act2 = a[REEF_CONV_ACT2];
+    float ra[T::STEPS];
+#pragma unroll
+    for (int s = 0; s < T::STEPS; ++s) {
+        const int c = s / 14, ky = (s % 14) / 2, kx0 = 4 * (s & 1);
+        const bool real = c < C && kx0 + kq < 7;
+        const float w = WL[i16 * K + min(c, C - 1) * 49 + ky * 7 + min(kx0 + kq, 6)];
+        ra[s] = real ? w : 0.0f;
+    }
     for (int g = wave; g < T::NG; g += 4) {
         const int r = g >> 1, gc = g & 1;
         const int j = min(16 * gc + i16, 28);          // columns past the 29 a tile needs: computed, never read

@@ -722,7 +722,7 @@ class GraphBuilder:
             n = k["name"]
             sym = n.split("#")[0]
             if sym == "reef_conv2d_sp7_g2":
-                shared[n] = (3 * 15 * 64 + 16 * (5 * 32 + 1) + 32) * 4 + 16     # TileSp7: input patch + pooled-from block
+                shared[n] = (3 * 15 * 64 + 16 * (5 * 32 + 1) + 32 + 16 * 3 * 49) * 4 + 16     # TileSp7: input patch, pooled-from block, weight rows
             elif sym.startswith("reef_conv2d_sdp_") or sym.startswith("reef_conv2d_xdp2_"):
                 # TileBlk: patch, the three layers' parameters, the front filter's result, the depthwise stage's
                 stem, G = sym.startswith("reef_conv2d_sdp_"), tiling.ROW_TILES[sym.split("_")[-1]]
