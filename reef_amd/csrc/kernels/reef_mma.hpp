@@ -1132,7 +1132,10 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     int pf = 0;
     int it = 0;
     bool left = false;
-    for (; it + NS <= nsteps; it += NS) {
+    // (groups whose refills all exist; the last whole group follows with the refills the remaining
+    // steps need and no others: a load outside the buffer brings nothing but still takes its turn in
+    // the vector-memory pipe, and a group of them cost a layer with nsteps == NS 1700 cycles)
+    for (; it + 2 * NS <= nsteps; it += NS) {
         if (Poll::enabled) {
             // the flag is read one group ahead; a wavefront that sees it tells the others
             // through LDS and all of them leave after the barrier below
@@ -1149,6 +1152,21 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
             load_step(s, it + s + NS);
             // keeps each step's refill behind its own MFMAs instead of at the end of the group
             __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    if (!left && it + NS <= nsteps) {
+        if (Poll::enabled && pf) {
+            *sflag = 1;
+            left = true;
+        } else {
+            if (Poll::enabled) pf = poll.load();
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                mma_stage(s);
+                if (it + s + NS < nsteps) load_step(s, it + s + NS);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            it += NS;
         }
     }
     if (!left) {
@@ -2370,7 +2388,9 @@ __device__ __forceinline__ bool gemm_nt_direct_body(const ReefOpDesc& d, int tas
     };
     int pf = 0, it = 0;
     bool left = false;
-    for (; it + NS <= nsteps; it += NS) {
+    // (groups whose refills all exist, then the last whole group with the refills the remaining steps
+    // need and no others, as in the convolution)
+    for (; it + 2 * NS <= nsteps; it += NS) {
         if (Poll::enabled) {
             if (pf) {
                 *sflag = 1;
@@ -2384,6 +2404,21 @@ __device__ __forceinline__ bool gemm_nt_direct_body(const ReefOpDesc& d, int tas
             mma_stage(s);
             load_step(s, it + s + NS);
             __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    if (!left && it + NS <= nsteps) {
+        if (Poll::enabled && pf) {
+            *sflag = 1;
+            left = true;
+        } else {
+            if (Poll::enabled) pf = poll.load();
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                mma_stage(s);
+                if (it + s + NS < nsteps) load_step(s, it + s + NS);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            it += NS;
         }
     }
     if (!left) {
