@@ -831,7 +831,9 @@ __device__ __forceinline__ float lane_from_right(float v) {  // lane i <- lane (
 // (zero-padded to whole groups): the 64 lanes of a wavefront read 1 KiB contiguous, aligned, per
 // group of four taps.  Measured on the 3x3 layers of ResNet-152: 1.4 us less per launch.  The
 // model generator writes the copy as a parameter of its own; attr WPACK names its pointer slot.
-template <int R, int TN, int TM, bool PRE, bool ROWS, bool PACKED, class Poll>
+// SHORT: the copy for layers with fewer steps than the NS the loads run ahead (the entry picks it):
+// only the stages that exist are fetched, and there is no refilling loop.
+template <int R, int TN, int TM, bool PRE, bool ROWS, bool PACKED, bool SHORT, class Poll>
 __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int task, char* smem_raw,
                                                    const Poll& poll) {
     static_assert(!PRE || R == 1, "the pre-activation form exists for 1-tap filters only");
@@ -966,7 +968,7 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     // their way.  (The waits the compiler places count loads in issue order, whatever it is.)
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
-        load_a(s, s);
+        if (!SHORT || s < nsteps) load_a(s, s);
         asm volatile("" ::: "memory");
     }
     unsigned vb[ROWS ? TN + 2 : TN][ROWS ? 1 : R];
@@ -1045,7 +1047,7 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     };
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
-        load_b(s, s);
+        if (!SHORT || s < nsteps) load_b(s, s);
         asm volatile("" ::: "memory");
     }
 
@@ -1135,7 +1137,7 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     // (groups whose refills all exist; the last whole group follows with the refills the remaining
     // steps need and no others: a load outside the buffer brings nothing but still takes its turn in
     // the vector-memory pipe, and a group of them cost a layer with nsteps == NS 1700 cycles)
-    for (; it + 2 * NS <= nsteps; it += NS) {
+    for (; !SHORT && it + 2 * NS <= nsteps; it += NS) {
         if (Poll::enabled) {
             // the flag is read one group ahead; a wavefront that sees it tells the others
             // through LDS and all of them leave after the barrier below
@@ -1154,7 +1156,7 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
             __builtin_amdgcn_sched_barrier(0);
         }
     }
-    if (!left && it + NS <= nsteps) {
+    if (!SHORT && !left && it + NS <= nsteps) {
         if (Poll::enabled && pf) {
             *sflag = 1;
             left = true;
