@@ -42,19 +42,7 @@ struct OpConvDirect {
     static constexpr bool CHECKS_FLAG_ITSELF = true;   // the body makes the wrapper's first flag check
     template <class P>
     static __device__ __forceinline__ bool run(const ReefOpDesc& d, int task, char* smem, const P& p) {
-        // A layer (or split) with fewer steps than the loads run ahead takes the copy that fetches only
-        // the stages that exist.  Plain 1-tap filters only, by measurement on one device in one
-        // process: MobileNetV2 -3 %, ResNet-152 and Inception-v3 -0.2 %; with the pre-activated
-        // filters included DenseNet-201 +4 %, with the multi-tap ones Inception-v3 +1.6 % (the
-        // conditional fetches make the compiler wait for a stage's loads in issue order, which
-        // costs a layer with cold operands more than the fetches saved).
-        if constexpr (R == 1 && !PRE) {
-            typedef DirectGeom<R, TN, TM, PRE, ROWS> G;
-            const int channels = min(d.attr[REEF_CONV_CIN], d.attr[REEF_CONV_K_CHUNK]);
-            if ((channels + G::STEP_C - 1) / G::STEP_C < G::NS)
-                return conv2d_direct_body<R, TN, TM, PRE, ROWS, PACKED, true>(d, task, smem, p);
-        }
-        return conv2d_direct_body<R, TN, TM, PRE, ROWS, PACKED, false>(d, task, smem, p);
+        return conv2d_direct_body<R, TN, TM, PRE, ROWS, PACKED>(d, task, smem, p);
     }
 };
 // the same with the weights read from their packed copy

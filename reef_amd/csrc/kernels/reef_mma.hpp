@@ -782,9 +782,21 @@ struct DirectGeom {
     static constexpr int NB = ROWS ? TN + 2 : TN * RC;
     // vector-memory instructions per step (PRE: two 128-bit loads each of input scale and shift)
     static constexpr int LOADS = TM * ((RC / 4) + (RC % 4)) + NB + (PRE ? 4 : 0);
-    // steps of loads in flight per wavefront: up to 60 load instructions, 2 to 6 (row form: 8) steps
-    static constexpr int NS_MAX = ROWS ? 8 : 6;
-    static constexpr int NS = 60 / LOADS < 2 ? 2 : (60 / LOADS > NS_MAX ? NS_MAX : 60 / LOADS);
+    // Steps of loads in flight per wavefront.  All of them are issued before the first MFMA, and a
+    // wavefront that is still issuing loads multiplies nothing: with 8 steps ahead (all of a 14x14
+    // row-form layer at a split of two) cycle stamps showed 4600 cycles of issue, then 6600 of K loop
+    // whose MFMAs alone need 4600.  Fewer steps ahead start the MFMAs while the later loads are
+    // still being issued behind them.  Picked per family by timing whole networks with the code
+    // objects side by side in one process (ResNet-152 1.180 -> 1.102 ms, DenseNet-201 1.26 -> 1.18):
+    //   row form 4 (3: +1.8 %, 5 and 6: +2.3 % on ResNet-152), d1 16x32 2 (3: +3.2 %), d1 16x16 4
+    //   (3 and 6 the same), p1 16x16 2 (3: +1 %, 4: +3.5 % on DenseNet-201), d9 16x16 3 (2, 4 the
+    //   same); the others 40 loads' worth, at least 2 and at most 4.
+    static constexpr int NS_GEN = 40 / LOADS < 2 ? 2 : (40 / LOADS > 4 ? 4 : 40 / LOADS);
+    static constexpr int NS = ROWS ? 4
+                            : (R == 1 && TN == 1 && TM == 1) ? (PRE ? 2 : 4)
+                            : (R == 1 && TN == 2 && TM == 1 && !PRE) ? 2
+                            : (R == 9 && TN == 1 && TM == 1) ? 3
+                            : NS_GEN;
 };
 
 // Row form (ROWS; 3x3 filters, stride 1, padding 1; symbols reef_conv2d_r9_g<G>[m2]): the tile is
@@ -831,9 +843,7 @@ __device__ __forceinline__ float lane_from_right(float v) {  // lane i <- lane (
 // (zero-padded to whole groups): the 64 lanes of a wavefront read 1 KiB contiguous, aligned, per
 // group of four taps.  Measured on the 3x3 layers of ResNet-152: 1.4 us less per launch.  The
 // model generator writes the copy as a parameter of its own; attr WPACK names its pointer slot.
-// SHORT: the copy for layers with fewer steps than the NS the loads run ahead (the entry picks it):
-// only the stages that exist are fetched, and there is no refilling loop.
-template <int R, int TN, int TM, bool PRE, bool ROWS, bool PACKED, bool SHORT, class Poll>
+template <int R, int TN, int TM, bool PRE, bool ROWS, bool PACKED, class Poll>
 __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int task, char* smem_raw,
                                                    const Poll& poll) {
     static_assert(!PRE || R == 1, "the pre-activation form exists for 1-tap filters only");
@@ -968,7 +978,7 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     // their way.  (The waits the compiler places count loads in issue order, whatever it is.)
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
-        if (!SHORT || s < nsteps) load_a(s, s);
+        load_a(s, s);
         asm volatile("" ::: "memory");
     }
     unsigned vb[ROWS ? TN + 2 : TN][ROWS ? 1 : R];
@@ -1047,7 +1057,7 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     };
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
-        if (!SHORT || s < nsteps) load_b(s, s);
+        load_b(s, s);
         asm volatile("" ::: "memory");
     }
 
@@ -1137,7 +1147,7 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
     // (groups whose refills all exist; the last whole group follows with the refills the remaining
     // steps need and no others: a load outside the buffer brings nothing but still takes its turn in
     // the vector-memory pipe, and a group of them cost a layer with nsteps == NS 1700 cycles)
-    for (; !SHORT && it + 2 * NS <= nsteps; it += NS) {
+    for (; it + 2 * NS <= nsteps; it += NS) {
         if (Poll::enabled) {
             // the flag is read one group ahead; a wavefront that sees it tells the others
             // through LDS and all of them leave after the barrier below
@@ -1156,7 +1166,7 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
             __builtin_amdgcn_sched_barrier(0);
         }
     }
-    if (!SHORT && !left && it + NS <= nsteps) {
+    if (!left && it + NS <= nsteps) {
         if (Poll::enabled && pf) {
             *sflag = 1;
             left = true;
@@ -2280,7 +2290,7 @@ __device__ __forceinline__ bool gemm_nt_direct_body(const ReefOpDesc& d, int tas
                                                     const Poll& poll) {
     typedef TileD16<TN, TM> TD;
     constexpr int LOADS = 2 * (TM + TN);
-    constexpr int NS = 60 / LOADS > 6 ? 6 : 60 / LOADS;
+    constexpr int NS = 3;      // steps of loads in flight (6: BERT-base +1.8 %, 4: +1.7 %, 2: +0.7 %, same process)
     float* smem = (float*)smem_raw;
     int* sflag = (int*)(smem + 4 * TD::SUBS * TD::PART);
     const int* a = d.attr;
