@@ -774,26 +774,30 @@ struct TileD16 {
 
 template <int R, int TN, int TM = 1, bool PRE = false, bool ROWS = false>
 struct DirectGeom {
-    static constexpr int CPL = R == 1 ? 8 : 1;   // channels per k slot and step
+    // channels per k slot and step.  1-tap filters: 4 -- a 128-bit load of weights per lane and step.
+    // (8 halves the steps, but a step is also the unit in which loads and MFMAs alternate: with 4,
+    // same process, ResNet-152 -2 %, Inception-v3 -1.4 %, MobileNetV2 -4.7 %, DenseNet-201 -2.4 %;
+    // with 2 the weights come as 32-bit loads and ResNet-152 is 5-12 % slower.)
+    static constexpr int CPL = R == 1 ? 4 : 1;
     static constexpr int RC = R * CPL;           // A values per lane and step (x TN B values and MFMAs)
     static constexpr int STEP_C = 16 * CPL;      // channels a workgroup consumes per step
     // B values a lane loads per step: every tap of every pixel group, or (row form) one value
     // per input row of the tile
     static constexpr int NB = ROWS ? TN + 2 : TN * RC;
     // vector-memory instructions per step (PRE: two 128-bit loads each of input scale and shift)
-    static constexpr int LOADS = TM * ((RC / 4) + (RC % 4)) + NB + (PRE ? 4 : 0);
+    static constexpr int LOADS = TM * ((RC / 4) + (RC % 4)) + NB + (PRE ? 2 * (RC / 4) : 0);
     // Steps of loads in flight per wavefront.  All of them are issued before the first MFMA, and a
     // wavefront that is still issuing loads multiplies nothing: with 8 steps ahead (all of a 14x14
     // row-form layer at a split of two) cycle stamps showed 4600 cycles of issue, then 6600 of K loop
     // whose MFMAs alone need 4600.  Fewer steps ahead start the MFMAs while the later loads are
     // still being issued behind them.  Picked per family by timing whole networks with the code
     // objects side by side in one process (ResNet-152 1.180 -> 1.102 ms, DenseNet-201 1.26 -> 1.18):
-    //   row form 4 (3: +1.8 %, 5 and 6: +2.3 % on ResNet-152), d1 16x32 2 (3: +3.2 %), d1 16x16 4
-    //   (3 and 6 the same), p1 16x16 2 (3: +1 %, 4: +3.5 % on DenseNet-201), d9 16x16 3 (2, 4 the
-    //   same); the others 40 loads' worth, at least 2 and at most 4.
+    //   row form 4 (3: +1.8 %, 5 and 6: +2.3 % on ResNet-152), d1 16x32 2 (3: +3.2 %), d1 16x16 and
+    //   p1 16x16 3 (2 to 5 within 0.5 %), d9 16x16 3 (2, 4 the same); the others 40 loads' worth, at
+    //   least 2 and at most 4.  (Steps of 1-tap filters are 64 channels.)
     static constexpr int NS_GEN = 40 / LOADS < 2 ? 2 : (40 / LOADS > 4 ? 4 : 40 / LOADS);
     static constexpr int NS = ROWS ? 4
-                            : (R == 1 && TN == 1 && TM == 1) ? (PRE ? 2 : 4)
+                            : (R == 1 && TN == 1 && TM == 1) ? 3
                             : (R == 1 && TN == 2 && TM == 1 && !PRE) ? 2
                             : (R == 9 && TN == 1 && TM == 1) ? 3
                             : NS_GEN;
@@ -932,7 +936,7 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
 
     constexpr int NB = G::NB;
     float ra[NS][TM][RC], rb[NS][NB];
-    float rps[NS][PRE ? 8 : 1], rpt[NS][PRE ? 8 : 1];
+    float rps[NS][PRE ? RC : 1], rpt[NS][PRE ? RC : 1];
     auto load_a = [&](int s, int step) {
         // offsets are below kOutside (a power of two), so or-ing it in moves them outside
         const unsigned outm = step < lane_steps ? 0u : kOutside;
@@ -1021,7 +1025,7 @@ __device__ __forceinline__ bool conv2d_direct_body(const ReefOpDesc& d_in, int t
             const unsigned op = vpre | outm;
             const unsigned sp = (unsigned)step * (unsigned)G::STEP_C * 4u;   // uniform
 #pragma unroll
-            for (int q = 0; q < 2; ++q) {
+            for (int q = 0; q < RC / 4; ++q) {
                 const f32x4 sc = __builtin_bit_cast(
                     f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_ps, (int)(op + 16u * q), (int)sp, 0));
                 const f32x4 sh = __builtin_bit_cast(
