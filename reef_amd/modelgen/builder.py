@@ -55,9 +55,12 @@ class Tensor:
 
 
 class GraphBuilder:
-    def __init__(self, name, seed=rng.BASE_SEED, weight_std=None):
+    def __init__(self, name, seed=rng.BASE_SEED, weight_std=None, under_load=False):
         self.name = name
         self.seed = seed
+        # the model is meant to run as a best-effort model beside others: tile choices measured
+        # with several clients on the device come before those measured alone (tuned.py)
+        self.under_load = under_load
         self.weight_std = weight_std   # fixed std (BERT: 0.02); None = He-normal
         self.storage = []
         self.kernels = []
@@ -230,7 +233,8 @@ class GraphBuilder:
             out = Tensor(out.idx, (cout,))
         t = force or tiling.choose(M, N, K, fused=fused_reduce, pointwise=(kh, kw) == (1, 1),
                                    taps=kh * kw, direct=tiling.direct_ok(cin, kh, kw),
-                                   rows=tiling.rows_ok(kh, kw, sh, sw, ph, pw), image=(Ho, Wo))
+                                   rows=tiling.rows_ok(kh, kw, sh, sw, ph, pw), image=(Ho, Wo),
+                                   under_load=self.under_load)
         if t.get("fused"):
             fused_reduce = True       # the measured table asks for the split folded into the launch
         pre = []

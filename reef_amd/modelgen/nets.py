@@ -186,7 +186,7 @@ def mobilenet_v2(image=(3, 224, 224), classes=1000, name="mobilenetv2", seed=rng
 
 
 def densenet(blocks=(6, 12, 48, 32), growth=32, image=(3, 224, 224), classes=1000, name="densenet201",
-             seed=rng.BASE_SEED, fuse_stem=True, pool_first=True):
+             seed=rng.BASE_SEED, fuse_stem=True, pool_first=True, under_load=False):
     """DenseNet-BC (201: blocks 6/12/48/32, growth 32): every layer reads the running
     concatenation through its own BN + ReLU (it cannot be folded into the producing
     convolution because each consumer has its own statistics; it is folded into the input
@@ -199,8 +199,10 @@ def densenet(blocks=(6, 12, 48, 32), growth=32, image=(3, 224, 224), classes=100
     concatenation through the BN + ReLU and the filter runs on a quarter of the pixels, writing
     straight into the next block's buffer -- a quarter of the transition's multiplications, same
     parameters in the same order; the network's last BN + ReLU is applied by the global average
-    pool as it reads.  False keeps the textbook order and a launch for that BN + ReLU."""
-    g = GraphBuilder(name, seed)
+    pool as it reads.  False keeps the textbook order and a launch for that BN + ReLU.
+    under_load: tile choices for a model that runs as a best-effort model beside others
+    (tuned.TUNED_UNDER_LOAD) instead of those for a model that has the device to itself."""
+    g = GraphBuilder(name, seed, under_load=under_load)
     x = g.input("data", image)
     fuse_stem = fuse_stem and image[0] <= 3
     y = None if fuse_stem else g.conv2d(x, 2 * growth, 7, 2, 3, bias=True, act=ACT_RELU)
@@ -440,8 +442,10 @@ def token_input(name, seq, vocab, seed=rng.BASE_SEED):
     return rng.randint(name + "/ids", seq, vocab, seed)
 
 
+# The networks of the benchmark configurations in the roles they have there: DenseNet-201 is a
+# best-effort model in every configuration that names it, so it is generated for that role.
 BUILDERS = {
     "resnet18": lambda: resnet(18), "resnet50": lambda: resnet(50), "resnet152": lambda: resnet(152),
-    "mobilenetv2": mobilenet_v2, "densenet201": densenet, "inceptionv3": inception_v3,
+    "mobilenetv2": mobilenet_v2, "densenet201": lambda: densenet(under_load=True), "inceptionv3": inception_v3,
     "bert_base": bert, "mocked_kernel": mocked_kernel,
 }

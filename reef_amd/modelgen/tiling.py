@@ -9,7 +9,7 @@ split-K to put a workgroup on every CU.
 """
 import math
 
-from .tuned import TUNED
+from .tuned import TUNED, TUNED_UNDER_LOAD
 
 # name -> (id, BM, BN, relative MFMA efficiency of the inner loop, workgroups per CU)
 TILES = {
@@ -154,12 +154,17 @@ def _steps_time(bm, bn, eff, steps):
 
 
 def choose(M, N, K, allow_split=True, tiles=None, max_split=32, fused=True, pointwise=False,
-           taps=1, direct=False, rows=False, image=None):
+           taps=1, direct=False, rows=False, image=None, under_load=False):
     """Returns dict(tile, tile_id, BM, BN, split_k, k_chunk, m_tiles, n_tiles, tasks).
     Measured choices (tuned.py) win over the analytic model for the shapes they cover; an entry
-    that names the direct tile counts only if the caller says the filter qualifies."""
+    that names the direct tile counts only if the caller says the filter qualifies.
+    under_load: the layer belongs to a model that shares the device with other streams; the
+    entries measured for that case (TUNED_UNDER_LOAD) come before those measured alone."""
     if allow_split and tiles is None and not fused:
-        hit = TUNED.get((M, N, K, 1 if pointwise else 0))
+        key = (M, N, K, 1 if pointwise else 0)
+        hit = TUNED.get(key)
+        if under_load and key in TUNED_UNDER_LOAD:
+            hit = TUNED_UNDER_LOAD[key] + (hit[2] if hit is not None else 0.0,)
         if hit is not None and hit[0] in ROW_TILES:
             if rows and image is not None:
                 t = forced_rows(hit[0], M, image[0], image[1], K, abs(hit[1]))

@@ -474,6 +474,27 @@ def test_tile_choice_outside_the_measured_table():
     assert 4.0 < tiling.direct_cost("16x32k4", g, True) < 12.0
 
 
+def test_a_model_generated_for_running_under_load_differs_in_its_splits_only():
+    """GraphBuilder(under_load=True) takes the tile choices measured with several clients on the
+    device where the table has them (tuned.TUNED_UNDER_LOAD): same kernels in the same order on
+    the same storages with the same parameters, a different split of K on the shapes listed."""
+    from reef_amd.modelgen import nets, tiling, tuned
+    for key, (tile, split) in tuned.TUNED_UNDER_LOAD.items():
+        assert key in tuned.TUNED and split < 0 and abs(split) > abs(tuned.TUNED[key][1])
+    M, N, K = 32, 196, 1152
+    alone = tiling.choose(M, N, K, fused=False, taps=9, direct=True, rows=True, image=(14, 14))
+    loaded = tiling.choose(M, N, K, fused=False, taps=9, direct=True, rows=True, image=(14, 14), under_load=True)
+    assert alone["tile"] == loaded["tile"] == "g1" and (alone["split_k"], loaded["split_k"]) == (2, 4)
+    assert loaded["fused"]
+    a, b = nets.densenet(blocks=(2, 2, 2, 2)), nets.densenet(blocks=(2, 2, 2, 2), under_load=True)
+    assert [k["name"] for k in a.kernels] == [k["name"] for k in b.kernels]
+    assert [k["args"] for k in a.kernels] == [k["args"] for k in b.kernels]
+    assert [p[0] for p in a.params] == [p[0] for p in b.params]
+    differing = [i for i, (x, y) in enumerate(zip(a.kernels, b.kernels)) if x["launch_params"] != y["launch_params"]]
+    assert differing and all(a.kernels[i]["launch_params"][0] < b.kernels[i]["launch_params"][0] for i in differing)
+    assert nets.BUILDERS["densenet201"]().under_load        # the benchmark's best-effort model
+
+
 def test_stream_drained_falls_back_to_the_query_of_a_backend_without_counters(fake):
     """reef_hal_stream_drained is what the padding loop asks between two real-time launches (the
     reference asks its runtime, scheduler.cpp:655-672 via GPUStreamEmpty); a backend that has no
