@@ -653,7 +653,7 @@ class GraphBuilder:
         if force_tile is not None:
             t = tiling.forced(force_tile, M, N, K, 1)
         else:
-            t = tiling.choose_gemm(M, N, K, batch, direct_ok)
+            t = tiling.choose_gemm(M, N, K, batch, direct_ok, under_load=self.under_load)
         direct = t["tile"] in tiling.GEMM_DIRECT_TILES
         assert direct_ok or not direct, "this GEMM has no direct form"
         args = [a.idx, b.idx, out.idx]

@@ -365,7 +365,8 @@ def inception_v3(image=(3, 299, 299), classes=1000, name="inceptionv3", seed=rng
 
 
 def bert(layers=12, hidden=768, heads=12, ffn=3072, seq=128, vocab=30522, name="bert_base",
-         seed=rng.BASE_SEED, attention_mask=False, fused_attention=True, fuse_layernorm=True):
+         seed=rng.BASE_SEED, attention_mask=False, fused_attention=True, fuse_layernorm=True,
+         under_load=False):
     """BERT encoder (base: 12 layers, hidden 768, 12 heads, FFN 3072, sequence 128), fp32,
     weights ~ N(0, 0.02).  Token ids are an int64 input, as in the reference's BERT model
     (resource/bert/bert.json storage[0]).  The per-head views of Q, K, V and of the context
@@ -383,8 +384,10 @@ def bert(layers=12, hidden=768, heads=12, ffn=3072, seq=128, vocab=30522, name="
     before the FFN) is not a launch of its own: the projection normalises the rows on the way into
     its tiles and writes them out for the next residual (reef_gemm_ntl_*); only the last
     LayerNorm of the network remains a kernel, and the residual sums are made by the epilogues
-    of the products in front -- 24 launches fewer, same parameters in the same order."""
-    g = GraphBuilder(name, seed, weight_std=0.02)
+    of the products in front -- 24 launches fewer, same parameters in the same order.
+    under_load: tile choices for a model that runs as a best-effort model beside others
+    (tuned.GEMM_UNDER_LOAD) instead of those for a model that has the device to itself."""
+    g = GraphBuilder(name, seed, weight_std=0.02, under_load=under_load)
     hd = hidden // heads
     ids = g.input("input0", (seq,), "int64")
     mask = g.input("attention_mask", (seq,), "uint1") if attention_mask else None
@@ -442,10 +445,11 @@ def token_input(name, seq, vocab, seed=rng.BASE_SEED):
     return rng.randint(name + "/ids", seq, vocab, seed)
 
 
-# The networks of the benchmark configurations in the roles they have there: DenseNet-201 is a
-# best-effort model in every configuration that names it, so it is generated for that role.
+# The networks of the benchmark configurations in the roles they have there: DenseNet-201 and
+# BERT-base are best-effort models in every configuration that names them, so they are generated
+# for that role (under_load).
 BUILDERS = {
     "resnet18": lambda: resnet(18), "resnet50": lambda: resnet(50), "resnet152": lambda: resnet(152),
     "mobilenetv2": mobilenet_v2, "densenet201": lambda: densenet(under_load=True), "inceptionv3": inception_v3,
-    "bert_base": bert, "mocked_kernel": mocked_kernel,
+    "bert_base": lambda: bert(under_load=True), "mocked_kernel": mocked_kernel,
 }

@@ -9,7 +9,7 @@ split-K to put a workgroup on every CU.
 """
 import math
 
-from .tuned import TUNED, TUNED_UNDER_LOAD
+from .tuned import TUNED, TUNED_UNDER_LOAD, GEMM_UNDER_LOAD
 
 # name -> (id, BM, BN, relative MFMA efficiency of the inner loop, workgroups per CU)
 TILES = {
@@ -54,7 +54,7 @@ GEMM_TILES = ("128x128", "64x64", "32x128", "32x32k4", "64x32k2")
 GEMM_DIRECT_TILES = ("16x16k4", "16x32k4", "32x32d4")   # reef_gemm_ntd_<tile>
 
 
-def choose_gemm(M, N, K, batch=1, direct_ok=False):
+def choose_gemm(M, N, K, batch=1, direct_ok=False, under_load=False):
     """Tile of a GEMM, and for a direct tile whether K is split in two across workgroups.
     Without a measured table: the staged choice of the analytic model, against the direct tiles
     (both operands K-contiguous) scored by the rule the batch-1 convolutions were found to
@@ -63,7 +63,14 @@ def choose_gemm(M, N, K, batch=1, direct_ok=False):
     launch through the pair slots) halves a workgroup's lines and doubles the workgroups, at a
     price measured on BERT-base's 128 x 768 x 3072 product (32x32d4: 25.8 us whole, 16.8 us
     split in two, against 19.4 us for 16x32k4 whole; splits of three and more meet on counters
-    and were slower throughout)."""
+    and were slower throughout).
+    under_load: the product belongs to a model that shares the device with other streams; a
+    choice measured for that case (tuned.GEMM_UNDER_LOAD) comes first."""
+    if under_load and direct_ok and batch == 1 and (M, N, K) in GEMM_UNDER_LOAD:
+        tile, split = GEMM_UNDER_LOAD[(M, N, K)]
+        t = forced(tile, M, N, K, 1)
+        t["gemm_split"] = split
+        return t
     staged = choose(M, N, K, allow_split=False, tiles=GEMM_TILES)
     if not direct_ok:
         return staged

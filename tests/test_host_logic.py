@@ -493,6 +493,15 @@ def test_a_model_generated_for_running_under_load_differs_in_its_splits_only():
     differing = [i for i, (x, y) in enumerate(zip(a.kernels, b.kernels)) if x["launch_params"] != y["launch_params"]]
     assert differing and all(a.kernels[i]["launch_params"][0] < b.kernels[i]["launch_params"][0] for i in differing)
     assert nets.BUILDERS["densenet201"]().under_load        # the benchmark's best-effort model
+    # matrix products: BERT-base's FFN-down product splits K in four instead of two
+    for (M, N, K), (tile, split) in tuned.GEMM_UNDER_LOAD.items():
+        alone, loaded = tiling.choose_gemm(M, N, K, 1, True), tiling.choose_gemm(M, N, K, 1, True, under_load=True)
+        assert (loaded["tile"], loaded["gemm_split"]) == (tile, split) != (alone["tile"], alone.get("gemm_split", 1))
+        assert tiling.choose_gemm(M, N, K, 2, True, under_load=True)["tile"] == tiling.choose_gemm(M, N, K, 2, True)["tile"]
+    a, b = nets.bert(layers=1), nets.bert(layers=1, under_load=True)
+    assert [k["name"] for k in a.kernels] == [k["name"] for k in b.kernels]
+    assert [p[0] for p in a.params] == [p[0] for p in b.params]
+    assert sum(x["launch_params"] != y["launch_params"] for x, y in zip(a.kernels, b.kernels)) == 1
 
 
 def test_stream_drained_falls_back_to_the_query_of_a_backend_without_counters(fake):
