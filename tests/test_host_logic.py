@@ -474,24 +474,27 @@ def test_tile_choice_outside_the_measured_table():
     assert 4.0 < tiling.direct_cost("16x32k4", g, True) < 12.0
 
 
-def test_a_model_generated_for_running_under_load_differs_in_its_splits_only():
+def test_a_model_generated_for_running_under_load_differs_in_its_tiles_and_splits_only():
     """GraphBuilder(under_load=True) takes the tile choices measured with several clients on the
     device where the table has them (tuned.TUNED_UNDER_LOAD): same kernels in the same order on
-    the same storages with the same parameters, a different split of K on the shapes listed."""
+    the same storages with the same parameters, a different tile or split of K on the shapes listed."""
     from reef_amd.modelgen import nets, tiling, tuned
     for key, (tile, split) in tuned.TUNED_UNDER_LOAD.items():
-        assert key in tuned.TUNED and split < 0 and abs(split) > abs(tuned.TUNED[key][1])
+        # a finer split of K folded inside the launch, or another tile
+        assert key in tuned.TUNED and (tile, split) != tuned.TUNED[key][:2]
+        assert (split < 0 and abs(split) > abs(tuned.TUNED[key][1])) or tile != tuned.TUNED[key][0]
     M, N, K = 32, 196, 1152
     alone = tiling.choose(M, N, K, fused=False, taps=9, direct=True, rows=True, image=(14, 14))
     loaded = tiling.choose(M, N, K, fused=False, taps=9, direct=True, rows=True, image=(14, 14), under_load=True)
     assert alone["tile"] == loaded["tile"] == "g1" and (alone["split_k"], loaded["split_k"]) == (2, 4)
     assert loaded["fused"]
     a, b = nets.densenet(blocks=(2, 2, 2, 2)), nets.densenet(blocks=(2, 2, 2, 2), under_load=True)
-    assert [k["name"] for k in a.kernels] == [k["name"] for k in b.kernels]
-    assert [k["args"] for k in a.kernels] == [k["args"] for k in b.kernels]
+    # the same convolutions on the same parameters; a tile that has a pre-activated form (p1) takes
+    # the BN + ReLU in front of it into its loads, so the model under load may have fewer launches
+    convs = lambda g: [k["attrs"][:12] for k in g.kernels if k["name"].startswith("reef_conv2d_")]
+    assert convs(a) == convs(b) and len(b.kernels) <= len(a.kernels)
     assert [p[0] for p in a.params] == [p[0] for p in b.params]
-    differing = [i for i, (x, y) in enumerate(zip(a.kernels, b.kernels)) if x["launch_params"] != y["launch_params"]]
-    assert differing and all(a.kernels[i]["launch_params"][0] < b.kernels[i]["launch_params"][0] for i in differing)
+    assert [k["launch_params"] for k in a.kernels] != [k["launch_params"] for k in b.kernels]
     assert nets.BUILDERS["densenet201"]().under_load        # the benchmark's best-effort model
     # matrix products: BERT-base's FFN-down product splits K in four instead of two
     for (M, N, K), (tile, split) in tuned.GEMM_UNDER_LOAD.items():
